@@ -1,0 +1,259 @@
+/*
+ * singa_hip.h — C ABI of the MI355X (gfx950) backward-pass + SGD-update engine for Apache SINGA.
+ *
+ * Every entry point is what a HIP `Device` / `tensor_math` specialisation / operation function in
+ * a SINGA tree would bind for the backward path.  Conventions:
+ *   - plain pointers and sizes only; all data pointers are DEVICE pointers unless named host_*;
+ *   - tensors are dense, row-major / NCHW, fp32 unless the suffix says otherwise;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); work is only enqueued,
+ *     never synchronised, except where stated;
+ *   - the return value is 0 on success, a positive hipError_t value when the HIP runtime failed,
+ *     or a negative SGH_E* code when the arguments were rejected on the host.  Nothing throws or
+ *     aborts: SINGA's glue wraps each call in CHECK_EQ(rc, 0) to keep its own abort-on-error
+ *     convention (reference: src/utils/logging.cc:105-110, include/singa/utils/cuda_utils.h:96-117);
+ *   - the library allocates device memory only inside sgh_malloc (the pool); kernels that need
+ *     scratch take an explicit workspace whose size sgh_*_workspace_bytes reports.
+ *
+ * Reference paths below are relative to the apache/singa source tree.
+ */
+#ifndef SINGA_HIP_H_
+#define SINGA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SGH_API __attribute__((visibility("default")))
+
+/* ---- error codes (negative: rejected on the host before any launch) */
+#define SGH_OK 0
+#define SGH_EINVAL (-1)     /* bad argument (null pointer, negative size, bad geometry) */
+#define SGH_EWORKSPACE (-2) /* workspace missing or too small */
+#define SGH_EUNSUPPORTED (-3)
+#define SGH_ELABEL (-4)     /* a class label was out of range (checked variant only) */
+#define SGH_ENOMEM (-5)
+
+/* Human-readable text for a return code (static storage). */
+SGH_API const char *sgh_error_string(int rc);
+/* Library version and the GPU architecture the code objects were built for ("gfx950"). */
+SGH_API const char *sgh_version(void);
+SGH_API const char *sgh_arch(void);
+
+/* =====================================================================================
+ * Device runtime.  Replaces what CudaGPU provides to SINGA:
+ *   include/singa/core/device.h:57-174 (Device), src/core/device/cuda_gpu.cc:56-209
+ *   (Setup, DoExec's stream, CopyToFrom, Malloc/Free, Sync, TimeProfilingDoExec) and the
+ *   DeviceMemPool of include/singa/core/memory.h:37-54 / src/core/memory/memory.cc.
+ * One sgh_device owns one HIP stream (default priority) and one caching memory pool on
+ * hipMalloc.  All pool blocks are recycled in submission order on that single stream, which
+ * is the invariant SINGA's Graph relies on when it frees blocks right after enqueueing their
+ * last consumer (src/core/scheduler/scheduler.cc:349-354).
+ * ===================================================================================== */
+typedef struct sgh_device sgh_device;
+
+SGH_API int sgh_device_count(int *count);
+/* Platform::CreateCudaGPUsOn analogue (src/core/device/platform.cc:137-160). */
+SGH_API int sgh_device_open(int gpu_id, sgh_device **out);
+SGH_API int sgh_device_close(sgh_device *dev);
+/* The stream behind Device::Exec for this device (hipStream_t as void*). */
+SGH_API void *sgh_device_stream(sgh_device *dev);
+/* Device::Sync (src/core/device/cuda_gpu.cc:206-209): blocks until the stream is idle. */
+SGH_API int sgh_device_sync(sgh_device *dev);
+
+/* DeviceMemPool::Malloc / Free (include/singa/core/memory.h:41-45).  Size-bucketed cache:
+ * a freed block goes back to its bucket and is handed out again without touching the driver.
+ * Like CudaGPU::Malloc the memory is NOT zero-filled (src/core/device/cuda_gpu.cc:187-197). */
+SGH_API int sgh_malloc(sgh_device *dev, void **ptr, size_t bytes);
+SGH_API int sgh_free(sgh_device *dev, void *ptr);
+/* DeviceMemPool::GetMemUsage: bytes handed out, bytes cached in the pool, driver calls made. */
+SGH_API int sgh_pool_stats(sgh_device *dev, size_t *in_use, size_t *cached, size_t *driver_allocs);
+/* Return every cached block to the driver. */
+SGH_API int sgh_pool_trim(sgh_device *dev);
+
+/* Device::CopyToFrom (src/core/device/cuda_gpu.cc:171-175).  kind: 0 H2H, 1 H2D, 2 D2H, 3 D2D
+ * (= core.proto CopyDirection, src/proto/core.proto:43-48).  D2H and H2D block until the
+ * copy has completed so the host may touch the buffer when the call returns. */
+SGH_API int sgh_memcpy(sgh_device *dev, void *dst, const void *src, size_t bytes, int kind);
+SGH_API int sgh_memset_f32(float *dst, float value, size_t n, void *stream);
+
+/* Per-op timing for Graph profiling (TimeProfilingDoExec / EvaluateTimeElapsed,
+ * src/core/device/cuda_gpu.cc:117-169): event pairs on the device stream. */
+typedef struct sgh_event sgh_event;
+SGH_API int sgh_event_create(sgh_event **ev);
+SGH_API int sgh_event_destroy(sgh_event *ev);
+SGH_API int sgh_event_record(sgh_event *ev, void *stream);
+/* Blocks on `stop`, then returns stop - start in milliseconds. */
+SGH_API int sgh_event_elapsed_ms(sgh_event *start, sgh_event *stop, float *ms);
+
+/* =====================================================================================
+ * tensor_math backward ops (HIP specialisations of src/core/tensor/tensor_math.h)
+ * ===================================================================================== */
+
+/* ReLUBackward<float, Lang>: tensor_math.h:175-179; CPU tensor_math_cpp.h:446-451;
+ * CUDA math_kernel.cu:253-261.  dx[i] = x[i] > 0 ? dy[i] : 0 (x = the ReLU input). */
+SGH_API int sgh_relu_bwd_f32(const float *dy, const float *x, float *dx, size_t n, void *stream);
+/* ReLU<float, Lang>: tensor_math_cpp.h:585-589 (needed to produce the backward's inputs). */
+SGH_API int sgh_relu_fwd_f32(const float *x, float *y, size_t n, void *stream);
+
+/* SoftmaxCrossEntropyBwd<float, Lang>: tensor_math.h:475-480; CPU tensor_math_cpp.h:1090-1119;
+ * CUDA math_kernel.cu:564-611; host wrapper src/core/tensor/tensor.cc:1717-1758.
+ * grad = (p - onehot(t)) * scale  (int_target = 1, t is int32 [batch]) or
+ * grad = (p - t / rowsum(t)) * scale (int_target = 0, t is int32 [batch, dim]).
+ * grad may alias p (the reference works in place on a clone of p).  scale = 1 reproduces the
+ * reference op; scale = 1/batch additionally fuses the "dx /= N" that follows it in
+ * python/singa/autograd.py:1319-1322.  Labels are trusted like on the reference GPU path;
+ * a label outside [0, dim) leaves its row as p * scale and raises the device-side error
+ * flag readable with sgh_softmax_ce_label_errors (the CPU reference aborts on negatives). */
+SGH_API int sgh_softmax_ce_bwd_f32(const float *p, const int32_t *t, float *grad, size_t batch,
+                                   size_t dim, int int_target, float scale, void *stream);
+/* Number of out-of-range labels seen since the last call (synchronises the stream). */
+SGH_API int sgh_softmax_ce_label_errors(void *stream, int *count);
+/* SoftMax<float, Lang> (rows) and ComputeCrossEntropy<float, Lang>: forward helpers,
+ * tensor_math_cpp.h:361-379, :1058-1088; CUDA tensor_math_cuda.h:1274-1339. */
+SGH_API int sgh_softmax_fwd_f32(const float *x, float *p, size_t batch, size_t dim, void *stream);
+SGH_API int sgh_cross_entropy_fwd_f32(const float *p, const int32_t *t, float *loss, size_t batch,
+                                      size_t dim, int int_target, void *stream);
+
+/* Axpy<float, Lang>, scalar and Tensor-alpha overloads: tensor_math.h:393-402;
+ * CPU tensor_math_cpp.h:788-823; CUDA tensor_math_cuda.h:1031-1072 (device pointer mode).
+ * y += alpha * x. */
+SGH_API int sgh_axpy_f32(float alpha, const float *x, float *y, size_t n, void *stream);
+SGH_API int sgh_axpy_devalpha_f32(const float *alpha_dev, const float *x, float *y, size_t n,
+                                  void *stream);
+
+/* EltwiseMult<float, Lang>: tensor_math.h:162-172; CPU tensor_math_cpp.h:432-444; CUDA
+ * tensor_math_cuda.h:300-362.  out = a * b; b_is_scalar = 1 reads b[0] for every element,
+ * which is the stride-0 broadcast view of "buf *= mom_value" (python/singa/opt.py:299-300)
+ * without materialising it.  out may alias a. */
+SGH_API int sgh_eltwise_mult_f32(const float *a, const float *b, int b_is_scalar, float *out,
+                                 size_t n, void *stream);
+/* Add<float, Lang> (Tensor::operator+=, src/core/tensor/tensor.cc:579-586): gradient fan-in
+ * of python/singa/autograd.py:204.  out may alias a or b. */
+SGH_API int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream);
+
+/* Fused SGD-momentum update = the four tensor ops of SGD.apply, python/singa/opt.py:269-310,
+ * in one pass:  [g += wd*p];  v = mu*v + (1-damp)*g;  g' = nesterov ? g + mu*v : v;
+ * p -= lr*g'.  wd == 0 and mu == 0 skip their terms exactly like the Python `if`s; with
+ * mu == 0, v may be NULL.  g is not written.
+ * hyper_dev (device variant) points at {lr, mu, damp, wd} as four consecutive device floats,
+ * the 1-element device tensors the reference keeps (opt.py:222-259). */
+SGH_API int sgh_sgd_momentum_f32(float *p, const float *g, float *v, size_t n, float lr, float mu,
+                                 float damp, float wd, int nesterov, void *stream);
+SGH_API int sgh_sgd_momentum_devhyper_f32(float *p, const float *g, float *v, size_t n,
+                                          const float *hyper_dev, int nesterov, void *stream);
+/* The same update for many parameter tensors in ONE launch (the per-parameter loop of
+ * Optimizer.call, python/singa/opt.py:107-111).  table_dev is a device array of `count`
+ * sgh_sgd_item; max_n is the largest item. */
+typedef struct sgh_sgd_item {
+  float *p;
+  const float *g;
+  float *v;
+  uint64_t n;
+} sgh_sgd_item;
+SGH_API int sgh_sgd_momentum_multi_f32(const sgh_sgd_item *table_dev, int count, size_t total_n,
+                                       float lr, float mu, float damp, float wd, int nesterov,
+                                       void *stream);
+
+/* GEMM<float, Lang>: tensor_math.h:444-448; CPU tensor_math_cpp.h:877-899 (cblas_sgemm,
+ * row-major).  C[M,N] = alpha * op(A) * op(B) + beta * C; lda/ldb/ldc are row pitches of the
+ * stored matrices.  Used by Linear backward: Mult(dy, W^T), Mult(x^T, dy)
+ * (python/singa/autograd.py:613-623). */
+SGH_API int sgh_gemm_f32(int transA, int transB, int M, int N, int K, float alpha, const float *A,
+                         int lda, const float *B, int ldb, float beta, float *C, int ldc,
+                         void *stream);
+/* SumRows<float, Lang> (Sum(dy, 0), src/core/tensor/tensor.cc:1523-1538): out[j] = sum_i m[i][j].
+ * Bias gradient of AddBias.backward (python/singa/autograd.py:696-709). */
+SGH_API int sgh_sum_rows_f32(const float *m, float *out, int rows, int cols, void *stream);
+/* AddRow (bias add of Linear forward, src/core/tensor/tensor.cc:1294-1316): m[i][j] += v[j]. */
+SGH_API int sgh_add_row_f32(const float *v, float *m, int rows, int cols, void *stream);
+
+/* =====================================================================================
+ * Operation entry points (the Gpu* functions of src/model/operation/{convolution,batchnorm,pooling}.cc)
+ * ===================================================================================== */
+
+/* Geometry of a ConvHandle (src/model/operation/convolution.h:43-90; ctor
+ * src/model/operation/convolution.cc:29-66).  P, Q are derived with the reference's integer
+ * division; sgh_conv_geom_init fills them and validates the rest. */
+typedef struct sgh_conv_geom {
+  int N, C, H, W;       /* input  [N, C, H, W]                    */
+  int K, R, S;          /* weight [K, C, R, S]                    */
+  int stride_h, stride_w, pad_h, pad_w;
+  int P, Q;             /* output [N, K, P, Q]                    */
+} sgh_conv_geom;
+SGH_API int sgh_conv_geom_init(sgh_conv_geom *g, int N, int C, int H, int W, int K, int R, int S,
+                               int stride_h, int stride_w, int pad_h, int pad_w);
+
+#define SGH_CONV_FWD 0
+#define SGH_CONV_DGRAD 1
+#define SGH_CONV_WGRAD 2
+/* Scratch bytes the given pass needs for this geometry (CudnnConvHandle::workspace_count,
+ * src/model/operation/convolution.cc:560-571). */
+SGH_API size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which);
+
+/* GpuConvBackwardx (src/model/operation/convolution.cc:634-656; native algorithm
+ * src/model/layer/convolution.cc:178-182 + Col2im :224-248):
+ * dx[n,c,h,w] = sum_{k,r,s} dy[n,k,p,q] * W[k,c,r,s], h = p*stride - pad + r. */
+SGH_API int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx,
+                               void *workspace, size_t ws_bytes, void *stream);
+/* GpuConvBackwardW (src/model/operation/convolution.cc:658-681; native algorithm
+ * src/model/layer/convolution.cc:166-177 + Im2col :197-222):
+ * dW[k,c,r,s] = sum_{n,p,q} dy[n,k,p,q] * x[n,c,p*stride-pad+r,q*stride-pad+s].
+ * The split reduction is summed in a fixed order: results are run-to-run identical. */
+SGH_API int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, float *dW,
+                               void *workspace, size_t ws_bytes, void *stream);
+/* GpuConvBackwardb (src/model/operation/convolution.cc:684-702; native CPU :425-440):
+ * db[k] = sum_{n,p,q} dy[n,k,p,q]. */
+SGH_API int sgh_conv_bgrad_f32(const sgh_conv_geom *g, const float *dy, float *db, void *stream);
+/* GpuConvForward (src/model/operation/convolution.cc:585-632); bias may be NULL. */
+SGH_API int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W,
+                             const float *bias, float *y, void *workspace, size_t ws_bytes,
+                             void *stream);
+
+/* GpuBatchNormForwardTraining (src/model/operation/batchnorm.cc:287-329), spatial mode:
+ * per-channel batch mean / biased variance over N*HW, y = gamma*(x-mean)*invstd + beta,
+ * running = (1-factor)*running + factor*batch (unbiased variance), saves (mean, invstd) with
+ * invstd = 1/sqrt(var + eps) in the slots Python calls (mean, var)
+ * (python/singa/autograd.py:1777-1781).  running_* may be NULL.
+ * workspace (both passes): sgh_bn_workspace_bytes(N, C, HW) bytes of per-channel partial sums. */
+SGH_API size_t sgh_bn_workspace_bytes(int N, int C, int HW);
+SGH_API int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float *beta,
+                                 float *running_mean, float *running_var, float factor, float eps,
+                                 float *y, float *save_mean, float *save_invstd, int N, int C,
+                                 int HW, void *workspace, size_t ws_bytes, void *stream);
+/* GpuBatchNormBackward (src/model/operation/batchnorm.cc:368-404):
+ * dbeta = sum dy, dgamma = sum dy*xhat, dx = gamma*invstd/M * (M*dy - dbeta - xhat*dgamma).
+ * dbeta = sum dy etc. are summed in a fixed order: results are run-to-run identical. */
+SGH_API int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma,
+                           const float *save_mean, const float *save_invstd, float *dx,
+                           float *dgamma, float *dbeta, int N, int C, int HW, void *workspace,
+                           size_t ws_bytes, void *stream);
+
+/* Geometry of a PoolingHandle (src/model/operation/pooling.h:40-71; ctor pooling.cc:27-52). */
+typedef struct sgh_pool_geom {
+  int N, C, H, W;
+  int kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w;
+  int P, Q;
+  int is_max;
+} sgh_pool_geom;
+SGH_API int sgh_pool_geom_init(sgh_pool_geom *g, int N, int C, int H, int W, int kernel_h,
+                               int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+                               int is_max);
+/* GpuPoolingForward (src/model/operation/pooling.cc:187-205).  Max: first maximum in
+ * row-major window order wins (src/model/layer/pooling.cc:189-196); avg: count-exclude-padding
+ * (pooling.cc:70-72, :172). */
+SGH_API int sgh_pool_fwd_f32(const sgh_pool_geom *g, const float *x, float *y, void *stream);
+/* GpuPoolingBackward (src/model/operation/pooling.cc:207-226), same (dy, x, y) arguments.
+ * Max: dy[n,c,p,q] is routed to the first-maximum position of its window (recomputed from x;
+ * y is accepted for signature parity and may be NULL), contributions of overlapping windows
+ * are added in ascending (p, q) order — the order of src/model/layer/pooling.cc:208-233 — so
+ * the result is bit-identical to the CPU loop.  Avg: dy / |clipped window| spread over the window. */
+SGH_API int sgh_pool_bwd_f32(const sgh_pool_geom *g, const float *dy, const float *x,
+                             const float *y, float *dx, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SINGA_HIP_H_ */

@@ -1,0 +1,248 @@
+// Spatial BatchNorm (NCHW fp32): forward-training (to produce the saved mean / inverse std the
+// backward consumes) and backward.
+//
+// Layout: channel c of image n is HW contiguous floats at ((n * C + c) * HW).  A channel's
+// reduction domain is therefore N runs of HW floats.  Both passes split every channel over
+// `S` workgroups (S chosen so the grid fills the chip), each workgroup reducing a contiguous
+// range of the channel's (n, hw) index space with 16-byte loads where HW % 4 == 0.
+// Reductions are a fixed tree (lane partials -> wavefront shuffle -> LDS -> ordered sum over
+// the S partials), so results are run-to-run identical.
+#include "common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+
+struct BnShape {
+  int N, C, HW;
+  int S;          // splits per channel
+  int per_split;  // elements of the (n, hw) space per split (multiple of 4 when HW % 4 == 0)
+};
+
+// Visit elements [lo, hi) of channel c's (n, hw) index space; F(x_value(s), index)
+template <int NT, class F4, class F1>
+__device__ __forceinline__ void channel_range(const BnShape s, int c, int lo, int hi, F4 f4, F1 f1) {
+  const int M = s.N * s.HW;
+  if (hi > M) hi = M;
+  if ((s.HW & 3) == 0) {
+    // lo and per_split are multiples of 4 and a float4 never straddles an image boundary
+    for (int i = lo + threadIdx.x * 4; i < hi; i += NT * 4) {
+      const int n = i / s.HW, r = i - n * s.HW;
+      f4((size_t(n) * s.C + c) * s.HW + r);
+    }
+  } else {
+    for (int i = lo + threadIdx.x; i < hi; i += NT) {
+      const int n = i / s.HW, r = i - n * s.HW;
+      f1((size_t(n) * s.C + c) * s.HW + r);
+    }
+  }
+}
+
+// ---- forward, pass 1: per (c, split) partial sum and sum of squares about a pivot ---------
+// The pivot (the channel's first element) keeps the single-pass variance well conditioned.
+__global__ __launch_bounds__(kBlock) void k_bn_fwd_partial(const float *__restrict__ x, float *__restrict__ part,
+                                                          BnShape s) {
+  __shared__ float red[16];
+  const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
+  const float pivot = x[size_t(c) * s.HW];
+  float a = 0.f, b = 0.f;
+  channel_range<kBlock>(
+      s, c, sp * s.per_split, (sp + 1) * s.per_split,
+      [&](size_t off) {
+        const float4 v = *reinterpret_cast<const float4 *>(x + off);
+        const float d0 = v.x - pivot, d1 = v.y - pivot, d2 = v.z - pivot, d3 = v.w - pivot;
+        a += (d0 + d1) + (d2 + d3);
+        b += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+      },
+      [&](size_t off) {
+        const float d = x[off] - pivot;
+        a += d;
+        b += d * d;
+      });
+  a = sgh_block_sum(a, red);
+  b = sgh_block_sum(b, red);
+  if (threadIdx.x == 0) {
+    part[(size_t(c) * s.S + sp) * 2 + 0] = a;
+    part[(size_t(c) * s.S + sp) * 2 + 1] = b;
+  }
+}
+
+// ---- forward, pass 2: finish statistics (every workgroup redoes the tiny S-sum), normalise --
+__global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const float *__restrict__ x, const float *__restrict__ gamma,
+                                                        const float *__restrict__ beta, const float *__restrict__ part,
+                                                        float *__restrict__ running_mean, float *__restrict__ running_var,
+                                                        float factor, float eps, float *__restrict__ y,
+                                                        float *__restrict__ save_mean, float *__restrict__ save_invstd,
+                                                        BnShape s) {
+  const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
+  const double M = double(s.N) * s.HW;
+  double a = 0, b = 0;
+  for (int i = 0; i < s.S; ++i) {
+    a += part[(size_t(c) * s.S + i) * 2 + 0];
+    b += part[(size_t(c) * s.S + i) * 2 + 1];
+  }
+  const float pivot = x[size_t(c) * s.HW];
+  const double dm = a / M;
+  double var = b / M - dm * dm;
+  if (var < 0) var = 0;
+  const float mean = float(double(pivot) + dm);
+  const float invstd = float(1.0 / sqrt(var + double(eps)));
+  if (sp == 0 && threadIdx.x == 0) {
+    save_mean[c] = mean;
+    save_invstd[c] = invstd;
+    if (running_mean) running_mean[c] = (1.f - factor) * running_mean[c] + factor * mean;
+    if (running_var) {
+      const double unb = M > 1 ? var * M / (M - 1) : var;
+      running_var[c] = (1.f - factor) * running_var[c] + factor * float(unb);
+    }
+  }
+  const float g = gamma[c], be = beta[c];
+  channel_range<kBlock>(
+      s, c, sp * s.per_split, (sp + 1) * s.per_split,
+      [&](size_t off) {
+        const float4 v = *reinterpret_cast<const float4 *>(x + off);
+        float4 r;
+        r.x = g * ((v.x - mean) * invstd) + be;
+        r.y = g * ((v.y - mean) * invstd) + be;
+        r.z = g * ((v.z - mean) * invstd) + be;
+        r.w = g * ((v.w - mean) * invstd) + be;
+        *reinterpret_cast<float4 *>(y + off) = r;
+      },
+      [&](size_t off) { y[off] = g * ((x[off] - mean) * invstd) + be; });
+}
+
+// ---- backward, pass 1: partial sum(dy) and sum(dy * xhat) ---------------------------------
+__global__ __launch_bounds__(kBlock) void k_bn_bwd_partial(const float *__restrict__ dy, const float *__restrict__ x,
+                                                          const float *__restrict__ save_mean,
+                                                          const float *__restrict__ save_invstd,
+                                                          float *__restrict__ part, BnShape s) {
+  __shared__ float red[16];
+  const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
+  const float mean = save_mean[c], invstd = save_invstd[c];
+  float a = 0.f, b = 0.f;
+  channel_range<kBlock>(
+      s, c, sp * s.per_split, (sp + 1) * s.per_split,
+      [&](size_t off) {
+        const float4 d = *reinterpret_cast<const float4 *>(dy + off);
+        const float4 v = *reinterpret_cast<const float4 *>(x + off);
+        a += (d.x + d.y) + (d.z + d.w);
+        b += (d.x * ((v.x - mean) * invstd) + d.y * ((v.y - mean) * invstd)) +
+             (d.z * ((v.z - mean) * invstd) + d.w * ((v.w - mean) * invstd));
+      },
+      [&](size_t off) {
+        const float d = dy[off];
+        a += d;
+        b += d * ((x[off] - mean) * invstd);
+      });
+  a = sgh_block_sum(a, red);
+  b = sgh_block_sum(b, red);
+  if (threadIdx.x == 0) {
+    part[(size_t(c) * s.S + sp) * 2 + 0] = a;
+    part[(size_t(c) * s.S + sp) * 2 + 1] = b;
+  }
+}
+
+// ---- backward, pass 2: dx = k * (dy - (dbeta + xhat * dgamma) / M), k = gamma * invstd -----
+__global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const float *__restrict__ dy, const float *__restrict__ x,
+                                                        const float *__restrict__ gamma,
+                                                        const float *__restrict__ save_mean,
+                                                        const float *__restrict__ save_invstd,
+                                                        const float *__restrict__ part, float *__restrict__ dx,
+                                                        float *__restrict__ dgamma, float *__restrict__ dbeta,
+                                                        BnShape s) {
+  const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
+  double a = 0, b = 0;
+  for (int i = 0; i < s.S; ++i) {
+    a += part[(size_t(c) * s.S + i) * 2 + 0];
+    b += part[(size_t(c) * s.S + i) * 2 + 1];
+  }
+  const float db = float(a), dg = float(b);
+  if (sp == 0 && threadIdx.x == 0) {
+    dbeta[c] = db;
+    dgamma[c] = dg;
+  }
+  const float mean = save_mean[c], invstd = save_invstd[c];
+  const float k = gamma[c] * invstd;
+  const float rM = float(1.0 / (double(s.N) * s.HW));
+  const float c0 = db * rM, c1 = dg * rM;
+  channel_range<kBlock>(
+      s, c, sp * s.per_split, (sp + 1) * s.per_split,
+      [&](size_t off) {
+        const float4 d = *reinterpret_cast<const float4 *>(dy + off);
+        const float4 v = *reinterpret_cast<const float4 *>(x + off);
+        float4 r;
+        r.x = k * (d.x - (c0 + ((v.x - mean) * invstd) * c1));
+        r.y = k * (d.y - (c0 + ((v.y - mean) * invstd) * c1));
+        r.z = k * (d.z - (c0 + ((v.z - mean) * invstd) * c1));
+        r.w = k * (d.w - (c0 + ((v.w - mean) * invstd) * c1));
+        *reinterpret_cast<float4 *>(dx + off) = r;
+      },
+      [&](size_t off) { dx[off] = k * (dy[off] - (c0 + ((x[off] - mean) * invstd) * c1)); });
+}
+
+inline bool shape_ok(int N, int C, int HW) {
+  return N > 0 && C > 0 && HW > 0 && size_t(N) * HW < 0x7fffffffu;
+}
+
+inline BnShape make_shape(int N, int C, int HW) {
+  BnShape s{N, C, HW, 1, 0};
+  const long M = long(N) * HW;
+  // aim at ~8 workgroups per CU in total, at least 2048 elements per workgroup
+  long want = (long(sgh_num_cus()) * 8 + C - 1) / C;
+  long max_by_work = (M + 2047) / 2048;
+  long S = want < max_by_work ? want : max_by_work;
+  if (S < 1) S = 1;
+  if (S > 1024) S = 1024;
+  long per = (M + S - 1) / S;
+  per = (per + 3) & ~3L;
+  S = (M + per - 1) / per;
+  s.S = int(S);
+  s.per_split = int(per);
+  return s;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
+  if (!shape_ok(N, C, HW)) return 0;
+  const BnShape s = make_shape(N, C, HW);
+  return size_t(C) * s.S * 2 * sizeof(float);
+}
+
+int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float *beta, float *running_mean,
+                         float *running_var, float factor, float eps, float *y, float *save_mean, float *save_invstd,
+                         int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  if (!shape_ok(N, C, HW) || !x || !gamma || !beta || !y || !save_mean || !save_invstd) return SGH_EINVAL;
+  const BnShape s = make_shape(N, C, HW);
+  if (!sgh_aligned16(x) || !sgh_aligned16(y)) return SGH_EINVAL;
+  if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
+  float *scratch = static_cast<float *>(workspace);
+  hipLaunchKernelGGL(k_bn_fwd_partial, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, scratch, s);
+  SGH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_bn_fwd_apply, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, gamma, beta, scratch,
+                     running_mean, running_var, factor, eps, y, save_mean, save_invstd, s);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const float *save_mean,
+                   const float *save_invstd, float *dx, float *dgamma, float *dbeta, int N, int C, int HW,
+                   void *workspace, size_t ws_bytes, void *stream) {
+  if (!shape_ok(N, C, HW) || !dy || !x || !gamma || !save_mean || !save_invstd || !dx || !dgamma || !dbeta)
+    return SGH_EINVAL;
+  if (!sgh_aligned16(x) || !sgh_aligned16(dy) || !sgh_aligned16(dx)) return SGH_EINVAL;
+  const BnShape s = make_shape(N, C, HW);
+  if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
+  float *part = static_cast<float *>(workspace);
+  hipLaunchKernelGGL(k_bn_bwd_partial, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, save_mean,
+                     save_invstd, part, s);
+  SGH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_bn_bwd_apply, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, gamma, save_mean,
+                     save_invstd, part, dx, dgamma, dbeta, s);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+}  // extern "C"

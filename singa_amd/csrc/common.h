@@ -1,0 +1,60 @@
+// Shared host/device helpers for the gfx950 kernels of the SINGA backward engine.
+#ifndef SINGA_AMD_CSRC_COMMON_H_
+#define SINGA_AMD_CSRC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "singa_hip.h"
+
+#define SGH_WAVE 64
+
+// Host-side: turn a hipError_t into the ABI's positive error code and leave the function.
+#define SGH_HIP_TRY(expr)                      \
+  do {                                         \
+    hipError_t sgh_e_ = (expr);                \
+    if (sgh_e_ != hipSuccess) return (int)sgh_e_; \
+  } while (0)
+
+// After a kernel launch: report launch-configuration errors without synchronising.
+#define SGH_LAUNCH_CHECK()                     \
+  do {                                         \
+    hipError_t sgh_e_ = hipGetLastError();     \
+    if (sgh_e_ != hipSuccess) return (int)sgh_e_; \
+  } while (0)
+
+static inline hipStream_t sgh_stream_of(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+static inline bool sgh_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Number of compute units of the current device (cached per process; one GPU per process).
+int sgh_num_cus();
+
+// Sum across the 64 lanes of a wavefront; every lane gets the total.
+__device__ __forceinline__ float sgh_wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ float sgh_wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Block-wide sum for blocks of up to 1024 threads; result valid in every thread.
+// `smem` must hold at least 16 floats.
+__device__ __forceinline__ float sgh_block_sum(float v, float *smem) {
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  v = sgh_wave_sum(v);
+  __syncthreads();
+  if (lane == 0) smem[wid] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += smem[i];
+  return t;
+}
+
+#endif  // SINGA_AMD_CSRC_COMMON_H_

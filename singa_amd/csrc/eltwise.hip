@@ -1,0 +1,555 @@
+// Bandwidth-bound tensor_math kernels of the backward path: ReLU backward, softmax-cross-entropy
+// backward, Axpy, EltwiseMult, Add, the fused SGD-momentum update and small row reductions.
+// Each moves its operands through HBM exactly once with 16-byte accesses; arithmetic keeps the
+// rounding sequence of the CPU reference (separate multiply and add, no contraction) so that
+// results are comparable bit for bit where the reference is elementwise.
+#include "common.h"
+
+// contraction is disabled per function where the reference rounds after each op
+#define SGH_NO_CONTRACT _Pragma("clang fp contract(off)")
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;  // float4 vectors in flight per thread per operand
+
+inline int grid_for(size_t nvec) {
+  size_t per_block = size_t(kBlock) * kUnroll;
+  size_t blocks = (nvec + per_block - 1) / per_block;
+  const size_t cap = size_t(sgh_num_cus()) * 16;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return int(blocks);
+}
+
+// ---------------------------------------------------------------------------------------
+// Generic streaming kernels: NIN read-only float streams + NIO read-write streams.
+// F::apply gets references to one element of each.
+// The vector body covers n/4 float4s with a grid-stride loop unrolled kUnroll times; the
+// scalar tail (n % 4) is done by the first threads of block 0.
+// ---------------------------------------------------------------------------------------
+template <class F>
+__global__ __launch_bounds__(kBlock) void k_map2_1(const float *a, const float *b, float *o, size_t n, F f) {
+  // no __restrict__: the in-place forms (y += alpha*x, a += b) alias an input with the output
+  const size_t nvec = n >> 2;
+  const float4 *a4 = reinterpret_cast<const float4 *>(a);
+  const float4 *b4 = reinterpret_cast<const float4 *>(b);
+  float4 *o4 = reinterpret_cast<float4 *>(o);
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+  for (; i + (kUnroll - 1) * stride < nvec; i += kUnroll * stride) {
+    float4 va[kUnroll], vb[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      va[u] = a4[i + u * stride];
+      vb[u] = b4[i + u * stride];
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      float4 r;
+      r.x = f(va[u].x, vb[u].x);
+      r.y = f(va[u].y, vb[u].y);
+      r.z = f(va[u].z, vb[u].z);
+      r.w = f(va[u].w, vb[u].w);
+      o4[i + u * stride] = r;
+    }
+  }
+  for (; i < nvec; i += stride) {
+    float4 va = a4[i], vb = b4[i], r;
+    r.x = f(va.x, vb.x);
+    r.y = f(va.y, vb.y);
+    r.z = f(va.z, vb.z);
+    r.w = f(va.w, vb.w);
+    o4[i] = r;
+  }
+  if (blockIdx.x == 0) {
+    const size_t t = (nvec << 2) + threadIdx.x;
+    if (t < n) o[t] = f(a[t], b[t]);
+  }
+}
+
+// scalar fallback for pointers that are not 16-byte aligned
+template <class F>
+__global__ __launch_bounds__(kBlock) void k_map2_1_scalar(const float *a, const float *b, float *o, size_t n, F f) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) o[i] = f(a[i], b[i]);
+}
+
+template <class F>
+int launch_map2(const float *a, const float *b, float *o, size_t n, F f, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!a || !b || !o) return SGH_EINVAL;
+  if (sgh_aligned16(a) && sgh_aligned16(b) && sgh_aligned16(o)) {
+    hipLaunchKernelGGL(k_map2_1<F>, dim3(grid_for(n >> 2)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o, n, f);
+  } else {
+    hipLaunchKernelGGL(k_map2_1_scalar<F>, dim3(grid_for(n)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o, n, f);
+  }
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+struct ReluBwd {
+  __device__ __forceinline__ float operator()(float dy, float x) const { return x > 0.f ? dy : 0.f; }
+};
+struct ReluFwd {  // second operand unused
+  __device__ __forceinline__ float operator()(float x, float) const { return x >= 0.f ? x : 0.f; }
+};
+struct AddOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+struct MulOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a * b; }
+};
+struct AxpyOp {  // (x, y) -> y + alpha * x, two roundings
+  float alpha;
+  __device__ __forceinline__ float operator()(float x, float y) const {
+    SGH_NO_CONTRACT
+    float t = alpha * x;
+    return y + t;
+  }
+};
+struct AxpyDevOp {
+  const float *alpha;
+  __device__ __forceinline__ float operator()(float x, float y) const {
+    SGH_NO_CONTRACT
+    float t = __ldg(alpha) * x;
+    return y + t;
+  }
+};
+struct MulScalarDevOp {  // second stream is ignored (aliased to the first by the launcher)
+  const float *s;
+  __device__ __forceinline__ float operator()(float a, float) const { return a * __ldg(s); }
+};
+
+// ---------------------------------------------------------------------------------------
+// unary (one read stream) variants for ReLU forward / scalar multiply / fill
+// ---------------------------------------------------------------------------------------
+template <class F>
+__global__ __launch_bounds__(kBlock) void k_map1_1(const float *a, float *o, size_t n, F f, int vec) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+  if (vec) {
+    const size_t nvec = n >> 2;
+    const float4 *a4 = reinterpret_cast<const float4 *>(a);
+    float4 *o4 = reinterpret_cast<float4 *>(o);
+    for (; i < nvec; i += stride) {
+      float4 v = a4[i], r;
+      r.x = f(v.x, 0.f);
+      r.y = f(v.y, 0.f);
+      r.z = f(v.z, 0.f);
+      r.w = f(v.w, 0.f);
+      o4[i] = r;
+    }
+    if (blockIdx.x == 0) {
+      const size_t t = (nvec << 2) + threadIdx.x;
+      if (t < n) o[t] = f(a[t], 0.f);
+    }
+  } else {
+    for (; i < n; i += stride) o[i] = f(a[i], 0.f);
+  }
+}
+
+template <class F>
+int launch_map1(const float *a, float *o, size_t n, F f, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!a || !o) return SGH_EINVAL;
+  const int vec = sgh_aligned16(a) && sgh_aligned16(o);
+  hipLaunchKernelGGL(k_map1_1<F>, dim3(grid_for(vec ? (n >> 2) : n)), dim3(kBlock), 0, sgh_stream_of(stream), a, o, n,
+                     f, vec);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+__global__ __launch_bounds__(kBlock) void k_fill(float *o, float v, size_t n) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) o[i] = v;
+}
+
+// ---------------------------------------------------------------------------------------
+// Fused SGD-momentum: streams p, g, v in; p, v out (5 * 4 bytes per parameter element).
+// ---------------------------------------------------------------------------------------
+struct SgdHyper {
+  float lr, mu, damp, wd;
+};
+
+__device__ __forceinline__ void sgd_one(float &p, float g, float &v, const SgdHyper h, int nesterov, bool has_v) {
+  SGH_NO_CONTRACT
+  const float one_minus_damp = 1.0f - h.damp;
+  const float minus_lr = 0.0f - h.lr;
+  if (h.wd != 0.f) {
+    float t = h.wd * p;
+    g = g + t;
+  }
+  if (has_v) {
+    float vi = v * h.mu;
+    float t = one_minus_damp * g;
+    vi = vi + t;
+    v = vi;
+    if (nesterov) {
+      float t2 = h.mu * vi;
+      g = g + t2;
+    } else {
+      g = vi;
+    }
+  }
+  float t = minus_lr * g;
+  p = p + t;
+}
+
+template <bool DEV_HYPER>
+__global__ __launch_bounds__(kBlock) void k_sgd(float *__restrict__ p, const float *__restrict__ g,
+                                               float *__restrict__ v, size_t n, SgdHyper hh,
+                                               const float *__restrict__ hyper_dev, int nesterov, int vec) {
+  SgdHyper h = hh;
+  if (DEV_HYPER) {
+    h.lr = __ldg(hyper_dev + 0);
+    h.mu = __ldg(hyper_dev + 1);
+    h.damp = __ldg(hyper_dev + 2);
+    h.wd = __ldg(hyper_dev + 3);
+  }
+  const bool has_v = (h.mu != 0.f) && v != nullptr;
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+  if (vec) {
+    const size_t nvec = n >> 2;
+    float4 *p4 = reinterpret_cast<float4 *>(p);
+    const float4 *g4 = reinterpret_cast<const float4 *>(g);
+    float4 *v4 = reinterpret_cast<float4 *>(v);
+    for (; i < nvec; i += stride) {
+      float4 pp = p4[i], gg = g4[i], vv = has_v ? v4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      sgd_one(pp.x, gg.x, vv.x, h, nesterov, has_v);
+      sgd_one(pp.y, gg.y, vv.y, h, nesterov, has_v);
+      sgd_one(pp.z, gg.z, vv.z, h, nesterov, has_v);
+      sgd_one(pp.w, gg.w, vv.w, h, nesterov, has_v);
+      p4[i] = pp;
+      if (has_v) v4[i] = vv;
+    }
+    if (blockIdx.x == 0) {
+      const size_t t = (nvec << 2) + threadIdx.x;
+      if (t < n) {
+        float pp = p[t], vv = has_v ? v[t] : 0.f;
+        sgd_one(pp, g[t], vv, h, nesterov, has_v);
+        p[t] = pp;
+        if (has_v) v[t] = vv;
+      }
+    }
+  } else {
+    for (; i < n; i += stride) {
+      float pp = p[i], vv = has_v ? v[i] : 0.f;
+      sgd_one(pp, g[i], vv, h, nesterov, has_v);
+      p[i] = pp;
+      if (has_v) v[i] = vv;
+    }
+  }
+}
+
+// Multi-tensor variant: block b walks the concatenation of all items in chunks of
+// kChunk elements; a chunk never crosses an item boundary (the table is scanned linearly,
+// 62 entries for ResNet-18).
+constexpr int kChunk = kBlock * 4 * 2;  // 2048 elements per block-iteration
+
+__global__ __launch_bounds__(kBlock) void k_sgd_multi(const sgh_sgd_item *__restrict__ table, int count, SgdHyper h,
+                                                     int nesterov) {
+  const bool use_v = h.mu != 0.f;
+  // chunk index space: sum over items of ceil(n / kChunk)
+  size_t chunk = blockIdx.x;
+  for (;;) {
+    // locate the item that owns this chunk
+    size_t c = chunk;
+    int it = 0;
+    for (; it < count; ++it) {
+      const size_t nc = (table[it].n + kChunk - 1) / kChunk;
+      if (c < nc) break;
+      c -= nc;
+    }
+    if (it >= count) return;
+    float *p = table[it].p;
+    const float *g = table[it].g;
+    float *v = table[it].v;
+    const size_t n = table[it].n;
+    const bool has_v = use_v && v != nullptr;
+    const size_t base = c * kChunk;
+    const size_t end = base + kChunk < n ? base + kChunk : n;
+    const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) |
+                       reinterpret_cast<uintptr_t>(has_v ? v : p)) & 15u) == 0;
+    if (vec) {
+      for (size_t e = base + size_t(threadIdx.x) * 4; e < end; e += size_t(kBlock) * 4) {
+        if (e + 4 <= end) {
+          float4 pp = *reinterpret_cast<float4 *>(p + e), gg = *reinterpret_cast<const float4 *>(g + e);
+          float4 vv = has_v ? *reinterpret_cast<float4 *>(v + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+          sgd_one(pp.x, gg.x, vv.x, h, nesterov, has_v);
+          sgd_one(pp.y, gg.y, vv.y, h, nesterov, has_v);
+          sgd_one(pp.z, gg.z, vv.z, h, nesterov, has_v);
+          sgd_one(pp.w, gg.w, vv.w, h, nesterov, has_v);
+          *reinterpret_cast<float4 *>(p + e) = pp;
+          if (has_v) *reinterpret_cast<float4 *>(v + e) = vv;
+        } else {
+          for (size_t t = e; t < end; ++t) {
+            float pp = p[t], vv = has_v ? v[t] : 0.f;
+            sgd_one(pp, g[t], vv, h, nesterov, has_v);
+            p[t] = pp;
+            if (has_v) v[t] = vv;
+          }
+        }
+      }
+    } else {
+      for (size_t t = base + threadIdx.x; t < end; t += kBlock) {
+        float pp = p[t], vv = has_v ? v[t] : 0.f;
+        sgd_one(pp, g[t], vv, h, nesterov, has_v);
+        p[t] = pp;
+        if (has_v) v[t] = vv;
+      }
+    }
+    chunk += gridDim.x;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Softmax cross-entropy: one 256-thread block per sample row.
+// ---------------------------------------------------------------------------------------
+__device__ int g_label_errors = 0;
+
+__global__ __launch_bounds__(kBlock) void k_softmax_ce_bwd(const float *__restrict__ p, const int32_t *__restrict__ t,
+                                                          float *__restrict__ grad, size_t dim, int int_target,
+                                                          float scale) {
+  __shared__ float red[16];
+  const size_t row = blockIdx.x;
+  const float *pr = p + row * dim;
+  float *gr = grad + row * dim;
+  if (int_target) {
+    const int label = t[row];
+    const bool ok = label >= 0 && size_t(label) < dim;
+    if (!ok && threadIdx.x == 0) atomicAdd(&g_label_errors, 1);
+    for (size_t j = threadIdx.x; j < dim; j += kBlock) {
+      float v = pr[j];
+      if (ok && j == size_t(label)) v = v - 1.0f;
+      gr[j] = v * scale;
+    }
+  } else {
+    const int32_t *tr = t + row * dim;
+    float s = 0.f;
+    for (size_t j = threadIdx.x; j < dim; j += kBlock) s += float(tr[j]);
+    s = sgh_block_sum(s, red);
+    for (size_t j = threadIdx.x; j < dim; j += kBlock) {
+      float v = pr[j] - float(tr[j]) / s;
+      gr[j] = v * scale;
+    }
+  }
+}
+
+// Row softmax with the numerically safe max subtraction (row max, not the CPU path's
+// zero-seeded max: the two agree whenever a row has a non-negative entry and differ only by
+// rounding otherwise).
+__global__ __launch_bounds__(kBlock) void k_softmax_fwd(const float *__restrict__ x, float *__restrict__ p, size_t dim) {
+  __shared__ float red[16];
+  const size_t row = blockIdx.x;
+  const float *xr = x + row * dim;
+  float *pr = p + row * dim;
+  float m = -3.402823466e38f;
+  for (size_t j = threadIdx.x; j < dim; j += kBlock) m = fmaxf(m, xr[j]);
+  m = sgh_wave_max(m);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  m = red[0];
+  for (int i = 1; i < kBlock / 64; ++i) m = fmaxf(m, red[i]);
+  float s = 0.f;
+  for (size_t j = threadIdx.x; j < dim; j += kBlock) {
+    float e = expf(xr[j] - m);
+    pr[j] = e;
+    s += e;
+  }
+  s = sgh_block_sum(s, red);
+  for (size_t j = threadIdx.x; j < dim; j += kBlock) pr[j] = pr[j] / s;
+}
+
+__global__ __launch_bounds__(kBlock) void k_ce_fwd(const float *__restrict__ p, const int32_t *__restrict__ t,
+                                                  float *__restrict__ loss, size_t dim, int int_target) {
+  __shared__ float red[16];
+  const size_t row = blockIdx.x;
+  const float *pr = p + row * dim;
+  if (int_target) {
+    if (threadIdx.x == 0) {
+      const int label = t[row];
+      if (label >= 0 && size_t(label) < dim) {
+        loss[row] = -logf(fmaxf(pr[label], 1.17549435e-38f));
+      } else {
+        atomicAdd(&g_label_errors, 1);
+        loss[row] = 0.f;
+      }
+    }
+  } else {
+    const int32_t *tr = t + row * dim;
+    float s = 0.f;
+    for (size_t j = threadIdx.x; j < dim; j += kBlock) s += float(tr[j]);
+    s = sgh_block_sum(s, red);
+    float l = 0.f;
+    for (size_t j = threadIdx.x; j < dim; j += kBlock)
+      l -= float(tr[j]) / s * logf(fmaxf(pr[j], 1.17549435e-38f));
+    l = sgh_block_sum(l, red);
+    if (threadIdx.x == 0) loss[row] = l;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Row reductions for Linear's bias:  out[j] = sum_i m[i][j]   and   m[i][j] += v[j]
+// ---------------------------------------------------------------------------------------
+// One thread per column, rows summed in ascending order (the order of the reference GEMV).
+__global__ __launch_bounds__(kBlock) void k_sum_rows(const float *__restrict__ m, float *__restrict__ out, int rows,
+                                                    int cols) {
+  const int j = blockIdx.x * kBlock + threadIdx.x;
+  if (j >= cols) return;
+  float s = 0.f;
+  for (int i = 0; i < rows; ++i) s += m[size_t(i) * cols + j];
+  out[j] = s;
+}
+
+__global__ __launch_bounds__(kBlock) void k_add_row(const float *__restrict__ v, float *__restrict__ m, size_t total,
+                                                   int cols) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) m[i] += v[i % cols];
+}
+
+}  // namespace
+
+extern "C" {
+
+int sgh_relu_bwd_f32(const float *dy, const float *x, float *dx, size_t n, void *stream) {
+  return launch_map2(dy, x, dx, n, ReluBwd{}, stream);
+}
+
+int sgh_relu_fwd_f32(const float *x, float *y, size_t n, void *stream) {
+  return launch_map1(x, y, n, ReluFwd{}, stream);
+}
+
+int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
+  return launch_map2(a, b, out, n, AddOp{}, stream);
+}
+
+int sgh_eltwise_mult_f32(const float *a, const float *b, int b_is_scalar, float *out, size_t n, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!a || !b || !out) return SGH_EINVAL;
+  if (b_is_scalar) return launch_map1(a, out, n, MulScalarDevOp{b}, stream);
+  return launch_map2(a, b, out, n, MulOp{}, stream);
+}
+
+int sgh_axpy_f32(float alpha, const float *x, float *y, size_t n, void *stream) {
+  return launch_map2(x, y, y, n, AxpyOp{alpha}, stream);
+}
+
+int sgh_axpy_devalpha_f32(const float *alpha_dev, const float *x, float *y, size_t n, void *stream) {
+  if (n != 0 && !alpha_dev) return SGH_EINVAL;
+  return launch_map2(x, y, y, n, AxpyDevOp{alpha_dev}, stream);
+}
+
+int sgh_memset_f32(float *dst, float value, size_t n, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!dst) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_fill, dim3(grid_for(n)), dim3(kBlock), 0, sgh_stream_of(stream), dst, value, n);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+static int sgd_launch(float *p, const float *g, float *v, size_t n, SgdHyper h, const float *hyper_dev, int nesterov,
+                      bool host_mu_nonzero_needs_v, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!p || !g) return SGH_EINVAL;
+  if (host_mu_nonzero_needs_v && !v) return SGH_EINVAL;
+  const int vec = sgh_aligned16(p) && sgh_aligned16(g) && (v == nullptr || sgh_aligned16(v));
+  const int grid = grid_for(vec ? (n >> 2) : n);
+  if (hyper_dev)
+    hipLaunchKernelGGL(k_sgd<true>, dim3(grid), dim3(kBlock), 0, sgh_stream_of(stream), p, g, v, n, h, hyper_dev,
+                       nesterov, vec);
+  else
+    hipLaunchKernelGGL(k_sgd<false>, dim3(grid), dim3(kBlock), 0, sgh_stream_of(stream), p, g, v, n, h, hyper_dev,
+                       nesterov, vec);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_sgd_momentum_f32(float *p, const float *g, float *v, size_t n, float lr, float mu, float damp, float wd,
+                         int nesterov, void *stream) {
+  return sgd_launch(p, g, v, n, SgdHyper{lr, mu, damp, wd}, nullptr, nesterov, mu != 0.f, stream);
+}
+
+int sgh_sgd_momentum_devhyper_f32(float *p, const float *g, float *v, size_t n, const float *hyper_dev, int nesterov,
+                                  void *stream) {
+  if (!hyper_dev) return SGH_EINVAL;
+  // mu lives on the device: a NULL v is only legal if mu turns out to be 0, which the kernel checks
+  return sgd_launch(p, g, v, n, SgdHyper{0, 0, 0, 0}, hyper_dev, nesterov, false, stream);
+}
+
+int sgh_sgd_momentum_multi_f32(const sgh_sgd_item *table_dev, int count, size_t total_n, float lr, float mu, float damp,
+                               float wd, int nesterov, void *stream) {
+  if (count == 0 || total_n == 0) return SGH_OK;
+  if (!table_dev || count < 0) return SGH_EINVAL;
+  size_t chunks = total_n / kChunk + size_t(count);  // upper bound on sum of per-item chunk counts
+  const size_t cap = size_t(sgh_num_cus()) * 8;
+  if (chunks > cap) chunks = cap;
+  hipLaunchKernelGGL(k_sgd_multi, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count,
+                     SgdHyper{lr, mu, damp, wd}, nesterov);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_softmax_ce_bwd_f32(const float *p, const int32_t *t, float *grad, size_t batch, size_t dim, int int_target,
+                           float scale, void *stream) {
+  if (batch == 0 || dim == 0) return SGH_OK;
+  if (!p || !t || !grad) return SGH_EINVAL;
+  if (batch > 0x7fffffffu) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_softmax_ce_bwd, dim3((unsigned)batch), dim3(kBlock), 0, sgh_stream_of(stream), p, t, grad, dim,
+                     int_target, scale);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_softmax_ce_label_errors(void *stream, int *count) {
+  if (!count) return SGH_EINVAL;
+  SGH_HIP_TRY(hipStreamSynchronize(sgh_stream_of(stream)));
+  int v = 0;
+  SGH_HIP_TRY(hipMemcpyFromSymbol(&v, HIP_SYMBOL(g_label_errors), sizeof(int), 0, hipMemcpyDeviceToHost));
+  const int zero = 0;
+  SGH_HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(g_label_errors), &zero, sizeof(int), 0, hipMemcpyHostToDevice));
+  *count = v;
+  return SGH_OK;
+}
+
+int sgh_softmax_fwd_f32(const float *x, float *p, size_t batch, size_t dim, void *stream) {
+  if (batch == 0 || dim == 0) return SGH_OK;
+  if (!x || !p || batch > 0x7fffffffu) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_softmax_fwd, dim3((unsigned)batch), dim3(kBlock), 0, sgh_stream_of(stream), x, p, dim);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_cross_entropy_fwd_f32(const float *p, const int32_t *t, float *loss, size_t batch, size_t dim, int int_target,
+                              void *stream) {
+  if (batch == 0 || dim == 0) return SGH_OK;
+  if (!p || !t || !loss || batch > 0x7fffffffu) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_ce_fwd, dim3((unsigned)batch), dim3(kBlock), 0, sgh_stream_of(stream), p, t, loss, dim,
+                     int_target);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_sum_rows_f32(const float *m, float *out, int rows, int cols, void *stream) {
+  if (rows < 0 || cols < 0) return SGH_EINVAL;
+  if (cols == 0) return SGH_OK;
+  if (!out || (rows > 0 && !m)) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_sum_rows, dim3((cols + kBlock - 1) / kBlock), dim3(kBlock), 0, sgh_stream_of(stream), m, out,
+                     rows, cols);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_add_row_f32(const float *v, float *m, int rows, int cols, void *stream) {
+  if (rows < 0 || cols < 0) return SGH_EINVAL;
+  const size_t total = size_t(rows) * cols;
+  if (total == 0) return SGH_OK;
+  if (!v || !m) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_add_row, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), v, m, total, cols);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+}  // extern "C"

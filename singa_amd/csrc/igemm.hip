@@ -1,0 +1,618 @@
+// fp32 MFMA GEMM core and the implicit-GEMM convolution passes built on it
+// (conv forward, dgrad, wgrad) plus the Linear-layer GEMM.
+//
+// One workgroup = 256 threads = 4 wavefronts in a 2 x 2 grid; the workgroup computes a
+// BM x BN tile of C, each wavefront a (BM/2) x (BN/2) sub-tile out of 32x32x2 fp32 MFMAs
+// (v_mfma_f32_32x32x2_f32: lane l feeds A[l%32][l/32] and B[l/32][l%32]; its 16 accumulators
+// hold C[8*(v/4) + 4*(l/32) + v%4][l%32]).
+//
+// Operands are staged through LDS in [k][m] / [k][n] order with a row pitch of (tile + 4)
+// floats: the MFMA operand reads (32 consecutive m for two consecutive k) and both kinds of
+// staging writes (threads consecutive in m, or consecutive in k) then touch every bank at most
+// twice per 64-lane access, which is the minimum.  Global loads for chunk i+1 are issued before
+// the MFMAs of chunk i and written to the other LDS buffer afterwards (one barrier per chunk).
+//
+// A "problem" supplies two loaders (how to fetch element (row, k) of A and (k, col) of B,
+// zero outside the valid range) and an epilogue (where C[m][n] goes).  The convolution loaders
+// perform im2col on the fly: no column matrix is ever materialised.
+#include "common.h"
+
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int NT = 256;
+constexpr int BK = 16;
+
+// ------------------------------------------------------------------------------------------
+// Thread -> staged element mapping.
+//   K-contiguous operand (consecutive k are consecutive in memory):
+//       kk = t % BK, row = t / BK + e * (NT / BK)
+//   M/N-contiguous operand (consecutive rows are consecutive in memory):
+//       row = t % ROWS, kk = t / ROWS + e * (NT / ROWS)
+// e = 0 .. ROWS * BK / NT - 1.
+// ------------------------------------------------------------------------------------------
+template <int ROWS, bool KCONTIG>
+struct StageMap {
+  static constexpr int E = ROWS * BK / NT;
+  static constexpr int ROW_STEP = KCONTIG ? NT / BK : 0;
+  static constexpr int K_STEP = KCONTIG ? 0 : NT / ROWS;
+  __device__ static __forceinline__ int row0(int t) { return KCONTIG ? t / BK : t % ROWS; }
+  __device__ static __forceinline__ int kk0(int t) { return KCONTIG ? t % BK : t / ROWS; }
+};
+
+template <int ROWS, bool KCONTIG>
+__device__ __forceinline__ void stage_store(float *lds /* [BK][ROWS + 4] */, const float (&r)[ROWS * BK / NT], int t) {
+  using M = StageMap<ROWS, KCONTIG>;
+  const int row0 = M::row0(t), kk0 = M::kk0(t);
+#pragma unroll
+  for (int e = 0; e < M::E; ++e) lds[(kk0 + e * M::K_STEP) * (ROWS + 4) + row0 + e * M::ROW_STEP] = r[e];
+}
+
+// ------------------------------------------------------------------------------------------
+// Loader 1: dense strided matrix.  element(row, k) = base[row * rs + k * ks]; whichever of
+// rs / ks is 1 decides KCONTIG.
+// ------------------------------------------------------------------------------------------
+template <int ROWS, bool KCONTIG>
+struct DenseLoader {
+  const float *base;
+  long rs, ks;
+  int rows, K;
+  __device__ __forceinline__ void init(int, int) {}
+  __device__ __forceinline__ void load(int tile_row0, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
+    using M = StageMap<ROWS, KCONTIG>;
+    const int row0 = tile_row0 + M::row0(t), kk0 = k0 + M::kk0(t);
+#pragma unroll
+    for (int e = 0; e < M::E; ++e) {
+      const int row = row0 + e * M::ROW_STEP, k = kk0 + e * M::K_STEP;
+      r[e] = (row < rows && k < k_end) ? base[row * rs + k * ks] : 0.f;
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------------------
+// Convolution geometry shared by the gather loaders.
+// ------------------------------------------------------------------------------------------
+struct ConvG {
+  int N, C, H, W, K, R, S, sh, sw, ph, pw, P, Q;
+};
+
+// ------------------------------------------------------------------------------------------
+// Loader 2: pixel gather for forward and dgrad (N-contiguous: a thread owns ONE pixel column of
+// the tile for the whole kernel and walks k).
+//   k index = tap * CP + ch, tap = r * S + s, CP = channel count rounded up to BK, so one
+//   BK-chunk has a single tap and the tap's validity test is done once per chunk per thread.
+//   FWD:   column = (n, p, q) of y;  source = x[n][ch][p*sh - ph + r][q*sw - pw + s]
+//   DGRAD: column = (n, h, w) of dx; source = dy[n][ch][(h + ph - r)/sh][(w + pw - s)/sw]
+//          (only where both divisions are exact and in range)
+// ------------------------------------------------------------------------------------------
+template <int ROWS, bool DGRAD>
+struct PixelGatherLoader {
+  const float *src;
+  ConvG g;
+  int CP;        // padded channel count of the k index
+  int src_ch;    // channels of the source tensor (C for fwd, K for dgrad)
+  int src_h, src_w;
+  int cols;      // valid columns (N * P * Q or N * H * W)
+  // per-thread state
+  long img_base;  // offset of image n in src
+  int a, b;       // (p, q) for fwd, (h, w) for dgrad
+  bool col_ok;
+
+  __device__ __forceinline__ void init(int tile_col0, int t) {
+    using M = StageMap<ROWS, false>;
+    const int col = tile_col0 + M::row0(t);
+    col_ok = col < cols;
+    const int plane = DGRAD ? g.H * g.W : g.P * g.Q;
+    const int wdt = DGRAD ? g.W : g.Q;
+    const int n = col / plane, rem = col - n * plane;
+    a = rem / wdt;
+    b = rem - a * wdt;
+    img_base = long(n) * src_ch * src_h * src_w;
+  }
+
+  __device__ __forceinline__ void load(int, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
+    using M = StageMap<ROWS, false>;
+    (void)k_end;
+    const int tap = k0 / CP, ch0 = k0 - tap * CP + M::kk0(t);
+    const int fr = tap / g.S, fs = tap - fr * g.S;
+    int y, x;
+    bool ok = col_ok;
+    if (DGRAD) {
+      const int hp = a + g.ph - fr, wp = b + g.pw - fs;
+      y = hp / g.sh;
+      x = wp / g.sw;
+      ok = ok && hp >= 0 && wp >= 0 && y * g.sh == hp && x * g.sw == wp && y < g.P && x < g.Q;
+    } else {
+      y = a * g.sh - g.ph + fr;
+      x = b * g.sw - g.pw + fs;
+      ok = ok && y >= 0 && y < g.H && x >= 0 && x < g.W;
+    }
+    const long plane = long(src_h) * src_w;
+    const float *p = src + img_base + long(y) * src_w + x;
+#pragma unroll
+    for (int e = 0; e < M::E; ++e) {
+      const int ch = ch0 + e * M::K_STEP;
+      r[e] = (ok && ch < src_ch) ? p[ch * plane] : 0.f;
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------------------
+// Loaders 3 and 4: wgrad.  The reduction index g = n * PQ + p * Q + q is contiguous in memory
+// for both operands, so both are K-contiguous.
+//   A(m = k_out, g) = dy[n][m][pq]
+//   B(g, j = (c, r, s) in KCRS order) = x[n][c][p*sh - ph + r][q*sw - pw + s]
+// ------------------------------------------------------------------------------------------
+template <int ROWS>
+struct WgradDyLoader {
+  const float *dy;
+  int K, PQ, G;  // G = N * PQ
+  __device__ __forceinline__ void init(int, int) {}
+  __device__ __forceinline__ void load(int tile_row0, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
+    using M = StageMap<ROWS, true>;
+    const int gi = k0 + M::kk0(t);
+    const bool ok = gi < k_end;
+    const int n = gi / PQ, pq = gi - n * PQ;
+    const float *p = dy + long(n) * K * PQ + pq;
+    const int row0 = tile_row0 + M::row0(t);
+#pragma unroll
+    for (int e = 0; e < M::E; ++e) {
+      const int row = row0 + e * M::ROW_STEP;
+      r[e] = (ok && row < K) ? p[long(row) * PQ] : 0.f;
+    }
+  }
+};
+
+template <int ROWS>
+struct WgradXLoader {
+  const float *x;
+  ConvG g;
+  int CRS;
+  // per-thread, per staged row: offset of (c, r - ph, s - pw) inside an image, and the tap shifts
+  int off[ROWS * BK / NT];
+  short dr[ROWS * BK / NT], ds[ROWS * BK / NT];
+  __device__ __forceinline__ void init(int tile_col0, int t) {
+    using M = StageMap<ROWS, true>;
+    const int RS = g.R * g.S;
+#pragma unroll
+    for (int e = 0; e < M::E; ++e) {
+      const int j = tile_col0 + M::row0(t) + e * M::ROW_STEP;
+      if (j < CRS) {
+        const int c = j / RS, rs = j - c * RS, fr = rs / g.S, fs = rs - fr * g.S;
+        dr[e] = short(fr - g.ph);
+        ds[e] = short(fs - g.pw);
+        off[e] = (c * g.H + (fr - g.ph)) * g.W + (fs - g.pw);
+      } else {
+        dr[e] = short(-30000);  // fails the row test below for every p
+        ds[e] = 0;
+        off[e] = 0;
+      }
+    }
+  }
+  __device__ __forceinline__ void load(int, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
+    using M = StageMap<ROWS, true>;
+    const int gi = k0 + M::kk0(t);
+    const bool ok = gi < k_end;
+    const int PQ = g.P * g.Q;
+    const int n = gi / PQ, pq = gi - n * PQ;
+    const int p = pq / g.Q, q = pq - p * g.Q;
+    const int h0 = p * g.sh, w0 = q * g.sw;
+    const float *base = x + long(n) * g.C * g.H * g.W + h0 * g.W + w0;
+#pragma unroll
+    for (int e = 0; e < M::E; ++e) {
+      const int h = h0 + dr[e], w = w0 + ds[e];
+      const bool v = ok && h >= 0 && h < g.H && w >= 0 && w < g.W;
+      r[e] = v ? base[off[e]] : 0.f;
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------------------
+// Epilogues
+// ------------------------------------------------------------------------------------------
+struct DenseStore {  // C[m * ldc + n] = alpha * acc + beta * C
+  float *C;
+  long ldc;
+  int M, N;
+  float alpha, beta;
+  __device__ __forceinline__ void operator()(int m, int n, float v) const {
+    if (m < M && n < N) {
+      float *p = C + m * ldc + n;
+      *p = beta == 0.f ? alpha * v : alpha * v + beta * *p;
+    }
+  }
+};
+
+struct NchwStore {  // out[(img * CH + m) * plane + rem] (+ bias[m]), column = img * plane + rem
+  float *out;
+  const float *bias;
+  int CH, plane, cols;
+  __device__ __forceinline__ void operator()(int m, int col, float v) const {
+    if (m < CH && col < cols) {
+      const int img = col / plane, rem = col - img * plane;
+      out[(long(img) * CH + m) * plane + rem] = bias ? v + bias[m] : v;
+    }
+  }
+};
+
+struct SplitStore {  // partial[split][m * N + n]
+  float *part;
+  int M, N;
+  __device__ __forceinline__ void operator()(int m, int n, float v) const {
+    if (m < M && n < N) part[long(blockIdx.z) * M * N + long(m) * N + n] = v;
+  }
+};
+
+// ------------------------------------------------------------------------------------------
+// The kernel.  grid = (M tiles, N tiles, K splits); split z covers chunks
+// [z * chunks_per_split, (z + 1) * chunks_per_split) of the reduction.
+// ------------------------------------------------------------------------------------------
+template <int BM, int BN, class LA, class LB, class ST, bool A_KCONTIG, bool B_KCONTIG>
+__global__ __launch_bounds__(NT) void k_igemm(LA la, LB lb, ST st, int Ktotal, int chunks_per_split) {
+  constexpr int PA = BM + 4, PB = BN + 4;
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  constexpr int EA = BM * BK / NT, EB = BN * BK / NT;
+  __shared__ float As[2][BK * PA];
+  __shared__ float Bs[2][BK * PB];
+
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const int k_begin = blockIdx.z * chunks_per_split * BK;
+  int k_end = k_begin + chunks_per_split * BK;
+  if (k_end > Ktotal) k_end = Ktotal;
+
+  la.init(m0, t);
+  lb.init(n0, t);
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  float ra[EA], rb[EB];
+  if (k_begin < k_end) {
+    la.load(m0, k_begin, k_end, t, ra);
+    lb.load(n0, k_begin, k_end, t, rb);
+    stage_store<BM, A_KCONTIG>(As[0], ra, t);
+    stage_store<BN, B_KCONTIG>(Bs[0], rb, t);
+  }
+  __syncthreads();
+
+  int cur = 0;
+  for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+    const bool more = k0 + BK < k_end;
+    if (more) {
+      la.load(m0, k0 + BK, k_end, t, ra);
+      lb.load(n0, k0 + BK, k_end, t, rb);
+    }
+    const float *as = As[cur] + (lane >> 5) * PA + wm * WM + (lane & 31);
+    const float *bs = Bs[cur] + (lane >> 5) * PB + wn * WN + (lane & 31);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      float a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = as[kk * PA + i * 32];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = bs[kk * PB + j * 32];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      stage_store<BM, A_KCONTIG>(As[cur ^ 1], ra, t);
+      stage_store<BN, B_KCONTIG>(Bs[cur ^ 1], rb, t);
+    }
+    __syncthreads();
+    cur ^= 1;
+  }
+
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * WM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        const int n = n0 + wn * WN + j * 32 + (lane & 31);
+        st(m, n, acc[i][j][v]);
+      }
+}
+
+// Ordered reduction of split-K partials: out[i] = sum_s part[s][i], s ascending.
+__global__ __launch_bounds__(NT) void k_split_reduce(const float *__restrict__ part, float *__restrict__ out, long n,
+                                                    int splits) {
+  const long stride = long(gridDim.x) * NT;
+  for (long i = long(blockIdx.x) * NT + threadIdx.x; i < n; i += stride) {
+    float s = 0.f;
+    for (int z = 0; z < splits; ++z) s += part[z * n + i];
+    out[i] = s;
+  }
+}
+
+// Weight re-layout for the pixel-gather passes:  W[K][C][R][S]  ->  Wt[tap][chp][m]
+//   forward: ch = c (padded to CP), m = k   -> Wt[(tap * CP + c) * K + k]
+//   dgrad:   ch = k (padded to KP), m = c   -> Wt[(tap * KP + k) * C + c]
+__global__ __launch_bounds__(NT) void k_weight_relayout(const float *__restrict__ W, float *__restrict__ Wt, int K, int C,
+                                                       int RS, int CHP, int dgrad) {
+  const long total = long(RS) * CHP * (dgrad ? C : K);
+  const long stride = long(gridDim.x) * NT;
+  const int Mdim = dgrad ? C : K;
+  for (long i = long(blockIdx.x) * NT + threadIdx.x; i < total; i += stride) {
+    const int m = int(i % Mdim);
+    const long rest = i / Mdim;
+    const int ch = int(rest % CHP), tap = int(rest / CHP);
+    float v = 0.f;
+    if (dgrad) {
+      if (ch < K) v = W[(long(ch) * C + m) * RS + tap];
+    } else {
+      if (ch < C) v = W[(long(m) * C + ch) * RS + tap];
+    }
+    Wt[i] = v;
+  }
+}
+
+// One thread per (k), summing dy over n, p, q is too serial; use one workgroup per k.
+__global__ __launch_bounds__(NT) void k_conv_bgrad(const float *__restrict__ dy, float *__restrict__ db, int N, int K,
+                                                  int PQ) {
+  __shared__ float red[16];
+  const int k = blockIdx.x;
+  float s = 0.f;
+  const int total = N * PQ;
+  for (int i = threadIdx.x; i < total; i += NT) {
+    const int n = i / PQ, r = i - n * PQ;
+    s += dy[(long(n) * K + k) * PQ + r];
+  }
+  s = sgh_block_sum(s, red);
+  if (threadIdx.x == 0) db[k] = s;
+}
+
+inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+inline ConvG to_g(const sgh_conv_geom *g) {
+  return ConvG{g->N, g->C, g->H, g->W, g->K, g->R, g->S, g->stride_h, g->stride_w, g->pad_h, g->pad_w, g->P, g->Q};
+}
+
+inline bool conv_ok(const sgh_conv_geom *g) {
+  if (!g) return false;
+  if (g->N <= 0 || g->C <= 0 || g->H <= 0 || g->W <= 0 || g->K <= 0 || g->R <= 0 || g->S <= 0 || g->stride_h <= 0 ||
+      g->stride_w <= 0 || g->pad_h < 0 || g->pad_w < 0 || g->P <= 0 || g->Q <= 0)
+    return false;
+  if (g->P != (g->H + 2 * g->pad_h - g->R) / g->stride_h + 1) return false;
+  if (g->Q != (g->W + 2 * g->pad_w - g->S) / g->stride_w + 1) return false;
+  if (g->pad_h > 16000 || g->pad_w > 16000 || g->R > 16000 || g->S > 16000) return false;
+  // all flattened index spaces are addressed with 32-bit ints inside the kernels
+  const size_t lim = 0x7fffffffu;
+  if (size_t(g->N) * g->C * g->H * g->W >= lim) return false;
+  if (size_t(g->N) * g->K * g->P * g->Q >= lim) return false;
+  if (size_t(g->K) * g->C * g->R * g->S >= lim) return false;
+  if (size_t(g->R) * g->S * (size_t(g->C > g->K ? g->C : g->K) + BK) >= lim) return false;
+  return true;
+}
+
+struct WgradPlan {
+  int bm, bn, splits, chunks_per_split;
+};
+
+inline WgradPlan plan_wgrad(const sgh_conv_geom *g) {
+  WgradPlan p;
+  const int CRS = g->C * g->R * g->S;
+  p.bm = g->K > 64 ? 128 : 64;
+  p.bn = CRS > 64 ? 128 : 64;
+  const long tiles = long((g->K + p.bm - 1) / p.bm) * ((CRS + p.bn - 1) / p.bn);
+  const long G = long(g->N) * g->P * g->Q;
+  const long chunks = (G + BK - 1) / BK;
+  long want = (long(sgh_num_cus()) * 2 + tiles - 1) / tiles;
+  long max_splits = chunks / 8;  // at least 8 chunks per split
+  if (max_splits < 1) max_splits = 1;
+  long s = want < max_splits ? want : max_splits;
+  if (s < 1) s = 1;
+  if (s > 1024) s = 1024;
+  p.chunks_per_split = int((chunks + s - 1) / s);
+  p.splits = int((chunks + p.chunks_per_split - 1) / p.chunks_per_split);
+  return p;
+}
+
+template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc>
+inline int launch_igemm(const LA &la, const LB &lb, const ST &st, int M, int N, int Ktotal, int splits,
+                        int chunks_per_split, hipStream_t stream) {
+  dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
+  if (grid.y > 65535u || grid.z > 65535u) return SGH_EUNSUPPORTED;
+  hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc>), grid, dim3(NT), 0, stream, la, lb, st, Ktotal,
+                     chunks_per_split);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+// ---- dense GEMM dispatch over the four transpose combinations and two tile sizes -----------
+template <int BM, int BN, bool AK, bool BKc>
+inline int gemm_tile(int M, int N, int K, float alpha, const float *A, long a_rs, long a_ks, const float *B, long b_rs,
+                     long b_ks, float beta, float *C, int ldc, hipStream_t stream) {
+  DenseLoader<BM, AK> la{A, a_rs, a_ks, M, K};
+  DenseLoader<BN, BKc> lb{B, b_rs, b_ks, N, K};
+  DenseStore st{C, ldc, M, N, alpha, beta};
+  const int chunks = (K + BK - 1) / BK;
+  return launch_igemm<BM, BN, DenseLoader<BM, AK>, DenseLoader<BN, BKc>, DenseStore, AK, BKc>(la, lb, st, M, N, K, 1,
+                                                                                               chunks, stream);
+}
+
+template <bool AK, bool BKc>
+inline int gemm_pick(int M, int N, int K, float alpha, const float *A, long a_rs, long a_ks, const float *B, long b_rs,
+                     long b_ks, float beta, float *C, int ldc, hipStream_t stream) {
+  const long tiles128 = long((M + 127) / 128) * ((N + 127) / 128);
+  if (M > 64 && N > 64 && tiles128 >= sgh_num_cus())
+    return gemm_tile<128, 128, AK, BKc>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, stream);
+  return gemm_tile<64, 64, AK, BKc>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+int sgh_conv_geom_init(sgh_conv_geom *g, int N, int C, int H, int W, int K, int R, int S, int stride_h, int stride_w,
+                       int pad_h, int pad_w) {
+  if (!g) return SGH_EINVAL;
+  if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || K <= 0 || R <= 0 || S <= 0 || stride_h <= 0 || stride_w <= 0 ||
+      pad_h < 0 || pad_w < 0)
+    return SGH_EINVAL;
+  if (H + 2 * pad_h < R || W + 2 * pad_w < S) return SGH_EINVAL;
+  g->N = N;
+  g->C = C;
+  g->H = H;
+  g->W = W;
+  g->K = K;
+  g->R = R;
+  g->S = S;
+  g->stride_h = stride_h;
+  g->stride_w = stride_w;
+  g->pad_h = pad_h;
+  g->pad_w = pad_w;
+  // ConvHandle's integer division (reference: src/model/operation/convolution.cc:56-59)
+  g->P = (H + 2 * pad_h - R) / stride_h + 1;
+  g->Q = (W + 2 * pad_w - S) / stride_w + 1;
+  return conv_ok(g) ? SGH_OK : SGH_EINVAL;
+}
+
+size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
+  if (!conv_ok(g)) return 0;
+  const size_t RS = size_t(g->R) * g->S;
+  switch (which) {
+    case SGH_CONV_FWD: return RS * round_up(g->C, BK) * g->K * sizeof(float);
+    case SGH_CONV_DGRAD: return RS * round_up(g->K, BK) * g->C * sizeof(float);
+    case SGH_CONV_WGRAD: {
+      const WgradPlan p = plan_wgrad(g);
+      return p.splits > 1 ? size_t(p.splits) * g->K * g->C * RS * sizeof(float) : 0;
+    }
+    default: return 0;
+  }
+}
+
+int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
+                       size_t ws_bytes, void *stream) {
+  if (!conv_ok(g) || !dy || !W || !dx) return SGH_EINVAL;
+  const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_DGRAD);
+  if (!workspace || ws_bytes < need) return SGH_EWORKSPACE;
+  hipStream_t s = sgh_stream_of(stream);
+  float *Wt = static_cast<float *>(workspace);
+  const int RS = g->R * g->S, KP = round_up(g->K, BK);
+  {
+    const long total = long(RS) * KP * g->C;
+    long blocks = (total + NT - 1) / NT;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
+    SGH_LAUNCH_CHECK();
+  }
+  const int M = g->C, Ncols = g->N * g->H * g->W, Ktot = RS * KP;
+  const int chunks = Ktot / BK;
+  NchwStore st{dx, nullptr, g->C, g->H * g->W, Ncols};
+  if (M > 64) {
+    DenseLoader<128, false> la{Wt, 1, long(g->C), M, Ktot};
+    PixelGatherLoader<128, true> lb{dy, to_g(g), KP, g->K, g->P, g->Q, Ncols, 0, 0, 0, false};
+    return launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+  }
+  DenseLoader<64, false> la{Wt, 1, long(g->C), M, Ktot};
+  PixelGatherLoader<128, true> lb{dy, to_g(g), KP, g->K, g->P, g->Q, Ncols, 0, 0, 0, false};
+  return launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
+      la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+}
+
+int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, const float *bias, float *y,
+                     void *workspace, size_t ws_bytes, void *stream) {
+  if (!conv_ok(g) || !x || !W || !y) return SGH_EINVAL;
+  const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_FWD);
+  if (!workspace || ws_bytes < need) return SGH_EWORKSPACE;
+  hipStream_t s = sgh_stream_of(stream);
+  float *Wt = static_cast<float *>(workspace);
+  const int RS = g->R * g->S, CP = round_up(g->C, BK);
+  {
+    const long total = long(RS) * CP * g->K;
+    long blocks = (total + NT - 1) / NT;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, CP, 0);
+    SGH_LAUNCH_CHECK();
+  }
+  const int M = g->K, Ncols = g->N * g->P * g->Q, Ktot = RS * CP;
+  const int chunks = Ktot / BK;
+  NchwStore st{y, bias, g->K, g->P * g->Q, Ncols};
+  if (M > 64) {
+    DenseLoader<128, false> la{Wt, 1, long(g->K), M, Ktot};
+    PixelGatherLoader<128, false> lb{x, to_g(g), CP, g->C, g->H, g->W, Ncols, 0, 0, 0, false};
+    return launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+  }
+  DenseLoader<64, false> la{Wt, 1, long(g->K), M, Ktot};
+  PixelGatherLoader<128, false> lb{x, to_g(g), CP, g->C, g->H, g->W, Ncols, 0, 0, 0, false};
+  return launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
+      la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+}
+
+int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
+                       size_t ws_bytes, void *stream) {
+  if (!conv_ok(g) || !dy || !x || !dW) return SGH_EINVAL;
+  const WgradPlan p = plan_wgrad(g);
+  const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_WGRAD);
+  if (need && (!workspace || ws_bytes < need)) return SGH_EWORKSPACE;
+  hipStream_t s = sgh_stream_of(stream);
+  const int CRS = g->C * g->R * g->S, PQ = g->P * g->Q;
+  const long G = long(g->N) * PQ;
+  if (G >= 0x7fffffffL) return SGH_EUNSUPPORTED;
+  float *part = p.splits > 1 ? static_cast<float *>(workspace) : dW;
+  SplitStore st{part, g->K, CRS};
+  int rc;
+#define SGH_WGRAD_CASE(BM_, BN_)                                                                                   \
+  {                                                                                                                \
+    WgradDyLoader<BM_> la{dy, g->K, PQ, int(G)};                                                                   \
+    WgradXLoader<BN_> lb;                                                                                          \
+    lb.x = x;                                                                                                      \
+    lb.g = to_g(g);                                                                                                \
+    lb.CRS = CRS;                                                                                                  \
+    rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true>(                    \
+        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s);                                           \
+  }
+  if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128)
+  else if (p.bm == 64 && p.bn == 128) SGH_WGRAD_CASE(64, 128)
+  else if (p.bm == 128 && p.bn == 64) SGH_WGRAD_CASE(128, 64)
+  else SGH_WGRAD_CASE(64, 64)
+#undef SGH_WGRAD_CASE
+  if (rc != SGH_OK) return rc;
+  if (p.splits > 1) {
+    const long n = long(g->K) * CRS;
+    long blocks = (n + NT - 1) / NT;
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(k_split_reduce, dim3(int(blocks)), dim3(NT), 0, s, part, dW, n, p.splits);
+    SGH_LAUNCH_CHECK();
+  }
+  return SGH_OK;
+}
+
+int sgh_conv_bgrad_f32(const sgh_conv_geom *g, const float *dy, float *db, void *stream) {
+  if (!conv_ok(g) || !dy || !db) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_conv_bgrad, dim3(g->K), dim3(NT), 0, sgh_stream_of(stream), dy, db, g->N, g->K, g->P * g->Q);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_gemm_f32(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, const float *B,
+                 int ldb, float beta, float *C, int ldc, void *stream) {
+  if (M < 0 || N < 0 || K < 0) return SGH_EINVAL;
+  if (M == 0 || N == 0) return SGH_OK;
+  if (!C || ldc < N) return SGH_EINVAL;
+  if (K > 0 && (!A || !B)) return SGH_EINVAL;
+  if (K > 0 && (lda < (transA ? M : K) || ldb < (transB ? K : N))) return SGH_EINVAL;
+  hipStream_t s = sgh_stream_of(stream);
+  // element(row, k) strides of each operand
+  const long a_rs = transA ? 1 : lda, a_ks = transA ? lda : 1;  // A(m, k)
+  const long b_rs = transB ? ldb : 1, b_ks = transB ? 1 : ldb;  // B(k, n) addressed as (n, k)
+  if (!transA && transB) return gemm_pick<true, true>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+  if (!transA && !transB) return gemm_pick<true, false>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+  if (transA && transB) return gemm_pick<false, true>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+  return gemm_pick<false, false>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,207 @@
+// Pooling forward/backward for NCHW fp32.
+//
+// Max-pool backward is a gather: one thread owns one dx element, visits the (at most
+// ceil(kh/sh) * ceil(kw/sw)) windows that contain it in ascending (p, q) order, recomputes each
+// window's first maximum (row-major scan, strict '>') and adds dy when the maximum sits on its
+// own element.  The additions therefore happen in exactly the order of the CPU scatter loop, so
+// dx is bit-identical to it and no atomics are needed.
+#include "common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+
+struct PoolG {
+  int H, W, P, Q, kh, kw, sh, sw, ph, pw;
+};
+
+// flat index (h * W + w) of the first maximum of window (p, q) in plane `b`; -1 if empty
+__device__ __forceinline__ int window_argmax(const float *__restrict__ b, const PoolG g, int p, int q, float *best_out) {
+  int hs = p * g.sh - g.ph, ws = q * g.sw - g.pw;
+  const int he = min(hs + g.kh, g.H), we = min(ws + g.kw, g.W);
+  hs = max(hs, 0);
+  ws = max(ws, 0);
+  float best = -3.402823466e38f;
+  int bi = -1;
+  for (int h = hs; h < he; ++h)
+    for (int w = ws; w < we; ++w) {
+      const float v = b[h * g.W + w];
+      if (v > best) {
+        best = v;
+        bi = h * g.W + w;
+      }
+    }
+  if (best_out) *best_out = best;
+  return bi;
+}
+
+__global__ __launch_bounds__(kBlock) void k_pool_max_fwd(const float *__restrict__ x, float *__restrict__ y, PoolG g,
+                                                        size_t total) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  const int PQ = g.P * g.Q;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
+    const size_t plane = i / PQ;
+    const int r = int(i - plane * PQ);
+    float best;
+    window_argmax(x + plane * size_t(g.H) * g.W, g, r / g.Q, r % g.Q, &best);
+    y[i] = best;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void k_pool_max_bwd(const float *__restrict__ dy, const float *__restrict__ x,
+                                                        float *__restrict__ dx, PoolG g, size_t total) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  const int HW = g.H * g.W, PQ = g.P * g.Q;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
+    const size_t plane = i / HW;
+    const int r = int(i - plane * HW);
+    const int h = r / g.W, w = r - h * g.W;
+    const float *xb = x + plane * size_t(HW);
+    const float *db = dy + plane * size_t(PQ);
+    // windows p with p*sh - ph <= h < p*sh - ph + kh
+    const int hp = h + g.ph, wp = w + g.pw;
+    const int p_lo = hp < g.kh ? 0 : (hp - g.kh) / g.sh + 1;
+    const int p_hi = min(hp / g.sh, g.P - 1);
+    const int q_lo = wp < g.kw ? 0 : (wp - g.kw) / g.sw + 1;
+    const int q_hi = min(wp / g.sw, g.Q - 1);
+    float s = 0.f;
+    for (int p = p_lo; p <= p_hi; ++p)
+      for (int q = q_lo; q <= q_hi; ++q)
+        if (window_argmax(xb, g, p, q, nullptr) == r) s += db[p * g.Q + q];
+    dx[i] = s;
+  }
+}
+
+__device__ __forceinline__ int window_count(const PoolG g, int p, int q, int *hs_, int *he_, int *ws_, int *we_) {
+  int hs = p * g.sh - g.ph, ws = q * g.sw - g.pw;
+  const int he = min(hs + g.kh, g.H), we = min(ws + g.kw, g.W);
+  hs = max(hs, 0);
+  ws = max(ws, 0);
+  *hs_ = hs;
+  *he_ = he;
+  *ws_ = ws;
+  *we_ = we;
+  return (he - hs) * (we - ws);  // count-exclude-padding
+}
+
+__global__ __launch_bounds__(kBlock) void k_pool_avg_fwd(const float *__restrict__ x, float *__restrict__ y, PoolG g,
+                                                        size_t total) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  const int PQ = g.P * g.Q;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
+    const size_t plane = i / PQ;
+    const int r = int(i - plane * PQ);
+    const float *b = x + plane * size_t(g.H) * g.W;
+    int hs, he, ws, we;
+    const int cnt = window_count(g, r / g.Q, r % g.Q, &hs, &he, &ws, &we);
+    float s = 0.f;
+    for (int h = hs; h < he; ++h)
+      for (int w = ws; w < we; ++w) s += b[h * g.W + w];
+    y[i] = s / float(cnt);
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void k_pool_avg_bwd(const float *__restrict__ dy, float *__restrict__ dx, PoolG g,
+                                                        size_t total) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  const int HW = g.H * g.W, PQ = g.P * g.Q;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
+    const size_t plane = i / HW;
+    const int r = int(i - plane * HW);
+    const int h = r / g.W, w = r - h * g.W;
+    const float *db = dy + plane * size_t(PQ);
+    const int hp = h + g.ph, wp = w + g.pw;
+    const int p_lo = hp < g.kh ? 0 : (hp - g.kh) / g.sh + 1;
+    const int p_hi = min(hp / g.sh, g.P - 1);
+    const int q_lo = wp < g.kw ? 0 : (wp - g.kw) / g.sw + 1;
+    const int q_hi = min(wp / g.sw, g.Q - 1);
+    float s = 0.f;
+    for (int p = p_lo; p <= p_hi; ++p)
+      for (int q = q_lo; q <= q_hi; ++q) {
+        int hs, he, ws, we;
+        const int cnt = window_count(g, p, q, &hs, &he, &ws, &we);
+        s += db[p * g.Q + q] / float(cnt);
+      }
+    dx[i] = s;
+  }
+}
+
+inline int grid_for(size_t n) {
+  size_t blocks = (n + kBlock - 1) / kBlock;
+  const size_t cap = size_t(sgh_num_cus()) * 32;
+  if (blocks > cap) blocks = cap;
+  return int(blocks < 1 ? 1 : blocks);
+}
+
+inline PoolG to_g(const sgh_pool_geom *g) {
+  return PoolG{g->H, g->W, g->P, g->Q, g->kernel_h, g->kernel_w, g->stride_h, g->stride_w, g->pad_h, g->pad_w};
+}
+
+inline bool geom_ok(const sgh_pool_geom *g) {
+  return g && g->N > 0 && g->C > 0 && g->H > 0 && g->W > 0 && g->kernel_h > 0 && g->kernel_w > 0 && g->stride_h > 0 &&
+         g->stride_w > 0 && g->pad_h >= 0 && g->pad_w >= 0 && g->P > 0 && g->Q > 0 &&
+         g->P == (g->H + 2 * g->pad_h - g->kernel_h) / g->stride_h + 1 &&
+         g->Q == (g->W + 2 * g->pad_w - g->kernel_w) / g->stride_w + 1 &&
+         // every window must overlap the image, else a max window would be empty
+         g->pad_h < g->kernel_h && g->pad_w < g->kernel_w &&
+         size_t(g->H) * g->W < 0x7fffffffu;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sgh_pool_geom_init(sgh_pool_geom *g, int N, int C, int H, int W, int kernel_h, int kernel_w, int stride_h,
+                       int stride_w, int pad_h, int pad_w, int is_max) {
+  if (!g) return SGH_EINVAL;
+  if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || kernel_h <= 0 || kernel_w <= 0 || stride_h <= 0 || stride_w <= 0 ||
+      pad_h < 0 || pad_w < 0)
+    return SGH_EINVAL;
+  if (H + 2 * pad_h < kernel_h || W + 2 * pad_w < kernel_w) return SGH_EINVAL;
+  g->N = N;
+  g->C = C;
+  g->H = H;
+  g->W = W;
+  g->kernel_h = kernel_h;
+  g->kernel_w = kernel_w;
+  g->stride_h = stride_h;
+  g->stride_w = stride_w;
+  g->pad_h = pad_h;
+  g->pad_w = pad_w;
+  // PoolingHandle's floor formula (reference: src/model/operation/pooling.cc:48-51)
+  g->P = (H + 2 * pad_h - kernel_h) / stride_h + 1;
+  g->Q = (W + 2 * pad_w - kernel_w) / stride_w + 1;
+  g->is_max = is_max ? 1 : 0;
+  return geom_ok(g) ? SGH_OK : SGH_EINVAL;
+}
+
+int sgh_pool_fwd_f32(const sgh_pool_geom *g, const float *x, float *y, void *stream) {
+  if (!geom_ok(g) || !x || !y) return SGH_EINVAL;
+  const size_t total = size_t(g->N) * g->C * g->P * g->Q;
+  if (g->is_max)
+    hipLaunchKernelGGL(k_pool_max_fwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), x, y, to_g(g),
+                       total);
+  else
+    hipLaunchKernelGGL(k_pool_avg_fwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), x, y, to_g(g),
+                       total);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_pool_bwd_f32(const sgh_pool_geom *g, const float *dy, const float *x, const float *y, float *dx,
+                     void *stream) {
+  (void)y;
+  if (!geom_ok(g) || !dy || !dx) return SGH_EINVAL;
+  if (g->is_max && !x) return SGH_EINVAL;
+  const size_t total = size_t(g->N) * g->C * g->H * g->W;
+  if (g->is_max)
+    hipLaunchKernelGGL(k_pool_max_bwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
+                       to_g(g), total);
+  else
+    hipLaunchKernelGGL(k_pool_avg_bwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, dx, to_g(g),
+                       total);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,227 @@
+// Device runtime behind the C ABI: one stream + one caching memory pool per opened device.
+// Mirrors what SINGA's CudaGPU + DeviceMemPool give the Tensor layer
+// (reference: src/core/device/cuda_gpu.cc:56-209, src/core/memory/memory.cc:32-118).
+#include <map>
+#include <mutex>
+#include <new>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+struct sgh_device {
+  int id = 0;
+  hipStream_t stream = nullptr;
+  std::mutex mu;
+  // free blocks keyed by their (rounded) size; blocks in use keyed by address
+  std::multimap<size_t, void *> free_blocks;
+  std::unordered_map<void *, size_t> live;
+  size_t in_use = 0, cached = 0, driver_allocs = 0;
+};
+
+struct sgh_event {
+  hipEvent_t ev;
+};
+
+static int g_num_cus = 0;
+
+int sgh_num_cus() {
+  if (g_num_cus > 0) return g_num_cus;
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) == hipSuccess &&
+      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+    g_num_cus = n;
+  else
+    g_num_cus = 256;
+  return g_num_cus;
+}
+
+// Pool granularity: 256 B up to 4 KiB, then power-of-two classes with four steps per octave
+// (worst-case slack 19 %), so a training loop that frees and re-allocates the same tensor
+// shapes every iteration always hits the cache.
+static size_t round_block(size_t bytes) {
+  if (bytes <= 4096) return (bytes + 255) & ~size_t(255);
+  size_t p = 4096;
+  while (p < bytes) p <<= 1;  // p >= bytes > p/2
+  const size_t step = p >> 3;  // eighth of the upper power = quarter of the lower one
+  size_t r = p >> 1;
+  while (r < bytes) r += step;
+  return r;
+}
+
+extern "C" {
+
+const char *sgh_error_string(int rc) {
+  switch (rc) {
+    case SGH_OK: return "ok";
+    case SGH_EINVAL: return "invalid argument";
+    case SGH_EWORKSPACE: return "workspace missing or too small";
+    case SGH_EUNSUPPORTED: return "unsupported configuration";
+    case SGH_ELABEL: return "class label out of range";
+    case SGH_ENOMEM: return "out of device memory";
+    default: break;
+  }
+  if (rc > 0) return hipGetErrorString(static_cast<hipError_t>(rc));
+  return "unknown error";
+}
+
+const char *sgh_version(void) { return "0.1.0"; }
+const char *sgh_arch(void) { return "gfx950"; }
+
+int sgh_device_count(int *count) {
+  if (!count) return SGH_EINVAL;
+  SGH_HIP_TRY(hipGetDeviceCount(count));
+  return SGH_OK;
+}
+
+int sgh_device_open(int gpu_id, sgh_device **out) {
+  if (!out || gpu_id < 0) return SGH_EINVAL;
+  int n = 0;
+  SGH_HIP_TRY(hipGetDeviceCount(&n));
+  if (gpu_id >= n) return SGH_EINVAL;
+  SGH_HIP_TRY(hipSetDevice(gpu_id));
+  sgh_device *d = new (std::nothrow) sgh_device();
+  if (!d) return SGH_ENOMEM;
+  d->id = gpu_id;
+  hipError_t e = hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    delete d;
+    return (int)e;
+  }
+  *out = d;
+  return SGH_OK;
+}
+
+int sgh_pool_trim(sgh_device *dev) {
+  if (!dev) return SGH_EINVAL;
+  std::lock_guard<std::mutex> lk(dev->mu);
+  SGH_HIP_TRY(hipStreamSynchronize(dev->stream));
+  for (auto &kv : dev->free_blocks) (void)hipFree(kv.second);
+  dev->free_blocks.clear();
+  dev->cached = 0;
+  return SGH_OK;
+}
+
+int sgh_device_close(sgh_device *dev) {
+  if (!dev) return SGH_EINVAL;
+  (void)hipSetDevice(dev->id);
+  (void)hipStreamSynchronize(dev->stream);
+  for (auto &kv : dev->free_blocks) (void)hipFree(kv.second);
+  for (auto &kv : dev->live) (void)hipFree(kv.first);
+  (void)hipStreamDestroy(dev->stream);
+  delete dev;
+  return SGH_OK;
+}
+
+void *sgh_device_stream(sgh_device *dev) { return dev ? reinterpret_cast<void *>(dev->stream) : nullptr; }
+
+int sgh_device_sync(sgh_device *dev) {
+  if (!dev) return SGH_EINVAL;
+  SGH_HIP_TRY(hipStreamSynchronize(dev->stream));
+  return SGH_OK;
+}
+
+int sgh_malloc(sgh_device *dev, void **ptr, size_t bytes) {
+  if (!dev || !ptr) return SGH_EINVAL;
+  if (bytes == 0) bytes = 1;
+  const size_t r = round_block(bytes);
+  std::lock_guard<std::mutex> lk(dev->mu);
+  auto it = dev->free_blocks.find(r);
+  void *p = nullptr;
+  if (it != dev->free_blocks.end()) {
+    p = it->second;
+    dev->free_blocks.erase(it);
+    dev->cached -= r;
+  } else {
+    hipError_t e = hipMalloc(&p, r);
+    if (e == hipErrorOutOfMemory && !dev->free_blocks.empty()) {
+      // give the cache back to the driver once and retry
+      (void)hipGetLastError();
+      (void)hipStreamSynchronize(dev->stream);
+      for (auto &kv : dev->free_blocks) (void)hipFree(kv.second);
+      dev->free_blocks.clear();
+      dev->cached = 0;
+      e = hipMalloc(&p, r);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return e == hipErrorOutOfMemory ? SGH_ENOMEM : (int)e;
+    }
+    dev->driver_allocs++;
+  }
+  dev->live.emplace(p, r);
+  dev->in_use += r;
+  *ptr = p;
+  return SGH_OK;
+}
+
+int sgh_free(sgh_device *dev, void *ptr) {
+  if (!dev) return SGH_EINVAL;
+  if (!ptr) return SGH_OK;
+  std::lock_guard<std::mutex> lk(dev->mu);
+  auto it = dev->live.find(ptr);
+  if (it == dev->live.end()) return SGH_EINVAL;
+  const size_t r = it->second;
+  dev->live.erase(it);
+  dev->in_use -= r;
+  // Work already enqueued on the device stream may still read the block; the next owner's
+  // work is enqueued behind it on the same stream, so immediate reuse is ordered correctly.
+  dev->free_blocks.emplace(r, ptr);
+  dev->cached += r;
+  return SGH_OK;
+}
+
+int sgh_pool_stats(sgh_device *dev, size_t *in_use, size_t *cached, size_t *driver_allocs) {
+  if (!dev) return SGH_EINVAL;
+  std::lock_guard<std::mutex> lk(dev->mu);
+  if (in_use) *in_use = dev->in_use;
+  if (cached) *cached = dev->cached;
+  if (driver_allocs) *driver_allocs = dev->driver_allocs;
+  return SGH_OK;
+}
+
+int sgh_memcpy(sgh_device *dev, void *dst, const void *src, size_t bytes, int kind) {
+  if (!dev || kind < 0 || kind > 3) return SGH_EINVAL;
+  if (bytes == 0) return SGH_OK;
+  if (!dst || !src) return SGH_EINVAL;
+  static const hipMemcpyKind kinds[4] = {hipMemcpyHostToHost, hipMemcpyHostToDevice,
+                                         hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice};
+  SGH_HIP_TRY(hipMemcpyAsync(dst, src, bytes, kinds[kind], dev->stream));
+  if (kind != 3) SGH_HIP_TRY(hipStreamSynchronize(dev->stream));
+  return SGH_OK;
+}
+
+int sgh_event_create(sgh_event **ev) {
+  if (!ev) return SGH_EINVAL;
+  sgh_event *e = new (std::nothrow) sgh_event();
+  if (!e) return SGH_ENOMEM;
+  hipError_t rc = hipEventCreate(&e->ev);
+  if (rc != hipSuccess) {
+    delete e;
+    return (int)rc;
+  }
+  *ev = e;
+  return SGH_OK;
+}
+
+int sgh_event_destroy(sgh_event *ev) {
+  if (!ev) return SGH_EINVAL;
+  (void)hipEventDestroy(ev->ev);
+  delete ev;
+  return SGH_OK;
+}
+
+int sgh_event_record(sgh_event *ev, void *stream) {
+  if (!ev) return SGH_EINVAL;
+  SGH_HIP_TRY(hipEventRecord(ev->ev, sgh_stream_of(stream)));
+  return SGH_OK;
+}
+
+int sgh_event_elapsed_ms(sgh_event *start, sgh_event *stop, float *ms) {
+  if (!start || !stop || !ms) return SGH_EINVAL;
+  SGH_HIP_TRY(hipEventSynchronize(stop->ev));
+  SGH_HIP_TRY(hipEventElapsedTime(ms, start->ev, stop->ev));
+  return SGH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,84 @@
+"""SGD with momentum as ``python/singa/opt.py`` defines it (class SGD :168-333), with the four
+tensor ops of ``SGD.apply`` (:269-310) replaced by one fused kernel launch per parameter, or by a
+single launch over all parameters (``apply_all``, the loop of ``Optimizer.call`` :107-111).
+
+    [g += weight_decay * p]
+    v  = momentum * v + (1 - dampening) * g
+    g' = g + momentum * v   (nesterov)   |   v   (otherwise)
+    p -= lr * g'
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from . import singa_wrap as singa
+from ._lib import check
+
+
+class SGD(object):
+
+    def __init__(self, lr=0.1, momentum=0, dampening=0, weight_decay=0, nesterov=False):
+        if momentum < 0.0:
+            raise ValueError("Invalid momentum value: {}".format(momentum))
+        if weight_decay < 0.0:
+            raise ValueError("Invalid weight_decay value: {}".format(weight_decay))
+        if nesterov and (momentum <= 0 or dampening != 0):
+            raise ValueError("Nesterov momentum requires a momentum and zero dampening")
+        self.lr = float(lr)
+        self.momentum = float(momentum)
+        self.dampening = float(dampening)
+        self.weight_decay = float(weight_decay)
+        self.nesterov = bool(nesterov)
+        self.moments = dict()
+        self.step_counter = 0
+        self._table = None
+        self._table_key = None
+
+    def _moment(self, name, p):
+        if name not in self.moments:
+            v = singa.Tensor(p.shape(), p.device(), p.data_type())
+            v.SetFloatValue(0.0)
+            self.moments[name] = v
+        return self.moments[name]
+
+    def apply(self, param_name, param_value, param_grad):
+        """One fused update of ``param_value`` (in place).  Unlike the reference the gradient
+        tensor is left untouched."""
+        assert param_value.shape() == param_grad.shape(), ("shape mismatch", param_value.shape(),
+                                                             param_grad.shape())
+        v = self._moment(param_name, param_value) if self.momentum != 0 else None
+        check(_lib.lib().sgh_sgd_momentum_f32(param_value.ptr, param_grad.ptr, v.ptr if v is not None else None,
+                                              param_value.Size(), self.lr, self.momentum, self.dampening,
+                                              self.weight_decay, int(self.nesterov), param_value.device().stream),
+              "sgh_sgd_momentum_f32")
+
+    def apply_all(self, named_params_grads):
+        """Update every (name, p, g) triple with ONE kernel launch.  The pointer table is built
+        once per distinct set of buffers and kept on the device."""
+        items = list(named_params_grads)
+        if not items:
+            return
+        dev = items[0][1].device()
+        key = tuple((n, p.ptr, g.ptr) for n, p, g in items)
+        if key != self._table_key:
+            arr = (_lib.SgdItem * len(items))()
+            total = 0
+            for i, (n, p, g) in enumerate(items):
+                assert p.shape() == g.shape(), ("shape mismatch", n)
+                v = self._moment(n, p) if self.momentum != 0 else None
+                arr[i].p, arr[i].g, arr[i].v, arr[i].n = p.ptr, g.ptr, (v.ptr if v is not None else None), p.Size()
+                total += p.Size()
+            nbytes = C.sizeof(arr)
+            table = singa.Tensor(((nbytes + 3) // 4,), dev, singa.kInt)
+            check(_lib.lib().sgh_memcpy(dev._h, table.ptr, C.addressof(arr), nbytes, 1), "sgh_memcpy H2D")
+            self._table, self._table_key, self._table_total = table, key, total
+        check(_lib.lib().sgh_sgd_momentum_multi_f32(self._table.ptr, len(items), self._table_total, self.lr,
+                                                    self.momentum, self.dampening, self.weight_decay,
+                                                    int(self.nesterov), dev.stream), "sgh_sgd_momentum_multi_f32")
+
+    def step(self):
+        self.step_counter += 1
+
+    def get_states(self):
+        return {k: v.to_numpy() for k, v in self.moments.items()}

@@ -1,0 +1,556 @@
+"""Host-side mirror of the slice of SINGA's ``singa_wrap`` (SWIG) module that the backward pass
+uses, bound to the gfx950 library through its C ABI.
+
+Names, argument order and meaning follow the reference so that code written against
+``singa_wrap`` for a non-CPU device reads the same here:
+
+* tensor functions: ``src/api/core_tensor.i`` (``ReLUBackward`` :344-355, ``Axpy`` :387-388,
+  ``Mult``, ``SoftmaxCrossEntropyBwd``, ``CrossEntropyFwd``, ``SoftMax``, ``Sum``, ``SumAll``,
+  ``__iadd__`` / ``__imul__``)
+* operation handles and functions: ``src/api/model_operation.i:121-191``
+  (``CudnnConvHandle``, ``GpuConvForward/Backwardx/BackwardW/Backwardb``,
+  ``CudnnBatchNormHandle``, ``GpuBatchNormForwardTraining/Backward``,
+  ``CudnnPoolingHandle``, ``GpuPoolingForward/Backward``)
+* device factory: ``python/singa/device.py:103-114`` (``create_cuda_gpu_on``)
+
+Every function only enqueues work on the device's stream; ``Device.Sync()`` or a copy to the
+host waits for it.  Errors raise ``SingaHipError`` (the reference aborts through CHECK).
+There is no CPU path in this module: without the built library and a GPU it cannot run.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import SingaHipError, check  # noqa: F401  (re-exported)
+
+# core.proto DataType values (src/proto/core.proto:26-34)
+kFloat32, kFloat16, kInt = 0, 1, 2
+# core.proto LangType (src/proto/core.proto:36-41); 3 is the value a HIP backend takes
+kCpp, kCuda, kOpencl, kHip = 0, 1, 2, 3
+
+_NP_OF = {kFloat32: np.float32, kInt: np.int32}
+_SIZE_OF = {kFloat32: 4, kInt: 4}
+
+USE_HIP = True
+
+
+def _L():
+    return _lib.lib()
+
+
+# ------------------------------------------------------------------------------------ device
+
+class HipGPU(object):
+    """Counterpart of ``CudaGPU`` (include/singa/core/device.h:57-174): one stream, one pool."""
+
+    def __init__(self, gpu_id=0):
+        h = C.c_void_p()
+        check(_L().sgh_device_open(int(gpu_id), C.byref(h)), "sgh_device_open")
+        self._h = h
+        self._id = int(gpu_id)
+        self.stream = _L().sgh_device_stream(h)
+
+    def id(self):
+        return self._id
+
+    def lang(self):
+        return kHip
+
+    def Sync(self):
+        check(_L().sgh_device_sync(self._h), "sgh_device_sync")
+
+    def GetAllocatedMem(self):
+        a, c, d = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        check(_L().sgh_pool_stats(self._h, C.byref(a), C.byref(c), C.byref(d)))
+        return a.value
+
+    def PoolStats(self):
+        a, c, d = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        check(_L().sgh_pool_stats(self._h, C.byref(a), C.byref(c), C.byref(d)))
+        return {"in_use": a.value, "cached": c.value, "driver_allocs": d.value}
+
+    # graph buffering is a property of SINGA's scheduler, not of this device
+    def graph_enabled(self):
+        return False
+
+    def EnableGraph(self, flag):
+        if flag:
+            raise SingaHipError("graph buffering lives in SINGA's scheduler; not available here")
+
+    def _malloc(self, nbytes):
+        p = C.c_void_p()
+        check(_L().sgh_malloc(self._h, C.byref(p), nbytes), "sgh_malloc")
+        return p.value
+
+    def _free(self, ptr):
+        if self._h is not None and _lib._lib is not None:
+            _lib._lib.sgh_free(self._h, C.c_void_p(ptr))
+
+
+_devices = {}
+
+
+def create_hip_gpu_on(device_id=0):
+    """``device.create_cuda_gpu_on`` analogue; devices are cached per id like
+    Platform::UsedDevice (src/core/device/platform.cc:137-160)."""
+    if device_id not in _devices:
+        _devices[device_id] = HipGPU(device_id)
+    return _devices[device_id]
+
+
+create_cuda_gpu_on = create_hip_gpu_on
+create_cuda_gpu = create_hip_gpu_on
+
+
+# ------------------------------------------------------------------------------------ tensor
+
+class _Block(object):
+    """Counterpart of ``Block`` (include/singa/core/common.h:64-97): a pool allocation freed
+    when the last Tensor referring to it goes away."""
+
+    def __init__(self, dev, nbytes, ptr=None, keepalive=None):
+        self.dev = dev
+        self.nbytes = nbytes
+        self.owned = ptr is None
+        self.ptr = dev._malloc(max(nbytes, 1)) if ptr is None else ptr
+        self.keepalive = keepalive
+
+    def __del__(self):
+        try:
+            if self.owned and self.ptr:
+                self.dev._free(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
+class Tensor(object):
+    """Counterpart of ``singa::Tensor`` as Python sees it (src/api/core_tensor.i:95-232):
+    dense row-major data on a HipGPU, plus a transpose flag for 2-D views."""
+
+    def __init__(self, shape=(), device=None, dtype=kFloat32, _block=None, _transposed=False):
+        if device is None:
+            raise SingaHipError("a HipGPU device is required (this module has no CPU path)")
+        if dtype not in _SIZE_OF:
+            raise SingaHipError("unsupported data type %r" % (dtype,))
+        self._shape = tuple(int(s) for s in shape)
+        self._dev = device
+        self._dtype = dtype
+        self._transposed = _transposed
+        self._block = _block if _block is not None else _Block(device, self.Size() * _SIZE_OF[dtype])
+
+    # --- reference accessors
+    def shape(self, axis=None):
+        return list(self._shape) if axis is None else self._shape[axis]
+
+    def nDim(self):
+        return len(self._shape)
+
+    def Size(self):
+        n = 1
+        for s in self._shape:
+            n *= s
+        return n
+
+    def MemSize(self):
+        return self.Size() * _SIZE_OF[self._dtype]
+
+    def data_type(self):
+        return self._dtype
+
+    def device(self):
+        return self._dev
+
+    def transpose(self):
+        return self._transposed
+
+    @property
+    def ptr(self):
+        return self._block.ptr
+
+    # --- views
+    def Reshape(self, shape):
+        shape = tuple(int(s) for s in shape)
+        t = Tensor(shape, self._dev, self._dtype, _block=self._block)
+        if t.Size() != self.Size():
+            raise SingaHipError("Reshape changes the element count")
+        if self._transposed:
+            raise SingaHipError("Reshape of a transposed view is not supported")
+        return t
+
+    def T(self):
+        if len(self._shape) != 2:
+            raise SingaHipError("T() needs a 2-D tensor")
+        return Tensor((self._shape[1], self._shape[0]), self._dev, self._dtype, _block=self._block,
+                      _transposed=not self._transposed)
+
+    def Clone(self):
+        t = Tensor(self._shape, self._dev, self._dtype, _transposed=self._transposed)
+        check(_L().sgh_memcpy(self._dev._h, t.ptr, self.ptr, self.MemSize(), 3), "sgh_memcpy D2D")
+        return t
+
+    # --- host transfers
+    def CopyFloatDataFromHostPtr(self, arr):
+        a = np.ascontiguousarray(arr, dtype=np.float32).ravel()
+        if a.size != self.Size() or self._dtype != kFloat32:
+            raise SingaHipError("size or type mismatch in CopyFloatDataFromHostPtr")
+        check(_L().sgh_memcpy(self._dev._h, self.ptr, a.ctypes.data, a.nbytes, 1), "sgh_memcpy H2D")
+
+    def CopyIntDataFromHostPtr(self, arr):
+        a = np.ascontiguousarray(arr, dtype=np.int32).ravel()
+        if a.size != self.Size() or self._dtype != kInt:
+            raise SingaHipError("size or type mismatch in CopyIntDataFromHostPtr")
+        check(_L().sgh_memcpy(self._dev._h, self.ptr, a.ctypes.data, a.nbytes, 1), "sgh_memcpy H2D")
+
+    def to_numpy(self):
+        out = np.empty(self.Size(), dtype=_NP_OF[self._dtype])
+        if out.size:
+            check(_L().sgh_memcpy(self._dev._h, out.ctypes.data, self.ptr, out.nbytes, 2), "sgh_memcpy D2H")
+        if self._transposed:
+            return out.reshape(self._shape[1], self._shape[0]).T.copy()
+        return out.reshape(self._shape)
+
+    def SetFloatValue(self, v):
+        check(_L().sgh_memset_f32(self.ptr, float(v), self.Size(), self._dev.stream), "sgh_memset_f32")
+
+    # --- arithmetic used by autograd / opt  (Tensor::operator+=, *=: src/core/tensor/tensor.cc:579-589)
+    def __iadd__(self, other):
+        _same(self, other)
+        check(_L().sgh_add_f32(self.ptr, other.ptr, self.ptr, self.Size(), self._dev.stream), "sgh_add_f32")
+        return self
+
+    def __imul__(self, other):
+        if isinstance(other, Tensor):
+            scalar = other.Size() == 1 and self.Size() != 1
+            if not scalar:
+                _same(self, other)
+            check(_L().sgh_eltwise_mult_f32(self.ptr, other.ptr, int(scalar), self.ptr, self.Size(),
+                                            self._dev.stream), "sgh_eltwise_mult_f32")
+        else:
+            s = from_numpy(np.array([other], dtype=np.float32), self._dev)
+            check(_L().sgh_eltwise_mult_f32(self.ptr, s.ptr, 1, self.ptr, self.Size(), self._dev.stream),
+                  "sgh_eltwise_mult_f32")
+        return self
+
+    def __itruediv__(self, d):
+        # Div(tensor, scalar) multiplies by the fp32 reciprocal (src/core/tensor/tensor_math.h:149-153)
+        return self.__imul__(float(np.float32(1.0) / np.float32(d)))
+
+
+def _same(a, b):
+    if a.Size() != b.Size() or a.data_type() != b.data_type():
+        raise SingaHipError("shape/type mismatch: %s vs %s" % (a.shape(), b.shape()))
+    if a.transpose() or b.transpose():
+        raise SingaHipError("elementwise ops need contiguous (non-transposed) tensors")
+
+
+def from_numpy(arr, device):
+    arr = np.asarray(arr)
+    if arr.dtype in (np.int32, np.int64):
+        t = Tensor(arr.shape, device, kInt)
+        t.CopyIntDataFromHostPtr(arr)
+    else:
+        t = Tensor(arr.shape, device, kFloat32)
+        t.CopyFloatDataFromHostPtr(arr)
+    return t
+
+
+def from_device_pointer(ptr, shape, device, dtype=kFloat32, keepalive=None):
+    """Wrap device memory owned by someone else (e.g. a torch tensor; pass it as keepalive)."""
+    t = Tensor.__new__(Tensor)
+    t._shape = tuple(int(s) for s in shape)
+    t._dev = device
+    t._dtype = dtype
+    t._transposed = False
+    t._block = _Block(device, t.Size() * _SIZE_OF[dtype], ptr=int(ptr), keepalive=keepalive)
+    return t
+
+
+def DefaultTranspose(t):
+    return t.T()
+
+
+def Reshape(t, shape):
+    return t.Reshape(shape)
+
+
+# ------------------------------------------------------------------------------------ tensor math
+
+def _like(t):
+    return Tensor(t.shape(), t.device(), t.data_type())
+
+
+def ReLU(x):
+    y = _like(x)
+    check(_L().sgh_relu_fwd_f32(x.ptr, y.ptr, x.Size(), x.device().stream), "sgh_relu_fwd_f32")
+    return y
+
+
+def ReLUBackward(dy, x):
+    """``singa.ReLUBackward(dy, x)`` (python/singa/autograd.py:432-439)."""
+    _same(dy, x)
+    dx = _like(dy)
+    check(_L().sgh_relu_bwd_f32(dy.ptr, x.ptr, dx.ptr, dy.Size(), dy.device().stream), "sgh_relu_bwd_f32")
+    return dx
+
+
+def SoftMax(x):
+    batch = x.shape(0) if x.nDim() == 2 else 1
+    p = _like(x)
+    check(_L().sgh_softmax_fwd_f32(x.ptr, p.ptr, batch, x.Size() // batch, x.device().stream),
+          "sgh_softmax_fwd_f32")
+    return p
+
+
+def _ce_dims(p, t):
+    if p.nDim() > 2 or t.nDim() > 2:
+        raise SingaHipError("cross entropy expects at most 2-D tensors")
+    if t.data_type() != kInt:
+        raise SingaHipError("the target tensor must hold int32 (the reference reads it as int)")
+    batch = p.shape(0) if p.nDim() == 2 else 1
+    dim = p.Size() // batch
+    int_target = t.Size() == batch
+    if not int_target and t.Size() != p.Size():
+        raise SingaHipError("target size matches neither [batch] nor [batch, dim]")
+    return batch, dim, int_target
+
+
+def CrossEntropyFwd(p, t):
+    batch, dim, int_target = _ce_dims(p, t)
+    loss = Tensor((batch,), p.device(), kFloat32)
+    check(_L().sgh_cross_entropy_fwd_f32(p.ptr, t.ptr, loss.ptr, batch, dim, int(int_target),
+                                         p.device().stream), "sgh_cross_entropy_fwd_f32")
+    return loss
+
+
+def SoftmaxCrossEntropyBwd(p, t, scale=1.0):
+    """``singa.SoftmaxCrossEntropyBwd(p, t)`` (src/core/tensor/tensor.cc:1717-1721): returns a new
+    tensor.  ``scale`` (not in the reference signature) fuses the ``dx /= N`` that follows it."""
+    batch, dim, int_target = _ce_dims(p, t)
+    g = _like(p)
+    check(_L().sgh_softmax_ce_bwd_f32(p.ptr, t.ptr, g.ptr, batch, dim, int(int_target), float(scale),
+                                      p.device().stream), "sgh_softmax_ce_bwd_f32")
+    return g
+
+
+def LabelErrors(device):
+    n = C.c_int()
+    check(_L().sgh_softmax_ce_label_errors(device.stream, C.byref(n)))
+    return n.value
+
+
+def Axpy(alpha, x, y):
+    """``singa.Axpy(alpha, x, y)``: y += alpha * x; alpha is a float or a 1-element device Tensor."""
+    _same(x, y)
+    if isinstance(alpha, Tensor):
+        if alpha.Size() != 1:
+            raise SingaHipError("Tensor alpha must have one element")
+        check(_L().sgh_axpy_devalpha_f32(alpha.ptr, x.ptr, y.ptr, x.Size(), x.device().stream),
+              "sgh_axpy_devalpha_f32")
+    else:
+        check(_L().sgh_axpy_f32(float(alpha), x.ptr, y.ptr, x.Size(), x.device().stream), "sgh_axpy_f32")
+
+
+def EltwiseMult(a, b, out=None):
+    out = _like(a) if out is None else out
+    scalar = b.Size() == 1 and a.Size() != 1
+    if not scalar:
+        _same(a, b)
+    check(_L().sgh_eltwise_mult_f32(a.ptr, b.ptr, int(scalar), out.ptr, a.Size(), a.device().stream),
+          "sgh_eltwise_mult_f32")
+    return out
+
+
+def __add__(a, b):
+    _same(a, b)
+    out = _like(a)
+    check(_L().sgh_add_f32(a.ptr, b.ptr, out.ptr, a.Size(), a.device().stream), "sgh_add_f32")
+    return out
+
+
+def Mult(A, B):
+    """``singa.Mult(A, B)`` for 2-D tensors (src/core/tensor/tensor.cc:1633-1706): the transpose
+    flags of the views select the GEMM variant, no data is moved."""
+    if A.nDim() != 2 or B.nDim() != 2 or A.shape(1) != B.shape(0):
+        raise SingaHipError("Mult shape mismatch %s x %s" % (A.shape(), B.shape()))
+    M, K, N = A.shape(0), A.shape(1), B.shape(1)
+    out = Tensor((M, N), A.device(), kFloat32)
+    tA, tB = A.transpose(), B.transpose()
+    lda = M if tA else K
+    ldb = K if tB else N
+    check(_L().sgh_gemm_f32(int(tA), int(tB), M, N, K, 1.0, A.ptr, lda, B.ptr, ldb, 0.0, out.ptr, N,
+                            A.device().stream), "sgh_gemm_f32")
+    return out
+
+
+def Sum(t, axis):
+    """``singa.Sum(t, 0)`` of a 2-D tensor: column sums (bias gradient of AddBias)."""
+    if t.nDim() != 2 or axis != 0 or t.transpose():
+        raise SingaHipError("only Sum(2-D tensor, 0) is on the backward path")
+    out = Tensor((t.shape(1),), t.device(), kFloat32)
+    check(_L().sgh_sum_rows_f32(t.ptr, out.ptr, t.shape(0), t.shape(1), t.device().stream), "sgh_sum_rows_f32")
+    return out
+
+
+def AddRow(v, m):
+    check(_L().sgh_add_row_f32(v.ptr, m.ptr, m.shape(0), m.shape(1), m.device().stream), "sgh_add_row_f32")
+
+
+# ------------------------------------------------------------------------------------ operations
+
+class CudnnConvHandle(object):
+    """Geometry + workspace of a convolution on the GPU device.  Same constructor arguments and
+    public fields as the reference's handle (src/model/operation/convolution.h:43-129; fields read
+    from Python: src/api/model_operation.i:37-54)."""
+
+    def __init__(self, x, kernel_size, stride, padding, in_channels, out_channels, bias, groups=1,
+                 workspace_byte_limit=1024 * 1024 * 1024, prefer="fastest"):
+        if groups != 1:
+            raise SingaHipError("grouped convolution is not on the backward path built here")
+        if x.nDim() != 4 or x.shape(1) != in_channels:
+            raise SingaHipError("the number of input channels mismatched.")
+        self.kernel_h, self.kernel_w = int(kernel_size[0]), int(kernel_size[1])
+        self.stride_h, self.stride_w = int(stride[0]), int(stride[1])
+        self.pad_h, self.pad_w = int(padding[0]), int(padding[1])
+        self.channels, self.num_filters = int(in_channels), int(out_channels)
+        self.group = groups
+        self.bias_term = bool(bias)
+        self.batchsize, _, self.height, self.width = x.shape()
+        self.geom = _lib.ConvGeom()
+        check(_L().sgh_conv_geom_init(C.byref(self.geom), self.batchsize, self.channels, self.height,
+                                      self.width, self.num_filters, self.kernel_h, self.kernel_w,
+                                      self.stride_h, self.stride_w, self.pad_h, self.pad_w),
+              "sgh_conv_geom_init")
+        self.conv_height, self.conv_width = self.geom.P, self.geom.Q
+        self.col_height = self.channels * self.kernel_h * self.kernel_w
+        self.col_width = self.conv_height * self.conv_width
+        self.imagesize = x.Size() // self.batchsize
+        need = max(_L().sgh_conv_workspace_bytes(C.byref(self.geom), w) for w in (0, 1, 2))
+        if need > workspace_byte_limit:
+            raise SingaHipError("workspace of %d bytes exceeds the limit" % need)
+        self.workspace_count = need // 4
+        self.workspace = Tensor((max(self.workspace_count, 1),), x.device(), kFloat32)
+
+    def _check_x(self, x):
+        if x.shape() != [self.batchsize, self.channels, self.height, self.width]:
+            raise SingaHipError("input sample shape should not change")
+
+    def _check_dy(self, dy):
+        if dy.shape() != [self.batchsize, self.num_filters, self.conv_height, self.conv_width]:
+            raise SingaHipError("dy shape does not match the handle")
+
+
+def GpuConvForward(x, W, b, h):
+    h._check_x(x)
+    y = Tensor((h.batchsize, h.num_filters, h.conv_height, h.conv_width), x.device(), kFloat32)
+    bias = b.ptr if (h.bias_term and b is not None) else None
+    check(_L().sgh_conv_fwd_f32(C.byref(h.geom), x.ptr, W.ptr, bias, y.ptr, h.workspace.ptr,
+                                h.workspace.MemSize(), x.device().stream), "sgh_conv_fwd_f32")
+    return y
+
+
+def GpuConvBackwardx(dy, W, x, h):
+    h._check_dy(dy)
+    dx = _like(x)
+    check(_L().sgh_conv_dgrad_f32(C.byref(h.geom), dy.ptr, W.ptr, dx.ptr, h.workspace.ptr,
+                                  h.workspace.MemSize(), dy.device().stream), "sgh_conv_dgrad_f32")
+    return dx
+
+
+def GpuConvBackwardW(dy, x, W, h):
+    h._check_dy(dy)
+    h._check_x(x)
+    dW = _like(W)
+    check(_L().sgh_conv_wgrad_f32(C.byref(h.geom), dy.ptr, x.ptr, dW.ptr, h.workspace.ptr,
+                                  h.workspace.MemSize(), dy.device().stream), "sgh_conv_wgrad_f32")
+    return dW
+
+
+def GpuConvBackwardb(dy, b, h):
+    h._check_dy(dy)
+    db = _like(b)
+    check(_L().sgh_conv_bgrad_f32(C.byref(h.geom), dy.ptr, db.ptr, dy.device().stream), "sgh_conv_bgrad_f32")
+    return db
+
+
+class CudnnBatchNormHandle(object):
+    """``CudnnBatchNormHandle(momentum, x)`` (src/model/operation/batchnorm.h:49-101)."""
+
+    def __init__(self, momentum, x):
+        self.factor = float(momentum)
+        self.is_2d = x.nDim() == 2
+        if self.is_2d:
+            self.batchsize, self.channels = x.shape()
+            self.height = self.width = 1
+        elif x.nDim() == 4:
+            self.batchsize, self.channels, self.height, self.width = x.shape()
+        else:
+            raise SingaHipError("BatchNorm expects a 2-D or 4-D input")
+        hw = self.height * self.width
+        nbytes = _L().sgh_bn_workspace_bytes(self.batchsize, self.channels, hw)
+        self.workspace = Tensor((max(nbytes // 4, 1),), x.device(), kFloat32)
+
+
+_BN_EPS = 1e-5  # CUDNN_BN_MIN_EPSILON, src/model/operation/batchnorm.cc:313
+
+
+def GpuBatchNormForwardTraining(h, x, scale, bias, running_mean, running_var):
+    """Returns ``[y, mean, var]`` where ``var`` holds the saved inverse standard deviation, and
+    updates the running statistics in place (src/model/operation/batchnorm.cc:287-329)."""
+    y = _like(x)
+    mean = Tensor((h.channels,), x.device(), kFloat32)
+    var = Tensor((h.channels,), x.device(), kFloat32)
+    check(_L().sgh_bn_fwd_train_f32(x.ptr, scale.ptr, bias.ptr,
+                                    running_mean.ptr if running_mean is not None else None,
+                                    running_var.ptr if running_var is not None else None,
+                                    h.factor, _BN_EPS, y.ptr, mean.ptr, var.ptr, h.batchsize, h.channels,
+                                    h.height * h.width, h.workspace.ptr, h.workspace.MemSize(),
+                                    x.device().stream), "sgh_bn_fwd_train_f32")
+    return [y, mean, var]
+
+
+def GpuBatchNormBackward(h, dy, x, scale, mean, var):
+    """Returns ``[dx, dscale, dbias]`` (src/model/operation/batchnorm.cc:368-404)."""
+    _same(dy, x)
+    dx = _like(dy)
+    ds = _like(scale)
+    db = _like(scale)
+    check(_L().sgh_bn_bwd_f32(dy.ptr, x.ptr, scale.ptr, mean.ptr, var.ptr, dx.ptr, ds.ptr, db.ptr,
+                              h.batchsize, h.channels, h.height * h.width, h.workspace.ptr,
+                              h.workspace.MemSize(), dy.device().stream), "sgh_bn_bwd_f32")
+    return [dx, ds, db]
+
+
+class CudnnPoolingHandle(object):
+    """``CudnnPoolingHandle(x, kernel, stride, padding, is_max)``
+    (src/model/operation/pooling.h:40-91)."""
+
+    def __init__(self, x, kernel_size, stride, padding, is_max=True):
+        if x.nDim() != 4:
+            raise SingaHipError("pooling expects a 4-D input")
+        self.kernel_h, self.kernel_w = int(kernel_size[0]), int(kernel_size[1])
+        self.stride_h, self.stride_w = int(stride[0]), int(stride[1])
+        self.pad_h, self.pad_w = int(padding[0]), int(padding[1])
+        self.batchsize, self.channels, self.height, self.width = x.shape()
+        self.is_max_pooling = bool(is_max)
+        self.geom = _lib.PoolGeom()
+        check(_L().sgh_pool_geom_init(C.byref(self.geom), self.batchsize, self.channels, self.height,
+                                      self.width, self.kernel_h, self.kernel_w, self.stride_h, self.stride_w,
+                                      self.pad_h, self.pad_w, int(self.is_max_pooling)), "sgh_pool_geom_init")
+        self.pooled_height, self.pooled_width = self.geom.P, self.geom.Q
+
+
+def GpuPoolingForward(h, x):
+    y = Tensor((h.batchsize, h.channels, h.pooled_height, h.pooled_width), x.device(), kFloat32)
+    check(_L().sgh_pool_fwd_f32(C.byref(h.geom), x.ptr, y.ptr, x.device().stream), "sgh_pool_fwd_f32")
+    return y
+
+
+def GpuPoolingBackward(h, dy, x, y):
+    if dy.shape() != [h.batchsize, h.channels, h.pooled_height, h.pooled_width]:
+        raise SingaHipError("dy shape does not match the handle")
+    dx = _like(x)
+    check(_L().sgh_pool_bwd_f32(C.byref(h.geom), dy.ptr, x.ptr, y.ptr if y is not None else None, dx.ptr,
+                                dy.device().stream), "sgh_pool_bwd_f32")
+    return dx

@@ -1,0 +1,77 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/singa_hip.h declares;
+host-only entry points (geometry, sizes, error strings) behave as documented."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from singa_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "singa_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"SGH_API\s+[\w\s\*]+?\b(sgh_\w+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    decl = declared_symbols()
+    assert len(decl) >= 40
+    assert sorted(_lib.SIGNATURES) == decl
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(_lib.LIBPATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_error_strings_and_identity():
+    lib = _lib.lib()
+    assert lib.sgh_arch() == b"gfx950"
+    assert lib.sgh_error_string(0) == b"ok"
+    assert b"workspace" in lib.sgh_error_string(-2)
+    assert b"invalid" in lib.sgh_error_string(-1)
+
+
+def test_conv_geometry_follows_reference_integer_division():
+    lib = _lib.lib()
+    g = _lib.ConvGeom()
+    # 7x7 stride 2 pad 3 on 224 -> 112 ; 3x3 stride 2 pad 1 on 56 -> 28 ; 1x1 stride 2 on 56 -> 28
+    for (H, R, s, p, P) in [(224, 7, 2, 3, 112), (56, 3, 2, 1, 28), (56, 1, 2, 0, 28), (3, 3, 2, 1, 2), (8, 3, 3, 1, 3)]:
+        assert lib.sgh_conv_geom_init(C.byref(g), 2, 3, H, H, 4, R, R, s, s, p, p) == 0
+        assert (g.P, g.Q) == (P, P)
+    assert lib.sgh_conv_geom_init(C.byref(g), 2, 3, 2, 2, 4, 5, 5, 1, 1, 0, 0) == -1  # kernel larger than padded input
+    assert lib.sgh_conv_geom_init(C.byref(g), 0, 3, 8, 8, 4, 3, 3, 1, 1, 0, 0) == -1
+    assert lib.sgh_conv_geom_init(None, 1, 3, 8, 8, 4, 3, 3, 1, 1, 0, 0) == -1
+
+
+def test_workspace_sizes():
+    lib = _lib.lib()
+    g = _lib.ConvGeom()
+    assert lib.sgh_conv_geom_init(C.byref(g), 64, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1) == 0
+    assert lib.sgh_conv_workspace_bytes(C.byref(g), _lib.SGH_CONV_DGRAD) == 9 * 64 * 64 * 4
+    assert lib.sgh_conv_workspace_bytes(C.byref(g), _lib.SGH_CONV_FWD) == 9 * 64 * 64 * 4
+    w = lib.sgh_conv_workspace_bytes(C.byref(g), _lib.SGH_CONV_WGRAD)
+    assert w % (64 * 64 * 9 * 4) == 0  # whole split-K partial copies of dW
+    assert lib.sgh_bn_workspace_bytes(64, 64, 56 * 56) >= 64 * 2 * 4
+    assert lib.sgh_bn_workspace_bytes(0, 64, 49) == 0
+
+
+def test_pool_geometry():
+    lib = _lib.lib()
+    g = _lib.PoolGeom()
+    assert lib.sgh_pool_geom_init(C.byref(g), 64, 64, 112, 112, 3, 3, 2, 2, 1, 1, 1) == 0
+    assert (g.P, g.Q) == (56, 56)
+    assert lib.sgh_pool_geom_init(C.byref(g), 64, 64, 7, 7, 7, 7, 1, 1, 0, 0, 0) == 0
+    assert (g.P, g.Q) == (1, 1)
+    # a pad as large as the kernel would make windows that see no input
+    assert lib.sgh_pool_geom_init(C.byref(g), 1, 1, 4, 4, 2, 2, 1, 1, 2, 2, 1) == -1
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(_lib.SingaHipError):
+        _lib.load(str(tmp_path / "nope.so"))

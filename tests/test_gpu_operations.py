@@ -1,0 +1,271 @@
+"""GPU parity: operation entry points (conv dgrad/wgrad/bias-grad, BatchNorm, pooling) against
+the CPU oracle, through the C ABI.
+
+Tolerances: max-pool routing and average pooling are bit-exact; conv and BatchNorm reductions
+are compared with the normalised L2 error ||gpu - cpu|| / ||cpu|| <= 1e-3 (fp32), the bound the
+task states for reductions whose summation order differs from the CPU's by construction."""
+import numpy as np
+import pytest
+
+from oracle import cpu_oracle as O
+from util import assert_bit_equal, nl2, randn, rng
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3   # stated bound; the observed error is printed and is typically < 1e-6
+
+
+@pytest.fixture(scope="module")
+def singa():
+    from singa_amd import singa_wrap
+    return singa_wrap
+
+
+def run_conv(singa, dev, x, w, b, dy, stride, pad):
+    N, C, H, W = x.shape
+    K, _, R, S = w.shape
+    xd, wd, dyd = singa.from_numpy(x, dev), singa.from_numpy(w, dev), singa.from_numpy(dy, dev)
+    h = singa.CudnnConvHandle(xd, (R, S), stride, pad, C, K, b is not None)
+    dx = singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy()
+    dw = singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy()
+    db = singa.GpuConvBackwardb(dyd, singa.from_numpy(b, dev), h).to_numpy() if b is not None else None
+    return h, dx, dw, db
+
+
+def test_conv_reference_vector(singa, dev, golden):
+    g = golden["conv"]
+    x = np.array(g["x"], np.float32).reshape(g["x_shape"])
+    w = np.array(g["w"], np.float32).reshape(g["w_shape"])
+    b = np.array(g["bias"], np.float32)
+    dy = np.array(g["dy"], np.float32).reshape(g["dy_shape"])
+    xd, wd, bd = singa.from_numpy(x, dev), singa.from_numpy(w, dev), singa.from_numpy(b, dev)
+    h = singa.CudnnConvHandle(xd, (3, 3), g["stride"], g["pad"], 1, 1, True)
+    assert (h.conv_height, h.conv_width, h.col_height, h.col_width) == (2, 2, 9, 4)
+    y = singa.GpuConvForward(xd, wd, bd, h).to_numpy()
+    np.testing.assert_allclose(y.ravel(), np.array(g["y"], np.float32), rtol=1e-6)
+    _, dx, dw, db = run_conv(singa, dev, x, w, b, dy, g["stride"], g["pad"])
+    dyf, wf, xf = dy.ravel(), w.ravel(), x.ravel()
+    for i, terms in enumerate(g["dx_terms"]):
+        np.testing.assert_allclose(dx.ravel()[i], sum(float(dyf[a]) * float(wf[c]) for a, c in terms), rtol=1e-6, atol=1e-7)
+    for i, terms in enumerate(g["dw_terms"]):
+        np.testing.assert_allclose(dw.ravel()[i], sum(float(dyf[a]) * float(xf[c]) for a, c in terms), rtol=1e-6)
+    np.testing.assert_allclose(db[0], float(dyf.sum()), rtol=1e-6)
+
+
+CONV_CASES = [
+    # N, C, H, W, K, R, S, stride, pad, bias
+    (2, 3, 7, 6, 4, 3, 3, (1, 1), (1, 1), True),
+    (2, 3, 9, 8, 5, 3, 3, (2, 2), (1, 1), False),
+    (2, 2, 6, 7, 3, 3, 2, (2, 1), (0, 1), True),          # non-square kernel / stride / pad
+    (3, 16, 8, 8, 32, 1, 1, (2, 2), (0, 0), False),       # 1x1 stride-2 downsample
+    (2, 3, 32, 32, 32, 5, 5, (1, 1), (2, 2), True),       # small-CNN conv1
+    (2, 32, 16, 16, 64, 5, 5, (1, 1), (2, 2), True),      # small-CNN conv2
+    (2, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3), False),      # ResNet stem (reduced image)
+    (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), False),     # stage-1 class
+    (2, 64, 14, 14, 128, 3, 3, (2, 2), (1, 1), False),    # stage transition
+    (2, 128, 7, 7, 128, 3, 3, (1, 1), (1, 1), False),     # odd spatial size
+    (1, 130, 9, 9, 70, 3, 3, (1, 1), (1, 1), False),      # channel counts that are not tile multiples
+    (4, 8, 5, 5, 8, 3, 3, (1, 1), (0, 0), False),         # no padding
+    (1, 1, 3, 3, 1, 3, 3, (1, 1), (2, 2), False),         # pad wider than half the kernel
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv_backward_vs_oracle(singa, dev, case):
+    N, C, H, W, K, R, S, stride, pad, bias = case
+    r = rng(abs(hash(case)) % 2**31)
+    x = randn(r, N, C, H, W)
+    w = (randn(r, K, C, R, S) * np.sqrt(2.0 / (C * R * S))).astype(np.float32)
+    b = randn(r, K) if bias else None
+    P, Q = (H + 2 * pad[0] - R) // stride[0] + 1, (W + 2 * pad[1] - S) // stride[1] + 1
+    dy = randn(r, N, K, P, Q)
+    h, dx, dw, db = run_conv(singa, dev, x, w, b, dy, stride, pad)
+    dx_o, dw_o = O.conv_bwd(dy, x, w, stride, pad)
+    e_dx, e_dw = nl2(dx, dx_o), nl2(dw, dw_o)
+    print("dgrad nl2 %.2e  wgrad nl2 %.2e" % (e_dx, e_dw))
+    assert e_dx < TOL and e_dw < TOL
+    if bias:
+        assert nl2(db, O.conv_bgrad(dy)) < TOL
+    # forward, which produces the activations the backward consumes
+    xd, wd = singa.from_numpy(x, dev), singa.from_numpy(w, dev)
+    y = singa.GpuConvForward(xd, wd, singa.from_numpy(b, dev) if bias else None, h).to_numpy()
+    assert nl2(y, O.conv_fwd(x, w, b, stride, pad)) < TOL
+
+
+def test_conv_wgrad_is_deterministic(singa, dev):
+    r = rng(4)
+    x, dy = randn(r, 8, 64, 28, 28), randn(r, 8, 64, 28, 28)
+    w = randn(r, 64, 64, 3, 3)
+    xd, wd, dyd = singa.from_numpy(x, dev), singa.from_numpy(w, dev), singa.from_numpy(dy, dev)
+    h = singa.CudnnConvHandle(xd, (3, 3), (1, 1), (1, 1), 64, 64, False)
+    a = singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy()
+    for _ in range(3):
+        assert_bit_equal(singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy(), a, "split-K reduction order")
+
+
+def test_conv_full_size_properties(singa, dev):
+    """BASELINE single-conv configuration (N64 C64 56x56 K64 3x3 s1 p1): too large for the CPU
+    oracle inside a test, so parity is checked through size-independent properties:
+    adjointness <conv(x,W),dy> = <x,dgrad(dy,W)> = <W,wgrad(dy,x)>, linearity in dy, and the
+    oracle on one image of the batch (dgrad is per-image; wgrad of a 1-image batch)."""
+    r = rng(2024)
+    N, C, H, K = 64, 64, 56, 64
+    x, dy = randn(r, N, C, H, H), randn(r, N, K, H, H)
+    w = (randn(r, K, C, 3, 3) * np.sqrt(2.0 / 576)).astype(np.float32)
+    xd, wd, dyd = singa.from_numpy(x, dev), singa.from_numpy(w, dev), singa.from_numpy(dy, dev)
+    h = singa.CudnnConvHandle(xd, (3, 3), (1, 1), (1, 1), C, K, True)
+    y = singa.GpuConvForward(xd, wd, None, h).to_numpy().astype(np.float64)
+    dx = singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy()
+    dw = singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy()
+    db = singa.GpuConvBackwardb(dyd, singa.from_numpy(np.zeros(K, np.float32), dev), h).to_numpy()
+    lhs = float((y * dy).sum())
+    assert abs(lhs - float((x.astype(np.float64) * dx).sum())) < 1e-4 * abs(lhs)
+    assert abs(lhs - float((w.astype(np.float64) * dw).sum())) < 1e-4 * abs(lhs)
+    np.testing.assert_allclose(db, dy.astype(np.float64).sum(axis=(0, 2, 3)), rtol=1e-4, atol=1e-2)
+    # oracle on image 5 (dgrad) and on a 2-image sub-batch (wgrad is additive over images)
+    dx5, _ = O.conv_bwd(dy[5:6], x[5:6], w, (1, 1), (1, 1), want_dw=False)
+    assert nl2(dx[5:6], dx5) < TOL
+    dys = dy.copy()
+    dys[2:] = 0
+    dw2 = singa.GpuConvBackwardW(singa.from_numpy(dys, dev), xd, wd, h).to_numpy()
+    _, dw2_o = O.conv_bwd(dy[:2], x[:2], w, (1, 1), (1, 1), want_dx=False)
+    assert nl2(dw2, dw2_o) < TOL
+    # linearity: dgrad(2*dy) == 2*dgrad(dy) exactly (scaling by a power of two)
+    dx2 = singa.GpuConvBackwardx(singa.from_numpy(dy * 2, dev), wd, xd, h).to_numpy()
+    assert_bit_equal(dx2, dx * 2, "dgrad linearity")
+
+
+def test_conv_argument_checks(singa, dev):
+    x = singa.from_numpy(np.zeros((2, 3, 8, 8), np.float32), dev)
+    with pytest.raises(singa.SingaHipError):
+        singa.CudnnConvHandle(x, (3, 3), (1, 1), (1, 1), 4, 8, False)  # channel mismatch
+    h = singa.CudnnConvHandle(x, (3, 3), (1, 1), (1, 1), 3, 8, False)
+    w = singa.from_numpy(np.zeros((8, 3, 3, 3), np.float32), dev)
+    with pytest.raises(singa.SingaHipError):
+        singa.GpuConvBackwardx(singa.from_numpy(np.zeros((2, 8, 7, 7), np.float32), dev), w, x, h)
+
+
+# ---------------------------------------------------------------------------------- pooling
+
+POOL_CASES = [
+    # N, C, H, W, kernel, stride, pad
+    (2, 3, 8, 8, (2, 2), (2, 2), (0, 0)),
+    (2, 4, 17, 17, (3, 3), (2, 2), (1, 1)),
+    (4, 64, 112, 112, (3, 3), (2, 2), (1, 1)),   # ResNet stem max-pool geometry (reduced batch)
+    (8, 32, 32, 32, (2, 2), (2, 2), (0, 0)),     # small-CNN pool 1
+    (1, 2, 7, 5, (3, 2), (1, 2), (1, 0)),
+    (2, 2, 6, 6, (2, 2), (3, 3), (0, 0)),        # stride > kernel: inputs outside every window
+    (4, 512, 7, 7, (7, 7), (1, 1), (0, 0)),      # ResNet global pool geometry
+]
+
+
+def test_pool_reference_vectors(singa, dev, golden):
+    g = golden["pool_max"]
+    x = np.array(g["x"], np.float32).reshape(g["x_shape"])
+    dy = np.array(g["dy"], np.float32).reshape(g["dy_shape"])
+    xd = singa.from_numpy(x, dev)
+    h = singa.CudnnPoolingHandle(xd, g["kernel"], g["stride"], g["pad"], True)
+    y = singa.GpuPoolingForward(h, xd)
+    assert y.to_numpy().ravel().tolist() == g["y"]
+    dx = singa.GpuPoolingBackward(h, singa.from_numpy(dy, dev), xd, y).to_numpy()
+    assert_bit_equal(dx.ravel(), np.array(g["dx"], np.float32), "test_pooling.cc vector")
+    g = golden["pool_api"]
+    x = np.array(g["x"], np.float32).reshape(g["x_shape"])
+    dy = np.array(g["dy"], np.float32).reshape(g["dy_shape"])
+    xd, dyd = singa.from_numpy(x, dev), singa.from_numpy(dy, dev)
+    for is_max, ky, kdx in ((True, "max_y", "max_dx"), (False, "avg_y", "avg_dx")):
+        h = singa.CudnnPoolingHandle(xd, g["kernel"], g["stride"], g["pad"], is_max)
+        y = singa.GpuPoolingForward(h, xd)
+        assert_bit_equal(y.to_numpy().ravel(), np.array(g[ky], np.float32), ky)
+        assert_bit_equal(singa.GpuPoolingBackward(h, dyd, xd, y).to_numpy().ravel(), np.array(g[kdx], np.float32), kdx)
+
+
+@pytest.mark.parametrize("case", POOL_CASES)
+@pytest.mark.parametrize("ties", [False, True])
+def test_max_pool_bit_exact(singa, dev, case, ties):
+    N, C, H, W, kernel, stride, pad = case
+    r = rng(H * 31 + W)
+    x = randn(r, N, C, H, W)
+    if ties:
+        x = np.round(x * 2).astype(np.float32)  # heavy ties: first maximum in row-major order wins
+    y_o, mask = O.pool_max_fwd(x, kernel, stride, pad)
+    dy = randn(r, *y_o.shape)
+    xd = singa.from_numpy(x, dev)
+    h = singa.CudnnPoolingHandle(xd, kernel, stride, pad, True)
+    y = singa.GpuPoolingForward(h, xd)
+    assert_bit_equal(y.to_numpy(), y_o, "max-pool forward")
+    dx = singa.GpuPoolingBackward(h, singa.from_numpy(dy, dev), xd, y).to_numpy()
+    assert_bit_equal(dx, O.pool_max_bwd(dy, mask, x.shape), "max-pool routing")
+
+
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_avg_pool_bit_exact(singa, dev, case):
+    N, C, H, W, kernel, stride, pad = case
+    r = rng(H * 37 + W)
+    x = randn(r, N, C, H, W)
+    xd = singa.from_numpy(x, dev)
+    h = singa.CudnnPoolingHandle(xd, kernel, stride, pad, False)
+    y = singa.GpuPoolingForward(h, xd)
+    y_o = O.pool_avg_fwd(x, kernel, stride, pad, include_pad=False)
+    assert nl2(y.to_numpy(), y_o) < 1e-6  # forward sums the window in the same order; division is IEEE
+    dy = randn(r, *y_o.shape)
+    dx = singa.GpuPoolingBackward(h, singa.from_numpy(dy, dev), xd, y).to_numpy()
+    assert_bit_equal(dx, O.pool_avg_bwd(dy, x.shape, kernel, stride, pad, include_pad=False), "avg-pool backward")
+
+
+# ---------------------------------------------------------------------------------- batch norm
+
+def test_bn_reference_vectors(singa, dev, golden):
+    g = golden["bn_cudnn"]
+    x = np.array(g["x"], np.float32).reshape(g["x_shape"])
+    dy = np.array(g["dy"], np.float32).reshape(g["x_shape"])
+    xd = singa.from_numpy(x, dev)
+    h = singa.CudnnBatchNormHandle(0.9, xd)
+    gamma, beta = singa.from_numpy(np.ones(2, np.float32), dev), singa.from_numpy(np.zeros(2, np.float32), dev)
+    rm, rv = singa.from_numpy(np.zeros(2, np.float32), dev), singa.from_numpy(np.zeros(2, np.float32), dev)
+    y, mean, var = singa.GpuBatchNormForwardTraining(h, xd, gamma, beta, rm, rv)
+    np.testing.assert_allclose(y.to_numpy().ravel(), np.array(g["y"], np.float32), atol=g["tol"])
+    dx, ds, db = singa.GpuBatchNormBackward(h, singa.from_numpy(dy, dev), xd, gamma, mean, var)
+    np.testing.assert_allclose(dx.to_numpy().ravel(), np.array(g["dx"], np.float32), atol=g["tol"])
+    np.testing.assert_allclose(ds.to_numpy(), np.array(g["dgamma"], np.float32), atol=g["tol"])
+    np.testing.assert_allclose(db.to_numpy(), np.array(g["dbeta"], np.float32), atol=g["tol"])
+    g = golden["bn_api"]
+    x = np.array(g["x"], np.float32).reshape(g["x_shape"])
+    xd = singa.from_numpy(x, dev)
+    h = singa.CudnnBatchNormHandle(0.1, xd)
+    gamma, beta = singa.from_numpy(np.ones(3, np.float32), dev), singa.from_numpy(np.zeros(3, np.float32), dev)
+    y, mean, var = singa.GpuBatchNormForwardTraining(h, xd, gamma, beta, None, None)
+    dx, _, _ = singa.GpuBatchNormBackward(h, xd, xd, gamma, mean, var)
+    np.testing.assert_allclose(dx.to_numpy().ravel(), np.array(g["dx"], np.float32), atol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 56, 56), (64, 512, 7, 7), (16, 128, 28, 28),
+                                   (2, 64, 112, 112), (32, 10)])
+def test_bn_vs_oracle(singa, dev, shape):
+    r = rng(sum(shape))
+    x = (randn(r, *shape) * 2 + 0.5).astype(np.float32)
+    dy = randn(r, *shape)
+    C = shape[1]
+    gamma, beta = (randn(r, C) * 0.2 + 1).astype(np.float32), randn(r, C)
+    rm, rv = randn(r, C), np.abs(randn(r, C))
+    rm_o, rv_o = rm.copy(), rv.copy()
+    y_o, mean_o, inv_o = O.bn_fwd_train(x, gamma, beta, rm_o, rv_o, factor=0.9)
+    dx_o, dg_o, db_o = O.bn_bwd(dy, x, gamma, mean_o, inv_o)
+    xd, gd, bd = singa.from_numpy(x, dev), singa.from_numpy(gamma, dev), singa.from_numpy(beta, dev)
+    rmd, rvd = singa.from_numpy(rm, dev), singa.from_numpy(rv, dev)
+    h = singa.CudnnBatchNormHandle(0.9, xd)
+    y, mean, var = singa.GpuBatchNormForwardTraining(h, xd, gd, bd, rmd, rvd)
+    assert nl2(y.to_numpy(), y_o) < TOL
+    assert nl2(mean.to_numpy(), mean_o) < 1e-4 and nl2(var.to_numpy(), inv_o) < 1e-4
+    assert nl2(rmd.to_numpy(), rm_o) < 1e-4 and nl2(rvd.to_numpy(), rv_o) < 1e-4
+    # backward fed with the ORACLE's saved statistics, so only the backward kernel is under test
+    dx, ds, db = singa.GpuBatchNormBackward(h, singa.from_numpy(dy, dev), xd, gd, singa.from_numpy(mean_o, dev),
+                                            singa.from_numpy(inv_o, dev))
+    e = (nl2(dx.to_numpy(), dx_o), nl2(ds.to_numpy(), dg_o), nl2(db.to_numpy(), db_o))
+    print("bn bwd nl2 dx %.2e dgamma %.2e dbeta %.2e" % e)
+    assert max(e) < TOL
+    # run-to-run identical
+    dx2, ds2, db2 = singa.GpuBatchNormBackward(h, singa.from_numpy(dy, dev), xd, gd, singa.from_numpy(mean_o, dev),
+                                               singa.from_numpy(inv_o, dev))
+    assert_bit_equal(dx2.to_numpy(), dx.to_numpy())
+    assert_bit_equal(ds2.to_numpy(), ds.to_numpy())

@@ -1,0 +1,216 @@
+"""GPU parity: tensor_math backward ops and the SGD update against the CPU oracle, through the
+C ABI (singa_amd.singa_wrap -> ctypes -> libsinga_hip.so).
+
+Tolerances: elementwise ops are compared bit for bit where the arithmetic is a single rounding
+per op (ReLU, Add, Mult, softmax-CE backward, Axpy and SGD with contraction off); where a
+library routine may legitimately round differently the bound is max relative error 1e-5."""
+import numpy as np
+import pytest
+
+from oracle import cpu_oracle as O
+from util import assert_bit_equal, max_rel_err, nl2, randn, rng
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [0, 1, 3, 4, 5, 255, 256, 1027, 4096, 100003, 1 << 20]
+
+
+@pytest.fixture(scope="module")
+def singa():
+    from singa_amd import singa_wrap
+    return singa_wrap
+
+
+def test_relu_reference_vector(singa, dev, golden):
+    g = golden["relu"]
+    x = singa.from_numpy(np.array(g["x"], np.float32).reshape(g["x_shape"]), dev)
+    dy = singa.from_numpy(np.array(g["dy"], np.float32).reshape(g["x_shape"]), dev)
+    assert singa.ReLU(x).to_numpy().ravel().tolist() == [np.float32(v) for v in g["y"]]
+    assert singa.ReLUBackward(dy, x).to_numpy().ravel().tolist() == g["dx"]
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_relu_backward(singa, dev, n):
+    r = rng(n + 1)
+    x, dy = randn(r, n), randn(r, n)
+    if n > 8:
+        x[::7] = 0.0      # gradient at exactly zero is zero
+        x[3::11] = -0.0
+    dx = singa.ReLUBackward(singa.from_numpy(dy, dev), singa.from_numpy(x, dev)).to_numpy()
+    assert_bit_equal(dx, O.relu_bwd(dy, x), "relu_bwd n=%d" % n)
+
+
+def test_relu_backward_stage1_shape_and_unaligned(singa, dev):
+    r = rng(99)
+    shape = (8, 64, 56, 56)
+    x, dy = randn(r, *shape), randn(r, *shape)
+    dx = singa.ReLUBackward(singa.from_numpy(dy, dev), singa.from_numpy(x, dev)).to_numpy()
+    assert_bit_equal(dx, O.relu_bwd(dy, x), "relu_bwd 4-D")
+    # pointers that are not 16-byte aligned take the scalar path
+    big = singa.from_numpy(np.concatenate([[0], x.ravel()[:1001]]).astype(np.float32), dev)
+    bigdy = singa.from_numpy(np.concatenate([[0], dy.ravel()[:1001]]).astype(np.float32), dev)
+    xs = singa.from_device_pointer(big.ptr + 4, (1001,), dev, keepalive=big)
+    dys = singa.from_device_pointer(bigdy.ptr + 4, (1001,), dev, keepalive=bigdy)
+    assert_bit_equal(singa.ReLUBackward(dys, xs).to_numpy(), O.relu_bwd(dy.ravel()[:1001], x.ravel()[:1001]), "unaligned")
+
+
+def test_softmax_ce_reference_vector(singa, dev, golden):
+    g = golden["softmax_ce"]
+    p = singa.SoftMax(singa.from_numpy(np.array(g["p"], np.float32).reshape(g["p_shape"]), dev))
+    for t in (np.array(g["t_index"], np.int32), np.array(g["t_onehot"], np.int32).reshape(2, 4)):
+        tt = singa.from_numpy(t, dev)
+        np.testing.assert_allclose(singa.CrossEntropyFwd(p, tt).to_numpy(), np.float32(-np.log(0.25)), rtol=4e-7)
+        np.testing.assert_allclose(singa.SoftmaxCrossEntropyBwd(p, tt).to_numpy().ravel(),
+                                   np.array(g["grad"], np.float32), rtol=4e-7)
+
+
+@pytest.mark.parametrize("batch,dim", [(1, 1), (2, 4), (128, 10), (64, 1000), (7, 1025), (3, 70001)])
+def test_softmax_ce_backward_bit_exact(singa, dev, batch, dim):
+    r = rng(batch * 131 + dim)
+    p = O.softmax(randn(r, batch, dim) * 3)
+    t = r.integers(0, dim, size=batch).astype(np.int32)
+    pd = singa.from_numpy(p, dev)
+    g = singa.SoftmaxCrossEntropyBwd(pd, singa.from_numpy(t, dev)).to_numpy()
+    assert_bit_equal(g, O.softmax_ce_bwd(p, t), "index target")
+    assert_bit_equal(pd.to_numpy(), p, "p must not be modified")
+    # fused /N (multiply by the fp32 reciprocal like the reference's Div)
+    scale = float(np.float32(1.0) / np.float32(batch))
+    g = singa.SoftmaxCrossEntropyBwd(pd, singa.from_numpy(t, dev), scale=scale).to_numpy()
+    assert_bit_equal(g, O.softmax_ce_bwd(p, t, div_by=batch), "index target, /N")
+    if dim <= 1025:
+        multi = np.eye(dim, dtype=np.int32)[t]
+        multi[:, 0] += 2
+        g = singa.SoftmaxCrossEntropyBwd(pd, singa.from_numpy(multi, dev)).to_numpy()
+        assert_bit_equal(g, O.softmax_ce_bwd(p, multi), "array target")
+
+
+def test_softmax_ce_label_edges(singa, dev):
+    p = O.softmax(randn(rng(5), 4, 6))
+    t = np.array([0, 5, 5, 0], np.int32)  # first and last class
+    g = singa.SoftmaxCrossEntropyBwd(singa.from_numpy(p, dev), singa.from_numpy(t, dev)).to_numpy()
+    assert_bit_equal(g, O.softmax_ce_bwd(p, t))
+    assert singa.LabelErrors(dev) == 0
+    bad = np.array([0, 6, -1, 1], np.int32)  # out of range: row left as p, error counted
+    g = singa.SoftmaxCrossEntropyBwd(singa.from_numpy(p, dev), singa.from_numpy(bad, dev)).to_numpy()
+    assert_bit_equal(g[1:3], p[1:3])
+    assert singa.LabelErrors(dev) == 2
+    assert singa.LabelErrors(dev) == 0
+
+
+def test_softmax_and_ce_forward(singa, dev):
+    r = rng(6)
+    x = randn(r, 64, 1000) * 5
+    p = singa.SoftMax(singa.from_numpy(x, dev))
+    assert max_rel_err(p.to_numpy(), O.softmax(x), floor=1e-12) < 1e-5
+    t = r.integers(0, 1000, size=64).astype(np.int32)
+    loss = singa.CrossEntropyFwd(p, singa.from_numpy(t, dev)).to_numpy()
+    assert max_rel_err(loss, O.cross_entropy_fwd(p.to_numpy(), t)) < 1e-5
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_axpy_mult_add(singa, dev, n):
+    r = rng(n + 17)
+    x, y = randn(r, n), randn(r, n)
+    yd = singa.from_numpy(y, dev)
+    singa.Axpy(0.37, singa.from_numpy(x, dev), yd)
+    exp = y.copy()
+    O.axpy(0.37, x, exp)
+    assert_bit_equal(yd.to_numpy(), exp, "Axpy scalar")
+    # Tensor alpha (1-element device tensor, as opt.SGD passes it)
+    alpha = singa.from_numpy(np.array([-0.05], np.float32), dev)
+    singa.Axpy(alpha, singa.from_numpy(x, dev), yd)
+    O.axpy(-0.05, x, exp)
+    assert_bit_equal(yd.to_numpy(), exp, "Axpy tensor alpha")
+    assert_bit_equal(singa.EltwiseMult(singa.from_numpy(x, dev), singa.from_numpy(y, dev)).to_numpy(),
+                     O.eltwise_mult(x, y), "EltwiseMult")
+    if n > 1:
+        buf = singa.from_numpy(x, dev)
+        buf *= singa.from_numpy(np.array([0.9], np.float32), dev)  # stride-0 broadcast of opt.py:299-300
+        assert_bit_equal(buf.to_numpy(), O.eltwise_mult(x, np.array([0.9], np.float32)), "buf *= mom")
+    acc = singa.from_numpy(x, dev)
+    acc += singa.from_numpy(y, dev)
+    assert_bit_equal(acc.to_numpy(), O.add(x, y), "+=")
+
+
+def test_sgd_reference_cases(singa, dev, golden):
+    from singa_amd import opt
+    g = golden["sgd"]
+    shape = tuple(g["shape"])
+    for c in g["cases"]:
+        sgd = opt.SGD(lr=c["lr"], momentum=c["mu"], weight_decay=c["wd"], nesterov=bool(c["nesterov"]))
+        w = singa.from_numpy(np.full(shape, c["w0"], np.float32), dev)
+        wo, vo = np.full(shape, c["w0"], np.float32), np.zeros(shape, np.float32)
+        for _ in range(c["steps"]):
+            grad = np.full(shape, c["g"], np.float32)
+            sgd.apply("w", w, singa.from_numpy(grad, dev))
+            sgd.step()
+            O.sgd_momentum(wo, grad, vo, c["lr"], mu=c["mu"], wd=c["wd"], nesterov=bool(c["nesterov"]))
+            assert_bit_equal(w.to_numpy(), wo, c["name"])
+
+
+@pytest.mark.parametrize("n", [1, 5, 4096, 100003, 2359296])
+@pytest.mark.parametrize("cfg", [(0.05, 0.9, 0.0, 0.0, False), (0.1, 0.9, 0.1, 1e-4, False), (0.01, 0.8, 0.0, 5e-4, True),
+                                 (0.05, 0.0, 0.0, 0.0, False)])
+def test_sgd_momentum_fused(singa, dev, n, cfg):
+    lr, mu, damp, wd, nesterov = cfg
+    from singa_amd import opt
+    r = rng(n)
+    p, v = randn(r, n), randn(r, n)
+    sgd = opt.SGD(lr=lr, momentum=mu, dampening=damp, weight_decay=wd, nesterov=nesterov)
+    pd = singa.from_numpy(p, dev)
+    if mu != 0:
+        sgd.moments["p"] = singa.from_numpy(v, dev)
+    for step in range(2):
+        g = randn(r, n)
+        sgd.apply("p", pd, singa.from_numpy(g, dev))
+        O.sgd_momentum(p, g, v, lr, mu=mu, damp=damp, wd=wd, nesterov=nesterov)
+    assert_bit_equal(pd.to_numpy(), p, "p")
+    if mu != 0:
+        assert_bit_equal(sgd.moments["p"].to_numpy(), v, "v")
+
+
+def test_sgd_multi_tensor_matches_per_tensor(singa, dev):
+    from singa_amd import opt
+    r = rng(77)
+    sizes = [1, 7, 64, 1000, 2048, 4099, 36864, 147456, 10]
+    ps = [randn(r, n) for n in sizes]
+    gs = [randn(r, n) for n in sizes]
+    a = opt.SGD(lr=0.05, momentum=0.9)
+    b = opt.SGD(lr=0.05, momentum=0.9)
+    pa = [singa.from_numpy(p, dev) for p in ps]
+    pb = [singa.from_numpy(p, dev) for p in ps]
+    for step in range(2):
+        for i, n in enumerate(sizes):
+            a.apply("p%d" % i, pa[i], singa.from_numpy(gs[i], dev))
+        b.apply_all([("p%d" % i, pb[i], singa.from_numpy(gs[i], dev)) for i in range(len(sizes))])
+    for i in range(len(sizes)):
+        assert_bit_equal(pa[i].to_numpy(), pb[i].to_numpy(), "multi p%d" % i)
+        assert_bit_equal(a.moments["p%d" % i].to_numpy(), b.moments["p%d" % i].to_numpy(), "multi v%d" % i)
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 784, 1000), (128, 1000, 10), (64, 512, 1000), (1, 1, 1), (65, 129, 33),
+                                   (300, 260, 515)])
+def test_linear_backward_gemms(singa, dev, M, N, K):
+    """Matmul.backward: dx = dy * W^T, dW = x^T * dy (python/singa/autograd.py:613-623)."""
+    r = rng(M + N + K)
+    x, W, dy = randn(r, M, N), randn(r, N, K), randn(r, M, K)
+    xd, Wd, dyd = (singa.from_numpy(a, dev) for a in (x, W, dy))
+    dx = singa.Mult(dyd, singa.DefaultTranspose(Wd)).to_numpy()
+    dW = singa.Mult(singa.DefaultTranspose(xd), dyd).to_numpy()
+    y = singa.Mult(xd, Wd).to_numpy()
+    assert nl2(dx, O.sgemm(dy, W, transB=True)) < 1e-5
+    assert nl2(dW, O.sgemm(x, dy, transA=True)) < 1e-5
+    assert nl2(y, O.sgemm(x, W)) < 1e-5
+    tt = singa.Mult(singa.DefaultTranspose(xd), singa.DefaultTranspose(singa.from_numpy(randn(r, K, M), dev)))
+    assert tt.shape() == [N, K]
+    db = singa.Sum(dyd, 0).to_numpy()
+    assert max_rel_err(db, O.sum_rows(dy), floor=1e-3) < 1e-5
+
+
+def test_pool_reuses_freed_blocks(singa, dev):
+    before = dev.PoolStats()["driver_allocs"]
+    for _ in range(20):
+        t = singa.Tensor((1 << 16,), dev)
+        t.SetFloatValue(1.0)
+        del t
+    assert dev.PoolStats()["driver_allocs"] - before <= 1
