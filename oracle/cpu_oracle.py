@@ -136,7 +136,7 @@ def cross_entropy_fwd(p, t):
     rc = lib().oracle_cross_entropy_fwd(pp, pt, C.c_int(t.size == batch), C.c_size_t(batch),
                                         C.c_size_t(p.size // batch), pl)
     if rc != 0:
-        raise ValueError("negative label")
+        raise ValueError("label out of range (rc=%d)" % rc)
     return loss
 
 
@@ -148,7 +148,7 @@ def softmax_ce_bwd(p, t, div_by=None):
     rc = lib().oracle_softmax_ce_bwd(g.ctypes.data_as(C.c_void_p), pt, C.c_int(t.size == batch),
                                      C.c_size_t(batch), C.c_size_t(g.size // batch))
     if rc != 0:
-        raise ValueError("negative label")
+        raise ValueError("label out of range (rc=%d)" % rc)
     if div_by is not None:
         lib().oracle_div_scalar(g.ctypes.data_as(C.c_void_p), C.c_float(div_by), C.c_size_t(g.size))
     return g

@@ -240,7 +240,7 @@ ORACLE_API void oracle_softmax(const float *x, float *p, size_t batch, size_t di
 }
 
 /* ComputeCrossEntropy<float, lang::Cpp>, src/core/tensor/tensor_math_cpp.h:1058-1088.
- * Returns -1 if a label is negative (the reference CHECK_GE aborts).
+ * Returns -1 if a label is negative (the reference CHECK_GE aborts), -2 if it is >= dim.
  * Pinned by test/singa/test_cross_entropy.cc:43-71. */
 ORACLE_API int oracle_cross_entropy_fwd(const float *p, const int *t, int int_target, size_t batch,
                                         size_t dim, float *loss) {
@@ -248,6 +248,7 @@ ORACLE_API int oracle_cross_entropy_fwd(const float *p, const int *t, int int_ta
     for (size_t i = 0; i < batch; ++i) {
       int k = t[i];
       if (k < 0) return -1;
+      if ((size_t)k >= dim) return -2; /* the reference reads out of bounds here; the oracle refuses */
       float pr = p[i * dim + k];
       loss[i] = -logf(pr > FLT_MIN ? pr : FLT_MIN);
     }
@@ -268,16 +269,17 @@ ORACLE_API int oracle_cross_entropy_fwd(const float *p, const int *t, int int_ta
 
 /* SoftmaxCrossEntropyBwd<float, lang::Cpp>, src/core/tensor/tensor_math_cpp.h:1090-1119,
  * in place on grad (which the caller pre-fills with p: src/core/tensor/tensor.cc:1717-1721).
- * The target is read as int32 in both modes.  Returns -1 on a negative label.
+ * The target is read as int32 in both modes.  Returns -1 on a negative label, -2 on one >= dim.
+ * All labels are validated before anything is written.
  * Pinned by test/singa/test_cross_entropy.cc:73-111. */
 ORACLE_API int oracle_softmax_ce_bwd(float *grad, const int *t, int int_target, size_t batch,
                                      size_t dim) {
   if (int_target) {
     for (size_t i = 0; i < batch; ++i) {
-      int k = t[i];
-      if (k < 0) return -1;
-      grad[i * dim + k] -= 1.0f;
+      if (t[i] < 0) return -1;
+      if ((size_t)t[i] >= dim) return -2; /* the reference writes out of bounds here; the oracle refuses */
     }
+    for (size_t i = 0; i < batch; ++i) grad[i * dim + t[i]] -= 1.0f;
   } else {
     for (size_t i = 0; i < batch; ++i) {
       float sum = 0.f;

@@ -72,6 +72,8 @@ def test_negative_label_is_rejected():
     p = np.full((2, 4), 0.25, dtype=np.float32)
     with pytest.raises(ValueError):
         O.softmax_ce_bwd(p, np.array([0, -1], dtype=np.int32))
+    with pytest.raises(ValueError):
+        O.softmax_ce_bwd(p, np.array([4, 0], dtype=np.int32))
 
 
 def test_bn_forward_cudnn_vector(golden):
