@@ -1,0 +1,145 @@
+#!/usr/bin/env python3
+"""Benchmark of the backward pass + SGD-momentum update on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): ResNet-18, N=64, 3x224x224, fp32,
+BatchNorm in training mode, 1000-class softmax cross-entropy, SGD momentum 0.9 -- the graph of the
+reference's examples/cnn/model/resnet.py.  One "step" = loss-gradient seed -> last parameter
+updated (every backward kernel in tape order plus the update of all 62 parameter tensors), on
+synthetic seeded inputs whose forward activations are already resident in HBM.
+
+Prints ONE JSON line: the whole-job images/s plus
+  roofline     -- the dominant kernel family (fp32 MFMA implicit-GEMM conv dgrad + wgrad):
+                  algorithmic FLOPs / measured kernel time (HIP events on the kernels' stream),
+                  against the MI355X fp32 matrix peak;
+  cpu_baseline -- the CPU oracle replaying the same tape on the host cores, on a bounded sample.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def collect_prof(lib):
+    n = C.c_int()
+    lib.sgh_prof_count(C.byref(n))
+    out = {}
+    buf = C.create_string_buffer(32)
+    for i in range(n.value):
+        ms, work = C.c_float(), C.c_double()
+        rc = lib.sgh_prof_get(i, buf, 32, C.byref(ms), C.byref(work))
+        if rc != 0:
+            raise RuntimeError("sgh_prof_get rc=%d" % rc)
+        d = out.setdefault(buf.value.decode(), {"launches": 0, "ms": 0.0, "flop": 0.0})
+        d["launches"] += 1
+        d["ms"] += ms.value
+        d["flop"] += work.value
+    return out
+
+
+def cpu_baseline(sample_batch):
+    """The CPU oracle (a restatement of SINGA's CppCPU algorithms) on the same tape, bounded."""
+    from oracle import cpu_oracle as O
+    from oracle.ops import OracleOps
+    from singa_amd import workloads as wl
+    ops = OracleOps()
+    net = wl.build("resnet18", ops)
+    x, labels = wl.make_inputs("resnet18", sample_batch)
+    net.forward(ops.from_numpy(x), ops.from_numpy(labels))
+    t0 = time.perf_counter()
+    net.backward_and_update()
+    dt = time.perf_counter() - t0
+    return {"value": round(sample_batch / dt, 3), "unit": "imgs/s", "cores": O.get_threads(), "kind": "port",
+            "sample": "one ResNet-18 backward+update step at batch %d (same graph and input distribution; "
+                      "%.1f s of CPU time)" % (sample_batch, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--config", default="resnet18")
+    ap.add_argument("--cpu-sample-batch", type=int, default=16)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--per-parameter-update", action="store_true",
+                    help="update each parameter right after its gradient (one launch each) instead of one fused launch")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch  # device synchronisation only; no torch op is on the measured path
+    from singa_amd import _lib
+    from singa_amd import singa_wrap as singa
+    from singa_amd import workloads as wl
+
+    lib = _lib.lib()
+    dev = singa.create_hip_gpu_on(0)
+    hip = wl.HipOps(dev)
+    net = wl.build(args.config, hip, lr=0.05, momentum=0.9)
+    x, labels = wl.make_inputs(args.config, args.batch)
+    net.forward(hip.from_numpy(x), hip.from_numpy(labels))
+    fused = not args.per_parameter_update
+
+    def sync():
+        dev.Sync()
+        torch.cuda.synchronize()
+
+    for _ in range(args.warmup):
+        net.backward_and_update(fused_update=fused)
+    sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        net.backward_and_update(fused_update=fused)
+    sync()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    imgs_per_s = args.batch * args.steps / elapsed
+
+    # kernel-level pass: every conv / GEMM launch bracketed by HIP events on the device stream
+    prof_steps = max(1, min(args.steps, 5))
+    lib.sgh_prof_enable(1)
+    for _ in range(prof_steps):
+        net.backward_and_update(fused_update=fused)
+    sync()
+    prof = collect_prof(lib)
+    lib.sgh_prof_enable(0)
+    conv = {k: prof[k] for k in ("conv_dgrad", "conv_wgrad") if k in prof}
+    flop = sum(v["flop"] for v in conv.values())
+    ms = sum(v["ms"] for v in conv.values())
+    launches = sum(v["launches"] for v in conv.values())
+    achieved = flop / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+    roofline = {
+        "bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+        "kernel": "k_igemm (fp32 MFMA implicit-GEMM conv dgrad + wgrad, %d launches/step)" % (launches // prof_steps),
+        "flop_per_step": flop / prof_steps, "kernel_ms_per_step": round(ms / prof_steps, 4),
+    }
+    for k, v in conv.items():
+        roofline[k + "_tflops"] = round(v["flop"] / (v["ms"] * 1e-3) / 1e12, 3) if v["ms"] > 0 else 0.0
+
+    out = {
+        "metric": "backward+update imgs/sec, ResNet-18 N=64 fp32", "value": round(imgs_per_s, 2), "unit": "imgs/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s backward+update, N=%d, 3x224x224, fp32, SGD momentum 0.9" % (args.config, args.batch),
+                   "update": "fused multi-tensor" if fused else "per parameter"},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

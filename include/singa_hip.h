@@ -88,6 +88,16 @@ SGH_API int sgh_event_record(sgh_event *ev, void *stream);
 /* Blocks on `stop`, then returns stop - start in milliseconds. */
 SGH_API int sgh_event_elapsed_ms(sgh_event *start, sgh_event *stop, float *ms);
 
+/* Kernel-level profiling: the per-node timing of SINGA's Graph (Device::SetVerbosity,
+ * TimeProfilingDoExec, Graph::PrintTimeProfiling: src/core/scheduler/scheduler.cc:240-295) at
+ * kernel granularity.  While enabled, every GEMM / implicit-GEMM launch of this library is
+ * bracketed by an event pair on its own stream and tagged ("conv_wgrad", "conv_dgrad",
+ * "conv_fwd", "gemm") with its algorithmic FLOP count.  sgh_prof_enable(1) clears old records.
+ * sgh_prof_get waits for record i to finish and returns its tag, duration and work. */
+SGH_API int sgh_prof_enable(int on);
+SGH_API int sgh_prof_count(int *n);
+SGH_API int sgh_prof_get(int i, char *tag, size_t tag_len, float *ms, double *work);
+
 /* =====================================================================================
  * tensor_math backward ops (HIP specialisations of src/core/tensor/tensor_math.h)
  * ===================================================================================== */

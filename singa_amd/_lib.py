@@ -53,6 +53,9 @@ SIGNATURES = {
     "sgh_event_destroy": (C.c_int, [vp]),
     "sgh_event_record": (C.c_int, [vp, vp]),
     "sgh_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
+    "sgh_prof_enable": (C.c_int, [C.c_int]),
+    "sgh_prof_count": (C.c_int, [C.POINTER(C.c_int)]),
+    "sgh_prof_get": (C.c_int, [C.c_int, C.c_char_p, sz, C.POINTER(C.c_float), C.POINTER(C.c_double)]),
     "sgh_relu_bwd_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_relu_fwd_f32": (C.c_int, [vp, vp, sz, vp]),
     "sgh_softmax_ce_bwd_f32": (C.c_int, [vp, vp, vp, sz, sz, C.c_int, C.c_float, vp]),

@@ -31,6 +31,11 @@ static inline bool sgh_aligned16(const void *p) { return (reinterpret_cast<uintp
 // Number of compute units of the current device (cached per process; one GPU per process).
 int sgh_num_cus();
 
+// Kernel-level profiling hooks (no-ops unless sgh_prof_enable(1) was called).
+bool sgh_prof_on();
+void sgh_prof_start(const char *tag, double work, hipStream_t s);
+void sgh_prof_stop(hipStream_t s);
+
 // Sum across the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float sgh_wave_sum(float v) {
 #pragma unroll

@@ -420,13 +420,20 @@ inline WgradPlan plan_wgrad(const sgh_conv_geom *g) {
 
 template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc>
 inline int launch_igemm(const LA &la, const LB &lb, const ST &st, int M, int N, int Ktotal, int splits,
-                        int chunks_per_split, hipStream_t stream) {
+                        int chunks_per_split, hipStream_t stream, const char *tag, double flops) {
   dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
   if (grid.y > 65535u || grid.z > 65535u) return SGH_EUNSUPPORTED;
+  sgh_prof_start(tag, flops, stream);
   hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc>), grid, dim3(NT), 0, stream, la, lb, st, Ktotal,
                      chunks_per_split);
+  sgh_prof_stop(stream);
   SGH_LAUNCH_CHECK();
   return SGH_OK;
+}
+
+// algorithmic FLOPs of one convolution pass: 2 * N * K * P * Q * C * R * S
+inline double conv_flops(const sgh_conv_geom *g) {
+  return 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S;
 }
 
 // ---- dense GEMM dispatch over the four transpose combinations and two tile sizes -----------
@@ -437,8 +444,8 @@ inline int gemm_tile(int M, int N, int K, float alpha, const float *A, long a_rs
   DenseLoader<BN, BKc> lb{B, b_rs, b_ks, N, K};
   DenseStore st{C, ldc, M, N, alpha, beta};
   const int chunks = (K + BK - 1) / BK;
-  return launch_igemm<BM, BN, DenseLoader<BM, AK>, DenseLoader<BN, BKc>, DenseStore, AK, BKc>(la, lb, st, M, N, K, 1,
-                                                                                               chunks, stream);
+  return launch_igemm<BM, BN, DenseLoader<BM, AK>, DenseLoader<BN, BKc>, DenseStore, AK, BKc>(
+      la, lb, st, M, N, K, 1, chunks, stream, "gemm", 2.0 * M * N * K);
 }
 
 template <bool AK, bool BKc>
@@ -514,12 +521,12 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
     DenseLoader<128, false> la{Wt, 1, long(g->C), M, Ktot};
     PixelGatherLoader<128, true> lb{dy, to_g(g), KP, g->K, g->P, g->Q, Ncols, 0, 0, 0, false};
     return launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_dgrad", conv_flops(g));
   }
   DenseLoader<64, false> la{Wt, 1, long(g->C), M, Ktot};
   PixelGatherLoader<128, true> lb{dy, to_g(g), KP, g->K, g->P, g->Q, Ncols, 0, 0, 0, false};
   return launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
-      la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+      la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_dgrad", conv_flops(g));
 }
 
 int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, const float *bias, float *y,
@@ -544,12 +551,12 @@ int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, con
     DenseLoader<128, false> la{Wt, 1, long(g->K), M, Ktot};
     PixelGatherLoader<128, false> lb{x, to_g(g), CP, g->C, g->H, g->W, Ncols, 0, 0, 0, false};
     return launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd", conv_flops(g));
   }
   DenseLoader<64, false> la{Wt, 1, long(g->K), M, Ktot};
   PixelGatherLoader<128, false> lb{x, to_g(g), CP, g->C, g->H, g->W, Ncols, 0, 0, 0, false};
   return launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
-      la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+      la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd", conv_flops(g));
 }
 
 int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
@@ -573,7 +580,7 @@ int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, 
     lb.g = to_g(g);                                                                                                \
     lb.CRS = CRS;                                                                                                  \
     rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true>(                    \
-        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s);                                           \
+        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s, "conv_wgrad", conv_flops(g));              \
   }
   if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128)
   else if (p.bm == 64 && p.bn == 128) SGH_WGRAD_CASE(64, 128)

@@ -36,6 +36,38 @@ int sgh_num_cus() {
   return g_num_cus;
 }
 
+// ---- kernel-level profiling records
+struct ProfRec {
+  const char *tag;
+  double work;
+  hipEvent_t a, b;
+};
+static std::vector<ProfRec> g_prof;
+static bool g_prof_on = false;
+
+bool sgh_prof_on() { return g_prof_on; }
+
+void sgh_prof_start(const char *tag, double work, hipStream_t s) {
+  if (!g_prof_on) return;
+  ProfRec r{tag, work, nullptr, nullptr};
+  if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) return;
+  (void)hipEventRecord(r.a, s);
+  g_prof.push_back(r);
+}
+
+void sgh_prof_stop(hipStream_t s) {
+  if (!g_prof_on || g_prof.empty()) return;
+  (void)hipEventRecord(g_prof.back().b, s);
+}
+
+static void prof_clear() {
+  for (auto &r : g_prof) {
+    if (r.a) (void)hipEventDestroy(r.a);
+    if (r.b) (void)hipEventDestroy(r.b);
+  }
+  g_prof.clear();
+}
+
 // Pool granularity: 256 B up to 4 KiB, then power-of-two classes with four steps per octave
 // (worst-case slack 19 %), so a training loop that frees and re-allocates the same tensor
 // shapes every iteration always hits the cache.
@@ -188,6 +220,32 @@ int sgh_memcpy(sgh_device *dev, void *dst, const void *src, size_t bytes, int ki
                                          hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice};
   SGH_HIP_TRY(hipMemcpyAsync(dst, src, bytes, kinds[kind], dev->stream));
   if (kind != 3) SGH_HIP_TRY(hipStreamSynchronize(dev->stream));
+  return SGH_OK;
+}
+
+int sgh_prof_enable(int on) {
+  if (on) prof_clear();
+  g_prof_on = on != 0;
+  return SGH_OK;
+}
+
+int sgh_prof_count(int *n) {
+  if (!n) return SGH_EINVAL;
+  *n = int(g_prof.size());
+  return SGH_OK;
+}
+
+int sgh_prof_get(int i, char *tag, size_t tag_len, float *ms, double *work) {
+  if (i < 0 || size_t(i) >= g_prof.size() || !ms) return SGH_EINVAL;
+  const ProfRec &r = g_prof[i];
+  SGH_HIP_TRY(hipEventSynchronize(r.b));
+  SGH_HIP_TRY(hipEventElapsedTime(ms, r.a, r.b));
+  if (work) *work = r.work;
+  if (tag && tag_len) {
+    size_t k = 0;
+    for (; r.tag[k] && k + 1 < tag_len; ++k) tag[k] = r.tag[k];
+    tag[k] = 0;
+  }
   return SGH_OK;
 }
 
