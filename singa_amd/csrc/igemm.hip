@@ -209,6 +209,104 @@ struct WgradXLoader {
 };
 
 // ------------------------------------------------------------------------------------------
+// Loaders 5 and 6 + epilogue: dgrad decomposed by output-pixel residue class.
+// With stride (sh, sw) the pixels h = ch + sh*hh, w = cw + sw*ww of class (ch, cw) receive
+// contributions only from the taps r = r0 + i*sh, s = s0 + j*sw (r0 = (ch + ph) % sh), and for
+// those p = hh + bh - i, q = ww + bw - j are exact.  Each class is therefore a dense stride-1
+// problem over its own tap subset: no MFMA work is spent on taps that cannot contribute
+// (a plain gather wastes 1 - 1/(sh*sw) of it).  blockIdx.z selects the class.
+//   k index inside a class = (i * ns + j) * KP + k_out
+//   class weights Wc[(tap_off + i*ns + j) * KP + k_out][c]  (k_weight_relayout_classes)
+// ------------------------------------------------------------------------------------------
+constexpr int kMaxClasses = 9;
+constexpr int kMaxTaps = 128;
+
+struct DgCls {
+  short ch, cw, r0, s0, nr, ns, bh, bw;
+  int Hc, Wc, tap_off;
+};
+struct DgClsTable {
+  DgCls c[kMaxClasses];
+};
+struct TapTable {  // class-ordered tap list: rs[t] = r * S + s
+  short rs[kMaxTaps];
+};
+
+template <int ROWS>
+struct DgradWLoader {  // A(m = c, k) = Wc[class][k][c], M-contiguous
+  const float *Wc;
+  int C, KP;
+  DgClsTable tab;
+  const float *base;
+  __device__ __forceinline__ void init(int, int) { base = Wc + long(tab.c[blockIdx.z].tap_off) * KP * C; }
+  __device__ __forceinline__ void load(int tile_row0, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
+    using M = StageMap<ROWS, false>;
+    const int row = tile_row0 + M::row0(t), kk0 = k0 + M::kk0(t);
+#pragma unroll
+    for (int e = 0; e < M::E; ++e) {
+      const int k = kk0 + e * M::K_STEP;
+      r[e] = (row < C && k < k_end) ? base[long(k) * C + row] : 0.f;
+    }
+  }
+};
+
+template <int ROWS>
+struct DgradDyLoader {  // B(k, col = (n, hh, ww) of the class), N-contiguous
+  const float *dy;
+  ConvG g;
+  int KP;
+  DgClsTable tab;
+  long img_base;
+  int hh, ww, cols;
+  bool col_ok;
+  DgCls c;
+  __device__ __forceinline__ void init(int tile_col0, int t) {
+    using M = StageMap<ROWS, false>;
+    c = tab.c[blockIdx.z];
+    const int plane = c.Hc * c.Wc;
+    cols = g.N * plane;
+    const int col = tile_col0 + M::row0(t);
+    col_ok = col < cols;
+    const int pl = plane > 0 ? plane : 1, wd = c.Wc > 0 ? c.Wc : 1;
+    const int n = col / pl, rem = col - n * pl;
+    hh = rem / wd;
+    ww = rem - hh * wd;
+    img_base = long(n) * g.K * g.P * g.Q;
+  }
+  __device__ __forceinline__ int ktotal() const { return int(c.nr) * c.ns * KP; }
+  __device__ __forceinline__ bool block_empty(int tile_col0) const { return tile_col0 >= cols; }
+  __device__ __forceinline__ void load(int, int k0, int, int t, float (&r)[ROWS * BK / NT]) const {
+    using M = StageMap<ROWS, false>;
+    const int tap = k0 / KP, ch0 = k0 - tap * KP + M::kk0(t);
+    const int i = tap / c.ns, j = tap - i * c.ns;
+    const int p = hh + c.bh - i, q = ww + c.bw - j;
+    const bool ok = col_ok && p >= 0 && p < g.P && q >= 0 && q < g.Q;
+    const int PQ = g.P * g.Q;
+    const float *src = dy + img_base + p * g.Q + q;
+#pragma unroll
+    for (int e = 0; e < M::E; ++e) {
+      const int ch = ch0 + e * M::K_STEP;
+      r[e] = (ok && ch < g.K) ? src[long(ch) * PQ] : 0.f;
+    }
+  }
+};
+
+struct DgradStore {  // dx[n][m][ch + sh*hh][cw + sw*ww]
+  float *dx;
+  ConvG g;
+  DgClsTable tab;
+  __device__ __forceinline__ void operator()(int m, int col, float v) const {
+    const DgCls c = tab.c[blockIdx.z];
+    const int plane = c.Hc * c.Wc;
+    if (m < g.C && col < g.N * plane) {
+      const int n = col / plane, rem = col - n * plane;
+      const int hh = rem / c.Wc, ww = rem - hh * c.Wc;
+      dx[((long(n) * g.C + m) * g.H + c.ch + g.sh * hh) * g.W + c.cw + g.sw * ww] = v;
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------------------
 // Epilogues
 // ------------------------------------------------------------------------------------------
 struct DenseStore {  // C[m * ldc + n] = alpha * acc + beta * C
@@ -248,7 +346,9 @@ struct SplitStore {  // partial[split][m * N + n]
 // The kernel.  grid = (M tiles, N tiles, K splits); split z covers chunks
 // [z * chunks_per_split, (z + 1) * chunks_per_split) of the reduction.
 // ------------------------------------------------------------------------------------------
-template <int BM, int BN, class LA, class LB, class ST, bool A_KCONTIG, bool B_KCONTIG>
+// With ZCLASS, blockIdx.z is a problem class instead (the B loader reports its reduction length
+// and whether this tile lies outside the class).
+template <int BM, int BN, class LA, class LB, class ST, bool A_KCONTIG, bool B_KCONTIG, bool ZCLASS = false>
 __global__ __launch_bounds__(NT) void k_igemm(LA la, LB lb, ST st, int Ktotal, int chunks_per_split) {
   constexpr int PA = BM + 4, PB = BN + 4;
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
@@ -259,12 +359,17 @@ __global__ __launch_bounds__(NT) void k_igemm(LA la, LB lb, ST st, int Ktotal, i
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
-  const int k_begin = blockIdx.z * chunks_per_split * BK;
+  int k_begin = blockIdx.z * chunks_per_split * BK;
   int k_end = k_begin + chunks_per_split * BK;
   if (k_end > Ktotal) k_end = Ktotal;
 
   la.init(m0, t);
   lb.init(n0, t);
+  if constexpr (ZCLASS) {
+    if (lb.block_empty(n0)) return;  // uniform over the workgroup, before any barrier
+    k_begin = 0;
+    k_end = lb.ktotal();
+  }
 
   v16f acc[TM][TN];
 #pragma unroll
@@ -357,6 +462,53 @@ __global__ __launch_bounds__(NT) void k_weight_relayout(const float *__restrict_
   }
 }
 
+// Class-ordered weight re-layout for the decomposed dgrad:
+//   Wc[(t * KP + k) * C + c] = W[k][c][taps.rs[t]],  t = position in the class-ordered tap list
+__global__ __launch_bounds__(NT) void k_weight_relayout_classes(const float *__restrict__ W, float *__restrict__ Wc,
+                                                               int K, int C, int RS, int KP, TapTable taps) {
+  const long total = long(RS) * KP * C;
+  const long stride = long(gridDim.x) * NT;
+  for (long i = long(blockIdx.x) * NT + threadIdx.x; i < total; i += stride) {
+    const int c = int(i % C);
+    const long rest = i / C;
+    const int k = int(rest % KP), tt = int(rest / KP);
+    Wc[i] = k < K ? W[(long(k) * C + c) * RS + taps.rs[tt]] : 0.f;
+  }
+}
+
+// Col2im as a gather (the scatter loop of the CPU algorithm turned inside out): one thread per
+// dx element adds the column entries of every tap that maps onto it, in ascending (r, s) order.
+//   dx[n][c][h][w] = sum_{r,s} dcol[(c*R + r)*S + s][n*PQ + p*Q + q],  p*sh = h + ph - r, q*sw = w + pw - s
+__global__ __launch_bounds__(NT) void k_col2im_gather(const float *__restrict__ dcol, float *__restrict__ dx, ConvG g,
+                                                     long total) {
+  const long stride = long(gridDim.x) * NT;
+  const int HW = g.H * g.W, PQ = g.P * g.Q;
+  const long ncols = long(g.N) * PQ;
+  for (long i = long(blockIdx.x) * NT + threadIdx.x; i < total; i += stride) {
+    const int w = int(i % g.W);
+    const long t1 = i / g.W;
+    const int h = int(t1 % g.H);
+    const long t2 = t1 / g.H;
+    const int c = int(t2 % g.C), n = int(t2 / g.C);
+    (void)HW;
+    float acc = 0.f;
+    for (int r = 0; r < g.R; ++r) {
+      const int hp = h + g.ph - r;
+      if (hp < 0) break;
+      const int p = hp / g.sh;
+      if (p * g.sh != hp || p >= g.P) continue;
+      for (int s = 0; s < g.S; ++s) {
+        const int wp = w + g.pw - s;
+        if (wp < 0) break;
+        const int q = wp / g.sw;
+        if (q * g.sw != wp || q >= g.Q) continue;
+        acc += dcol[long((c * g.R + r) * g.S + s) * ncols + long(n) * PQ + p * g.Q + q];
+      }
+    }
+    dx[i] = acc;
+  }
+}
+
 // One thread per (k), summing dy over n, p, q is too serial; use one workgroup per k.
 __global__ __launch_bounds__(NT) void k_conv_bgrad(const float *__restrict__ dy, float *__restrict__ db, int N, int K,
                                                   int PQ) {
@@ -418,15 +570,15 @@ inline WgradPlan plan_wgrad(const sgh_conv_geom *g) {
   return p;
 }
 
-template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc>
+template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc, bool ZCLASS = false>
 inline int launch_igemm(const LA &la, const LB &lb, const ST &st, int M, int N, int Ktotal, int splits,
                         int chunks_per_split, hipStream_t stream, const char *tag, double flops) {
   dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
   if (grid.y > 65535u || grid.z > 65535u) return SGH_EUNSUPPORTED;
-  sgh_prof_start(tag, flops, stream);
-  hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc>), grid, dim3(NT), 0, stream, la, lb, st, Ktotal,
+  if (tag) sgh_prof_start(tag, flops, stream);
+  hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc, ZCLASS>), grid, dim3(NT), 0, stream, la, lb, st, Ktotal,
                      chunks_per_split);
-  sgh_prof_stop(stream);
+  if (tag) sgh_prof_stop(stream);
   SGH_LAUNCH_CHECK();
   return SGH_OK;
 }
@@ -455,6 +607,18 @@ inline int gemm_pick(int M, int N, int K, float alpha, const float *A, long a_rs
   if (M > 64 && N > 64 && tiles128 >= sgh_num_cus())
     return gemm_tile<128, 128, AK, BKc>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, stream);
   return gemm_tile<64, 64, AK, BKc>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, stream);
+}
+
+// Which algorithm a dgrad of this geometry uses.
+enum DgradPath { kDgradColumns, kDgradClasses, kDgradGather };
+
+inline DgradPath dgrad_path(const sgh_conv_geom *g) {
+  const size_t RS = size_t(g->R) * g->S;
+  // few input channels: the C x pixels output tile would waste most of a 64-row MFMA tile, so run
+  // the dense GEMM dcol = W^T * dy (CRS rows) and fold the columns back with a gather
+  if (g->C < 32 && RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float) <= (size_t(2) << 30)) return kDgradColumns;
+  if (g->stride_h * g->stride_w <= kMaxClasses && RS <= size_t(kMaxTaps)) return kDgradClasses;
+  return kDgradGather;
 }
 
 }  // namespace
@@ -490,7 +654,9 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
   const size_t RS = size_t(g->R) * g->S;
   switch (which) {
     case SGH_CONV_FWD: return RS * round_up(g->C, BK) * g->K * sizeof(float);
-    case SGH_CONV_DGRAD: return RS * round_up(g->K, BK) * g->C * sizeof(float);
+    case SGH_CONV_DGRAD:
+      if (dgrad_path(g) == kDgradColumns) return RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float);
+      return RS * round_up(g->K, BK) * g->C * sizeof(float);
     case SGH_CONV_WGRAD: {
       const WgradPlan p = plan_wgrad(g);
       return p.splits > 1 ? size_t(p.splits) * g->K * g->C * RS * sizeof(float) : 0;
@@ -505,28 +671,104 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
   const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_DGRAD);
   if (!workspace || ws_bytes < need) return SGH_EWORKSPACE;
   hipStream_t s = sgh_stream_of(stream);
-  float *Wt = static_cast<float *>(workspace);
   const int RS = g->R * g->S, KP = round_up(g->K, BK);
-  {
+  const DgradPath path = dgrad_path(g);
+  int rc = SGH_OK;
+  sgh_prof_start("conv_dgrad", conv_flops(g), s);
+
+  if (path == kDgradColumns) {
+    float *dcol = static_cast<float *>(workspace);
+    const int CRS = g->C * RS, Ncols = g->N * g->P * g->Q;
+    DenseLoader<64, false> la{W, 1, long(CRS), CRS, g->K};
+    ConvG fake{g->N, g->K, g->P, g->Q, g->K, 1, 1, 1, 1, 0, 0, g->P, g->Q};
+    PixelGatherLoader<128, false> lb{dy, fake, KP, g->K, g->P, g->Q, Ncols, 0, 0, 0, false};
+    DenseStore st{dcol, long(Ncols), CRS, Ncols, 1.f, 0.f};
+    rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DenseStore, false, false>(
+        la, lb, st, CRS, Ncols, g->K, 1, (g->K + BK - 1) / BK, s, nullptr, 0);
+    if (rc == SGH_OK) {
+      const long total = long(g->N) * g->C * g->H * g->W;
+      long blocks = (total + NT - 1) / NT;
+      const long cap = long(sgh_num_cus()) * 32;
+      if (blocks > cap) blocks = cap;
+      hipLaunchKernelGGL(k_col2im_gather, dim3(int(blocks)), dim3(NT), 0, s, dcol, dx, to_g(g), total);
+      if (hipGetLastError() != hipSuccess) rc = SGH_EINVAL;
+    }
+  } else if (path == kDgradClasses) {
+    float *Wc = static_cast<float *>(workspace);
+    DgClsTable tab;
+    TapTable taps;
+    int ncls = 0, tap_off = 0, max_cols = 0;
+    for (int ch = 0; ch < g->stride_h; ++ch)
+      for (int cw = 0; cw < g->stride_w; ++cw) {
+        DgCls &c = tab.c[ncls++];
+        const int r0 = (ch + g->pad_h) % g->stride_h, s0 = (cw + g->pad_w) % g->stride_w;
+        c.ch = short(ch);
+        c.cw = short(cw);
+        c.r0 = short(r0);
+        c.s0 = short(s0);
+        c.nr = short(r0 < g->R ? (g->R - r0 + g->stride_h - 1) / g->stride_h : 0);
+        c.ns = short(s0 < g->S ? (g->S - s0 + g->stride_w - 1) / g->stride_w : 0);
+        if (c.nr == 0 || c.ns == 0) c.nr = c.ns = 0;
+        c.bh = short((ch + g->pad_h - r0) / g->stride_h);
+        c.bw = short((cw + g->pad_w - s0) / g->stride_w);
+        c.Hc = ch < g->H ? (g->H - ch + g->stride_h - 1) / g->stride_h : 0;
+        c.Wc = cw < g->W ? (g->W - cw + g->stride_w - 1) / g->stride_w : 0;
+        c.tap_off = tap_off;
+        for (int i = 0; i < c.nr; ++i)
+          for (int j = 0; j < c.ns; ++j)
+            taps.rs[tap_off + i * c.ns + j] = short((r0 + i * g->stride_h) * g->S + (s0 + j * g->stride_w));
+        tap_off += c.nr * c.ns;
+        const int cols = g->N * c.Hc * c.Wc;
+        if (cols > max_cols) max_cols = cols;
+      }
+    for (int i = tap_off; i < kMaxTaps; ++i) taps.rs[i] = 0;
+    for (int i = ncls; i < kMaxClasses; ++i) tab.c[i] = tab.c[0];
+    {
+      const long total = long(tap_off) * KP * g->C;
+      long blocks = (total + NT - 1) / NT;
+      if (blocks > 4096) blocks = 4096;
+      if (total > 0)
+        hipLaunchKernelGGL(k_weight_relayout_classes, dim3(int(blocks)), dim3(NT), 0, s, W, Wc, g->K, g->C, RS, KP,
+                           taps);
+    }
+    const int M = g->C;
+    DgradStore st{dx, to_g(g), tab};
+    if (M > 64) {
+      DgradWLoader<128> la{Wc, g->C, KP, tab, nullptr};
+      DgradDyLoader<128> lb;
+      lb.dy = dy;
+      lb.g = to_g(g);
+      lb.KP = KP;
+      lb.tab = tab;
+      rc = launch_igemm<128, 128, DgradWLoader<128>, DgradDyLoader<128>, DgradStore, false, false, true>(
+          la, lb, st, M, max_cols, 0, ncls, 0, s, nullptr, 0);
+    } else {
+      DgradWLoader<64> la{Wc, g->C, KP, tab, nullptr};
+      DgradDyLoader<128> lb;
+      lb.dy = dy;
+      lb.g = to_g(g);
+      lb.KP = KP;
+      lb.tab = tab;
+      rc = launch_igemm<64, 128, DgradWLoader<64>, DgradDyLoader<128>, DgradStore, false, false, true>(
+          la, lb, st, M, max_cols, 0, ncls, 0, s, nullptr, 0);
+    }
+  } else {
+    float *Wt = static_cast<float *>(workspace);
     const long total = long(RS) * KP * g->C;
     long blocks = (total + NT - 1) / NT;
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
-    SGH_LAUNCH_CHECK();
-  }
-  const int M = g->C, Ncols = g->N * g->H * g->W, Ktot = RS * KP;
-  const int chunks = Ktot / BK;
-  NchwStore st{dx, nullptr, g->C, g->H * g->W, Ncols};
-  if (M > 64) {
+    const int M = g->C, Ncols = g->N * g->H * g->W, Ktot = RS * KP;
+    NchwStore st{dx, nullptr, g->C, g->H * g->W, Ncols};
     DenseLoader<128, false> la{Wt, 1, long(g->C), M, Ktot};
     PixelGatherLoader<128, true> lb{dy, to_g(g), KP, g->K, g->P, g->Q, Ncols, 0, 0, 0, false};
-    return launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_dgrad", conv_flops(g));
+    rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
+        la, lb, st, M, Ncols, Ktot, 1, Ktot / BK, s, nullptr, 0);
   }
-  DenseLoader<64, false> la{Wt, 1, long(g->C), M, Ktot};
-  PixelGatherLoader<128, true> lb{dy, to_g(g), KP, g->K, g->P, g->Q, Ncols, 0, 0, 0, false};
-  return launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
-      la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_dgrad", conv_flops(g));
+  sgh_prof_stop(s);
+  if (rc != SGH_OK) return rc;
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
 }
 
 int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, const float *bias, float *y,
@@ -572,6 +814,7 @@ int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, 
   float *part = p.splits > 1 ? static_cast<float *>(workspace) : dW;
   SplitStore st{part, g->K, CRS};
   int rc;
+  sgh_prof_start("conv_wgrad", conv_flops(g), s);
 #define SGH_WGRAD_CASE(BM_, BN_)                                                                                   \
   {                                                                                                                \
     WgradDyLoader<BM_> la{dy, g->K, PQ, int(G)};                                                                   \
@@ -580,21 +823,25 @@ int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, 
     lb.g = to_g(g);                                                                                                \
     lb.CRS = CRS;                                                                                                  \
     rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true>(                    \
-        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s, "conv_wgrad", conv_flops(g));              \
+        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s, nullptr, 0);                               \
   }
   if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128)
   else if (p.bm == 64 && p.bn == 128) SGH_WGRAD_CASE(64, 128)
   else if (p.bm == 128 && p.bn == 64) SGH_WGRAD_CASE(128, 64)
   else SGH_WGRAD_CASE(64, 64)
 #undef SGH_WGRAD_CASE
-  if (rc != SGH_OK) return rc;
+  if (rc != SGH_OK) {
+    sgh_prof_stop(s);
+    return rc;
+  }
   if (p.splits > 1) {
     const long n = long(g->K) * CRS;
     long blocks = (n + NT - 1) / NT;
     if (blocks > 2048) blocks = 2048;
     hipLaunchKernelGGL(k_split_reduce, dim3(int(blocks)), dim3(NT), 0, s, part, dW, n, p.splits);
-    SGH_LAUNCH_CHECK();
   }
+  sgh_prof_stop(s);
+  SGH_LAUNCH_CHECK();
   return SGH_OK;
 }
 

@@ -67,6 +67,14 @@ CONV_CASES = [
     (1, 130, 9, 9, 70, 3, 3, (1, 1), (1, 1), False),      # channel counts that are not tile multiples
     (4, 8, 5, 5, 8, 3, 3, (1, 1), (0, 0), False),         # no padding
     (1, 1, 3, 3, 1, 3, 3, (1, 1), (2, 2), False),         # pad wider than half the kernel
+    (2, 40, 9, 11, 24, 3, 3, (2, 2), (1, 1), False),      # stride 2, odd image: residue classes of unequal size
+    (2, 34, 10, 10, 20, 3, 3, (3, 3), (1, 1), False),     # stride 3: nine residue classes
+    (3, 64, 8, 8, 128, 1, 1, (2, 2), (0, 0), False),      # 1x1 stride 2: three classes receive no tap at all
+    (1, 32, 12, 12, 16, 5, 5, (2, 2), (2, 2), False),
+    (2, 32, 8, 8, 32, 2, 2, (2, 2), (0, 0), False),       # kernel == stride
+    (1, 32, 7, 7, 16, 1, 1, (3, 3), (0, 0), False),       # kernel smaller than stride
+    (2, 36, 9, 7, 33, 3, 2, (2, 1), (1, 0), True),        # mixed strides, non-square kernel
+    (2, 4, 12, 12, 8, 3, 3, (2, 2), (1, 1), False),       # few input channels: column-GEMM + gather path, strided
 ]
 
 
