@@ -24,6 +24,21 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int NT = 256;
 constexpr int BK = 16;
 
+// Global operands are read through buffer loads: the hardware range check makes an out-of-range
+// byte offset return 0, which gives zero padding / tile tails without a branch per element.
+// Every operand tensor is therefore limited to < 2 GiB (SINGA's Device::Malloc(int) caps a Block
+// at that size anyway: include/singa/core/device.h:142).
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int kOOB = int(0x80000000u);
+__device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
+}
+// `ok` must be built with bitwise '&' (no short-circuit) so that the load stays straight-line code.
+__device__ __forceinline__ float buf_ld(rsrc_t r, int elem_off, int ok) {
+  const int m = -ok;  // all ones when valid
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, ((elem_off << 2) & m) | (kOOB & ~m), 0, 0));
+}
+
 // ------------------------------------------------------------------------------------------
 // Thread -> staged element mapping.
 //   K-contiguous operand (consecutive k are consecutive in memory):
@@ -56,16 +71,18 @@ __device__ __forceinline__ void stage_store(float *lds /* [BK][ROWS + 4] */, con
 template <int ROWS, bool KCONTIG>
 struct DenseLoader {
   const float *base;
-  long rs, ks;
+  int rs, ks;
   int rows, K;
+  unsigned bytes;
   __device__ __forceinline__ void init(int, int) {}
   __device__ __forceinline__ void load(int tile_row0, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
     using M = StageMap<ROWS, KCONTIG>;
+    const rsrc_t rc = make_rsrc(base, bytes);
     const int row0 = tile_row0 + M::row0(t), kk0 = k0 + M::kk0(t);
 #pragma unroll
     for (int e = 0; e < M::E; ++e) {
       const int row = row0 + e * M::ROW_STEP, k = kk0 + e * M::K_STEP;
-      r[e] = (row < rows && k < k_end) ? base[row * rs + k * ks] : 0.f;
+      r[e] = buf_ld(rc, row * rs + k * ks, int(row < rows) & int(k < k_end));
     }
   }
 };
@@ -94,8 +111,9 @@ struct PixelGatherLoader {
   int src_ch;    // channels of the source tensor (C for fwd, K for dgrad)
   int src_h, src_w;
   int cols;      // valid columns (N * P * Q or N * H * W)
+  unsigned bytes;
   // per-thread state
-  long img_base;  // offset of image n in src
+  int img_base;  // offset of image n in src
   int a, b;       // (p, q) for fwd, (h, w) for dgrad
   bool col_ok;
 
@@ -108,12 +126,13 @@ struct PixelGatherLoader {
     const int n = col / plane, rem = col - n * plane;
     a = rem / wdt;
     b = rem - a * wdt;
-    img_base = long(n) * src_ch * src_h * src_w;
+    img_base = n * src_ch * src_h * src_w;
   }
 
   __device__ __forceinline__ void load(int, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
     using M = StageMap<ROWS, false>;
     (void)k_end;
+    const rsrc_t rc = make_rsrc(src, bytes);
     const int tap = k0 / CP, ch0 = k0 - tap * CP + M::kk0(t);
     const int fr = tap / g.S, fs = tap - fr * g.S;
     int y, x;
@@ -122,18 +141,18 @@ struct PixelGatherLoader {
       const int hp = a + g.ph - fr, wp = b + g.pw - fs;
       y = hp / g.sh;
       x = wp / g.sw;
-      ok = ok && hp >= 0 && wp >= 0 && y * g.sh == hp && x * g.sw == wp && y < g.P && x < g.Q;
+      ok = ok & (hp >= 0) & (wp >= 0) & (y * g.sh == hp) & (x * g.sw == wp) & (y < g.P) & (x < g.Q);
     } else {
       y = a * g.sh - g.ph + fr;
       x = b * g.sw - g.pw + fs;
-      ok = ok && y >= 0 && y < g.H && x >= 0 && x < g.W;
+      ok = ok & (unsigned(y) < unsigned(g.H)) & (unsigned(x) < unsigned(g.W));
     }
-    const long plane = long(src_h) * src_w;
-    const float *p = src + img_base + long(y) * src_w + x;
+    const int plane = src_h * src_w;
+    const int p = img_base + y * src_w + x;
 #pragma unroll
     for (int e = 0; e < M::E; ++e) {
       const int ch = ch0 + e * M::K_STEP;
-      r[e] = (ok && ch < src_ch) ? p[ch * plane] : 0.f;
+      r[e] = buf_ld(rc, p + ch * plane, int(ok) & int(ch < src_ch));
     }
   }
 };
@@ -148,18 +167,20 @@ template <int ROWS>
 struct WgradDyLoader {
   const float *dy;
   int K, PQ, G;  // G = N * PQ
+  unsigned bytes;
   __device__ __forceinline__ void init(int, int) {}
   __device__ __forceinline__ void load(int tile_row0, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
     using M = StageMap<ROWS, true>;
+    const rsrc_t rc = make_rsrc(dy, bytes);
     const int gi = k0 + M::kk0(t);
     const bool ok = gi < k_end;
     const int n = gi / PQ, pq = gi - n * PQ;
-    const float *p = dy + long(n) * K * PQ + pq;
+    const int p = n * K * PQ + pq;
     const int row0 = tile_row0 + M::row0(t);
 #pragma unroll
     for (int e = 0; e < M::E; ++e) {
       const int row = row0 + e * M::ROW_STEP;
-      r[e] = (ok && row < K) ? p[long(row) * PQ] : 0.f;
+      r[e] = buf_ld(rc, p + row * PQ, int(ok) & int(row < K));
     }
   }
 };
@@ -169,6 +190,7 @@ struct WgradXLoader {
   const float *x;
   ConvG g;
   int CRS;
+  unsigned bytes;
   // per-thread, per staged row: offset of (c, r - ph, s - pw) inside an image, and the tap shifts
   int off[ROWS * BK / NT];
   short dr[ROWS * BK / NT], ds[ROWS * BK / NT];
@@ -198,12 +220,14 @@ struct WgradXLoader {
     const int n = gi / PQ, pq = gi - n * PQ;
     const int p = pq / g.Q, q = pq - p * g.Q;
     const int h0 = p * g.sh, w0 = q * g.sw;
-    const float *base = x + long(n) * g.C * g.H * g.W + h0 * g.W + w0;
+    const int base = n * g.C * g.H * g.W + h0 * g.W + w0;
+    const rsrc_t rc = make_rsrc(x, bytes);
 #pragma unroll
     for (int e = 0; e < M::E; ++e) {
       const int h = h0 + dr[e], w = w0 + ds[e];
-      const bool v = ok && h >= 0 && h < g.H && w >= 0 && w < g.W;
-      r[e] = v ? base[off[e]] : 0.f;
+      // unsigned compares fold the two-sided range checks
+      const int v = int(ok) & int(unsigned(h) < unsigned(g.H)) & int(unsigned(w) < unsigned(g.W));
+      r[e] = buf_ld(rc, base + off[e], v);
     }
   }
 };
@@ -236,16 +260,18 @@ template <int ROWS>
 struct DgradWLoader {  // A(m = c, k) = Wc[class][k][c], M-contiguous
   const float *Wc;
   int C, KP;
-  DgClsTable tab;
-  const float *base;
-  __device__ __forceinline__ void init(int, int) { base = Wc + long(tab.c[blockIdx.z].tap_off) * KP * C; }
+  const DgCls *tab;  // class table in device memory (written by k_weight_relayout_classes)
+  unsigned bytes;
+  int base;
+  __device__ __forceinline__ void init(int, int) { base = tab[blockIdx.z].tap_off * KP * C; }
   __device__ __forceinline__ void load(int tile_row0, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
     using M = StageMap<ROWS, false>;
+    const rsrc_t rc = make_rsrc(Wc, bytes);
     const int row = tile_row0 + M::row0(t), kk0 = k0 + M::kk0(t);
 #pragma unroll
     for (int e = 0; e < M::E; ++e) {
       const int k = kk0 + e * M::K_STEP;
-      r[e] = (row < C && k < k_end) ? base[long(k) * C + row] : 0.f;
+      r[e] = buf_ld(rc, base + k * C + row, int(row < C) & int(k < k_end));
     }
   }
 };
@@ -255,14 +281,15 @@ struct DgradDyLoader {  // B(k, col = (n, hh, ww) of the class), N-contiguous
   const float *dy;
   ConvG g;
   int KP;
-  DgClsTable tab;
-  long img_base;
+  const DgCls *tab;
+  unsigned bytes;
+  int img_base;
   int hh, ww, cols;
   bool col_ok;
   DgCls c;
   __device__ __forceinline__ void init(int tile_col0, int t) {
     using M = StageMap<ROWS, false>;
-    c = tab.c[blockIdx.z];
+    c = tab[blockIdx.z];
     const int plane = c.Hc * c.Wc;
     cols = g.N * plane;
     const int col = tile_col0 + M::row0(t);
@@ -271,7 +298,7 @@ struct DgradDyLoader {  // B(k, col = (n, hh, ww) of the class), N-contiguous
     const int n = col / pl, rem = col - n * pl;
     hh = rem / wd;
     ww = rem - hh * wd;
-    img_base = long(n) * g.K * g.P * g.Q;
+    img_base = n * g.K * g.P * g.Q;
   }
   __device__ __forceinline__ int ktotal() const { return int(c.nr) * c.ns * KP; }
   __device__ __forceinline__ bool block_empty(int tile_col0) const { return tile_col0 >= cols; }
@@ -280,13 +307,14 @@ struct DgradDyLoader {  // B(k, col = (n, hh, ww) of the class), N-contiguous
     const int tap = k0 / KP, ch0 = k0 - tap * KP + M::kk0(t);
     const int i = tap / c.ns, j = tap - i * c.ns;
     const int p = hh + c.bh - i, q = ww + c.bw - j;
-    const bool ok = col_ok && p >= 0 && p < g.P && q >= 0 && q < g.Q;
+    const int ok = int(col_ok) & int(unsigned(p) < unsigned(g.P)) & int(unsigned(q) < unsigned(g.Q));
     const int PQ = g.P * g.Q;
-    const float *src = dy + img_base + p * g.Q + q;
+    const int src = img_base + p * g.Q + q;
+    const rsrc_t rc = make_rsrc(dy, bytes);
 #pragma unroll
     for (int e = 0; e < M::E; ++e) {
       const int ch = ch0 + e * M::K_STEP;
-      r[e] = (ok && ch < g.K) ? src[long(ch) * PQ] : 0.f;
+      r[e] = buf_ld(rc, src + ch * PQ, int(ok) & int(ch < g.K));
     }
   }
 };
@@ -294,9 +322,9 @@ struct DgradDyLoader {  // B(k, col = (n, hh, ww) of the class), N-contiguous
 struct DgradStore {  // dx[n][m][ch + sh*hh][cw + sw*ww]
   float *dx;
   ConvG g;
-  DgClsTable tab;
+  const DgCls *tab;
   __device__ __forceinline__ void operator()(int m, int col, float v) const {
-    const DgCls c = tab.c[blockIdx.z];
+    const DgCls c = tab[blockIdx.z];
     const int plane = c.Hc * c.Wc;
     if (m < g.C && col < g.N * plane) {
       const int n = col / plane, rem = col - n * plane;
@@ -397,17 +425,27 @@ __global__ __launch_bounds__(NT) void k_igemm(LA la, LB lb, ST st, int Ktotal, i
     }
     const float *as = As[cur] + (lane >> 5) * PA + wm * WM + (lane & 31);
     const float *bs = Bs[cur] + (lane >> 5) * PB + wn * WN + (lane & 31);
+    // operand fragments are double-buffered in registers: the LDS reads of k-step kk+2 are in
+    // flight while the MFMAs of k-step kk execute
+    float a[2][TM], b[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a[0][i] = as[i * 32];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b[0][j] = bs[j * 32];
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 2) {
-      float a[TM], b[TN];
+      const int cb = (kk >> 1) & 1, nb = cb ^ 1;
+      if (kk + 2 < BK) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a[i] = as[kk * PA + i * 32];
+        for (int i = 0; i < TM; ++i) a[nb][i] = as[(kk + 2) * PA + i * 32];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) b[j] = bs[kk * PB + j * 32];
+        for (int j = 0; j < TN; ++j) b[nb][j] = bs[(kk + 2) * PB + j * 32];
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cb][i], b[cb][j], acc[i][j], 0, 0, 0);
     }
     if (more) {
       stage_store<BM, A_KCONTIG>(As[cur ^ 1], ra, t);
@@ -465,7 +503,16 @@ __global__ __launch_bounds__(NT) void k_weight_relayout(const float *__restrict_
 // Class-ordered weight re-layout for the decomposed dgrad:
 //   Wc[(t * KP + k) * C + c] = W[k][c][taps.rs[t]],  t = position in the class-ordered tap list
 __global__ __launch_bounds__(NT) void k_weight_relayout_classes(const float *__restrict__ W, float *__restrict__ Wc,
-                                                               int K, int C, int RS, int KP, TapTable taps) {
+                                                               int K, int C, int RS, int KP, TapTable taps,
+                                                               DgClsTable tab, DgCls *__restrict__ tab_out) {
+  if (blockIdx.x == 0 && threadIdx.x < kMaxClasses) {
+    // static indexing keeps the by-value table in SGPRs
+    DgCls c = tab.c[0];
+#pragma unroll
+    for (int i = 1; i < kMaxClasses; ++i)
+      if (int(threadIdx.x) == i) c = tab.c[i];
+    tab_out[threadIdx.x] = c;
+  }
   const long total = long(RS) * KP * C;
   const long stride = long(gridDim.x) * NT;
   for (long i = long(blockIdx.x) * NT + threadIdx.x; i < total; i += stride) {
@@ -530,6 +577,8 @@ inline ConvG to_g(const sgh_conv_geom *g) {
   return ConvG{g->N, g->C, g->H, g->W, g->K, g->R, g->S, g->stride_h, g->stride_w, g->pad_h, g->pad_w, g->P, g->Q};
 }
 
+constexpr size_t kMaxOperandBytes = size_t(1) << 31;  // buffer-load addressing limit per tensor
+
 inline bool conv_ok(const sgh_conv_geom *g) {
   if (!g) return false;
   if (g->N <= 0 || g->C <= 0 || g->H <= 0 || g->W <= 0 || g->K <= 0 || g->R <= 0 || g->S <= 0 || g->stride_h <= 0 ||
@@ -538,13 +587,45 @@ inline bool conv_ok(const sgh_conv_geom *g) {
   if (g->P != (g->H + 2 * g->pad_h - g->R) / g->stride_h + 1) return false;
   if (g->Q != (g->W + 2 * g->pad_w - g->S) / g->stride_w + 1) return false;
   if (g->pad_h > 16000 || g->pad_w > 16000 || g->R > 16000 || g->S > 16000) return false;
-  // all flattened index spaces are addressed with 32-bit ints inside the kernels
-  const size_t lim = 0x7fffffffu;
+  // every tensor is addressed with 32-bit byte offsets inside the kernels
+  const size_t lim = kMaxOperandBytes / sizeof(float);
   if (size_t(g->N) * g->C * g->H * g->W >= lim) return false;
   if (size_t(g->N) * g->K * g->P * g->Q >= lim) return false;
-  if (size_t(g->K) * g->C * g->R * g->S >= lim) return false;
-  if (size_t(g->R) * g->S * (size_t(g->C > g->K ? g->C : g->K) + BK) >= lim) return false;
+  if (size_t(g->R) * g->S * (size_t(g->C) + BK) * (size_t(g->K) + BK) >= lim) return false;
   return true;
+}
+
+inline unsigned bytes_of(size_t elems) { return unsigned(elems * sizeof(float)); }
+
+// ---- loader factories (host) -------------------------------------------------------------
+template <int ROWS, bool KC>
+inline DenseLoader<ROWS, KC> dense_loader(const float *base, long rs, long ks, int rows, int K) {
+  DenseLoader<ROWS, KC> l;
+  l.base = base;
+  l.rs = int(rs);
+  l.ks = int(ks);
+  l.rows = rows;
+  l.K = K;
+  const size_t extent = (rows > 0 && K > 0) ? size_t(rows - 1) * rs + size_t(K - 1) * ks + 1 : 0;
+  l.bytes = bytes_of(extent);
+  return l;
+}
+
+template <int ROWS, bool DG>
+inline PixelGatherLoader<ROWS, DG> gather_loader(const float *src, const ConvG &g, int CP, int src_ch, int src_h,
+                                                 int src_w, int cols) {
+  PixelGatherLoader<ROWS, DG> l;
+  l.src = src;
+  l.g = g;
+  l.CP = CP;
+  l.src_ch = src_ch;
+  l.src_h = src_h;
+  l.src_w = src_w;
+  l.cols = cols;
+  l.bytes = bytes_of(size_t(g.N) * src_ch * src_h * src_w);
+  l.img_base = l.a = l.b = 0;
+  l.col_ok = false;
+  return l;
 }
 
 struct WgradPlan {
@@ -572,15 +653,12 @@ inline WgradPlan plan_wgrad(const sgh_conv_geom *g) {
 
 template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc, bool ZCLASS = false>
 inline int launch_igemm(const LA &la, const LB &lb, const ST &st, int M, int N, int Ktotal, int splits,
-                        int chunks_per_split, hipStream_t stream, const char *tag, double flops) {
+                        int chunks_per_split, hipStream_t stream) {
   dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
   if (grid.y > 65535u || grid.z > 65535u) return SGH_EUNSUPPORTED;
-  if (tag) sgh_prof_start(tag, flops, stream);
   hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc, ZCLASS>), grid, dim3(NT), 0, stream, la, lb, st, Ktotal,
                      chunks_per_split);
-  if (tag) sgh_prof_stop(stream);
-  SGH_LAUNCH_CHECK();
-  return SGH_OK;
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
 // algorithmic FLOPs of one convolution pass: 2 * N * K * P * Q * C * R * S
@@ -592,12 +670,12 @@ inline double conv_flops(const sgh_conv_geom *g) {
 template <int BM, int BN, bool AK, bool BKc>
 inline int gemm_tile(int M, int N, int K, float alpha, const float *A, long a_rs, long a_ks, const float *B, long b_rs,
                      long b_ks, float beta, float *C, int ldc, hipStream_t stream) {
-  DenseLoader<BM, AK> la{A, a_rs, a_ks, M, K};
-  DenseLoader<BN, BKc> lb{B, b_rs, b_ks, N, K};
+  auto la = dense_loader<BM, AK>(A, a_rs, a_ks, M, K);
+  auto lb = dense_loader<BN, BKc>(B, b_rs, b_ks, N, K);
   DenseStore st{C, ldc, M, N, alpha, beta};
   const int chunks = (K + BK - 1) / BK;
-  return launch_igemm<BM, BN, DenseLoader<BM, AK>, DenseLoader<BN, BKc>, DenseStore, AK, BKc>(
-      la, lb, st, M, N, K, 1, chunks, stream, "gemm", 2.0 * M * N * K);
+  return launch_igemm<BM, BN, DenseLoader<BM, AK>, DenseLoader<BN, BKc>, DenseStore, AK, BKc>(la, lb, st, M, N, K, 1,
+                                                                                               chunks, stream);
 }
 
 template <bool AK, bool BKc>
@@ -616,10 +694,12 @@ inline DgradPath dgrad_path(const sgh_conv_geom *g) {
   const size_t RS = size_t(g->R) * g->S;
   // few input channels: the C x pixels output tile would waste most of a 64-row MFMA tile, so run
   // the dense GEMM dcol = W^T * dy (CRS rows) and fold the columns back with a gather
-  if (g->C < 32 && RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float) <= (size_t(2) << 30)) return kDgradColumns;
+  if (g->C < 32 && RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float) < kMaxOperandBytes) return kDgradColumns;
   if (g->stride_h * g->stride_w <= kMaxClasses && RS <= size_t(kMaxTaps)) return kDgradClasses;
   return kDgradGather;
 }
+
+inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
 }  // namespace
 
@@ -656,7 +736,7 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
     case SGH_CONV_FWD: return RS * round_up(g->C, BK) * g->K * sizeof(float);
     case SGH_CONV_DGRAD:
       if (dgrad_path(g) == kDgradColumns) return RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float);
-      return RS * round_up(g->K, BK) * g->C * sizeof(float);
+      return align256(RS * round_up(g->K, BK) * g->C * sizeof(float)) + align256(sizeof(DgClsTable));
     case SGH_CONV_WGRAD: {
       const WgradPlan p = plan_wgrad(g);
       return p.splits > 1 ? size_t(p.splits) * g->K * g->C * RS * sizeof(float) : 0;
@@ -679,22 +759,23 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
   if (path == kDgradColumns) {
     float *dcol = static_cast<float *>(workspace);
     const int CRS = g->C * RS, Ncols = g->N * g->P * g->Q;
-    DenseLoader<64, false> la{W, 1, long(CRS), CRS, g->K};
+    auto la = dense_loader<64, false>(W, 1, CRS, CRS, g->K);
     ConvG fake{g->N, g->K, g->P, g->Q, g->K, 1, 1, 1, 1, 0, 0, g->P, g->Q};
-    PixelGatherLoader<128, false> lb{dy, fake, KP, g->K, g->P, g->Q, Ncols, 0, 0, 0, false};
+    auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
     DenseStore st{dcol, long(Ncols), CRS, Ncols, 1.f, 0.f};
     rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DenseStore, false, false>(
-        la, lb, st, CRS, Ncols, g->K, 1, (g->K + BK - 1) / BK, s, nullptr, 0);
+        la, lb, st, CRS, Ncols, g->K, 1, (g->K + BK - 1) / BK, s);
     if (rc == SGH_OK) {
       const long total = long(g->N) * g->C * g->H * g->W;
       long blocks = (total + NT - 1) / NT;
       const long cap = long(sgh_num_cus()) * 32;
       if (blocks > cap) blocks = cap;
       hipLaunchKernelGGL(k_col2im_gather, dim3(int(blocks)), dim3(NT), 0, s, dcol, dx, to_g(g), total);
-      if (hipGetLastError() != hipSuccess) rc = SGH_EINVAL;
     }
   } else if (path == kDgradClasses) {
     float *Wc = static_cast<float *>(workspace);
+    const size_t wc_bytes = size_t(RS) * KP * g->C * sizeof(float);
+    DgCls *tab_dev = reinterpret_cast<DgCls *>(static_cast<char *>(workspace) + align256(wc_bytes));
     DgClsTable tab;
     TapTable taps;
     int ncls = 0, tap_off = 0, max_cols = 0;
@@ -727,30 +808,26 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
       const long total = long(tap_off) * KP * g->C;
       long blocks = (total + NT - 1) / NT;
       if (blocks > 4096) blocks = 4096;
-      if (total > 0)
-        hipLaunchKernelGGL(k_weight_relayout_classes, dim3(int(blocks)), dim3(NT), 0, s, W, Wc, g->K, g->C, RS, KP,
-                           taps);
+      if (blocks < 1) blocks = 1;  // the class table is written even when no tap survives
+      hipLaunchKernelGGL(k_weight_relayout_classes, dim3(int(blocks)), dim3(NT), 0, s, W, Wc, g->K, g->C, RS, KP, taps,
+                         tab, tab_dev);
     }
     const int M = g->C;
-    DgradStore st{dx, to_g(g), tab};
+    DgradStore st{dx, to_g(g), tab_dev};
+    DgradDyLoader<128> lb;
+    lb.dy = dy;
+    lb.g = to_g(g);
+    lb.KP = KP;
+    lb.tab = tab_dev;
+    lb.bytes = bytes_of(size_t(g->N) * g->K * g->P * g->Q);
     if (M > 64) {
-      DgradWLoader<128> la{Wc, g->C, KP, tab, nullptr};
-      DgradDyLoader<128> lb;
-      lb.dy = dy;
-      lb.g = to_g(g);
-      lb.KP = KP;
-      lb.tab = tab;
+      DgradWLoader<128> la{Wc, g->C, KP, tab_dev, unsigned(wc_bytes), 0};
       rc = launch_igemm<128, 128, DgradWLoader<128>, DgradDyLoader<128>, DgradStore, false, false, true>(
-          la, lb, st, M, max_cols, 0, ncls, 0, s, nullptr, 0);
+          la, lb, st, M, max_cols, 0, ncls, 0, s);
     } else {
-      DgradWLoader<64> la{Wc, g->C, KP, tab, nullptr};
-      DgradDyLoader<128> lb;
-      lb.dy = dy;
-      lb.g = to_g(g);
-      lb.KP = KP;
-      lb.tab = tab;
+      DgradWLoader<64> la{Wc, g->C, KP, tab_dev, unsigned(wc_bytes), 0};
       rc = launch_igemm<64, 128, DgradWLoader<64>, DgradDyLoader<128>, DgradStore, false, false, true>(
-          la, lb, st, M, max_cols, 0, ncls, 0, s, nullptr, 0);
+          la, lb, st, M, max_cols, 0, ncls, 0, s);
     }
   } else {
     float *Wt = static_cast<float *>(workspace);
@@ -760,10 +837,10 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
     hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
     const int M = g->C, Ncols = g->N * g->H * g->W, Ktot = RS * KP;
     NchwStore st{dx, nullptr, g->C, g->H * g->W, Ncols};
-    DenseLoader<128, false> la{Wt, 1, long(g->C), M, Ktot};
-    PixelGatherLoader<128, true> lb{dy, to_g(g), KP, g->K, g->P, g->Q, Ncols, 0, 0, 0, false};
+    auto la = dense_loader<128, false>(Wt, 1, g->C, M, Ktot);
+    auto lb = gather_loader<128, true>(dy, to_g(g), KP, g->K, g->P, g->Q, Ncols);
     rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, Ktot / BK, s, nullptr, 0);
+        la, lb, st, M, Ncols, Ktot, 1, Ktot / BK, s);
   }
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
@@ -779,26 +856,31 @@ int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, con
   hipStream_t s = sgh_stream_of(stream);
   float *Wt = static_cast<float *>(workspace);
   const int RS = g->R * g->S, CP = round_up(g->C, BK);
+  sgh_prof_start("conv_fwd", conv_flops(g), s);
   {
     const long total = long(RS) * CP * g->K;
     long blocks = (total + NT - 1) / NT;
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, CP, 0);
-    SGH_LAUNCH_CHECK();
   }
   const int M = g->K, Ncols = g->N * g->P * g->Q, Ktot = RS * CP;
   const int chunks = Ktot / BK;
   NchwStore st{y, bias, g->K, g->P * g->Q, Ncols};
+  auto lb = gather_loader<128, false>(x, to_g(g), CP, g->C, g->H, g->W, Ncols);
+  int rc;
   if (M > 64) {
-    DenseLoader<128, false> la{Wt, 1, long(g->K), M, Ktot};
-    PixelGatherLoader<128, false> lb{x, to_g(g), CP, g->C, g->H, g->W, Ncols, 0, 0, 0, false};
-    return launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd", conv_flops(g));
+    auto la = dense_loader<128, false>(Wt, 1, g->K, M, Ktot);
+    rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+  } else {
+    auto la = dense_loader<64, false>(Wt, 1, g->K, M, Ktot);
+    rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s);
   }
-  DenseLoader<64, false> la{Wt, 1, long(g->K), M, Ktot};
-  PixelGatherLoader<128, false> lb{x, to_g(g), CP, g->C, g->H, g->W, Ncols, 0, 0, 0, false};
-  return launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
-      la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd", conv_flops(g));
+  sgh_prof_stop(s);
+  if (rc != SGH_OK) return rc;
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
 }
 
 int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
@@ -810,37 +892,34 @@ int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, 
   hipStream_t s = sgh_stream_of(stream);
   const int CRS = g->C * g->R * g->S, PQ = g->P * g->Q;
   const long G = long(g->N) * PQ;
-  if (G >= 0x7fffffffL) return SGH_EUNSUPPORTED;
   float *part = p.splits > 1 ? static_cast<float *>(workspace) : dW;
   SplitStore st{part, g->K, CRS};
   int rc;
   sgh_prof_start("conv_wgrad", conv_flops(g), s);
 #define SGH_WGRAD_CASE(BM_, BN_)                                                                                   \
   {                                                                                                                \
-    WgradDyLoader<BM_> la{dy, g->K, PQ, int(G)};                                                                   \
+    WgradDyLoader<BM_> la{dy, g->K, PQ, int(G), bytes_of(size_t(G) * g->K)};                                       \
     WgradXLoader<BN_> lb;                                                                                          \
     lb.x = x;                                                                                                      \
     lb.g = to_g(g);                                                                                                \
     lb.CRS = CRS;                                                                                                  \
+    lb.bytes = bytes_of(size_t(g->N) * g->C * g->H * g->W);                                                        \
     rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true>(                    \
-        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s, nullptr, 0);                               \
+        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s);                                           \
   }
   if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128)
   else if (p.bm == 64 && p.bn == 128) SGH_WGRAD_CASE(64, 128)
   else if (p.bm == 128 && p.bn == 64) SGH_WGRAD_CASE(128, 64)
   else SGH_WGRAD_CASE(64, 64)
 #undef SGH_WGRAD_CASE
-  if (rc != SGH_OK) {
-    sgh_prof_stop(s);
-    return rc;
-  }
-  if (p.splits > 1) {
+  if (rc == SGH_OK && p.splits > 1) {
     const long n = long(g->K) * CRS;
     long blocks = (n + NT - 1) / NT;
     if (blocks > 2048) blocks = 2048;
     hipLaunchKernelGGL(k_split_reduce, dim3(int(blocks)), dim3(NT), 0, s, part, dW, n, p.splits);
   }
   sgh_prof_stop(s);
+  if (rc != SGH_OK) return rc;
   SGH_LAUNCH_CHECK();
   return SGH_OK;
 }
@@ -859,14 +938,21 @@ int sgh_gemm_f32(int transA, int transB, int M, int N, int K, float alpha, const
   if (!C || ldc < N) return SGH_EINVAL;
   if (K > 0 && (!A || !B)) return SGH_EINVAL;
   if (K > 0 && (lda < (transA ? M : K) || ldb < (transB ? K : N))) return SGH_EINVAL;
+  // operands are addressed with 32-bit byte offsets
+  const size_t a_ext = size_t(transA ? K : M) * lda, b_ext = size_t(transB ? N : K) * ldb;
+  if (a_ext * sizeof(float) >= kMaxOperandBytes || b_ext * sizeof(float) >= kMaxOperandBytes) return SGH_EUNSUPPORTED;
   hipStream_t s = sgh_stream_of(stream);
   // element(row, k) strides of each operand
   const long a_rs = transA ? 1 : lda, a_ks = transA ? lda : 1;  // A(m, k)
   const long b_rs = transB ? ldb : 1, b_ks = transB ? 1 : ldb;  // B(k, n) addressed as (n, k)
-  if (!transA && transB) return gemm_pick<true, true>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
-  if (!transA && !transB) return gemm_pick<true, false>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
-  if (transA && transB) return gemm_pick<false, true>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
-  return gemm_pick<false, false>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+  int rc;
+  sgh_prof_start("gemm", 2.0 * M * N * K, s);
+  if (!transA && transB) rc = gemm_pick<true, true>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+  else if (!transA && !transB) rc = gemm_pick<true, false>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+  else if (transA && transB) rc = gemm_pick<false, true>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+  else rc = gemm_pick<false, false>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+  sgh_prof_stop(s);
+  return rc;
 }
 
 }  // extern "C"
