@@ -1,20 +1,29 @@
 // fp32 MFMA GEMM core and the implicit-GEMM convolution passes built on it
 // (conv forward, dgrad, wgrad) plus the Linear-layer GEMM.
 //
-// One workgroup = 256 threads = 4 wavefronts in a 2 x 2 grid; the workgroup computes a
-// BM x BN tile of C, each wavefront a (BM/2) x (BN/2) sub-tile out of 32x32x2 fp32 MFMAs
+// One workgroup = 256 threads = 4 wavefronts in a WGM x WGN grid; the workgroup computes a
+// BM x BN tile of C, each wavefront a (BM/WGM) x (BN/WGN) sub-tile out of 32x32x2 fp32 MFMAs
 // (v_mfma_f32_32x32x2_f32: lane l feeds A[l%32][l/32] and B[l/32][l%32]; its 16 accumulators
 // hold C[8*(v/4) + 4*(l/32) + v%4][l%32]).
 //
 // Operands are staged through LDS in [k][m] / [k][n] order with a row pitch of (tile + 4)
 // floats: the MFMA operand reads (32 consecutive m for two consecutive k) and both kinds of
 // staging writes (threads consecutive in m, or consecutive in k) then touch every bank at most
-// twice per 64-lane access, which is the minimum.  Global loads for chunk i+1 are issued before
-// the MFMAs of chunk i and written to the other LDS buffer afterwards (one barrier per chunk).
+// twice per 64-lane access, which is the minimum.
+//
+// Software pipeline of one BK-chunk (8 MFMA k-steps):
+//   - the LDS operand fragments of k-step s+1 are fetched into a second register set before the
+//     MFMAs of k-step s are issued;
+//   - the global loads of the NEXT chunk (address arithmetic included) are spread over the
+//     k-steps and issued right behind each step's MFMAs, so their VALU work and latency hide
+//     under the matrix pipeline;
+//   - after the last k-step the loaded registers go to the other LDS buffer (one barrier per chunk).
 //
 // A "problem" supplies two loaders (how to fetch element (row, k) of A and (k, col) of B,
 // zero outside the valid range) and an epilogue (where C[m][n] goes).  The convolution loaders
 // perform im2col on the fly: no column matrix is ever materialised.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace {
@@ -23,6 +32,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int NT = 256;
 constexpr int BK = 16;
+constexpr int KSTEPS = BK / 2;
 
 // Global operands are read through buffer loads: the hardware range check makes an out-of-range
 // byte offset return 0, which gives zero padding / tile tails without a branch per element.
@@ -64,26 +74,31 @@ __device__ __forceinline__ void stage_store(float *lds /* [BK][ROWS + 4] */, con
   for (int e = 0; e < M::E; ++e) lds[(kk0 + e * M::K_STEP) * (ROWS + 4) + row0 + e * M::ROW_STEP] = r[e];
 }
 
+// Every loader has:   init(tile0, t)          once per kernel (per-thread constants)
+//                     prepare(tile0, k0, k_end, t)   once per chunk (per-chunk index arithmetic)
+//                     get(e)                   element e of the chunk prepared last
+
 // ------------------------------------------------------------------------------------------
 // Loader 1: dense strided matrix.  element(row, k) = base[row * rs + k * ks]; whichever of
 // rs / ks is 1 decides KCONTIG.
 // ------------------------------------------------------------------------------------------
 template <int ROWS, bool KCONTIG>
 struct DenseLoader {
+  using M = StageMap<ROWS, KCONTIG>;
   const float *base;
   int rs, ks;
   int rows, K;
   unsigned bytes;
+  int row0_, kk0_, kend_;
   __device__ __forceinline__ void init(int, int) {}
-  __device__ __forceinline__ void load(int tile_row0, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
-    using M = StageMap<ROWS, KCONTIG>;
-    const rsrc_t rc = make_rsrc(base, bytes);
-    const int row0 = tile_row0 + M::row0(t), kk0 = k0 + M::kk0(t);
-#pragma unroll
-    for (int e = 0; e < M::E; ++e) {
-      const int row = row0 + e * M::ROW_STEP, k = kk0 + e * M::K_STEP;
-      r[e] = buf_ld(rc, row * rs + k * ks, int(row < rows) & int(k < k_end));
-    }
+  __device__ __forceinline__ void prepare(int tile_row0, int k0, int k_end, int t) {
+    row0_ = tile_row0 + M::row0(t);
+    kk0_ = k0 + M::kk0(t);
+    kend_ = k_end;
+  }
+  __device__ __forceinline__ float get(int e) const {
+    const int row = row0_ + e * M::ROW_STEP, k = kk0_ + e * M::K_STEP;
+    return buf_ld(make_rsrc(base, bytes), row * rs + k * ks, int(row < rows) & int(k < kend_));
   }
 };
 
@@ -105,6 +120,7 @@ struct ConvG {
 // ------------------------------------------------------------------------------------------
 template <int ROWS, bool DGRAD>
 struct PixelGatherLoader {
+  using M = StageMap<ROWS, false>;
   const float *src;
   ConvG g;
   int CP;        // padded channel count of the k index
@@ -114,11 +130,12 @@ struct PixelGatherLoader {
   unsigned bytes;
   // per-thread state
   int img_base;  // offset of image n in src
-  int a, b;       // (p, q) for fwd, (h, w) for dgrad
+  int a, b;      // (p, q) for fwd, (h, w) for dgrad
   bool col_ok;
+  // per-chunk state
+  int p_, ch0_, ok_;
 
   __device__ __forceinline__ void init(int tile_col0, int t) {
-    using M = StageMap<ROWS, false>;
     const int col = tile_col0 + M::row0(t);
     col_ok = col < cols;
     const int plane = DGRAD ? g.H * g.W : g.P * g.Q;
@@ -129,14 +146,12 @@ struct PixelGatherLoader {
     img_base = n * src_ch * src_h * src_w;
   }
 
-  __device__ __forceinline__ void load(int, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
-    using M = StageMap<ROWS, false>;
-    (void)k_end;
-    const rsrc_t rc = make_rsrc(src, bytes);
-    const int tap = k0 / CP, ch0 = k0 - tap * CP + M::kk0(t);
+  __device__ __forceinline__ void prepare(int, int k0, int, int t) {
+    const int tap = k0 / CP;
+    ch0_ = k0 - tap * CP + M::kk0(t);
     const int fr = tap / g.S, fs = tap - fr * g.S;
     int y, x;
-    bool ok = col_ok;
+    int ok = col_ok;
     if (DGRAD) {
       const int hp = a + g.ph - fr, wp = b + g.pw - fs;
       y = hp / g.sh;
@@ -147,13 +162,13 @@ struct PixelGatherLoader {
       x = b * g.sw - g.pw + fs;
       ok = ok & (unsigned(y) < unsigned(g.H)) & (unsigned(x) < unsigned(g.W));
     }
-    const int plane = src_h * src_w;
-    const int p = img_base + y * src_w + x;
-#pragma unroll
-    for (int e = 0; e < M::E; ++e) {
-      const int ch = ch0 + e * M::K_STEP;
-      r[e] = buf_ld(rc, p + ch * plane, int(ok) & int(ch < src_ch));
-    }
+    ok_ = ok;
+    p_ = img_base + y * src_w + x;
+  }
+
+  __device__ __forceinline__ float get(int e) const {
+    const int ch = ch0_ + e * M::K_STEP;
+    return buf_ld(make_rsrc(src, bytes), p_ + ch * (src_h * src_w), ok_ & int(ch < src_ch));
   }
 };
 
@@ -165,28 +180,28 @@ struct PixelGatherLoader {
 // ------------------------------------------------------------------------------------------
 template <int ROWS>
 struct WgradDyLoader {
+  using M = StageMap<ROWS, true>;
   const float *dy;
   int K, PQ, G;  // G = N * PQ
   unsigned bytes;
+  int row0_, p_, ok_;
   __device__ __forceinline__ void init(int, int) {}
-  __device__ __forceinline__ void load(int tile_row0, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
-    using M = StageMap<ROWS, true>;
-    const rsrc_t rc = make_rsrc(dy, bytes);
+  __device__ __forceinline__ void prepare(int tile_row0, int k0, int k_end, int t) {
     const int gi = k0 + M::kk0(t);
-    const bool ok = gi < k_end;
+    ok_ = gi < k_end;
     const int n = gi / PQ, pq = gi - n * PQ;
-    const int p = n * K * PQ + pq;
-    const int row0 = tile_row0 + M::row0(t);
-#pragma unroll
-    for (int e = 0; e < M::E; ++e) {
-      const int row = row0 + e * M::ROW_STEP;
-      r[e] = buf_ld(rc, p + row * PQ, int(ok) & int(row < K));
-    }
+    p_ = n * K * PQ + pq;
+    row0_ = tile_row0 + M::row0(t);
+  }
+  __device__ __forceinline__ float get(int e) const {
+    const int row = row0_ + e * M::ROW_STEP;
+    return buf_ld(make_rsrc(dy, bytes), p_ + row * PQ, ok_ & int(row < K));
   }
 };
 
 template <int ROWS>
 struct WgradXLoader {
+  using M = StageMap<ROWS, true>;
   const float *x;
   ConvG g;
   int CRS;
@@ -194,8 +209,8 @@ struct WgradXLoader {
   // per-thread, per staged row: offset of (c, r - ph, s - pw) inside an image, and the tap shifts
   int off[ROWS * BK / NT];
   short dr[ROWS * BK / NT], ds[ROWS * BK / NT];
+  int h0_, w0_, base_, ok_;
   __device__ __forceinline__ void init(int tile_col0, int t) {
-    using M = StageMap<ROWS, true>;
     const int RS = g.R * g.S;
 #pragma unroll
     for (int e = 0; e < M::E; ++e) {
@@ -212,23 +227,21 @@ struct WgradXLoader {
       }
     }
   }
-  __device__ __forceinline__ void load(int, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
-    using M = StageMap<ROWS, true>;
+  __device__ __forceinline__ void prepare(int, int k0, int k_end, int t) {
     const int gi = k0 + M::kk0(t);
-    const bool ok = gi < k_end;
+    ok_ = gi < k_end;
     const int PQ = g.P * g.Q;
     const int n = gi / PQ, pq = gi - n * PQ;
     const int p = pq / g.Q, q = pq - p * g.Q;
-    const int h0 = p * g.sh, w0 = q * g.sw;
-    const int base = n * g.C * g.H * g.W + h0 * g.W + w0;
-    const rsrc_t rc = make_rsrc(x, bytes);
-#pragma unroll
-    for (int e = 0; e < M::E; ++e) {
-      const int h = h0 + dr[e], w = w0 + ds[e];
-      // unsigned compares fold the two-sided range checks
-      const int v = int(ok) & int(unsigned(h) < unsigned(g.H)) & int(unsigned(w) < unsigned(g.W));
-      r[e] = buf_ld(rc, base + off[e], v);
-    }
+    h0_ = p * g.sh;
+    w0_ = q * g.sw;
+    base_ = n * g.C * g.H * g.W + h0_ * g.W + w0_;
+  }
+  __device__ __forceinline__ float get(int e) const {
+    const int h = h0_ + dr[e], w = w0_ + ds[e];
+    // unsigned compares fold the two-sided range checks
+    const int v = ok_ & int(unsigned(h) < unsigned(g.H)) & int(unsigned(w) < unsigned(g.W));
+    return buf_ld(make_rsrc(x, bytes), base_ + off[e], v);
   }
 };
 
@@ -258,26 +271,28 @@ struct TapTable {  // class-ordered tap list: rs[t] = r * S + s
 
 template <int ROWS>
 struct DgradWLoader {  // A(m = c, k) = Wc[class][k][c], M-contiguous
+  using M = StageMap<ROWS, false>;
   const float *Wc;
   int C, KP;
   const DgCls *tab;  // class table in device memory (written by k_weight_relayout_classes)
   unsigned bytes;
   int base;
+  int row_, kk0_, kend_;
   __device__ __forceinline__ void init(int, int) { base = tab[blockIdx.z].tap_off * KP * C; }
-  __device__ __forceinline__ void load(int tile_row0, int k0, int k_end, int t, float (&r)[ROWS * BK / NT]) const {
-    using M = StageMap<ROWS, false>;
-    const rsrc_t rc = make_rsrc(Wc, bytes);
-    const int row = tile_row0 + M::row0(t), kk0 = k0 + M::kk0(t);
-#pragma unroll
-    for (int e = 0; e < M::E; ++e) {
-      const int k = kk0 + e * M::K_STEP;
-      r[e] = buf_ld(rc, base + k * C + row, int(row < C) & int(k < k_end));
-    }
+  __device__ __forceinline__ void prepare(int tile_row0, int k0, int k_end, int t) {
+    row_ = tile_row0 + M::row0(t);
+    kk0_ = k0 + M::kk0(t);
+    kend_ = k_end;
+  }
+  __device__ __forceinline__ float get(int e) const {
+    const int k = kk0_ + e * M::K_STEP;
+    return buf_ld(make_rsrc(Wc, bytes), base + k * C + row_, int(row_ < C) & int(k < kend_));
   }
 };
 
 template <int ROWS>
 struct DgradDyLoader {  // B(k, col = (n, hh, ww) of the class), N-contiguous
+  using M = StageMap<ROWS, false>;
   const float *dy;
   ConvG g;
   int KP;
@@ -287,8 +302,8 @@ struct DgradDyLoader {  // B(k, col = (n, hh, ww) of the class), N-contiguous
   int hh, ww, cols;
   bool col_ok;
   DgCls c;
+  int src_, ch0_, ok_;
   __device__ __forceinline__ void init(int tile_col0, int t) {
-    using M = StageMap<ROWS, false>;
     c = tab[blockIdx.z];
     const int plane = c.Hc * c.Wc;
     cols = g.N * plane;
@@ -302,20 +317,18 @@ struct DgradDyLoader {  // B(k, col = (n, hh, ww) of the class), N-contiguous
   }
   __device__ __forceinline__ int ktotal() const { return int(c.nr) * c.ns * KP; }
   __device__ __forceinline__ bool block_empty(int tile_col0) const { return tile_col0 >= cols; }
-  __device__ __forceinline__ void load(int, int k0, int, int t, float (&r)[ROWS * BK / NT]) const {
-    using M = StageMap<ROWS, false>;
-    const int tap = k0 / KP, ch0 = k0 - tap * KP + M::kk0(t);
-    const int i = tap / c.ns, j = tap - i * c.ns;
+  __device__ __forceinline__ void prepare(int, int k0, int, int t) {
+    const int tap = k0 / KP;
+    ch0_ = k0 - tap * KP + M::kk0(t);
+    const int ns = c.ns > 0 ? c.ns : 1;
+    const int i = tap / ns, j = tap - i * ns;
     const int p = hh + c.bh - i, q = ww + c.bw - j;
-    const int ok = int(col_ok) & int(unsigned(p) < unsigned(g.P)) & int(unsigned(q) < unsigned(g.Q));
-    const int PQ = g.P * g.Q;
-    const int src = img_base + p * g.Q + q;
-    const rsrc_t rc = make_rsrc(dy, bytes);
-#pragma unroll
-    for (int e = 0; e < M::E; ++e) {
-      const int ch = ch0 + e * M::K_STEP;
-      r[e] = buf_ld(rc, src + ch * PQ, int(ok) & int(ch < g.K));
-    }
+    ok_ = int(col_ok) & int(unsigned(p) < unsigned(g.P)) & int(unsigned(q) < unsigned(g.Q));
+    src_ = img_base + p * g.Q + q;
+  }
+  __device__ __forceinline__ float get(int e) const {
+    const int ch = ch0_ + e * M::K_STEP;
+    return buf_ld(make_rsrc(dy, bytes), src_ + ch * (g.P * g.Q), ok_ & int(ch < g.K));
   }
 };
 
@@ -373,19 +386,23 @@ struct SplitStore {  // partial[split][m * N + n]
 // ------------------------------------------------------------------------------------------
 // The kernel.  grid = (M tiles, N tiles, K splits); split z covers chunks
 // [z * chunks_per_split, (z + 1) * chunks_per_split) of the reduction.
-// ------------------------------------------------------------------------------------------
 // With ZCLASS, blockIdx.z is a problem class instead (the B loader reports its reduction length
 // and whether this tile lies outside the class).
-template <int BM, int BN, class LA, class LB, class ST, bool A_KCONTIG, bool B_KCONTIG, bool ZCLASS = false>
+// ------------------------------------------------------------------------------------------
+template <int BM, int BN, class LA, class LB, class ST, bool A_KCONTIG, bool B_KCONTIG, bool ZCLASS = false,
+          int WGM = 2>
 __global__ __launch_bounds__(NT) void k_igemm(LA la, LB lb, ST st, int Ktotal, int chunks_per_split) {
+  // the four wavefronts form a WGM x WGN grid over the tile
+  constexpr int WGN = 4 / WGM;
   constexpr int PA = BM + 4, PB = BN + 4;
-  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
-  constexpr int EA = BM * BK / NT, EB = BN * BK / NT;
+  constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+  static_assert(TM >= 1 && TN >= 1 && WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
+  constexpr int EA = BM * BK / NT, EB = BN * BK / NT, ET = EA + EB;
   __shared__ float As[2][BK * PA];
   __shared__ float Bs[2][BK * PB];
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
   int k_begin = blockIdx.z * chunks_per_split * BK;
   int k_end = k_begin + chunks_per_split * BK;
@@ -409,8 +426,12 @@ __global__ __launch_bounds__(NT) void k_igemm(LA la, LB lb, ST st, int Ktotal, i
 
   float ra[EA], rb[EB];
   if (k_begin < k_end) {
-    la.load(m0, k_begin, k_end, t, ra);
-    lb.load(n0, k_begin, k_end, t, rb);
+    la.prepare(m0, k_begin, k_end, t);
+    lb.prepare(n0, k_begin, k_end, t);
+#pragma unroll
+    for (int e = 0; e < EA; ++e) ra[e] = la.get(e);
+#pragma unroll
+    for (int e = 0; e < EB; ++e) rb[e] = lb.get(e);
     stage_store<BM, A_KCONTIG>(As[0], ra, t);
     stage_store<BN, B_KCONTIG>(Bs[0], rb, t);
   }
@@ -418,36 +439,43 @@ __global__ __launch_bounds__(NT) void k_igemm(LA la, LB lb, ST st, int Ktotal, i
 
   int cur = 0;
   for (int k0 = k_begin; k0 < k_end; k0 += BK) {
-    const bool more = k0 + BK < k_end;
-    if (more) {
-      la.load(m0, k0 + BK, k_end, t, ra);
-      lb.load(n0, k0 + BK, k_end, t, rb);
-    }
+    // the next chunk is always fetched: past the end every loader yields zeros (or, for the
+    // gather loaders, values that are never stored), which keeps this loop free of branches
+    la.prepare(m0, k0 + BK, k_end, t);
+    lb.prepare(n0, k0 + BK, k_end, t);
+
     const float *as = As[cur] + (lane >> 5) * PA + wm * WM + (lane & 31);
     const float *bs = Bs[cur] + (lane >> 5) * PB + wn * WN + (lane & 31);
-    // operand fragments are double-buffered in registers: the LDS reads of k-step kk+2 are in
-    // flight while the MFMAs of k-step kk execute
     float a[2][TM], b[2][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i) a[0][i] = as[i * 32];
 #pragma unroll
     for (int j = 0; j < TN; ++j) b[0][j] = bs[j * 32];
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 2) {
-      const int cb = (kk >> 1) & 1, nb = cb ^ 1;
-      if (kk + 2 < BK) {
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int cb = s & 1, nb = cb ^ 1;
+      if (s + 1 < KSTEPS) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) a[nb][i] = as[(kk + 2) * PA + i * 32];
+        for (int i = 0; i < TM; ++i) a[nb][i] = as[(2 * s + 2) * PA + i * 32];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) b[nb][j] = bs[(kk + 2) * PB + j * 32];
+        for (int j = 0; j < TN; ++j) b[nb][j] = bs[(2 * s + 2) * PB + j * 32];
       }
+      __builtin_amdgcn_sched_barrier(0);  // operand prefetch stays ahead of this k-step's MFMAs
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cb][i], b[cb][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);  // this k-step's share of the next chunk's global loads
+#pragma unroll
+      for (int q = 0; q < ET; ++q) {
+        if (q * KSTEPS / ET == s) {
+          if (q < EA) ra[q] = la.get(q);
+          else rb[q - EA] = lb.get(q - EA);
+        }
+      }
     }
-    if (more) {
+    if (k0 + BK < k_end) {
       stage_store<BM, A_KCONTIG>(As[cur ^ 1], ra, t);
       stage_store<BN, B_KCONTIG>(Bs[cur ^ 1], rb, t);
     }
@@ -608,6 +636,7 @@ inline DenseLoader<ROWS, KC> dense_loader(const float *base, long rs, long ks, i
   l.K = K;
   const size_t extent = (rows > 0 && K > 0) ? size_t(rows - 1) * rs + size_t(K - 1) * ks + 1 : 0;
   l.bytes = bytes_of(extent);
+  l.row0_ = l.kk0_ = l.kend_ = 0;
   return l;
 }
 
@@ -625,6 +654,7 @@ inline PixelGatherLoader<ROWS, DG> gather_loader(const float *src, const ConvG &
   l.bytes = bytes_of(size_t(g.N) * src_ch * src_h * src_w);
   l.img_base = l.a = l.b = 0;
   l.col_ok = false;
+  l.p_ = l.ch0_ = l.ok_ = 0;
   return l;
 }
 
@@ -637,6 +667,20 @@ inline WgradPlan plan_wgrad(const sgh_conv_geom *g) {
   const int CRS = g->C * g->R * g->S;
   p.bm = g->K > 64 ? 128 : 64;
   p.bn = CRS > 64 ? 128 : 64;
+  // 64 output channels: a 64 x 256 tile (wavefronts 1 x 4, 64 x 64 each) keeps four MFMAs per
+  // operand fetch, which a 64 x 128 tile (32 x 64 per wavefront) cannot
+  if (p.bm == 64 && CRS >= 256) p.bn = 256;
+  // 576 = 64 channels x 9 taps is exactly three 192-wide tiles (a 128- or 256-wide tile would
+  // spend 10 % / 25 % of its MFMAs on padding columns)
+  if (p.bm == 64 && CRS % 192 == 0 && CRS % 256 != 0) p.bn = 192;
+  if (const char *e = getenv("SGH_WGRAD_TILE")) {
+    const int v = atoi(e);
+    static const int bm[6] = {128, 64, 128, 64, 64, 64}, bn[6] = {128, 128, 64, 64, 256, 192};
+    if (v >= 0 && v <= 5) {
+      p.bm = bm[v];
+      p.bn = bn[v];
+    }
+  }
   const long tiles = long((g->K + p.bm - 1) / p.bm) * ((CRS + p.bn - 1) / p.bn);
   const long G = long(g->N) * g->P * g->Q;
   const long chunks = (G + BK - 1) / BK;
@@ -651,13 +695,13 @@ inline WgradPlan plan_wgrad(const sgh_conv_geom *g) {
   return p;
 }
 
-template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc, bool ZCLASS = false>
+template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc, bool ZCLASS = false, int WGM = 2>
 inline int launch_igemm(const LA &la, const LB &lb, const ST &st, int M, int N, int Ktotal, int splits,
                         int chunks_per_split, hipStream_t stream) {
   dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
   if (grid.y > 65535u || grid.z > 65535u) return SGH_EUNSUPPORTED;
-  hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc, ZCLASS>), grid, dim3(NT), 0, stream, la, lb, st, Ktotal,
-                     chunks_per_split);
+  hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc, ZCLASS, WGM>), grid, dim3(NT), 0, stream, la, lb, st,
+                     Ktotal, chunks_per_split);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -685,6 +729,27 @@ inline int gemm_pick(int M, int N, int K, float alpha, const float *A, long a_rs
   if (M > 64 && N > 64 && tiles128 >= sgh_num_cus())
     return gemm_tile<128, 128, AK, BKc>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, stream);
   return gemm_tile<64, 64, AK, BKc>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, stream);
+}
+
+// Tile choice for an M x N problem launched `z` times: 0 = 128x128, 1 = 64x128, 2 = 128x64,
+// 3 = 64x64.  The largest tile that still yields at least two workgroups per CU wins; a small
+// problem takes the smallest tile.  An environment variable (value 0..3) overrides the choice,
+// the counterpart of the reference's CUDNN_CONV_ALG switch
+// (reference: src/model/operation/convolution.cc:453-457).
+inline int pick_tile(const char *env, int M, int N, int z) {
+  if (const char *e = getenv(env)) {
+    const int v = atoi(e);
+    if (v >= 0 && v <= 3) return v;
+  }
+  static const int bm[4] = {128, 64, 128, 64}, bn[4] = {128, 128, 64, 64};
+  const long want = 2L * sgh_num_cus();
+  for (int i = 0; i < 4; ++i) {
+    if (bm[i] == 128 && M <= 64) continue;
+    if (bn[i] == 128 && N <= 64) continue;
+    const long blocks = long((M + bm[i] - 1) / bm[i]) * ((N + bn[i] - 1) / bn[i]) * z;
+    if (blocks >= want) return i;
+  }
+  return (M <= 64) ? (N <= 64 ? 3 : 1) : 3;
 }
 
 // Which algorithm a dgrad of this geometry uses.
@@ -814,21 +879,24 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
     }
     const int M = g->C;
     DgradStore st{dx, to_g(g), tab_dev};
-    DgradDyLoader<128> lb;
-    lb.dy = dy;
-    lb.g = to_g(g);
-    lb.KP = KP;
-    lb.tab = tab_dev;
-    lb.bytes = bytes_of(size_t(g->N) * g->K * g->P * g->Q);
-    if (M > 64) {
-      DgradWLoader<128> la{Wc, g->C, KP, tab_dev, unsigned(wc_bytes), 0};
-      rc = launch_igemm<128, 128, DgradWLoader<128>, DgradDyLoader<128>, DgradStore, false, false, true>(
-          la, lb, st, M, max_cols, 0, ncls, 0, s);
-    } else {
-      DgradWLoader<64> la{Wc, g->C, KP, tab_dev, unsigned(wc_bytes), 0};
-      rc = launch_igemm<64, 128, DgradWLoader<64>, DgradDyLoader<128>, DgradStore, false, false, true>(
-          la, lb, st, M, max_cols, 0, ncls, 0, s);
-    }
+    const int tile = pick_tile("SGH_DGRAD_TILE", M, max_cols, ncls);
+#define SGH_DGRAD_CASE(BM_, BN_)                                                                              \
+  {                                                                                                           \
+    DgradWLoader<BM_> la{Wc, g->C, KP, tab_dev, unsigned(wc_bytes), 0, 0, 0, 0};                              \
+    DgradDyLoader<BN_> lb;                                                                                    \
+    lb.dy = dy;                                                                                               \
+    lb.g = to_g(g);                                                                                           \
+    lb.KP = KP;                                                                                               \
+    lb.tab = tab_dev;                                                                                         \
+    lb.bytes = bytes_of(size_t(g->N) * g->K * g->P * g->Q);                                                   \
+    rc = launch_igemm<BM_, BN_, DgradWLoader<BM_>, DgradDyLoader<BN_>, DgradStore, false, false, true>(       \
+        la, lb, st, M, max_cols, 0, ncls, 0, s);                                                              \
+  }
+    if (tile == 0) SGH_DGRAD_CASE(128, 128)
+    else if (tile == 1) SGH_DGRAD_CASE(64, 128)
+    else if (tile == 2) SGH_DGRAD_CASE(128, 64)
+    else SGH_DGRAD_CASE(64, 64)
+#undef SGH_DGRAD_CASE
   } else {
     float *Wt = static_cast<float *>(workspace);
     const long total = long(RS) * KP * g->C;
@@ -896,21 +964,23 @@ int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, 
   SplitStore st{part, g->K, CRS};
   int rc;
   sgh_prof_start("conv_wgrad", conv_flops(g), s);
-#define SGH_WGRAD_CASE(BM_, BN_)                                                                                   \
+#define SGH_WGRAD_CASE(BM_, BN_, WGM_)                                                                             \
   {                                                                                                                \
-    WgradDyLoader<BM_> la{dy, g->K, PQ, int(G), bytes_of(size_t(G) * g->K)};                                       \
+    WgradDyLoader<BM_> la{dy, g->K, PQ, int(G), bytes_of(size_t(G) * g->K), 0, 0, 0};                              \
     WgradXLoader<BN_> lb;                                                                                          \
     lb.x = x;                                                                                                      \
     lb.g = to_g(g);                                                                                                \
     lb.CRS = CRS;                                                                                                  \
     lb.bytes = bytes_of(size_t(g->N) * g->C * g->H * g->W);                                                        \
-    rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true>(                    \
+    rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true, false, WGM_>(       \
         la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s);                                           \
   }
-  if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128)
-  else if (p.bm == 64 && p.bn == 128) SGH_WGRAD_CASE(64, 128)
-  else if (p.bm == 128 && p.bn == 64) SGH_WGRAD_CASE(128, 64)
-  else SGH_WGRAD_CASE(64, 64)
+  if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128, 2)
+  else if (p.bm == 64 && p.bn == 256) SGH_WGRAD_CASE(64, 256, 1)
+  else if (p.bm == 64 && p.bn == 192) SGH_WGRAD_CASE(64, 192, 2)
+  else if (p.bm == 64 && p.bn == 128) SGH_WGRAD_CASE(64, 128, 2)
+  else if (p.bm == 128 && p.bn == 64) SGH_WGRAD_CASE(128, 64, 2)
+  else SGH_WGRAD_CASE(64, 64, 2)
 #undef SGH_WGRAD_CASE
   if (rc == SGH_OK && p.splits > 1) {
     const long n = long(g->K) * CRS;
