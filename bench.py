@@ -134,6 +134,9 @@ def main():
     }
     for k, v in conv.items():
         roofline[k + "_tflops"] = round(v["flop"] / (v["ms"] * 1e-3) / 1e12, 3) if v["ms"] > 0 else 0.0
+    # whole entry points (weight re-layout, split-K reduction and column gather kernels included)
+    ops_ms = sum(prof[k]["ms"] for k in ("conv_dgrad_op", "conv_wgrad_op") if k in prof)
+    roofline["entry_points_ms_per_step"] = round(ops_ms / prof_steps, 4)
 
     out = {
         "metric": "backward+update imgs/sec, ResNet-18 N=64 fp32", "value": round(imgs_per_s, 2), "unit": "imgs/s",

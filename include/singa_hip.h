@@ -91,8 +91,10 @@ SGH_API int sgh_event_elapsed_ms(sgh_event *start, sgh_event *stop, float *ms);
 /* Kernel-level profiling: the per-node timing of SINGA's Graph (Device::SetVerbosity,
  * TimeProfilingDoExec, Graph::PrintTimeProfiling: src/core/scheduler/scheduler.cc:240-295) at
  * kernel granularity.  While enabled, every GEMM / implicit-GEMM launch of this library is
- * bracketed by an event pair on its own stream and tagged ("conv_wgrad", "conv_dgrad",
- * "conv_fwd", "gemm") with its algorithmic FLOP count.  sgh_prof_enable(1) clears old records.
+ * bracketed by an event pair on its own stream and tagged with its algorithmic FLOP count:
+ * "conv_wgrad" / "conv_dgrad" / "conv_fwd" cover the MFMA kernel alone, "conv_*_op" the whole
+ * entry point (weight re-layout, split-K reduction and column-gather kernels included), "gemm"
+ * a dense GEMM.  Records nest.  sgh_prof_enable(1) clears old records.
  * sgh_prof_get waits for record i to finish and returns its tag, duration and work. */
 SGH_API int sgh_prof_enable(int on);
 SGH_API int sgh_prof_count(int *n);

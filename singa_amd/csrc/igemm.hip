@@ -697,11 +697,13 @@ inline WgradPlan plan_wgrad(const sgh_conv_geom *g) {
 
 template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc, bool ZCLASS = false, int WGM = 2>
 inline int launch_igemm(const LA &la, const LB &lb, const ST &st, int M, int N, int Ktotal, int splits,
-                        int chunks_per_split, hipStream_t stream) {
+                        int chunks_per_split, hipStream_t stream, const char *tag = nullptr, double flops = 0) {
   dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
   if (grid.y > 65535u || grid.z > 65535u) return SGH_EUNSUPPORTED;
+  if (tag) sgh_prof_start(tag, flops, stream);  // kernel-level record: this launch only
   hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc, ZCLASS, WGM>), grid, dim3(NT), 0, stream, la, lb, st,
                      Ktotal, chunks_per_split);
+  if (tag) sgh_prof_stop(stream);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -819,7 +821,7 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
   const int RS = g->R * g->S, KP = round_up(g->K, BK);
   const DgradPath path = dgrad_path(g);
   int rc = SGH_OK;
-  sgh_prof_start("conv_dgrad", conv_flops(g), s);
+  sgh_prof_start("conv_dgrad_op", conv_flops(g), s);
 
   if (path == kDgradColumns) {
     float *dcol = static_cast<float *>(workspace);
@@ -829,7 +831,7 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
     auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
     DenseStore st{dcol, long(Ncols), CRS, Ncols, 1.f, 0.f};
     rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DenseStore, false, false>(
-        la, lb, st, CRS, Ncols, g->K, 1, (g->K + BK - 1) / BK, s);
+        la, lb, st, CRS, Ncols, g->K, 1, (g->K + BK - 1) / BK, s, "conv_dgrad", conv_flops(g));
     if (rc == SGH_OK) {
       const long total = long(g->N) * g->C * g->H * g->W;
       long blocks = (total + NT - 1) / NT;
@@ -890,7 +892,7 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
     lb.tab = tab_dev;                                                                                         \
     lb.bytes = bytes_of(size_t(g->N) * g->K * g->P * g->Q);                                                   \
     rc = launch_igemm<BM_, BN_, DgradWLoader<BM_>, DgradDyLoader<BN_>, DgradStore, false, false, true>(       \
-        la, lb, st, M, max_cols, 0, ncls, 0, s);                                                              \
+        la, lb, st, M, max_cols, 0, ncls, 0, s, "conv_dgrad", conv_flops(g));                                 \
   }
     if (tile == 0) SGH_DGRAD_CASE(128, 128)
     else if (tile == 1) SGH_DGRAD_CASE(64, 128)
@@ -908,7 +910,7 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
     auto la = dense_loader<128, false>(Wt, 1, g->C, M, Ktot);
     auto lb = gather_loader<128, true>(dy, to_g(g), KP, g->K, g->P, g->Q, Ncols);
     rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, Ktot / BK, s);
+        la, lb, st, M, Ncols, Ktot, 1, Ktot / BK, s, "conv_dgrad", conv_flops(g));
   }
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
@@ -924,7 +926,7 @@ int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, con
   hipStream_t s = sgh_stream_of(stream);
   float *Wt = static_cast<float *>(workspace);
   const int RS = g->R * g->S, CP = round_up(g->C, BK);
-  sgh_prof_start("conv_fwd", conv_flops(g), s);
+  sgh_prof_start("conv_fwd_op", conv_flops(g), s);
   {
     const long total = long(RS) * CP * g->K;
     long blocks = (total + NT - 1) / NT;
@@ -939,11 +941,11 @@ int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, con
   if (M > 64) {
     auto la = dense_loader<128, false>(Wt, 1, g->K, M, Ktot);
     rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd", conv_flops(g));
   } else {
     auto la = dense_loader<64, false>(Wt, 1, g->K, M, Ktot);
     rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, chunks, s);
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd", conv_flops(g));
   }
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
@@ -963,7 +965,7 @@ int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, 
   float *part = p.splits > 1 ? static_cast<float *>(workspace) : dW;
   SplitStore st{part, g->K, CRS};
   int rc;
-  sgh_prof_start("conv_wgrad", conv_flops(g), s);
+  sgh_prof_start("conv_wgrad_op", conv_flops(g), s);
 #define SGH_WGRAD_CASE(BM_, BN_, WGM_)                                                                             \
   {                                                                                                                \
     WgradDyLoader<BM_> la{dy, g->K, PQ, int(G), bytes_of(size_t(G) * g->K), 0, 0, 0};                              \
@@ -973,7 +975,7 @@ int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, 
     lb.CRS = CRS;                                                                                                  \
     lb.bytes = bytes_of(size_t(g->N) * g->C * g->H * g->W);                                                        \
     rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true, false, WGM_>(       \
-        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s);                                           \
+        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s, "conv_wgrad", conv_flops(g));              \
   }
   if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128, 2)
   else if (p.bm == 64 && p.bn == 256) SGH_WGRAD_CASE(64, 256, 1)

@@ -43,6 +43,7 @@ struct ProfRec {
   hipEvent_t a, b;
 };
 static std::vector<ProfRec> g_prof;
+static std::vector<size_t> g_prof_open;  // indices of records whose stop event is not recorded yet (nesting)
 static bool g_prof_on = false;
 
 bool sgh_prof_on() { return g_prof_on; }
@@ -52,12 +53,14 @@ void sgh_prof_start(const char *tag, double work, hipStream_t s) {
   ProfRec r{tag, work, nullptr, nullptr};
   if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) return;
   (void)hipEventRecord(r.a, s);
+  g_prof_open.push_back(g_prof.size());
   g_prof.push_back(r);
 }
 
 void sgh_prof_stop(hipStream_t s) {
-  if (!g_prof_on || g_prof.empty()) return;
-  (void)hipEventRecord(g_prof.back().b, s);
+  if (!g_prof_on || g_prof_open.empty()) return;
+  (void)hipEventRecord(g_prof[g_prof_open.back()].b, s);
+  g_prof_open.pop_back();
 }
 
 static void prof_clear() {
@@ -66,6 +69,7 @@ static void prof_clear() {
     if (r.b) (void)hipEventDestroy(r.b);
   }
   g_prof.clear();
+  g_prof_open.clear();
 }
 
 // Pool granularity: 256 B up to 4 KiB, then power-of-two classes with four steps per octave
