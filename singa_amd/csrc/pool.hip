@@ -72,6 +72,67 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd(const float *__restrict
   }
 }
 
+// Tiled max-pool backward: one workgroup owns a band of TH rows of one (n, c) plane of dx.
+//   1. the x rows every window touching the band needs are staged in LDS (read from HBM once),
+//   2. each of those windows gets its first-maximum position (flat h * W + w) into LDS,
+//   3. each dx element of the band adds dy over the windows that contain it, in ascending (p, q)
+//      order, when the window's maximum sits on it -- the same order as the CPU scatter loop.
+// x, dy and dx each cross HBM once (plus the band halo of x).
+__global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__restrict__ dy, const float *__restrict__ x,
+                                                              float *__restrict__ dx, PoolG g, int TH, int bands,
+                                                              int max_xrows) {
+  extern __shared__ float smem[];
+  float *xs = smem;                                              // [max_xrows][W]
+  int *widx = reinterpret_cast<int *>(smem + max_xrows * g.W);   // [windows rows][Q]
+  const int plane = blockIdx.x / bands, band = blockIdx.x - plane * bands;
+  const int h0 = band * TH, h1 = min(h0 + TH, g.H);
+  // windows p with [p*sh - ph, p*sh - ph + kh) overlapping [h0, h1)
+  const int lo_num = h0 + g.ph - g.kh + 1;
+  const int p_lo = lo_num <= 0 ? 0 : (lo_num + g.sh - 1) / g.sh;
+  const int p_hi = min((h1 - 1 + g.ph) / g.sh, g.P - 1);
+  const int xr0 = max(p_lo * g.sh - g.ph, 0), xr1 = min(p_hi * g.sh - g.ph + g.kh, g.H);  // x rows [xr0, xr1)
+  const float *xb = x + size_t(plane) * g.H * g.W;
+  const float *db = dy + size_t(plane) * g.P * g.Q;
+  float *ob = dx + size_t(plane) * g.H * g.W;
+  const int nx = (xr1 - xr0) * g.W;
+  for (int i = threadIdx.x; i < nx; i += kBlock) xs[i] = xb[xr0 * g.W + i];
+  __syncthreads();
+  const int np = p_hi - p_lo + 1;
+  for (int i = threadIdx.x; i < np * g.Q; i += kBlock) {
+    const int p = p_lo + i / g.Q, q = i % g.Q;
+    int hs = p * g.sh - g.ph, ws = q * g.sw - g.pw;
+    const int he = min(hs + g.kh, g.H), we = min(ws + g.kw, g.W);
+    hs = max(hs, 0);
+    ws = max(ws, 0);
+    float best = -3.402823466e38f;
+    int bi = -1;
+    for (int h = hs; h < he; ++h)
+      for (int w = ws; w < we; ++w) {
+        const float v = xs[(h - xr0) * g.W + w];
+        if (v > best) {
+          best = v;
+          bi = h * g.W + w;
+        }
+      }
+    widx[i] = bi;
+  }
+  __syncthreads();
+  const int nd = (h1 - h0) * g.W;
+  for (int i = threadIdx.x; i < nd; i += kBlock) {
+    const int h = h0 + i / g.W, w = i % g.W, r = h * g.W + w;
+    const int hp = h + g.ph, wp = w + g.pw;
+    const int pl = hp < g.kh ? 0 : (hp - g.kh) / g.sh + 1;
+    const int ph_ = min(hp / g.sh, g.P - 1);
+    const int ql = wp < g.kw ? 0 : (wp - g.kw) / g.sw + 1;
+    const int qh = min(wp / g.sw, g.Q - 1);
+    float s = 0.f;
+    for (int p = pl; p <= ph_; ++p)
+      for (int q = ql; q <= qh; ++q)
+        if (widx[(p - p_lo) * g.Q + q] == r) s += db[p * g.Q + q];
+    ob[r] = s;
+  }
+}
+
 __device__ __forceinline__ int window_count(const PoolG g, int p, int q, int *hs_, int *he_, int *ws_, int *we_) {
   int hs = p * g.sh - g.ph, ws = q * g.sw - g.pw;
   const int he = min(hs + g.kh, g.H), we = min(ws + g.kw, g.W);
@@ -194,10 +255,24 @@ int sgh_pool_bwd_f32(const sgh_pool_geom *g, const float *dy, const float *x, co
   if (!geom_ok(g) || !dy || !dx) return SGH_EINVAL;
   if (g->is_max && !x) return SGH_EINVAL;
   const size_t total = size_t(g->N) * g->C * g->H * g->W;
-  if (g->is_max)
-    hipLaunchKernelGGL(k_pool_max_bwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
-                       to_g(g), total);
-  else
+  if (g->is_max) {
+    // band height: about 8 dx elements per thread
+    int TH = 2048 / g->W;
+    if (TH < 1) TH = 1;
+    if (TH > g->H) TH = g->H;
+    const int bands = (g->H + TH - 1) / TH;
+    const int max_np = (TH + g->kernel_h - 2) / g->stride_h + 2;
+    const int max_xrows = (max_np - 1) * g->stride_h + g->kernel_h;
+    const size_t lds = (size_t(max_xrows) * g->W + size_t(max_np) * g->Q) * sizeof(float);
+    const size_t blocks = size_t(g->N) * g->C * bands;
+    if (lds <= 48 * 1024 && blocks < 0x7fffffffu && g->W <= 2048) {
+      hipLaunchKernelGGL(k_pool_max_bwd_tiled, dim3((unsigned)blocks), dim3(kBlock), lds, sgh_stream_of(stream), dy, x,
+                         dx, to_g(g), TH, bands, max_xrows);
+    } else {
+      hipLaunchKernelGGL(k_pool_max_bwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
+                         to_g(g), total);
+    }
+  } else
     hipLaunchKernelGGL(k_pool_avg_bwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, dx, to_g(g),
                        total);
   SGH_LAUNCH_CHECK();
