@@ -36,6 +36,12 @@ bool sgh_prof_on();
 void sgh_prof_start(const char *tag, double work, hipStream_t s);
 void sgh_prof_stop(hipStream_t s);
 
+// 3x3 stride-1 weight gradient with a shared LDS input tile (wgrad3x3.hip).  *_run returns
+// SGH_EUNSUPPORTED for geometries it does not cover; *_workspace_bytes is 0 for those.
+size_t sgh_wgrad3x3_workspace_bytes(const sgh_conv_geom *g);
+int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
+                     size_t ws_bytes, hipStream_t s);
+
 // Sum across the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float sgh_wave_sum(float v) {
 #pragma unroll
