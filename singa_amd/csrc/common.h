@@ -42,6 +42,13 @@ size_t sgh_wgrad3x3_workspace_bytes(const sgh_conv_geom *g);
 int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
                      size_t ws_bytes, hipStream_t s);
 
+// 3x3 stride-1 pad-1 data gradient with a shared LDS gradient tile (dgrad3x3.hip).
+// `wt` = weights re-laid as [tap][KP][C], KP = K rounded up to 16.
+bool sgh_dgrad3x3_supported(const sgh_conv_geom *g);
+size_t sgh_dgrad3x3_partial_bytes(const sgh_conv_geom *g);  // scratch for split-reduction partial images
+int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, int KP, float *dx, float *partials,
+                     hipStream_t s);
+
 // Sum across the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float sgh_wave_sum(float v) {
 #pragma unroll

@@ -1,0 +1,323 @@
+// Data gradient of 3x3, stride-1, pad-1 convolutions with an LDS gradient tile shared by all
+// nine taps.
+//
+//   dx[n][c][h][w] = sum_{k,r,s} dy[n][k][h + 1 - r][w + 1 - s] * W[k][c][r][s]
+//
+// GEMM view: M = C (128 per workgroup), N = 128 consecutive pixels of the flattened (n, h, w)
+// index, reduction = (k, tap).  The reduction runs in chunks of 16 output channels k; per chunk
+// the workgroup stages in LDS
+//   dyS[kc][vrow][col]   the dy rows its 128 pixels touch (one halo row above / below, halo
+//                        columns, zero padding materialised).  Rows are addressed in a "virtual
+//                        row" space in which every image owns P + 2 rows (a zero row on top and
+//                        at the bottom), so a tile may straddle image boundaries;
+//   Ws[kc][m]            the 16 x 128 weight slice of ONE tap, double-buffered across taps.
+// Every tap reads its B operand from the same dy tile at a compile-time offset, so the inner loop
+// is nothing but LDS reads and MFMAs: no address arithmetic, no predicates, and each dy element is
+// fetched from global memory once per chunk instead of nine times.
+// 512 threads = 8 wavefronts in a 2 (M) x 4 (N) grid, 64 x 32 per wavefront
+// (v_mfma_f32_32x32x2_f32); two wavefronts per SIMD so that one's staging work overlaps the
+// other's MFMAs.
+#include <stdlib.h>
+
+#include "common.h"
+
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+constexpr int NT = 512;
+constexpr int BN = 128, KC = 16;
+constexpr int kOOB = int(0x80000000u);
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
+}
+
+struct D3Args {
+  const float *dy, *wt;   // wt: re-laid weights [tap][KP][C]
+  float *dx;
+  int N, C, H, W, K, KP;  // P == H, Q == W (3x3, stride 1, pad 1)
+  int total_pix;          // N * H * W
+  int chunks_per_split;   // reduction chunks (16 channels of k each) per grid.z slice
+  long split_stride;      // elements between the partial outputs of consecutive slices
+  unsigned dy_bytes, wt_bytes;
+};
+
+// LOGP: log2 of the LDS row pitch (>= W + 2); VR: virtual rows held per channel.
+// BM: output channels per workgroup (64 or 128; the wavefront tile is (BM/2) x 32).
+template <int BM, int LOGP, int VR>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_dgrad3x3(D3Args a) {
+  constexpr int PA = BM + 4;                // weight tile pitch (16-byte aligned rows for 128-bit LDS writes)
+  constexpr int TM = BM / 64;               // 32-row MFMA tiles per wavefront
+  constexpr int PITCHP = 1 << LOGP;
+  constexpr int VRP = VR * PITCHP;          // floats per channel slab
+  constexpr int CHS = VRP + 4;              // channel stride in LDS
+  constexpr int DSLOTS = KC * VRP / NT;     // dy elements per thread per chunk
+  constexpr int SPT = (DSLOTS + 8) / 9;     // dy slots fetched per tap step
+  static_assert(KC * VRP % NT == 0 && (NT % VRP == 0 || VRP % NT == 0), "slab must tile over the threads");
+
+  extern __shared__ float smem[];
+  float *Ws = smem;                         // [2][KC][PA]
+  float *dyS = smem + 2 * KC * PA;          // [2][KC][CHS]
+
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 wavefronts, 64 x 32 each
+  const int c0 = blockIdx.x * BM;
+  const int pix0 = blockIdx.y * BN;
+  const int HW = a.H * a.W, VH = a.H + 2;
+  const rsrc_t rdy = make_rsrc(a.dy, a.dy_bytes), rw = make_rsrc(a.wt, a.wt_bytes);
+
+  // first virtual row of the slab: the row above the tile's first pixel row
+  const int n_first = pix0 / HW, h_first = (pix0 - n_first * HW) / a.W;
+  const int vbase = n_first * VH + h_first;  // virtual row of dy row (h_first - 1)
+
+  // ---- dy slab loader: per-thread, per-slot constants (tile-invariant across chunks) -------
+  // slab element index i = e * NT + t  ->  kc = i / VRP, within = i % VRP, vr = within >> LOGP,
+  // col = within & (PITCHP - 1);  dy row p = (vbase + vr) % VH - 1 of image (vbase + vr) / VH,
+  // dy column q = col - 1.
+  int goff[DSLOTS];   // element offset relative to channel k0 (negative: always zero)
+  int loff[DSLOTS];   // LDS offset inside a dy buffer
+#pragma unroll
+  for (int e = 0; e < DSLOTS; ++e) {
+    const int i = e * NT + t, kc = i / VRP, within = i - kc * VRP, vr = within >> LOGP, col = within & (PITCHP - 1);
+    const int v = vbase + vr, n = v / VH, p = v - n * VH - 1, q = col - 1;
+    const bool ok = n < a.N && unsigned(p) < unsigned(a.H) && unsigned(q) < unsigned(a.W);
+    goff[e] = ok ? ((n * a.K + kc) * a.H + p) * a.W + q : -1;
+    loff[e] = kc * CHS + within;
+  }
+  auto dy_get = [&](int e, int k0) -> float {
+    const int kc = (e * NT + t) / VRP;
+    const int ok = int(goff[e] >= 0) & int(k0 + kc < a.K);
+    const int m = -ok;
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                         rdy, (((goff[e] + k0 * HW) << 2) & m) | (kOOB & ~m), 0, 0));
+  };
+
+  // ---- weight tile loader: one 128-bit load per thread per tap step ------------------------
+  // (BM == 64: the upper half of the threads has no weight element to fetch)
+  constexpr int WV = BM / 4;                     // float4 per weight row
+  const int w_kc = t / WV, w_m = (t % WV) * 4;   // 16 rows x WV float4
+  auto w_get = [&](int tap, int k0) -> v4f {
+    const int row = tap * a.KP + k0 + w_kc;
+    const int ok = int(c0 + w_m + 3 < a.C) & int(w_kc < KC);
+    const int m = -ok;
+    return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+                                       rw, (((row * a.C + c0 + w_m) << 2) & m) | (kOOB & ~m), 0, 0));
+  };
+  auto w_put = [&](v4f v, float *dst) {
+    if (BM == 128 || w_kc < KC) *reinterpret_cast<v4f *>(dst + w_kc * PA + w_m) = v;
+  };
+
+  // ---- this lane's pixel (B operand column) ------------------------------------------------
+  const int pix = pix0 + wn * 32 + (lane & 31);
+  const int pixc = pix < a.total_pix ? pix : a.total_pix - 1;  // a tail lane computes a valid pixel, stores nothing
+  const int pn = pixc / HW, prem = pixc - pn * HW, ph_ = prem / a.W, pw_ = prem - ph_ * a.W;
+  // LDS offset of tap (r = 2, s = 2); tap (r, s) adds (2 - r) * PITCHP + (2 - s):
+  //   dy row h + 1 - r  ->  virtual row pn*VH + h + 2 - r ; slab column of q = w + 1 - s is w + 2 - s
+  const int boff = (pn * VH + ph_ - vbase) * PITCHP + pw_ + (lane >> 5) * CHS;
+  const int aoff = (lane >> 5) * PA + wm * (BM / 2) + (lane & 31);
+
+  v16f acc[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+
+  const int nchunks = a.KP / KC;
+  const int ch_begin = blockIdx.z * a.chunks_per_split;
+  const int ch_end = min(ch_begin + a.chunks_per_split, nchunks);
+
+  // prologue: the first chunk's dy slab and tap 0's weights
+#pragma unroll
+  for (int e = 0; e < DSLOTS; ++e) dyS[loff[e]] = dy_get(e, ch_begin * KC);
+  w_put(w_get(0, ch_begin * KC), Ws);
+  __syncthreads();
+
+  int dcur = 0, wcur = 0;
+  for (int ch = ch_begin; ch < ch_end; ++ch) {
+    const int k0 = ch * KC, k1 = k0 + KC;   // k1: next chunk (loads past the end are masked)
+    const float *dys = dyS + dcur * (KC * CHS) + boff;
+    float *dyn = dyS + (dcur ^ 1) * (KC * CHS);
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) {
+      const int r = tap / 3, s = tap - r * 3;
+      const int toff = (2 - r) * PITCHP + (2 - s);
+      const float *ws = Ws + wcur * (KC * PA) + aoff;
+      // next step's weights (the next chunk's tap 0 after tap 8) and a share of its dy slab
+      const v4f wnext = tap < 8 ? w_get(tap + 1, k0) : w_get(0, k1);
+      float dl[SPT];
+#pragma unroll
+      for (int j = 0; j < SPT; ++j) {
+        const int e = tap * SPT + j;
+        dl[j] = e < DSLOTS ? dy_get(e < DSLOTS ? e : 0, k1) : 0.f;
+      }
+#pragma unroll
+      for (int kk = 0; kk < KC; kk += 2) {
+        const float b = dys[kk * CHS + toff];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(ws[kk * PA + i * 32], b, acc[i], 0, 0, 0);
+      }
+      w_put(wnext, Ws + (wcur ^ 1) * (KC * PA));
+#pragma unroll
+      for (int j = 0; j < SPT; ++j) {
+        const int e = tap * SPT + j;
+        if (e < DSLOTS) dyn[loff[e]] = dl[j];
+      }
+      __syncthreads();
+      wcur ^= 1;
+    }
+    dcur ^= 1;
+  }
+
+  // epilogue: dx[n][c][h][w], this lane's pixel, rows c0 + wm*64 + i*32 + 8*(v/4) + 4*(lane/32) + v%4
+  if (pix < a.total_pix) {
+    float *o = a.dx + size_t(blockIdx.z) * a.split_stride + size_t(pn) * a.C * HW + prem;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (c < a.C) o[size_t(c) * HW] = acc[i][v];
+      }
+  }
+}
+
+// out[i] = sum over slices (ascending) of part[z][i]
+__global__ __launch_bounds__(256) void k_dgrad3x3_reduce(const float *__restrict__ part, float *__restrict__ out, long n4,
+                                                        int splits) {
+  const long stride = long(gridDim.x) * 256;
+  const v4f *p4 = reinterpret_cast<const v4f *>(part);
+  v4f *o4 = reinterpret_cast<v4f *>(out);
+  for (long i = long(blockIdx.x) * 256 + threadIdx.x; i < n4; i += stride) {
+    v4f s = p4[i];
+    for (int z = 1; z < splits; ++z) s += p4[z * n4 + i];
+    o4[i] = s;
+  }
+}
+
+struct D3Plan {
+  bool ok;
+  int bm, logp, vr, splits, chunks_per_split;
+  size_t lds;
+};
+
+inline D3Plan plan(const sgh_conv_geom *g) {
+  D3Plan p{};
+  p.ok = false;
+  if (g->R != 3 || g->S != 3 || g->stride_h != 1 || g->stride_w != 1 || g->pad_h != 1 || g->pad_w != 1) return p;
+  if (g->C < 64 || g->C % 4 != 0 || g->W + 2 > 64 || g->W < 2) return p;
+  if (getenv("SGH_DGRAD3X3_OFF")) return p;
+  p.logp = g->W + 2 <= 16 ? 4 : (g->W + 2 <= 32 ? 5 : 6);
+  // virtual rows a 128-pixel tile can touch: its pixel rows, one halo row each side, and two
+  // zero rows per image boundary it crosses
+  const int rows = (BN + g->W - 2) / g->W + 1;
+  const int crossings = (BN - 1) / (g->H * g->W) + 1;
+  const int need = rows + 2 + 2 * crossings;
+  if (p.logp == 6) p.vr = 8;
+  else if (p.logp == 5) p.vr = 16;
+  else p.vr = need <= 16 ? 16 : 32;
+  if (need > p.vr) return p;
+  p.bm = (g->C % 128 == 0 || g->C > 192) ? 128 : 64;
+  if (const char *e = getenv("SGH_DGRAD3X3_BM")) p.bm = atoi(e) == 64 ? 64 : 128;
+  const size_t chs = size_t(p.vr) * (1u << p.logp) + 4;
+  p.lds = (size_t(2) * KC * (p.bm + 4) + size_t(2) * KC * chs) * sizeof(float);
+  if (p.lds > 160 * 1024) return p;
+  const size_t lim = size_t(1) << 31;
+  const size_t dx_elems = size_t(g->N) * g->C * g->H * g->W;
+  if (size_t(g->N) * g->K * g->P * g->Q * 4 >= lim || dx_elems * 4 >= lim) return p;
+  if (size_t(g->N) * (g->H + 2) + p.vr >= lim / 64) return p;
+  // split the reduction when the tile grid cannot fill the chip (one workgroup per CU fits);
+  // the partial images are summed in slice order, so results stay run-to-run identical
+  const long tiles = long((g->C + p.bm - 1) / p.bm) * ((long(g->N) * g->H * g->W + BN - 1) / BN);
+  const int nchunks = (g->K + KC - 1) / KC;
+  // (three quarters of the CUs busy with unsplit work beats a full chip that also has to write,
+  // re-read and sum partial images)
+  long s = (3L * sgh_num_cus() / 4 + tiles - 1) / tiles;
+  if (s > nchunks / 4) s = nchunks / 4;
+  if (s > 8) s = 8;
+  if (s < 1) s = 1;
+  if (dx_elems % 4 != 0) s = 1;
+  if (const char *e = getenv("SGH_DGRAD3X3_SPLITS")) s = atoi(e) > 0 ? atoi(e) : s;
+  p.chunks_per_split = int((nchunks + s - 1) / s);
+  p.splits = (nchunks + p.chunks_per_split - 1) / p.chunks_per_split;
+  p.ok = true;
+  return p;
+}
+
+template <int BM, int LOGP, int VR>
+int launch(const D3Args &a, const D3Plan &p, dim3 grid, hipStream_t s) {
+  auto kern = k_dgrad3x3<BM, LOGP, VR>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            160 * 1024) != hipSuccess)
+      return SGH_EUNSUPPORTED;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(NT), p.lds, s, a);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
+}  // namespace
+
+bool sgh_dgrad3x3_supported(const sgh_conv_geom *g) { return plan(g).ok; }
+
+// Extra workspace (bytes, after the re-laid weights) for split-reduction partial images.
+size_t sgh_dgrad3x3_partial_bytes(const sgh_conv_geom *g) {
+  const D3Plan p = plan(g);
+  if (!p.ok || p.splits <= 1) return 0;
+  return size_t(p.splits) * g->N * g->C * g->H * g->W * sizeof(float);
+}
+
+// `wt` holds the weights re-laid as [tap][KP][C] (KP = K rounded up to 16, zero rows beyond K);
+// `partials` is sgh_dgrad3x3_partial_bytes(g) bytes of scratch (may be NULL when that is 0).
+int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, int KP, float *dx, float *partials,
+                     hipStream_t s) {
+  const D3Plan p = plan(g);
+  if (!p.ok) return SGH_EUNSUPPORTED;
+  if (p.splits > 1 && !partials) return SGH_EWORKSPACE;
+  D3Args a;
+  a.dy = dy;
+  a.wt = wt;
+  a.dx = p.splits > 1 ? partials : dx;
+  a.N = g->N;
+  a.C = g->C;
+  a.H = g->H;
+  a.W = g->W;
+  a.K = g->K;
+  a.KP = KP;
+  a.total_pix = g->N * g->H * g->W;
+  a.chunks_per_split = p.chunks_per_split;
+  a.split_stride = long(g->N) * g->C * g->H * g->W;
+  a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 4);
+  a.wt_bytes = unsigned(size_t(9) * KP * g->C * 4);
+  dim3 grid((g->C + p.bm - 1) / p.bm, (a.total_pix + BN - 1) / BN, p.splits);
+  if (grid.y > 65535u) return SGH_EUNSUPPORTED;
+  int rc = SGH_EUNSUPPORTED;
+  sgh_prof_start("conv_dgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
+#define D3_CASE(BM_, LOGP_, VR_) \
+  if (p.bm == BM_ && p.logp == LOGP_ && p.vr == VR_) rc = launch<BM_, LOGP_, VR_>(a, p, grid, s);
+  D3_CASE(128, 6, 8)
+  D3_CASE(64, 6, 8)
+  D3_CASE(128, 5, 16)
+  D3_CASE(64, 5, 16)
+  D3_CASE(128, 4, 16)
+  D3_CASE(64, 4, 16)
+  D3_CASE(128, 4, 32)
+  D3_CASE(64, 4, 32)
+#undef D3_CASE
+  sgh_prof_stop(s);
+  if (rc != SGH_OK) return rc;
+  if (p.splits > 1) {
+    const long n4 = a.split_stride / 4;
+    long blocks = (n4 + 255) / 256;
+    const long cap = long(sgh_num_cus()) * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(k_dgrad3x3_reduce, dim3(int(blocks)), dim3(256), 0, s, partials, dx, n4, p.splits);
+    if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
+  }
+  return SGH_OK;
+}

@@ -755,13 +755,14 @@ inline int pick_tile(const char *env, int M, int N, int z) {
 }
 
 // Which algorithm a dgrad of this geometry uses.
-enum DgradPath { kDgradColumns, kDgradClasses, kDgradGather };
+enum DgradPath { kDgradColumns, kDgradTile3x3, kDgradClasses, kDgradGather };
 
 inline DgradPath dgrad_path(const sgh_conv_geom *g) {
   const size_t RS = size_t(g->R) * g->S;
   // few input channels: the C x pixels output tile would waste most of a 64-row MFMA tile, so run
   // the dense GEMM dcol = W^T * dy (CRS rows) and fold the columns back with a gather
   if (g->C < 32 && RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float) < kMaxOperandBytes) return kDgradColumns;
+  if (sgh_dgrad3x3_supported(g)) return kDgradTile3x3;
   if (g->stride_h * g->stride_w <= kMaxClasses && RS <= size_t(kMaxTaps)) return kDgradClasses;
   return kDgradGather;
 }
@@ -803,7 +804,8 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
     case SGH_CONV_FWD: return RS * round_up(g->C, BK) * g->K * sizeof(float);
     case SGH_CONV_DGRAD:
       if (dgrad_path(g) == kDgradColumns) return RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float);
-      return align256(RS * round_up(g->K, BK) * g->C * sizeof(float)) + align256(sizeof(DgClsTable));
+      return align256(RS * round_up(g->K, BK) * g->C * sizeof(float)) + align256(sizeof(DgClsTable)) +
+             sgh_dgrad3x3_partial_bytes(g);
     case SGH_CONV_WGRAD: {
       const size_t tiled = sgh_wgrad3x3_workspace_bytes(g);
       if (tiled) return tiled;
@@ -841,6 +843,16 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
       if (blocks > cap) blocks = cap;
       hipLaunchKernelGGL(k_col2im_gather, dim3(int(blocks)), dim3(NT), 0, s, dcol, dx, to_g(g), total);
     }
+  } else if (path == kDgradTile3x3) {
+    float *Wt = static_cast<float *>(workspace);
+    const long total = long(RS) * KP * g->C;
+    long blocks = (total + NT - 1) / NT;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
+    float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) +
+                                                align256(size_t(RS) * KP * g->C * sizeof(float)) +
+                                                align256(sizeof(DgClsTable)));
+    rc = sgh_dgrad3x3_run(g, dy, Wt, KP, dx, partials, s);
   } else if (path == kDgradClasses) {
     float *Wc = static_cast<float *>(workspace);
     const size_t wc_bytes = size_t(RS) * KP * g->C * sizeof(float);
