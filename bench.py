@@ -108,6 +108,7 @@ def main():
     t0 = time.perf_counter()
     for _ in range(args.steps):
         net.backward_and_update(fused_update=fused)
+    t_enqueued = time.perf_counter() - t0   # host time to enqueue every launch of the timed steps
     sync()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
@@ -145,6 +146,7 @@ def main():
         "config": {"workload": "%s backward+update, N=%d, 3x224x224, fp32, SGD momentum 0.9" % (args.config, args.batch),
                    "update": "fused multi-tensor" if fused else "per parameter"},
         "roofline": roofline,
+        "host_enqueue_ms_per_step": round(t_enqueued / args.steps * 1e3, 4),
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.config, args.cpu_sample_batch, args.cpu_budget_s)

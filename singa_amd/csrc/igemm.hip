@@ -554,33 +554,42 @@ __global__ __launch_bounds__(NT) void k_weight_relayout_classes(const float *__r
 // Col2im as a gather (the scatter loop of the CPU algorithm turned inside out): one thread per
 // dx element adds the column entries of every tap that maps onto it, in ascending (r, s) order.
 //   dx[n][c][h][w] = sum_{r,s} dcol[(c*R + r)*S + s][n*PQ + p*Q + q],  p*sh = h + ph - r, q*sw = w + pw - s
+// Only the taps of the element's residue class are visited (r = r0, r0 + sh, ...), and the
+// threads of a wavefront take elements of ONE class along w (w = cw + sw * j, j consecutive), so
+// that for a fixed tap they read consecutive q: coalesced reads of dcol, stride-sw writes of dx.
 __global__ __launch_bounds__(NT) void k_col2im_gather(const float *__restrict__ dcol, float *__restrict__ dx, ConvG g,
                                                      long total) {
   const long stride = long(gridDim.x) * NT;
-  const int HW = g.H * g.W, PQ = g.P * g.Q;
+  const int PQ = g.P * g.Q;
   const long ncols = long(g.N) * PQ;
-  for (long i = long(blockIdx.x) * NT + threadIdx.x; i < total; i += stride) {
-    const int w = int(i % g.W);
-    const long t1 = i / g.W;
-    const int h = int(t1 % g.H);
-    const long t2 = t1 / g.H;
+  const int WJ = (g.W + g.sw - 1) / g.sw;  // elements per class along w (the last class may be shorter)
+  const long rowlen = long(WJ) * g.sw;      // iteration space per row: sw classes x WJ
+  const long total_it = long(g.N) * g.C * g.H * rowlen;
+  (void)total;
+  for (long i = long(blockIdx.x) * NT + threadIdx.x; i < total_it; i += stride) {
+    const int it = int(i % rowlen);
+    const long row = i / rowlen;
+    const int cw = it / WJ, j = it - cw * WJ;
+    const int w = cw + g.sw * j;
+    if (w >= g.W) continue;
+    const int h = int(row % g.H);
+    const long t2 = row / g.H;
     const int c = int(t2 % g.C), n = int(t2 / g.C);
-    (void)HW;
+    const int r0 = (h + g.ph) % g.sh, s0 = (w + g.pw) % g.sw;
     float acc = 0.f;
-    for (int r = 0; r < g.R; ++r) {
-      const int hp = h + g.ph - r;
-      if (hp < 0) break;
-      const int p = hp / g.sh;
-      if (p * g.sh != hp || p >= g.P) continue;
-      for (int s = 0; s < g.S; ++s) {
-        const int wp = w + g.pw - s;
-        if (wp < 0) break;
-        const int q = wp / g.sw;
-        if (q * g.sw != wp || q >= g.Q) continue;
-        acc += dcol[long((c * g.R + r) * g.S + s) * ncols + long(n) * PQ + p * g.Q + q];
+    for (int r = r0; r < g.R; r += g.sh) {
+      const int p = (h + g.ph - r) / g.sh;  // exact by construction
+      if (h + g.ph - r < 0) break;
+      if (p >= g.P) continue;
+      const float *src = dcol + long((c * g.R + r) * g.S) * ncols + long(n) * PQ + p * g.Q;
+      for (int s = s0; s < g.S; s += g.sw) {
+        const int wq = w + g.pw - s;
+        if (wq < 0) break;
+        const int q = wq / g.sw;
+        if (q < g.Q) acc += src[long(s) * ncols + q];
       }
     }
-    dx[i] = acc;
+    dx[(row * g.W) + w] = acc;
   }
 }
 
@@ -837,7 +846,7 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
     rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DenseStore, false, false>(
         la, lb, st, CRS, Ncols, g->K, 1, (g->K + BK - 1) / BK, s, "conv_dgrad", conv_flops(g));
     if (rc == SGH_OK) {
-      const long total = long(g->N) * g->C * g->H * g->W;
+      const long total = long(g->N) * g->C * g->H * (long((g->W + g->stride_w - 1) / g->stride_w) * g->stride_w);
       long blocks = (total + NT - 1) / NT;
       const long cap = long(sgh_num_cus()) * 32;
       if (blocks > cap) blocks = cap;

@@ -246,20 +246,39 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     }
 }
 
-// dW[k][c][tap] = sum over splits (ascending) of partial[z][tap][k][c]
+// dW[k][c][tap] = sum over splits of partial[z][tap][k][c], in a fixed order.
+// A workgroup takes 64 consecutive (k, c) pairs.  Its 256 threads form 4 z-lanes x 64 pairs:
+// lane zl sums the splits z = zl, zl + 4, ... (ascending) of all nine taps, the four lane sums are
+// added in lane order, and the 576 results are transposed through LDS so that they leave as one
+// contiguous run.  The summation order depends only on `splits`: results are run-to-run identical.
 __global__ __launch_bounds__(256) void k_wgrad3x3_reduce(const float *__restrict__ part, float *__restrict__ dW, int K,
-                                                       int C, int splits) {
-  const long n = long(K) * C * 9;
-  const long stride = long(gridDim.x) * 256;
+                                                        int C, int splits) {
+  __shared__ float lanes[4][9][64];
+  __shared__ float tile[64 * 9];
   const long KC = long(K) * C;
-  for (long i = long(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
-    // i enumerates (tap, k, c) so that reads are coalesced; the write is the strided one
-    const int tap = int(i / KC);
-    const long kc = i - tap * KC;
-    float s = 0.f;
-    for (int z = 0; z < splits; ++z) s += part[(long(z) * 9 + tap) * KC + kc];
-    dW[kc * 9 + tap] = s;
+  const long kc0 = long(blockIdx.x) * 64;
+  const int e = threadIdx.x & 63, zl = threadIdx.x >> 6;
+  const long kc = kc0 + e;
+  float s[9];
+#pragma unroll
+  for (int tap = 0; tap < 9; ++tap) s[tap] = 0.f;
+  if (kc < KC) {
+    for (int z = zl; z < splits; z += 4) {
+      const float *pz = part + long(z) * 9 * KC + kc;
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap) s[tap] += pz[tap * KC];
+    }
   }
+#pragma unroll
+  for (int tap = 0; tap < 9; ++tap) lanes[zl][tap][e] = s[tap];
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * 9; i += 256) {
+    const int tap = i >> 6, ee = i & 63;
+    tile[ee * 9 + tap] = ((lanes[0][tap][ee] + lanes[1][tap][ee]) + lanes[2][tap][ee]) + lanes[3][tap][ee];
+  }
+  __syncthreads();
+  const long nvalid = (KC - kc0 < 64 ? KC - kc0 : 64) * 9;
+  for (int i = threadIdx.x; i < nvalid; i += 256) dW[kc0 * 9 + i] = tile[i];
 }
 
 struct W3Plan {
@@ -369,9 +388,7 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
 #undef W3_CASE
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
-  const long n = long(g->K) * g->C * 9;
-  long blocks = (n + 255) / 256;
-  if (blocks > 4096) blocks = 4096;
+  const long blocks = (long(g->K) * g->C + 63) / 64;
   hipLaunchKernelGGL(k_wgrad3x3_reduce, dim3(int(blocks)), dim3(256), 0, s, a.part, dW, g->K, g->C, 2 * p.splits);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
