@@ -27,15 +27,12 @@ typedef __amdgpu_buffer_rsrc_t rsrc_t;
 constexpr int NT = 512;
 constexpr int UPIXP = 64;        // padded pixels per unit (k dimension of one unit)
 constexpr int kOOB = int(0x80000000u);
+constexpr int kFar = 0x40000000;  // byte offset past any image (images are < 1 GiB); kFar + kFar = kOOB
+constexpr int TABN = 72;          // window-offset table entries: 64 pixels + the look-ahead of the last k-steps
 
 __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
 }
-__device__ __forceinline__ float buf_ld(rsrc_t r, int elem_off, int ok) {
-  const int m = -ok;
-  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, ((elem_off << 2) & m) | (kOOB & ~m), 0, 0));
-}
-
 struct W3Args {
   const float *dy, *x;
   float *part;           // [splits][9][K][C]
@@ -43,15 +40,23 @@ struct W3Args {
   int RU;                // output rows per unit
   int units_per_image;   // ceil(P / RU)
   int total_units, units_per_split;
-  unsigned dy_bytes, x_bytes;
 };
 
-// LOGP: log2 of the LDS row pitch (>= W + 2); ROWS = RU + 2 slab rows.
+// LOGP: log2 of the LDS row pitch (>= W + 2 * pad_w); ROWS = RU + 2 slab rows.
 // 512 threads = 8 wavefronts: wavefronts 0-3 and 4-7 each tile the same (BM/32) x (BC/32) output
 // block but take the first / second half of every unit's k-steps, and write separate partials
 // (split index 2*z + half).  Two wavefronts per SIMD share one LDS tile, so one wavefront's
 // address arithmetic and memory waits overlap the other's MFMAs (within a single wavefront
 // VALU work does not overlap its own MFMAs).
+//
+// Vector-ALU work per MFMA is kept minimal, because it is paid in MFMA issue slots:
+//   * every staging slot of a thread is "thread constant + unit-uniform term": the thread part is
+//     computed once per kernel, the uniform part on the scalar unit, and the k-step loop is fully
+//     unrolled so that slot indices and LDS write offsets are immediates (one v_add per load);
+//   * image, channel and row bounds are enforced by the buffer descriptor (one per image) and by
+//     an out-of-range offset, not by per-lane predicates;
+//   * the LDS offset of a pixel's 3x3 window comes from a 64-entry table built once per kernel
+//     (one for full units, one for the short last unit of an image).
 template <int BM, int BC, int LOGP, int ROWS>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_wgrad3x3(W3Args a) {
   constexpr int PITCHP = 1 << LOGP;
@@ -61,28 +66,42 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   constexpr int ZPAD = 3 * PITCHP;                   // always-zero area read by the padded pixels of a short unit
   constexpr int WGC = BC / 32, WGM = 4 / WGC;
   static_assert(BM == WGM * 32, "four wavefronts of 32 rows x 32 channels per half");
+  constexpr int CPB = NT >> LOGP;                    // channels staged per pass of the 512 threads
+  static_assert(BC % CPB == 0, "channel tile is a whole number of staging passes");
   constexpr int DSLOTS = BM * UPIXP / NT;            // dy elements per thread per unit
-  constexpr int XSLOTS = (BC * ROWS * PITCHP + NT - 1) / NT;
-  constexpr int G = 2;                               // k-steps per software-pipeline group
-  constexpr int NGMAX = UPIXP / 2 / 2 / G;           // groups per wavefront for a full unit
-  constexpr int DPG = (DSLOTS + NGMAX - 1) / NGMAX + 1;
-  constexpr int XPG = (XSLOTS + NGMAX - 1) / NGMAX + 1;
+  constexpr int XSLOTS = (BC / CPB) * ROWS;          // x elements per thread per unit
+  constexpr int NSMAX = UPIXP / 4;                   // k-steps of one wavefront in a full unit
+  constexpr int NSFIT = 12;                          // the slots are spread over this many k-steps
+  constexpr int DPS = (DSLOTS + NSFIT - 1) / NSFIT;
+  constexpr int XPS = (XSLOTS + NSFIT - 1) / NSFIT;
+  constexpr int LAT = 3;                             // a load issued in k-step i is written to LDS after k-step i + LAT
 
   extern __shared__ float smem[];
   float *dyS = smem;                                  // [2][UPIXP][PA]
-  float *xS = smem + 2 * UPIXP * PA;                  // [2][BC][CHS], then ZPAD zeros, then 64 dummy words
+  float *xS = smem + 2 * UPIXP * PA;                  // [2][BC][CHS]
+  float *zeroS = xS + 2 * XBUF;                       // ZPAD zeros
+  int *tab = reinterpret_cast<int *>(zeroS + ZPAD);   // [2][TABN] window offsets per pixel
 
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int half = wave >> 2, w4 = wave & 3;
   const int wm = w4 / WGC, wc = w4 % WGC;
   const int k0 = blockIdx.x * BM, c0 = blockIdx.y * BC;
   const int u_begin = blockIdx.z * a.units_per_split;
   const int u_end = min(u_begin + a.units_per_split, a.total_units);
-  const rsrc_t rdy = make_rsrc(a.dy, a.dy_bytes), rx = make_rsrc(a.x, a.x_bytes);
   const int PQ = a.P * a.Q, HW = a.H * a.W;
+  const unsigned dy_img_bytes = unsigned(a.K) * PQ * 4u, x_img_bytes = unsigned(a.C) * HW * 4u;
 
-  // the zero area is written once; the slabs (pad columns included) are fully rewritten per unit
+  // the zero area and the pad columns are written once; staging only rewrites the image columns
   for (int i = t; i < 2 * XBUF + ZPAD; i += NT) xS[i] = 0.f;
+  // window offset of pixel `pix` in a full unit (table 0) and in an image's last unit (table 1)
+  if (t < 2 * TABN) {
+    const int which = t >= TABN, pix = t - which * TABN;
+    const int tail_rows = a.P % a.RU;
+    const int upix = (which && tail_rows ? tail_rows : a.RU) * a.Q;
+    const int row = pix / a.Q, q = pix - row * a.Q;
+    tab[t] = pix < upix ? row * PITCHP + q : 0x7fffffff;
+  }
 
   v16f acc[9];
 #pragma unroll
@@ -90,56 +109,65 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
 
-  // ---- per-unit loaders -------------------------------------------------------------------
-  auto unit_geom = [&](int u, int &n, int &p0, int &upix) {
+  // ---- staging roles of this thread (unit independent) ---------------------------------------
+  // dy: pixel t % 64 of output channel k0 + t / 64 + 8 * e           -> dyS[pixel][channel]
+  // x : column t % PITCHP of channel c0 + t / PITCHP + CPB * (e / ROWS), slab row e % ROWS
+  const int pixt = t & (UPIXP - 1), tm = t >> 6;
+  const int td4 = (tm * PQ + pixt) * 4;
+  const int dw_off = pixt * PA + tm;
+  const int tcol = t & (PITCHP - 1), tch = t >> LOGP;
+  const int wcol = tcol - a.pw;
+  // a pad column loads out of range (zero) and rewrites its own zero
+  const int tx4 = unsigned(wcol) < unsigned(a.W) ? (tch * HW + wcol) * 4 : kFar;
+  const int xw_off = tch * CHS + tcol;
+
+  auto unit_geom = [&](int u, int &n, int &p0, int &rows) {
     n = u / a.units_per_image;
     p0 = (u - n * a.units_per_image) * a.RU;
-    const int rows = min(a.RU, a.P - p0);
-    upix = rows * a.Q;
+    rows = min(a.RU, a.P - p0);
   };
-  auto dy_get = [&](int e, int n, int p0, int upix) -> float {
-    const int idx = e * NT + t, pix = idx & (UPIXP - 1), m = idx >> 6;
-    const int ok = int(unsigned(e) < unsigned(DSLOTS)) & int(pix < upix) & int(k0 + m < a.K);
-    return buf_ld(rdy, (n * a.K + k0 + m) * PQ + p0 * a.Q + pix, ok);
+  // byte offsets inside image n; `vd` is the thread part, already out of range for a padded pixel
+  auto dy_voff = [&](int e, int vd, int p0) -> int { return vd + ((k0 + 8 * e) * PQ + p0 * a.Q) * 4; };
+  auto x_voff = [&](int e, int p0) -> int {
+    const int ce = e / ROWS, row = e - ce * ROWS;
+    const int h = p0 - a.ph + row;
+    const int sx = unsigned(h) < unsigned(a.H) ? ((c0 + CPB * ce) * HW + h * a.W) * 4 : kFar;
+    return tx4 + sx;  // kFar + kFar = 2^31, kFar + valid < 2^31 but past any image: both out of range
   };
-  // The staging writes are branch-free: a slot outside the slab goes to a per-lane dummy word, so
-  // that a k-step group stays one straight-line scheduling region.
-  float *const dummy = xS + 2 * XBUF + ZPAD + lane;
-  auto dy_put = [&](int e, float v, float *dst) {
-    const int idx = e * NT + t, pix = idx & (UPIXP - 1), m = idx >> 6;
-    float *p = unsigned(e) < unsigned(DSLOTS) ? dst + pix * PA + m : dummy;
-    *p = v;
+  auto x_dst = [&](int e) -> int {
+    const int ce = e / ROWS, row = e - ce * ROWS;
+    return xw_off + ce * (CPB * CHS) + row * PITCHP;
   };
-  auto x_get = [&](int e, int n, int p0, int live) -> float {
-    const int idx = e * NT + t, col = idx & (PITCHP - 1), rc = idx >> LOGP, c = rc / ROWS, row = rc - c * ROWS;
-    const int h = p0 - a.ph + row, w = col - a.pw;
-    const int ok = live & int(e >= 0) & int(c < BC) & int(c0 + c < a.C) & int(unsigned(h) < unsigned(a.H)) &
-                   int(unsigned(w) < unsigned(a.W));
-    return buf_ld(rx, (n * a.C + c0 + c) * HW + h * a.W + w, ok);
-  };
-  auto x_put = [&](int e, float v, float *dst) {
-    const int idx = e * NT + t, col = idx & (PITCHP - 1), rc = idx >> LOGP, c = rc / ROWS, row = rc - c * ROWS;
-    float *p = (e >= 0) & (c < BC) ? dst + c * CHS + row * PITCHP + col : dummy;
-    *p = v;
+  auto ld = [&](rsrc_t r, int voff) -> float {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, 0, 0));
   };
 
   if (u_begin < u_end) {
-    int n, p0, upix;
-    unit_geom(u_begin, n, p0, upix);
+    int n, p0, rows;
+    unit_geom(u_begin, n, p0, rows);
+    const rsrc_t rdy = make_rsrc(a.dy + size_t(n) * a.K * PQ, dy_img_bytes);
+    const rsrc_t rx = make_rsrc(a.x + size_t(n) * a.C * HW, x_img_bytes);
+    const int vd = pixt < rows * a.Q ? td4 : kOOB;
     __syncthreads();  // zero fill done before the first slab lands
-    for (int e = 0; e < DSLOTS; ++e) dy_put(e, dy_get(e, n, p0, upix), dyS);
-    for (int e = 0; e < XSLOTS; ++e) x_put(e, x_get(e, n, p0, 1), xS);
+#pragma unroll
+    for (int e = 0; e < DSLOTS; ++e) dyS[dw_off + 8 * e] = ld(rdy, dy_voff(e, vd, p0));
+#pragma unroll
+    for (int e = 0; e < XSLOTS; ++e) xS[x_dst(e)] = ld(rx, x_voff(e, p0));
   }
   __syncthreads();
 
   int cur = 0;
   for (int u = u_begin; u < u_end; ++u) {
-    int n, p0, upix;
-    unit_geom(u, n, p0, upix);
-    int nn, np0, nupix;
+    int n, p0, rows;
+    unit_geom(u, n, p0, rows);
+    const int upix = rows * a.Q;
+    int nn, np0, nrows;
     const bool more = u + 1 < u_end;
-    unit_geom(more ? u + 1 : u, nn, np0, nupix);
-    if (!more) nupix = 0;
+    unit_geom(more ? u + 1 : u, nn, np0, nrows);
+    // no next unit: an empty descriptor makes every staging load return zero
+    const rsrc_t rdy = make_rsrc(a.dy + size_t(nn) * a.K * PQ, more ? dy_img_bytes : 0u);
+    const rsrc_t rx = make_rsrc(a.x + size_t(nn) * a.C * HW, more ? x_img_bytes : 0u);
+    const int vd = pixt < nrows * a.Q ? td4 : kOOB;
 
     const float *dcur = dyS + cur * (UPIXP * PA);
     const float *xcur = xS + cur * XBUF;
@@ -149,86 +177,65 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     // this wavefront's share of the unit's k-steps (two pixels each)
     const int ksteps = (upix + 1) >> 1;
     const int khalf = (ksteps + 1) >> 1;
-    const int s_begin = half ? khalf : 0, s_end = half ? ksteps : khalf;
-    const int nsteps = s_end - s_begin;
-    const int ngroups = nsteps / G;
+    const int s_begin = half ? khalf : 0;
+    const int nsteps = half ? ksteps - khalf : khalf;
 
-    // A operand: dyS[pix][m]; B operand: xS[c][pixoff(pix) + r*PITCHP + s]
-    const float *ap = dcur + (lane >> 5) * PA + wm * 32 + (lane & 31);
+    // A operand: dyS[pix][m]; B operand: xS[c][window(pix) + r*PITCHP + s]; pix = 2*step + lane/32
+    const float *ap = dcur + (2 * s_begin + (lane >> 5)) * PA + wm * 32 + (lane & 31);
     const float *bp = xcur + (wc * 32 + (lane & 31)) * CHS;
-    const int zoff = int((xS + 2 * XBUF) - bp);  // this lane's offset of the zero area
-    // running (column, LDS offset) of this lane's pixel: pix = 2*step + lane/32  (Q >= 2)
-    const int pix0 = 2 * s_begin + (lane >> 5);
-    const int row0 = pix0 / a.Q;
-    int q = pix0 - row0 * a.Q, off = row0 * PITCHP + q;
+    const int zoff = int(zeroS - bp);  // this lane's offset of the zero area (beyond every window offset)
+    const int *tb = tab + (rows != a.RU ? TABN : 0) + 2 * s_begin + (lane >> 5);
 
-    // Operand fragments of k-step s+1 are fetched while the MFMAs of k-step s run.
+    // Operand fragments of k-step i+1 are fetched while the MFMAs of k-step i run; the window
+    // offset of k-step i+2 is fetched one step earlier still.
     float av[2], bv[2][9];
-    auto fetch = [&](int step, int buf) {
-      av[buf] = ap[(2 * step) * PA];
+    int tv[3];
+    auto frag = [&](int i, int buf, int tval) {
+      av[buf] = ap[2 * i * PA];
       // a pixel past the unit's end has a zero dy column; its x operand comes from the zero area
       // so that no stale LDS value can meet it
-      const int o = (2 * step + (lane >> 5)) < upix ? off : zoff;
+      const float *w = bp + min(tval, zoff);
 #pragma unroll
       for (int r = 0; r < 3; ++r)
 #pragma unroll
-        for (int s = 0; s < 3; ++s) bv[buf][r * 3 + s] = bp[o + r * PITCHP + s];
-      q += 2;
-      off += 2;
-      if (q >= a.Q) {
-        q -= a.Q;
-        off += PITCHP - a.Q;
-      }
+        for (int s = 0; s < 3; ++s) bv[buf][r * 3 + s] = w[r * PITCHP + s];
     };
     auto mfmas = [&](int buf) {
 #pragma unroll
       for (int i = 0; i < 9; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[buf], bv[buf][i], acc[i], 0, 0, 0);
     };
 
-    fetch(s_begin, 0);
-    // Global loads issued in group g are written to LDS at the end of group g + 1.
-    float pd[DPG], px[XPG];
+    tv[0] = tb[0];
+    tv[1] = tb[2];
+    frag(0, 0, tv[0]);
+    float st[LAT + 1][DPS + XPS];
 #pragma unroll
-    for (int j = 0; j < DPG; ++j) pd[j] = 0.f;
+    for (int i = 0; i < NSMAX + LAT; ++i) {
+      if (i < NSMAX && i < nsteps) {
 #pragma unroll
-    for (int j = 0; j < XPG; ++j) px[j] = 0.f;
-    for (int g = 0; g < ngroups; ++g) {
-      float ld[DPG], lx[XPG];
+        for (int j = 0; j < DPS; ++j)
+          if (i * DPS + j < DSLOTS) st[i % (LAT + 1)][j] = ld(rdy, dy_voff(i * DPS + j, vd, np0));
 #pragma unroll
-      for (int j = 0; j < DPG; ++j) ld[j] = dy_get(g * DPG + j, nn, np0, nupix);
-#pragma unroll
-      for (int j = 0; j < XPG; ++j) lx[j] = x_get(g * XPG + j, nn, np0, int(more));
-#pragma unroll
-      for (int s2 = 0; s2 < G; ++s2) {
-        fetch(s_begin + g * G + s2 + 1, (s2 + 1) & 1);
-        mfmas(s2 & 1);
+        for (int j = 0; j < XPS; ++j)
+          if (i * XPS + j < XSLOTS) st[i % (LAT + 1)][DPS + j] = ld(rx, x_voff(i * XPS + j, np0));
+        tv[(i + 2) % 3] = tb[2 * (i + 2)];
+        frag(i + 1, (i + 1) & 1, tv[(i + 1) % 3]);
+        mfmas(i & 1);
       }
-      // previous group's loads (for g == 0 the slot index is negative: dummy word); written even
-      // when no unit follows -- the other buffer is simply not read again
+      if (i >= LAT && i - LAT < nsteps) {
+        const int w = i - LAT;
 #pragma unroll
-      for (int j = 0; j < DPG; ++j) dy_put((g - 1) * DPG + j, pd[j], dnxt);
+        for (int j = 0; j < DPS; ++j)
+          if (w * DPS + j < DSLOTS) dnxt[dw_off + 8 * (w * DPS + j)] = st[w % (LAT + 1)][j];
 #pragma unroll
-      for (int j = 0; j < XPG; ++j) x_put((g - 1) * XPG + j, px[j], xnxt);
-#pragma unroll
-      for (int j = 0; j < DPG; ++j) pd[j] = ld[j];
-#pragma unroll
-      for (int j = 0; j < XPG; ++j) px[j] = lx[j];
+        for (int j = 0; j < XPS; ++j)
+          if (w * XPS + j < XSLOTS) xnxt[x_dst(w * XPS + j)] = st[w % (LAT + 1)][DPS + j];
+      }
     }
-    if (ngroups > 0) {
-#pragma unroll
-      for (int j = 0; j < DPG; ++j) dy_put((ngroups - 1) * DPG + j, pd[j], dnxt);
-#pragma unroll
-      for (int j = 0; j < XPG; ++j) x_put((ngroups - 1) * XPG + j, px[j], xnxt);
-    }
-    for (int step = s_begin + ngroups * G; step < s_end; ++step) {
-      // fragments sit in buffer 0 here (an even number of steps per group keeps the parity)
-      mfmas(0);
-      fetch(step + 1, 0);
-    }
-    // slots not reached by a short unit's groups
+    // slots not reached by a short unit's k-steps
     if (more) {
-      for (int e = ngroups * DPG; e < DSLOTS; ++e) dy_put(e, dy_get(e, nn, np0, nupix), dnxt);
-      for (int e = ngroups * XPG; e < XSLOTS; ++e) x_put(e, x_get(e, nn, np0, 1), xnxt);
+      for (int e = nsteps * DPS; e < DSLOTS; ++e) dnxt[dw_off + 8 * e] = ld(rdy, dy_voff(e, vd, np0));
+      for (int e = nsteps * XPS; e < XSLOTS; ++e) xnxt[x_dst(e)] = ld(rx, x_voff(e, np0));
     }
     __syncthreads();
     cur ^= 1;
@@ -296,7 +303,9 @@ inline W3Plan plan(const sgh_conv_geom *g) {
   if (getenv("SGH_WGRAD3X3_OFF")) return p;
   // instantiated slabs: pitch 64 x 3 rows (RU 1), pitch 32 x 4 rows (RU 2), pitch 16 x 6 rows (RU 4),
   // pitch 16 x 9 rows (RU 7: a whole 7x7 plane)
-  p.logp = g->W + 2 <= 16 ? 4 : (g->W + 2 <= 32 ? 5 : 6);
+  const int cols = g->W + 2 * g->pad_w;  // slab columns a window can touch
+  if (cols > 64) return p;
+  p.logp = cols <= 16 ? 4 : (cols <= 32 ? 5 : 6);
   if (p.logp == 6) p.ru = 1;
   else if (p.logp == 5) p.ru = 2;
   else p.ru = (7 * g->Q <= UPIXP && g->P >= 7) ? 7 : 4;
@@ -317,10 +326,10 @@ inline W3Plan plan(const sgh_conv_geom *g) {
   p.units_per_split = int((p.total_units + s - 1) / s);
   p.splits = (p.total_units + p.units_per_split - 1) / p.units_per_split;
   const int pitchp = 1 << p.logp, chs = p.rows * pitchp + 1;
-  p.lds = (size_t(2) * UPIXP * (p.bm + 1) + size_t(2) * p.bc * chs + 3 * pitchp + 64) * sizeof(float);
+  p.lds = (size_t(2) * UPIXP * (p.bm + 1) + size_t(2) * p.bc * chs + 3 * pitchp + 2 * TABN) * sizeof(float);
   if (p.lds > 160 * 1024) return p;
-  if (size_t(g->N) * g->K * g->P * g->Q * 4 >= (size_t(1) << 31) || size_t(g->N) * g->C * g->H * g->W * 4 >= (size_t(1) << 31))
-    return p;
+  // staging offsets are 32-bit byte offsets inside one image, with kFar as the out-of-range mark
+  if (size_t(g->K) * g->P * g->Q * 4 >= size_t(kFar) || size_t(g->C) * g->H * g->W * 4 >= size_t(kFar)) return p;
   p.ok = true;
   return p;
 }
@@ -370,8 +379,6 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
   a.units_per_image = p.upi;
   a.total_units = p.total_units;
   a.units_per_split = p.units_per_split;
-  a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 4);
-  a.x_bytes = unsigned(size_t(g->N) * g->C * g->H * g->W * 4);
   dim3 grid((g->K + p.bm - 1) / p.bm, (g->C + p.bc - 1) / p.bc, p.splits);
   int rc = SGH_EUNSUPPORTED;
   sgh_prof_start("conv_wgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
