@@ -30,6 +30,9 @@ typedef __amdgpu_buffer_rsrc_t rsrc_t;
 constexpr int NT = 512;
 constexpr int BN = 128, KC = 16;
 constexpr int kOOB = int(0x80000000u);
+#ifndef D3_LAT
+#define D3_LAT 2
+#endif
 
 __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
@@ -47,6 +50,13 @@ struct D3Args {
 
 // LOGP: log2 of the LDS row pitch (>= W + 2); VR: virtual rows held per channel.
 // BM: output channels per workgroup (64 or 128; the wavefront tile is (BM/2) x 32).
+//
+// The reduction is a flat sequence of tap steps (chunk, tap).  Global loads run LAT steps ahead of
+// their LDS write: the data written at the end of step q (tap q+1's weights, a ninth of the next
+// chunk's dy slab) was requested at the start of step q - LAT and waits in registers, so a
+// request has LAT + 1 steps of MFMA time to return.  Every load address is "thread constant +
+// scalar term" (one vector add); the thread constant is out of range for elements that must read
+// as zero, and K is a multiple of 16, so no per-load predicate is left.
 template <int BM, int LOGP, int VR>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_dgrad3x3(D3Args a) {
   constexpr int PA = BM + 4;                // weight tile pitch (16-byte aligned rows for 128-bit LDS writes)
@@ -56,13 +66,18 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   constexpr int CHS = VRP + 4;              // channel stride in LDS
   constexpr int DSLOTS = KC * VRP / NT;     // dy elements per thread per chunk
   constexpr int SPT = (DSLOTS + 8) / 9;     // dy slots fetched per tap step
+  constexpr int SUB = VRP > NT ? VRP / NT : 1;   // passes of the 512 threads over one channel slab
+  constexpr int KPP = VRP > NT ? 1 : NT / VRP;   // channels covered by one pass
+  constexpr int LAT = D3_LAT;               // tap steps between a load and its LDS write
   static_assert(KC * VRP % NT == 0 && (NT % VRP == 0 || VRP % NT == 0), "slab must tile over the threads");
+  static_assert(9 % (LAT + 1) == 0, "the staging registers rotate with the tap index");
 
   extern __shared__ float smem[];
   float *Ws = smem;                         // [2][KC][PA]
   float *dyS = smem + 2 * KC * PA;          // [2][KC][CHS]
 
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 wavefronts, 64 x 32 each
   const int c0 = blockIdx.x * BM;
   const int pix0 = blockIdx.y * BN;
@@ -73,41 +88,37 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int n_first = pix0 / HW, h_first = (pix0 - n_first * HW) / a.W;
   const int vbase = n_first * VH + h_first;  // virtual row of dy row (h_first - 1)
 
-  // ---- dy slab loader: per-thread, per-slot constants (tile-invariant across chunks) -------
-  // slab element index i = e * NT + t  ->  kc = i / VRP, within = i % VRP, vr = within >> LOGP,
-  // col = within & (PITCHP - 1);  dy row p = (vbase + vr) % VH - 1 of image (vbase + vr) / VH,
-  // dy column q = col - 1.
-  int goff[DSLOTS];   // element offset relative to channel k0 (negative: always zero)
-  int loff[DSLOTS];   // LDS offset inside a dy buffer
+  // ---- dy slab loader ------------------------------------------------------------------------
+  // slot e covers channel kc = (e / SUB) * KPP + tkc and slab element within = (e % SUB) * NT + tw:
+  // virtual row vr = within >> LOGP, column col = within % PITCHP; dy row p = (vbase + vr) % VH - 1
+  // of image (vbase + vr) / VH, dy column q = col - 1.  The byte offset splits into a thread part
+  // g0 (kOOB for halo / padding elements) and the scalar (k0 + (e / SUB) * KPP) * HW * 4.
+  const int tkc = VRP > NT ? 0 : t / VRP, tw = VRP > NT ? t : t % VRP;
+  int g0[SUB];
 #pragma unroll
-  for (int e = 0; e < DSLOTS; ++e) {
-    const int i = e * NT + t, kc = i / VRP, within = i - kc * VRP, vr = within >> LOGP, col = within & (PITCHP - 1);
+  for (int sub = 0; sub < SUB; ++sub) {
+    const int within = sub * NT + tw, vr = within >> LOGP, col = within & (PITCHP - 1);
     const int v = vbase + vr, n = v / VH, p = v - n * VH - 1, q = col - 1;
     const bool ok = n < a.N && unsigned(p) < unsigned(a.H) && unsigned(q) < unsigned(a.W);
-    goff[e] = ok ? ((n * a.K + kc) * a.H + p) * a.W + q : -1;
-    loff[e] = kc * CHS + within;
+    g0[sub] = ok ? (((n * a.K + tkc) * a.H + p) * a.W + q) * 4 : kOOB;
   }
+  const int l0 = tkc * CHS + tw;
   auto dy_get = [&](int e, int k0) -> float {
-    const int kc = (e * NT + t) / VRP;
-    const int ok = int(goff[e] >= 0) & int(k0 + kc < a.K);
-    const int m = -ok;
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                         rdy, (((goff[e] + k0 * HW) << 2) & m) | (kOOB & ~m), 0, 0));
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_raw_buffer_load_b32(rdy, g0[e % SUB] + (k0 + (e / SUB) * KPP) * HW * 4, 0, 0));
   };
+  auto dy_loff = [&](int e) -> int { return l0 + (e / SUB) * KPP * CHS + (e % SUB) * NT; };
 
   // ---- weight tile loader: one 128-bit load per thread per tap step ------------------------
   // (BM == 64: the upper half of the threads has no weight element to fetch)
   constexpr int WV = BM / 4;                     // float4 per weight row
   const int w_kc = t / WV, w_m = (t % WV) * 4;   // 16 rows x WV float4
+  const int w0 = (c0 + w_m + 3 < a.C) && (w_kc < KC) ? (w_kc * a.C + c0 + w_m) * 4 : kOOB;
   auto w_get = [&](int tap, int k0) -> v4f {
-    const int row = tap * a.KP + k0 + w_kc;
-    const int ok = int(c0 + w_m + 3 < a.C) & int(w_kc < KC);
-    const int m = -ok;
-    return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
-                                       rw, (((row * a.C + c0 + w_m) << 2) & m) | (kOOB & ~m), 0, 0));
+    return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rw, w0 + (tap * a.KP + k0) * a.C * 4, 0, 0));
   };
   auto w_put = [&](v4f v, float *dst) {
-    if (BM == 128 || w_kc < KC) *reinterpret_cast<v4f *>(dst + w_kc * PA + w_m) = v;
+    if (BM == 128 || wave < 4) *reinterpret_cast<v4f *>(dst + w_kc * PA + w_m) = v;
   };
 
   // ---- this lane's pixel (B operand column) ------------------------------------------------
@@ -129,15 +140,33 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int ch_begin = blockIdx.z * a.chunks_per_split;
   const int ch_end = min(ch_begin + a.chunks_per_split, nchunks);
 
-  // prologue: the first chunk's dy slab and tap 0's weights
+  // Staging registers.  Step q (tap q % 9 of chunk q / 9) requests what step q + LAT writes: the
+  // weights of step q + LAT + 1 and dy slots [td * SPT, (td + 1) * SPT) of the chunk after step
+  // q + LAT's, td = (q + LAT) % 9.  Requests past the last chunk land in buffers nobody reads.
+  v4f wst[LAT + 1];
+  float dst[LAT + 1][SPT];
+  auto request = [&](int tq, int ch) {  // tq: tap index relative to chunk ch (negative during warm-up)
+    const int slot = ((tq % (LAT + 1)) + LAT + 1) % (LAT + 1);
+    const int qw = tq + LAT + 1, qd = tq + LAT;
+    wst[slot] = w_get(qw % 9, (ch + qw / 9) * KC);
 #pragma unroll
-  for (int e = 0; e < DSLOTS; ++e) dyS[loff[e]] = dy_get(e, ch_begin * KC);
+    for (int j = 0; j < SPT; ++j) {
+      const int e = (qd % 9) * SPT + j;
+      if (e < DSLOTS) dst[slot][j] = dy_get(e, (ch + 1 + qd / 9) * KC);
+    }
+  };
+
+  // prologue: the first chunk's dy slab and tap 0's weights, then the requests of the LAT steps
+  // that would have preceded step 0
+#pragma unroll
+  for (int e = 0; e < DSLOTS; ++e) dyS[dy_loff(e)] = dy_get(e, ch_begin * KC);
   w_put(w_get(0, ch_begin * KC), Ws);
+#pragma unroll
+  for (int tq = -LAT; tq < 0; ++tq) request(tq, ch_begin);
   __syncthreads();
 
   int dcur = 0, wcur = 0;
   for (int ch = ch_begin; ch < ch_end; ++ch) {
-    const int k0 = ch * KC, k1 = k0 + KC;   // k1: next chunk (loads past the end are masked)
     const float *dys = dyS + dcur * (KC * CHS) + boff;
     float *dyn = dyS + (dcur ^ 1) * (KC * CHS);
 #pragma unroll
@@ -145,14 +174,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
       const int r = tap / 3, s = tap - r * 3;
       const int toff = (2 - r) * PITCHP + (2 - s);
       const float *ws = Ws + wcur * (KC * PA) + aoff;
-      // next step's weights (the next chunk's tap 0 after tap 8) and a share of its dy slab
-      const v4f wnext = tap < 8 ? w_get(tap + 1, k0) : w_get(0, k1);
-      float dl[SPT];
-#pragma unroll
-      for (int j = 0; j < SPT; ++j) {
-        const int e = tap * SPT + j;
-        dl[j] = e < DSLOTS ? dy_get(e < DSLOTS ? e : 0, k1) : 0.f;
-      }
+      request(tap, ch);
 #pragma unroll
       for (int kk = 0; kk < KC; kk += 2) {
         const float b = dys[kk * CHS + toff];
@@ -160,11 +182,13 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         for (int i = 0; i < TM; ++i)
           acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(ws[kk * PA + i * 32], b, acc[i], 0, 0, 0);
       }
-      w_put(wnext, Ws + (wcur ^ 1) * (KC * PA));
+      // what step (tap - LAT) requested: tap + 1's weights and this tap's share of the next slab
+      const int slot = ((tap - LAT) % (LAT + 1) + LAT + 1) % (LAT + 1);
+      w_put(wst[slot], Ws + (wcur ^ 1) * (KC * PA));
 #pragma unroll
       for (int j = 0; j < SPT; ++j) {
         const int e = tap * SPT + j;
-        if (e < DSLOTS) dyn[loff[e]] = dl[j];
+        if (e < DSLOTS) dyn[dy_loff(e)] = dst[slot][j];
       }
       __syncthreads();
       wcur ^= 1;
@@ -208,7 +232,7 @@ inline D3Plan plan(const sgh_conv_geom *g) {
   D3Plan p{};
   p.ok = false;
   if (g->R != 3 || g->S != 3 || g->stride_h != 1 || g->stride_w != 1 || g->pad_h != 1 || g->pad_w != 1) return p;
-  if (g->C < 64 || g->C % 4 != 0 || g->W + 2 > 64 || g->W < 2) return p;
+  if (g->C < 64 || g->C % 4 != 0 || g->K % KC != 0 || g->W + 2 > 64 || g->W < 2) return p;
   if (getenv("SGH_DGRAD3X3_OFF")) return p;
   p.logp = g->W + 2 <= 16 ? 4 : (g->W + 2 <= 32 ? 5 : 6);
   // virtual rows a 128-pixel tile can touch: its pixel rows, one halo row each side, and two
