@@ -15,8 +15,9 @@
 // is nothing but LDS reads and MFMAs: no address arithmetic, no predicates, and each dy element is
 // fetched from global memory once per chunk instead of nine times.
 // 512 threads = 8 wavefronts in a 2 (M) x 4 (N) grid, 64 x 32 per wavefront
-// (v_mfma_f32_32x32x2_f32); two wavefronts per SIMD so that one's staging work overlaps the
-// other's MFMAs.
+// (v_mfma_f32_32x32x2_f32).  The LDS footprint is at most 80 KB and the kernel needs fewer than
+// 128 registers, so two workgroups (four wavefronts per SIMD) share a CU and one's staging work
+// and barriers overlap the other's MFMAs.
 #include <stdlib.h>
 
 #include "common.h"
@@ -58,12 +59,12 @@ struct D3Args {
 // scalar term" (one vector add); the thread constant is out of range for elements that must read
 // as zero, and K is a multiple of 16, so no per-load predicate is left.
 template <int BM, int LOGP, int VR>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_dgrad3x3(D3Args a) {
-  constexpr int PA = BM + 4;                // weight tile pitch (16-byte aligned rows for 128-bit LDS writes)
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void k_dgrad3x3(D3Args a) {
+  constexpr int PA = BM;                    // weight tile pitch
   constexpr int TM = BM / 64;               // 32-row MFMA tiles per wavefront
   constexpr int PITCHP = 1 << LOGP;
   constexpr int VRP = VR * PITCHP;          // floats per channel slab
-  constexpr int CHS = VRP + 4;              // channel stride in LDS
+  constexpr int CHS = VRP;                   // channel stride in LDS (a wavefront's two 32-lane halves are served separately)
   constexpr int DSLOTS = KC * VRP / NT;     // dy elements per thread per chunk
   constexpr int SPT = (DSLOTS + 8) / 9;     // dy slots fetched per tap step
   constexpr int SUB = VRP > NT ? VRP / NT : 1;   // passes of the 512 threads over one channel slab
@@ -246,8 +247,8 @@ inline D3Plan plan(const sgh_conv_geom *g) {
   if (need > p.vr) return p;
   p.bm = (g->C % 128 == 0 || g->C > 192) ? 128 : 64;
   if (const char *e = getenv("SGH_DGRAD3X3_BM")) p.bm = atoi(e) == 64 ? 64 : 128;
-  const size_t chs = size_t(p.vr) * (1u << p.logp) + 4;
-  p.lds = (size_t(2) * KC * (p.bm + 4) + size_t(2) * KC * chs) * sizeof(float);
+  const size_t chs = size_t(p.vr) * (1u << p.logp);
+  p.lds = (size_t(2) * KC * (p.bm) + size_t(2) * KC * chs) * sizeof(float);
   if (p.lds > 160 * 1024) return p;
   const size_t lim = size_t(1) << 31;
   const size_t dx_elems = size_t(g->N) * g->C * g->H * g->W;
