@@ -44,10 +44,10 @@ struct W3Args {
 
 // LOGP: log2 of the LDS row pitch (>= W + 2 * pad_w); ROWS = RU + 2 slab rows.
 // 512 threads = 8 wavefronts: wavefronts 0-3 and 4-7 each tile the same (BM/32) x (BC/32) output
-// block but take the first / second half of every unit's k-steps, and write separate partials
-// (split index 2*z + half).  Two wavefronts per SIMD share one LDS tile, so one wavefront's
-// address arithmetic and memory waits overlap the other's MFMAs (within a single wavefront
-// VALU work does not overlap its own MFMAs).
+// block but take the first / second half of every unit's k-steps; their accumulators are summed
+// through LDS at the end.  Two wavefronts per SIMD share one LDS tile, so one wavefront's address
+// arithmetic and memory waits overlap the other's MFMAs (within a single wavefront VALU work does
+// not overlap its own MFMAs).
 //
 // Vector-ALU work per MFMA is kept minimal, because it is paid in MFMA issue slots:
 //   * every staging slot of a thread is "thread constant + unit-uniform term": the thread part is
@@ -241,36 +241,76 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     cur ^= 1;
   }
 
-  // partial[2*z + half][tap][k][c]
-  float *pz = a.part + size_t(blockIdx.z * 2 + half) * 9 * a.K * a.C;
+  // The two halves' accumulators are summed through LDS (the staging buffers are free now):
+  // the first half ends up owning taps 0-4 and the second taps 5-8, so that one partial per
+  // workgroup goes to memory and both halves share the stores.
+  {
+    constexpr int T0 = 5;  // taps kept by the first half
+    float *xch = smem + lane;
+    const int wbase = w4 * 16 * 64;
+    if (half == 1) {
 #pragma unroll
-  for (int i = 0; i < 9; ++i)
+      for (int i = 0; i < T0; ++i)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int m = k0 + wm * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-      const int c = c0 + wc * 32 + (lane & 31);
-      if (m < a.K && c < a.C) pz[(size_t(i) * a.K + m) * a.C + c] = acc[i][v];
+        for (int v = 0; v < 16; ++v) xch[(i * 4 * 16 + v) * 64 + wbase] = acc[i][v];
     }
+    __syncthreads();
+    if (half == 0) {
+#pragma unroll
+      for (int i = 0; i < T0; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][v] += xch[(i * 4 * 16 + v) * 64 + wbase];
+    }
+    __syncthreads();
+    if (half == 0) {
+#pragma unroll
+      for (int i = T0; i < 9; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) xch[((i - T0) * 4 * 16 + v) * 64 + wbase] = acc[i][v];
+    }
+    __syncthreads();
+    if (half == 1) {
+#pragma unroll
+      for (int i = T0; i < 9; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][v] += xch[((i - T0) * 4 * 16 + v) * 64 + wbase];
+    }
+    // partial[z][tap][k][c]
+    float *pz = a.part + size_t(blockIdx.z) * 9 * a.K * a.C;
+    const int c = c0 + wc * 32 + (lane & 31);
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+      if ((i < T0) != (half == 0)) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = k0 + wm * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (m < a.K && c < a.C) pz[(size_t(i) * a.K + m) * a.C + c] = acc[i][v];
+      }
+    }
+  }
 }
 
 // dW[k][c][tap] = sum over splits of partial[z][tap][k][c], in a fixed order.
-// A workgroup takes 64 consecutive (k, c) pairs.  Its 256 threads form 4 z-lanes x 64 pairs:
-// lane zl sums the splits z = zl, zl + 4, ... (ascending) of all nine taps, the four lane sums are
-// added in lane order, and the 576 results are transposed through LDS so that they leave as one
-// contiguous run.  The summation order depends only on `splits`: results are run-to-run identical.
+// A workgroup takes EP consecutive (k, c) pairs.  Its 256 threads form ZL = 256 / EP z-lanes x EP
+// pairs: lane zl sums the splits z = zl, zl + ZL, ... (ascending) of all nine taps, the lane sums
+// are added in lane order, and the 9 * EP results are transposed through LDS so that they leave as
+// one contiguous run.  EP is chosen from the layer shape alone, so the summation order depends
+// only on the shape: results are run-to-run identical.
+template <int EP>
 __global__ __launch_bounds__(256) void k_wgrad3x3_reduce(const float *__restrict__ part, float *__restrict__ dW, int K,
                                                         int C, int splits) {
-  __shared__ float lanes[4][9][64];
-  __shared__ float tile[64 * 9];
+  constexpr int ZL = 256 / EP;
+  __shared__ float lanes[ZL][9][EP];
+  __shared__ float tile[EP * 9];
   const long KC = long(K) * C;
-  const long kc0 = long(blockIdx.x) * 64;
-  const int e = threadIdx.x & 63, zl = threadIdx.x >> 6;
+  const long kc0 = long(blockIdx.x) * EP;
+  const int e = threadIdx.x % EP, zl = threadIdx.x / EP;
   const long kc = kc0 + e;
   float s[9];
 #pragma unroll
   for (int tap = 0; tap < 9; ++tap) s[tap] = 0.f;
   if (kc < KC) {
-    for (int z = zl; z < splits; z += 4) {
+    for (int z = zl; z < splits; z += ZL) {
       const float *pz = part + long(z) * 9 * KC + kc;
 #pragma unroll
       for (int tap = 0; tap < 9; ++tap) s[tap] += pz[tap * KC];
@@ -279,12 +319,15 @@ __global__ __launch_bounds__(256) void k_wgrad3x3_reduce(const float *__restrict
 #pragma unroll
   for (int tap = 0; tap < 9; ++tap) lanes[zl][tap][e] = s[tap];
   __syncthreads();
-  for (int i = threadIdx.x; i < 64 * 9; i += 256) {
-    const int tap = i >> 6, ee = i & 63;
-    tile[ee * 9 + tap] = ((lanes[0][tap][ee] + lanes[1][tap][ee]) + lanes[2][tap][ee]) + lanes[3][tap][ee];
+  for (int i = threadIdx.x; i < EP * 9; i += 256) {
+    const int tap = i / EP, ee = i % EP;
+    float r = lanes[0][tap][ee];
+#pragma unroll
+    for (int l = 1; l < ZL; ++l) r += lanes[l][tap][ee];
+    tile[ee * 9 + tap] = r;
   }
   __syncthreads();
-  const long nvalid = (KC - kc0 < 64 ? KC - kc0 : 64) * 9;
+  const long nvalid = (KC - kc0 < EP ? KC - kc0 : EP) * 9;
   for (int i = threadIdx.x; i < nvalid; i += 256) dW[kc0 * 9 + i] = tile[i];
 }
 
@@ -327,7 +370,7 @@ inline W3Plan plan(const sgh_conv_geom *g) {
   p.splits = (p.total_units + p.units_per_split - 1) / p.units_per_split;
   const int pitchp = 1 << p.logp, chs = p.rows * pitchp + 1;
   p.lds = (size_t(2) * UPIXP * (p.bm + 1) + size_t(2) * p.bc * chs + 3 * pitchp + 2 * TABN) * sizeof(float);
-  if (p.lds > 160 * 1024) return p;
+  if (p.lds > 160 * 1024 || p.lds < size_t(5) * 4096 * sizeof(float)) return p;  // (the epilogue exchanges 5 taps through LDS)
   // staging offsets are 32-bit byte offsets inside one image, with kFar as the out-of-range mark
   if (size_t(g->K) * g->P * g->Q * 4 >= size_t(kFar) || size_t(g->C) * g->H * g->W * 4 >= size_t(kFar)) return p;
   p.ok = true;
@@ -352,7 +395,7 @@ int launch(const W3Args &a, const W3Plan &p, dim3 grid, hipStream_t s) {
 
 size_t sgh_wgrad3x3_workspace_bytes(const sgh_conv_geom *g) {
   const W3Plan p = plan(g);
-  return p.ok ? size_t(2) * p.splits * 9 * g->K * g->C * sizeof(float) : 0;
+  return p.ok ? size_t(p.splits) * 9 * g->K * g->C * sizeof(float) : 0;
 }
 
 // Returns SGH_EUNSUPPORTED when the geometry is not covered (the caller then uses the generic path).
@@ -360,7 +403,7 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
                      size_t ws_bytes, hipStream_t s) {
   const W3Plan p = plan(g);
   if (!p.ok) return SGH_EUNSUPPORTED;
-  const size_t need = size_t(2) * p.splits * 9 * g->K * g->C * sizeof(float);
+  const size_t need = size_t(p.splits) * 9 * g->K * g->C * sizeof(float);
   if (!workspace || ws_bytes < need) return SGH_EWORKSPACE;
   W3Args a;
   a.dy = dy;
@@ -395,7 +438,14 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
 #undef W3_CASE
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
-  const long blocks = (long(g->K) * g->C + 63) / 64;
-  hipLaunchKernelGGL(k_wgrad3x3_reduce, dim3(int(blocks)), dim3(256), 0, s, a.part, dW, g->K, g->C, 2 * p.splits);
+  // pairs per reduction workgroup: small layers take fewer pairs and more z-lanes per workgroup
+  const long kc = long(g->K) * g->C;
+  const int cus = sgh_num_cus();
+  if (kc / 64 >= cus)
+    hipLaunchKernelGGL(k_wgrad3x3_reduce<64>, dim3(int((kc + 63) / 64)), dim3(256), 0, s, a.part, dW, g->K, g->C, p.splits);
+  else if (kc / 32 >= cus)
+    hipLaunchKernelGGL(k_wgrad3x3_reduce<32>, dim3(int((kc + 31) / 32)), dim3(256), 0, s, a.part, dW, g->K, g->C, p.splits);
+  else
+    hipLaunchKernelGGL(k_wgrad3x3_reduce<16>, dim3(int((kc + 15) / 16)), dim3(256), 0, s, a.part, dW, g->K, g->C, p.splits);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
