@@ -1,17 +1,18 @@
-// Weight gradient of 3x3 stride-1 convolutions with an LDS input tile shared by all nine taps.
+// Weight gradient of 3x3 convolutions (stride 1 or 2) with an LDS input tile shared by all nine taps.
 //
-//   dW[k][c][r][s] = sum_{n,p,q} dy[n][k][p][q] * x[n][c][p - ph + r][q - pw + s]
+//   dW[k][c][r][s] = sum_{n,p,q} dy[n][k][p][q] * x[n][c][p*stride - ph + r][q*stride - pw + s]
 //
 // A workgroup owns BM output channels x BC input channels x 9 taps and walks "units" of the
 // reduction: RU consecutive output rows of one image (<= 64 pixels).  Per unit it stages in LDS
 //   dyS[pixel][m]            the BM x (RU*Q) slice of dy (MFMA A operand, k = pixel),
-//   xS[c][row][col]          the BC x (RU+2) x (W+2) input slab, zero padding materialised,
-// and every tap (r, s) reads its B operand from the SAME slab at offset r*pitch + s.  Each input
-// element is therefore fetched once per unit instead of once per tap, the address arithmetic of an
-// im2col gather disappears from the inner loop, and one operand fetch feeds nine MFMAs.
+//   xS[c][row][col]          the BC x ((RU-1)*stride+3) x (W+2) input slab, zero padding materialised,
+// and every tap (r, s) reads its B operand from the SAME slab at offset r*pitch + s from the
+// pixel's window origin.  Each input element is therefore fetched once per unit instead of once
+// per tap, the address arithmetic of an im2col gather disappears from the inner loop, and one
+// operand fetch feeds nine MFMAs.
 // The four wavefronts tile (BM/32) x (BC/32); each holds 9 accumulator tiles of 32x32
 // (v_mfma_f32_32x32x2_f32: 144 accumulator registers).  The next unit's global loads are spread
-// over the k-step groups of the current unit and land in the other LDS buffer.
+// over the k-steps of the current unit and land in the other LDS buffer.
 //
 // The reduction is split over workgroups (grid.z); partials are written as [split][tap][K][C] and
 // summed in ascending split order by k_wgrad3x3_reduce: results are run-to-run identical.
@@ -36,7 +37,7 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
 struct W3Args {
   const float *dy, *x;
   float *part;           // [splits][9][K][C]
-  int N, C, H, W, K, P, Q, ph, pw;
+  int N, C, H, W, K, P, Q, ph, pw, stride;
   int RU;                // output rows per unit
   int units_per_image;   // ceil(P / RU)
   int total_units, units_per_split;
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const int tail_rows = a.P % a.RU;
     const int upix = (which && tail_rows ? tail_rows : a.RU) * a.Q;
     const int row = pix / a.Q, q = pix - row * a.Q;
-    tab[t] = pix < upix ? row * PITCHP + q : 0x7fffffff;
+    tab[t] = pix < upix ? (row * PITCHP + q) * a.stride : 0x7fffffff;
   }
 
   v16f acc[9];
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   auto dy_voff = [&](int e, int vd, int p0) -> int { return vd + ((k0 + 8 * e) * PQ + p0 * a.Q) * 4; };
   auto x_voff = [&](int e, int p0) -> int {
     const int ce = e / ROWS, row = e - ce * ROWS;
-    const int h = p0 - a.ph + row;
+    const int h = p0 * a.stride - a.ph + row;
     const int sx = unsigned(h) < unsigned(a.H) ? ((c0 + CPB * ce) * HW + h * a.W) * 4 : kFar;
     return tx4 + sx;  // kFar + kFar = 2^31, kFar + valid < 2^31 but past any image: both out of range
   };
@@ -340,20 +341,27 @@ struct W3Plan {
 inline W3Plan plan(const sgh_conv_geom *g) {
   W3Plan p{};
   p.ok = false;
-  if (g->R != 3 || g->S != 3 || g->stride_h != 1 || g->stride_w != 1) return p;
+  if (g->R != 3 || g->S != 3 || g->stride_h != g->stride_w || (g->stride_h != 1 && g->stride_h != 2)) return p;
+  const int st = g->stride_h;
   if (g->pad_h > 2 || g->pad_w > 2) return p;
   if (g->W + 2 > 64 || g->Q < 2 || g->Q > 64 || g->C < 32 || g->K < 64) return p;
   if (getenv("SGH_WGRAD3X3_OFF")) return p;
-  // instantiated slabs: pitch 64 x 3 rows (RU 1), pitch 32 x 4 rows (RU 2), pitch 16 x 6 rows (RU 4),
-  // pitch 16 x 9 rows (RU 7: a whole 7x7 plane)
+  // instantiated slabs, stride 1: pitch 64 x 3 rows (RU 1), pitch 32 x 4 rows (RU 2), pitch 16 x 6 rows
+  // (RU 4), pitch 16 x 9 rows (RU 7: a whole 7x7 plane); stride 2: pitch 64 x 5 rows (RU 2), pitch 32 x 9
+  // rows (RU 4), pitch 16 x 15 rows (RU 7)
   const int cols = g->W + 2 * g->pad_w;  // slab columns a window can touch
   if (cols > 64) return p;
   p.logp = cols <= 16 ? 4 : (cols <= 32 ? 5 : 6);
-  if (p.logp == 6) p.ru = 1;
-  else if (p.logp == 5) p.ru = 2;
-  else p.ru = (7 * g->Q <= UPIXP && g->P >= 7) ? 7 : 4;
+  if (st == 1) {
+    if (p.logp == 6) p.ru = 1;
+    else if (p.logp == 5) p.ru = 2;
+    else p.ru = (7 * g->Q <= UPIXP && g->P >= 7) ? 7 : 4;
+  } else {
+    p.ru = p.logp == 6 ? 2 : (p.logp == 5 ? 4 : 7);
+    if (g->K < 128) return p;  // only the 128 x 32 tile is instantiated for the taller stride-2 slabs
+  }
   if (p.ru > g->P || p.ru * g->Q > UPIXP) return p;
-  p.rows = p.ru + 2;
+  p.rows = (p.ru - 1) * st + 3;
   p.bm = g->K >= 128 ? 128 : 64;
   p.bc = p.bm == 128 ? 32 : 64;
   if (p.bc == 64 && g->C < 64) return p;
@@ -418,6 +426,7 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
   a.Q = g->Q;
   a.ph = g->pad_h;
   a.pw = g->pad_w;
+  a.stride = g->stride_h;
   a.RU = p.ru;
   a.units_per_image = p.upi;
   a.total_units = p.total_units;
@@ -435,6 +444,9 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
   W3_CASE(64, 64, 4, 6)
   W3_CASE(128, 32, 4, 9)
   W3_CASE(64, 64, 4, 9)
+  W3_CASE(128, 32, 6, 5)
+  W3_CASE(128, 32, 5, 9)
+  W3_CASE(128, 32, 4, 15)
 #undef W3_CASE
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
