@@ -73,63 +73,84 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd(const float *__restrict
 }
 
 // Tiled max-pool backward: one workgroup owns a band of TH rows of one (n, c) plane of dx.
-//   1. the x rows every window touching the band needs are staged in LDS (read from HBM once),
+//   1. the x rows every window touching the band needs and the dy rows of those windows are
+//      staged in LDS (both are contiguous runs of the plane: 128-bit copies when aligned),
 //   2. each of those windows gets its first-maximum position (flat h * W + w) into LDS,
 //   3. each dx element of the band adds dy over the windows that contain it, in ascending (p, q)
 //      order, when the window's maximum sits on it -- the same order as the CPU scatter loop.
+// The 256 threads form 64 columns x 4 rows, so no per-element division is needed: a thread's
+// column window range is fixed, and the per-row window range is computed once per band row.
 // x, dy and dx each cross HBM once (plus the band halo of x).
 __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__restrict__ dy, const float *__restrict__ x,
                                                               float *__restrict__ dx, PoolG g, int TH, int bands,
-                                                              int max_xrows) {
+                                                              int max_xrows, int max_np) {
   extern __shared__ float smem[];
-  float *xs = smem;                                              // [max_xrows][W]
-  int *widx = reinterpret_cast<int *>(smem + max_xrows * g.W);   // [windows rows][Q]
+  float *xs = smem;                                               // [max_xrows][W]
+  float *ds = xs + max_xrows * g.W;                               // [max_np][Q]
+  int *widx = reinterpret_cast<int *>(ds + max_np * g.Q);         // [max_np][Q]
+  int *prange = widx + max_np * g.Q;                              // [TH][2]: first / last window row of a band row
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int plane = blockIdx.x / bands, band = blockIdx.x - plane * bands;
   const int h0 = band * TH, h1 = min(h0 + TH, g.H);
   // windows p with [p*sh - ph, p*sh - ph + kh) overlapping [h0, h1)
   const int lo_num = h0 + g.ph - g.kh + 1;
   const int p_lo = lo_num <= 0 ? 0 : (lo_num + g.sh - 1) / g.sh;
   const int p_hi = min((h1 - 1 + g.ph) / g.sh, g.P - 1);
-  const int xr0 = max(p_lo * g.sh - g.ph, 0), xr1 = min(p_hi * g.sh - g.ph + g.kh, g.H);  // x rows [xr0, xr1)
-  const float *xb = x + size_t(plane) * g.H * g.W;
-  const float *db = dy + size_t(plane) * g.P * g.Q;
-  float *ob = dx + size_t(plane) * g.H * g.W;
-  const int nx = (xr1 - xr0) * g.W;
-  for (int i = threadIdx.x; i < nx; i += kBlock) xs[i] = xb[xr0 * g.W + i];
-  __syncthreads();
   const int np = p_hi - p_lo + 1;
-  for (int i = threadIdx.x; i < np * g.Q; i += kBlock) {
-    const int p = p_lo + i / g.Q, q = i % g.Q;
-    int hs = p * g.sh - g.ph, ws = q * g.sw - g.pw;
-    const int he = min(hs + g.kh, g.H), we = min(ws + g.kw, g.W);
-    hs = max(hs, 0);
-    ws = max(ws, 0);
-    float best = -3.402823466e38f;
-    int bi = -1;
-    for (int h = hs; h < he; ++h)
-      for (int w = ws; w < we; ++w) {
-        const float v = xs[(h - xr0) * g.W + w];
-        if (v > best) {
-          best = v;
-          bi = h * g.W + w;
-        }
-      }
-    widx[i] = bi;
+  const int xr0 = max(p_lo * g.sh - g.ph, 0), xr1 = min(p_hi * g.sh - g.ph + g.kh, g.H);  // x rows [xr0, xr1)
+  const float *xb = x + size_t(plane) * g.H * g.W + xr0 * g.W;
+  const float *db = dy + size_t(plane) * g.P * g.Q + p_lo * g.Q;
+  float *ob = dx + size_t(plane) * g.H * g.W;
+  const int nx = (xr1 - xr0) * g.W, nd = np > 0 ? np * g.Q : 0;
+  if (((reinterpret_cast<uintptr_t>(xb) | reinterpret_cast<uintptr_t>(xs)) & 15u) == 0 && (nx & 3) == 0) {
+    const float4 *s4 = reinterpret_cast<const float4 *>(xb);
+    float4 *d4 = reinterpret_cast<float4 *>(xs);
+    for (int i = threadIdx.x; i < (nx >> 2); i += kBlock) d4[i] = s4[i];
+  } else {
+    for (int i = threadIdx.x; i < nx; i += kBlock) xs[i] = xb[i];
+  }
+  for (int i = threadIdx.x; i < nd; i += kBlock) ds[i] = db[i];
+  for (int i = threadIdx.x; i < h1 - h0; i += kBlock) {
+    const int hp = h0 + i + g.ph;
+    prange[2 * i] = (hp < g.kh ? 0 : (hp - g.kh) / g.sh + 1) - p_lo;
+    prange[2 * i + 1] = min(hp / g.sh, g.P - 1) - p_lo;
   }
   __syncthreads();
-  const int nd = (h1 - h0) * g.W;
-  for (int i = threadIdx.x; i < nd; i += kBlock) {
-    const int h = h0 + i / g.W, w = i % g.W, r = h * g.W + w;
-    const int hp = h + g.ph, wp = w + g.pw;
-    const int pl = hp < g.kh ? 0 : (hp - g.kh) / g.sh + 1;
-    const int ph_ = min(hp / g.sh, g.P - 1);
+  for (int pp = ty; pp < np; pp += 4) {
+    int hs = (p_lo + pp) * g.sh - g.ph;
+    const int he = min(hs + g.kh, g.H);
+    hs = max(hs, 0);
+    for (int q = tx; q < g.Q; q += 64) {
+      int ws = q * g.sw - g.pw;
+      const int we = min(ws + g.kw, g.W);
+      ws = max(ws, 0);
+      float best = -3.402823466e38f;
+      int bi = -1;
+      for (int h = hs; h < he; ++h)
+        for (int w = ws; w < we; ++w) {
+          const float v = xs[(h - xr0) * g.W + w];
+          if (v > best) {
+            best = v;
+            bi = h * g.W + w;
+          }
+        }
+      widx[pp * g.Q + q] = bi;
+    }
+  }
+  __syncthreads();
+  for (int w = tx; w < g.W; w += 64) {
+    const int wp = w + g.pw;
     const int ql = wp < g.kw ? 0 : (wp - g.kw) / g.sw + 1;
     const int qh = min(wp / g.sw, g.Q - 1);
-    float s = 0.f;
-    for (int p = pl; p <= ph_; ++p)
-      for (int q = ql; q <= qh; ++q)
-        if (widx[(p - p_lo) * g.Q + q] == r) s += db[p * g.Q + q];
-    ob[r] = s;
+    for (int hh = ty; hh < h1 - h0; hh += 4) {
+      const int r = (h0 + hh) * g.W + w;
+      const int pl = prange[2 * hh], ph_ = prange[2 * hh + 1];
+      float s = 0.f;
+      for (int p = pl; p <= ph_; ++p)
+        for (int q = ql; q <= qh; ++q)
+          if (widx[p * g.Q + q] == r) s += ds[p * g.Q + q];
+      ob[r] = s;
+    }
   }
 }
 
@@ -256,18 +277,20 @@ int sgh_pool_bwd_f32(const sgh_pool_geom *g, const float *dy, const float *x, co
   if (g->is_max && !x) return SGH_EINVAL;
   const size_t total = size_t(g->N) * g->C * g->H * g->W;
   if (g->is_max) {
-    // band height: about 8 dx elements per thread
-    int TH = 2048 / g->W;
+    // band height: about 24 KB of x rows per workgroup, bands of equal height
+    int TH = 6144 / g->W - g->kernel_h;
     if (TH < 1) TH = 1;
     if (TH > g->H) TH = g->H;
-    const int bands = (g->H + TH - 1) / TH;
+    int bands = (g->H + TH - 1) / TH;
+    TH = (g->H + bands - 1) / bands;
+    bands = (g->H + TH - 1) / TH;
     const int max_np = (TH + g->kernel_h - 2) / g->stride_h + 2;
     const int max_xrows = (max_np - 1) * g->stride_h + g->kernel_h;
-    const size_t lds = (size_t(max_xrows) * g->W + size_t(max_np) * g->Q) * sizeof(float);
+    const size_t lds = (size_t(max_xrows) * g->W + size_t(2) * max_np * g->Q + size_t(2) * TH) * sizeof(float);
     const size_t blocks = size_t(g->N) * g->C * bands;
     if (lds <= 48 * 1024 && blocks < 0x7fffffffu && g->W <= 2048) {
       hipLaunchKernelGGL(k_pool_max_bwd_tiled, dim3((unsigned)blocks), dim3(kBlock), lds, sgh_stream_of(stream), dy, x,
-                         dx, to_g(g), TH, bands, max_xrows);
+                         dx, to_g(g), TH, bands, max_xrows, max_np);
     } else {
       hipLaunchKernelGGL(k_pool_max_bwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
                          to_g(g), total);
