@@ -81,9 +81,19 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd(const float *__restrict
 // The 256 threads form 64 columns x 4 rows, so no per-element division is needed: a thread's
 // column window range is fixed, and the per-row window range is computed once per band row.
 // x, dy and dx each cross HBM once (plus the band halo of x).
+// KH/KW/SH/SW > 0 fix the window at compile time: the scans are then fully unrolled, every LDS
+// read of a window or of a dx element is issued before the first compare, and out-of-range
+// positions are predicated instead of branched over.  0 = read the geometry at run time.
+template <int KH, int KW, int SH, int SW>
 __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__restrict__ dy, const float *__restrict__ x,
                                                               float *__restrict__ dx, PoolG g, int TH, int bands,
                                                               int max_xrows, int max_np) {
+  if (KH > 0) {
+    g.kh = KH;
+    g.kw = KW;
+    g.sh = SH;
+    g.sw = SW;
+  }
   extern __shared__ float smem[];
   float *xs = smem;                                               // [max_xrows][W]
   float *ds = xs + max_xrows * g.W;                               // [max_np][Q]
@@ -105,6 +115,7 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__re
   if (((reinterpret_cast<uintptr_t>(xb) | reinterpret_cast<uintptr_t>(xs)) & 15u) == 0 && (nx & 3) == 0) {
     const float4 *s4 = reinterpret_cast<const float4 *>(xb);
     float4 *d4 = reinterpret_cast<float4 *>(xs);
+#pragma unroll 4
     for (int i = threadIdx.x; i < (nx >> 2); i += kBlock) d4[i] = s4[i];
   } else {
     for (int i = threadIdx.x; i < nx; i += kBlock) xs[i] = xb[i];
@@ -117,27 +128,47 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__re
   }
   __syncthreads();
   for (int pp = ty; pp < np; pp += 4) {
-    int hs = (p_lo + pp) * g.sh - g.ph;
-    const int he = min(hs + g.kh, g.H);
-    hs = max(hs, 0);
+    const int hs0 = (p_lo + pp) * g.sh - g.ph;
     for (int q = tx; q < g.Q; q += 64) {
-      int ws = q * g.sw - g.pw;
-      const int we = min(ws + g.kw, g.W);
-      ws = max(ws, 0);
+      const int ws0 = q * g.sw - g.pw;
       float best = -3.402823466e38f;
       int bi = -1;
-      for (int h = hs; h < he; ++h)
-        for (int w = ws; w < we; ++w) {
-          const float v = xs[(h - xr0) * g.W + w];
-          if (v > best) {
-            best = v;
-            bi = h * g.W + w;
+      if (KH > 0) {
+        float v[KH > 0 ? KH * KW : 1];
+#pragma unroll
+        for (int dh = 0; dh < KH; ++dh)
+#pragma unroll
+          for (int dw = 0; dw < KW; ++dw) {
+            const int h = hs0 + dh, w = ws0 + dw;
+            const bool ok = unsigned(h) < unsigned(g.H) && unsigned(w) < unsigned(g.W);
+            const float xv = xs[ok ? (h - xr0) * g.W + w : 0];
+            v[dh * KW + dw] = ok ? xv : -3.402823466e38f;
           }
-        }
+#pragma unroll
+        for (int dh = 0; dh < KH; ++dh)
+#pragma unroll
+          for (int dw = 0; dw < KW; ++dw)
+            if (v[dh * KW + dw] > best) {
+              best = v[dh * KW + dw];
+              bi = (hs0 + dh) * g.W + ws0 + dw;
+            }
+      } else {
+        const int hs = max(hs0, 0), he = min(hs0 + g.kh, g.H);
+        const int ws = max(ws0, 0), we = min(ws0 + g.kw, g.W);
+        for (int h = hs; h < he; ++h)
+          for (int w = ws; w < we; ++w) {
+            const float v = xs[(h - xr0) * g.W + w];
+            if (v > best) {
+              best = v;
+              bi = h * g.W + w;
+            }
+          }
+      }
       widx[pp * g.Q + q] = bi;
     }
   }
   __syncthreads();
+  constexpr int NWH = KH > 0 ? (KH + SH - 1) / SH : 1, NWW = KW > 0 ? (KW + SW - 1) / SW : 1;  // windows over one element
   for (int w = tx; w < g.W; w += 64) {
     const int wp = w + g.pw;
     const int ql = wp < g.kw ? 0 : (wp - g.kw) / g.sw + 1;
@@ -146,9 +177,27 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__re
       const int r = (h0 + hh) * g.W + w;
       const int pl = prange[2 * hh], ph_ = prange[2 * hh + 1];
       float s = 0.f;
-      for (int p = pl; p <= ph_; ++p)
-        for (int q = ql; q <= qh; ++q)
-          if (widx[p * g.Q + q] == r) s += ds[p * g.Q + q];
+      if (KH > 0) {
+        int wi[NWH * NWW];
+        float dv[NWH * NWW];
+#pragma unroll
+        for (int dp = 0; dp < NWH; ++dp)
+#pragma unroll
+          for (int dq = 0; dq < NWW; ++dq) {
+            const bool ok = pl + dp <= ph_ && ql + dq <= qh;
+            const int o = ok ? (pl + dp) * g.Q + ql + dq : 0;
+            wi[dp * NWW + dq] = ok ? widx[o] : -2;
+            dv[dp * NWW + dq] = ds[o];
+          }
+        // s is never -0.0 (it starts at +0.0), so adding +0.0 for a window that does not match
+        // leaves it bit-identical to skipping the addition
+#pragma unroll
+        for (int i = 0; i < NWH * NWW; ++i) s += wi[i] == r ? dv[i] : 0.f;
+      } else {
+        for (int p = pl; p <= ph_; ++p)
+          for (int q = ql; q <= qh; ++q)
+            if (widx[p * g.Q + q] == r) s += ds[p * g.Q + q];
+      }
       ob[r] = s;
     }
   }
@@ -277,8 +326,9 @@ int sgh_pool_bwd_f32(const sgh_pool_geom *g, const float *dy, const float *x, co
   if (g->is_max && !x) return SGH_EINVAL;
   const size_t total = size_t(g->N) * g->C * g->H * g->W;
   if (g->is_max) {
-    // band height: about 24 KB of x rows per workgroup, bands of equal height
-    int TH = 6144 / g->W - g->kernel_h;
+    // band height: about 12 KB of x rows per workgroup (measured optimum: enough workgroups per CU to
+    // overlap one's staging with another's scans), bands of equal height
+    int TH = 3072 / g->W - g->kernel_h;
     if (TH < 1) TH = 1;
     if (TH > g->H) TH = g->H;
     int bands = (g->H + TH - 1) / TH;
@@ -289,8 +339,15 @@ int sgh_pool_bwd_f32(const sgh_pool_geom *g, const float *dy, const float *x, co
     const size_t lds = (size_t(max_xrows) * g->W + size_t(2) * max_np * g->Q + size_t(2) * TH) * sizeof(float);
     const size_t blocks = size_t(g->N) * g->C * bands;
     if (lds <= 48 * 1024 && blocks < 0x7fffffffu && g->W <= 2048) {
-      hipLaunchKernelGGL(k_pool_max_bwd_tiled, dim3((unsigned)blocks), dim3(kBlock), lds, sgh_stream_of(stream), dy, x,
-                         dx, to_g(g), TH, bands, max_xrows, max_np);
+      auto kern = k_pool_max_bwd_tiled<0, 0, 0, 0>;
+      if (g->kernel_h == 3 && g->kernel_w == 3 && g->stride_h == 2 && g->stride_w == 2)
+        kern = k_pool_max_bwd_tiled<3, 3, 2, 2>;
+      else if (g->kernel_h == 2 && g->kernel_w == 2 && g->stride_h == 2 && g->stride_w == 2)
+        kern = k_pool_max_bwd_tiled<2, 2, 2, 2>;
+      else if (g->kernel_h == 3 && g->kernel_w == 3 && g->stride_h == 1 && g->stride_w == 1)
+        kern = k_pool_max_bwd_tiled<3, 3, 1, 1>;
+      hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBlock), lds, sgh_stream_of(stream), dy, x, dx, to_g(g), TH,
+                         bands, max_xrows, max_np);
     } else {
       hipLaunchKernelGGL(k_pool_max_bwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
                          to_g(g), total);
