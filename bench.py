@@ -8,7 +8,7 @@ updated (every backward kernel in tape order plus the update of all 62 parameter
 synthetic seeded inputs whose forward activations are already resident in HBM.
 
 Prints ONE JSON line: the whole-job images/s plus
-  roofline     -- the dominant kernel family (fp32 MFMA implicit-GEMM conv dgrad + wgrad):
+  roofline     -- the dominant kernel family (fp32 MFMA conv dgrad + wgrad kernels):
                   algorithmic FLOPs / measured kernel time (HIP events on the kernels' stream),
                   against the MI355X fp32 matrix peak;
   cpu_baseline -- the CPU oracle replaying the same tape on the host cores, on a bounded sample.
@@ -130,7 +130,8 @@ def main():
     roofline = {
         "bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
-        "kernel": "k_igemm (fp32 MFMA implicit-GEMM conv dgrad + wgrad, %d launches/step)" % (launches // prof_steps),
+        "kernel": "fp32 MFMA conv dgrad + wgrad kernels (k_dgrad3x3, k_wgrad3x3, k_igemm; %d launches/step)"
+                  % (launches // prof_steps),
         "flop_per_step": flop / prof_steps, "kernel_ms_per_step": round(ms / prof_steps, 4),
     }
     for k, v in conv.items():
