@@ -36,11 +36,17 @@ bool sgh_prof_on();
 void sgh_prof_start(const char *tag, double work, hipStream_t s);
 void sgh_prof_stop(hipStream_t s);
 
-// 3x3 stride-1 weight gradient with a shared LDS input tile (wgrad3x3.hip).  *_run returns
+// 3x3 (stride 1 or 2) weight gradient with a shared LDS input tile (wgrad3x3.hip).  *_run returns
 // SGH_EUNSUPPORTED for geometries it does not cover; *_workspace_bytes is 0 for those.
 size_t sgh_wgrad3x3_workspace_bytes(const sgh_conv_geom *g);
 int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
                      size_t ws_bytes, hipStream_t s);
+
+// Weight gradient for few input channels and a large filter (C*R*S in 65..160: the 7x7 stem),
+// wgrad_fewc.hip.  Same conventions as the 3x3 kernel above.
+size_t sgh_wgrad_fewc_workspace_bytes(const sgh_conv_geom *g);
+int sgh_wgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
+                       size_t ws_bytes, hipStream_t s);
 
 // 3x3 stride-1 pad-1 data gradient with a shared LDS gradient tile (dgrad3x3.hip).
 // `wt` = weights re-laid as [tap][KP][C], KP = K rounded up to 16.

@@ -818,6 +818,8 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
     case SGH_CONV_WGRAD: {
       const size_t tiled = sgh_wgrad3x3_workspace_bytes(g);
       if (tiled) return tiled;
+      const size_t fewc = sgh_wgrad_fewc_workspace_bytes(g);
+      if (fewc) return fewc;
       const WgradPlan p = plan_wgrad(g);
       return p.splits > 1 ? size_t(p.splits) * g->K * g->C * RS * sizeof(float) : 0;
     }
@@ -979,11 +981,17 @@ int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, con
 int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
                        size_t ws_bytes, void *stream) {
   if (!conv_ok(g) || !dy || !x || !dW) return SGH_EINVAL;
-  if (sgh_wgrad3x3_workspace_bytes(g)) {  // 3x3 stride 1: shared-input-tile kernel
+  if (sgh_wgrad3x3_workspace_bytes(g)) {  // 3x3, stride 1 or 2: shared-input-tile kernel
     sgh_prof_start("conv_wgrad_op", conv_flops(g), sgh_stream_of(stream));
     const int rc3 = sgh_wgrad3x3_run(g, dy, x, dW, workspace, ws_bytes, sgh_stream_of(stream));
     sgh_prof_stop(sgh_stream_of(stream));
     return rc3;
+  }
+  if (sgh_wgrad_fewc_workspace_bytes(g)) {  // few input channels, large filter (the stem)
+    sgh_prof_start("conv_wgrad_op", conv_flops(g), sgh_stream_of(stream));
+    const int rcf = sgh_wgrad_fewc_run(g, dy, x, dW, workspace, ws_bytes, sgh_stream_of(stream));
+    sgh_prof_stop(sgh_stream_of(stream));
+    return rcf;
   }
   const WgradPlan p = plan_wgrad(g);
   const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_WGRAD);

@@ -75,6 +75,9 @@ CONV_CASES = [
     (1, 32, 7, 7, 16, 1, 1, (3, 3), (0, 0), False),       # kernel smaller than stride
     (2, 36, 9, 7, 33, 3, 2, (2, 1), (1, 0), True),        # mixed strides, non-square kernel
     (2, 4, 12, 12, 8, 3, 3, (2, 2), (1, 1), False),       # few input channels: column-GEMM + gather path, strided
+    (1, 3, 224, 224, 64, 7, 7, (2, 2), (3, 3), False),    # ResNet stem at full image size
+    (3, 3, 40, 40, 96, 7, 7, (2, 2), (3, 3), True),       # stem-like, output channels over two 64-row tiles (second partial)
+    (2, 2, 24, 24, 40, 7, 7, (1, 1), (3, 3), False),      # few-channel large-filter path at stride 1
 ]
 
 
