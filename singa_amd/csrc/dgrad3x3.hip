@@ -1,5 +1,5 @@
-// Data gradient of 3x3, stride-1, pad-1 convolutions with an LDS gradient tile shared by all
-// nine taps.
+// Data gradient of 3x3, pad-1 convolutions (stride 1; stride 2 on even images) with an LDS gradient
+// tile shared by all nine taps.
 //
 //   dx[n][c][h][w] = sum_{k,r,s} dy[n][k][h + 1 - r][w + 1 - s] * W[k][c][r][s]
 //
@@ -42,8 +42,9 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
 struct D3Args {
   const float *dy, *wt;   // wt: re-laid weights [tap][KP][C]
   float *dx;
-  int N, C, H, W, K, KP;  // P == H, Q == W (3x3, stride 1, pad 1)
-  int total_pix;          // N * H * W
+  int N, C, H, W, K, KP;  // dx is N x C x H x W
+  int P, Q;               // dy is N x K x P x Q (stride 1: P == H, Q == W; stride 2: H == 2P, W == 2Q)
+  int total_pix;          // N * P * Q: pixels of the tile index space
   int chunks_per_split;   // reduction chunks (16 channels of k each) per grid.z slice
   long split_stride;      // elements between the partial outputs of consecutive slices
   unsigned dy_bytes, wt_bytes;
@@ -58,8 +59,15 @@ struct D3Args {
 // request has LAT + 1 steps of MFMA time to return.  Every load address is "thread constant +
 // scalar term" (one vector add); the thread constant is out of range for elements that must read
 // as zero, and K is a multiple of 16, so no per-load predicate is left.
-template <int BM, int LOGP, int VR>
+//
+// S2 (stride 2, pad 1, even H and W): the tile index space is the P x Q grid of one residue class
+// (h, w) = (2i + a, 2j + b); all four classes of a pixel block are accumulated by the same
+// workgroup (tap (r, s) belongs to class a = (r != 1), b = (s != 1) and reads dy[i + (r == 0)]
+// [j + (s == 0)]), so no MFMA is spent on the zeros of a dilated gradient, every tap is still a
+// compile-time LDS offset, and a lane stores its 2 x 2 output block as two 8-byte writes.
+template <int BM, int LOGP, int VR, bool S2>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void k_dgrad3x3(D3Args a) {
+  constexpr int NCLS = S2 ? 4 : 1;          // residue classes accumulated side by side
   constexpr int PA = BM;                    // weight tile pitch
   constexpr int TM = BM / 64;               // 32-row MFMA tiles per wavefront
   constexpr int PITCHP = 1 << LOGP;
@@ -82,31 +90,33 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
   const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 wavefronts, 64 x 32 each
   const int c0 = blockIdx.x * BM;
   const int pix0 = blockIdx.y * BN;
-  const int HW = a.H * a.W, VH = a.H + 2;
+  const int HW = a.H * a.W, PQ = a.P * a.Q;
+  const int VH = S2 ? a.P + 1 : a.P + 2;    // virtual rows per image: its dy rows plus the zero rows a tap can reach
   const rsrc_t rdy = make_rsrc(a.dy, a.dy_bytes), rw = make_rsrc(a.wt, a.wt_bytes);
 
   // first virtual row of the slab: the row above the tile's first pixel row
-  const int n_first = pix0 / HW, h_first = (pix0 - n_first * HW) / a.W;
-  const int vbase = n_first * VH + h_first;  // virtual row of dy row (h_first - 1)
+  const int n_first = pix0 / PQ, h_first = (pix0 - n_first * PQ) / a.Q;
+  const int vbase = n_first * VH + h_first;  // stride 1: virtual row of dy row (h_first - 1); stride 2: of row h_first
 
   // ---- dy slab loader ------------------------------------------------------------------------
   // slot e covers channel kc = (e / SUB) * KPP + tkc and slab element within = (e % SUB) * NT + tw:
   // virtual row vr = within >> LOGP, column col = within % PITCHP; dy row p = (vbase + vr) % VH - 1
   // of image (vbase + vr) / VH, dy column q = col - 1.  The byte offset splits into a thread part
-  // g0 (kOOB for halo / padding elements) and the scalar (k0 + (e / SUB) * KPP) * HW * 4.
+  // g0 (kOOB for halo / padding elements) and the scalar (k0 + (e / SUB) * KPP) * P * Q * 4.
+  // (Stride 2: no halo row above or column to the left, p = (vbase + vr) % VH, q = col.)
   const int tkc = VRP > NT ? 0 : t / VRP, tw = VRP > NT ? t : t % VRP;
   int g0[SUB];
 #pragma unroll
   for (int sub = 0; sub < SUB; ++sub) {
     const int within = sub * NT + tw, vr = within >> LOGP, col = within & (PITCHP - 1);
-    const int v = vbase + vr, n = v / VH, p = v - n * VH - 1, q = col - 1;
-    const bool ok = n < a.N && unsigned(p) < unsigned(a.H) && unsigned(q) < unsigned(a.W);
-    g0[sub] = ok ? (((n * a.K + tkc) * a.H + p) * a.W + q) * 4 : kOOB;
+    const int v = vbase + vr, n = v / VH, p = v - n * VH - (S2 ? 0 : 1), q = col - (S2 ? 0 : 1);
+    const bool ok = n < a.N && unsigned(p) < unsigned(a.P) && unsigned(q) < unsigned(a.Q);
+    g0[sub] = ok ? (((n * a.K + tkc) * a.P + p) * a.Q + q) * 4 : kOOB;
   }
   const int l0 = tkc * CHS + tw;
   auto dy_get = [&](int e, int k0) -> float {
     return __builtin_bit_cast(
-        float, __builtin_amdgcn_raw_buffer_load_b32(rdy, g0[e % SUB] + (k0 + (e / SUB) * KPP) * HW * 4, 0, 0));
+        float, __builtin_amdgcn_raw_buffer_load_b32(rdy, g0[e % SUB] + (k0 + (e / SUB) * KPP) * PQ * 4, 0, 0));
   };
   auto dy_loff = [&](int e) -> int { return l0 + (e / SUB) * KPP * CHS + (e % SUB) * NT; };
 
@@ -125,15 +135,15 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
   // ---- this lane's pixel (B operand column) ------------------------------------------------
   const int pix = pix0 + wn * 32 + (lane & 31);
   const int pixc = pix < a.total_pix ? pix : a.total_pix - 1;  // a tail lane computes a valid pixel, stores nothing
-  const int pn = pixc / HW, prem = pixc - pn * HW, ph_ = prem / a.W, pw_ = prem - ph_ * a.W;
+  const int pn = pixc / PQ, prem = pixc - pn * PQ, ph_ = prem / a.Q, pw_ = prem - ph_ * a.Q;
   // LDS offset of tap (r = 2, s = 2); tap (r, s) adds (2 - r) * PITCHP + (2 - s):
   //   dy row h + 1 - r  ->  virtual row pn*VH + h + 2 - r ; slab column of q = w + 1 - s is w + 2 - s
   const int boff = (pn * VH + ph_ - vbase) * PITCHP + pw_ + (lane >> 5) * CHS;
   const int aoff = (lane >> 5) * PA + wm * (BM / 2) + (lane & 31);
 
-  v16f acc[TM];
+  v16f acc[NCLS * TM];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < NCLS * TM; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
 
@@ -173,7 +183,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap) {
       const int r = tap / 3, s = tap - r * 3;
-      const int toff = (2 - r) * PITCHP + (2 - s);
+      const int toff = S2 ? (r == 0) * PITCHP + (s == 0) : (2 - r) * PITCHP + (2 - s);
+      const int cls = S2 ? 2 * (r != 1) + (s != 1) : 0;
       const float *ws = Ws + wcur * (KC * PA) + aoff;
       request(tap, ch);
 #pragma unroll
@@ -181,7 +192,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
         const float b = dys[kk * CHS + toff];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-          acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(ws[kk * PA + i * 32], b, acc[i], 0, 0, 0);
+          acc[cls * TM + i] =
+              __builtin_amdgcn_mfma_f32_32x32x2f32(ws[kk * PA + i * 32], b, acc[cls * TM + i], 0, 0, 0);
       }
       // what step (tap - LAT) requested: tap + 1's weights and this tap's share of the next slab
       const int slot = ((tap - LAT) % (LAT + 1) + LAT + 1) % (LAT + 1);
@@ -197,16 +209,32 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
     dcur ^= 1;
   }
 
-  // epilogue: dx[n][c][h][w], this lane's pixel, rows c0 + wm*64 + i*32 + 8*(v/4) + 4*(lane/32) + v%4
+  // epilogue: dx[n][c][h][w], this lane's pixel, rows c0 + wm*(BM/2) + i*32 + 8*(v/4) + 4*(lane/32) + v%4
   if (pix < a.total_pix) {
-    float *o = a.dx + size_t(blockIdx.z) * a.split_stride + size_t(pn) * a.C * HW + prem;
+    if (S2) {
+      typedef float v2f __attribute__((ext_vector_type(2)));
+      float *o = a.dx + size_t(blockIdx.z) * a.split_stride + size_t(pn) * a.C * HW + (2 * ph_) * a.W + 2 * pw_;
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (c < a.C) o[size_t(c) * HW] = acc[i][v];
-      }
+        for (int v = 0; v < 16; ++v) {
+          const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+          if (c < a.C) {
+            float *oc = o + size_t(c) * HW;
+            *reinterpret_cast<v2f *>(oc) = v2f{acc[0 * TM + i][v], acc[1 * TM + i][v]};
+            *reinterpret_cast<v2f *>(oc + a.W) = v2f{acc[2 * TM + i][v], acc[3 * TM + i][v]};
+          }
+        }
+    } else {
+      float *o = a.dx + size_t(blockIdx.z) * a.split_stride + size_t(pn) * a.C * HW + prem;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+          if (c < a.C) o[size_t(c) * HW] = acc[i][v];
+        }
+    }
   }
 }
 
@@ -224,7 +252,7 @@ __global__ __launch_bounds__(256) void k_dgrad3x3_reduce(const float *__restrict
 }
 
 struct D3Plan {
-  bool ok;
+  bool ok, s2;
   int bm, logp, vr, splits, chunks_per_split;
   size_t lds;
 };
@@ -232,31 +260,45 @@ struct D3Plan {
 inline D3Plan plan(const sgh_conv_geom *g) {
   D3Plan p{};
   p.ok = false;
-  if (g->R != 3 || g->S != 3 || g->stride_h != 1 || g->stride_w != 1 || g->pad_h != 1 || g->pad_w != 1) return p;
-  if (g->C < 64 || g->C % 4 != 0 || g->K % KC != 0 || g->W + 2 > 64 || g->W < 2) return p;
+  if (g->R != 3 || g->S != 3 || g->pad_h != 1 || g->pad_w != 1 || g->stride_h != g->stride_w) return p;
+  p.s2 = g->stride_h == 2;
+  if (g->stride_h != 1 && !p.s2) return p;
+  if (p.s2 && (g->H != 2 * g->P || g->W != 2 * g->Q)) return p;  // even image: four residue classes of equal size
+  if (g->C < 64 || g->C % 4 != 0 || g->K % KC != 0 || g->Q < 2) return p;
   if (getenv("SGH_DGRAD3X3_OFF")) return p;
-  p.logp = g->W + 2 <= 16 ? 4 : (g->W + 2 <= 32 ? 5 : 6);
-  // virtual rows a 128-pixel tile can touch: its pixel rows, one halo row each side, and two
-  // zero rows per image boundary it crosses
-  const int rows = (BN + g->W - 2) / g->W + 1;
-  const int crossings = (BN - 1) / (g->H * g->W) + 1;
-  const int need = rows + 2 + 2 * crossings;
-  if (p.logp == 6) p.vr = 8;
-  else if (p.logp == 5) p.vr = 16;
-  else p.vr = need <= 16 ? 16 : 32;
+  // slab columns: stride 1 has a halo column on both sides, stride 2 one zero column on the right
+  const int cols = p.s2 ? g->Q + 1 : g->Q + 2;
+  if (cols > 64) return p;
+  p.logp = cols <= 8 ? 3 : (cols <= 16 ? 4 : (cols <= 32 ? 5 : 6));
+  if (!p.s2 && p.logp < 4) p.logp = 4;
+  // virtual rows a 128-pixel tile can touch: its pixel rows, the halo rows (stride 1: one each
+  // side; stride 2: one below), and the zero rows of every image boundary it crosses
+  const int rows = (BN + g->Q - 2) / g->Q + 1;
+  const int crossings = (BN - 1) / (g->P * g->Q) + 1;
+  const int need = p.s2 ? rows + 1 + crossings : rows + 2 + 2 * crossings;
+  if (p.s2) {
+    // instantiated: pitch 32 x 8 rows, pitch 16 x 16 rows, pitch 8 x 32 rows (256 floats per channel)
+    if (p.logp == 6) return p;
+    p.vr = 256 >> p.logp;
+    p.bm = 64;  // four classes x 16 accumulators per 32-row tile: the 64-row tile keeps two workgroups per CU
+  } else {
+    if (p.logp == 6) p.vr = 8;
+    else if (p.logp == 5) p.vr = 16;
+    else p.vr = need <= 16 ? 16 : 32;
+    p.bm = (g->C % 128 == 0 || g->C > 192) ? 128 : 64;
+    if (const char *e = getenv("SGH_DGRAD3X3_BM")) p.bm = atoi(e) == 64 ? 64 : 128;
+  }
   if (need > p.vr) return p;
-  p.bm = (g->C % 128 == 0 || g->C > 192) ? 128 : 64;
-  if (const char *e = getenv("SGH_DGRAD3X3_BM")) p.bm = atoi(e) == 64 ? 64 : 128;
   const size_t chs = size_t(p.vr) * (1u << p.logp);
   p.lds = (size_t(2) * KC * (p.bm) + size_t(2) * KC * chs) * sizeof(float);
   if (p.lds > 160 * 1024) return p;
   const size_t lim = size_t(1) << 31;
   const size_t dx_elems = size_t(g->N) * g->C * g->H * g->W;
   if (size_t(g->N) * g->K * g->P * g->Q * 4 >= lim || dx_elems * 4 >= lim) return p;
-  if (size_t(g->N) * (g->H + 2) + p.vr >= lim / 64) return p;
+  if (size_t(g->N) * (g->P + 2) + p.vr >= lim / 64) return p;
   // split the reduction when the tile grid cannot fill the chip (one workgroup per CU fits);
   // the partial images are summed in slice order, so results stay run-to-run identical
-  const long tiles = long((g->C + p.bm - 1) / p.bm) * ((long(g->N) * g->H * g->W + BN - 1) / BN);
+  const long tiles = long((g->C + p.bm - 1) / p.bm) * ((long(g->N) * g->P * g->Q + BN - 1) / BN);
   const int nchunks = (g->K + KC - 1) / KC;
   // (three quarters of the CUs busy with unsplit work beats a full chip that also has to write,
   // re-read and sum partial images)
@@ -272,9 +314,9 @@ inline D3Plan plan(const sgh_conv_geom *g) {
   return p;
 }
 
-template <int BM, int LOGP, int VR>
+template <int BM, int LOGP, int VR, bool S2>
 int launch(const D3Args &a, const D3Plan &p, dim3 grid, hipStream_t s) {
-  auto kern = k_dgrad3x3<BM, LOGP, VR>;
+  auto kern = k_dgrad3x3<BM, LOGP, VR, S2>;
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -314,7 +356,9 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   a.W = g->W;
   a.K = g->K;
   a.KP = KP;
-  a.total_pix = g->N * g->H * g->W;
+  a.P = g->P;
+  a.Q = g->Q;
+  a.total_pix = g->N * g->P * g->Q;
   a.chunks_per_split = p.chunks_per_split;
   a.split_stride = long(g->N) * g->C * g->H * g->W;
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 4);
@@ -324,7 +368,9 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   int rc = SGH_EUNSUPPORTED;
   sgh_prof_start("conv_dgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
 #define D3_CASE(BM_, LOGP_, VR_) \
-  if (p.bm == BM_ && p.logp == LOGP_ && p.vr == VR_) rc = launch<BM_, LOGP_, VR_>(a, p, grid, s);
+  if (!p.s2 && p.bm == BM_ && p.logp == LOGP_ && p.vr == VR_) rc = launch<BM_, LOGP_, VR_, false>(a, p, grid, s);
+#define D3_CASE_S2(LOGP_, VR_) \
+  if (p.s2 && p.bm == 64 && p.logp == LOGP_ && p.vr == VR_) rc = launch<64, LOGP_, VR_, true>(a, p, grid, s);
   D3_CASE(128, 6, 8)
   D3_CASE(64, 6, 8)
   D3_CASE(128, 5, 16)
@@ -333,7 +379,11 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   D3_CASE(64, 4, 16)
   D3_CASE(128, 4, 32)
   D3_CASE(64, 4, 32)
+  D3_CASE_S2(5, 8)
+  D3_CASE_S2(4, 16)
+  D3_CASE_S2(3, 32)
 #undef D3_CASE
+#undef D3_CASE_S2
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
   if (p.splits > 1) {

@@ -75,6 +75,9 @@ CONV_CASES = [
     (1, 32, 7, 7, 16, 1, 1, (3, 3), (0, 0), False),       # kernel smaller than stride
     (2, 36, 9, 7, 33, 3, 2, (2, 1), (1, 0), True),        # mixed strides, non-square kernel
     (2, 4, 12, 12, 8, 3, 3, (2, 2), (1, 1), False),       # few input channels: column-GEMM + gather path, strided
+    (1, 64, 56, 56, 128, 3, 3, (2, 2), (1, 1), False),    # stage transitions at full spatial size: four residue
+    (2, 128, 28, 28, 64, 3, 3, (2, 2), (1, 1), False),    #   classes per workgroup, tiles crossing image boundaries
+    (5, 68, 14, 14, 48, 3, 3, (2, 2), (1, 1), True),      #   (7x7 class grid: up to 3 crossings), ragged channel counts
     (1, 3, 224, 224, 64, 7, 7, (2, 2), (3, 3), False),    # ResNet stem at full image size
     (3, 3, 40, 40, 96, 7, 7, (2, 2), (3, 3), True),       # stem-like, output channels over two 64-row tiles (second partial)
     (2, 2, 24, 24, 40, 7, 7, (1, 1), (3, 3), False),      # few-channel large-filter path at stride 1
