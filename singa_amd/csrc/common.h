@@ -55,6 +55,13 @@ size_t sgh_dgrad3x3_partial_bytes(const sgh_conv_geom *g);  // scratch for split
 int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, int KP, float *dx, float *partials,
                      hipStream_t s);
 
+// Stride-2 data gradient for at most four input channels and a large filter (the 7x7 stem),
+// dgrad_fewc.hip: direct 16-row MFMA kernel, W in its native [K][C][R][S] layout.
+bool sgh_dgrad_fewc_supported(const sgh_conv_geom *g);
+size_t sgh_dgrad_fewc_workspace_bytes(const sgh_conv_geom *g);
+int sgh_dgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
+                       size_t ws_bytes, hipStream_t s);
+
 // Sum across the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float sgh_wave_sum(float v) {
 #pragma unroll

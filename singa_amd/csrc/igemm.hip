@@ -764,10 +764,12 @@ inline int pick_tile(const char *env, int M, int N, int z) {
 }
 
 // Which algorithm a dgrad of this geometry uses.
-enum DgradPath { kDgradColumns, kDgradTile3x3, kDgradClasses, kDgradGather };
+enum DgradPath { kDgradFewC, kDgradColumns, kDgradTile3x3, kDgradClasses, kDgradGather };
 
 inline DgradPath dgrad_path(const sgh_conv_geom *g) {
   const size_t RS = size_t(g->R) * g->S;
+  // at most four input channels, stride 2, large filter (the stem): direct 16-row MFMA kernel
+  if (sgh_dgrad_fewc_supported(g)) return kDgradFewC;
   // few input channels: the C x pixels output tile would waste most of a 64-row MFMA tile, so run
   // the dense GEMM dcol = W^T * dy (CRS rows) and fold the columns back with a gather
   if (g->C < 32 && RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float) < kMaxOperandBytes) return kDgradColumns;
@@ -812,6 +814,7 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
   switch (which) {
     case SGH_CONV_FWD: return RS * round_up(g->C, BK) * g->K * sizeof(float);
     case SGH_CONV_DGRAD:
+      if (dgrad_path(g) == kDgradFewC) return sgh_dgrad_fewc_workspace_bytes(g);
       if (dgrad_path(g) == kDgradColumns) return RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float);
       return align256(RS * round_up(g->K, BK) * g->C * sizeof(float)) + align256(sizeof(DgClsTable)) +
              sgh_dgrad3x3_partial_bytes(g);
@@ -838,7 +841,9 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
   int rc = SGH_OK;
   sgh_prof_start("conv_dgrad_op", conv_flops(g), s);
 
-  if (path == kDgradColumns) {
+  if (path == kDgradFewC) {
+    rc = sgh_dgrad_fewc_run(g, dy, W, dx, workspace, ws_bytes, s);
+  } else if (path == kDgradColumns) {
     float *dcol = static_cast<float *>(workspace);
     const int CRS = g->C * RS, Ncols = g->N * g->P * g->Q;
     auto la = dense_loader<64, false>(W, 1, CRS, CRS, g->K);

@@ -81,6 +81,8 @@ CONV_CASES = [
     (1, 3, 224, 224, 64, 7, 7, (2, 2), (3, 3), False),    # ResNet stem at full image size
     (3, 3, 40, 40, 96, 7, 7, (2, 2), (3, 3), True),       # stem-like, output channels over two 64-row tiles (second partial)
     (2, 2, 24, 24, 40, 7, 7, (1, 1), (3, 3), False),      # few-channel large-filter path at stride 1
+    (2, 4, 24, 24, 16, 5, 5, (2, 2), (2, 2), False),      # direct few-channel dgrad: 5x5 (three offsets per dimension), C = 4
+    (2, 1, 16, 16, 8, 7, 7, (2, 2), (3, 3), True),        # direct few-channel dgrad: one channel
 ]
 
 
