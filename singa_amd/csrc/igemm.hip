@@ -506,6 +506,27 @@ __global__ __launch_bounds__(NT) void k_split_reduce(const float *__restrict__ p
   }
 }
 
+// The same sum for small outputs with many splits: 16 z-lanes x 16 elements per workgroup, lane zl
+// sums z = zl, zl + 16, ... (ascending), the lane sums are added in lane order.  Which of the two
+// kernels runs depends on the shape only, so results stay run-to-run identical.
+__global__ __launch_bounds__(256) void k_split_reduce_lanes(const float *__restrict__ part, float *__restrict__ out,
+                                                           long n, int splits) {
+  __shared__ float lanes[16][16];
+  const int e = threadIdx.x & 15, zl = threadIdx.x >> 4;
+  const long i = long(blockIdx.x) * 16 + e;
+  float s = 0.f;
+  if (i < n)
+    for (int z = zl; z < splits; z += 16) s += part[long(z) * n + i];
+  lanes[zl][e] = s;
+  __syncthreads();
+  if (threadIdx.x < 16 && i < n) {
+    float r = lanes[0][e];
+#pragma unroll
+    for (int l = 1; l < 16; ++l) r += lanes[l][e];
+    out[i] = r;
+  }
+}
+
 // Weight re-layout for the pixel-gather passes:  W[K][C][R][S]  ->  Wt[tap][chp][m]
 //   forward: ch = c (padded to CP), m = k   -> Wt[(tap * CP + c) * K + k]
 //   dgrad:   ch = k (padded to KP), m = c   -> Wt[(tap * KP + k) * C + c]
@@ -1028,9 +1049,13 @@ int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, 
 #undef SGH_WGRAD_CASE
   if (rc == SGH_OK && p.splits > 1) {
     const long n = long(g->K) * CRS;
-    long blocks = (n + NT - 1) / NT;
-    if (blocks > 2048) blocks = 2048;
-    hipLaunchKernelGGL(k_split_reduce, dim3(int(blocks)), dim3(NT), 0, s, part, dW, n, p.splits);
+    if (p.splits >= 32 && n <= long(sgh_num_cus()) * 16 * 64) {
+      hipLaunchKernelGGL(k_split_reduce_lanes, dim3(int((n + 15) / 16)), dim3(256), 0, s, part, dW, n, p.splits);
+    } else {
+      long blocks = (n + NT - 1) / NT;
+      if (blocks > 2048) blocks = 2048;
+      hipLaunchKernelGGL(k_split_reduce, dim3(int(blocks)), dim3(NT), 0, s, part, dW, n, p.splits);
+    }
   }
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
