@@ -26,6 +26,10 @@ if ROOT not in sys.path:
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes the 40 conv dgrad/wgrad MFMA launches of one default step move (fetched + written), from the
+# rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, each scaled by what the same counter reads for
+# a streaming kernel of known size (ReLU forward: 1.998 and 1.000).  Valid for the default workload only.
+CONV_HBM_BYTES_PER_STEP = 5.56e9
 
 
 def collect_prof(lib):
@@ -129,7 +133,9 @@ def main():
     achieved = flop / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
     roofline = {
         "bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+        "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+        "traffic": CONV_HBM_BYTES_PER_STEP if (args.config == "resnet18" and args.batch == 64) else None,
+        "traffic_unit": "HBM bytes per step over the same launches (PMC, calibrated)",
         "kernel": "fp32 MFMA conv dgrad + wgrad kernels (k_dgrad3x3, k_wgrad3x3, k_igemm; %d launches/step)"
                   % (launches // prof_steps),
         "flop_per_step": flop / prof_steps, "kernel_ms_per_step": round(ms / prof_steps, 4),
