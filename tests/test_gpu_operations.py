@@ -75,6 +75,13 @@ CONV_CASES = [
     (1, 32, 7, 7, 16, 1, 1, (3, 3), (0, 0), False),       # kernel smaller than stride
     (2, 36, 9, 7, 33, 3, 2, (2, 1), (1, 0), True),        # mixed strides, non-square kernel
     (2, 4, 12, 12, 8, 3, 3, (2, 2), (1, 1), False),       # few input channels: column-GEMM + gather path, strided
+    (2, 32, 12, 12, 64, 3, 3, (1, 1), (0, 0), False),     # shared-slab wgrad without padding
+    (2, 64, 10, 10, 64, 3, 3, (1, 1), (2, 2), False),     # ... with padding 2 (output larger than input)
+    (2, 32, 13, 13, 128, 3, 3, (2, 2), (1, 1), False),    # ... stride 2 on an odd image (dgrad: residue-class GEMMs)
+    (2, 32, 16, 16, 128, 3, 3, (2, 2), (0, 0), True),     # ... stride 2 without padding
+    (1, 32, 62, 62, 64, 3, 3, (1, 1), (1, 1), False),     # widest rows the 64-column slab holds
+    (1, 64, 30, 30, 64, 3, 3, (1, 1), (1, 1), False),     # widest rows the 32-column slab holds
+    (3, 96, 9, 20, 160, 3, 3, (1, 1), (1, 1), False),     # non-square image, channel tails in both tile dimensions
     (1, 64, 56, 56, 128, 3, 3, (2, 2), (1, 1), False),    # stage transitions at full spatial size: four residue
     (2, 128, 28, 28, 64, 3, 3, (2, 2), (1, 1), False),    #   classes per workgroup, tiles crossing image boundaries
     (5, 68, 14, 14, 48, 3, 3, (2, 2), (1, 1), True),      #   (7x7 class grid: up to 3 crossings), ragged channel counts
