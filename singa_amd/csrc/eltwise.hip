@@ -12,6 +12,10 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kUnroll = 4;  // float4 vectors in flight per thread per operand
+// Streaming operands are read and written with non-temporal accesses: measured in the ResNet-18
+// backward step this is faster than default caching for the large early-layer tensors and neutral
+// for the small ones.
+constexpr bool kNonTemporal = true;
 
 inline int grid_for(size_t nvec) {
   size_t per_block = size_t(kBlock) * kUnroll;
@@ -31,35 +35,42 @@ inline int grid_for(size_t nvec) {
 template <class F>
 __global__ __launch_bounds__(kBlock) void k_map2_1(const float *a, const float *b, float *o, size_t n, F f) {
   // no __restrict__: the in-place forms (y += alpha*x, a += b) alias an input with the output
+  typedef float v4f_ __attribute__((ext_vector_type(4)));
   const size_t nvec = n >> 2;
-  const float4 *a4 = reinterpret_cast<const float4 *>(a);
-  const float4 *b4 = reinterpret_cast<const float4 *>(b);
-  float4 *o4 = reinterpret_cast<float4 *>(o);
-  const size_t stride = size_t(gridDim.x) * kBlock;
-  size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
-  for (; i + (kUnroll - 1) * stride < nvec; i += kUnroll * stride) {
-    float4 va[kUnroll], vb[kUnroll];
+  const v4f_ *a4 = reinterpret_cast<const v4f_ *>(a);
+  const v4f_ *b4 = reinterpret_cast<const v4f_ *>(b);
+  v4f_ *o4 = reinterpret_cast<v4f_ *>(o);
+  // a workgroup takes kUnroll * kBlock consecutive vectors per pass (16 KB per stream), so that
+  // neighbouring workgroups stream neighbouring DRAM pages
+  const size_t step = size_t(gridDim.x) * (kBlock * kUnroll);
+  size_t i = size_t(blockIdx.x) * (kBlock * kUnroll) + threadIdx.x;
+  for (; i + (kUnroll - 1) * kBlock < nvec; i += step) {
+    v4f_ va[kUnroll], vb[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      va[u] = a4[i + u * stride];
-      vb[u] = b4[i + u * stride];
+      va[u] = kNonTemporal ? __builtin_nontemporal_load(a4 + i + u * kBlock) : a4[i + u * kBlock];
+      vb[u] = kNonTemporal ? __builtin_nontemporal_load(b4 + i + u * kBlock) : b4[i + u * kBlock];
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      float4 r;
-      r.x = f(va[u].x, vb[u].x);
-      r.y = f(va[u].y, vb[u].y);
-      r.z = f(va[u].z, vb[u].z);
-      r.w = f(va[u].w, vb[u].w);
-      o4[i + u * stride] = r;
+      v4f_ r;
+      r[0] = f(va[u][0], vb[u][0]);
+      r[1] = f(va[u][1], vb[u][1]);
+      r[2] = f(va[u][2], vb[u][2]);
+      r[3] = f(va[u][3], vb[u][3]);
+      if (kNonTemporal) __builtin_nontemporal_store(r, o4 + i + u * kBlock);
+      else o4[i + u * kBlock] = r;
     }
   }
-  for (; i < nvec; i += stride) {
-    float4 va = a4[i], vb = b4[i], r;
-    r.x = f(va.x, vb.x);
-    r.y = f(va.y, vb.y);
-    r.z = f(va.z, vb.z);
-    r.w = f(va.w, vb.w);
+  // the last, partial pass of the workgroup that owns it
+  for (; i < nvec; i += kBlock) {
+    if (i / (kBlock * kUnroll) % gridDim.x != blockIdx.x) break;
+    const v4f_ va = a4[i], vb = b4[i];
+    v4f_ r;
+    r[0] = f(va[0], vb[0]);
+    r[1] = f(va[1], vb[1]);
+    r[2] = f(va[2], vb[2]);
+    r[3] = f(va[3], vb[3]);
     o4[i] = r;
   }
   if (blockIdx.x == 0) {

@@ -34,6 +34,7 @@ class SGD(object):
         self.step_counter = 0
         self._table = None
         self._table_key = None
+        self._tables = {}
 
     def _moment(self, name, p):
         if name not in self.moments:
@@ -55,12 +56,19 @@ class SGD(object):
 
     def apply_all(self, named_params_grads):
         """Update every (name, p, g) triple with ONE kernel launch.  The pointer table is built
-        once per distinct set of buffers and kept on the device."""
+        once per distinct set of buffers and kept on the device; the memory pool hands the
+        gradient buffers out in a short cycle of address sets, so a few tables are cached and a
+        steady-state step uploads nothing (an upload is a blocking copy that would drain the
+        stream at the end of every step)."""
         items = list(named_params_grads)
         if not items:
             return
         dev = items[0][1].device()
         key = tuple((n, p.ptr, g.ptr) for n, p, g in items)
+        cached = self._tables.get(key)
+        if cached is not None:
+            self._table, self._table_total = cached
+            self._table_key = key
         if key != self._table_key:
             arr = (_lib.SgdItem * len(items))()
             total = 0
@@ -73,6 +81,9 @@ class SGD(object):
             table = singa.Tensor(((nbytes + 3) // 4,), dev, singa.kInt)
             check(_lib.lib().sgh_memcpy(dev._h, table.ptr, C.addressof(arr), nbytes, 1), "sgh_memcpy H2D")
             self._table, self._table_key, self._table_total = table, key, total
+            if len(self._tables) >= 16:
+                self._tables.pop(next(iter(self._tables)))
+            self._tables[key] = (table, total)
         check(_lib.lib().sgh_sgd_momentum_multi_f32(self._table.ptr, len(items), self._table_total, self.lr,
                                                     self.momentum, self.dampening, self.weight_decay,
                                                     int(self.nesterov), dev.stream), "sgh_sgd_momentum_multi_f32")
