@@ -17,18 +17,61 @@ struct BnShape {
   int N, C, HW;
   int S;          // splits per channel
   int per_split;  // elements of the (n, hw) space per split (multiple of 4 when HW % 4 == 0)
+  int stream;     // tensor too large to stay cache resident between kernels: non-temporal loads
 };
 
-// Visit elements [lo, hi) of channel c's (n, hw) index space; F(x_value(s), index)
-template <int NT, class F4, class F1>
-__device__ __forceinline__ void channel_range(const BnShape s, int c, int lo, int hi, F4 f4, F1 f1) {
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// Visit elements [lo, hi) of channel c's (n, hw) index space.  The 16-byte path loads four
+// float4 of x (and of dy when `dy` is not null) per thread before the first use, so that eight
+// loads are in flight per thread, and tracks (image, offset) incrementally instead of dividing.
+// f4(offset, x4, dy4) / f1(offset) do the arithmetic and any store.
+template <int NT, bool STREAM, class F4, class F1>
+__device__ __forceinline__ void channel_range_impl(const BnShape s, int c, int lo, int hi, const float *__restrict__ x,
+                                                   const float *__restrict__ dy, F4 f4, F1 f1) {
   const int M = s.N * s.HW;
   if (hi > M) hi = M;
   if ((s.HW & 3) == 0) {
     // lo and per_split are multiples of 4 and a float4 never straddles an image boundary
-    for (int i = lo + threadIdx.x * 4; i < hi; i += NT * 4) {
-      const int n = i / s.HW, r = i - n * s.HW;
-      f4((size_t(n) * s.C + c) * s.HW + r);
+    constexpr int U = 4;
+    int i = lo + threadIdx.x * 4;
+    int n = i / s.HW, r = i - n * s.HW;
+    for (; i + (U - 1) * NT * 4 < hi; i += U * NT * 4) {
+      size_t off[U];
+      v4f xv[U], dv[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        off[u] = (size_t(n) * s.C + c) * s.HW + r;
+        r += NT * 4;
+        while (r >= s.HW) {
+          r -= s.HW;
+          ++n;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (STREAM) {
+          xv[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(x + off[u]));
+          if (dy) dv[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(dy + off[u]));
+        } else {
+          xv[u] = *reinterpret_cast<const v4f *>(x + off[u]);
+          if (dy) dv[u] = *reinterpret_cast<const v4f *>(dy + off[u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) f4(off[u], xv[u], dv[u]);
+    }
+    for (; i < hi; i += NT * 4) {
+      const size_t off = (size_t(n) * s.C + c) * s.HW + r;
+      v4f dv = {0.f, 0.f, 0.f, 0.f};
+      const v4f xv = *reinterpret_cast<const v4f *>(x + off);
+      if (dy) dv = *reinterpret_cast<const v4f *>(dy + off);
+      f4(off, xv, dv);
+      r += NT * 4;
+      while (r >= s.HW) {
+        r -= s.HW;
+        ++n;
+      }
     }
   } else {
     for (int i = lo + threadIdx.x; i < hi; i += NT) {
@@ -36,6 +79,13 @@ __device__ __forceinline__ void channel_range(const BnShape s, int c, int lo, in
       f1((size_t(n) * s.C + c) * s.HW + r);
     }
   }
+}
+
+template <int NT, class F4, class F1>
+__device__ __forceinline__ void channel_range(const BnShape s, int c, int lo, int hi, const float *__restrict__ x,
+                                              const float *__restrict__ dy, F4 f4, F1 f1) {
+  if (s.stream) channel_range_impl<NT, true>(s, c, lo, hi, x, dy, f4, f1);
+  else channel_range_impl<NT, false>(s, c, lo, hi, x, dy, f4, f1);
 }
 
 // ---- forward, pass 1: per (c, split) partial sum and sum of squares about a pivot ---------
@@ -47,10 +97,9 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_partial(const float *__restri
   const float pivot = x[size_t(c) * s.HW];
   float a = 0.f, b = 0.f;
   channel_range<kBlock>(
-      s, c, sp * s.per_split, (sp + 1) * s.per_split,
-      [&](size_t off) {
-        const float4 v = *reinterpret_cast<const float4 *>(x + off);
-        const float d0 = v.x - pivot, d1 = v.y - pivot, d2 = v.z - pivot, d3 = v.w - pivot;
+      s, c, sp * s.per_split, (sp + 1) * s.per_split, x, nullptr,
+      [&](size_t, v4f v, v4f) {
+        const float d0 = v[0] - pivot, d1 = v[1] - pivot, d2 = v[2] - pivot, d3 = v[3] - pivot;
         a += (d0 + d1) + (d2 + d3);
         b += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
       },
@@ -98,15 +147,14 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const float *__restrict
   }
   const float g = gamma[c], be = beta[c];
   channel_range<kBlock>(
-      s, c, sp * s.per_split, (sp + 1) * s.per_split,
-      [&](size_t off) {
-        const float4 v = *reinterpret_cast<const float4 *>(x + off);
-        float4 r;
-        r.x = g * ((v.x - mean) * invstd) + be;
-        r.y = g * ((v.y - mean) * invstd) + be;
-        r.z = g * ((v.z - mean) * invstd) + be;
-        r.w = g * ((v.w - mean) * invstd) + be;
-        *reinterpret_cast<float4 *>(y + off) = r;
+      s, c, sp * s.per_split, (sp + 1) * s.per_split, x, nullptr,
+      [&](size_t off, v4f v, v4f) {
+        v4f r;
+        r[0] = g * ((v[0] - mean) * invstd) + be;
+        r[1] = g * ((v[1] - mean) * invstd) + be;
+        r[2] = g * ((v[2] - mean) * invstd) + be;
+        r[3] = g * ((v[3] - mean) * invstd) + be;
+        *reinterpret_cast<v4f *>(y + off) = r;
       },
       [&](size_t off) { y[off] = g * ((x[off] - mean) * invstd) + be; });
 }
@@ -121,13 +169,11 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_partial(const float *__restri
   const float mean = save_mean[c], invstd = save_invstd[c];
   float a = 0.f, b = 0.f;
   channel_range<kBlock>(
-      s, c, sp * s.per_split, (sp + 1) * s.per_split,
-      [&](size_t off) {
-        const float4 d = *reinterpret_cast<const float4 *>(dy + off);
-        const float4 v = *reinterpret_cast<const float4 *>(x + off);
-        a += (d.x + d.y) + (d.z + d.w);
-        b += (d.x * ((v.x - mean) * invstd) + d.y * ((v.y - mean) * invstd)) +
-             (d.z * ((v.z - mean) * invstd) + d.w * ((v.w - mean) * invstd));
+      s, c, sp * s.per_split, (sp + 1) * s.per_split, x, dy,
+      [&](size_t, v4f v, v4f d) {
+        a += (d[0] + d[1]) + (d[2] + d[3]);
+        b += (d[0] * ((v[0] - mean) * invstd) + d[1] * ((v[1] - mean) * invstd)) +
+             (d[2] * ((v[2] - mean) * invstd) + d[3] * ((v[3] - mean) * invstd));
       },
       [&](size_t off) {
         const float d = dy[off];
@@ -166,16 +212,14 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const float *__restrict
   const float rM = float(1.0 / (double(s.N) * s.HW));
   const float c0 = db * rM, c1 = dg * rM;
   channel_range<kBlock>(
-      s, c, sp * s.per_split, (sp + 1) * s.per_split,
-      [&](size_t off) {
-        const float4 d = *reinterpret_cast<const float4 *>(dy + off);
-        const float4 v = *reinterpret_cast<const float4 *>(x + off);
-        float4 r;
-        r.x = k * (d.x - (c0 + ((v.x - mean) * invstd) * c1));
-        r.y = k * (d.y - (c0 + ((v.y - mean) * invstd) * c1));
-        r.z = k * (d.z - (c0 + ((v.z - mean) * invstd) * c1));
-        r.w = k * (d.w - (c0 + ((v.w - mean) * invstd) * c1));
-        *reinterpret_cast<float4 *>(dx + off) = r;
+      s, c, sp * s.per_split, (sp + 1) * s.per_split, x, dy,
+      [&](size_t off, v4f v, v4f d) {
+        v4f r;
+        r[0] = k * (d[0] - (c0 + ((v[0] - mean) * invstd) * c1));
+        r[1] = k * (d[1] - (c0 + ((v[1] - mean) * invstd) * c1));
+        r[2] = k * (d[2] - (c0 + ((v[2] - mean) * invstd) * c1));
+        r[3] = k * (d[3] - (c0 + ((v[3] - mean) * invstd) * c1));
+        *reinterpret_cast<v4f *>(dx + off) = r;
       },
       [&](size_t off) { dx[off] = k * (dy[off] - (c0 + ((x[off] - mean) * invstd) * c1)); });
 }
@@ -185,7 +229,9 @@ inline bool shape_ok(int N, int C, int HW) {
 }
 
 inline BnShape make_shape(int N, int C, int HW) {
-  BnShape s{N, C, HW, 1, 0};
+  // (measured: non-temporal loads gain 20 % on the 205 MB stem tensors and lose a few per cent on
+  // tensors the previous kernel left in the 256 MB Infinity Cache)
+  BnShape s{N, C, HW, 1, 0, size_t(N) * C * HW * sizeof(float) >= (size_t(96) << 20) ? 1 : 0};
   const long M = long(N) * HW;
   // aim at ~8 workgroups per CU in total, at least 2048 elements per workgroup
   long want = (long(sgh_num_cus()) * 8 + C - 1) / C;
