@@ -259,26 +259,62 @@ __global__ __launch_bounds__(kBlock) void k_sgd(float *__restrict__ p, const flo
   }
 }
 
-// Multi-tensor variant: block b walks the concatenation of all items in chunks of
-// kChunk elements; a chunk never crosses an item boundary (the table is scanned linearly,
-// 62 entries for ResNet-18).
-constexpr int kChunk = kBlock * 4 * 2;  // 2048 elements per block-iteration
+// Multi-tensor variant: block b walks the concatenation of all items in chunks of kChunk elements;
+// a chunk never crosses an item boundary.  Each workgroup first builds the prefix sums of the
+// items' chunk counts in LDS (one parallel pass over the table), then finds the owner of its
+// chunks by walking that array forward (its chunk indices only grow), so the table costs one
+// global read per item per workgroup instead of a dependent scan per chunk.  All of a thread's
+// 16-byte loads of a chunk are issued before the first store.
+constexpr int kSgdVec = 4;                        // float4 per thread per tensor per chunk
+constexpr int kChunk = kBlock * 4 * kSgdVec;      // 4096 elements per block-iteration
+constexpr int kSgdTab = 2048;                     // items whose prefix sums fit the LDS table
 
 __global__ __launch_bounds__(kBlock) void k_sgd_multi(const sgh_sgd_item *__restrict__ table, int count, SgdHyper h,
                                                      int nesterov) {
+  __shared__ unsigned pre[kSgdTab + 1];  // pre[i] = chunks of items 0 .. i-1
   const bool use_v = h.mu != 0.f;
+  const bool lds_tab = count <= kSgdTab;
+  if (lds_tab) {
+    for (int i = threadIdx.x; i < count; i += kBlock) pre[i + 1] = unsigned((table[i].n + kChunk - 1) / kChunk);
+    if (threadIdx.x == 0) pre[0] = 0;
+    __syncthreads();
+    if (threadIdx.x < 64) {  // wavefront 0: inclusive scan in tiles of 64 with a running carry
+      unsigned carry = 0;
+      for (int base = 0; base < count; base += 64) {
+        const int i = base + threadIdx.x;
+        unsigned v = i < count ? pre[i + 1] : 0u;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const unsigned u = __shfl_up(v, o, 64);
+          if (int(threadIdx.x) >= o) v += u;
+        }
+        v += carry;
+        if (i < count) pre[i + 1] = v;
+        carry = __shfl(v, 63, 64);
+      }
+    }
+    __syncthreads();
+  }
   // chunk index space: sum over items of ceil(n / kChunk)
   size_t chunk = blockIdx.x;
+  int it = 0;
+  size_t it_first = 0;  // first chunk of item `it` (linear-scan fallback only)
   for (;;) {
     // locate the item that owns this chunk
-    size_t c = chunk;
-    int it = 0;
-    for (; it < count; ++it) {
-      const size_t nc = (table[it].n + kChunk - 1) / kChunk;
-      if (c < nc) break;
-      c -= nc;
+    size_t c;
+    if (lds_tab) {
+      if (chunk >= pre[count]) return;
+      while (chunk >= pre[it + 1]) ++it;
+      c = chunk - pre[it];
+    } else {
+      for (; it < count; ++it) {
+        const size_t nc = (table[it].n + kChunk - 1) / kChunk;
+        if (chunk - it_first < nc) break;
+        it_first += nc;
+      }
+      if (it >= count) return;
+      c = chunk - it_first;
     }
-    if (it >= count) return;
     float *p = table[it].p;
     const float *g = table[it].g;
     float *v = table[it].v;
@@ -288,7 +324,27 @@ __global__ __launch_bounds__(kBlock) void k_sgd_multi(const sgh_sgd_item *__rest
     const size_t end = base + kChunk < n ? base + kChunk : n;
     const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) |
                        reinterpret_cast<uintptr_t>(has_v ? v : p)) & 15u) == 0;
-    if (vec) {
+    if (vec && base + kChunk <= n) {
+      // a full chunk: kSgdVec float4 per thread per tensor, all loaded before the first store
+      float4 pp[kSgdVec], gg[kSgdVec], vv[kSgdVec];
+#pragma unroll
+      for (int u = 0; u < kSgdVec; ++u) {
+        const size_t e = base + (size_t(u) * kBlock + threadIdx.x) * 4;
+        pp[u] = *reinterpret_cast<const float4 *>(p + e);
+        gg[u] = *reinterpret_cast<const float4 *>(g + e);
+        vv[u] = has_v ? *reinterpret_cast<const float4 *>(v + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < kSgdVec; ++u) {
+        const size_t e = base + (size_t(u) * kBlock + threadIdx.x) * 4;
+        sgd_one(pp[u].x, gg[u].x, vv[u].x, h, nesterov, has_v);
+        sgd_one(pp[u].y, gg[u].y, vv[u].y, h, nesterov, has_v);
+        sgd_one(pp[u].z, gg[u].z, vv[u].z, h, nesterov, has_v);
+        sgd_one(pp[u].w, gg[u].w, vv[u].w, h, nesterov, has_v);
+        *reinterpret_cast<float4 *>(p + e) = pp[u];
+        if (has_v) *reinterpret_cast<float4 *>(v + e) = vv[u];
+      }
+    } else if (vec) {
       for (size_t e = base + size_t(threadIdx.x) * 4; e < end; e += size_t(kBlock) * 4) {
         if (e + 4 <= end) {
           float4 pp = *reinterpret_cast<float4 *>(p + e), gg = *reinterpret_cast<const float4 *>(g + e);
