@@ -168,37 +168,72 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__re
     }
   }
   __syncthreads();
-  constexpr int NWH = KH > 0 ? (KH + SH - 1) / SH : 1, NWW = KW > 0 ? (KW + SW - 1) / SW : 1;  // windows over one element
-  for (int w = tx; w < g.W; w += 64) {
-    const int wp = w + g.pw;
-    const int ql = wp < g.kw ? 0 : (wp - g.kw) / g.sw + 1;
-    const int qh = min(wp / g.sw, g.Q - 1);
-    for (int hh = ty; hh < h1 - h0; hh += 4) {
-      const int r = (h0 + hh) * g.W + w;
-      const int pl = prange[2 * hh], ph_ = prange[2 * hh + 1];
-      float s = 0.f;
-      if (KH > 0) {
-        int wi[NWH * NWW];
-        float dv[NWH * NWW];
+  if (KH > 0) {
+    // A thread owns an SH x SW block of dx.  The windows that can contain any of its elements are
+    // NBH x NBW consecutive ones; their arg-max positions and dy values are read once and serve
+    // the whole block (a window whose maximum sits on element r necessarily contains r, so
+    // testing the position is enough).
+    constexpr int SHc = KH > 0 ? SH : 1, SWc = KW > 0 ? SW : 1;
+    constexpr int NBH = KH > 0 ? (KH + SH - 2) / SHc + 1 : 1, NBW = KW > 0 ? (KW + SW - 2) / SWc + 1 : 1;
+    const int nbh = (h1 - h0 + SHc - 1) / SHc, nbw = (g.W + SWc - 1) / SWc;
+    for (int bj = tx; bj < nbw; bj += 64) {
+      const int w0 = bj * SWc, wp0 = w0 + g.pw;
+      const int ql0 = wp0 < g.kw ? 0 : (wp0 - g.kw) / g.sw + 1;
+      for (int bi = ty; bi < nbh; bi += 4) {
+        const int hb = h0 + bi * SHc, hp0 = hb + g.ph;
+        const int pl0 = (hp0 < g.kh ? 0 : (hp0 - g.kh) / g.sh + 1) - p_lo;
+        int wi[NBH * NBW];
+        float dv[NBH * NBW];
 #pragma unroll
-        for (int dp = 0; dp < NWH; ++dp)
+        for (int dp = 0; dp < NBH; ++dp)
 #pragma unroll
-          for (int dq = 0; dq < NWW; ++dq) {
-            const bool ok = pl + dp <= ph_ && ql + dq <= qh;
-            const int o = ok ? (pl + dp) * g.Q + ql + dq : 0;
-            wi[dp * NWW + dq] = ok ? widx[o] : -2;
-            dv[dp * NWW + dq] = ds[o];
+          for (int dq = 0; dq < NBW; ++dq) {
+            const bool ok = pl0 + dp < np && ql0 + dq < g.Q;
+            const int o = ok ? (pl0 + dp) * g.Q + ql0 + dq : 0;
+            wi[dp * NBW + dq] = ok ? widx[o] : -2;
+            dv[dp * NBW + dq] = ds[o];
           }
-        // s is never -0.0 (it starts at +0.0), so adding +0.0 for a window that does not match
-        // leaves it bit-identical to skipping the addition
 #pragma unroll
-        for (int i = 0; i < NWH * NWW; ++i) s += wi[i] == r ? dv[i] : 0.f;
-      } else {
+        for (int a = 0; a < SHc; ++a) {
+          const int h = hb + a;
+          if (h >= h1) break;
+          float out[SWc];
+#pragma unroll
+          for (int b2 = 0; b2 < SWc; ++b2) {
+            const int r = h * g.W + w0 + b2;
+            // s is never -0.0 (it starts at +0.0), so adding +0.0 for a window that does not match
+            // leaves it bit-identical to skipping the addition; ascending (p, q) order as on the CPU
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < NBH * NBW; ++i) s += wi[i] == r ? dv[i] : 0.f;
+            out[b2] = s;
+          }
+          float *o = ob + h * g.W + w0;
+          if (SWc == 2 && w0 + 1 < g.W && (reinterpret_cast<uintptr_t>(o) & 7u) == 0) {
+            typedef float v2f __attribute__((ext_vector_type(2)));
+            *reinterpret_cast<v2f *>(o) = v2f{out[0], out[SWc - 1]};
+          } else {
+#pragma unroll
+            for (int b2 = 0; b2 < SWc; ++b2)
+              if (w0 + b2 < g.W) o[b2] = out[b2];
+          }
+        }
+      }
+    }
+  } else {
+    for (int w = tx; w < g.W; w += 64) {
+      const int wp = w + g.pw;
+      const int ql = wp < g.kw ? 0 : (wp - g.kw) / g.sw + 1;
+      const int qh = min(wp / g.sw, g.Q - 1);
+      for (int hh = ty; hh < h1 - h0; hh += 4) {
+        const int r = (h0 + hh) * g.W + w;
+        const int pl = prange[2 * hh], ph_ = prange[2 * hh + 1];
+        float s = 0.f;
         for (int p = pl; p <= ph_; ++p)
           for (int q = ql; q <= qh; ++q)
             if (widx[p * g.Q + q] == r) s += ds[p * g.Q + q];
+        ob[r] = s;
       }
-      ob[r] = s;
     }
   }
 }
