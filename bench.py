@@ -136,7 +136,7 @@ def main():
         "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
         "traffic": CONV_HBM_BYTES_PER_STEP if (args.config == "resnet18" and args.batch == 64) else None,
         "traffic_unit": "HBM bytes per step over the same launches (PMC, calibrated)",
-        "kernel": "fp32 MFMA conv dgrad + wgrad kernels (k_dgrad3x3, k_wgrad3x3, k_igemm; %d launches/step)"
+        "kernel": "fp32 MFMA conv dgrad + wgrad kernels (k_dgrad3x3, k_wgrad3x3, k_dgrad_fewc, k_wgrad_fewc, k_igemm; %d launches/step)"
                   % (launches // prof_steps),
         "flop_per_step": flop / prof_steps, "kernel_ms_per_step": round(ms / prof_steps, 4),
     }
