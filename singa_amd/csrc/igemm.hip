@@ -375,6 +375,33 @@ struct NchwStore {  // out[(img * CH + m) * plane + rem] (+ bias[m]), column = i
   }
 };
 
+// Data gradient of a 1x1, pad-0, stride-s convolution: GEMM column (img, p, q) lands on
+// dx[img][m][s*p][s*q] and the other positions of its s x s block are zero.  A lane writes the
+// whole block, so dx is produced in one pass without a separate zero fill.
+struct DilateStore {
+  float *dx;
+  int C, H, W, P, Q, sh, sw, cols;
+  __device__ __forceinline__ void operator()(int m, int col, float v) const {
+    if (m < C && col < cols) {
+      const int PQ = P * Q;
+      const int img = col / PQ, rem = col - img * PQ, p = rem / Q, q = rem - p * Q;
+      float *o = dx + ((long(img) * C + m) * H + p * sh) * W + q * sw;
+      if (sh == 2 && sw == 2 && p * 2 + 1 < H && q * 2 + 1 < W && (reinterpret_cast<uintptr_t>(o) & 7u) == 0 &&
+          (W & 1) == 0) {
+        typedef float v2f __attribute__((ext_vector_type(2)));
+        *reinterpret_cast<v2f *>(o) = v2f{v, 0.f};
+        *reinterpret_cast<v2f *>(o + W) = v2f{0.f, 0.f};
+      } else {
+        // rows / columns of the block that fall outside the image (odd sizes) are skipped; the
+        // last block of a row / column also covers the remainder beyond s * Q (s * P)
+        const int he = p == P - 1 ? H - p * sh : sh, we = q == Q - 1 ? W - q * sw : sw;
+        for (int a = 0; a < he; ++a)
+          for (int b = 0; b < we; ++b) o[a * W + b] = (a == 0 && b == 0) ? v : 0.f;
+      }
+    }
+  }
+};
+
 struct SplitStore {  // partial[split][m * N + n]
   float *part;
   int M, N;
@@ -785,12 +812,15 @@ inline int pick_tile(const char *env, int M, int N, int z) {
 }
 
 // Which algorithm a dgrad of this geometry uses.
-enum DgradPath { kDgradFewC, kDgradColumns, kDgradTile3x3, kDgradClasses, kDgradGather };
+enum DgradPath { kDgradFewC, kDgradPointwise, kDgradColumns, kDgradTile3x3, kDgradClasses, kDgradGather };
 
 inline DgradPath dgrad_path(const sgh_conv_geom *g) {
   const size_t RS = size_t(g->R) * g->S;
   // at most four input channels, stride 2, large filter (the stem): direct 16-row MFMA kernel
   if (sgh_dgrad_fewc_supported(g)) return kDgradFewC;
+  // 1x1 without padding: a plain GEMM over the output pixels whose store dilates by the stride
+  if (RS == 1 && g->pad_h == 0 && g->pad_w == 0 && g->C >= 32 && !getenv("SGH_DGRAD_POINTWISE_OFF"))
+    return kDgradPointwise;
   // few input channels: the C x pixels output tile would waste most of a 64-row MFMA tile, so run
   // the dense GEMM dcol = W^T * dy (CRS rows) and fold the columns back with a gather
   if (g->C < 32 && RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float) < kMaxOperandBytes) return kDgradColumns;
@@ -836,6 +866,7 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
     case SGH_CONV_FWD: return RS * round_up(g->C, BK) * g->K * sizeof(float);
     case SGH_CONV_DGRAD:
       if (dgrad_path(g) == kDgradFewC) return sgh_dgrad_fewc_workspace_bytes(g);
+      if (dgrad_path(g) == kDgradPointwise) return 0;
       if (dgrad_path(g) == kDgradColumns) return RS * g->C * size_t(g->N) * g->P * g->Q * sizeof(float);
       return align256(RS * round_up(g->K, BK) * g->C * sizeof(float)) + align256(sizeof(DgClsTable)) +
              sgh_dgrad3x3_partial_bytes(g);
@@ -855,7 +886,7 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
                        size_t ws_bytes, void *stream) {
   if (!conv_ok(g) || !dy || !W || !dx) return SGH_EINVAL;
   const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_DGRAD);
-  if (!workspace || ws_bytes < need) return SGH_EWORKSPACE;
+  if (need && (!workspace || ws_bytes < need)) return SGH_EWORKSPACE;
   hipStream_t s = sgh_stream_of(stream);
   const int RS = g->R * g->S, KP = round_up(g->K, BK);
   const DgradPath path = dgrad_path(g);
@@ -864,6 +895,29 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
 
   if (path == kDgradFewC) {
     rc = sgh_dgrad_fewc_run(g, dy, W, dx, workspace, ws_bytes, s);
+  } else if (path == kDgradPointwise) {
+    // dx block (img, m, p, q) = sum_k W[k][m] * dy[img][k][p][q]: A(m, k) = W[k * C + m] in its native layout
+    const int Ncols = g->N * g->P * g->Q;
+    ConvG fake{g->N, g->K, g->P, g->Q, g->K, 1, 1, 1, 1, 0, 0, g->P, g->Q};
+    DilateStore st{dx, g->C, g->H, g->W, g->P, g->Q, g->stride_h, g->stride_w, Ncols};
+    const int chunks = (g->K + BK - 1) / BK;
+    const long tiles128 = long((g->C + 127) / 128) * ((Ncols + 127) / 128);
+    if (g->C > 64 && tiles128 >= sgh_num_cus()) {
+      auto la = dense_loader<128, false>(W, 1, g->C, g->C, g->K);
+      auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
+      rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, DilateStore, false, false>(
+          la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad", conv_flops(g));
+    } else if (long((g->C + 63) / 64) * ((Ncols + 127) / 128) >= sgh_num_cus()) {
+      auto la = dense_loader<64, false>(W, 1, g->C, g->C, g->K);
+      auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
+      rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DilateStore, false, false>(
+          la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad", conv_flops(g));
+    } else {
+      auto la = dense_loader<64, false>(W, 1, g->C, g->C, g->K);
+      auto lb = gather_loader<64, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
+      rc = launch_igemm<64, 64, DenseLoader<64, false>, PixelGatherLoader<64, false>, DilateStore, false, false>(
+          la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad", conv_flops(g));
+    }
   } else if (path == kDgradColumns) {
     float *dcol = static_cast<float *>(workspace);
     const int CRS = g->C * RS, Ncols = g->N * g->P * g->Q;
