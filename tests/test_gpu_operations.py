@@ -126,32 +126,42 @@ def test_conv_wgrad_is_deterministic(singa, dev):
         assert_bit_equal(singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy(), a, "split-K reduction order")
 
 
-def test_conv_full_size_properties(singa, dev):
-    """BASELINE single-conv configuration (N64 C64 56x56 K64 3x3 s1 p1): too large for the CPU
-    oracle inside a test, so parity is checked through size-independent properties:
-    adjointness <conv(x,W),dy> = <x,dgrad(dy,W)> = <W,wgrad(dy,x)>, linearity in dy, and the
-    oracle on one image of the batch (dgrad is per-image; wgrad of a 1-image batch)."""
+@pytest.mark.parametrize("shape", [
+    (64, 64, 56, 64, 3, 1, 1),     # BASELINE single-conv configuration
+    (64, 3, 224, 64, 7, 2, 3),     # ResNet stem: few-channel wgrad / direct dgrad kernels
+    (64, 64, 56, 128, 3, 2, 1),    # stage transition: residue-class shared-tile dgrad, stride-2 slab wgrad
+    (64, 256, 14, 512, 1, 2, 0),   # downsample: pointwise dgrad with dilating store
+])
+def test_conv_full_size_properties(singa, dev, shape):
+    """Convolutions at the benchmark's full batch are too large for the CPU oracle inside a test,
+    so parity is checked through size-independent properties: adjointness
+    <conv(x,W),dy> = <x,dgrad(dy,W)> = <W,wgrad(dy,x)>, linearity in dy, and the oracle on one image
+    of the batch (dgrad is per-image; wgrad of a 2-image batch)."""
     r = rng(2024)
-    N, C, H, K = 64, 64, 56, 64
-    x, dy = randn(r, N, C, H, H), randn(r, N, K, H, H)
-    w = (randn(r, K, C, 3, 3) * np.sqrt(2.0 / 576)).astype(np.float32)
-    xd, wd, dyd = singa.from_numpy(x, dev), singa.from_numpy(w, dev), singa.from_numpy(dy, dev)
-    h = singa.CudnnConvHandle(xd, (3, 3), (1, 1), (1, 1), C, K, True)
+    N, C, H, K, R, st, pd = shape
+    x = randn(r, N, C, H, H)
+    w = (randn(r, K, C, R, R) * np.sqrt(2.0 / (C * R * R))).astype(np.float32)
+    xd, wd = singa.from_numpy(x, dev), singa.from_numpy(w, dev)
+    h = singa.CudnnConvHandle(xd, (R, R), (st, st), (pd, pd), C, K, True)
+    P = h.conv_height
+    dy = randn(r, N, K, P, P)
+    dyd = singa.from_numpy(dy, dev)
     y = singa.GpuConvForward(xd, wd, None, h).to_numpy().astype(np.float64)
     dx = singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy()
     dw = singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy()
     db = singa.GpuConvBackwardb(dyd, singa.from_numpy(np.zeros(K, np.float32), dev), h).to_numpy()
     lhs = float((y * dy).sum())
-    assert abs(lhs - float((x.astype(np.float64) * dx).sum())) < 1e-4 * abs(lhs)
-    assert abs(lhs - float((w.astype(np.float64) * dw).sum())) < 1e-4 * abs(lhs)
+    scale = float(np.sqrt((y * y).sum() * (dy.astype(np.float64) ** 2).sum()))  # |<y,dy>| can be small: bound by norms
+    assert abs(lhs - float((x.astype(np.float64) * dx).sum())) < 1e-5 * scale
+    assert abs(lhs - float((w.astype(np.float64) * dw).sum())) < 1e-5 * scale
     np.testing.assert_allclose(db, dy.astype(np.float64).sum(axis=(0, 2, 3)), rtol=1e-4, atol=1e-2)
     # oracle on image 5 (dgrad) and on a 2-image sub-batch (wgrad is additive over images)
-    dx5, _ = O.conv_bwd(dy[5:6], x[5:6], w, (1, 1), (1, 1), want_dw=False)
+    dx5, _ = O.conv_bwd(dy[5:6], x[5:6], w, (st, st), (pd, pd), want_dw=False)
     assert nl2(dx[5:6], dx5) < TOL
     dys = dy.copy()
     dys[2:] = 0
     dw2 = singa.GpuConvBackwardW(singa.from_numpy(dys, dev), xd, wd, h).to_numpy()
-    _, dw2_o = O.conv_bwd(dy[:2], x[:2], w, (1, 1), (1, 1), want_dx=False)
+    _, dw2_o = O.conv_bwd(dy[:2], x[:2], w, (st, st), (pd, pd), want_dx=False)
     assert nl2(dw2, dw2_o) < TOL
     # linearity: dgrad(2*dy) == 2*dgrad(dy) exactly (scaling by a power of two)
     dx2 = singa.GpuConvBackwardx(singa.from_numpy(dy * 2, dev), wd, xd, h).to_numpy()
