@@ -41,6 +41,7 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
 
 struct D3Args {
   const float *dy, *wt;   // wt: re-laid weights [tap][KP][C]
+  const float *bias;      // per output channel, added in the epilogue (NULL: none; unused with split reduction)
   float *dx;
   int N, C, H, W, K, KP;  // dx is N x C x H x W
   int P, Q;               // dy is N x K x P x Q (stride 1: P == H, Q == W; stride 2: H == 2P, W == 2Q)
@@ -232,21 +233,25 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-          if (c < a.C) o[size_t(c) * HW] = acc[i][v];
+          if (c < a.C) o[size_t(c) * HW] = a.bias ? acc[i][v] + a.bias[c] : acc[i][v];
         }
     }
   }
 }
 
-// out[i] = sum over slices (ascending) of part[z][i]
+// out[i] = sum over slices (ascending) of part[z][i] (+ bias of element i's channel)
 __global__ __launch_bounds__(256) void k_dgrad3x3_reduce(const float *__restrict__ part, float *__restrict__ out, long n4,
-                                                        int splits) {
+                                                        int splits, const float *__restrict__ bias, int HW, int C) {
   const long stride = long(gridDim.x) * 256;
   const v4f *p4 = reinterpret_cast<const v4f *>(part);
   v4f *o4 = reinterpret_cast<v4f *>(out);
   for (long i = long(blockIdx.x) * 256 + threadIdx.x; i < n4; i += stride) {
     v4f s = p4[i];
     for (int z = 1; z < splits; ++z) s += p4[z * n4 + i];
+    if (bias) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[j] += bias[((4 * i + j) / HW) % C];
+    }
     o4[i] = s;
   }
 }
@@ -342,7 +347,7 @@ size_t sgh_dgrad3x3_partial_bytes(const sgh_conv_geom *g) {
 // `wt` holds the weights re-laid as [tap][KP][C] (KP = K rounded up to 16, zero rows beyond K);
 // `partials` is sgh_dgrad3x3_partial_bytes(g) bytes of scratch (may be NULL when that is 0).
 int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, int KP, float *dx, float *partials,
-                     hipStream_t s) {
+                     hipStream_t s, const char *tag, const float *bias) {
   const D3Plan p = plan(g);
   if (!p.ok) return SGH_EUNSUPPORTED;
   if (p.splits > 1 && !partials) return SGH_EWORKSPACE;
@@ -350,6 +355,7 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   a.dy = dy;
   a.wt = wt;
   a.dx = p.splits > 1 ? partials : dx;
+  a.bias = p.splits > 1 ? nullptr : bias;  // with split reduction the bias is added by the reduction kernel
   a.N = g->N;
   a.C = g->C;
   a.H = g->H;
@@ -366,7 +372,7 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   dim3 grid((g->C + p.bm - 1) / p.bm, (a.total_pix + BN - 1) / BN, p.splits);
   if (grid.y > 65535u) return SGH_EUNSUPPORTED;
   int rc = SGH_EUNSUPPORTED;
-  sgh_prof_start("conv_dgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
+  sgh_prof_start(tag, 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
 #define D3_CASE(BM_, LOGP_, VR_) \
   if (!p.s2 && p.bm == BM_ && p.logp == LOGP_ && p.vr == VR_) rc = launch<BM_, LOGP_, VR_, false>(a, p, grid, s);
 #define D3_CASE_S2(LOGP_, VR_) \
@@ -391,7 +397,8 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
     long blocks = (n4 + 255) / 256;
     const long cap = long(sgh_num_cus()) * 16;
     if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL(k_dgrad3x3_reduce, dim3(int(blocks)), dim3(256), 0, s, partials, dx, n4, p.splits);
+    hipLaunchKernelGGL(k_dgrad3x3_reduce, dim3(int(blocks)), dim3(256), 0, s, partials, dx, n4, p.splits, bias,
+                       g->H * g->W, g->C);
     if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
   }
   return SGH_OK;

@@ -555,10 +555,15 @@ __global__ __launch_bounds__(256) void k_split_reduce_lanes(const float *__restr
 }
 
 // Weight re-layout for the pixel-gather passes:  W[K][C][R][S]  ->  Wt[tap][chp][m]
-//   forward: ch = c (padded to CP), m = k   -> Wt[(tap * CP + c) * K + k]
-//   dgrad:   ch = k (padded to KP), m = c   -> Wt[(tap * KP + k) * C + c]
+//   forward (mode 0): ch = c (padded to CP), m = k   -> Wt[(tap * CP + c) * K + k]
+//   dgrad   (mode 1): ch = k (padded to KP), m = c   -> Wt[(tap * KP + k) * C + c]
+//   forward with the taps in reverse order (mode 2): as mode 0 from W[..][RS - 1 - tap]; a
+//   correlation with the flipped filter is what the shared-tile data-gradient kernel computes,
+//   so that kernel then evaluates the forward convolution
 __global__ __launch_bounds__(NT) void k_weight_relayout(const float *__restrict__ W, float *__restrict__ Wt, int K, int C,
                                                        int RS, int CHP, int dgrad) {
+  const bool flip = dgrad == 2;
+  if (flip) dgrad = 0;
   const long total = long(RS) * CHP * (dgrad ? C : K);
   const long stride = long(gridDim.x) * NT;
   const int Mdim = dgrad ? C : K;
@@ -570,7 +575,7 @@ __global__ __launch_bounds__(NT) void k_weight_relayout(const float *__restrict_
     if (dgrad) {
       if (ch < K) v = W[(long(ch) * C + m) * RS + tap];
     } else {
-      if (ch < C) v = W[(long(m) * C + ch) * RS + tap];
+      if (ch < C) v = W[(long(m) * C + ch) * RS + (flip ? RS - 1 - tap : tap)];
     }
     Wt[i] = v;
   }
@@ -831,6 +836,17 @@ inline DgradPath dgrad_path(const sgh_conv_geom *g) {
 
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
+// A 3x3 stride-1 pad-1 forward convolution is the data gradient of the channel-swapped problem
+// with the filter taps reversed; `gt` receives that problem when the shared-tile kernel covers it.
+inline bool fwd_as_dgrad(const sgh_conv_geom *g, sgh_conv_geom *gt) {
+  if (g->R != 3 || g->S != 3 || g->stride_h != 1 || g->stride_w != 1 || g->pad_h != 1 || g->pad_w != 1) return false;
+  if (g->C % BK != 0) return false;  // the reduction (input channels) runs in whole chunks
+  *gt = *g;
+  gt->C = g->K;
+  gt->K = g->C;
+  return sgh_dgrad3x3_supported(gt);
+}
+
 }  // namespace
 
 extern "C" {
@@ -863,7 +879,11 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
   if (!conv_ok(g)) return 0;
   const size_t RS = size_t(g->R) * g->S;
   switch (which) {
-    case SGH_CONV_FWD: return RS * round_up(g->C, BK) * g->K * sizeof(float);
+    case SGH_CONV_FWD: {
+      sgh_conv_geom gt;
+      const size_t wt = RS * round_up(g->C, BK) * g->K * sizeof(float);
+      return fwd_as_dgrad(g, &gt) ? align256(wt) + sgh_dgrad3x3_partial_bytes(&gt) : wt;
+    }
     case SGH_CONV_DGRAD:
       if (dgrad_path(g) == kDgradFewC) return sgh_dgrad_fewc_workspace_bytes(g);
       if (dgrad_path(g) == kDgradPointwise) return 0;
@@ -943,7 +963,7 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
     float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) +
                                                 align256(size_t(RS) * KP * g->C * sizeof(float)) +
                                                 align256(sizeof(DgClsTable)));
-    rc = sgh_dgrad3x3_run(g, dy, Wt, KP, dx, partials, s);
+    rc = sgh_dgrad3x3_run(g, dy, Wt, KP, dx, partials, s, "conv_dgrad", nullptr);
   } else if (path == kDgradClasses) {
     float *Wc = static_cast<float *>(workspace);
     const size_t wc_bytes = size_t(RS) * KP * g->C * sizeof(float);
@@ -1032,6 +1052,19 @@ int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, con
   float *Wt = static_cast<float *>(workspace);
   const int RS = g->R * g->S, CP = round_up(g->C, BK);
   sgh_prof_start("conv_fwd_op", conv_flops(g), s);
+  sgh_conv_geom gt;
+  if (fwd_as_dgrad(g, &gt)) {
+    // 3x3 stride 1 pad 1: the shared-tile kernel on the channel-swapped problem with reversed taps
+    const long total = long(RS) * CP * g->K;
+    long blocks = (total + NT - 1) / NT;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, CP, 2);
+    float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) +
+                                                align256(size_t(RS) * CP * g->K * sizeof(float)));
+    const int rc3 = sgh_dgrad3x3_run(&gt, x, Wt, CP, y, partials, s, "conv_fwd", bias);
+    sgh_prof_stop(s);
+    return rc3;
+  }
   {
     const long total = long(RS) * CP * g->K;
     long blocks = (total + NT - 1) / NT;

@@ -61,9 +61,9 @@ CONV_CASES = [
     (2, 3, 32, 32, 32, 5, 5, (1, 1), (2, 2), True),       # small-CNN conv1
     (2, 32, 16, 16, 64, 5, 5, (1, 1), (2, 2), True),      # small-CNN conv2
     (2, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3), False),      # ResNet stem (reduced image)
-    (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), False),     # stage-1 class
+    (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), True),      # stage-1 class (forward: shared-tile kernel with bias)
     (2, 64, 14, 14, 128, 3, 3, (2, 2), (1, 1), False),    # stage transition
-    (2, 128, 7, 7, 128, 3, 3, (1, 1), (1, 1), False),     # odd spatial size
+    (2, 128, 7, 7, 128, 3, 3, (1, 1), (1, 1), True),      # odd spatial size (forward bias added by the split reduction)
     (1, 130, 9, 9, 70, 3, 3, (1, 1), (1, 1), False),      # channel counts that are not tile multiples
     (4, 8, 5, 5, 8, 3, 3, (1, 1), (0, 0), False),         # no padding
     (1, 1, 3, 3, 1, 3, 3, (1, 1), (2, 2), False),         # pad wider than half the kernel
