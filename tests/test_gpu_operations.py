@@ -302,3 +302,58 @@ def test_bn_vs_oracle(singa, dev, shape):
                                                singa.from_numpy(inv_o, dev))
     assert_bit_equal(dx2.to_numpy(), dx.to_numpy())
     assert_bit_equal(ds2.to_numpy(), ds.to_numpy())
+
+
+def _random_conv_cases(count, seed):
+    """Seeded geometry sweep aimed at the planning logic of the specialised kernels: channel counts
+    around the 32 / 64 / 128 tile edges, image sizes around the 16 / 32 / 64-column slab limits,
+    strides 1-2, 1x1 / 3x3 / 5x5 / 7x7 filters, every legal padding."""
+    r = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        R = int(r.choice([1, 3, 3, 3, 5, 7]))
+        st = int(r.choice([1, 1, 2]))
+        pd = int(r.integers(0, R // 2 + 2))
+        C = int(r.choice([1, 3, 4, 16, 31, 32, 33, 48, 64, 65, 96, 128, 130]))
+        K = int(r.choice([8, 16, 32, 48, 63, 64, 65, 96, 128, 144]))
+        H = int(r.integers(max(R - 2 * pd, 1), 34)) if r.random() < 0.7 else int(r.choice([56, 58, 62, 63]))
+        W = H if r.random() < 0.6 else int(r.integers(max(R - 2 * pd, 1), 40))
+        if H + 2 * pd < R or W + 2 * pd < R:
+            continue
+        N = int(r.integers(1, 4))
+        P, Q = (H + 2 * pd - R) // st + 1, (W + 2 * pd - R) // st + 1
+        if N * K * P * Q * C * R * R > 4e8:   # keep the CPU oracle quick
+            continue
+        cases.append((N, C, H, W, K, R, R, (st, st), (pd, pd), bool(r.random() < 0.3)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_conv_cases(48, 20240607))
+def test_conv_geometry_sweep(singa, dev, case):
+    test_conv_backward_vs_oracle(singa, dev, case)
+
+
+def _shared_tile_cases(count, seed):
+    """3x3 pad-1 geometries the shared-tile kernels accept (C >= 64, K a multiple of 16), over image
+    sizes that move the slab pitch / rows-per-tile choices and make tiles straddle images."""
+    r = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        st = int(r.choice([1, 1, 2]))
+        C = int(r.choice([64, 68, 96, 128, 192, 256]))
+        K = int(r.choice([64, 80, 96, 128, 160, 256]))
+        H = int(r.integers(2, 32)) * (2 if st == 2 else 1)
+        W = int(r.integers(2, 32)) * (2 if st == 2 else 1)
+        if st == 1 and r.random() < 0.5:
+            H, W = int(r.integers(2, 63)), int(r.integers(2, 63))
+        N = int(r.integers(1, 6))
+        P, Q = (H + 2 - 3) // st + 1, (W + 2 - 3) // st + 1
+        if N * K * P * Q * C * 9 > 6e8:
+            continue
+        cases.append((N, C, H, W, K, 3, 3, (st, st), (1, 1), bool(r.random() < 0.3)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _shared_tile_cases(40, 777))
+def test_conv_shared_tile_sweep(singa, dev, case):
+    test_conv_backward_vs_oracle(singa, dev, case)
