@@ -146,6 +146,32 @@ SGH_API int sgh_eltwise_mult_f32(const float *a, const float *b, int b_is_scalar
  * of python/singa/autograd.py:204.  out may alias a or b. */
 SGH_API int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream);
 
+/* -------------------------------------------------------------------------------------
+ * 16-bit storage variants: IEEE binary16 ("f16", the reference's half_float::half / __half
+ * tensors) and bfloat16 ("bf16") travel as uint16_t arrays.  Arithmetic is fp32 with one
+ * rounding to nearest-even on store, like the reference's half kernels
+ * (__half2float / __float2half in src/core/tensor/math_kernel.cu).
+ * ------------------------------------------------------------------------------------- */
+/* CastCopy<float, half, Lang> / CastCopy<half, float, Lang> (Tensor::AsType):
+ * src/core/tensor/tensor_math_cuda.h:193-208, math_kernel.cu float2half / half2float. */
+SGH_API int sgh_cast_f32_to_f16(const float *src, uint16_t *dst, size_t n, void *stream);
+SGH_API int sgh_cast_f16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream);
+SGH_API int sgh_cast_f32_to_bf16(const float *src, uint16_t *dst, size_t n, void *stream);
+SGH_API int sgh_cast_bf16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream);
+/* ReLUBackward<half, Lang>: tensor_math_cuda.h:665-674, math_kernel.cu:261-271.  Follows the
+ * CPU rule dx = x > 0 ? dy : 0 (the CUDA half kernel alone passes the gradient at x == 0). */
+SGH_API int sgh_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream);
+SGH_API int sgh_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream);
+/* Add / EltwiseMult<half, Lang>: tensor_math_cuda.h:345-362, math_kernel.cu:111-117, :353-359.
+ * out may alias an input. */
+SGH_API int sgh_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream);
+SGH_API int sgh_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream);
+SGH_API int sgh_eltwise_mult_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream);
+SGH_API int sgh_eltwise_mult_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream);
+/* Axpy<half, Lang> (scalar alpha): tensor_math_cuda.h:1064-1072 (cublasAxpyEx, fp32 compute). */
+SGH_API int sgh_axpy_f16(float alpha, const uint16_t *x, uint16_t *y, size_t n, void *stream);
+SGH_API int sgh_axpy_bf16(float alpha, const uint16_t *x, uint16_t *y, size_t n, void *stream);
+
 /* Fused SGD-momentum update = the four tensor ops of SGD.apply, python/singa/opt.py:269-310,
  * in one pass:  [g += wd*p];  v = mu*v + (1-damp)*g;  g' = nesterov ? g + mu*v : v;
  * p -= lr*g'.  wd == 0 and mu == 0 skip their terms exactly like the Python `if`s; with

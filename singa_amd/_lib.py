@@ -66,6 +66,18 @@ SIGNATURES = {
     "sgh_axpy_devalpha_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_eltwise_mult_f32": (C.c_int, [vp, vp, C.c_int, vp, sz, vp]),
     "sgh_add_f32": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_cast_f32_to_f16": (C.c_int, [vp, vp, sz, vp]),
+    "sgh_cast_f16_to_f32": (C.c_int, [vp, vp, sz, vp]),
+    "sgh_cast_f32_to_bf16": (C.c_int, [vp, vp, sz, vp]),
+    "sgh_cast_bf16_to_f32": (C.c_int, [vp, vp, sz, vp]),
+    "sgh_relu_bwd_f16": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_relu_bwd_bf16": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_add_f16": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_add_bf16": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_eltwise_mult_f16": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_eltwise_mult_bf16": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_axpy_f16": (C.c_int, [C.c_float, vp, vp, sz, vp]),
+    "sgh_axpy_bf16": (C.c_int, [C.c_float, vp, vp, sz, vp]),
     "sgh_sgd_momentum_f32": (C.c_int, [vp, vp, vp, sz, C.c_float, C.c_float, C.c_float, C.c_float,
                                        C.c_int, vp]),
     "sgh_sgd_momentum_devhyper_f32": (C.c_int, [vp, vp, vp, sz, vp, C.c_int, vp]),

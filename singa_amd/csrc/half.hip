@@ -1,0 +1,235 @@
+// 16-bit storage variants of the bandwidth-bound backward ops: IEEE binary16 ("f16") and bfloat16
+// ("bf16") tensors travel as uint16_t arrays; arithmetic is fp32 with ONE rounding (to nearest,
+// ties to even) when a result is stored, which is what the reference's half kernels do through
+// __half2float / __float2half (src/core/tensor/math_kernel.cu:111-117, :261-271, :353-375).
+// ReLU backward keeps the CPU rule (gradient 0 at x == 0), not the CUDA half kernel's '>='.
+//
+// Each thread moves 16 bytes (8 elements) per access; a workgroup streams contiguous 16 KB
+// chunks, as in the fp32 kernels.
+#include "common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;
+
+typedef unsigned short u16;
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+struct F16 {
+  static __device__ __forceinline__ float load(u16 b) {
+    _Float16 h;
+    __builtin_memcpy(&h, &b, 2);
+    return float(h);
+  }
+  static __device__ __forceinline__ u16 store(float f) {
+    const _Float16 h = _Float16(f);  // v_cvt_f16_f32: round to nearest even
+    u16 b;
+    __builtin_memcpy(&b, &h, 2);
+    return b;
+  }
+};
+
+struct BF16 {
+  static __device__ __forceinline__ float load(u16 b) { return __builtin_bit_cast(float, unsigned(b) << 16); }
+  static __device__ __forceinline__ u16 store(float f) {
+    unsigned u = __builtin_bit_cast(unsigned, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return u16((u >> 16) | 0x40u);  // NaN stays a (quiet) NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                      // round to nearest even
+    return u16(u >> 16);
+  }
+};
+
+struct F32 {};  // marker for the fp32 side of a cast
+
+inline int grid_for(size_t nvec) {
+  size_t per_block = size_t(kBlock) * kUnroll;
+  size_t blocks = (nvec + per_block - 1) / per_block;
+  const size_t cap = size_t(sgh_num_cus()) * 16;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return int(blocks);
+}
+
+// out = f(a, b) over 16-bit tensors; vectors of 8 elements
+template <class T, class F>
+__global__ __launch_bounds__(kBlock) void k_map2_h(const u16 *a, const u16 *b, u16 *o, size_t n, F f, int vec) {
+  if (vec) {
+    const size_t nvec = n >> 3;
+    const v4u *a4 = reinterpret_cast<const v4u *>(a);
+    const v4u *b4 = reinterpret_cast<const v4u *>(b);
+    v4u *o4 = reinterpret_cast<v4u *>(o);
+    const size_t step = size_t(gridDim.x) * (kBlock * kUnroll);
+    for (size_t base = size_t(blockIdx.x) * (kBlock * kUnroll); base < nvec; base += step) {
+      v4u va[kUnroll], vb[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const size_t i = base + u * kBlock + threadIdx.x;
+        if (i < nvec) {
+          va[u] = a4[i];
+          vb[u] = b4[i];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const size_t i = base + u * kBlock + threadIdx.x;
+        if (i < nvec) {
+          v4u r;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float lo = f(T::load(u16(va[u][j] & 0xffffu)), T::load(u16(vb[u][j] & 0xffffu)));
+            const float hi = f(T::load(u16(va[u][j] >> 16)), T::load(u16(vb[u][j] >> 16)));
+            r[j] = unsigned(T::store(lo)) | (unsigned(T::store(hi)) << 16);
+          }
+          o4[i] = r;
+        }
+      }
+    }
+    if (blockIdx.x == 0) {
+      const size_t t = (nvec << 3) + threadIdx.x;
+      if (t < n) o[t] = T::store(f(T::load(a[t]), T::load(b[t])));
+    }
+  } else {
+    const size_t stride = size_t(gridDim.x) * kBlock;
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride)
+      o[i] = T::store(f(T::load(a[i]), T::load(b[i])));
+  }
+}
+
+template <class T, class F>
+int launch_map2_h(const uint16_t *a, const uint16_t *b, uint16_t *o, size_t n, F f, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!a || !b || !o) return SGH_EINVAL;
+  const int vec = sgh_aligned16(a) && sgh_aligned16(b) && sgh_aligned16(o);
+  hipLaunchKernelGGL((k_map2_h<T, F>), dim3(grid_for(vec ? n >> 3 : n)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o,
+                     n, f, vec);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+struct ReluBwd {
+  __device__ __forceinline__ float operator()(float dy, float x) const { return x > 0.f ? dy : 0.f; }
+};
+struct AddOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+struct MulOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a * b; }
+};
+struct AxpyOp {  // (x, y) -> y + alpha * x in fp32 (two fp32 roundings, then the storage rounding)
+  float alpha;
+  __device__ __forceinline__ float operator()(float x, float y) const {
+#pragma clang fp contract(off)
+    const float t = alpha * x;
+    return y + t;
+  }
+};
+
+// casts: fp32 <-> 16-bit, 8 elements per thread per access on the 16-bit side
+template <class T>
+__global__ __launch_bounds__(kBlock) void k_cast_to16(const float *__restrict__ src, u16 *__restrict__ dst, size_t n,
+                                                     int vec) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  if (vec) {
+    const size_t nvec = n >> 3;
+    const float4 *s4 = reinterpret_cast<const float4 *>(src);
+    v4u *d4 = reinterpret_cast<v4u *>(dst);
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += stride) {
+      const float4 x0 = s4[2 * i], x1 = s4[2 * i + 1];
+      v4u r;
+      r[0] = unsigned(T::store(x0.x)) | (unsigned(T::store(x0.y)) << 16);
+      r[1] = unsigned(T::store(x0.z)) | (unsigned(T::store(x0.w)) << 16);
+      r[2] = unsigned(T::store(x1.x)) | (unsigned(T::store(x1.y)) << 16);
+      r[3] = unsigned(T::store(x1.z)) | (unsigned(T::store(x1.w)) << 16);
+      d4[i] = r;
+    }
+    if (blockIdx.x == 0) {
+      const size_t t = (nvec << 3) + threadIdx.x;
+      if (t < n) dst[t] = T::store(src[t]);
+    }
+  } else {
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) dst[i] = T::store(src[i]);
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void k_cast_from16(const u16 *__restrict__ src, float *__restrict__ dst, size_t n,
+                                                       int vec) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  if (vec) {
+    const size_t nvec = n >> 3;
+    const v4u *s4 = reinterpret_cast<const v4u *>(src);
+    float4 *d4 = reinterpret_cast<float4 *>(dst);
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += stride) {
+      const v4u v = s4[i];
+      d4[2 * i] = make_float4(T::load(u16(v[0] & 0xffffu)), T::load(u16(v[0] >> 16)), T::load(u16(v[1] & 0xffffu)),
+                              T::load(u16(v[1] >> 16)));
+      d4[2 * i + 1] = make_float4(T::load(u16(v[2] & 0xffffu)), T::load(u16(v[2] >> 16)), T::load(u16(v[3] & 0xffffu)),
+                                  T::load(u16(v[3] >> 16)));
+    }
+    if (blockIdx.x == 0) {
+      const size_t t = (nvec << 3) + threadIdx.x;
+      if (t < n) dst[t] = T::load(src[t]);
+    }
+  } else {
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) dst[i] = T::load(src[i]);
+  }
+}
+
+template <class T>
+int cast_to16(const float *src, uint16_t *dst, size_t n, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!src || !dst) return SGH_EINVAL;
+  const int vec = sgh_aligned16(src) && sgh_aligned16(dst);
+  hipLaunchKernelGGL(k_cast_to16<T>, dim3(grid_for(vec ? n >> 3 : n)), dim3(kBlock), 0, sgh_stream_of(stream), src, dst, n,
+                     vec);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+template <class T>
+int cast_from16(const uint16_t *src, float *dst, size_t n, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!src || !dst) return SGH_EINVAL;
+  const int vec = sgh_aligned16(src) && sgh_aligned16(dst);
+  hipLaunchKernelGGL(k_cast_from16<T>, dim3(grid_for(vec ? n >> 3 : n)), dim3(kBlock), 0, sgh_stream_of(stream), src, dst,
+                     n, vec);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sgh_cast_f32_to_f16(const float *src, uint16_t *dst, size_t n, void *stream) { return cast_to16<F16>(src, dst, n, stream); }
+int sgh_cast_f16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream) { return cast_from16<F16>(src, dst, n, stream); }
+int sgh_cast_f32_to_bf16(const float *src, uint16_t *dst, size_t n, void *stream) { return cast_to16<BF16>(src, dst, n, stream); }
+int sgh_cast_bf16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream) { return cast_from16<BF16>(src, dst, n, stream); }
+
+int sgh_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream) {
+  return launch_map2_h<F16>(dy, x, dx, n, ReluBwd{}, stream);
+}
+int sgh_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream) {
+  return launch_map2_h<BF16>(dy, x, dx, n, ReluBwd{}, stream);
+}
+int sgh_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  return launch_map2_h<F16>(a, b, out, n, AddOp{}, stream);
+}
+int sgh_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  return launch_map2_h<BF16>(a, b, out, n, AddOp{}, stream);
+}
+int sgh_eltwise_mult_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  return launch_map2_h<F16>(a, b, out, n, MulOp{}, stream);
+}
+int sgh_eltwise_mult_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  return launch_map2_h<BF16>(a, b, out, n, MulOp{}, stream);
+}
+int sgh_axpy_f16(float alpha, const uint16_t *x, uint16_t *y, size_t n, void *stream) {
+  return launch_map2_h<F16>(x, y, y, n, AxpyOp{alpha}, stream);
+}
+int sgh_axpy_bf16(float alpha, const uint16_t *x, uint16_t *y, size_t n, void *stream) {
+  return launch_map2_h<BF16>(x, y, y, n, AxpyOp{alpha}, stream);
+}
+
+}  // extern "C"

@@ -26,11 +26,37 @@ from ._lib import SingaHipError, check  # noqa: F401  (re-exported)
 
 # core.proto DataType values (src/proto/core.proto:26-34)
 kFloat32, kFloat16, kInt = 0, 1, 2
+# bfloat16 storage is not a SINGA data type; the value lies outside core.proto's range
+kBFloat16 = 100
 # core.proto LangType (src/proto/core.proto:36-41); 3 is the value a HIP backend takes
 kCpp, kCuda, kOpencl, kHip = 0, 1, 2, 3
 
-_NP_OF = {kFloat32: np.float32, kInt: np.int32}
-_SIZE_OF = {kFloat32: 4, kInt: 4}
+_NP_OF = {kFloat32: np.float32, kInt: np.int32, kFloat16: np.float16, kBFloat16: np.uint16}
+_SIZE_OF = {kFloat32: 4, kInt: 4, kFloat16: 2, kBFloat16: 2}
+_SUFFIX = {kFloat32: "f32", kFloat16: "f16", kBFloat16: "bf16"}
+
+
+def _fn(name, t):
+    """The entry point of `name` for t's data type: sgh_<name>_<f32|f16|bf16>."""
+    sfx = _SUFFIX.get(t.data_type())
+    if sfx is None:
+        raise SingaHipError("%s: unsupported data type %r" % (name, t.data_type()))
+    full = "sgh_%s_%s" % (name, sfx)
+    return getattr(_L(), full), full
+
+
+def bf16_bits_to_float(bits):
+    """uint16 bfloat16 payloads -> float32 values (exact)."""
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def float_to_bf16_bits(a):
+    """float32 -> bfloat16 payloads, round to nearest even (NaN stays NaN)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = (u & 0x7fffffff) > 0x7f800000
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return r
 
 USE_HIP = True
 
@@ -203,10 +229,36 @@ class Tensor(object):
             raise SingaHipError("size or type mismatch in CopyIntDataFromHostPtr")
         check(_L().sgh_memcpy(self._dev._h, self.ptr, a.ctypes.data, a.nbytes, 1), "sgh_memcpy H2D")
 
+    def CopyHalfDataFromHostPtr(self, arr):
+        """float16 values (kFloat16) or raw uint16 bfloat16 payloads (kBFloat16)."""
+        a = np.ascontiguousarray(arr, dtype=_NP_OF[self._dtype]).ravel()
+        if a.size != self.Size() or self._dtype not in (kFloat16, kBFloat16):
+            raise SingaHipError("size or type mismatch in CopyHalfDataFromHostPtr")
+        check(_L().sgh_memcpy(self._dev._h, self.ptr, a.ctypes.data, a.nbytes, 1), "sgh_memcpy H2D")
+
+    def AsType(self, dtype):
+        """``Tensor::AsType`` (src/core/tensor/tensor.cc:197-214) between fp32 and a 16-bit type."""
+        if dtype == self._dtype:
+            return self
+        if self._transposed:
+            raise SingaHipError("AsType of a transposed view is not supported")
+        out = Tensor(self._shape, self._dev, dtype)
+        if self._dtype == kFloat32 and dtype in (kFloat16, kBFloat16):
+            name = "sgh_cast_f32_to_%s" % _SUFFIX[dtype]
+        elif dtype == kFloat32 and self._dtype in (kFloat16, kBFloat16):
+            name = "sgh_cast_%s_to_f32" % _SUFFIX[self._dtype]
+        else:
+            raise SingaHipError("AsType %r -> %r is not on the backward path" % (self._dtype, dtype))
+        check(getattr(_L(), name)(self.ptr, out.ptr, self.Size(), self._dev.stream), name)
+        return out
+
     def to_numpy(self):
+        """fp32 / int32 / float16 arrays; bfloat16 tensors come back as float32 values."""
         out = np.empty(self.Size(), dtype=_NP_OF[self._dtype])
         if out.size:
             check(_L().sgh_memcpy(self._dev._h, out.ctypes.data, self.ptr, out.nbytes, 2), "sgh_memcpy D2H")
+        if self._dtype == kBFloat16:
+            out = bf16_bits_to_float(out)
         if self._transposed:
             return out.reshape(self._shape[1], self._shape[0]).T.copy()
         return out.reshape(self._shape)
@@ -217,7 +269,8 @@ class Tensor(object):
     # --- arithmetic used by autograd / opt  (Tensor::operator+=, *=: src/core/tensor/tensor.cc:579-589)
     def __iadd__(self, other):
         _same(self, other)
-        check(_L().sgh_add_f32(self.ptr, other.ptr, self.ptr, self.Size(), self._dev.stream), "sgh_add_f32")
+        fn, name = _fn("add", self)
+        check(fn(self.ptr, other.ptr, self.ptr, self.Size(), self._dev.stream), name)
         return self
 
     def __imul__(self, other):
@@ -247,6 +300,10 @@ def _same(a, b):
 
 def from_numpy(arr, device):
     arr = np.asarray(arr)
+    if arr.dtype == np.float16:
+        t = Tensor(arr.shape, device, kFloat16)
+        t.CopyHalfDataFromHostPtr(arr)
+        return t
     if arr.dtype in (np.int32, np.int64):
         t = Tensor(arr.shape, device, kInt)
         t.CopyIntDataFromHostPtr(arr)
@@ -291,7 +348,8 @@ def ReLUBackward(dy, x):
     """``singa.ReLUBackward(dy, x)`` (python/singa/autograd.py:432-439)."""
     _same(dy, x)
     dx = _like(dy)
-    check(_L().sgh_relu_bwd_f32(dy.ptr, x.ptr, dx.ptr, dy.Size(), dy.device().stream), "sgh_relu_bwd_f32")
+    fn, name = _fn("relu_bwd", dy)
+    check(fn(dy.ptr, x.ptr, dx.ptr, dy.Size(), dy.device().stream), name)
     return dx
 
 
@@ -349,7 +407,8 @@ def Axpy(alpha, x, y):
         check(_L().sgh_axpy_devalpha_f32(alpha.ptr, x.ptr, y.ptr, x.Size(), x.device().stream),
               "sgh_axpy_devalpha_f32")
     else:
-        check(_L().sgh_axpy_f32(float(alpha), x.ptr, y.ptr, x.Size(), x.device().stream), "sgh_axpy_f32")
+        fn, name = _fn("axpy", x)
+        check(fn(float(alpha), x.ptr, y.ptr, x.Size(), x.device().stream), name)
 
 
 def EltwiseMult(a, b, out=None):
@@ -357,6 +416,12 @@ def EltwiseMult(a, b, out=None):
     scalar = b.Size() == 1 and a.Size() != 1
     if not scalar:
         _same(a, b)
+    if a.data_type() != kFloat32:
+        if scalar:
+            raise SingaHipError("scalar EltwiseMult is fp32 only")
+        fn, name = _fn("eltwise_mult", a)
+        check(fn(a.ptr, b.ptr, out.ptr, a.Size(), a.device().stream), name)
+        return out
     check(_L().sgh_eltwise_mult_f32(a.ptr, b.ptr, int(scalar), out.ptr, a.Size(), a.device().stream),
           "sgh_eltwise_mult_f32")
     return out
@@ -365,7 +430,8 @@ def EltwiseMult(a, b, out=None):
 def __add__(a, b):
     _same(a, b)
     out = _like(a)
-    check(_L().sgh_add_f32(a.ptr, b.ptr, out.ptr, a.Size(), a.device().stream), "sgh_add_f32")
+    fn, name = _fn("add", a)
+    check(fn(a.ptr, b.ptr, out.ptr, a.Size(), a.device().stream), name)
     return out
 
 

@@ -1,0 +1,90 @@
+"""16-bit storage variants (binary16 and bfloat16) of the elementwise backward ops and the casts,
+checked bit for bit against numpy: numpy's float32 -> float16 conversion rounds to nearest even, as
+the kernels do, and the bfloat16 reference rounding is written out in singa_wrap.float_to_bf16_bits.
+(The reference has no CPU half arithmetic to restate: its half_float type is "for labeling only",
+src/core/tensor/tensor_math_cuda.h:195; the CUDA kernels compute in fp32 and round once.)"""
+import numpy as np
+import pytest
+
+from util import rng
+
+pytestmark = pytest.mark.gpu
+
+@pytest.fixture(scope="module")
+def singa():
+    from singa_amd import singa_wrap
+    return singa_wrap
+
+
+SIZES = [1, 7, 8, 9, 1000, 4096 + 3, 64 * 1024 + 5, 3 * 1000 * 1000 + 1]
+
+
+def _special(r, n):
+    """N(0,1) values salted with zeros, signed zeros, subnormals, huge values, infinities and NaN."""
+    a = r.standard_normal(n).astype(np.float32)
+    if n >= 64:
+        a[1:64:7] = [0.0, -0.0, 1e-7, -1e-7, 6.0e-5, 65504.0, 65520.0, 1e38, np.inf][: len(a[1:64:7])]
+        a[5] = np.nan
+    return a
+
+
+def _to(singa, dev, a32, kind):
+    if kind == "f16":
+        with np.errstate(over="ignore"):
+            h = a32.astype(np.float16)
+        return singa.from_numpy(h, dev), h.astype(np.float32)
+    bits = singa.float_to_bf16_bits(a32)
+    t = singa.Tensor(a32.shape, dev, singa.kBFloat16)
+    t.CopyHalfDataFromHostPtr(bits)
+    return t, singa.bf16_bits_to_float(bits)
+
+
+def _round(singa, a32, kind):
+    """fp32 result -> the values the 16-bit store keeps (as float32)."""
+    if kind == "f16":
+        with np.errstate(over="ignore"):
+            return a32.astype(np.float16).astype(np.float32)
+    return singa.bf16_bits_to_float(singa.float_to_bf16_bits(a32))
+
+
+def _same_bits(got, want, what):
+    g, w = np.asarray(got, np.float32).ravel(), np.asarray(want, np.float32).ravel()
+    both_nan = np.isnan(g) & np.isnan(w)
+    bad = (g.view(np.uint32) != w.view(np.uint32)) & ~both_nan
+    assert not bad.any(), "%s: %d of %d differ, first at %d: %r vs %r" % (
+        what, bad.sum(), g.size, np.argmax(bad), g[np.argmax(bad)], w[np.argmax(bad)])
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("n", SIZES)
+def test_casts(singa, dev, kind, n):
+    r = rng(n)
+    a = _special(r, n)
+    dtype = singa.kFloat16 if kind == "f16" else singa.kBFloat16
+    t = singa.from_numpy(a, dev).AsType(dtype)
+    assert t.data_type() == dtype and t.MemSize() == 2 * n
+    _same_bits(t.to_numpy(), _round(singa, a, kind), "fp32 -> " + kind)
+    back = t.AsType(singa.kFloat32)
+    _same_bits(back.to_numpy(), _round(singa, a, kind), kind + " -> fp32")
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("n", SIZES)
+def test_relu_backward_add_mult_axpy(singa, dev, kind, n):
+    r = rng(1000 + n)
+    dyt, dy = _to(singa, dev, _special(r, n), kind)
+    xt, x = _to(singa, dev, _special(r, n), kind)
+    # ReLU backward: a select, so exact; gradient 0 at x == 0 (and at -0.0, NaN)
+    _same_bits(singa.ReLUBackward(dyt, xt).to_numpy(), np.where(x > 0, dy, np.float32(0)), "relu_bwd " + kind)
+    with np.errstate(invalid="ignore", over="ignore"):
+        _same_bits(singa.__add__(dyt, xt).to_numpy(), _round(singa, dy + x, kind), "add " + kind)
+        _same_bits(singa.EltwiseMult(dyt, xt).to_numpy(), _round(singa, dy * x, kind), "mult " + kind)
+        alpha = np.float32(-0.05)
+        want = _round(singa, x + alpha * dy, kind)     # two fp32 roundings, then the storage rounding
+        singa.Axpy(float(alpha), dyt, xt)              # xt += alpha * dyt
+        _same_bits(xt.to_numpy(), want, "axpy " + kind)
+    # in place accumulate (gradient fan-in)
+    at, a = _to(singa, dev, r.standard_normal(n).astype(np.float32), kind)
+    bt, b = _to(singa, dev, r.standard_normal(n).astype(np.float32), kind)
+    at += bt
+    _same_bits(at.to_numpy(), _round(singa, a + b, kind), "iadd " + kind)

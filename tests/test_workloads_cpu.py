@@ -62,3 +62,17 @@ def test_small_resnet_step_runs_and_learns():
         l1 = float(np.mean(net.forward(xs, ls)))
     assert dxin.shape == x.shape          # the stem's dgrad is computed like SINGA does
     assert np.isfinite(l1) and l1 < l0    # three steps on one batch reduce its loss
+
+
+def test_bf16_host_rounding():
+    """float_to_bf16_bits is the reference rounding the GPU tests compare with: ties to even,
+    carries into the exponent, infinities and NaN preserved."""
+    from singa_amd.singa_wrap import bf16_bits_to_float, float_to_bf16_bits
+    a = np.array([1.0, 1.00390625, 1.01171875, 3.4e38, -0.0, np.inf, -np.inf], np.float32)
+    b = float_to_bf16_bits(a)
+    assert list(b[:3]) == [0x3F80, 0x3F80, 0x3F82]          # tie -> even (down), tie -> even (up)
+    assert b[3] == 0x7F80 and b[4] == 0x8000 and b[5] == 0x7F80 and b[6] == 0xFF80   # overflow rounds to inf
+    assert np.isnan(bf16_bits_to_float(float_to_bf16_bits(np.array([np.nan], np.float32)))).all()
+    x = np.random.default_rng(0).standard_normal(1000).astype(np.float32)
+    y = bf16_bits_to_float(float_to_bf16_bits(x))
+    assert np.abs(y - x).max() <= np.abs(x).max() * 2.0 ** -8
