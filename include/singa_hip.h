@@ -268,6 +268,25 @@ SGH_API int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma,
                            const float *save_mean, const float *save_invstd, float *dx,
                            float *dgamma, float *dbeta, int N, int C, int HW, void *workspace,
                            size_t ws_bytes, void *stream);
+/* The same two operations on 16-bit activations (x, y, dy, dx binary16 or bfloat16) with fp32
+ * gamma / beta / statistics / parameter gradients -- cuDNN's convention for half tensors, which
+ * the reference's handle selects from the input's data type (batchnorm.cc:261-285). */
+SGH_API int sgh_bn_fwd_train_f16(const uint16_t *x, const float *gamma, const float *beta,
+                                 float *running_mean, float *running_var, float factor, float eps,
+                                 uint16_t *y, float *save_mean, float *save_invstd, int N, int C,
+                                 int HW, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_fwd_train_bf16(const uint16_t *x, const float *gamma, const float *beta,
+                                  float *running_mean, float *running_var, float factor, float eps,
+                                  uint16_t *y, float *save_mean, float *save_invstd, int N, int C,
+                                  int HW, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma,
+                           const float *save_mean, const float *save_invstd, uint16_t *dx,
+                           float *dgamma, float *dbeta, int N, int C, int HW, void *workspace,
+                           size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma,
+                            const float *save_mean, const float *save_invstd, uint16_t *dx,
+                            float *dgamma, float *dbeta, int N, int C, int HW, void *workspace,
+                            size_t ws_bytes, void *stream);
 
 /* Geometry of a PoolingHandle (src/model/operation/pooling.h:40-71; ctor pooling.cc:27-52). */
 typedef struct sgh_pool_geom {

@@ -8,6 +8,7 @@
 // Reductions are a fixed tree (lane partials -> wavefront shuffle -> LDS -> ordered sum over
 // the S partials), so results are run-to-run identical.
 #include "common.h"
+#include "storage.h"
 
 namespace {
 
@@ -20,29 +21,29 @@ struct BnShape {
   int stream;     // tensor too large to stay cache resident between kernels: non-temporal loads
 };
 
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-// Visit elements [lo, hi) of channel c's (n, hw) index space.  The 16-byte path loads four
-// float4 of x (and of dy when `dy` is not null) per thread before the first use, so that eight
-// loads are in flight per thread, and tracks (image, offset) incrementally instead of dividing.
-// f4(offset, x4, dy4) / f1(offset) do the arithmetic and any store.
-template <int NT, bool STREAM, class F4, class F1>
-__device__ __forceinline__ void channel_range_impl(const BnShape s, int c, int lo, int hi, const float *__restrict__ x,
-                                                   const float *__restrict__ dy, F4 f4, F1 f1) {
+// Visit elements [lo, hi) of channel c's (n, hw) index space.  S is the storage type (storage.h):
+// the 16-byte path loads four vectors of x (and of dy when `dy` is not null) per thread before the
+// first use, so that eight loads are in flight per thread, and tracks (image, offset) incrementally
+// instead of dividing.  fv(offset, x[VEC], dy[VEC]) / f1(offset) do the arithmetic and any store.
+template <int NT, bool STREAM, class S, class FV, class F1>
+__device__ __forceinline__ void channel_range_impl(const BnShape s, int c, int lo, int hi,
+                                                   const typename S::elem *__restrict__ x,
+                                                   const typename S::elem *__restrict__ dy, FV fv, F1 f1) {
+  constexpr int V = S::VEC;
   const int M = s.N * s.HW;
   if (hi > M) hi = M;
-  if ((s.HW & 3) == 0) {
-    // lo and per_split are multiples of 4 and a float4 never straddles an image boundary
+  if (s.HW % V == 0) {
+    // lo and per_split are multiples of V and a vector never straddles an image boundary
     constexpr int U = 4;
-    int i = lo + threadIdx.x * 4;
+    int i = lo + threadIdx.x * V;
     int n = i / s.HW, r = i - n * s.HW;
-    for (; i + (U - 1) * NT * 4 < hi; i += U * NT * 4) {
+    for (; i + (U - 1) * NT * V < hi; i += U * NT * V) {
       size_t off[U];
-      v4f xv[U], dv[U];
+      float xv[U][V], dv[U][V];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         off[u] = (size_t(n) * s.C + c) * s.HW + r;
-        r += NT * 4;
+        r += NT * V;
         while (r >= s.HW) {
           r -= s.HW;
           ++n;
@@ -50,24 +51,19 @@ __device__ __forceinline__ void channel_range_impl(const BnShape s, int c, int l
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        if (STREAM) {
-          xv[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(x + off[u]));
-          if (dy) dv[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(dy + off[u]));
-        } else {
-          xv[u] = *reinterpret_cast<const v4f *>(x + off[u]);
-          if (dy) dv[u] = *reinterpret_cast<const v4f *>(dy + off[u]);
-        }
+        S::template load16<STREAM>(x + off[u], xv[u]);
+        if (dy) S::template load16<STREAM>(dy + off[u], dv[u]);
       }
 #pragma unroll
-      for (int u = 0; u < U; ++u) f4(off[u], xv[u], dv[u]);
+      for (int u = 0; u < U; ++u) fv(off[u], xv[u], dv[u]);
     }
-    for (; i < hi; i += NT * 4) {
+    for (; i < hi; i += NT * V) {
       const size_t off = (size_t(n) * s.C + c) * s.HW + r;
-      v4f dv = {0.f, 0.f, 0.f, 0.f};
-      const v4f xv = *reinterpret_cast<const v4f *>(x + off);
-      if (dy) dv = *reinterpret_cast<const v4f *>(dy + off);
-      f4(off, xv, dv);
-      r += NT * 4;
+      float xv[V], dv[V];
+      S::template load16<false>(x + off, xv);
+      if (dy) S::template load16<false>(dy + off, dv);
+      fv(off, xv, dv);
+      r += NT * V;
       while (r >= s.HW) {
         r -= s.HW;
         ++n;
@@ -81,30 +77,34 @@ __device__ __forceinline__ void channel_range_impl(const BnShape s, int c, int l
   }
 }
 
-template <int NT, class F4, class F1>
-__device__ __forceinline__ void channel_range(const BnShape s, int c, int lo, int hi, const float *__restrict__ x,
-                                              const float *__restrict__ dy, F4 f4, F1 f1) {
-  if (s.stream) channel_range_impl<NT, true>(s, c, lo, hi, x, dy, f4, f1);
-  else channel_range_impl<NT, false>(s, c, lo, hi, x, dy, f4, f1);
+template <int NT, class S, class FV, class F1>
+__device__ __forceinline__ void channel_range(const BnShape s, int c, int lo, int hi, const typename S::elem *__restrict__ x,
+                                              const typename S::elem *__restrict__ dy, FV fv, F1 f1) {
+  if (s.stream) channel_range_impl<NT, true, S>(s, c, lo, hi, x, dy, fv, f1);
+  else channel_range_impl<NT, false, S>(s, c, lo, hi, x, dy, fv, f1);
 }
 
 // ---- forward, pass 1: per (c, split) partial sum and sum of squares about a pivot ---------
 // The pivot (the channel's first element) keeps the single-pass variance well conditioned.
-__global__ __launch_bounds__(kBlock) void k_bn_fwd_partial(const float *__restrict__ x, float *__restrict__ part,
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_bn_fwd_partial(const typename S::elem *__restrict__ x, float *__restrict__ part,
                                                           BnShape s) {
   __shared__ float red[16];
   const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
-  const float pivot = x[size_t(c) * s.HW];
+  const float pivot = S::ld(x + size_t(c) * s.HW);
   float a = 0.f, b = 0.f;
-  channel_range<kBlock>(
+  channel_range<kBlock, S>(
       s, c, sp * s.per_split, (sp + 1) * s.per_split, x, nullptr,
-      [&](size_t, v4f v, v4f) {
-        const float d0 = v[0] - pivot, d1 = v[1] - pivot, d2 = v[2] - pivot, d3 = v[3] - pivot;
-        a += (d0 + d1) + (d2 + d3);
-        b += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+      [&](size_t, const float *v, const float *) {
+#pragma unroll
+        for (int q = 0; q < S::VEC; q += 4) {
+          const float d0 = v[q] - pivot, d1 = v[q + 1] - pivot, d2 = v[q + 2] - pivot, d3 = v[q + 3] - pivot;
+          a += (d0 + d1) + (d2 + d3);
+          b += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+        }
       },
       [&](size_t off) {
-        const float d = x[off] - pivot;
+        const float d = S::ld(x + off) - pivot;
         a += d;
         b += d * d;
       });
@@ -117,12 +117,13 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_partial(const float *__restri
 }
 
 // ---- forward, pass 2: finish statistics (every workgroup redoes the tiny S-sum), normalise --
-__global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const float *__restrict__ x, const float *__restrict__ gamma,
-                                                        const float *__restrict__ beta, const float *__restrict__ part,
-                                                        float *__restrict__ running_mean, float *__restrict__ running_var,
-                                                        float factor, float eps, float *__restrict__ y,
-                                                        float *__restrict__ save_mean, float *__restrict__ save_invstd,
-                                                        BnShape s) {
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const typename S::elem *__restrict__ x,
+                                                        const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                        const float *__restrict__ part, float *__restrict__ running_mean,
+                                                        float *__restrict__ running_var, float factor, float eps,
+                                                        typename S::elem *__restrict__ y, float *__restrict__ save_mean,
+                                                        float *__restrict__ save_invstd, BnShape s) {
   const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
   const double M = double(s.N) * s.HW;
   double a = 0, b = 0;
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const float *__restrict
     a += part[(size_t(c) * s.S + i) * 2 + 0];
     b += part[(size_t(c) * s.S + i) * 2 + 1];
   }
-  const float pivot = x[size_t(c) * s.HW];
+  const float pivot = S::ld(x + size_t(c) * s.HW);
   const double dm = a / M;
   double var = b / M - dm * dm;
   if (var < 0) var = 0;
@@ -146,21 +147,21 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const float *__restrict
     }
   }
   const float g = gamma[c], be = beta[c];
-  channel_range<kBlock>(
+  channel_range<kBlock, S>(
       s, c, sp * s.per_split, (sp + 1) * s.per_split, x, nullptr,
-      [&](size_t off, v4f v, v4f) {
-        v4f r;
-        r[0] = g * ((v[0] - mean) * invstd) + be;
-        r[1] = g * ((v[1] - mean) * invstd) + be;
-        r[2] = g * ((v[2] - mean) * invstd) + be;
-        r[3] = g * ((v[3] - mean) * invstd) + be;
-        *reinterpret_cast<v4f *>(y + off) = r;
+      [&](size_t off, const float *v, const float *) {
+        float r[S::VEC];
+#pragma unroll
+        for (int q = 0; q < S::VEC; ++q) r[q] = g * ((v[q] - mean) * invstd) + be;
+        S::store16(y + off, r);
       },
-      [&](size_t off) { y[off] = g * ((x[off] - mean) * invstd) + be; });
+      [&](size_t off) { S::st(y + off, g * ((S::ld(x + off) - mean) * invstd) + be); });
 }
 
 // ---- backward, pass 1: partial sum(dy) and sum(dy * xhat) ---------------------------------
-__global__ __launch_bounds__(kBlock) void k_bn_bwd_partial(const float *__restrict__ dy, const float *__restrict__ x,
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_bn_bwd_partial(const typename S::elem *__restrict__ dy,
+                                                          const typename S::elem *__restrict__ x,
                                                           const float *__restrict__ save_mean,
                                                           const float *__restrict__ save_invstd,
                                                           float *__restrict__ part, BnShape s) {
@@ -168,17 +169,20 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_partial(const float *__restri
   const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
   const float mean = save_mean[c], invstd = save_invstd[c];
   float a = 0.f, b = 0.f;
-  channel_range<kBlock>(
+  channel_range<kBlock, S>(
       s, c, sp * s.per_split, (sp + 1) * s.per_split, x, dy,
-      [&](size_t, v4f v, v4f d) {
-        a += (d[0] + d[1]) + (d[2] + d[3]);
-        b += (d[0] * ((v[0] - mean) * invstd) + d[1] * ((v[1] - mean) * invstd)) +
-             (d[2] * ((v[2] - mean) * invstd) + d[3] * ((v[3] - mean) * invstd));
+      [&](size_t, const float *v, const float *d) {
+#pragma unroll
+        for (int q = 0; q < S::VEC; q += 4) {
+          a += (d[q] + d[q + 1]) + (d[q + 2] + d[q + 3]);
+          b += (d[q] * ((v[q] - mean) * invstd) + d[q + 1] * ((v[q + 1] - mean) * invstd)) +
+               (d[q + 2] * ((v[q + 2] - mean) * invstd) + d[q + 3] * ((v[q + 3] - mean) * invstd));
+        }
       },
       [&](size_t off) {
-        const float d = dy[off];
+        const float d = S::ld(dy + off);
         a += d;
-        b += d * ((x[off] - mean) * invstd);
+        b += d * ((S::ld(x + off) - mean) * invstd);
       });
   a = sgh_block_sum(a, red);
   b = sgh_block_sum(b, red);
@@ -189,11 +193,13 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_partial(const float *__restri
 }
 
 // ---- backward, pass 2: dx = k * (dy - (dbeta + xhat * dgamma) / M), k = gamma * invstd -----
-__global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const float *__restrict__ dy, const float *__restrict__ x,
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const typename S::elem *__restrict__ dy,
+                                                        const typename S::elem *__restrict__ x,
                                                         const float *__restrict__ gamma,
                                                         const float *__restrict__ save_mean,
                                                         const float *__restrict__ save_invstd,
-                                                        const float *__restrict__ part, float *__restrict__ dx,
+                                                        const float *__restrict__ part, typename S::elem *__restrict__ dx,
                                                         float *__restrict__ dgamma, float *__restrict__ dbeta,
                                                         BnShape s) {
   const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
@@ -211,27 +217,28 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const float *__restrict
   const float k = gamma[c] * invstd;
   const float rM = float(1.0 / (double(s.N) * s.HW));
   const float c0 = db * rM, c1 = dg * rM;
-  channel_range<kBlock>(
+  channel_range<kBlock, S>(
       s, c, sp * s.per_split, (sp + 1) * s.per_split, x, dy,
-      [&](size_t off, v4f v, v4f d) {
-        v4f r;
-        r[0] = k * (d[0] - (c0 + ((v[0] - mean) * invstd) * c1));
-        r[1] = k * (d[1] - (c0 + ((v[1] - mean) * invstd) * c1));
-        r[2] = k * (d[2] - (c0 + ((v[2] - mean) * invstd) * c1));
-        r[3] = k * (d[3] - (c0 + ((v[3] - mean) * invstd) * c1));
-        *reinterpret_cast<v4f *>(dx + off) = r;
+      [&](size_t off, const float *v, const float *d) {
+        float r[S::VEC];
+#pragma unroll
+        for (int q = 0; q < S::VEC; ++q) r[q] = k * (d[q] - (c0 + ((v[q] - mean) * invstd) * c1));
+        S::store16(dx + off, r);
       },
-      [&](size_t off) { dx[off] = k * (dy[off] - (c0 + ((x[off] - mean) * invstd) * c1)); });
+      [&](size_t off) {
+        S::st(dx + off, k * (S::ld(dy + off) - (c0 + ((S::ld(x + off) - mean) * invstd) * c1)));
+      });
 }
 
 inline bool shape_ok(int N, int C, int HW) {
   return N > 0 && C > 0 && HW > 0 && size_t(N) * HW < 0x7fffffffu;
 }
 
-inline BnShape make_shape(int N, int C, int HW) {
+// `vec`: elements per 16-byte access of the storage type; `esize`: bytes per element
+inline BnShape make_shape(int N, int C, int HW, int vec, int esize) {
   // (measured: non-temporal loads gain 20 % on the 205 MB stem tensors and lose a few per cent on
   // tensors the previous kernel left in the 256 MB Infinity Cache)
-  BnShape s{N, C, HW, 1, 0, size_t(N) * C * HW * sizeof(float) >= (size_t(96) << 20) ? 1 : 0};
+  BnShape s{N, C, HW, 1, 0, size_t(N) * C * HW * esize >= (size_t(96) << 20) ? 1 : 0};
   const long M = long(N) * HW;
   // aim at ~8 workgroups per CU in total, at least 2048 elements per workgroup
   long want = (long(sgh_num_cus()) * 8 + C - 1) / C;
@@ -240,11 +247,47 @@ inline BnShape make_shape(int N, int C, int HW) {
   if (S < 1) S = 1;
   if (S > 1024) S = 1024;
   long per = (M + S - 1) / S;
-  per = (per + 3) & ~3L;
+  per = (per + vec - 1) / vec * vec;
   S = (M + per - 1) / per;
   s.S = int(S);
   s.per_split = int(per);
   return s;
+}
+
+template <class S>
+int bn_fwd_train(const typename S::elem *x, const float *gamma, const float *beta, float *running_mean,
+                 float *running_var, float factor, float eps, typename S::elem *y, float *save_mean, float *save_invstd,
+                 int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  if (!shape_ok(N, C, HW) || !x || !gamma || !beta || !y || !save_mean || !save_invstd) return SGH_EINVAL;
+  const BnShape s = make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem)));
+  if (!sgh_aligned16(x) || !sgh_aligned16(y)) return SGH_EINVAL;
+  if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
+  float *scratch = static_cast<float *>(workspace);
+  hipLaunchKernelGGL(k_bn_fwd_partial<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, scratch, s);
+  SGH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_bn_fwd_apply<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, gamma, beta, scratch,
+                     running_mean, running_var, factor, eps, y, save_mean, save_invstd, s);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+template <class S>
+int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *gamma, const float *save_mean,
+           const float *save_invstd, typename S::elem *dx, float *dgamma, float *dbeta, int N, int C, int HW,
+           void *workspace, size_t ws_bytes, void *stream) {
+  if (!shape_ok(N, C, HW) || !dy || !x || !gamma || !save_mean || !save_invstd || !dx || !dgamma || !dbeta)
+    return SGH_EINVAL;
+  if (!sgh_aligned16(x) || !sgh_aligned16(dy) || !sgh_aligned16(dx)) return SGH_EINVAL;
+  const BnShape s = make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem)));
+  if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
+  float *part = static_cast<float *>(workspace);
+  hipLaunchKernelGGL(k_bn_bwd_partial<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, save_mean,
+                     save_invstd, part, s);
+  SGH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_bn_bwd_apply<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, gamma, save_mean,
+                     save_invstd, part, dx, dgamma, dbeta, s);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
 }
 
 }  // namespace
@@ -253,42 +296,44 @@ extern "C" {
 
 size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
   if (!shape_ok(N, C, HW)) return 0;
-  const BnShape s = make_shape(N, C, HW);
-  return size_t(C) * s.S * 2 * sizeof(float);
+  // one size for every storage type: the larger of the fp32 and the 16-bit split counts
+  const int s4 = make_shape(N, C, HW, 4, 4).S, s8 = make_shape(N, C, HW, 8, 2).S;
+  return size_t(C) * (s4 > s8 ? s4 : s8) * 2 * sizeof(float);
 }
 
 int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float *beta, float *running_mean,
                          float *running_var, float factor, float eps, float *y, float *save_mean, float *save_invstd,
                          int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
-  if (!shape_ok(N, C, HW) || !x || !gamma || !beta || !y || !save_mean || !save_invstd) return SGH_EINVAL;
-  const BnShape s = make_shape(N, C, HW);
-  if (!sgh_aligned16(x) || !sgh_aligned16(y)) return SGH_EINVAL;
-  if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
-  float *scratch = static_cast<float *>(workspace);
-  hipLaunchKernelGGL(k_bn_fwd_partial, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, scratch, s);
-  SGH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_bn_fwd_apply, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, gamma, beta, scratch,
-                     running_mean, running_var, factor, eps, y, save_mean, save_invstd, s);
-  SGH_LAUNCH_CHECK();
-  return SGH_OK;
+  return bn_fwd_train<StF32>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C, HW,
+                             workspace, ws_bytes, stream);
+}
+int sgh_bn_fwd_train_f16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
+                         float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
+                         float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  return bn_fwd_train<StF16>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C, HW,
+                             workspace, ws_bytes, stream);
+}
+int sgh_bn_fwd_train_bf16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
+                          float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
+                          float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  return bn_fwd_train<StBF16>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C,
+                              HW, workspace, ws_bytes, stream);
 }
 
 int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const float *save_mean,
                    const float *save_invstd, float *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                    void *workspace, size_t ws_bytes, void *stream) {
-  if (!shape_ok(N, C, HW) || !dy || !x || !gamma || !save_mean || !save_invstd || !dx || !dgamma || !dbeta)
-    return SGH_EINVAL;
-  if (!sgh_aligned16(x) || !sgh_aligned16(dy) || !sgh_aligned16(dx)) return SGH_EINVAL;
-  const BnShape s = make_shape(N, C, HW);
-  if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
-  float *part = static_cast<float *>(workspace);
-  hipLaunchKernelGGL(k_bn_bwd_partial, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, save_mean,
-                     save_invstd, part, s);
-  SGH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_bn_bwd_apply, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, gamma, save_mean,
-                     save_invstd, part, dx, dgamma, dbeta, s);
-  SGH_LAUNCH_CHECK();
-  return SGH_OK;
+  return bn_bwd<StF32>(dy, x, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes, stream);
+}
+int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
+                   const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
+                   void *workspace, size_t ws_bytes, void *stream) {
+  return bn_bwd<StF16>(dy, x, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes, stream);
+}
+int sgh_bn_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
+                    const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
+                    void *workspace, size_t ws_bytes, void *stream) {
+  return bn_bwd<StBF16>(dy, x, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes, stream);
 }
 
 }  // extern "C"

@@ -7,6 +7,7 @@
 // Each thread moves 16 bytes (8 elements) per access; a workgroup streams contiguous 16 KB
 // chunks, as in the fp32 kernels.
 #include "common.h"
+#include "storage.h"
 
 namespace {
 
@@ -17,30 +18,14 @@ typedef unsigned short u16;
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 struct F16 {
-  static __device__ __forceinline__ float load(u16 b) {
-    _Float16 h;
-    __builtin_memcpy(&h, &b, 2);
-    return float(h);
-  }
-  static __device__ __forceinline__ u16 store(float f) {
-    const _Float16 h = _Float16(f);  // v_cvt_f16_f32: round to nearest even
-    u16 b;
-    __builtin_memcpy(&b, &h, 2);
-    return b;
-  }
+  static __device__ __forceinline__ float load(u16 b) { return sgh_f16_to_f32(b); }
+  static __device__ __forceinline__ u16 store(float f) { return sgh_f32_to_f16(f); }
 };
 
 struct BF16 {
-  static __device__ __forceinline__ float load(u16 b) { return __builtin_bit_cast(float, unsigned(b) << 16); }
-  static __device__ __forceinline__ u16 store(float f) {
-    unsigned u = __builtin_bit_cast(unsigned, f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return u16((u >> 16) | 0x40u);  // NaN stays a (quiet) NaN
-    u += 0x7fffu + ((u >> 16) & 1u);                                      // round to nearest even
-    return u16(u >> 16);
-  }
+  static __device__ __forceinline__ float load(u16 b) { return sgh_bf16_to_f32(b); }
+  static __device__ __forceinline__ u16 store(float f) { return sgh_f32_to_bf16(f); }
 };
-
-struct F32 {};  // marker for the fp32 side of a cast
 
 inline int grid_for(size_t nvec) {
   size_t per_block = size_t(kBlock) * kUnroll;

@@ -1,0 +1,78 @@
+// Storage types of the bandwidth-bound kernels.  Arithmetic is always fp32; a storage type says
+// how 16 bytes of a tensor turn into floats and back: fp32 (4 elements), IEEE binary16 and
+// bfloat16 (8 elements, carried as uint16_t).  Stores round to nearest, ties to even.
+#ifndef SINGA_AMD_CSRC_STORAGE_H_
+#define SINGA_AMD_CSRC_STORAGE_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef float sgh_v4f __attribute__((ext_vector_type(4)));
+typedef unsigned int sgh_v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float sgh_f16_to_f32(uint16_t b) {
+  _Float16 h;
+  __builtin_memcpy(&h, &b, 2);
+  return float(h);
+}
+__device__ __forceinline__ uint16_t sgh_f32_to_f16(float f) {
+  const _Float16 h = _Float16(f);  // v_cvt_f16_f32: round to nearest even
+  uint16_t b;
+  __builtin_memcpy(&b, &h, 2);
+  return b;
+}
+__device__ __forceinline__ float sgh_bf16_to_f32(uint16_t b) { return __builtin_bit_cast(float, unsigned(b) << 16); }
+__device__ __forceinline__ uint16_t sgh_f32_to_bf16(float f) {
+  unsigned u = __builtin_bit_cast(unsigned, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40u);  // NaN stays a (quiet) NaN
+  u += 0x7fffu + ((u >> 16) & 1u);                                          // round to nearest even
+  return uint16_t(u >> 16);
+}
+
+struct StF32 {
+  typedef float elem;
+  static constexpr int VEC = 4;
+  static __device__ __forceinline__ float ld(const elem *p) { return *p; }
+  static __device__ __forceinline__ void st(elem *p, float v) { *p = v; }
+  template <bool NT>
+  static __device__ __forceinline__ void load16(const elem *p, float *out) {
+    const sgh_v4f v = NT ? __builtin_nontemporal_load(reinterpret_cast<const sgh_v4f *>(p))
+                         : *reinterpret_cast<const sgh_v4f *>(p);
+    out[0] = v[0];
+    out[1] = v[1];
+    out[2] = v[2];
+    out[3] = v[3];
+  }
+  static __device__ __forceinline__ void store16(elem *p, const float *in) {
+    *reinterpret_cast<sgh_v4f *>(p) = sgh_v4f{in[0], in[1], in[2], in[3]};
+  }
+};
+
+template <float (*LD)(uint16_t), uint16_t (*ST)(float)>
+struct St16 {
+  typedef uint16_t elem;
+  static constexpr int VEC = 8;
+  static __device__ __forceinline__ float ld(const elem *p) { return LD(*p); }
+  static __device__ __forceinline__ void st(elem *p, float v) { *p = ST(v); }
+  template <bool NT>
+  static __device__ __forceinline__ void load16(const elem *p, float *out) {
+    const sgh_v4u v = NT ? __builtin_nontemporal_load(reinterpret_cast<const sgh_v4u *>(p))
+                         : *reinterpret_cast<const sgh_v4u *>(p);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      out[2 * j] = LD(uint16_t(v[j] & 0xffffu));
+      out[2 * j + 1] = LD(uint16_t(v[j] >> 16));
+    }
+  }
+  static __device__ __forceinline__ void store16(elem *p, const float *in) {
+    sgh_v4u r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = unsigned(ST(in[2 * j])) | (unsigned(ST(in[2 * j + 1])) << 16);
+    *reinterpret_cast<sgh_v4u *>(p) = r;
+  }
+};
+
+typedef St16<sgh_f16_to_f32, sgh_f32_to_f16> StF16;
+typedef St16<sgh_bf16_to_f32, sgh_f32_to_bf16> StBF16;
+
+#endif  // SINGA_AMD_CSRC_STORAGE_H_

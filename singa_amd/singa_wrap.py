@@ -567,12 +567,12 @@ def GpuBatchNormForwardTraining(h, x, scale, bias, running_mean, running_var):
     y = _like(x)
     mean = Tensor((h.channels,), x.device(), kFloat32)
     var = Tensor((h.channels,), x.device(), kFloat32)
-    check(_L().sgh_bn_fwd_train_f32(x.ptr, scale.ptr, bias.ptr,
-                                    running_mean.ptr if running_mean is not None else None,
-                                    running_var.ptr if running_var is not None else None,
-                                    h.factor, _BN_EPS, y.ptr, mean.ptr, var.ptr, h.batchsize, h.channels,
-                                    h.height * h.width, h.workspace.ptr, h.workspace.MemSize(),
-                                    x.device().stream), "sgh_bn_fwd_train_f32")
+    fn, name = _fn("bn_fwd_train", x)  # 16-bit activations keep fp32 scale / bias / statistics
+    check(fn(x.ptr, scale.ptr, bias.ptr,
+             running_mean.ptr if running_mean is not None else None,
+             running_var.ptr if running_var is not None else None,
+             h.factor, _BN_EPS, y.ptr, mean.ptr, var.ptr, h.batchsize, h.channels,
+             h.height * h.width, h.workspace.ptr, h.workspace.MemSize(), x.device().stream), name)
     return [y, mean, var]
 
 
@@ -582,9 +582,10 @@ def GpuBatchNormBackward(h, dy, x, scale, mean, var):
     dx = _like(dy)
     ds = _like(scale)
     db = _like(scale)
-    check(_L().sgh_bn_bwd_f32(dy.ptr, x.ptr, scale.ptr, mean.ptr, var.ptr, dx.ptr, ds.ptr, db.ptr,
-                              h.batchsize, h.channels, h.height * h.width, h.workspace.ptr,
-                              h.workspace.MemSize(), dy.device().stream), "sgh_bn_bwd_f32")
+    fn, name = _fn("bn_bwd", dy)
+    check(fn(dy.ptr, x.ptr, scale.ptr, mean.ptr, var.ptr, dx.ptr, ds.ptr, db.ptr,
+             h.batchsize, h.channels, h.height * h.width, h.workspace.ptr,
+             h.workspace.MemSize(), dy.device().stream), name)
     return [dx, ds, db]
 
 

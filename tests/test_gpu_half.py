@@ -88,3 +88,33 @@ def test_relu_backward_add_mult_axpy(singa, dev, kind, n):
     bt, b = _to(singa, dev, r.standard_normal(n).astype(np.float32), kind)
     at += bt
     _same_bits(at.to_numpy(), _round(singa, a + b, kind), "iadd " + kind)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 28, 28), (16, 32, 8, 8), (3, 7, 4, 2)])
+def test_batchnorm_16bit_storage(singa, dev, kind, shape):
+    """BN forward-training / backward on 16-bit activations with fp32 parameters and statistics:
+    the fp32 CPU oracle on the same (already rounded) inputs, outputs compared at the 16-bit
+    tolerance of 1e-2 normalised L2; statistics and parameter gradients stay fp32 (1e-3)."""
+    from oracle import cpu_oracle as O
+    from util import nl2
+    r = rng(sum(shape))
+    N, C, H, W = shape
+    xt, x = _to(singa, dev, (r.standard_normal(shape) * 2 + 0.5).astype(np.float32), kind)
+    dyt, dy = _to(singa, dev, r.standard_normal(shape).astype(np.float32), kind)
+    gamma = (1 + 0.1 * r.standard_normal(C)).astype(np.float32)
+    beta = (0.1 * r.standard_normal(C)).astype(np.float32)
+    h = singa.CudnnBatchNormHandle(0.9, xt)
+    gd, bd = singa.from_numpy(gamma, dev), singa.from_numpy(beta, dev)
+    rm, rv = singa.from_numpy(np.zeros(C, np.float32), dev), singa.from_numpy(np.ones(C, np.float32), dev)
+    y, mean, var = singa.GpuBatchNormForwardTraining(h, xt, gd, bd, rm, rv)
+    assert y.data_type() == xt.data_type() and mean.data_type() == singa.kFloat32
+    y_o, mean_o, invstd_o = O.bn_fwd_train(x, gamma, beta, np.zeros(C, np.float32), np.ones(C, np.float32), 0.9, 1e-5)
+    assert nl2(y.to_numpy(), y_o) < 1e-2
+    np.testing.assert_allclose(mean.to_numpy(), mean_o, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(var.to_numpy(), invstd_o, rtol=1e-4)
+    dx, ds, db = singa.GpuBatchNormBackward(h, dyt, xt, gd, mean, var)
+    dx_o, ds_o, db_o = O.bn_bwd(dy, x, gamma, mean_o, invstd_o)
+    assert dx.data_type() == xt.data_type()
+    assert nl2(dx.to_numpy(), dx_o) < 1e-2
+    assert nl2(ds.to_numpy(), ds_o) < 1e-3 and nl2(db.to_numpy(), db_o) < 1e-3
