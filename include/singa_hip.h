@@ -309,6 +309,14 @@ SGH_API int sgh_pool_fwd_f32(const sgh_pool_geom *g, const float *x, float *y, v
  * the result is bit-identical to the CPU loop.  Avg: dy / |clipped window| spread over the window. */
 SGH_API int sgh_pool_bwd_f32(const sgh_pool_geom *g, const float *dy, const float *x,
                              const float *y, float *dx, void *stream);
+/* Pooling on 16-bit tensors: comparisons and sums in fp32 (conversion keeps order, so the routing
+ * of the max gradient is that of the stored values), one rounding on store. */
+SGH_API int sgh_pool_fwd_f16(const sgh_pool_geom *g, const uint16_t *x, uint16_t *y, void *stream);
+SGH_API int sgh_pool_fwd_bf16(const sgh_pool_geom *g, const uint16_t *x, uint16_t *y, void *stream);
+SGH_API int sgh_pool_bwd_f16(const sgh_pool_geom *g, const uint16_t *dy, const uint16_t *x,
+                             const uint16_t *y, uint16_t *dx, void *stream);
+SGH_API int sgh_pool_bwd_bf16(const sgh_pool_geom *g, const uint16_t *dy, const uint16_t *x,
+                              const uint16_t *y, uint16_t *dx, void *stream);
 
 #ifdef __cplusplus
 }

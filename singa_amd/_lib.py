@@ -106,6 +106,10 @@ SIGNATURES = {
     "sgh_pool_geom_init": (C.c_int, [C.POINTER(PoolGeom)] + [C.c_int] * 11),
     "sgh_pool_fwd_f32": (C.c_int, [C.POINTER(PoolGeom), vp, vp, vp]),
     "sgh_pool_bwd_f32": (C.c_int, [C.POINTER(PoolGeom), vp, vp, vp, vp, vp]),
+    "sgh_pool_fwd_f16": (C.c_int, [C.POINTER(PoolGeom), vp, vp, vp]),
+    "sgh_pool_fwd_bf16": (C.c_int, [C.POINTER(PoolGeom), vp, vp, vp]),
+    "sgh_pool_bwd_f16": (C.c_int, [C.POINTER(PoolGeom), vp, vp, vp, vp, vp]),
+    "sgh_pool_bwd_bf16": (C.c_int, [C.POINTER(PoolGeom), vp, vp, vp, vp, vp]),
 }
 
 SGH_CONV_FWD, SGH_CONV_DGRAD, SGH_CONV_WGRAD = 0, 1, 2

@@ -6,6 +6,7 @@
 // own element.  The additions therefore happen in exactly the order of the CPU scatter loop, so
 // dx is bit-identical to it and no atomics are needed.
 #include "common.h"
+#include "storage.h"
 
 namespace {
 
@@ -16,7 +17,9 @@ struct PoolG {
 };
 
 // flat index (h * W + w) of the first maximum of window (p, q) in plane `b`; -1 if empty
-__device__ __forceinline__ int window_argmax(const float *__restrict__ b, const PoolG g, int p, int q, float *best_out) {
+template <class S>
+__device__ __forceinline__ int window_argmax(const typename S::elem *__restrict__ b, const PoolG g, int p, int q,
+                                             float *best_out) {
   int hs = p * g.sh - g.ph, ws = q * g.sw - g.pw;
   const int he = min(hs + g.kh, g.H), we = min(ws + g.kw, g.W);
   hs = max(hs, 0);
@@ -25,7 +28,7 @@ __device__ __forceinline__ int window_argmax(const float *__restrict__ b, const 
   int bi = -1;
   for (int h = hs; h < he; ++h)
     for (int w = ws; w < we; ++w) {
-      const float v = b[h * g.W + w];
+      const float v = S::ld(b + h * g.W + w);
       if (v > best) {
         best = v;
         bi = h * g.W + w;
@@ -35,29 +38,32 @@ __device__ __forceinline__ int window_argmax(const float *__restrict__ b, const 
   return bi;
 }
 
-__global__ __launch_bounds__(kBlock) void k_pool_max_fwd(const float *__restrict__ x, float *__restrict__ y, PoolG g,
-                                                        size_t total) {
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_pool_max_fwd(const typename S::elem *__restrict__ x,
+                                                        typename S::elem *__restrict__ y, PoolG g, size_t total) {
   const size_t stride = size_t(gridDim.x) * kBlock;
   const int PQ = g.P * g.Q;
   for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
     const size_t plane = i / PQ;
     const int r = int(i - plane * PQ);
     float best;
-    window_argmax(x + plane * size_t(g.H) * g.W, g, r / g.Q, r % g.Q, &best);
-    y[i] = best;
+    window_argmax<S>(x + plane * size_t(g.H) * g.W, g, r / g.Q, r % g.Q, &best);
+    S::st(y + i, best);
   }
 }
 
-__global__ __launch_bounds__(kBlock) void k_pool_max_bwd(const float *__restrict__ dy, const float *__restrict__ x,
-                                                        float *__restrict__ dx, PoolG g, size_t total) {
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_pool_max_bwd(const typename S::elem *__restrict__ dy,
+                                                        const typename S::elem *__restrict__ x,
+                                                        typename S::elem *__restrict__ dx, PoolG g, size_t total) {
   const size_t stride = size_t(gridDim.x) * kBlock;
   const int HW = g.H * g.W, PQ = g.P * g.Q;
   for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
     const size_t plane = i / HW;
     const int r = int(i - plane * HW);
     const int h = r / g.W, w = r - h * g.W;
-    const float *xb = x + plane * size_t(HW);
-    const float *db = dy + plane * size_t(PQ);
+    const typename S::elem *xb = x + plane * size_t(HW);
+    const typename S::elem *db = dy + plane * size_t(PQ);
     // windows p with p*sh - ph <= h < p*sh - ph + kh
     const int hp = h + g.ph, wp = w + g.pw;
     const int p_lo = hp < g.kh ? 0 : (hp - g.kh) / g.sh + 1;
@@ -67,8 +73,8 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd(const float *__restrict
     float s = 0.f;
     for (int p = p_lo; p <= p_hi; ++p)
       for (int q = q_lo; q <= q_hi; ++q)
-        if (window_argmax(xb, g, p, q, nullptr) == r) s += db[p * g.Q + q];
-    dx[i] = s;
+        if (window_argmax<S>(xb, g, p, q, nullptr) == r) s += S::ld(db + p * g.Q + q);
+    S::st(dx + i, s);
   }
 }
 
@@ -84,10 +90,11 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd(const float *__restrict
 // KH/KW/SH/SW > 0 fix the window at compile time: the scans are then fully unrolled, every LDS
 // read of a window or of a dx element is issued before the first compare, and out-of-range
 // positions are predicated instead of branched over.  0 = read the geometry at run time.
-template <int KH, int KW, int SH, int SW>
-__global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__restrict__ dy, const float *__restrict__ x,
-                                                              float *__restrict__ dx, PoolG g, int TH, int bands,
-                                                              int max_xrows, int max_np) {
+template <int KH, int KW, int SH, int SW, class S>
+__global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const typename S::elem *__restrict__ dy,
+                                                              const typename S::elem *__restrict__ x,
+                                                              typename S::elem *__restrict__ dx, PoolG g, int TH,
+                                                              int bands, int max_xrows, int max_np) {
   if (KH > 0) {
     g.kh = KH;
     g.kw = KW;
@@ -108,19 +115,24 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__re
   const int p_hi = min((h1 - 1 + g.ph) / g.sh, g.P - 1);
   const int np = p_hi - p_lo + 1;
   const int xr0 = max(p_lo * g.sh - g.ph, 0), xr1 = min(p_hi * g.sh - g.ph + g.kh, g.H);  // x rows [xr0, xr1)
-  const float *xb = x + size_t(plane) * g.H * g.W + xr0 * g.W;
-  const float *db = dy + size_t(plane) * g.P * g.Q + p_lo * g.Q;
-  float *ob = dx + size_t(plane) * g.H * g.W;
+  const typename S::elem *xb = x + size_t(plane) * g.H * g.W + xr0 * g.W;
+  const typename S::elem *db = dy + size_t(plane) * g.P * g.Q + p_lo * g.Q;
+  typename S::elem *ob = dx + size_t(plane) * g.H * g.W;
   const int nx = (xr1 - xr0) * g.W, nd = np > 0 ? np * g.Q : 0;
-  if (((reinterpret_cast<uintptr_t>(xb) | reinterpret_cast<uintptr_t>(xs)) & 15u) == 0 && (nx & 3) == 0) {
-    const float4 *s4 = reinterpret_cast<const float4 *>(xb);
-    float4 *d4 = reinterpret_cast<float4 *>(xs);
+  // 16 bytes of the storage type per access when the run is aligned (LDS holds floats)
+  constexpr int V = S::VEC;
+  if ((reinterpret_cast<uintptr_t>(xb) & 15u) == 0 && nx % V == 0) {
 #pragma unroll 4
-    for (int i = threadIdx.x; i < (nx >> 2); i += kBlock) d4[i] = s4[i];
+    for (int i = threadIdx.x; i < nx / V; i += kBlock) {
+      float v[V];
+      S::template load16<false>(xb + i * V, v);
+#pragma unroll
+      for (int j = 0; j < V; ++j) xs[i * V + j] = v[j];
+    }
   } else {
-    for (int i = threadIdx.x; i < nx; i += kBlock) xs[i] = xb[i];
+    for (int i = threadIdx.x; i < nx; i += kBlock) xs[i] = S::ld(xb + i);
   }
-  for (int i = threadIdx.x; i < nd; i += kBlock) ds[i] = db[i];
+  for (int i = threadIdx.x; i < nd; i += kBlock) ds[i] = S::ld(db + i);
   for (int i = threadIdx.x; i < h1 - h0; i += kBlock) {
     const int hp = h0 + i + g.ph;
     prange[2 * i] = (hp < g.kh ? 0 : (hp - g.kh) / g.sh + 1) - p_lo;
@@ -208,14 +220,14 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__re
             for (int i = 0; i < NBH * NBW; ++i) s += wi[i] == r ? dv[i] : 0.f;
             out[b2] = s;
           }
-          float *o = ob + h * g.W + w0;
-          if (SWc == 2 && w0 + 1 < g.W && (reinterpret_cast<uintptr_t>(o) & 7u) == 0) {
+          typename S::elem *o = ob + h * g.W + w0;
+          if (V == 4 && SWc == 2 && w0 + 1 < g.W && (reinterpret_cast<uintptr_t>(o) & 7u) == 0) {
             typedef float v2f __attribute__((ext_vector_type(2)));
             *reinterpret_cast<v2f *>(o) = v2f{out[0], out[SWc - 1]};
           } else {
 #pragma unroll
             for (int b2 = 0; b2 < SWc; ++b2)
-              if (w0 + b2 < g.W) o[b2] = out[b2];
+              if (w0 + b2 < g.W) S::st(o + b2, out[b2]);
           }
         }
       }
@@ -232,7 +244,7 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const float *__re
         for (int p = pl; p <= ph_; ++p)
           for (int q = ql; q <= qh; ++q)
             if (widx[p * g.Q + q] == r) s += ds[p * g.Q + q];
-        ob[r] = s;
+        S::st(ob + r, s);
       }
     }
   }
@@ -250,32 +262,34 @@ __device__ __forceinline__ int window_count(const PoolG g, int p, int q, int *hs
   return (he - hs) * (we - ws);  // count-exclude-padding
 }
 
-__global__ __launch_bounds__(kBlock) void k_pool_avg_fwd(const float *__restrict__ x, float *__restrict__ y, PoolG g,
-                                                        size_t total) {
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_pool_avg_fwd(const typename S::elem *__restrict__ x,
+                                                        typename S::elem *__restrict__ y, PoolG g, size_t total) {
   const size_t stride = size_t(gridDim.x) * kBlock;
   const int PQ = g.P * g.Q;
   for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
     const size_t plane = i / PQ;
     const int r = int(i - plane * PQ);
-    const float *b = x + plane * size_t(g.H) * g.W;
+    const typename S::elem *b = x + plane * size_t(g.H) * g.W;
     int hs, he, ws, we;
     const int cnt = window_count(g, r / g.Q, r % g.Q, &hs, &he, &ws, &we);
     float s = 0.f;
     for (int h = hs; h < he; ++h)
-      for (int w = ws; w < we; ++w) s += b[h * g.W + w];
-    y[i] = s / float(cnt);
+      for (int w = ws; w < we; ++w) s += S::ld(b + h * g.W + w);
+    S::st(y + i, s / float(cnt));
   }
 }
 
-__global__ __launch_bounds__(kBlock) void k_pool_avg_bwd(const float *__restrict__ dy, float *__restrict__ dx, PoolG g,
-                                                        size_t total) {
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_pool_avg_bwd(const typename S::elem *__restrict__ dy,
+                                                        typename S::elem *__restrict__ dx, PoolG g, size_t total) {
   const size_t stride = size_t(gridDim.x) * kBlock;
   const int HW = g.H * g.W, PQ = g.P * g.Q;
   for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
     const size_t plane = i / HW;
     const int r = int(i - plane * HW);
     const int h = r / g.W, w = r - h * g.W;
-    const float *db = dy + plane * size_t(PQ);
+    const typename S::elem *db = dy + plane * size_t(PQ);
     const int hp = h + g.ph, wp = w + g.pw;
     const int p_lo = hp < g.kh ? 0 : (hp - g.kh) / g.sh + 1;
     const int p_hi = min(hp / g.sh, g.P - 1);
@@ -286,9 +300,9 @@ __global__ __launch_bounds__(kBlock) void k_pool_avg_bwd(const float *__restrict
       for (int q = q_lo; q <= q_hi; ++q) {
         int hs, he, ws, we;
         const int cnt = window_count(g, p, q, &hs, &he, &ws, &we);
-        s += db[p * g.Q + q] / float(cnt);
+        s += S::ld(db + p * g.Q + q) / float(cnt);
       }
-    dx[i] = s;
+    S::st(dx + i, s);
   }
 }
 
@@ -311,6 +325,61 @@ inline bool geom_ok(const sgh_pool_geom *g) {
          // every window must overlap the image, else a max window would be empty
          g->pad_h < g->kernel_h && g->pad_w < g->kernel_w &&
          size_t(g->H) * g->W < 0x7fffffffu;
+}
+
+template <class S>
+int pool_fwd(const sgh_pool_geom *g, const typename S::elem *x, typename S::elem *y, void *stream) {
+  if (!geom_ok(g) || !x || !y) return SGH_EINVAL;
+  const size_t total = size_t(g->N) * g->C * g->P * g->Q;
+  if (g->is_max)
+    hipLaunchKernelGGL(k_pool_max_fwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), x, y, to_g(g),
+                       total);
+  else
+    hipLaunchKernelGGL(k_pool_avg_fwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), x, y, to_g(g),
+                       total);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+template <class S>
+int pool_bwd(const sgh_pool_geom *g, const typename S::elem *dy, const typename S::elem *x, const typename S::elem *y,
+             typename S::elem *dx, void *stream) {
+  (void)y;
+  if (!geom_ok(g) || !dy || !dx) return SGH_EINVAL;
+  if (g->is_max && !x) return SGH_EINVAL;
+  const size_t total = size_t(g->N) * g->C * g->H * g->W;
+  if (g->is_max) {
+    // band height: about 12 KB of x rows per workgroup (measured optimum: enough workgroups per CU to
+    // overlap one's staging with another's scans), bands of equal height
+    int TH = 3072 / g->W - g->kernel_h;
+    if (TH < 1) TH = 1;
+    if (TH > g->H) TH = g->H;
+    int bands = (g->H + TH - 1) / TH;
+    TH = (g->H + bands - 1) / bands;
+    bands = (g->H + TH - 1) / TH;
+    const int max_np = (TH + g->kernel_h - 2) / g->stride_h + 2;
+    const int max_xrows = (max_np - 1) * g->stride_h + g->kernel_h;
+    const size_t lds = (size_t(max_xrows) * g->W + size_t(2) * max_np * g->Q + size_t(2) * TH) * sizeof(float);
+    const size_t blocks = size_t(g->N) * g->C * bands;
+    if (lds <= 48 * 1024 && blocks < 0x7fffffffu && g->W <= 2048) {
+      auto kern = k_pool_max_bwd_tiled<0, 0, 0, 0, S>;
+      if (g->kernel_h == 3 && g->kernel_w == 3 && g->stride_h == 2 && g->stride_w == 2)
+        kern = k_pool_max_bwd_tiled<3, 3, 2, 2, S>;
+      else if (g->kernel_h == 2 && g->kernel_w == 2 && g->stride_h == 2 && g->stride_w == 2)
+        kern = k_pool_max_bwd_tiled<2, 2, 2, 2, S>;
+      else if (g->kernel_h == 3 && g->kernel_w == 3 && g->stride_h == 1 && g->stride_w == 1)
+        kern = k_pool_max_bwd_tiled<3, 3, 1, 1, S>;
+      hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBlock), lds, sgh_stream_of(stream), dy, x, dx, to_g(g), TH,
+                         bands, max_xrows, max_np);
+    } else {
+      hipLaunchKernelGGL(k_pool_max_bwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
+                         to_g(g), total);
+    }
+  } else
+    hipLaunchKernelGGL(k_pool_avg_bwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, dx, to_g(g),
+                       total);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
 }
 
 }  // namespace
@@ -342,56 +411,25 @@ int sgh_pool_geom_init(sgh_pool_geom *g, int N, int C, int H, int W, int kernel_
 }
 
 int sgh_pool_fwd_f32(const sgh_pool_geom *g, const float *x, float *y, void *stream) {
-  if (!geom_ok(g) || !x || !y) return SGH_EINVAL;
-  const size_t total = size_t(g->N) * g->C * g->P * g->Q;
-  if (g->is_max)
-    hipLaunchKernelGGL(k_pool_max_fwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), x, y, to_g(g),
-                       total);
-  else
-    hipLaunchKernelGGL(k_pool_avg_fwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), x, y, to_g(g),
-                       total);
-  SGH_LAUNCH_CHECK();
-  return SGH_OK;
+  return pool_fwd<StF32>(g, x, y, stream);
 }
-
+int sgh_pool_fwd_f16(const sgh_pool_geom *g, const uint16_t *x, uint16_t *y, void *stream) {
+  return pool_fwd<StF16>(g, x, y, stream);
+}
+int sgh_pool_fwd_bf16(const sgh_pool_geom *g, const uint16_t *x, uint16_t *y, void *stream) {
+  return pool_fwd<StBF16>(g, x, y, stream);
+}
 int sgh_pool_bwd_f32(const sgh_pool_geom *g, const float *dy, const float *x, const float *y, float *dx,
                      void *stream) {
-  (void)y;
-  if (!geom_ok(g) || !dy || !dx) return SGH_EINVAL;
-  if (g->is_max && !x) return SGH_EINVAL;
-  const size_t total = size_t(g->N) * g->C * g->H * g->W;
-  if (g->is_max) {
-    // band height: about 12 KB of x rows per workgroup (measured optimum: enough workgroups per CU to
-    // overlap one's staging with another's scans), bands of equal height
-    int TH = 3072 / g->W - g->kernel_h;
-    if (TH < 1) TH = 1;
-    if (TH > g->H) TH = g->H;
-    int bands = (g->H + TH - 1) / TH;
-    TH = (g->H + bands - 1) / bands;
-    bands = (g->H + TH - 1) / TH;
-    const int max_np = (TH + g->kernel_h - 2) / g->stride_h + 2;
-    const int max_xrows = (max_np - 1) * g->stride_h + g->kernel_h;
-    const size_t lds = (size_t(max_xrows) * g->W + size_t(2) * max_np * g->Q + size_t(2) * TH) * sizeof(float);
-    const size_t blocks = size_t(g->N) * g->C * bands;
-    if (lds <= 48 * 1024 && blocks < 0x7fffffffu && g->W <= 2048) {
-      auto kern = k_pool_max_bwd_tiled<0, 0, 0, 0>;
-      if (g->kernel_h == 3 && g->kernel_w == 3 && g->stride_h == 2 && g->stride_w == 2)
-        kern = k_pool_max_bwd_tiled<3, 3, 2, 2>;
-      else if (g->kernel_h == 2 && g->kernel_w == 2 && g->stride_h == 2 && g->stride_w == 2)
-        kern = k_pool_max_bwd_tiled<2, 2, 2, 2>;
-      else if (g->kernel_h == 3 && g->kernel_w == 3 && g->stride_h == 1 && g->stride_w == 1)
-        kern = k_pool_max_bwd_tiled<3, 3, 1, 1>;
-      hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBlock), lds, sgh_stream_of(stream), dy, x, dx, to_g(g), TH,
-                         bands, max_xrows, max_np);
-    } else {
-      hipLaunchKernelGGL(k_pool_max_bwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
-                         to_g(g), total);
-    }
-  } else
-    hipLaunchKernelGGL(k_pool_avg_bwd, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, dx, to_g(g),
-                       total);
-  SGH_LAUNCH_CHECK();
-  return SGH_OK;
+  return pool_bwd<StF32>(g, dy, x, y, dx, stream);
+}
+int sgh_pool_bwd_f16(const sgh_pool_geom *g, const uint16_t *dy, const uint16_t *x, const uint16_t *y, uint16_t *dx,
+                     void *stream) {
+  return pool_bwd<StF16>(g, dy, x, y, dx, stream);
+}
+int sgh_pool_bwd_bf16(const sgh_pool_geom *g, const uint16_t *dy, const uint16_t *x, const uint16_t *y, uint16_t *dx,
+                      void *stream) {
+  return pool_bwd<StBF16>(g, dy, x, y, dx, stream);
 }
 
 }  // extern "C"

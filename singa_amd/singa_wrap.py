@@ -609,15 +609,18 @@ class CudnnPoolingHandle(object):
 
 
 def GpuPoolingForward(h, x):
-    y = Tensor((h.batchsize, h.channels, h.pooled_height, h.pooled_width), x.device(), kFloat32)
-    check(_L().sgh_pool_fwd_f32(C.byref(h.geom), x.ptr, y.ptr, x.device().stream), "sgh_pool_fwd_f32")
+    y = Tensor((h.batchsize, h.channels, h.pooled_height, h.pooled_width), x.device(), x.data_type())
+    fn, name = _fn("pool_fwd", x)
+    check(fn(C.byref(h.geom), x.ptr, y.ptr, x.device().stream), name)
     return y
 
 
 def GpuPoolingBackward(h, dy, x, y):
     if dy.shape() != [h.batchsize, h.channels, h.pooled_height, h.pooled_width]:
         raise SingaHipError("dy shape does not match the handle")
+    if dy.data_type() != x.data_type():
+        raise SingaHipError("dy and x differ in data type")
     dx = _like(x)
-    check(_L().sgh_pool_bwd_f32(C.byref(h.geom), dy.ptr, x.ptr, y.ptr if y is not None else None, dx.ptr,
-                                dy.device().stream), "sgh_pool_bwd_f32")
+    fn, name = _fn("pool_bwd", x)
+    check(fn(C.byref(h.geom), dy.ptr, x.ptr, y.ptr if y is not None else None, dx.ptr, dy.device().stream), name)
     return dx

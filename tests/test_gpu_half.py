@@ -118,3 +118,37 @@ def test_batchnorm_16bit_storage(singa, dev, kind, shape):
     assert dx.data_type() == xt.data_type()
     assert nl2(dx.to_numpy(), dx_o) < 1e-2
     assert nl2(ds.to_numpy(), ds_o) < 1e-3 and nl2(db.to_numpy(), db_o) < 1e-3
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("case", [
+    (2, 3, 8, 8, (2, 2), (2, 2), (0, 0)),
+    (2, 4, 17, 17, (3, 3), (2, 2), (1, 1)),
+    (2, 16, 112, 112, (3, 3), (2, 2), (1, 1)),   # ResNet stem max-pool geometry (tiled kernel, 16-byte staging)
+    (1, 2, 7, 5, (3, 2), (1, 2), (1, 0)),
+    (3, 8, 14, 14, (3, 3), (1, 1), (1, 1)),
+])
+def test_pooling_16bit_storage(singa, dev, kind, case):
+    """Max pooling on 16-bit tensors routes the gradient like the CPU algorithm on the stored
+    values (the 16-bit grid makes ties frequent: first maximum wins) and sums overlapping
+    windows in fp32 with one rounding: bit-exact against the fp32 oracle on the same inputs,
+    rounded once.  Average pooling: same rounding rule."""
+    from oracle import cpu_oracle as O
+    N, C, H, W, kernel, stride, pad = case
+    r = rng(sum(case[:4]) + 3)
+    xt, x = _to(singa, dev, np.round(r.standard_normal((N, C, H, W)) * 4).astype(np.float32) / 4, kind)  # many ties
+    h = singa.CudnnPoolingHandle(xt, kernel, stride, pad, True)
+    y = singa.GpuPoolingForward(h, xt)
+    y_o, mask = O.pool_max_fwd(x, kernel, stride, pad)
+    _same_bits(y.to_numpy(), y_o, "max-pool forward " + kind)       # a maximum of stored values is a stored value
+    dyt, dy = _to(singa, dev, r.standard_normal(y_o.shape).astype(np.float32), kind)
+    dx = singa.GpuPoolingBackward(h, dyt, xt, y)
+    dx_o = O.pool_max_bwd(dy, mask, x.shape)
+    _same_bits(dx.to_numpy(), _round(singa, dx_o, kind), "max-pool backward " + kind)
+    ha = singa.CudnnPoolingHandle(xt, kernel, stride, pad, False)
+    ya = singa.GpuPoolingForward(ha, xt)
+    _same_bits(ya.to_numpy(), _round(singa, O.pool_avg_fwd(x, kernel, stride, pad, include_pad=False), kind),
+               "avg-pool forward " + kind)
+    dxa = singa.GpuPoolingBackward(ha, dyt, xt, ya)
+    _same_bits(dxa.to_numpy(), _round(singa, O.pool_avg_bwd(dy, x.shape, kernel, stride, pad, include_pad=False), kind),
+               "avg-pool backward " + kind)
