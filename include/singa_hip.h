@@ -250,6 +250,29 @@ SGH_API int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float
                              const float *bias, float *y, void *workspace, size_t ws_bytes,
                              void *stream);
 
+/* The three convolution passes on 16-bit tensors (x, W, y and their gradients all binary16 or
+ * all bfloat16, as a reference handle built from a half input runs them:
+ * src/model/operation/convolution.cc:444-572).  Arithmetic: the operands are widened to fp32 in
+ * the workspace, the fp32 MFMA kernels accumulate in fp32, the result is rounded once.
+ * Workspace: sgh_conv_workspace_bytes_h(g, which) bytes. */
+SGH_API size_t sgh_conv_workspace_bytes_h(const sgh_conv_geom *g, int which);
+SGH_API int sgh_conv_dgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W,
+                               uint16_t *dx, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_conv_dgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W,
+                                uint16_t *dx, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_conv_wgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x,
+                               uint16_t *dW, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_conv_wgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x,
+                                uint16_t *dW, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_conv_bgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db, void *stream);
+SGH_API int sgh_conv_bgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db, void *stream);
+SGH_API int sgh_conv_fwd_f16(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W,
+                             const uint16_t *bias, uint16_t *y, void *workspace, size_t ws_bytes,
+                             void *stream);
+SGH_API int sgh_conv_fwd_bf16(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W,
+                              const uint16_t *bias, uint16_t *y, void *workspace, size_t ws_bytes,
+                              void *stream);
+
 /* GpuBatchNormForwardTraining (src/model/operation/batchnorm.cc:287-329), spatial mode:
  * per-channel batch mean / biased variance over N*HW, y = gamma*(x-mean)*invstd + beta,
  * running = (1-factor)*running + factor*batch (unbiased variance), saves (mean, invstd) with

@@ -93,6 +93,15 @@ SIGNATURES = {
     "sgh_conv_wgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_bgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp]),
     "sgh_conv_fwd_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
+    "sgh_conv_workspace_bytes_h": (sz, [C.POINTER(ConvGeom), C.c_int]),
+    "sgh_conv_dgrad_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
+    "sgh_conv_dgrad_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
+    "sgh_conv_wgrad_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
+    "sgh_conv_wgrad_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
+    "sgh_conv_bgrad_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp]),
+    "sgh_conv_bgrad_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp]),
+    "sgh_conv_fwd_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
+    "sgh_conv_fwd_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
     "sgh_bn_workspace_bytes": (sz, [C.c_int, C.c_int, C.c_int]),
     "sgh_bn_fwd_train_f32": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
                                        C.c_int, C.c_int, vp, sz, vp]),

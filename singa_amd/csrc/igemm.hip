@@ -25,6 +25,7 @@
 #include <stdlib.h>
 
 #include "common.h"
+#include "storage.h"
 
 namespace {
 
@@ -647,18 +648,19 @@ __global__ __launch_bounds__(NT) void k_col2im_gather(const float *__restrict__ 
 }
 
 // One thread per (k), summing dy over n, p, q is too serial; use one workgroup per k.
-__global__ __launch_bounds__(NT) void k_conv_bgrad(const float *__restrict__ dy, float *__restrict__ db, int N, int K,
-                                                  int PQ) {
+template <class S>
+__global__ __launch_bounds__(NT) void k_conv_bgrad(const typename S::elem *__restrict__ dy,
+                                                  typename S::elem *__restrict__ db, int N, int K, int PQ) {
   __shared__ float red[16];
   const int k = blockIdx.x;
   float s = 0.f;
   const int total = N * PQ;
   for (int i = threadIdx.x; i < total; i += NT) {
     const int n = i / PQ, r = i - n * PQ;
-    s += dy[(long(n) * K + k) * PQ + r];
+    s += S::ld(dy + (long(n) * K + k) * PQ + r);
   }
   s = sgh_block_sum(s, red);
-  if (threadIdx.x == 0) db[k] = s;
+  if (threadIdx.x == 0) S::st(db + k, s);
 }
 
 inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
@@ -1152,7 +1154,8 @@ int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, 
 
 int sgh_conv_bgrad_f32(const sgh_conv_geom *g, const float *dy, float *db, void *stream) {
   if (!conv_ok(g) || !dy || !db) return SGH_EINVAL;
-  hipLaunchKernelGGL(k_conv_bgrad, dim3(g->K), dim3(NT), 0, sgh_stream_of(stream), dy, db, g->N, g->K, g->P * g->Q);
+  hipLaunchKernelGGL(k_conv_bgrad<StF32>, dim3(g->K), dim3(NT), 0, sgh_stream_of(stream), dy, db, g->N, g->K,
+                     g->P * g->Q);
   SGH_LAUNCH_CHECK();
   return SGH_OK;
 }
@@ -1179,6 +1182,111 @@ int sgh_gemm_f32(int transA, int transB, int M, int N, int K, float alpha, const
   else rc = gemm_pick<false, false>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
   sgh_prof_stop(s);
   return rc;
+}
+
+
+// ---- 16-bit storage (binary16 / bfloat16) --------------------------------------------------
+// The tensors are converted to fp32 in the workspace, the fp32 kernels above do the arithmetic
+// (fp32 MFMA, fp32 accumulation) and the result is rounded once on the way out.  The workspace
+// holds the three fp32 copies followed by the fp32 pass's own workspace.
+namespace {
+
+struct HalfPlan {
+  size_t a_elems, b_elems, out_elems, inner;  // the two inputs, the output, the fp32 pass's workspace
+  size_t total() const { return align256(a_elems * 4) + align256(b_elems * 4) + align256(out_elems * 4) + inner; }
+};
+
+inline HalfPlan half_plan(const sgh_conv_geom *g, int which) {
+  const size_t x = size_t(g->N) * g->C * g->H * g->W, y = size_t(g->N) * g->K * g->P * g->Q;
+  const size_t w = size_t(g->K) * g->C * g->R * g->S;
+  HalfPlan p{};
+  p.inner = sgh_conv_workspace_bytes(g, which);
+  if (which == SGH_CONV_DGRAD) p.a_elems = y, p.b_elems = w, p.out_elems = x;
+  else if (which == SGH_CONV_WGRAD) p.a_elems = y, p.b_elems = x, p.out_elems = w;
+  else p.a_elems = x, p.b_elems = w, p.out_elems = y;
+  return p;
+}
+
+typedef int (*cast_in_fn)(const uint16_t *, float *, size_t, void *);
+typedef int (*cast_out_fn)(const float *, uint16_t *, size_t, void *);
+
+// which: SGH_CONV_*; (a, b) are the pass's two tensor inputs in the order of its fp32 entry point
+int conv_half(const sgh_conv_geom *g, int which, const uint16_t *a, const uint16_t *b, const uint16_t *bias,
+              uint16_t *out, void *workspace, size_t ws_bytes, void *stream, cast_in_fn in, cast_out_fn outc) {
+  if (!conv_ok(g) || !a || !b || !out) return SGH_EINVAL;
+  const HalfPlan p = half_plan(g, which);
+  if (!workspace || ws_bytes < p.total() + (bias ? align256(size_t(g->K) * 4) : 0)) return SGH_EWORKSPACE;
+  char *w = static_cast<char *>(workspace);
+  float *a32 = reinterpret_cast<float *>(w);
+  float *b32 = reinterpret_cast<float *>(w + align256(p.a_elems * 4));
+  float *o32 = reinterpret_cast<float *>(w + align256(p.a_elems * 4) + align256(p.b_elems * 4));
+  char *inner = w + align256(p.a_elems * 4) + align256(p.b_elems * 4) + align256(p.out_elems * 4);
+  float *bias32 = nullptr;
+  int rc = in(a, a32, p.a_elems, stream);
+  if (rc == SGH_OK) rc = in(b, b32, p.b_elems, stream);
+  if (rc == SGH_OK && bias) {
+    bias32 = reinterpret_cast<float *>(inner + p.inner);
+    rc = in(bias, bias32, size_t(g->K), stream);
+  }
+  if (rc != SGH_OK) return rc;
+  if (which == SGH_CONV_DGRAD) rc = sgh_conv_dgrad_f32(g, a32, b32, o32, inner, p.inner, stream);
+  else if (which == SGH_CONV_WGRAD) rc = sgh_conv_wgrad_f32(g, a32, b32, o32, inner, p.inner, stream);
+  else rc = sgh_conv_fwd_f32(g, a32, b32, bias32, o32, inner, p.inner, stream);
+  if (rc != SGH_OK) return rc;
+  return outc(o32, out, p.out_elems, stream);
+}
+
+}  // namespace
+
+int sgh_conv_bgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db, void *stream) {
+  if (!conv_ok(g) || !dy || !db) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_conv_bgrad<StF16>, dim3(g->K), dim3(NT), 0, sgh_stream_of(stream), dy, db, g->N, g->K,
+                     g->P * g->Q);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+int sgh_conv_bgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db, void *stream) {
+  if (!conv_ok(g) || !dy || !db) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_conv_bgrad<StBF16>, dim3(g->K), dim3(NT), 0, sgh_stream_of(stream), dy, db, g->N, g->K,
+                     g->P * g->Q);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+size_t sgh_conv_workspace_bytes_h(const sgh_conv_geom *g, int which) {
+  if (!conv_ok(g) || which < 0 || which > 2) return 0;
+  return half_plan(g, which).total() + (which == SGH_CONV_FWD ? align256(size_t(g->K) * 4) : 0);
+}
+
+int sgh_conv_dgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
+                       size_t ws_bytes, void *stream) {
+  return conv_half(g, SGH_CONV_DGRAD, dy, W, nullptr, dx, workspace, ws_bytes, stream, sgh_cast_f16_to_f32,
+                   sgh_cast_f32_to_f16);
+}
+int sgh_conv_dgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
+                        size_t ws_bytes, void *stream) {
+  return conv_half(g, SGH_CONV_DGRAD, dy, W, nullptr, dx, workspace, ws_bytes, stream, sgh_cast_bf16_to_f32,
+                   sgh_cast_f32_to_bf16);
+}
+int sgh_conv_wgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x, uint16_t *dW, void *workspace,
+                       size_t ws_bytes, void *stream) {
+  return conv_half(g, SGH_CONV_WGRAD, dy, x, nullptr, dW, workspace, ws_bytes, stream, sgh_cast_f16_to_f32,
+                   sgh_cast_f32_to_f16);
+}
+int sgh_conv_wgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x, uint16_t *dW, void *workspace,
+                        size_t ws_bytes, void *stream) {
+  return conv_half(g, SGH_CONV_WGRAD, dy, x, nullptr, dW, workspace, ws_bytes, stream, sgh_cast_bf16_to_f32,
+                   sgh_cast_f32_to_bf16);
+}
+int sgh_conv_fwd_f16(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
+                     void *workspace, size_t ws_bytes, void *stream) {
+  return conv_half(g, SGH_CONV_FWD, x, W, bias, y, workspace, ws_bytes, stream, sgh_cast_f16_to_f32,
+                   sgh_cast_f32_to_f16);
+}
+int sgh_conv_fwd_bf16(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
+                      void *workspace, size_t ws_bytes, void *stream) {
+  return conv_half(g, SGH_CONV_FWD, x, W, bias, y, workspace, ws_bytes, stream, sgh_cast_bf16_to_f32,
+                   sgh_cast_f32_to_bf16);
 }
 
 }  // extern "C"

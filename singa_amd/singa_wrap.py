@@ -492,7 +492,10 @@ class CudnnConvHandle(object):
         self.col_height = self.channels * self.kernel_h * self.kernel_w
         self.col_width = self.conv_height * self.conv_width
         self.imagesize = x.Size() // self.batchsize
-        need = max(_L().sgh_conv_workspace_bytes(C.byref(self.geom), w) for w in (0, 1, 2))
+        # a handle built from a 16-bit input runs every pass on 16-bit tensors (convolution.cc:444-572)
+        self.dtype = x.data_type()
+        ws_fn = _L().sgh_conv_workspace_bytes if self.dtype == kFloat32 else _L().sgh_conv_workspace_bytes_h
+        need = max(ws_fn(C.byref(self.geom), w) for w in (0, 1, 2))
         if need > workspace_byte_limit:
             raise SingaHipError("workspace of %d bytes exceeds the limit" % need)
         self.workspace_count = need // 4
@@ -509,18 +512,20 @@ class CudnnConvHandle(object):
 
 def GpuConvForward(x, W, b, h):
     h._check_x(x)
-    y = Tensor((h.batchsize, h.num_filters, h.conv_height, h.conv_width), x.device(), kFloat32)
+    y = Tensor((h.batchsize, h.num_filters, h.conv_height, h.conv_width), x.device(), x.data_type())
     bias = b.ptr if (h.bias_term and b is not None) else None
-    check(_L().sgh_conv_fwd_f32(C.byref(h.geom), x.ptr, W.ptr, bias, y.ptr, h.workspace.ptr,
-                                h.workspace.MemSize(), x.device().stream), "sgh_conv_fwd_f32")
+    fn, name = _fn("conv_fwd", x)
+    check(fn(C.byref(h.geom), x.ptr, W.ptr, bias, y.ptr, h.workspace.ptr, h.workspace.MemSize(),
+             x.device().stream), name)
     return y
 
 
 def GpuConvBackwardx(dy, W, x, h):
     h._check_dy(dy)
     dx = _like(x)
-    check(_L().sgh_conv_dgrad_f32(C.byref(h.geom), dy.ptr, W.ptr, dx.ptr, h.workspace.ptr,
-                                  h.workspace.MemSize(), dy.device().stream), "sgh_conv_dgrad_f32")
+    fn, name = _fn("conv_dgrad", dy)
+    check(fn(C.byref(h.geom), dy.ptr, W.ptr, dx.ptr, h.workspace.ptr, h.workspace.MemSize(),
+             dy.device().stream), name)
     return dx
 
 
@@ -528,15 +533,17 @@ def GpuConvBackwardW(dy, x, W, h):
     h._check_dy(dy)
     h._check_x(x)
     dW = _like(W)
-    check(_L().sgh_conv_wgrad_f32(C.byref(h.geom), dy.ptr, x.ptr, dW.ptr, h.workspace.ptr,
-                                  h.workspace.MemSize(), dy.device().stream), "sgh_conv_wgrad_f32")
+    fn, name = _fn("conv_wgrad", dy)
+    check(fn(C.byref(h.geom), dy.ptr, x.ptr, dW.ptr, h.workspace.ptr, h.workspace.MemSize(),
+             dy.device().stream), name)
     return dW
 
 
 def GpuConvBackwardb(dy, b, h):
     h._check_dy(dy)
     db = _like(b)
-    check(_L().sgh_conv_bgrad_f32(C.byref(h.geom), dy.ptr, db.ptr, dy.device().stream), "sgh_conv_bgrad_f32")
+    fn, name = _fn("conv_bgrad", dy)
+    check(fn(C.byref(h.geom), dy.ptr, db.ptr, dy.device().stream), name)
     return db
 
 

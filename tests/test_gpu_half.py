@@ -152,3 +152,38 @@ def test_pooling_16bit_storage(singa, dev, kind, case):
     dxa = singa.GpuPoolingBackward(ha, dyt, xt, ya)
     _same_bits(dxa.to_numpy(), _round(singa, O.pool_avg_bwd(dy, x.shape, kernel, stride, pad, include_pad=False), kind),
                "avg-pool backward " + kind)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("case", [
+    (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), True),      # shared-tile kernels
+    (2, 64, 14, 14, 128, 3, 3, (2, 2), (1, 1), False),    # stride-2 residue classes
+    (2, 3, 32, 32, 64, 7, 7, (2, 2), (3, 3), False),      # stem kernels
+    (3, 64, 8, 8, 128, 1, 1, (2, 2), (0, 0), False),      # pointwise
+    (2, 5, 9, 7, 6, 3, 2, (2, 1), (1, 0), True),          # generic path
+])
+def test_conv_16bit_storage(singa, dev, kind, case):
+    """Convolution passes on 16-bit tensors: operands widened to fp32, fp32 accumulation, one
+    rounding of the result.  Checked against the fp32 CPU oracle on the same stored inputs at the
+    16-bit tolerance (1e-2 normalised L2; the rounding of the result alone is about 3e-4 for
+    binary16 and 2e-3 for bfloat16)."""
+    from oracle import cpu_oracle as O
+    from util import nl2
+    N, C, H, W, K, R, S, stride, pad, bias = case
+    r = rng(sum(case[:7]) + 11)
+    xt, x = _to(singa, dev, r.standard_normal((N, C, H, W)).astype(np.float32), kind)
+    wt, w = _to(singa, dev, (r.standard_normal((K, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32), kind)
+    bt, b = _to(singa, dev, r.standard_normal(K).astype(np.float32), kind) if bias else (None, None)
+    h = singa.CudnnConvHandle(xt, (R, S), stride, pad, C, K, bias)
+    y = singa.GpuConvForward(xt, wt, bt, h)
+    assert y.data_type() == xt.data_type()
+    assert nl2(y.to_numpy(), O.conv_fwd(x, w, b, stride, pad)) < 1e-2
+    dyt, dy = _to(singa, dev, r.standard_normal(y.shape()).astype(np.float32), kind)
+    dx = singa.GpuConvBackwardx(dyt, wt, xt, h)
+    dw = singa.GpuConvBackwardW(dyt, xt, wt, h)
+    dx_o, dw_o = O.conv_bwd(dy, x, w, stride, pad)
+    assert dx.data_type() == xt.data_type() and dw.data_type() == xt.data_type()
+    assert nl2(dx.to_numpy(), dx_o) < 1e-2 and nl2(dw.to_numpy(), dw_o) < 1e-2
+    if bias:
+        db = singa.GpuConvBackwardb(dyt, bt, h)
+        assert nl2(db.to_numpy(), O.conv_bgrad(dy)) < 1e-2
