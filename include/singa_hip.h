@@ -194,6 +194,23 @@ typedef struct sgh_sgd_item {
 SGH_API int sgh_sgd_momentum_multi_f32(const sgh_sgd_item *table_dev, int count, size_t total_n,
                                        float lr, float mu, float damp, float wd, int nesterov,
                                        void *stream);
+/* The same update on 16-bit gradients.
+ * sgh_sgd_momentum_f16 / _bf16: p, g, v all 16-bit, as opt.SGD(dtype=float16) keeps them
+ *   (python/singa/opt.py:283-284); fp32 arithmetic, p and v rounded once per step (the
+ *   reference's four unfused half ops round after each op: parity at the 16-bit tolerance).
+ * sgh_sgd_momentum_master_f16 / _bf16: mixed precision -- fp32 master weights and fp32 momentum
+ *   are updated from the 16-bit gradient, and p_out receives the master rounded to 16 bits
+ *   (the working copy the next forward pass reads).  No counterpart in the reference's opt.py. */
+SGH_API int sgh_sgd_momentum_f16(uint16_t *p, const uint16_t *g, uint16_t *v, size_t n, float lr,
+                                 float mu, float damp, float wd, int nesterov, void *stream);
+SGH_API int sgh_sgd_momentum_bf16(uint16_t *p, const uint16_t *g, uint16_t *v, size_t n, float lr,
+                                  float mu, float damp, float wd, int nesterov, void *stream);
+SGH_API int sgh_sgd_momentum_master_f16(float *p_master, const uint16_t *g, float *v,
+                                        uint16_t *p_out, size_t n, float lr, float mu, float damp,
+                                        float wd, int nesterov, void *stream);
+SGH_API int sgh_sgd_momentum_master_bf16(float *p_master, const uint16_t *g, float *v,
+                                         uint16_t *p_out, size_t n, float lr, float mu, float damp,
+                                         float wd, int nesterov, void *stream);
 
 /* GEMM<float, Lang>: tensor_math.h:444-448; CPU tensor_math_cpp.h:877-899 (cblas_sgemm,
  * row-major).  C[M,N] = alpha * op(A) * op(B) + beta * C; lda/ldb/ldc are row pitches of the

@@ -83,6 +83,12 @@ SIGNATURES = {
     "sgh_sgd_momentum_devhyper_f32": (C.c_int, [vp, vp, vp, sz, vp, C.c_int, vp]),
     "sgh_sgd_momentum_multi_f32": (C.c_int, [vp, C.c_int, sz, C.c_float, C.c_float, C.c_float,
                                              C.c_float, C.c_int, vp]),
+    "sgh_sgd_momentum_f16": (C.c_int, [vp, vp, vp, sz, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, vp]),
+    "sgh_sgd_momentum_bf16": (C.c_int, [vp, vp, vp, sz, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, vp]),
+    "sgh_sgd_momentum_master_f16": (C.c_int, [vp, vp, vp, vp, sz, C.c_float, C.c_float, C.c_float, C.c_float,
+                                              C.c_int, vp]),
+    "sgh_sgd_momentum_master_bf16": (C.c_int, [vp, vp, vp, vp, sz, C.c_float, C.c_float, C.c_float, C.c_float,
+                                               C.c_int, vp]),
     "sgh_gemm_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, vp, C.c_int,
                                vp, C.c_int, C.c_float, vp, C.c_int, vp]),
     "sgh_sum_rows_f32": (C.c_int, [vp, vp, C.c_int, C.c_int, vp]),

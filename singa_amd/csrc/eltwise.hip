@@ -4,6 +4,7 @@
 // rounding sequence of the CPU reference (separate multiply and add, no contraction) so that
 // results are comparable bit for bit where the reference is elementwise.
 #include "common.h"
+#include "sgd_math.h"
 
 // contraction is disabled per function where the reference rounds after each op
 #define SGH_NO_CONTRACT _Pragma("clang fp contract(off)")
@@ -184,34 +185,6 @@ __global__ __launch_bounds__(kBlock) void k_fill(float *o, float v, size_t n) {
 // ---------------------------------------------------------------------------------------
 // Fused SGD-momentum: streams p, g, v in; p, v out (5 * 4 bytes per parameter element).
 // ---------------------------------------------------------------------------------------
-struct SgdHyper {
-  float lr, mu, damp, wd;
-};
-
-__device__ __forceinline__ void sgd_one(float &p, float g, float &v, const SgdHyper h, int nesterov, bool has_v) {
-  SGH_NO_CONTRACT
-  const float one_minus_damp = 1.0f - h.damp;
-  const float minus_lr = 0.0f - h.lr;
-  if (h.wd != 0.f) {
-    float t = h.wd * p;
-    g = g + t;
-  }
-  if (has_v) {
-    float vi = v * h.mu;
-    float t = one_minus_damp * g;
-    vi = vi + t;
-    v = vi;
-    if (nesterov) {
-      float t2 = h.mu * vi;
-      g = g + t2;
-    } else {
-      g = vi;
-    }
-  }
-  float t = minus_lr * g;
-  p = p + t;
-}
-
 template <bool DEV_HYPER>
 __global__ __launch_bounds__(kBlock) void k_sgd(float *__restrict__ p, const float *__restrict__ g,
                                                float *__restrict__ v, size_t n, SgdHyper hh,

@@ -8,6 +8,7 @@
 // chunks, as in the fp32 kernels.
 #include "common.h"
 #include "storage.h"
+#include "sgd_math.h"
 
 namespace {
 
@@ -183,9 +184,64 @@ int cast_from16(const uint16_t *src, float *dst, size_t n, void *stream) {
   return SGH_OK;
 }
 
+// Fused SGD-momentum on 16-bit gradients.
+//   MASTER = false: p, g, v all 16-bit (opt.SGD constructed with dtype float16): fp32 arithmetic,
+//                   p and v rounded once per step;
+//   MASTER = true : fp32 master weights p32 and fp32 momentum v32 are updated from the 16-bit
+//                   gradient and the 16-bit working copy p16 is refreshed from the master.
+template <class T, bool MASTER>
+__global__ __launch_bounds__(kBlock) void k_sgd_h(u16 *__restrict__ p16, const u16 *__restrict__ g16,
+                                                 u16 *__restrict__ v16, float *__restrict__ p32,
+                                                 float *__restrict__ v32, size_t n, SgdHyper h, int nesterov) {
+  const bool has_v = h.mu != 0.f && (MASTER ? v32 != nullptr : v16 != nullptr);
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) {
+    float pp = MASTER ? p32[i] : T::load(p16[i]);
+    float vv = has_v ? (MASTER ? v32[i] : T::load(v16[i])) : 0.f;
+    sgd_one(pp, T::load(g16[i]), vv, h, nesterov, has_v);
+    if (MASTER) {
+      p32[i] = pp;
+      if (has_v) v32[i] = vv;
+    } else if (has_v) {
+      v16[i] = T::store(vv);
+    }
+    p16[i] = T::store(pp);
+  }
+}
+
+template <class T, bool MASTER>
+int sgd_h(uint16_t *p16, const uint16_t *g16, uint16_t *v16, float *p32, float *v32, size_t n, float lr, float mu,
+          float damp, float wd, int nesterov, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!p16 || !g16 || (MASTER && !p32)) return SGH_EINVAL;
+  if (mu != 0.f && (MASTER ? !v32 : !v16)) return SGH_EINVAL;
+  hipLaunchKernelGGL((k_sgd_h<T, MASTER>), dim3(grid_for(n)), dim3(kBlock), 0, sgh_stream_of(stream), p16, g16, v16, p32,
+                     v32, n, SgdHyper{lr, mu, damp, wd}, nesterov);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+int sgh_sgd_momentum_f16(uint16_t *p, const uint16_t *g, uint16_t *v, size_t n, float lr, float mu, float damp,
+                         float wd, int nesterov, void *stream) {
+  return sgd_h<F16, false>(p, g, v, nullptr, nullptr, n, lr, mu, damp, wd, nesterov, stream);
+}
+int sgh_sgd_momentum_bf16(uint16_t *p, const uint16_t *g, uint16_t *v, size_t n, float lr, float mu, float damp,
+                          float wd, int nesterov, void *stream) {
+  return sgd_h<BF16, false>(p, g, v, nullptr, nullptr, n, lr, mu, damp, wd, nesterov, stream);
+}
+int sgh_sgd_momentum_master_f16(float *p_master, const uint16_t *g, float *v, uint16_t *p_out, size_t n, float lr,
+                                float mu, float damp, float wd, int nesterov, void *stream) {
+  return sgd_h<F16, true>(p_out, g, nullptr, p_master, v, n, lr, mu, damp, wd, nesterov, stream);
+}
+int sgh_sgd_momentum_master_bf16(float *p_master, const uint16_t *g, float *v, uint16_t *p_out, size_t n, float lr,
+                                 float mu, float damp, float wd, int nesterov, void *stream) {
+  return sgd_h<BF16, true>(p_out, g, nullptr, p_master, v, n, lr, mu, damp, wd, nesterov, stream);
+}
+
 
 int sgh_cast_f32_to_f16(const float *src, uint16_t *dst, size_t n, void *stream) { return cast_to16<F16>(src, dst, n, stream); }
 int sgh_cast_f16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream) { return cast_from16<F16>(src, dst, n, stream); }

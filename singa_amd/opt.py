@@ -31,6 +31,7 @@ class SGD(object):
         self.weight_decay = float(weight_decay)
         self.nesterov = bool(nesterov)
         self.moments = dict()
+        self.masters = dict()
         self.step_counter = 0
         self._table = None
         self._table_key = None
@@ -38,8 +39,13 @@ class SGD(object):
 
     def _moment(self, name, p):
         if name not in self.moments:
-            v = singa.Tensor(p.shape(), p.device(), p.data_type())
-            v.SetFloatValue(0.0)
+            if p.data_type() == singa.kFloat32:
+                v = singa.Tensor(p.shape(), p.device(), singa.kFloat32)
+                v.SetFloatValue(0.0)
+            else:  # zeros in a 16-bit type: cast fp32 zeros
+                z = singa.Tensor(p.shape(), p.device(), singa.kFloat32)
+                z.SetFloatValue(0.0)
+                v = z.AsType(p.data_type())
             self.moments[name] = v
         return self.moments[name]
 
@@ -48,11 +54,30 @@ class SGD(object):
         tensor is left untouched."""
         assert param_value.shape() == param_grad.shape(), ("shape mismatch", param_value.shape(),
                                                              param_grad.shape())
+        if param_value.data_type() != param_grad.data_type():
+            raise singa.SingaHipError("parameter and gradient differ in data type")
         v = self._moment(param_name, param_value) if self.momentum != 0 else None
-        check(_lib.lib().sgh_sgd_momentum_f32(param_value.ptr, param_grad.ptr, v.ptr if v is not None else None,
-                                              param_value.Size(), self.lr, self.momentum, self.dampening,
-                                              self.weight_decay, int(self.nesterov), param_value.device().stream),
-              "sgh_sgd_momentum_f32")
+        name = "sgh_sgd_momentum_" + singa._SUFFIX[param_value.data_type()]   # f32 / f16 / bf16
+        check(getattr(_lib.lib(), name)(param_value.ptr, param_grad.ptr, v.ptr if v is not None else None,
+                                        param_value.Size(), self.lr, self.momentum, self.dampening,
+                                        self.weight_decay, int(self.nesterov), param_value.device().stream), name)
+
+    def apply_master(self, param_name, param_value, param_grad):
+        """Mixed precision: ``param_value`` / ``param_grad`` are 16-bit; an fp32 master copy of the
+        parameter (created from it on first use) and an fp32 momentum buffer are updated, and
+        ``param_value`` is refreshed from the master."""
+        if param_value.data_type() not in (singa.kFloat16, singa.kBFloat16):
+            raise singa.SingaHipError("apply_master expects 16-bit parameters")
+        if param_value.data_type() != param_grad.data_type() or param_value.shape() != param_grad.shape():
+            raise singa.SingaHipError("parameter and gradient differ in shape or data type")
+        if param_name not in self.masters:
+            self.masters[param_name] = param_value.AsType(singa.kFloat32)
+        master = self.masters[param_name]
+        v = self._moment(param_name, master) if self.momentum != 0 else None
+        name = "sgh_sgd_momentum_master_" + singa._SUFFIX[param_value.data_type()]
+        check(getattr(_lib.lib(), name)(master.ptr, param_grad.ptr, v.ptr if v is not None else None, param_value.ptr,
+                                        param_value.Size(), self.lr, self.momentum, self.dampening,
+                                        self.weight_decay, int(self.nesterov), param_value.device().stream), name)
 
     def apply_all(self, named_params_grads):
         """Update every (name, p, g) triple with ONE kernel launch.  The pointer table is built

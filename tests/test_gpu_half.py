@@ -187,3 +187,50 @@ def test_conv_16bit_storage(singa, dev, kind, case):
     if bias:
         db = singa.GpuConvBackwardb(dyt, bt, h)
         assert nl2(db.to_numpy(), O.conv_bgrad(dy)) < 1e-2
+
+
+def _sgd_ref(p, g, v, lr, mu, damp, wd, nesterov):
+    """The four ops of SGD.apply in fp32, each product / sum rounded separately."""
+    f = np.float32
+    p, g, v = p.astype(f), g.astype(f), v.astype(f)
+    if wd != 0:
+        g = g + f(wd) * p
+    if mu != 0:
+        v = v * f(mu) + (f(1.0) - f(damp)) * g
+        g = g + f(mu) * v if nesterov else v
+    p = p + (f(0.0) - f(lr)) * g
+    return p, v
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("hyper", [(0.05, 0.9, 0.0, 0.0, False), (0.1, 0.9, 0.0, 1e-4, True), (0.01, 0.0, 0.0, 5e-4, False),
+                                   (0.05, 0.5, 0.1, 0.0, False)])
+def test_sgd_on_16bit_gradients(singa, dev, kind, hyper):
+    from singa_amd import opt
+    lr, mu, damp, wd, nesterov = hyper
+    r = rng(int(lr * 1000) + int(mu * 10))
+    n = 70001
+    # (a) everything 16-bit: two steps, p and v rounded once per step
+    pt, p = _to(singa, dev, r.standard_normal(n).astype(np.float32), kind)
+    sgd = opt.SGD(lr=lr, momentum=mu, dampening=damp, weight_decay=wd, nesterov=nesterov)
+    v = np.zeros(n, np.float32)
+    for _ in range(2):
+        gt, g = _to(singa, dev, r.standard_normal(n).astype(np.float32), kind)
+        sgd.apply("w", pt, gt)
+        p, v = _sgd_ref(p, g, v, lr, mu, damp, wd, nesterov)
+        p, v = _round(singa, p, kind), _round(singa, v, kind)
+        _same_bits(pt.to_numpy(), p, "16-bit SGD p " + kind)
+        if mu != 0:
+            _same_bits(sgd.moments["w"].to_numpy(), v, "16-bit SGD v " + kind)
+    # (b) fp32 master weights and momentum, 16-bit working copy
+    pt, p = _to(singa, dev, r.standard_normal(n).astype(np.float32), kind)
+    sgd = opt.SGD(lr=lr, momentum=mu, dampening=damp, weight_decay=wd, nesterov=nesterov)
+    v = np.zeros(n, np.float32)
+    for _ in range(3):
+        gt, g = _to(singa, dev, r.standard_normal(n).astype(np.float32), kind)
+        sgd.apply_master("w", pt, gt)
+        p, v = _sgd_ref(p, g, v, lr, mu, damp, wd, nesterov)     # the master stays fp32 between steps
+        _same_bits(sgd.masters["w"].to_numpy(), p, "master p " + kind)
+        _same_bits(pt.to_numpy(), _round(singa, p, kind), "working copy " + kind)
+        if mu != 0:
+            _same_bits(sgd.moments["w"].to_numpy(), v, "master v " + kind)
