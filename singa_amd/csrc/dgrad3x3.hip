@@ -41,13 +41,18 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
 
 struct D3Args {
   const float *dy, *wt;   // wt: re-laid weights [tap][KP][C]
-  const float *bias;      // per output channel, added in the epilogue (NULL: none; unused with split reduction)
+  const float *bias;      // per output channel, added when a tile is finished (NULL: none)
   float *dx;
   int N, C, H, W, K, KP;  // dx is N x C x H x W
   int P, Q;               // dy is N x K x P x Q (stride 1: P == H, Q == W; stride 2: H == 2P, W == 2Q)
   int total_pix;          // N * P * Q: pixels of the tile index space
-  int chunks_per_split;   // reduction chunks (16 channels of k each) per grid.z slice
-  long split_stride;      // elements between the partial outputs of consecutive slices
+  // Work assignment (1-D grid).  Tile t = (pixel tile t / ctiles, channel tile t % ctiles).  Workgroups
+  // [0, dp_tiles) take one whole tile each; workgroup dp_tiles + g takes units
+  // [g * sk_units / sk_wgs, (g + 1) * sk_units / sk_wgs) of the remaining tiles, a unit being one
+  // reduction chunk of one tile (unit u = tile dp_tiles + u / nchunks, chunk u % nchunks).
+  int ctiles, dp_tiles, sk_wgs;
+  long sk_units;
+  float *partials;        // [sk_wgs][2][classes * BM * BN]: a workgroup's first / last incomplete tile
   unsigned dy_bytes, wt_bytes;
 };
 
@@ -89,11 +94,35 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 wavefronts, 64 x 32 each
-  const int c0 = blockIdx.x * BM;
-  const int pix0 = blockIdx.y * BN;
   const int HW = a.H * a.W, PQ = a.P * a.Q;
   const int VH = S2 ? a.P + 1 : a.P + 2;    // virtual rows per image: its dy rows plus the zero rows a tap can reach
   const rsrc_t rdy = make_rsrc(a.dy, a.dy_bytes), rw = make_rsrc(a.wt, a.wt_bytes);
+  const int nchunks = a.KP / KC;
+
+  // ---- this workgroup's work: one whole tile, or a run of (tile, chunk) units that may span tiles
+  const bool stream = int(blockIdx.x) >= a.dp_tiles;
+  const int sk_g = int(blockIdx.x) - a.dp_tiles;
+  long u = stream ? sk_g * a.sk_units / a.sk_wgs : 0;
+  const long u_end = stream ? (sk_g + 1) * a.sk_units / a.sk_wgs : 0;
+  const int first_tile = int(u / nchunks);
+  for (bool again = true; again;) {
+  int tile, ch_begin, ch_end, tile_rel = 0;
+  if (!stream) {
+    tile = blockIdx.x;
+    ch_begin = 0;
+    ch_end = nchunks;
+    again = false;
+  } else {
+    if (u >= u_end) break;
+    tile_rel = int(u / nchunks);
+    tile = a.dp_tiles + tile_rel;
+    ch_begin = int(u - long(tile_rel) * nchunks);
+    ch_end = int(min(long(nchunks), ch_begin + (u_end - u)));
+    u += ch_end - ch_begin;
+  }
+  const bool whole = ch_begin == 0 && ch_end == nchunks;
+  const int c0 = (tile % a.ctiles) * BM;
+  const int pix0 = (tile / a.ctiles) * BN;
 
   // first virtual row of the slab: the row above the tile's first pixel row
   const int n_first = pix0 / PQ, h_first = (pix0 - n_first * PQ) / a.Q;
@@ -147,10 +176,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
   for (int i = 0; i < NCLS * TM; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
-
-  const int nchunks = a.KP / KC;
-  const int ch_begin = blockIdx.z * a.chunks_per_split;
-  const int ch_end = min(ch_begin + a.chunks_per_split, nchunks);
 
   // Staging registers.  Step q (tap q % 9 of chunk q / 9) requests what step q + LAT writes: the
   // weights of step q + LAT + 1 and dy slots [td * SPT, (td + 1) * SPT) of the chunk after step
@@ -210,55 +235,116 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
     dcur ^= 1;
   }
 
-  // epilogue: dx[n][c][h][w], this lane's pixel, rows c0 + wm*(BM/2) + i*32 + 8*(v/4) + 4*(lane/32) + v%4
-  if (pix < a.total_pix) {
+  // epilogue.  A finished tile goes to dx[n][c][h][w] (this lane's pixel, rows c0 + wm*(BM/2) + i*32 +
+  // 8*(v/4) + 4*(lane/32) + v%4); an incomplete one to this workgroup's partial slot as
+  // [class][row][pixel], to be summed by k_dgrad3x3_fixup.
+  // (the lane term is laundered through an empty asm so that the epilogue's address arithmetic is
+  // not hoisted out of the segment loop, where it would occupy registers during the MFMA loop)
+  int lhalf = lane >> 5;
+  asm volatile("" : "+v"(lhalf));
+  if (!whole) {
+    float *ps = a.partials + (size_t(sk_g) * 2 + (tile_rel == first_tile ? 0 : 1)) * (NCLS * BM * BN) +
+                (wm * (BM / 2) + 4 * lhalf) * BN + wn * 32 + (lane & 31);
+#pragma unroll
+    for (int cl = 0; cl < NCLS; ++cl)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) ps[(cl * BM + i * 32 + 8 * (v >> 2) + (v & 3)) * BN] = acc[cl * TM + i][v];
+  } else if (pix < a.total_pix) {
     if (S2) {
       typedef float v2f __attribute__((ext_vector_type(2)));
-      float *o = a.dx + size_t(blockIdx.z) * a.split_stride + size_t(pn) * a.C * HW + (2 * ph_) * a.W + 2 * pw_;
+      float *o = a.dx + size_t(pn) * a.C * HW + (2 * ph_) * a.W + 2 * pw_;
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+          const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * lhalf + (v & 3);
           if (c < a.C) {
+            const float bb = a.bias ? a.bias[c] : 0.f;
             float *oc = o + size_t(c) * HW;
-            *reinterpret_cast<v2f *>(oc) = v2f{acc[0 * TM + i][v], acc[1 * TM + i][v]};
-            *reinterpret_cast<v2f *>(oc + a.W) = v2f{acc[2 * TM + i][v], acc[3 * TM + i][v]};
+            *reinterpret_cast<v2f *>(oc) = v2f{acc[0 * TM + i][v] + bb, acc[1 * TM + i][v] + bb};
+            *reinterpret_cast<v2f *>(oc + a.W) = v2f{acc[2 * TM + i][v] + bb, acc[3 * TM + i][v] + bb};
           }
         }
     } else {
-      float *o = a.dx + size_t(blockIdx.z) * a.split_stride + size_t(pn) * a.C * HW + prem;
+      float *o = a.dx + size_t(pn) * a.C * HW + prem;
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+          const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * lhalf + (v & 3);
           if (c < a.C) o[size_t(c) * HW] = a.bias ? acc[i][v] + a.bias[c] : acc[i][v];
         }
     }
   }
+  }  // next segment (the last tap step ended with a barrier: the LDS buffers are free)
 }
 
-// out[i] = sum over slices (ascending) of part[z][i] (+ bias of element i's channel)
-__global__ __launch_bounds__(256) void k_dgrad3x3_reduce(const float *__restrict__ part, float *__restrict__ out, long n4,
-                                                        int splits, const float *__restrict__ bias, int HW, int C) {
-  const long stride = long(gridDim.x) * 256;
-  const v4f *p4 = reinterpret_cast<const v4f *>(part);
-  v4f *o4 = reinterpret_cast<v4f *>(out);
-  for (long i = long(blockIdx.x) * 256 + threadIdx.x; i < n4; i += stride) {
-    v4f s = p4[i];
-    for (int z = 1; z < splits; ++z) s += p4[z * n4 + i];
-    if (bias) {
+// Finishes the tiles that several workgroups shared: tile r of the shared region covers units
+// [r * nchunks, (r + 1) * nchunks); the workgroups whose unit ranges meet it are visited in
+// ascending order (= ascending chunk order) and their partial tiles summed, so the result does
+// not depend on timing.  A tile that one workgroup computed alone was already stored by it.
+template <int BM, bool S2>
+__global__ __launch_bounds__(256) void k_dgrad3x3_fixup(D3Args a) {
+  constexpr int NCLS = S2 ? 4 : 1;
+  const int nchunks = a.KP / KC;
+  const int r = blockIdx.x;
+  const long x0 = long(r) * nchunks, x1 = x0 + nchunks - 1;
+  auto start = [&](long g) -> long { return g * a.sk_units / a.sk_wgs; };
+  auto owner = [&](long x) -> int {
+    long g = x * a.sk_wgs / a.sk_units;
+    while (g + 1 < a.sk_wgs && start(g + 1) <= x) ++g;
+    while (g > 0 && start(g) > x) --g;
+    return int(g);
+  };
+  const int g_lo = owner(x0), g_hi = owner(x1);
+  if (g_lo == g_hi) return;
+  const int tile = a.dp_tiles + r;
+  const int c0 = (tile % a.ctiles) * BM, pix0 = (tile / a.ctiles) * BN;
+  const int HW = a.H * a.W, PQ = a.P * a.Q;
+  // a block covers 8 rows of the tile, a thread 4 consecutive pixels of one row
+  typedef float v4f __attribute__((ext_vector_type(4)));
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  const int m = blockIdx.y * 8 + (threadIdx.x >> 5), col = (threadIdx.x & 31) * 4;
+  const int c = c0 + m;
+  if (c >= a.C) return;
+  v4f s[NCLS];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s[j] += bias[((4 * i + j) / HW) % C];
+  for (int cl = 0; cl < NCLS; ++cl) s[cl] = v4f{0.f, 0.f, 0.f, 0.f};
+  for (int g = g_lo; g <= g_hi; ++g) {
+    const int slot = int(start(g) / nchunks) == r ? 0 : 1;
+    const float *ps = a.partials + (size_t(g) * 2 + slot) * (NCLS * BM * BN) + m * BN + col;
+#pragma unroll
+    for (int cl = 0; cl < NCLS; ++cl) s[cl] += *reinterpret_cast<const v4f *>(ps + cl * BM * BN);
+  }
+  const float bb = a.bias ? a.bias[c] : 0.f;
+  int pix = pix0 + col;
+  int pn = pix / PQ, prem = pix - pn * PQ;
+  if (!S2 && (PQ & 3) == 0 && pix + 3 < a.total_pix) {  // the four pixels lie in one image, 16-byte aligned
+    *reinterpret_cast<v4f *>(a.dx + (size_t(pn) * a.C + c) * HW + prem) = s[0] + bb;
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j, ++pix) {
+    if (pix >= a.total_pix) break;
+    if (S2) {
+      const int i = prem / a.Q, jj = prem - i * a.Q;
+      float *o = a.dx + (size_t(pn) * a.C + c) * HW + (2 * i) * a.W + 2 * jj;
+      *reinterpret_cast<v2f *>(o) = v2f{s[0][j] + bb, s[NCLS > 1 ? 1 : 0][j] + bb};
+      *reinterpret_cast<v2f *>(o + a.W) = v2f{s[NCLS > 2 ? 2 : 0][j] + bb, s[NCLS > 3 ? 3 : 0][j] + bb};
+    } else {
+      a.dx[(size_t(pn) * a.C + c) * HW + prem] = s[0][j] + bb;
     }
-    o4[i] = s;
+    if (++prem == PQ) prem = 0, ++pn;
   }
 }
 
 struct D3Plan {
   bool ok, s2;
-  int bm, logp, vr, splits, chunks_per_split;
+  int bm, logp, vr;
+  int ctiles, tiles, dp_tiles, sk_wgs;  // whole-tile workgroups, then sk_wgs workgroups sharing the rest
+  long sk_units;
   size_t lds;
 };
 
@@ -301,20 +387,20 @@ inline D3Plan plan(const sgh_conv_geom *g) {
   const size_t dx_elems = size_t(g->N) * g->C * g->H * g->W;
   if (size_t(g->N) * g->K * g->P * g->Q * 4 >= lim || dx_elems * 4 >= lim) return p;
   if (size_t(g->N) * (g->P + 2) + p.vr >= lim / 64) return p;
-  // split the reduction when the tile grid cannot fill the chip (one workgroup per CU fits);
-  // the partial images are summed in slice order, so results stay run-to-run identical
-  const long tiles = long((g->C + p.bm - 1) / p.bm) * ((long(g->N) * g->P * g->Q + BN - 1) / BN);
+  // Work balance.  Whole multiples of the CU count of tiles run one tile per workgroup; the
+  // remaining tiles (all of them when there are fewer tiles than CUs) are cut into (tile, chunk)
+  // units and dealt evenly to one workgroup per CU (two per CU measured slower: twice the
+  // partial tiles to write and sum), so that no CU is left with a whole extra tile while others idle.  Tiles shared between workgroups are finished by
+  // k_dgrad3x3_fixup in a fixed order: results stay run-to-run identical.
+  const int cus = sgh_num_cus();
   const int nchunks = (g->K + KC - 1) / KC;
-  // (three quarters of the CUs busy with unsplit work beats a full chip that also has to write,
-  // re-read and sum partial images)
-  long s = (3L * sgh_num_cus() / 4 + tiles - 1) / tiles;
-  if (s > nchunks / 4) s = nchunks / 4;
-  if (s > 8) s = 8;
-  if (s < 1) s = 1;
-  if (dx_elems % 4 != 0) s = 1;
-  if (const char *e = getenv("SGH_DGRAD3X3_SPLITS")) s = atoi(e) > 0 ? atoi(e) : s;
-  p.chunks_per_split = int((nchunks + s - 1) / s);
-  p.splits = (nchunks + p.chunks_per_split - 1) / p.chunks_per_split;
+  p.ctiles = (g->C + p.bm - 1) / p.bm;
+  const long tiles = long(p.ctiles) * ((long(g->N) * g->P * g->Q + BN - 1) / BN);
+  if (tiles >= (long(1) << 30)) return p;
+  p.tiles = int(tiles);
+  p.dp_tiles = int(tiles / cus * cus);
+  p.sk_units = long(p.tiles - p.dp_tiles) * nchunks;
+  p.sk_wgs = int(p.sk_units < cus ? p.sk_units : cus);
   p.ok = true;
   return p;
 }
@@ -340,8 +426,8 @@ bool sgh_dgrad3x3_supported(const sgh_conv_geom *g) { return plan(g).ok; }
 // Extra workspace (bytes, after the re-laid weights) for split-reduction partial images.
 size_t sgh_dgrad3x3_partial_bytes(const sgh_conv_geom *g) {
   const D3Plan p = plan(g);
-  if (!p.ok || p.splits <= 1) return 0;
-  return size_t(p.splits) * g->N * g->C * g->H * g->W * sizeof(float);
+  if (!p.ok || p.sk_wgs == 0) return 0;
+  return size_t(p.sk_wgs) * 2 * (p.s2 ? 4 : 1) * p.bm * BN * sizeof(float);
 }
 
 // `wt` holds the weights re-laid as [tap][KP][C] (KP = K rounded up to 16, zero rows beyond K);
@@ -350,12 +436,12 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
                      hipStream_t s, const char *tag, const float *bias) {
   const D3Plan p = plan(g);
   if (!p.ok) return SGH_EUNSUPPORTED;
-  if (p.splits > 1 && !partials) return SGH_EWORKSPACE;
+  if (p.sk_wgs > 0 && !partials) return SGH_EWORKSPACE;
   D3Args a;
   a.dy = dy;
   a.wt = wt;
-  a.dx = p.splits > 1 ? partials : dx;
-  a.bias = p.splits > 1 ? nullptr : bias;  // with split reduction the bias is added by the reduction kernel
+  a.bias = bias;
+  a.dx = dx;
   a.N = g->N;
   a.C = g->C;
   a.H = g->H;
@@ -365,12 +451,14 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   a.P = g->P;
   a.Q = g->Q;
   a.total_pix = g->N * g->P * g->Q;
-  a.chunks_per_split = p.chunks_per_split;
-  a.split_stride = long(g->N) * g->C * g->H * g->W;
+  a.ctiles = p.ctiles;
+  a.dp_tiles = p.dp_tiles;
+  a.sk_wgs = p.sk_wgs;
+  a.sk_units = p.sk_units;
+  a.partials = partials;
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 4);
   a.wt_bytes = unsigned(size_t(9) * KP * g->C * 4);
-  dim3 grid((g->C + p.bm - 1) / p.bm, (a.total_pix + BN - 1) / BN, p.splits);
-  if (grid.y > 65535u) return SGH_EUNSUPPORTED;
+  dim3 grid(unsigned(p.dp_tiles + p.sk_wgs), 1, 1);
   int rc = SGH_EUNSUPPORTED;
   sgh_prof_start(tag, 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
 #define D3_CASE(BM_, LOGP_, VR_) \
@@ -392,13 +480,12 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
 #undef D3_CASE_S2
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
-  if (p.splits > 1) {
-    const long n4 = a.split_stride / 4;
-    long blocks = (n4 + 255) / 256;
-    const long cap = long(sgh_num_cus()) * 16;
-    if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL(k_dgrad3x3_reduce, dim3(int(blocks)), dim3(256), 0, s, partials, dx, n4, p.splits, bias,
-                       g->H * g->W, g->C);
+  if (p.sk_wgs > 0) {
+    const int shared_tiles = p.tiles - p.dp_tiles;
+    const dim3 fgrid(shared_tiles, p.bm / 8);
+    if (p.s2) hipLaunchKernelGGL((k_dgrad3x3_fixup<64, true>), fgrid, dim3(256), 0, s, a);
+    else if (p.bm == 64) hipLaunchKernelGGL((k_dgrad3x3_fixup<64, false>), fgrid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((k_dgrad3x3_fixup<128, false>), fgrid, dim3(256), 0, s, a);
     if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
   }
   return SGH_OK;

@@ -126,6 +126,27 @@ def test_conv_wgrad_is_deterministic(singa, dev):
         assert_bit_equal(singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy(), a, "split-K reduction order")
 
 
+@pytest.mark.parametrize("n,c,hw,k,stride", [
+    (40, 64, 56, 64, 1),     # 980 tiles: three whole rounds of tiles plus a shared remainder
+    (16, 256, 14, 256, 1),   # fewer tiles than CUs: every tile is shared between workgroups
+    (16, 64, 28, 128, 2),    # residue-class kernel, four partial classes per shared tile
+])
+def test_conv_dgrad_is_deterministic(singa, dev, n, c, hw, k, stride):
+    """Tiles shared between workgroups are summed in a fixed order: repeated runs agree bit for bit,
+    and one image of the batch agrees with the oracle."""
+    r = rng(11)
+    p = hw // stride
+    x, dy = randn(r, n, c, hw, hw), randn(r, n, k, p, p)
+    w = randn(r, k, c, 3, 3)
+    xd, wd, dyd = singa.from_numpy(x, dev), singa.from_numpy(w, dev), singa.from_numpy(dy, dev)
+    h = singa.CudnnConvHandle(xd, (3, 3), (stride, stride), (1, 1), c, k, False)
+    a = singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy()
+    for _ in range(3):
+        assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), a, "shared-tile summation order")
+    dx_o, _ = O.conv_bwd(dy[-1:], x[-1:], w, (stride, stride), (1, 1), want_dw=False)
+    assert nl2(a[-1:], dx_o) < TOL
+
+
 @pytest.mark.parametrize("shape", [
     (64, 64, 56, 64, 3, 1, 1),     # BASELINE single-conv configuration
     (64, 3, 224, 64, 7, 2, 3),     # ResNet stem: few-channel wgrad / direct dgrad kernels
