@@ -64,6 +64,15 @@ size_t sgh_dgrad_fewc_workspace_bytes(const sgh_conv_geom *g);
 int sgh_dgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
                        size_t ws_bytes, hipStream_t s);
 
+// Convolution gradients on 16-bit tensors with the 16-bit matrix instructions (conv16.hip).
+// *_workspace_bytes is 0 and the run functions return SGH_EUNSUPPORTED for geometries they do not
+// cover (strides above 2, K not a multiple of 8 for the data gradient, tensors of 2^31 elements).
+size_t sgh_conv16_workspace_bytes(const sgh_conv_geom *g, int which);
+int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x, uint16_t *dW, void *workspace,
+                     size_t ws_bytes, bool bf16, hipStream_t s);
+int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
+                     size_t ws_bytes, bool bf16, hipStream_t s);
+
 // Sum across the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float sgh_wave_sum(float v) {
 #pragma unroll

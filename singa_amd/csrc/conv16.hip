@@ -1,0 +1,606 @@
+// Convolution gradients on 16-bit tensors (IEEE binary16 / bfloat16, NCHW) with the 16-bit matrix
+// instructions of gfx950: v_mfma_f32_32x32x16_{f16,bf16}, fp32 accumulation, one rounding at the
+// store.  Reference entry points: ConvBackwardx / ConvBackwardW, src/model/operation/convolution.cc
+// :634-681 (cuDNN with half tensors); formulas as in igemm.hip.
+//
+// Both MFMA operands hold, per lane, EIGHT CONSECUTIVE reduction indices of one tile row (lane l:
+// row l % 32, indices 8 * (l / 32) .. + 7), so both LDS tiles are kept as [row][reduction] with the
+// reduction index contiguous (pitch 64 + 8 halves: ds_read_b128, conflict-free).  Which eight
+// indices share an octet is irrelevant as long as both operands agree, which is what makes NCHW
+// usable without a layout change:
+//
+//   weight gradient  dW[k][(c,r,s)] = sum_{n,p,q} dy[n,k,p,q] * x[n,c,p*st-pad+r,q*st-pad+s]
+//     The reduction runs over pixels, contiguous in memory for both operands.  An octet is 8
+//     consecutive q of one output row (the last octet of a row is partly empty: at most 12.5 % of
+//     the MFMA work for Q = 7, 14, 28, none for 56 and 112); 1x1 stride-1 layers are passed in with
+//     the image plane as one row.  dy octets are 16-byte loads; an x octet is the 16 (stride 2: 32)
+//     bytes at the tap's offset, loaded unaligned and masked at the image border.
+//   data gradient    dx[c][(n,h,w)]  = sum_{r,s,k} W[k,c,r,s] * dy[n,k,(h+pad-r)/st,(w+pad-s)/st]
+//     The reduction runs over k, strided in memory, while pixels are contiguous: a thread loads one
+//     dword (two neighbouring pixels) for each of 8 consecutive k and transposes them into two
+//     octets with v_perm_b32 (the selector also encodes which of the two pixels exist for the
+//     tap, so border handling costs nothing extra).  Weights are re-laid as [tap][C][K] in 16 bits.
+//     Stride 2 is handled by residue class: output pixels (2i+a, 2j+b) of one class form their own
+//     pixel space with a stride-1 gradient window, and only the taps of that class are visited.
+//
+// 256 threads = 2 x 2 wavefronts, workgroup tile 128 (or 64) x 128, reduction chunk 64, LDS and
+// register double buffering.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "storage.h"
+
+namespace {
+
+constexpr int NT = 256, BN = 128, KC = 64, PITCH = KC + 8;  // PITCH in 16-bit elements
+constexpr int kOOB = int(0x80000000u);
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, int(bytes), 0x00020000);
+}
+
+template <bool BF16>
+__device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0,
+                                                   0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
+                                                  0);
+}
+
+template <bool BF16>
+__device__ __forceinline__ uint16_t round16(float v) {
+  return BF16 ? sgh_f32_to_bf16(v) : sgh_f32_to_f16(v);
+}
+
+// keeps elements j in [lo, hi) of an octet, zeroes the others
+__device__ __forceinline__ u32x4 mask_range(u32x4 v, int lo, int hi) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const unsigned m = ((2 * d >= lo && 2 * d < hi) ? 0xffffu : 0u) | ((2 * d + 1 >= lo && 2 * d + 1 < hi) ? 0xffff0000u : 0u);
+    v[d] &= m;
+  }
+  return v;
+}
+
+// element-wise guarded load of elements j in [lo, hi) at p[off + j * STEP]
+template <int STEP>
+__device__ __forceinline__ u32x4 load_elems(const uint16_t *p, long off, int lo, int hi) {
+  u32x4 v = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if (j >= lo && j < hi) v[j >> 1] |= unsigned(p[off + long(j) * STEP]) << (16 * (j & 1));
+  return v;
+}
+
+__device__ __forceinline__ u32x4 load16b(const uint16_t *p) {  // 16 bytes at any 2-byte alignment
+  u32x4 v;
+  __builtin_memcpy(&v, p, 16);
+  return v;
+}
+
+// One reduction chunk (64 indices = four MFMA steps) of a wavefront's (TM*32) x 64 tile.
+template <int TM, bool BF16>
+__device__ __forceinline__ void mma_chunk(const uint16_t *As, const uint16_t *Bs, int arow, int brow, int lh,
+                                          f32x16 (&acc)[TM][2]) {
+#pragma unroll
+  for (int j = 0; j < KC / 16; ++j) {
+    u32x4 av[TM], bv[2];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) av[i] = *reinterpret_cast<const u32x4 *>(As + (arow + i * 32) * PITCH + (2 * j + lh) * 8);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) bv[i] = *reinterpret_cast<const u32x4 *>(Bs + (brow + i * 32) * PITCH + (2 * j + lh) * 8);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int jn = 0; jn < 2; ++jn) acc[i][jn] = mfma<BF16>(av[i], bv[jn], acc[i][jn]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// weight gradient
+// ------------------------------------------------------------------------------------------------
+struct W16Args {
+  const uint16_t *dy, *x;
+  float *partial;  // [splits][K][CRS]
+  int N, C, H, W, K, P, Q, R, S, pad_h, pad_w;
+  int QO;          // octets per output row: ceil(Q / 8)
+  int CRS, mtiles;
+  int chunks, chunks_per_split;  // a chunk = 8 octets = 8 units (n, p, octet)
+  long dy_elems, x_elems;
+};
+
+template <int BM, int STRIDE, bool BF16>
+__global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
+  extern __shared__ __align__(16) uint16_t lds16[];
+  constexpr int TM = BM / 64, ASLOTS = BM * 8 / NT, BSLOTS = BN * 8 / NT;
+  uint16_t *const As0 = lds16, *const Bs0 = lds16 + BM * PITCH;
+  uint16_t *const As1 = lds16 + (BM + BN) * PITCH, *const Bs1 = As1 + BM * PITCH;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, lh = lane >> 5;
+  const int m0 = (int(blockIdx.x) % a.mtiles) * BM, n0 = (int(blockIdx.x) / a.mtiles) * BN;
+  const int split = blockIdx.y;
+  const int c_begin = split * a.chunks_per_split;
+  const int c_end = min(a.chunks, c_begin + a.chunks_per_split);
+  const int oct = t & 7, rb = t >> 3;
+  const int PQ = a.P * a.Q, HW = a.H * a.W, RS = a.R * a.S;
+
+  // this thread's unit (n, p, qo) in the current chunk, and the step of 8 units to the next chunk
+  const int PQO = a.P * a.QO;
+  int n, p, qo;
+  {
+    const long unit = long(c_begin) * 8 + oct;
+    n = int(unit / PQO);
+    const int rem = int(unit - long(n) * PQO);
+    p = rem / a.QO;
+    qo = rem - p * a.QO;
+  }
+  const int dn = 8 / PQO, dp = (8 - dn * PQO) / a.QO, dq = 8 - dn * PQO - dp * a.QO;
+  auto advance = [&]() {
+    qo += dq;
+    if (qo >= a.QO) qo -= a.QO, ++p;
+    p += dp;
+    if (p >= a.P) p -= a.P, ++n;
+    n += dn;
+  };
+
+  int aoff[ASLOTS];
+  bool aok[ASLOTS];
+#pragma unroll
+  for (int i = 0; i < ASLOTS; ++i) {
+    const int k = m0 + rb + 32 * i;
+    aok[i] = k < a.K;
+    aoff[i] = k * PQ;
+  }
+  int bconst[BSLOTS], br[BSLOTS], bs[BSLOTS];
+  bool bok[BSLOTS];
+#pragma unroll
+  for (int i = 0; i < BSLOTS; ++i) {
+    const int col = n0 + rb + 32 * i;
+    bok[i] = col < a.CRS;
+    const int c = col / RS, tap = col - c * RS, r = tap / a.S;
+    br[i] = r - a.pad_h;
+    bs[i] = tap - r * a.S - a.pad_w;
+    bconst[i] = c * HW;
+  }
+
+  u32x4 ra[ASLOTS], rbv[BSLOTS];
+  auto load = [&]() {
+    const int nv = min(8, a.Q - 8 * qo);
+    const bool unit_ok = n < a.N;
+    const long abase = long(n) * a.K * PQ + p * a.Q + 8 * qo;
+#pragma unroll
+    for (int i = 0; i < ASLOTS; ++i) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (unit_ok && aok[i]) {
+        const long off = abase + aoff[i];
+        if (off + 8 <= a.dy_elems) {
+          v = load16b(a.dy + off);
+          if (nv < 8) v = mask_range(v, 0, nv);
+        } else {
+          v = load_elems<1>(a.dy, off, 0, nv);
+        }
+      }
+      ra[i] = v;
+    }
+    const long xbase = long(n) * a.C * HW;
+#pragma unroll
+    for (int i = 0; i < BSLOTS; ++i) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      const int h = p * STRIDE + br[i], col0 = 8 * STRIDE * qo + bs[i];
+      const int lo = col0 < 0 ? (-col0 + STRIDE - 1) / STRIDE : 0;
+      const int hi = min(nv, (a.W - col0 + STRIDE - 1) / STRIDE);
+      if (unit_ok && bok[i] && h >= 0 && h < a.H && hi > lo) {
+        const long off = xbase + bconst[i] + h * a.W + col0;
+        if (off >= 0 && off + 8 * STRIDE <= a.x_elems) {
+          if (STRIDE == 1) {
+            v = load16b(a.x + off);
+          } else {  // 16 elements, every other one wanted
+            const u32x4 v0 = load16b(a.x + off), v1 = load16b(a.x + off + 8);
+            v[0] = __builtin_amdgcn_perm(v0[1], v0[0], 0x05040100u);
+            v[1] = __builtin_amdgcn_perm(v0[3], v0[2], 0x05040100u);
+            v[2] = __builtin_amdgcn_perm(v1[1], v1[0], 0x05040100u);
+            v[3] = __builtin_amdgcn_perm(v1[3], v1[2], 0x05040100u);
+          }
+          if (lo > 0 || hi < 8) v = mask_range(v, lo, hi);
+        } else {
+          v = load_elems<STRIDE>(a.x, off, lo, hi);
+        }
+      }
+      rbv[i] = v;
+    }
+    advance();
+  };
+  auto stage = [&](uint16_t *As, uint16_t *Bs) {
+#pragma unroll
+    for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 32 * i) * PITCH + oct * 8) = ra[i];
+#pragma unroll
+    for (int i = 0; i < BSLOTS; ++i) *reinterpret_cast<u32x4 *>(Bs + (rb + 32 * i) * PITCH + oct * 8) = rbv[i];
+  };
+
+  f32x16 acc[TM][2];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  if (c_begin < c_end) {
+    load();
+    stage(As0, Bs0);
+    __syncthreads();
+    for (int c = c_begin; c < c_end; ++c) {
+      const bool cur1 = (c - c_begin) & 1, more = c + 1 < c_end;
+      if (more) load();
+      mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, wm * (TM * 32) + l32, wn * 64 + l32, lh, acc);
+      if (more) stage(cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
+      __syncthreads();
+    }
+  }
+
+  float *out = a.partial + size_t(split) * a.K * a.CRS;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int jn = 0; jn < 2; ++jn) {
+      const int col = n0 + wn * 64 + jn * 32 + l32;
+      if (col >= a.CRS) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+        if (row < a.K) out[size_t(row) * a.CRS + col] = acc[i][jn][v];
+      }
+    }
+}
+
+// dW = round16(sum over splits, ascending): run-to-run identical
+template <bool BF16>
+__global__ __launch_bounds__(256) void k_wgrad16_reduce(const float *partial, int splits, size_t n, uint16_t *dW) {
+  const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int z = 0; z < splits; ++z) s += partial[size_t(z) * n + i];
+  dW[i] = round16<BF16>(s);
+}
+
+// ------------------------------------------------------------------------------------------------
+// data gradient
+// ------------------------------------------------------------------------------------------------
+struct D16Args {
+  const uint16_t *dy, *wt;  // wt: [tap][CP][KP], zero-filled padding
+  uint16_t *dx;
+  int N, C, H, W, K, P, Q, R, S, stride, pad_h, pad_w;
+  int KP, CP, mtiles;
+  int cls_tile0[5];  // first pixel tile of each residue class (stride^2 classes), then the total
+  unsigned dy_bytes;
+};
+
+constexpr unsigned kSelLo = 0x05040100u, kSelHi = 0x07060302u, kSelZero = 0x0c0c0c0cu;
+
+template <int BM, bool BF16>
+__global__ __launch_bounds__(NT) void k_dgrad16(D16Args a) {
+  extern __shared__ __align__(16) uint16_t lds16[];
+  constexpr int TM = BM / 64, ASLOTS = BM * 8 / NT;
+  uint16_t *const As0 = lds16, *const Bs0 = lds16 + BM * PITCH;
+  uint16_t *const As1 = lds16 + (BM + BN) * PITCH, *const Bs1 = As1 + BM * PITCH;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lh = lane >> 5;
+  const int m0 = (int(blockIdx.x) % a.mtiles) * BM, pt = int(blockIdx.x) / a.mtiles;
+  const int st = a.stride, PQ = a.P * a.Q, HW = a.H * a.W;
+  int cls = 0;
+  while (pt >= a.cls_tile0[cls + 1]) ++cls;
+  const int ca = cls / st, cb = cls - ca * st;
+  // the class's pixel space: rows are padded to an even width so that a pixel pair never
+  // straddles two rows (an odd width costs one dummy pixel per row)
+  const int Hc = (a.H - ca + st - 1) / st, Wreal = (a.W - cb + st - 1) / st, Wc = (Wreal + 1) & ~1, HWc = Hc * Wc;
+  const long cnt = long(a.N) * HWc;
+  const long pix0 = long(pt - a.cls_tile0[cls]) * BN;
+  const rsrc_t rdy = make_rsrc(a.dy, a.dy_bytes);
+
+  // B loader: pixel pair pp of the tile, k octets kq and kq + 4 of the chunk
+  const int pp = lane, kq = wave;
+  const long pixA = pix0 + 2 * pp, pixB = pixA + 1;
+  const int nA = int(pixA / HWc), remA = int(pixA - long(nA) * HWc), iA = remA / Wc, jA = remA - iA * Wc;
+  int voff = kOOB;  // byte offset of the dword holding both pixels (kOOB: neither exists)
+  unsigned selA = kSelZero, selB = kSelZero;
+  auto set_tap = [&](int tap) {
+    const int r = tap / a.S, s = tap - r * a.S;
+    const int dr = (ca + a.pad_h - r) / st, ds = (cb + a.pad_w - s) / st;  // exact for the taps of this class
+    const int p = iA + dr, q0 = jA + ds;
+    const bool row = p >= 0 && p < a.P;
+    const bool memA = row && q0 >= 0 && q0 < a.Q, memB = row && q0 + 1 >= 0 && q0 + 1 < a.Q;
+    const int base = ((nA * a.K) * a.P + p) * a.Q + q0;
+    bool hiA = false, loB = false;
+    if (memA && memB) voff = base * 2;
+    else if (memA) voff = (base - 1) * 2, hiA = true;   // pixel A sits in the high half
+    else if (memB) voff = (base + 1) * 2, loB = true;   // pixel B sits in the low half
+    else voff = kOOB;
+    selA = (memA && pixA < cnt) ? (hiA ? kSelHi : kSelLo) : kSelZero;
+    selB = (memB && pixB < cnt && jA + 1 < Wreal) ? (loB ? kSelLo : kSelHi) : kSelZero;
+  };
+  auto tap_in_class = [&](int tap) {
+    const int r = tap / a.S, s = tap - r * a.S;
+    return (ca + a.pad_h - r) % st == 0 && (cb + a.pad_w - s) % st == 0;
+  };
+  const int RS = a.R * a.S, nkc = a.KP / KC;
+  auto next_tap = [&](int tap) {
+    while (tap < RS && !tap_in_class(tap)) ++tap;
+    return tap;
+  };
+
+  const int oct = t & 7, rb = t >> 3;
+  u32x4 ra[ASLOTS];
+  unsigned rd[2][8];   // the pair's dword for 8 consecutive k
+  auto load = [&](int tap, int kc) {
+#pragma unroll
+    for (int i = 0; i < ASLOTS; ++i)
+      ra[i] = *reinterpret_cast<const u32x4 *>(a.wt + (size_t(tap) * a.CP + m0 + rb + 32 * i) * a.KP + kc * KC + oct * 8);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int kb = kc * KC + (kq + 4 * i) * 8;
+      if (kb < a.K) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          rd[i][j] = unsigned(__builtin_amdgcn_raw_buffer_load_b32(rdy, voff, (kb + j) * PQ * 2, 0));
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) rd[i][j] = 0u;
+      }
+    }
+  };
+  auto stage = [&](uint16_t *As, uint16_t *Bs) {
+#pragma unroll
+    for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 32 * i) * PITCH + oct * 8) = ra[i];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      u32x4 vA, vB;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        vA[d] = __builtin_amdgcn_perm(rd[i][2 * d + 1], rd[i][2 * d], selA);
+        vB[d] = __builtin_amdgcn_perm(rd[i][2 * d + 1], rd[i][2 * d], selB);
+      }
+      *reinterpret_cast<u32x4 *>(Bs + (2 * pp) * PITCH + (kq + 4 * i) * 8) = vA;
+      *reinterpret_cast<u32x4 *>(Bs + (2 * pp + 1) * PITCH + (kq + 4 * i) * 8) = vB;
+    }
+  };
+
+  f32x16 acc[TM][2];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  int tap = next_tap(0), kc = 0;
+  if (tap < RS) {
+    set_tap(tap);
+    load(tap, kc);
+    stage(As0, Bs0);
+    __syncthreads();
+    bool cur1 = false;
+    while (true) {
+      int ntap = tap, nk = kc + 1;
+      if (nk == nkc) nk = 0, ntap = next_tap(tap + 1);
+      const bool more = ntap < RS;
+      if (more) {
+        if (ntap != tap) set_tap(ntap);   // the staged registers were already packed with the old selectors
+        load(ntap, nk);
+      }
+      mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, wm * (TM * 32) + l32, wn * 64 + l32, lh, acc);
+      if (!more) break;
+      stage(cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
+      __syncthreads();
+      cur1 = !cur1;
+      tap = ntap;
+      kc = nk;
+    }
+  }
+
+  // epilogue: lane's pixel column, 16 channel rows per accumulator
+#pragma unroll
+  for (int jn = 0; jn < 2; ++jn) {
+    const long pix = pix0 + wn * 64 + jn * 32 + l32;
+    if (pix >= cnt) continue;
+    const int n = int(pix / HWc), rem = int(pix - long(n) * HWc), i_ = rem / Wc, j_ = rem - i_ * Wc;
+    if (j_ >= Wreal) continue;
+    uint16_t *o = a.dx + (size_t(n) * a.C) * HW + (st * i_ + ca) * a.W + st * j_ + cb;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int c = m0 + wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+        if (c < a.C) o[size_t(c) * HW] = round16<BF16>(acc[i][jn][v]);
+      }
+  }
+}
+
+// wt[tap][c][k] (c < CP, k < KP; zero beyond C / K) from W[k][c][r][s]
+__global__ __launch_bounds__(256) void k_relayout16(const uint16_t *W, uint16_t *wt, int K, int C, int RS, int KP, int CP) {
+  const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x, n = size_t(RS) * CP * KP;
+  if (i >= n) return;
+  const int k = int(i % KP), c = int((i / KP) % CP), tap = int(i / (size_t(KP) * CP));
+  wt[i] = (k < K && c < C) ? W[(size_t(k) * C + c) * RS + tap] : uint16_t(0);
+}
+
+inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+
+constexpr size_t kLds128 = size_t(2) * (128 + BN) * PITCH * 2, kLds64 = size_t(2) * (64 + BN) * PITCH * 2;
+
+template <typename Kern>
+bool allow_lds(Kern kern, size_t bytes) {
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             int(bytes)) == hipSuccess;
+}
+
+struct W16Plan {
+  bool ok;
+  int bm, stride, mtiles, ntiles, chunks, splits, cps;
+  sgh_conv_geom f;  // the geometry the kernel sees (1x1 stride-1 layers: image plane as one row)
+  int QO;
+};
+
+W16Plan wplan(const sgh_conv_geom *g) {
+  W16Plan p{};
+  if (g->stride_h != g->stride_w || (g->stride_h != 1 && g->stride_h != 2)) return p;
+  const size_t lim = size_t(1) << 31;
+  const size_t xe = size_t(g->N) * g->C * g->H * g->W, ye = size_t(g->N) * g->K * g->P * g->Q;
+  if (xe >= lim || ye >= lim || size_t(g->K) * g->C * g->R * g->S >= lim) return p;
+  p.f = *g;
+  if (g->R == 1 && g->S == 1 && g->stride_h == 1 && g->pad_h == 0 && g->pad_w == 0) {
+    p.f.H = 1, p.f.W = g->H * g->W, p.f.P = 1, p.f.Q = g->P * g->Q;
+  }
+  p.stride = g->stride_h;
+  p.bm = g->K <= 64 ? 64 : 128;
+  p.mtiles = (g->K + p.bm - 1) / p.bm;
+  p.ntiles = (g->C * g->R * g->S + BN - 1) / BN;
+  p.QO = (p.f.Q + 7) / 8;
+  const long units = long(p.f.N) * p.f.P * p.QO;
+  p.chunks = int((units + 7) / 8);
+  // enough splits of the reduction for two workgroups per CU, at least 4 chunks each
+  const int tiles = p.mtiles * p.ntiles, want = (2 * sgh_num_cus() + tiles - 1) / tiles;
+  int splits = want < 1 ? 1 : want;
+  if (splits > (p.chunks + 3) / 4) splits = (p.chunks + 3) / 4;
+  if (splits < 1) splits = 1;
+  p.cps = (p.chunks + splits - 1) / splits;
+  p.splits = (p.chunks + p.cps - 1) / p.cps;
+  if (p.splits < 1) p.splits = 1;
+  p.ok = true;
+  return p;
+}
+
+struct D16Plan {
+  bool ok;
+  int bm, mtiles, KP, CP, tiles;
+  int cls_tile0[5];
+};
+
+D16Plan dplan(const sgh_conv_geom *g) {
+  D16Plan p{};
+  const int st = g->stride_h;
+  if (g->stride_h != g->stride_w || (st != 1 && st != 2)) return p;
+  if (g->K % 8 != 0 || g->Q < 2 || g->C < 16) return p;  // (a 64-row tile is mostly empty below 16 channels)
+  const size_t lim = size_t(1) << 30;  // byte offsets of dy stay below 2^31
+  if (size_t(g->N) * g->K * g->P * g->Q >= lim || size_t(g->N) * g->C * g->H * g->W >= 2 * lim) return p;
+  p.bm = g->C <= 64 ? 64 : 128;
+  p.mtiles = (g->C + p.bm - 1) / p.bm;
+  p.CP = p.mtiles * p.bm;
+  p.KP = (g->K + KC - 1) / KC * KC;
+  long tiles = 0;
+  for (int cls = 0; cls < st * st; ++cls) {
+    const int ca = cls / st, cb = cls % st;
+    const int Hc = (g->H - ca + st - 1) / st, Wc = ((g->W - cb + st - 1) / st + 1) & ~1;  // rows padded to even
+    p.cls_tile0[cls] = int(tiles);
+    tiles += (long(g->N) * Hc * Wc + BN - 1) / BN;
+  }
+  for (int cls = st * st; cls < 5; ++cls) p.cls_tile0[cls] = int(tiles);
+  if (tiles * p.mtiles >= (long(1) << 30)) return p;
+  p.tiles = int(tiles);
+  p.ok = true;
+  return p;
+}
+
+template <int BM, int STRIDE, bool BF16>
+int launch_w(const W16Args &a, const W16Plan &p, hipStream_t s) {
+  auto kern = k_wgrad16<BM, STRIDE, BF16>;
+  const size_t lds = BM == 128 ? kLds128 : kLds64;
+  static bool attr = false;
+  if (!attr) {
+    if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
+    attr = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(p.mtiles * p.ntiles, p.splits), dim3(NT), lds, s, a);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
+template <int BM, bool BF16>
+int launch_d(const D16Args &a, const D16Plan &p, hipStream_t s) {
+  auto kern = k_dgrad16<BM, BF16>;
+  const size_t lds = BM == 128 ? kLds128 : kLds64;
+  static bool attr = false;
+  if (!attr) {
+    if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
+    attr = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(p.tiles * p.mtiles), dim3(NT), lds, s, a);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
+}  // namespace
+
+size_t sgh_conv16_workspace_bytes(const sgh_conv_geom *g, int which) {
+  if (which == SGH_CONV_WGRAD) {
+    const W16Plan p = wplan(g);
+    return p.ok ? align256(size_t(p.splits) * g->K * g->C * g->R * g->S * sizeof(float)) : 0;
+  }
+  if (which == SGH_CONV_DGRAD) {
+    const D16Plan p = dplan(g);
+    return p.ok ? align256(size_t(g->R) * g->S * p.CP * p.KP * sizeof(uint16_t)) : 0;
+  }
+  return 0;
+}
+
+int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x, uint16_t *dW, void *workspace,
+                     size_t ws_bytes, bool bf16, hipStream_t s) {
+  const W16Plan p = wplan(g);
+  if (!p.ok) return SGH_EUNSUPPORTED;
+  if (!workspace || ws_bytes < sgh_conv16_workspace_bytes(g, SGH_CONV_WGRAD)) return SGH_EWORKSPACE;
+  W16Args a{};
+  a.dy = dy, a.x = x, a.partial = static_cast<float *>(workspace);
+  a.N = p.f.N, a.C = p.f.C, a.H = p.f.H, a.W = p.f.W, a.K = p.f.K, a.P = p.f.P, a.Q = p.f.Q;
+  a.R = p.f.R, a.S = p.f.S, a.pad_h = p.f.pad_h, a.pad_w = p.f.pad_w;
+  a.QO = p.QO, a.CRS = g->C * g->R * g->S, a.mtiles = p.mtiles;
+  a.chunks = p.chunks, a.chunks_per_split = p.cps;
+  a.dy_elems = long(g->N) * g->K * g->P * g->Q, a.x_elems = long(g->N) * g->C * g->H * g->W;
+  const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
+  sgh_prof_start("conv_wgrad16", flops, s);
+  int rc;
+  if (p.bm == 128) {
+    if (p.stride == 1) rc = bf16 ? launch_w<128, 1, true>(a, p, s) : launch_w<128, 1, false>(a, p, s);
+    else rc = bf16 ? launch_w<128, 2, true>(a, p, s) : launch_w<128, 2, false>(a, p, s);
+  } else {
+    if (p.stride == 1) rc = bf16 ? launch_w<64, 1, true>(a, p, s) : launch_w<64, 1, false>(a, p, s);
+    else rc = bf16 ? launch_w<64, 2, true>(a, p, s) : launch_w<64, 2, false>(a, p, s);
+  }
+  sgh_prof_stop(s);
+  if (rc != SGH_OK) return rc;
+  const size_t n = size_t(g->K) * a.CRS;
+  if (bf16) hipLaunchKernelGGL(k_wgrad16_reduce<true>, dim3(unsigned((n + 255) / 256)), dim3(256), 0, s, a.partial, p.splits, n, dW);
+  else hipLaunchKernelGGL(k_wgrad16_reduce<false>, dim3(unsigned((n + 255) / 256)), dim3(256), 0, s, a.partial, p.splits, n, dW);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
+int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
+                     size_t ws_bytes, bool bf16, hipStream_t s) {
+  const D16Plan p = dplan(g);
+  if (!p.ok) return SGH_EUNSUPPORTED;
+  if (!workspace || ws_bytes < sgh_conv16_workspace_bytes(g, SGH_CONV_DGRAD)) return SGH_EWORKSPACE;
+  uint16_t *wt = static_cast<uint16_t *>(workspace);
+  const int RS = g->R * g->S;
+  const size_t nw = size_t(RS) * p.CP * p.KP;
+  hipLaunchKernelGGL(k_relayout16, dim3(unsigned((nw + 255) / 256)), dim3(256), 0, s, W, wt, g->K, g->C, RS, p.KP, p.CP);
+  if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
+  D16Args a{};
+  a.dy = dy, a.wt = wt, a.dx = dx;
+  a.N = g->N, a.C = g->C, a.H = g->H, a.W = g->W, a.K = g->K, a.P = g->P, a.Q = g->Q, a.R = g->R, a.S = g->S;
+  a.stride = g->stride_h, a.pad_h = g->pad_h, a.pad_w = g->pad_w;
+  a.KP = p.KP, a.CP = p.CP, a.mtiles = p.mtiles;
+  for (int i = 0; i < 5; ++i) a.cls_tile0[i] = p.cls_tile0[i];
+  a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2);
+  const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
+  sgh_prof_start("conv_dgrad16", flops, s);
+  int rc;
+  if (p.bm == 128) rc = bf16 ? launch_d<128, true>(a, p, s) : launch_d<128, false>(a, p, s);
+  else rc = bf16 ? launch_d<64, true>(a, p, s) : launch_d<64, false>(a, p, s);
+  sgh_prof_stop(s);
+  return rc;
+}

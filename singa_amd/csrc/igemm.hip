@@ -1214,6 +1214,15 @@ typedef int (*cast_out_fn)(const float *, uint16_t *, size_t, void *);
 int conv_half(const sgh_conv_geom *g, int which, const uint16_t *a, const uint16_t *b, const uint16_t *bias,
               uint16_t *out, void *workspace, size_t ws_bytes, void *stream, cast_in_fn in, cast_out_fn outc) {
   if (!conv_ok(g) || !a || !b || !out) return SGH_EINVAL;
+  // the gradients run on the 16-bit matrix instructions where conv16.hip covers the geometry;
+  // everything else (and the forward pass) computes in fp32 on widened copies
+  if (which != SGH_CONV_FWD && sgh_conv16_workspace_bytes(g, which) != 0 && !getenv("SGH_CONV16_OFF")) {
+    const bool bf16 = in == sgh_cast_bf16_to_f32;
+    const int rc = which == SGH_CONV_DGRAD
+                       ? sgh_conv16_dgrad(g, a, b, out, workspace, ws_bytes, bf16, sgh_stream_of(stream))
+                       : sgh_conv16_wgrad(g, a, b, out, workspace, ws_bytes, bf16, sgh_stream_of(stream));
+    if (rc != SGH_EUNSUPPORTED) return rc;
+  }
   const HalfPlan p = half_plan(g, which);
   if (!workspace || ws_bytes < p.total() + (bias ? align256(size_t(g->K) * 4) : 0)) return SGH_EWORKSPACE;
   char *w = static_cast<char *>(workspace);
@@ -1255,7 +1264,9 @@ int sgh_conv_bgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db
 
 size_t sgh_conv_workspace_bytes_h(const sgh_conv_geom *g, int which) {
   if (!conv_ok(g) || which < 0 || which > 2) return 0;
-  return half_plan(g, which).total() + (which == SGH_CONV_FWD ? align256(size_t(g->K) * 4) : 0);
+  const size_t wide = half_plan(g, which).total() + (which == SGH_CONV_FWD ? align256(size_t(g->K) * 4) : 0);
+  const size_t native = sgh_conv16_workspace_bytes(g, which);
+  return wide > native ? wide : native;
 }
 
 int sgh_conv_dgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,

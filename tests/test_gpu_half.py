@@ -189,6 +189,58 @@ def test_conv_16bit_storage(singa, dev, kind, case):
         assert nl2(db.to_numpy(), O.conv_bgrad(dy)) < 1e-2
 
 
+def _grad16_cases(count, seed):
+    """Seeded geometries for the 16-bit matrix-instruction gradient kernels: output rows of 1..3
+    octets with partly empty last octets, odd and even widths (paired and single-pixel gradient
+    loads), strides 1-2 with every residue class, channel counts around the 64 / 128 tile edges and
+    K both below and above one 64-wide reduction chunk."""
+    r = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        R = int(r.choice([1, 1, 3, 3, 3, 5, 7]))
+        st = int(r.choice([1, 1, 2]))
+        pd = int(r.integers(0, R // 2 + 1))
+        C = int(r.choice([3, 16, 40, 64, 65, 128, 136]))
+        K = int(r.choice([8, 24, 64, 72, 128, 136]))
+        H = int(r.integers(max(R - 2 * pd, 2), 30))
+        W = H if r.random() < 0.5 else int(r.integers(max(R - 2 * pd, 2), 36))
+        N = int(r.integers(1, 5))
+        P, Q = (H + 2 * pd - R) // st + 1, (W + 2 * pd - R) // st + 1
+        if P < 1 or Q < 2 or N * K * P * Q * C * R * R > 3e8:
+            continue
+        cases.append((N, C, H, W, K, R, R, (st, st), (pd, pd)))
+    return cases
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("case", _grad16_cases(40, 777) + [
+    (2, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1)),      # ResNet stage-1 3x3
+    (2, 256, 14, 14, 64, 1, 1, (1, 1), (0, 0)),     # bottleneck reduce: plane of 196 = 24.5 octets
+    (3, 64, 7, 7, 256, 1, 1, (1, 1), (0, 0)),       # odd plane: single-pixel gradient loads
+    (2, 128, 28, 28, 256, 1, 1, (2, 2), (0, 0)),    # downsample
+    (1, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3)),       # stem
+])
+def test_conv_gradients_16bit_matrix_kernels(singa, dev, kind, case):
+    """dgrad / wgrad on the 16-bit MFMA kernels against the fp32 CPU oracle on the same stored
+    inputs (1e-2 normalised L2), plus run-to-run identity of the split weight gradient."""
+    from oracle import cpu_oracle as O
+    from util import nl2
+    N, C, H, W, K, R, S, stride, pad = case
+    r = rng(sum(case[:7]) + 5)
+    xt, x = _to(singa, dev, r.standard_normal((N, C, H, W)).astype(np.float32), kind)
+    wt, w = _to(singa, dev, (r.standard_normal((K, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32), kind)
+    h = singa.CudnnConvHandle(xt, (R, S), stride, pad, C, K, False)
+    P, Q = (H + 2 * pad[0] - R) // stride[0] + 1, (W + 2 * pad[1] - S) // stride[1] + 1
+    dyt, dy = _to(singa, dev, r.standard_normal((N, K, P, Q)).astype(np.float32), kind)
+    dx = singa.GpuConvBackwardx(dyt, wt, xt, h)
+    dw = singa.GpuConvBackwardW(dyt, xt, wt, h)
+    dx_o, dw_o = O.conv_bwd(dy, x, w, stride, pad)
+    e = nl2(dx.to_numpy(), dx_o), nl2(dw.to_numpy(), dw_o)
+    print("16-bit gradients nl2: dx %.2e dw %.2e" % e)
+    assert max(e) < 1e-2
+    _same_bits(singa.GpuConvBackwardW(dyt, xt, wt, h).to_numpy(), dw.to_numpy(), "wgrad run-to-run")
+
+
 def _sgd_ref(p, g, v, lr, mu, damp, wd, nesterov):
     """The four ops of SGD.apply in fp32, each product / sum rounded separately."""
     f = np.float32
