@@ -112,7 +112,7 @@ struct W16Args {
   float *partial;  // [splits][K][CRS]
   int N, C, H, W, K, P, Q, R, S, pad_h, pad_w;
   int QO;          // octets per output row: ceil(Q / 8)
-  int CRS, mtiles;
+  int CRS, mtiles, tiles, splits;
   int chunks, chunks_per_split;  // a chunk = 8 octets = 8 units (n, p, octet)
   long dy_elems, x_elems;
 };
@@ -125,8 +125,13 @@ __global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
   uint16_t *const As1 = lds16 + (BM + BN) * PITCH, *const Bs1 = As1 + BM * PITCH;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
-  const int m0 = (int(blockIdx.x) % a.mtiles) * BM, n0 = (int(blockIdx.x) / a.mtiles) * BN;
-  const int split = blockIdx.y;
+  // Workgroup w runs on XCD w % 8 (each XCD has its own L2).  All tiles of one split of the
+  // reduction read the same dy rows, so a split's tiles are given to one XCD: split = 8 * (slot /
+  // tiles) + w % 8 with slot = w / 8.
+  const int slot = int(blockIdx.x) >> 3, tile = slot % a.tiles;
+  const int split = (slot / a.tiles) * 8 + (int(blockIdx.x) & 7);
+  if (split >= a.splits) return;
+  const int m0 = (tile % a.mtiles) * BM, n0 = (tile / a.mtiles) * BN;
   const int c_begin = split * a.chunks_per_split;
   const int c_end = min(a.chunks, c_begin + a.chunks_per_split);
   const int oct = t & 7, rb = t >> 3;
@@ -151,78 +156,89 @@ __global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
     n += dn;
   };
 
+  // Loads are issued for the next chunk before the MFMA steps of the current one and only
+  // touched (masked, compacted) when they are written to LDS afterwards, so their latency hides
+  // behind the matrix work.  Offsets are bytes into buffer descriptors; kOOB reads as zero.
+  const rsrc_t rdy = make_rsrc(a.dy, unsigned(a.dy_elems * 2)), rx = make_rsrc(a.x, unsigned(a.x_elems * 2));
   int aoff[ASLOTS];
-  bool aok[ASLOTS];
 #pragma unroll
   for (int i = 0; i < ASLOTS; ++i) {
     const int k = m0 + rb + 32 * i;
-    aok[i] = k < a.K;
-    aoff[i] = k * PQ;
+    aoff[i] = k < a.K ? k * PQ : -1;
   }
-  int bconst[BSLOTS], br[BSLOTS], bs[BSLOTS];
-  bool bok[BSLOTS];
+  int boff[BSLOTS], br[BSLOTS], bs[BSLOTS];
 #pragma unroll
   for (int i = 0; i < BSLOTS; ++i) {
     const int col = n0 + rb + 32 * i;
-    bok[i] = col < a.CRS;
     const int c = col / RS, tap = col - c * RS, r = tap / a.S;
     br[i] = r - a.pad_h;
     bs[i] = tap - r * a.S - a.pad_w;
-    bconst[i] = c * HW;
+    boff[i] = c * HW + br[i] * a.W + bs[i];
+    if (col >= a.CRS) br[i] = -(1 << 28);  // (a row that is never inside the image)
   }
 
-  u32x4 ra[ASLOTS], rbv[BSLOTS];
-  auto load = [&]() {
+  struct Stage {                   // one chunk in flight
+    u32x4 ra[ASLOTS], rbv[BSLOTS][STRIDE];
+    int a_nv, a_tail[ASLOTS];      // valid elements of the dy octet; element offset of a slot on the guarded path, or -1
+    int b_lohi[BSLOTS], b_tail[BSLOTS];
+  };
+  auto load = [&](Stage &g) {
     const int nv = min(8, a.Q - 8 * qo);
     const bool unit_ok = n < a.N;
-    const long abase = long(n) * a.K * PQ + p * a.Q + 8 * qo;
+    g.a_nv = nv;
+    const int abase = n * a.K * PQ + p * a.Q + 8 * qo;
 #pragma unroll
     for (int i = 0; i < ASLOTS; ++i) {
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (unit_ok && aok[i]) {
-        const long off = abase + aoff[i];
-        if (off + 8 <= a.dy_elems) {
-          v = load16b(a.dy + off);
-          if (nv < 8) v = mask_range(v, 0, nv);
-        } else {
-          v = load_elems<1>(a.dy, off, 0, nv);
-        }
-      }
-      ra[i] = v;
+      const int off = abase + aoff[i];
+      const bool ok = unit_ok && aoff[i] >= 0;
+      const bool tail = ok && off + 8 > int(a.dy_elems);  // the 16 bytes would cross the end of the tensor
+      g.a_tail[i] = tail ? off : -1;
+      g.ra[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rdy, ok && !tail ? off * 2 : kOOB, 0, 0));
     }
-    const long xbase = long(n) * a.C * HW;
+    const int xbase = n * a.C * HW + p * STRIDE * a.W + 8 * STRIDE * qo;
 #pragma unroll
     for (int i = 0; i < BSLOTS; ++i) {
-      u32x4 v = {0u, 0u, 0u, 0u};
       const int h = p * STRIDE + br[i], col0 = 8 * STRIDE * qo + bs[i];
       const int lo = col0 < 0 ? (-col0 + STRIDE - 1) / STRIDE : 0;
       const int hi = min(nv, (a.W - col0 + STRIDE - 1) / STRIDE);
-      if (unit_ok && bok[i] && h >= 0 && h < a.H && hi > lo) {
-        const long off = xbase + bconst[i] + h * a.W + col0;
-        if (off >= 0 && off + 8 * STRIDE <= a.x_elems) {
-          if (STRIDE == 1) {
-            v = load16b(a.x + off);
-          } else {  // 16 elements, every other one wanted
-            const u32x4 v0 = load16b(a.x + off), v1 = load16b(a.x + off + 8);
-            v[0] = __builtin_amdgcn_perm(v0[1], v0[0], 0x05040100u);
-            v[1] = __builtin_amdgcn_perm(v0[3], v0[2], 0x05040100u);
-            v[2] = __builtin_amdgcn_perm(v1[1], v1[0], 0x05040100u);
-            v[3] = __builtin_amdgcn_perm(v1[3], v1[2], 0x05040100u);
-          }
-          if (lo > 0 || hi < 8) v = mask_range(v, lo, hi);
-        } else {
-          v = load_elems<STRIDE>(a.x, off, lo, hi);
-        }
+      const bool ok = unit_ok && unsigned(h) < unsigned(a.H) && hi > lo;
+      const int off = xbase + boff[i];
+      const bool tail = ok && (off < 0 || off + 8 * STRIDE > int(a.x_elems));
+      g.b_lohi[i] = ok ? (lo | (hi << 8)) : 0;
+      g.b_tail[i] = tail ? 1 : 0;
+      const int voff = ok && !tail ? off * 2 : kOOB;
+#pragma unroll
+      for (int u = 0; u < STRIDE; ++u)
+        g.rbv[i][u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, voff, 16 * u, 0));
+      if (tail) {  // first / last row of the tensor: element loads (rare; keeps every access inside the tensor)
+        g.rbv[i][0] = load_elems<STRIDE>(a.x, off, lo, hi);
+        g.b_lohi[i] = 8 << 8;
       }
-      rbv[i] = v;
     }
     advance();
   };
-  auto stage = [&](uint16_t *As, uint16_t *Bs) {
+  auto stage = [&](const Stage &g, uint16_t *As, uint16_t *Bs) {
 #pragma unroll
-    for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 32 * i) * PITCH + oct * 8) = ra[i];
+    for (int i = 0; i < ASLOTS; ++i) {
+      u32x4 v = g.ra[i];
+      if (g.a_tail[i] >= 0) v = load_elems<1>(a.dy, g.a_tail[i], 0, g.a_nv);
+      else if (g.a_nv < 8) v = mask_range(v, 0, g.a_nv);
+      *reinterpret_cast<u32x4 *>(As + (rb + 32 * i) * PITCH + oct * 8) = v;
+    }
 #pragma unroll
-    for (int i = 0; i < BSLOTS; ++i) *reinterpret_cast<u32x4 *>(Bs + (rb + 32 * i) * PITCH + oct * 8) = rbv[i];
+    for (int i = 0; i < BSLOTS; ++i) {
+      u32x4 v = g.rbv[i][0];
+      if (STRIDE == 2 && !g.b_tail[i]) {  // 16 elements loaded, every other one wanted
+        const u32x4 v1 = g.rbv[i][STRIDE - 1];
+        const u32x4 v0 = v;
+        v[0] = __builtin_amdgcn_perm(v0[1], v0[0], 0x05040100u);
+        v[1] = __builtin_amdgcn_perm(v0[3], v0[2], 0x05040100u);
+        v[2] = __builtin_amdgcn_perm(v1[1], v1[0], 0x05040100u);
+        v[3] = __builtin_amdgcn_perm(v1[3], v1[2], 0x05040100u);
+      }
+      if (g.b_lohi[i] != (8 << 8)) v = mask_range(v, g.b_lohi[i] & 0xff, g.b_lohi[i] >> 8);
+      *reinterpret_cast<u32x4 *>(Bs + (rb + 32 * i) * PITCH + oct * 8) = v;
+    }
   };
 
   f32x16 acc[TM][2];
@@ -233,15 +249,20 @@ __global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
+  // Chunk c is computed from LDS buffer c & 1 while the loads of chunk c + 1 are in flight; they are
+  // written to the other buffer after the MFMA steps.  (Holding two chunks in registers to cover
+  // more latency costs the second workgroup per CU and measured slower.)
   if (c_begin < c_end) {
-    load();
-    stage(As0, Bs0);
+    Stage g;
+    const int arow = wm * (TM * 32) + l32, brow = wn * 64 + l32;
+    load(g);
+    stage(g, As0, Bs0);
     __syncthreads();
     for (int c = c_begin; c < c_end; ++c) {
       const bool cur1 = (c - c_begin) & 1, more = c + 1 < c_end;
-      if (more) load();
-      mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, wm * (TM * 32) + l32, wn * 64 + l32, lh, acc);
-      if (more) stage(cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
+      if (more) load(g);
+      mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, arow, brow, lh, acc);
+      if (more) stage(g, cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
       __syncthreads();
     }
   }
@@ -261,14 +282,27 @@ __global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
     }
 }
 
-// dW = round16(sum over splits, ascending): run-to-run identical
-template <bool BF16>
-__global__ __launch_bounds__(256) void k_wgrad16_reduce(const float *partial, int splits, size_t n, uint16_t *dW) {
-  const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
-  if (i >= n) return;
+// dW = round16(sum over splits).  A workgroup takes EP consecutive elements; its 256 threads form
+// ZL = 256 / EP z-lanes: lane zl sums the splits zl, zl + ZL, ... in ascending order and the lane
+// sums are added in lane order, so the result depends on the shape only: run-to-run identical.
+template <int EP, bool BF16>
+__global__ __launch_bounds__(256) void k_wgrad16_reduce(const float *__restrict__ partial, int splits, size_t n,
+                                                        uint16_t *__restrict__ dW) {
+  constexpr int ZL = 256 / EP;
+  __shared__ float lanes[ZL][EP];
+  const int e = threadIdx.x % EP, zl = threadIdx.x / EP;
+  const size_t i = size_t(blockIdx.x) * EP + e;
   float s = 0.f;
-  for (int z = 0; z < splits; ++z) s += partial[size_t(z) * n + i];
-  dW[i] = round16<BF16>(s);
+  if (i < n)
+    for (int z = zl; z < splits; z += ZL) s += partial[size_t(z) * n + i];
+  lanes[zl][e] = s;
+  __syncthreads();
+  if (zl == 0 && i < n) {
+    float r = lanes[0][e];
+#pragma unroll
+    for (int l = 1; l < ZL; ++l) r += lanes[l][e];
+    dW[i] = round16<BF16>(r);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -278,7 +312,7 @@ struct D16Args {
   const uint16_t *dy, *wt;  // wt: [tap][CP][KP], zero-filled padding
   uint16_t *dx;
   int N, C, H, W, K, P, Q, R, S, stride, pad_h, pad_w;
-  int KP, CP, mtiles;
+  int KP, CP, mtiles, ptiles;
   int cls_tile0[5];  // first pixel tile of each residue class (stride^2 classes), then the total
   unsigned dy_bytes;
 };
@@ -293,7 +327,11 @@ __global__ __launch_bounds__(NT) void k_dgrad16(D16Args a) {
   uint16_t *const As1 = lds16 + (BM + BN) * PITCH, *const Bs1 = As1 + BM * PITCH;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lh = lane >> 5;
-  const int m0 = (int(blockIdx.x) % a.mtiles) * BM, pt = int(blockIdx.x) / a.mtiles;
+  // XCD-aware ids (workgroup w runs on XCD w % 8): the channel tiles of one pixel tile read the
+  // same gradient pixels and share an XCD's L2.
+  const int slot = int(blockIdx.x) >> 3, pt = (slot / a.mtiles) * 8 + (int(blockIdx.x) & 7);
+  if (pt >= a.ptiles) return;
+  const int m0 = (slot % a.mtiles) * BM;
   const int st = a.stride, PQ = a.P * a.Q, HW = a.H * a.W;
   int cls = 0;
   while (pt >= a.cls_tile0[cls + 1]) ++cls;
@@ -452,7 +490,7 @@ struct W16Plan {
 W16Plan wplan(const sgh_conv_geom *g) {
   W16Plan p{};
   if (g->stride_h != g->stride_w || (g->stride_h != 1 && g->stride_h != 2)) return p;
-  const size_t lim = size_t(1) << 31;
+  const size_t lim = size_t(1) << 30;  // byte offsets into x and dy stay below 2^31
   const size_t xe = size_t(g->N) * g->C * g->H * g->W, ye = size_t(g->N) * g->K * g->P * g->Q;
   if (xe >= lim || ye >= lim || size_t(g->K) * g->C * g->R * g->S >= lim) return p;
   p.f = *g;
@@ -518,7 +556,7 @@ int launch_w(const W16Args &a, const W16Plan &p, hipStream_t s) {
     if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
     attr = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.mtiles * p.ntiles, p.splits), dim3(NT), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(unsigned(p.mtiles * p.ntiles) * 8u * unsigned((p.splits + 7) / 8)), dim3(NT), lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -531,7 +569,7 @@ int launch_d(const D16Args &a, const D16Plan &p, hipStream_t s) {
     if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
     attr = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.tiles * p.mtiles), dim3(NT), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(unsigned((p.tiles + 7) / 8) * 8u * unsigned(p.mtiles)), dim3(NT), lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -558,7 +596,7 @@ int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
   a.dy = dy, a.x = x, a.partial = static_cast<float *>(workspace);
   a.N = p.f.N, a.C = p.f.C, a.H = p.f.H, a.W = p.f.W, a.K = p.f.K, a.P = p.f.P, a.Q = p.f.Q;
   a.R = p.f.R, a.S = p.f.S, a.pad_h = p.f.pad_h, a.pad_w = p.f.pad_w;
-  a.QO = p.QO, a.CRS = g->C * g->R * g->S, a.mtiles = p.mtiles;
+  a.QO = p.QO, a.CRS = g->C * g->R * g->S, a.mtiles = p.mtiles, a.tiles = p.mtiles * p.ntiles, a.splits = p.splits;
   a.chunks = p.chunks, a.chunks_per_split = p.cps;
   a.dy_elems = long(g->N) * g->K * g->P * g->Q, a.x_elems = long(g->N) * g->C * g->H * g->W;
   const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
@@ -574,8 +612,15 @@ int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
   const size_t n = size_t(g->K) * a.CRS;
-  if (bf16) hipLaunchKernelGGL(k_wgrad16_reduce<true>, dim3(unsigned((n + 255) / 256)), dim3(256), 0, s, a.partial, p.splits, n, dW);
-  else hipLaunchKernelGGL(k_wgrad16_reduce<false>, dim3(unsigned((n + 255) / 256)), dim3(256), 0, s, a.partial, p.splits, n, dW);
+  if (n / 64 >= size_t(2 * sgh_num_cus()) || p.splits < 16) {
+    const dim3 grid(unsigned((n + 63) / 64));
+    if (bf16) hipLaunchKernelGGL((k_wgrad16_reduce<64, true>), grid, dim3(256), 0, s, a.partial, p.splits, n, dW);
+    else hipLaunchKernelGGL((k_wgrad16_reduce<64, false>), grid, dim3(256), 0, s, a.partial, p.splits, n, dW);
+  } else {  // few elements, many splits: more z-lanes
+    const dim3 grid(unsigned((n + 15) / 16));
+    if (bf16) hipLaunchKernelGGL((k_wgrad16_reduce<16, true>), grid, dim3(256), 0, s, a.partial, p.splits, n, dW);
+    else hipLaunchKernelGGL((k_wgrad16_reduce<16, false>), grid, dim3(256), 0, s, a.partial, p.splits, n, dW);
+  }
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -593,7 +638,7 @@ int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
   a.dy = dy, a.wt = wt, a.dx = dx;
   a.N = g->N, a.C = g->C, a.H = g->H, a.W = g->W, a.K = g->K, a.P = g->P, a.Q = g->Q, a.R = g->R, a.S = g->S;
   a.stride = g->stride_h, a.pad_h = g->pad_h, a.pad_w = g->pad_w;
-  a.KP = p.KP, a.CP = p.CP, a.mtiles = p.mtiles;
+  a.KP = p.KP, a.CP = p.CP, a.mtiles = p.mtiles, a.ptiles = p.tiles;
   for (int i = 0; i < 5; ++i) a.cls_tile0[i] = p.cls_tile0[i];
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2);
   const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
