@@ -27,6 +27,8 @@
 // register double buffering.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "storage.h"
 
@@ -118,11 +120,14 @@ struct W16Args {
 };
 
 template <int BM, int STRIDE, bool BF16>
-__global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_wgrad16(W16Args a) {
   extern __shared__ __align__(16) uint16_t lds16[];
   constexpr int TM = BM / 64, ASLOTS = BM * 8 / NT, BSLOTS = BN * 8 / NT;
   uint16_t *const As0 = lds16, *const Bs0 = lds16 + BM * PITCH;
   uint16_t *const As1 = lds16 + (BM + BN) * PITCH, *const Bs1 = As1 + BM * PITCH;
+  // octet masks by valid element range: lut[lo * 9 + hi] keeps elements lo <= j < hi (branch-free
+  // border handling: one LDS read and four ANDs per octet)
+  u32x4 *const lut = reinterpret_cast<u32x4 *>(lds16 + 2 * (BM + BN) * PITCH);
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
   // Workgroup w runs on XCD w % 8 (each XCD has its own L2).  All tiles of one split of the
@@ -131,6 +136,8 @@ __global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
   const int slot = int(blockIdx.x) >> 3, tile = slot % a.tiles;
   const int split = (slot / a.tiles) * 8 + (int(blockIdx.x) & 7);
   if (split >= a.splits) return;
+  if (t < 81) lut[t] = mask_range(u32x4{~0u, ~0u, ~0u, ~0u}, t / 9, t % 9);
+  __syncthreads();
   const int m0 = (tile % a.mtiles) * BM, n0 = (tile / a.mtiles) * BN;
   const int c_begin = split * a.chunks_per_split;
   const int c_end = min(a.chunks, c_begin + a.chunks_per_split);
@@ -179,20 +186,21 @@ __global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
 
   struct Stage {                   // one chunk in flight
     u32x4 ra[ASLOTS], rbv[BSLOTS][STRIDE];
-    int a_nv, a_tail[ASLOTS];      // valid elements of the dy octet; element offset of a slot on the guarded path, or -1
-    int b_lohi[BSLOTS], b_tail[BSLOTS];
+    int a_nv;                      // valid elements of the dy octet
+    int b_lohi[BSLOTS];            // lo * 9 + hi for the valid element range [lo, hi) of each x octet
   };
-  auto load = [&](Stage &g) {
+  auto load = [&](Stage &g, auto tails) {
     const int nv = min(8, a.Q - 8 * qo);
     const bool unit_ok = n < a.N;
     g.a_nv = nv;
     const int abase = n * a.K * PQ + p * a.Q + 8 * qo;
+    bool any_tail = false;
 #pragma unroll
     for (int i = 0; i < ASLOTS; ++i) {
       const int off = abase + aoff[i];
       const bool ok = unit_ok && aoff[i] >= 0;
       const bool tail = ok && off + 8 > int(a.dy_elems);  // the 16 bytes would cross the end of the tensor
-      g.a_tail[i] = tail ? off : -1;
+      any_tail |= tail;
       g.ra[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rdy, ok && !tail ? off * 2 : kOOB, 0, 0));
     }
     const int xbase = n * a.C * HW + p * STRIDE * a.W + 8 * STRIDE * qo;
@@ -204,31 +212,49 @@ __global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
       const bool ok = unit_ok && unsigned(h) < unsigned(a.H) && hi > lo;
       const int off = xbase + boff[i];
       const bool tail = ok && (off < 0 || off + 8 * STRIDE > int(a.x_elems));
-      g.b_lohi[i] = ok ? (lo | (hi << 8)) : 0;
-      g.b_tail[i] = tail ? 1 : 0;
+      any_tail |= tail;
+      g.b_lohi[i] = ok ? lo * 9 + hi : 0;
       const int voff = ok && !tail ? off * 2 : kOOB;
 #pragma unroll
       for (int u = 0; u < STRIDE; ++u)
         g.rbv[i][u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, voff, 16 * u, 0));
-      if (tail) {  // first / last row of the tensor: element loads (rare; keeps every access inside the tensor)
-        g.rbv[i][0] = load_elems<STRIDE>(a.x, off, lo, hi);
-        g.b_lohi[i] = 8 << 8;
+    }
+    // Octets whose 16 bytes would start before or end after the tensor (its first / last rows only)
+    // are fetched element by element, so that no access leaves the tensor.  Rare, and the only
+    // place where this function waits for memory.
+    if (decltype(tails)::value && any_tail) {
+#pragma unroll
+      for (int i = 0; i < ASLOTS; ++i) {
+        const int off = abase + aoff[i];
+        if (unit_ok && aoff[i] >= 0 && off + 8 > int(a.dy_elems)) g.ra[i] = load_elems<1>(a.dy, off, 0, nv);
+      }
+#pragma unroll
+      for (int i = 0; i < BSLOTS; ++i) {
+        const int h = p * STRIDE + br[i], col0 = 8 * STRIDE * qo + bs[i];
+        const int lo = col0 < 0 ? (-col0 + STRIDE - 1) / STRIDE : 0;
+        const int hi = min(nv, (a.W - col0 + STRIDE - 1) / STRIDE);
+        const int off = xbase + boff[i];
+        if (unit_ok && unsigned(h) < unsigned(a.H) && hi > lo && (off < 0 || off + 8 * STRIDE > int(a.x_elems))) {
+          const u32x4 v = load_elems<STRIDE>(a.x, off, lo, hi);  // already compacted and masked
+          g.rbv[i][0] = v;
+          if (STRIDE == 2) {  // (spread again so that the common compaction below reproduces v)
+            g.rbv[i][0] = u32x4{v[0] & 0xffffu, v[0] >> 16, v[1] & 0xffffu, v[1] >> 16};
+            g.rbv[i][STRIDE - 1] = u32x4{v[2] & 0xffffu, v[2] >> 16, v[3] & 0xffffu, v[3] >> 16};
+          }
+          g.b_lohi[i] = 8;
+        }
       }
     }
     advance();
   };
   auto stage = [&](const Stage &g, uint16_t *As, uint16_t *Bs) {
+    const u32x4 ma = lut[g.a_nv];
 #pragma unroll
-    for (int i = 0; i < ASLOTS; ++i) {
-      u32x4 v = g.ra[i];
-      if (g.a_tail[i] >= 0) v = load_elems<1>(a.dy, g.a_tail[i], 0, g.a_nv);
-      else if (g.a_nv < 8) v = mask_range(v, 0, g.a_nv);
-      *reinterpret_cast<u32x4 *>(As + (rb + 32 * i) * PITCH + oct * 8) = v;
-    }
+    for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 32 * i) * PITCH + oct * 8) = g.ra[i] & ma;
 #pragma unroll
     for (int i = 0; i < BSLOTS; ++i) {
       u32x4 v = g.rbv[i][0];
-      if (STRIDE == 2 && !g.b_tail[i]) {  // 16 elements loaded, every other one wanted
+      if (STRIDE == 2) {  // 16 elements loaded, every other one wanted
         const u32x4 v1 = g.rbv[i][STRIDE - 1];
         const u32x4 v0 = v;
         v[0] = __builtin_amdgcn_perm(v0[1], v0[0], 0x05040100u);
@@ -236,8 +262,7 @@ __global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
         v[2] = __builtin_amdgcn_perm(v1[1], v1[0], 0x05040100u);
         v[3] = __builtin_amdgcn_perm(v1[3], v1[2], 0x05040100u);
       }
-      if (g.b_lohi[i] != (8 << 8)) v = mask_range(v, g.b_lohi[i] & 0xff, g.b_lohi[i] >> 8);
-      *reinterpret_cast<u32x4 *>(Bs + (rb + 32 * i) * PITCH + oct * 8) = v;
+      *reinterpret_cast<u32x4 *>(Bs + (rb + 32 * i) * PITCH + oct * 8) = v & lut[g.b_lohi[i]];
     }
   };
 
@@ -249,22 +274,48 @@ __global__ __launch_bounds__(NT) void k_wgrad16(W16Args a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  // Chunk c is computed from LDS buffer c & 1 while the loads of chunk c + 1 are in flight; they are
-  // written to the other buffer after the MFMA steps.  (Holding two chunks in registers to cover
-  // more latency costs the second workgroup per CU and measured slower.)
-  if (c_begin < c_end) {
-    Stage g;
-    const int arow = wm * (TM * 32) + l32, brow = wn * 64 + l32;
-    load(g);
-    stage(g, As0, Bs0);
-    __syncthreads();
-    for (int c = c_begin; c < c_end; ++c) {
-      const bool cur1 = (c - c_begin) & 1, more = c + 1 < c_end;
-      if (more) load(g);
-      mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, arow, brow, lh, acc);
-      if (more) stage(g, cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
+  const int arow = wm * (TM * 32) + l32, brow = wn * 64 + l32;
+  auto run = [&](auto tails) {
+    if constexpr (STRIDE == 1) {
+      // Chunk c is computed from LDS buffer c & 1 while chunk c + 1 waits in registers (stage set
+      // (c + 1) & 1) and the loads of chunk c + 2 are issued: two chunks of memory latency are covered.
+      Stage g0, g1;
+      load(g0, tails);
+      stage(g0, As0, Bs0);
+      if (c_begin + 1 < c_end) load(g1, tails);
       __syncthreads();
+      for (int c = c_begin; c < c_end; c += 2) {
+        if (c + 2 < c_end) load(g0, tails);
+        mma_chunk<TM, BF16>(As0, Bs0, arow, brow, lh, acc);
+        if (c + 1 >= c_end) break;
+        stage(g1, As1, Bs1);
+        __syncthreads();
+        if (c + 3 < c_end) load(g1, tails);
+        mma_chunk<TM, BF16>(As1, Bs1, arow, brow, lh, acc);
+        if (c + 2 < c_end) stage(g0, As0, Bs0);
+        __syncthreads();
+      }
+    } else {
+      // (stride 2 holds twice the x registers per chunk: one chunk in flight, or the kernel spills)
+      Stage g;
+      load(g, tails);
+      stage(g, As0, Bs0);
+      __syncthreads();
+      for (int c = c_begin; c < c_end; ++c) {
+        const bool cur1 = (c - c_begin) & 1, more = c + 1 < c_end;
+        if (more) load(g, tails);
+        mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, arow, brow, lh, acc);
+        if (more) stage(g, cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
+        __syncthreads();
+      }
     }
+  };
+  // Only the first chunk (x rows before the first image) and the chunks of the last two output
+  // rows of the last image can hold an octet that would reach outside a tensor; every other
+  // workgroup runs the loop without that code.
+  if (c_begin < c_end) {
+    if (c_begin == 0 || c_end + (2 * a.QO + 7) / 8 + 1 >= a.chunks) run(std::true_type{});
+    else run(std::false_type{});
   }
 
   float *out = a.partial + size_t(split) * a.K * a.CRS;
@@ -472,6 +523,7 @@ __global__ __launch_bounds__(256) void k_relayout16(const uint16_t *W, uint16_t 
 
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
+constexpr size_t kLutBytes = 81 * 16;  // wgrad: octet mask table behind the tiles
 constexpr size_t kLds128 = size_t(2) * (128 + BN) * PITCH * 2, kLds64 = size_t(2) * (64 + BN) * PITCH * 2;
 
 template <typename Kern>
@@ -504,14 +556,20 @@ W16Plan wplan(const sgh_conv_geom *g) {
   p.QO = (p.f.Q + 7) / 8;
   const long units = long(p.f.N) * p.f.P * p.QO;
   p.chunks = int((units + 7) / 8);
-  // enough splits of the reduction for two workgroups per CU, at least 4 chunks each
-  const int tiles = p.mtiles * p.ntiles, want = (2 * sgh_num_cus() + tiles - 1) / tiles;
-  int splits = want < 1 ? 1 : want;
-  if (splits > (p.chunks + 3) / 4) splits = (p.chunks + 3) / 4;
-  if (splits < 1) splits = 1;
-  p.cps = (p.chunks + splits - 1) / splits;
-  p.splits = (p.chunks + p.cps - 1) / p.cps;
-  if (p.splits < 1) p.splits = 1;
+  // Splits of the reduction: the chip holds 2 workgroups per CU at a time; among 1..4 such rounds
+  // take the split count whose (rounds x chunks per split) is smallest, i.e. avoid a last round
+  // that is mostly empty.  Every split gets at least 4 chunks.
+  const int tiles = p.mtiles * p.ntiles, slots = 2 * sgh_num_cus();
+  long best = -1;
+  for (int r = 1; r <= 4; ++r) {
+    int s = slots * r / tiles;
+    if (s < 1) s = 1;
+    if (s > (p.chunks + 3) / 4) s = (p.chunks + 3) / 4;
+    if (s < 1) s = 1;
+    const int cps = (p.chunks + s - 1) / s, s2 = (p.chunks + cps - 1) / cps;
+    const long rounds = (long(tiles) * s2 + slots - 1) / slots, cost = rounds * (cps + 2);  // (+2: prologue, epilogue)
+    if (best < 0 || cost < best) best = cost, p.cps = cps, p.splits = s2;
+  }
   p.ok = true;
   return p;
 }
@@ -550,7 +608,7 @@ D16Plan dplan(const sgh_conv_geom *g) {
 template <int BM, int STRIDE, bool BF16>
 int launch_w(const W16Args &a, const W16Plan &p, hipStream_t s) {
   auto kern = k_wgrad16<BM, STRIDE, BF16>;
-  const size_t lds = BM == 128 ? kLds128 : kLds64;
+  const size_t lds = (BM == 128 ? kLds128 : kLds64) + kLutBytes;
   static bool attr = false;
   if (!attr) {
     if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
