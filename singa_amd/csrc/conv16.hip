@@ -365,7 +365,7 @@ struct D16Args {
   int N, C, H, W, K, P, Q, R, S, stride, pad_h, pad_w;
   int KP, CP, mtiles, ptiles;
   int cls_tile0[5];  // first pixel tile of each residue class (stride^2 classes), then the total
-  unsigned dy_bytes;
+  unsigned dy_bytes, wt_bytes;
 };
 
 constexpr unsigned kSelLo = 0x05040100u, kSelHi = 0x07060302u, kSelZero = 0x0c0c0c0cu;
@@ -400,38 +400,37 @@ __global__ __launch_bounds__(NT) void k_dgrad16(D16Args a) {
   const int nA = int(pixA / HWc), remA = int(pixA - long(nA) * HWc), iA = remA / Wc, jA = remA - iA * Wc;
   int voff = kOOB;  // byte offset of the dword holding both pixels (kOOB: neither exists)
   unsigned selA = kSelZero, selB = kSelZero;
-  auto set_tap = [&](int tap) {
-    const int r = tap / a.S, s = tap - r * a.S;
-    const int dr = (ca + a.pad_h - r) / st, ds = (cb + a.pad_w - s) / st;  // exact for the taps of this class
-    const int p = iA + dr, q0 = jA + ds;
-    const bool row = p >= 0 && p < a.P;
-    const bool memA = row && q0 >= 0 && q0 < a.Q, memB = row && q0 + 1 >= 0 && q0 + 1 < a.Q;
+  // The taps of this class are r = r0 + st * ti, s = s0 + st * tj (ti < nr, tj < ns): those with
+  // (ca + pad_h - r) and (cb + pad_w - s) divisible by the stride; the gradient pixel of tap
+  // (ti, tj) is (i + dr0 - ti, j + ds0 - tj).  (st is 1 or 2: shifts, no divisions.)
+  const int sh = st - 1;
+  const int r0 = (ca + a.pad_h) & sh, s0 = (cb + a.pad_w) & sh;
+  const int nr = r0 < a.R ? (a.R - r0 + sh) >> sh : 0, ns = s0 < a.S ? (a.S - s0 + sh) >> sh : 0;
+  const int dr0 = (ca + a.pad_h - r0) >> sh, ds0 = (cb + a.pad_w - s0) >> sh;
+  const bool pixA_ok = pixA < cnt, pixB_ok = pixB < cnt && jA + 1 < Wreal;
+  auto set_tap = [&](int ti, int tj) {
+    const int p = iA + dr0 - ti, q0 = jA + ds0 - tj;
+    const bool row = unsigned(p) < unsigned(a.P);
+    const bool memA = row && unsigned(q0) < unsigned(a.Q), memB = row && unsigned(q0 + 1) < unsigned(a.Q);
     const int base = ((nA * a.K) * a.P + p) * a.Q + q0;
-    bool hiA = false, loB = false;
-    if (memA && memB) voff = base * 2;
-    else if (memA) voff = (base - 1) * 2, hiA = true;   // pixel A sits in the high half
-    else if (memB) voff = (base + 1) * 2, loB = true;   // pixel B sits in the low half
-    else voff = kOOB;
-    selA = (memA && pixA < cnt) ? (hiA ? kSelHi : kSelLo) : kSelZero;
-    selB = (memB && pixB < cnt && jA + 1 < Wreal) ? (loB ? kSelLo : kSelHi) : kSelZero;
+    // both pixels exist: their dword; only A: the dword before (A in the high half); only B: the
+    // dword after (B in the low half) -- the load never leaves the row
+    voff = memA ? (memB ? base * 2 : (base - 1) * 2) : (memB ? (base + 1) * 2 : kOOB);
+    selA = memA && pixA_ok ? (memB ? kSelLo : kSelHi) : kSelZero;
+    selB = memB && pixB_ok ? (memA ? kSelHi : kSelLo) : kSelZero;
   };
-  auto tap_in_class = [&](int tap) {
-    const int r = tap / a.S, s = tap - r * a.S;
-    return (ca + a.pad_h - r) % st == 0 && (cb + a.pad_w - s) % st == 0;
-  };
-  const int RS = a.R * a.S, nkc = a.KP / KC;
-  auto next_tap = [&](int tap) {
-    while (tap < RS && !tap_in_class(tap)) ++tap;
-    return tap;
-  };
+  const int nkc = a.KP / KC;
 
   const int oct = t & 7, rb = t >> 3;
   u32x4 ra[ASLOTS];
   unsigned rd[2][8];   // the pair's dword for 8 consecutive k
+  const rsrc_t rwt = make_rsrc(a.wt, a.wt_bytes);
+  const int woff = ((m0 + rb) * a.KP + oct * 8) * 2;
   auto load = [&](int tap, int kc) {
+    const int wso = (tap * a.CP * a.KP + kc * KC) * 2;
 #pragma unroll
     for (int i = 0; i < ASLOTS; ++i)
-      ra[i] = *reinterpret_cast<const u32x4 *>(a.wt + (size_t(tap) * a.CP + m0 + rb + 32 * i) * a.KP + kc * KC + oct * 8);
+      ra[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rwt, woff + 32 * i * a.KP * 2, wso, 0));
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int kb = kc * KC + (kq + 4 * i) * 8;
@@ -470,28 +469,29 @@ __global__ __launch_bounds__(NT) void k_dgrad16(D16Args a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  int tap = next_tap(0), kc = 0;
-  if (tap < RS) {
-    set_tap(tap);
-    load(tap, kc);
+  if (nr > 0 && ns > 0) {
+    int ti = 0, tj = 0, kc = 0;
+    set_tap(ti, tj);
+    load((r0 + st * ti) * a.S + s0 + st * tj, kc);
     stage(As0, Bs0);
     __syncthreads();
     bool cur1 = false;
     while (true) {
-      int ntap = tap, nk = kc + 1;
-      if (nk == nkc) nk = 0, ntap = next_tap(tap + 1);
-      const bool more = ntap < RS;
+      bool newtap = false;
+      if (++kc == nkc) {
+        kc = 0, newtap = true;
+        if (++tj == ns) tj = 0, ++ti;
+      }
+      const bool more = ti < nr;
       if (more) {
-        if (ntap != tap) set_tap(ntap);   // the staged registers were already packed with the old selectors
-        load(ntap, nk);
+        if (newtap) set_tap(ti, tj);   // (the registers of the previous chunk were packed with the old selectors)
+        load((r0 + st * ti) * a.S + s0 + st * tj, kc);
       }
       mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, wm * (TM * 32) + l32, wn * 64 + l32, lh, acc);
       if (!more) break;
       stage(cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
       __syncthreads();
       cur1 = !cur1;
-      tap = ntap;
-      kc = nk;
     }
   }
 
@@ -587,10 +587,6 @@ D16Plan dplan(const sgh_conv_geom *g) {
   if (g->K % 8 != 0 || g->Q < 2 || g->C < 16) return p;  // (a 64-row tile is mostly empty below 16 channels)
   const size_t lim = size_t(1) << 30;  // byte offsets of dy stay below 2^31
   if (size_t(g->N) * g->K * g->P * g->Q >= lim || size_t(g->N) * g->C * g->H * g->W >= 2 * lim) return p;
-  p.bm = g->C <= 64 ? 64 : 128;
-  p.mtiles = (g->C + p.bm - 1) / p.bm;
-  p.CP = p.mtiles * p.bm;
-  p.KP = (g->K + KC - 1) / KC * KC;
   long tiles = 0;
   for (int cls = 0; cls < st * st; ++cls) {
     const int ca = cls / st, cb = cls % st;
@@ -599,7 +595,12 @@ D16Plan dplan(const sgh_conv_geom *g) {
     tiles += (long(g->N) * Hc * Wc + BN - 1) / BN;
   }
   for (int cls = st * st; cls < 5; ++cls) p.cls_tile0[cls] = int(tiles);
-  if (tiles * p.mtiles >= (long(1) << 30)) return p;
+  // 64-row channel tiles when 128-row ones would leave CUs without a workgroup
+  p.bm = (g->C <= 64 || tiles * ((g->C + 127) / 128) < sgh_num_cus() * 5 / 4) ? 64 : 128;
+  p.mtiles = (g->C + p.bm - 1) / p.bm;
+  p.CP = p.mtiles * p.bm;
+  p.KP = (g->K + KC - 1) / KC * KC;
+  if (tiles * p.mtiles >= (long(1) << 30) || size_t(g->R) * g->S * p.CP * p.KP >= lim) return p;
   p.tiles = int(tiles);
   p.ok = true;
   return p;
@@ -699,6 +700,7 @@ int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
   a.KP = p.KP, a.CP = p.CP, a.mtiles = p.mtiles, a.ptiles = p.tiles;
   for (int i = 0; i < 5; ++i) a.cls_tile0[i] = p.cls_tile0[i];
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2);
+  a.wt_bytes = unsigned(nw * 2);
   const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
   sgh_prof_start("conv_dgrad16", flops, s);
   int rc;

@@ -121,6 +121,54 @@ class HipOps(object):
     def make_sgd(self, lr, momentum):
         return hip_opt.SGD(lr=lr, momentum=momentum)
 
+    # precision boundary of a mixed-precision graph (identity here)
+    def to_compute(self, x):
+        return x
+
+    def to_storage(self, x):
+        return x
+
+
+class _MixedSGD(hip_opt.SGD):
+    """16-bit parameters are updated through an fp32 master copy and fp32 momentum
+    (``SGD.apply_master``); fp32 parameters as usual."""
+
+    def apply(self, name, p, g):
+        if p.data_type() != singa.kFloat32:
+            return self.apply_master(name, p, g)
+        return super(_MixedSGD, self).apply(name, p, g)
+
+
+class HalfHipOps(HipOps):
+    """Mixed precision as the reference trains in half (``layer.py:684-696`` casts the conv / linear
+    parameters to the input's type; cuDNN keeps BatchNorm parameters and statistics in fp32):
+    4-D tensors -- activations, their gradients and convolution weights -- are stored in `dtype`
+    (binary16 or bfloat16), BatchNorm parameters / statistics and the classifier head stay fp32,
+    16-bit weights are updated through fp32 master copies."""
+
+    def __init__(self, dev, dtype):
+        HipOps.__init__(self, dev)
+        self.dtype = dtype
+        self.name = "hip-" + singa._SUFFIX[dtype]
+
+    def from_numpy(self, a):
+        t = singa.from_numpy(a, self.dev)
+        return t.AsType(self.dtype) if np.ndim(a) == 4 else t
+
+    def relu(self, x):
+        if x.data_type() == singa.kFloat32:
+            return singa.ReLU(x)
+        return singa.ReLUBackward(x, x)   # y = x > 0 ? x : 0, the same selection
+
+    def to_compute(self, x):
+        return x.AsType(singa.kFloat32)
+
+    def to_storage(self, x):
+        return x.AsType(self.dtype)
+
+    def make_sgd(self, lr, momentum):
+        return _MixedSGD(lr=lr, momentum=momentum)
+
 
 # ------------------------------------------------------------------------------------ layers
 
@@ -221,6 +269,20 @@ class Flatten(_Layer):
         return self.ops.reshape(dy, self.shape)
 
 
+class Cast(_Layer):
+    """Precision boundary in front of the classifier head: storage type -> fp32 and back for the
+    gradient (``Tensor::AsType``); the identity for an all-fp32 graph."""
+
+    def __init__(self, ops, name):
+        self.ops, self.name = ops, name
+
+    def fwd(self, x):
+        return self.ops.to_compute(x) if hasattr(self.ops, "to_compute") else x
+
+    def bwd(self, dy, grads):
+        return self.ops.to_storage(dy) if hasattr(self.ops, "to_storage") else dy
+
+
 class Linear(_Layer):
     params = ("W", "b")
 
@@ -280,6 +342,58 @@ class BasicBlock(_Layer):
                                              grads), grads)
         if d_res is d_add:
             # the first-arrived buffer is another op's input gradient: accumulate into the fresh one
+            return self.ops.accumulate(d_main, d_res)
+        return self.ops.accumulate(d_res, d_main)
+
+
+class Bottleneck(_Layer):
+    """examples/cnn/model/resnet.py:68-120: 1x1 reduce, 3x3 (carries the stride), 1x1 expand (x4)."""
+
+    expansion = 4
+
+    def __init__(self, ops, name, rng, inplanes, planes, stride, downsample):
+        self.ops, self.name = ops, name
+        out = planes * self.expansion
+        self.conv1 = Conv(ops, name + ".conv1", he_normal(rng, planes, inplanes, 1, 1), None, (1, 1), (0, 0))
+        self.bn1 = BatchNorm(ops, name + ".bn1", planes)
+        self.relu1 = ReLU(ops, name + ".relu1")
+        self.conv2 = Conv(ops, name + ".conv2", he_normal(rng, planes, planes, 3, 3), None, (stride, stride), (1, 1))
+        self.bn2 = BatchNorm(ops, name + ".bn2", planes)
+        self.relu2 = ReLU(ops, name + ".relu2")
+        self.conv3 = Conv(ops, name + ".conv3", he_normal(rng, out, planes, 1, 1), None, (1, 1), (0, 0))
+        self.bn3 = BatchNorm(ops, name + ".bn3", out)
+        self.relu3 = ReLU(ops, name + ".relu3")
+        self.ds_conv = self.ds_bn = None
+        if downsample:
+            self.ds_conv = Conv(ops, name + ".downsample.conv", he_normal(rng, out, inplanes, 1, 1), None,
+                                (stride, stride), (0, 0))
+            self.ds_bn = BatchNorm(ops, name + ".downsample.bn", out)
+
+    def sublayers(self):
+        ls = [self.conv1, self.bn1, self.relu1, self.conv2, self.bn2, self.relu2, self.conv3, self.bn3, self.relu3]
+        if self.ds_conv is not None:
+            ls += [self.ds_conv, self.ds_bn]
+        return ls
+
+    def fwd(self, x):
+        out = self.relu1.fwd(self.bn1.fwd(self.conv1.fwd(x)))
+        out = self.relu2.fwd(self.bn2.fwd(self.conv2.fwd(out)))
+        out = self.bn3.fwd(self.conv3.fwd(out))
+        residual = x
+        if self.ds_conv is not None:
+            residual = self.ds_bn.fwd(self.ds_conv.fwd(x))
+        return self.relu3.fwd(self.ops.add(out, residual))
+
+    def bwd(self, dy, grads):
+        d_add = self.relu3.bwd(dy, grads)
+        if self.ds_conv is not None:   # the stack pops the residual branch first, as in BasicBlock
+            d_res = self.ds_conv.bwd(self.ds_bn.bwd(d_add, grads), grads)
+        else:
+            d_res = d_add
+        d = self.conv3.bwd(self.bn3.bwd(d_add, grads), grads)
+        d = self.conv2.bwd(self.bn2.bwd(self.relu2.bwd(d, grads), grads), grads)
+        d_main = self.conv1.bwd(self.bn1.bwd(self.relu1.bwd(d, grads), grads), grads)
+        if d_res is d_add:
             return self.ops.accumulate(d_main, d_res)
         return self.ops.accumulate(d_res, d_main)
 
@@ -406,6 +520,32 @@ def build_resnet18(ops, rng, lr=0.05, momentum=0.9, classes=1000, in_ch=3, width
     return Net(ops, layers, lr, momentum)
 
 
+def build_resnet50(ops, rng, lr=0.05, momentum=0.9, classes=1000, in_ch=3, widths=(64, 128, 256, 512),
+                   blocks=(3, 4, 6, 3), final_pool=7):
+    """examples/cnn/model/resnet.py:121-185 with Bottleneck blocks (resnet50: stages [3, 4, 6, 3])."""
+    layers = [
+        Conv(ops, "conv1", he_normal(rng, widths[0], in_ch, 7, 7), None, (2, 2), (3, 3)),
+        BatchNorm(ops, "bn1", widths[0]),
+        ReLU(ops, "relu"),
+        Pool(ops, "maxpool", (3, 3), (2, 2), (1, 1), True),
+    ]
+    inplanes = widths[0]
+    for si, (planes, nb) in enumerate(zip(widths, blocks)):
+        stride = 1 if si == 0 else 2
+        for bi in range(nb):
+            s = stride if bi == 0 else 1
+            ds = bi == 0 and (s != 1 or inplanes != planes * Bottleneck.expansion)
+            layers.append(Bottleneck(ops, "layer%d.%d" % (si + 1, bi), rng, inplanes, planes, s, ds))
+            inplanes = planes * Bottleneck.expansion
+    layers += [
+        Pool(ops, "avgpool", (final_pool, final_pool), (1, 1), (0, 0), False),
+        Flatten(ops, "flatten"),
+        Cast(ops, "head_precision"),
+        Linear(ops, "fc", he_normal(rng, inplanes, classes), np.zeros(classes, np.float32)),
+    ]
+    return Net(ops, layers, lr, momentum)
+
+
 # ------------------------------------------------------------------------------------ configurations
 
 CONFIGS = {
@@ -416,15 +556,23 @@ CONFIGS = {
     # reduced variants used where a CPU implementation has to keep up
     "smoke_cnn": (build_cnn, {"image": 16, "c1": 8, "c2": 16}, (3, 16, 16), 10, 4),
     "resnet18_small": (build_resnet18, {"classes": 100, "final_pool": 2}, (3, 64, 64), 100, 2),
+    # bottleneck network of the half-precision configuration (run with HalfHipOps), and a narrow one
+    "resnet50": (build_resnet50, {}, (3, 224, 224), 1000, 128),
+    "resnet50_small": (build_resnet50, {"classes": 100, "final_pool": 2, "widths": (16, 32, 64, 128)},
+                       (3, 64, 64), 100, 4),
 }
 
 SEED_BASE = 0x5167A000
+# per-configuration seed offsets (fixed numbers, so that adding a configuration leaves the inputs of
+# the others unchanged)
+_SEED_INDEX = {"cnn": 0, "mlp": 1, "resnet18": 2, "resnet18_small": 3, "smoke_cnn": 4, "resnet50": 5,
+               "resnet50_small": 6}
 
 
 def make_inputs(name, batch=None):
     builder, kw, xshape, classes, default_batch = CONFIGS[name]
     batch = batch or default_batch
-    r = np.random.default_rng(SEED_BASE + 17 * (sorted(CONFIGS).index(name) + 1) + batch)
+    r = np.random.default_rng(SEED_BASE + 17 * (_SEED_INDEX[name] + 1) + batch)
     x = r.standard_normal((batch,) + xshape).astype(np.float32)
     labels = r.integers(0, classes, size=batch).astype(np.int32)
     return x, labels
@@ -432,7 +580,7 @@ def make_inputs(name, batch=None):
 
 def build(name, ops, lr=0.05, momentum=0.9):
     builder, kw, _, _, _ = CONFIGS[name]
-    wr = np.random.default_rng(SEED_BASE + 1000 + sorted(CONFIGS).index(name))
+    wr = np.random.default_rng(SEED_BASE + 1000 + _SEED_INDEX[name])
     return builder(ops, wr, lr=lr, momentum=momentum, **kw)
 
 
@@ -463,13 +611,13 @@ def _nl2(a, b):
     return float(np.linalg.norm(a - b) / (d if d > 0 else 1.0))
 
 
-def run_parity_case(name, dev, checker_ops, batch=None, steps=1, share_activations=True):
+def run_parity_case(name, dev, checker_ops, batch=None, steps=1, share_activations=True, hip_ops=None):
     """Replays configuration `name` on the GPU and on `checker_ops` (an ops implementation handed
     in by the caller, e.g. the test-suite's CPU oracle) from identical inputs.  Both run their own
     forward (loss and logits are compared); with share_activations the GPU backward then consumes
     the checker's saved activations, so the reported errors are those of the backward kernels
     alone.  Returns per-tensor normalised L2 errors of every gradient and updated parameter."""
-    hip = HipOps(dev)
+    hip = hip_ops if hip_ops is not None else HipOps(dev)
     if not hasattr(checker_ops, "from_numpy"):
         raise TypeError("checker_ops must implement the ops interface")
     x, labels = make_inputs(name, batch)
