@@ -25,6 +25,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_16BIT_MFMA_TFLOPS = 2500.0   # dense fp16 / bf16 matrix peak
 PEAK_HBM_GBS = 8000.0
 # HBM bytes the 40 conv dgrad/wgrad MFMA launches of one default step move (fetched + written), from the
 # rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, each scaled by what the same counter reads for
@@ -82,6 +83,9 @@ def main():
     ap.add_argument("--cpu-sample-batch", type=int, default=32)
     ap.add_argument("--cpu-budget-s", type=float, default=10.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--storage", default="f32", choices=["f32", "f16", "bf16"],
+                    help="f16 / bf16: the mixed-precision tape (16-bit activations, gradients and conv weights, "
+                         "fp32 BatchNorm statistics and master weights), e.g. --config resnet50 --batch 128")
     ap.add_argument("--per-parameter-update", action="store_true",
                     help="update each parameter right after its gradient (one launch each) instead of one fused launch")
     args = ap.parse_args()
@@ -96,11 +100,12 @@ def main():
 
     lib = _lib.lib()
     dev = singa.create_hip_gpu_on(0)
-    hip = wl.HipOps(dev)
+    half = args.storage != "f32"
+    hip = wl.HalfHipOps(dev, singa.kFloat16 if args.storage == "f16" else singa.kBFloat16) if half else wl.HipOps(dev)
     net = wl.build(args.config, hip, lr=0.05, momentum=0.9)
     x, labels = wl.make_inputs(args.config, args.batch)
     net.forward(hip.from_numpy(x), hip.from_numpy(labels))
-    fused = not args.per_parameter_update
+    fused = not args.per_parameter_update and not half   # (the single-launch update covers fp32 parameters)
 
     def sync():
         dev.Sync()
@@ -126,17 +131,20 @@ def main():
     sync()
     prof = collect_prof(lib)
     lib.sgh_prof_enable(0)
-    conv = {k: prof[k] for k in ("conv_dgrad", "conv_wgrad") if k in prof}
+    conv = {k: prof[k] for k in ("conv_dgrad", "conv_wgrad", "conv_dgrad16", "conv_wgrad16") if k in prof}
     flop = sum(v["flop"] for v in conv.values())
     ms = sum(v["ms"] for v in conv.values())
     launches = sum(v["launches"] for v in conv.values())
     achieved = flop / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+    peak = PEAK_16BIT_MFMA_TFLOPS if half else PEAK_FP32_MFMA_TFLOPS
     roofline = {
-        "bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+        "bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
+        "frac": round(achieved / peak, 4),
         "traffic": CONV_HBM_BYTES_PER_STEP if (args.config == "resnet18" and args.batch == 64) else None,
         "traffic_unit": "HBM bytes per step over the same launches (PMC, calibrated)",
-        "kernel": "fp32 MFMA conv dgrad + wgrad kernels (k_dgrad3x3, k_wgrad3x3, k_dgrad_fewc, k_wgrad_fewc, k_igemm; %d launches/step)"
+        "kernel": ("16-bit MFMA conv dgrad + wgrad kernels (k_dgrad16, k_wgrad16; fp32 kernels for the stem dgrad; %d launches/step)"
+                   if half else
+                   "fp32 MFMA conv dgrad + wgrad kernels (k_dgrad3x3, k_wgrad3x3, k_dgrad_fewc, k_wgrad_fewc, k_igemm; %d launches/step)")
                   % (launches // prof_steps),
         "flop_per_step": flop / prof_steps, "kernel_ms_per_step": round(ms / prof_steps, 4),
     }
@@ -147,10 +155,13 @@ def main():
     roofline["entry_points_ms_per_step"] = round(ops_ms / prof_steps, 4)
 
     out = {
-        "metric": "backward+update imgs/sec, ResNet-18 N=64 fp32", "value": round(imgs_per_s, 2), "unit": "imgs/s",
+        "metric": "backward+update imgs/sec, ResNet-18 N=64 fp32" if (args.config == "resnet18" and not half and args.batch == 64)
+                  else "backward+update imgs/sec, %s N=%d %s" % (args.config, args.batch, args.storage),
+        "value": round(imgs_per_s, 2), "unit": "imgs/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "%s backward+update, N=%d, 3x224x224, fp32, SGD momentum 0.9" % (args.config, args.batch),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.storage, "data": "synthetic",
+        "config": {"workload": "%s backward+update, N=%d, 3x224x224, %s, SGD momentum 0.9" % (
+                       args.config, args.batch, "fp32" if not half else args.storage + " storage / fp32 accumulate, statistics and master weights"),
                    "update": "fused multi-tensor" if fused else "per parameter"},
         "roofline": roofline,
         "host_enqueue_ms_per_step": round(t_enqueued / args.steps * 1e3, 4),
