@@ -308,6 +308,17 @@ SGH_API int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma,
                            const float *save_mean, const float *save_invstd, float *dx,
                            float *dgamma, float *dbeta, int N, int C, int HW, void *workspace,
                            size_t ws_bytes, void *stream);
+/* ReLUBackward followed by GpuBatchNormBackward in one pass, for a ReLU whose input is this
+ * BatchNorm's output (python/singa/autograd.py:432-439 then batchnorm.cc:368-404; the tape of
+ * conv -> BatchNorm -> ReLU, examples/cnn/model/resnet.py:54-60).  `dy` is the gradient behind the
+ * ReLU; the BatchNorm output y = gamma*xhat + beta is recomputed from x exactly as the forward
+ * kernel stored it, and the gradient entering the BatchNorm is dy where y > 0, else 0.  Same
+ * outputs as the two separate calls, three tensor passes less.  *_f16 / *_bf16 below likewise. */
+SGH_API int sgh_bn_relu_bwd_f32(const float *dy, const float *x, const float *gamma,
+                                const float *beta, const float *save_mean,
+                                const float *save_invstd, float *dx, float *dgamma, float *dbeta,
+                                int N, int C, int HW, void *workspace, size_t ws_bytes,
+                                void *stream);
 /* The same two operations on 16-bit activations (x, y, dy, dx binary16 or bfloat16) with fp32
  * gamma / beta / statistics / parameter gradients -- cuDNN's convention for half tensors, which
  * the reference's handle selects from the input's data type (batchnorm.cc:261-285). */
@@ -327,6 +338,16 @@ SGH_API int sgh_bn_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *
                             const float *save_mean, const float *save_invstd, uint16_t *dx,
                             float *dgamma, float *dbeta, int N, int C, int HW, void *workspace,
                             size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma,
+                                const float *beta, const float *save_mean,
+                                const float *save_invstd, uint16_t *dx, float *dgamma,
+                                float *dbeta, int N, int C, int HW, void *workspace,
+                                size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma,
+                                 const float *beta, const float *save_mean,
+                                 const float *save_invstd, uint16_t *dx, float *dgamma,
+                                 float *dbeta, int N, int C, int HW, void *workspace,
+                                 size_t ws_bytes, void *stream);
 
 /* Geometry of a PoolingHandle (src/model/operation/pooling.h:40-71; ctor pooling.cc:27-52). */
 typedef struct sgh_pool_geom {

@@ -117,6 +117,9 @@ SIGNATURES = {
     "sgh_bn_fwd_train_bf16": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
                                         C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_bwd_f16": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_relu_bwd_f32": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_relu_bwd_f16": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_relu_bwd_bf16": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_bwd_bf16": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, sz, vp]),
     "sgh_pool_geom_init": (C.c_int, [C.POINTER(PoolGeom)] + [C.c_int] * 11),
     "sgh_pool_fwd_f32": (C.c_int, [C.POINTER(PoolGeom), vp, vp, vp]),

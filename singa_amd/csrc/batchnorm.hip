@@ -84,6 +84,12 @@ __device__ __forceinline__ void channel_range(const BnShape s, int c, int lo, in
   else channel_range_impl<NT, false, S>(s, c, lo, hi, x, dy, fv, f1);
 }
 
+// y = gamma * xhat + beta, written so that forward and the fused ReLU backward (which recomputes y
+// to find the elements the ReLU passed) round identically.
+__device__ __forceinline__ float bn_out(float v, float mean, float invstd, float g, float be) {
+  return __builtin_fmaf(g, (v - mean) * invstd, be);
+}
+
 // ---- forward, pass 1: per (c, split) partial sum and sum of squares about a pivot ---------
 // The pivot (the channel's first element) keeps the single-pass variance well conditioned.
 template <class S>
@@ -152,38 +158,51 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const typename S::elem 
       [&](size_t off, const float *v, const float *) {
         float r[S::VEC];
 #pragma unroll
-        for (int q = 0; q < S::VEC; ++q) r[q] = g * ((v[q] - mean) * invstd) + be;
+        for (int q = 0; q < S::VEC; ++q) r[q] = bn_out(v[q], mean, invstd, g, be);
         S::store16(y + off, r);
       },
-      [&](size_t off) { S::st(y + off, g * ((S::ld(x + off) - mean) * invstd) + be); });
+      [&](size_t off) { S::st(y + off, bn_out(S::ld(x + off), mean, invstd, g, be)); });
 }
 
 // ---- backward, pass 1: partial sum(dy) and sum(dy * xhat) ---------------------------------
-template <class S>
+// RELU: dy is the gradient behind a ReLU that consumed this BatchNorm's output; the gradient that
+// reaches the BatchNorm is dy where the recomputed output is > 0 and 0 elsewhere (ReLUBackward's
+// rule), applied on the fly instead of by a kernel of its own.
+template <class S, bool RELU>
 __global__ __launch_bounds__(kBlock) void k_bn_bwd_partial(const typename S::elem *__restrict__ dy,
                                                           const typename S::elem *__restrict__ x,
+                                                          const float *__restrict__ gamma, const float *__restrict__ beta,
                                                           const float *__restrict__ save_mean,
                                                           const float *__restrict__ save_invstd,
                                                           float *__restrict__ part, BnShape s) {
   __shared__ float red[16];
   const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
   const float mean = save_mean[c], invstd = save_invstd[c];
-  float a = 0.f, b = 0.f;
+  const float g = RELU ? gamma[c] : 0.f, be = RELU ? beta[c] : 0.f;
+  auto gate = [&](float d, float v) { return !RELU || S::stored(bn_out(v, mean, invstd, g, be)) > 0.f ? d : 0.f; };
+  // (the products are accumulated with explicit fused multiply-adds: the fused and the plain
+  // instantiation then round identically whatever the compiler does around the gate)
+  float a = 0.f, b = 0.f, b1 = 0.f;
   channel_range<kBlock, S>(
       s, c, sp * s.per_split, (sp + 1) * s.per_split, x, dy,
       [&](size_t, const float *v, const float *d) {
 #pragma unroll
         for (int q = 0; q < S::VEC; q += 4) {
-          a += (d[q] + d[q + 1]) + (d[q + 2] + d[q + 3]);
-          b += (d[q] * ((v[q] - mean) * invstd) + d[q + 1] * ((v[q + 1] - mean) * invstd)) +
-               (d[q + 2] * ((v[q + 2] - mean) * invstd) + d[q + 3] * ((v[q + 3] - mean) * invstd));
+          const float d0 = gate(d[q], v[q]), d1 = gate(d[q + 1], v[q + 1]), d2 = gate(d[q + 2], v[q + 2]),
+                      d3 = gate(d[q + 3], v[q + 3]);
+          a += (d0 + d1) + (d2 + d3);
+          b = __builtin_fmaf(d0, (v[q] - mean) * invstd, b);
+          b1 = __builtin_fmaf(d1, (v[q + 1] - mean) * invstd, b1);
+          b = __builtin_fmaf(d2, (v[q + 2] - mean) * invstd, b);
+          b1 = __builtin_fmaf(d3, (v[q + 3] - mean) * invstd, b1);
         }
       },
       [&](size_t off) {
-        const float d = S::ld(dy + off);
+        const float v = S::ld(x + off), d = gate(S::ld(dy + off), v);
         a += d;
-        b += d * ((S::ld(x + off) - mean) * invstd);
+        b = __builtin_fmaf(d, (v - mean) * invstd, b);
       });
+  b += b1;
   a = sgh_block_sum(a, red);
   b = sgh_block_sum(b, red);
   if (threadIdx.x == 0) {
@@ -193,10 +212,10 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_partial(const typename S::ele
 }
 
 // ---- backward, pass 2: dx = k * (dy - (dbeta + xhat * dgamma) / M), k = gamma * invstd -----
-template <class S>
+template <class S, bool RELU>
 __global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const typename S::elem *__restrict__ dy,
                                                         const typename S::elem *__restrict__ x,
-                                                        const float *__restrict__ gamma,
+                                                        const float *__restrict__ gamma, const float *__restrict__ beta,
                                                         const float *__restrict__ save_mean,
                                                         const float *__restrict__ save_invstd,
                                                         const float *__restrict__ part, typename S::elem *__restrict__ dx,
@@ -214,19 +233,23 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const typename S::elem 
     dgamma[c] = dg;
   }
   const float mean = save_mean[c], invstd = save_invstd[c];
-  const float k = gamma[c] * invstd;
+  const float g = gamma[c], be = RELU ? beta[c] : 0.f;
+  const float k = g * invstd;
   const float rM = float(1.0 / (double(s.N) * s.HW));
   const float c0 = db * rM, c1 = dg * rM;
+  auto gate = [&](float d, float v) { return !RELU || S::stored(bn_out(v, mean, invstd, g, be)) > 0.f ? d : 0.f; };
   channel_range<kBlock, S>(
       s, c, sp * s.per_split, (sp + 1) * s.per_split, x, dy,
       [&](size_t off, const float *v, const float *d) {
         float r[S::VEC];
 #pragma unroll
-        for (int q = 0; q < S::VEC; ++q) r[q] = k * (d[q] - (c0 + ((v[q] - mean) * invstd) * c1));
+        for (int q = 0; q < S::VEC; ++q)
+          r[q] = k * (gate(d[q], v[q]) - __builtin_fmaf((v[q] - mean) * invstd, c1, c0));
         S::store16(dx + off, r);
       },
       [&](size_t off) {
-        S::st(dx + off, k * (S::ld(dy + off) - (c0 + ((S::ld(x + off) - mean) * invstd) * c1)));
+        const float v = S::ld(x + off);
+        S::st(dx + off, k * (gate(S::ld(dy + off), v) - __builtin_fmaf((v - mean) * invstd, c1, c0)));
       });
 }
 
@@ -271,21 +294,30 @@ int bn_fwd_train(const typename S::elem *x, const float *gamma, const float *bet
   return SGH_OK;
 }
 
+// beta != NULL selects the fused ReLU + BatchNorm backward
 template <class S>
-int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *gamma, const float *save_mean,
-           const float *save_invstd, typename S::elem *dx, float *dgamma, float *dbeta, int N, int C, int HW,
-           void *workspace, size_t ws_bytes, void *stream) {
+int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *gamma, const float *beta,
+           const float *save_mean, const float *save_invstd, typename S::elem *dx, float *dgamma, float *dbeta, int N,
+           int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   if (!shape_ok(N, C, HW) || !dy || !x || !gamma || !save_mean || !save_invstd || !dx || !dgamma || !dbeta)
     return SGH_EINVAL;
   if (!sgh_aligned16(x) || !sgh_aligned16(dy) || !sgh_aligned16(dx)) return SGH_EINVAL;
   const BnShape s = make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem)));
   if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
   float *part = static_cast<float *>(workspace);
-  hipLaunchKernelGGL(k_bn_bwd_partial<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, save_mean,
-                     save_invstd, part, s);
-  SGH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_bn_bwd_apply<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, gamma, save_mean,
-                     save_invstd, part, dx, dgamma, dbeta, s);
+  const dim3 grid(C * s.S), block(kBlock);
+  hipStream_t st = sgh_stream_of(stream);
+  if (beta) {
+    hipLaunchKernelGGL((k_bn_bwd_partial<S, true>), grid, block, 0, st, dy, x, gamma, beta, save_mean, save_invstd, part, s);
+    SGH_LAUNCH_CHECK();
+    hipLaunchKernelGGL((k_bn_bwd_apply<S, true>), grid, block, 0, st, dy, x, gamma, beta, save_mean, save_invstd, part,
+                       dx, dgamma, dbeta, s);
+  } else {
+    hipLaunchKernelGGL((k_bn_bwd_partial<S, false>), grid, block, 0, st, dy, x, gamma, beta, save_mean, save_invstd, part, s);
+    SGH_LAUNCH_CHECK();
+    hipLaunchKernelGGL((k_bn_bwd_apply<S, false>), grid, block, 0, st, dy, x, gamma, beta, save_mean, save_invstd, part,
+                       dx, dgamma, dbeta, s);
+  }
   SGH_LAUNCH_CHECK();
   return SGH_OK;
 }
@@ -323,17 +355,42 @@ int sgh_bn_fwd_train_bf16(const uint16_t *x, const float *gamma, const float *be
 int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const float *save_mean,
                    const float *save_invstd, float *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                    void *workspace, size_t ws_bytes, void *stream) {
-  return bn_bwd<StF32>(dy, x, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes, stream);
+  return bn_bwd<StF32>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                       stream);
 }
 int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                    const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                    void *workspace, size_t ws_bytes, void *stream) {
-  return bn_bwd<StF16>(dy, x, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes, stream);
+  return bn_bwd<StF16>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                       stream);
 }
 int sgh_bn_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                     const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                     void *workspace, size_t ws_bytes, void *stream) {
-  return bn_bwd<StBF16>(dy, x, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes, stream);
+  return bn_bwd<StBF16>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                        stream);
+}
+
+int sgh_bn_relu_bwd_f32(const float *dy, const float *x, const float *gamma, const float *beta, const float *save_mean,
+                        const float *save_invstd, float *dx, float *dgamma, float *dbeta, int N, int C, int HW,
+                        void *workspace, size_t ws_bytes, void *stream) {
+  if (!beta) return SGH_EINVAL;
+  return bn_bwd<StF32>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                       stream);
+}
+int sgh_bn_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *beta,
+                        const float *save_mean, const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta,
+                        int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  if (!beta) return SGH_EINVAL;
+  return bn_bwd<StF16>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                       stream);
+}
+int sgh_bn_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *beta,
+                         const float *save_mean, const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta,
+                         int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  if (!beta) return SGH_EINVAL;
+  return bn_bwd<StBF16>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                        stream);
 }
 
 }  // extern "C"

@@ -34,6 +34,7 @@ struct StF32 {
   static constexpr int VEC = 4;
   static __device__ __forceinline__ float ld(const elem *p) { return *p; }
   static __device__ __forceinline__ void st(elem *p, float v) { *p = v; }
+  static __device__ __forceinline__ float stored(float v) { return v; }  // the value a store keeps
   template <bool NT>
   static __device__ __forceinline__ void load16(const elem *p, float *out) {
     const sgh_v4f v = NT ? __builtin_nontemporal_load(reinterpret_cast<const sgh_v4f *>(p))
@@ -54,6 +55,7 @@ struct St16 {
   static constexpr int VEC = 8;
   static __device__ __forceinline__ float ld(const elem *p) { return LD(*p); }
   static __device__ __forceinline__ void st(elem *p, float v) { *p = ST(v); }
+  static __device__ __forceinline__ float stored(float v) { return LD(ST(v)); }  // the value a store keeps
   template <bool NT>
   static __device__ __forceinline__ void load16(const elem *p, float *out) {
     const sgh_v4u v = NT ? __builtin_nontemporal_load(reinterpret_cast<const sgh_v4u *>(p))

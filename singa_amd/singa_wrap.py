@@ -596,6 +596,22 @@ def GpuBatchNormBackward(h, dy, x, scale, mean, var):
     return [dx, ds, db]
 
 
+def GpuBatchNormReLUBackward(h, dy, x, scale, bias, mean, var):
+    """``GpuBatchNormBackward(h, ReLUBackward(dy, y), x, scale, mean, var)`` for ``y`` = this
+    BatchNorm's output, in one pass: ``y`` is recomputed from ``x`` instead of being read, and the
+    ReLU's gradient is never written (the conv -> BatchNorm -> ReLU tape of
+    examples/cnn/model/resnet.py:54-60).  Returns ``[dx, dscale, dbias]``."""
+    _same(dy, x)
+    dx = _like(dy)
+    ds = _like(scale)
+    db = _like(scale)
+    fn, name = _fn("bn_relu_bwd", dy)
+    check(fn(dy.ptr, x.ptr, scale.ptr, bias.ptr, mean.ptr, var.ptr, dx.ptr, ds.ptr, db.ptr,
+             h.batchsize, h.channels, h.height * h.width, h.workspace.ptr,
+             h.workspace.MemSize(), dy.device().stream), name)
+    return [dx, ds, db]
+
+
 class CudnnPoolingHandle(object):
     """``CudnnPoolingHandle(x, kernel, stride, padding, is_max)``
     (src/model/operation/pooling.h:40-91)."""

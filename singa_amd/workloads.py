@@ -105,6 +105,12 @@ class HipOps(object):
     def bn_bwd(self, h, dy, x, g, mean, var):
         return singa.GpuBatchNormBackward(h, dy, x, g, mean, var)
 
+    # cross-op fusion the tape permits: the ReLU behind a BatchNorm folded into its backward
+    fuse_bn_relu = True
+
+    def bn_relu_bwd(self, h, dy, x, g, b, mean, var):
+        return singa.GpuBatchNormReLUBackward(h, dy, x, g, b, mean, var)
+
     def conv_bwd_x(self, dy, W, x, h):
         return singa.GpuConvBackwardx(dy, W, x, h)
 
@@ -228,6 +234,16 @@ class BatchNorm(_Layer):
         grads(self.name + ".bias", self.bias, db)
         return dx
 
+    def bwd_through_relu(self, relu, dy, grads):
+        """Backward of ``relu(self(x))``: ReLU.backward then BatchNorm.backward, as one fused call
+        where the ops implementation offers it."""
+        if not getattr(self.ops, "fuse_bn_relu", False):
+            return self.bwd(relu.bwd(dy, grads), grads)
+        dx, ds, db = self.ops.bn_relu_bwd(self.h, dy, self.x, self.scale, self.bias, self.mean, self.var)
+        grads(self.name + ".scale", self.scale, ds)
+        grads(self.name + ".bias", self.bias, db)
+        return dx
+
 
 class ReLU(_Layer):
     def __init__(self, ops, name):
@@ -338,8 +354,8 @@ class BasicBlock(_Layer):
             d_res = self.ds_conv.bwd(self.ds_bn.bwd(d_add, grads), grads)
         else:
             d_res = d_add
-        d_main = self.conv1.bwd(self.bn1.bwd(self.relu1.bwd(self.conv2.bwd(self.bn2.bwd(d_add, grads), grads), grads),
-                                             grads), grads)
+        d_main = self.conv1.bwd(self.bn1.bwd_through_relu(self.relu1, self.conv2.bwd(self.bn2.bwd(d_add, grads), grads),
+                                                          grads), grads)
         if d_res is d_add:
             # the first-arrived buffer is another op's input gradient: accumulate into the fresh one
             return self.ops.accumulate(d_main, d_res)
@@ -391,8 +407,8 @@ class Bottleneck(_Layer):
         else:
             d_res = d_add
         d = self.conv3.bwd(self.bn3.bwd(d_add, grads), grads)
-        d = self.conv2.bwd(self.bn2.bwd(self.relu2.bwd(d, grads), grads), grads)
-        d_main = self.conv1.bwd(self.bn1.bwd(self.relu1.bwd(d, grads), grads), grads)
+        d = self.conv2.bwd(self.bn2.bwd_through_relu(self.relu2, d, grads), grads)
+        d_main = self.conv1.bwd(self.bn1.bwd_through_relu(self.relu1, d, grads), grads)
         if d_res is d_add:
             return self.ops.accumulate(d_main, d_res)
         return self.ops.accumulate(d_res, d_main)
@@ -464,8 +480,15 @@ class Net(object):
         dy = ops.softmax_ce_bwd(self.p, self.t, self.batch)
         if keep_grads:
             self.grad_log["logits"] = dy
-        for l in reversed(self.layers):
-            dy = l.bwd(dy, grads)
+        rev = list(reversed(self.layers))
+        i = 0
+        while i < len(rev):
+            if isinstance(rev[i], ReLU) and i + 1 < len(rev) and isinstance(rev[i + 1], BatchNorm):
+                dy = rev[i + 1].bwd_through_relu(rev[i], dy, grads)   # the stem's conv -> BatchNorm -> ReLU
+                i += 2
+            else:
+                dy = rev[i].bwd(dy, grads)
+                i += 1
         if keep_grads:
             self.grad_log["input"] = dy
         if fused_update:

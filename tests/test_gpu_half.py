@@ -120,6 +120,46 @@ def test_batchnorm_16bit_storage(singa, dev, kind, shape):
     assert nl2(ds.to_numpy(), ds_o) < 1e-3 and nl2(db.to_numpy(), db_o) < 1e-3
 
 
+@pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 28, 28), (16, 32, 8, 8), (3, 7, 4, 2),
+                                   (32, 64, 56, 56)])
+def test_fused_relu_batchnorm_backward(singa, dev, kind, shape):
+    """The fused ReLU + BatchNorm backward equals ReLUBackward followed by GpuBatchNormBackward on
+    the forward's own output BIT FOR BIT (the recomputed output selects the same elements as the
+    stored one, zeros and 16-bit underflow included), in every storage type; and it matches the
+    oracle's composition of the two ops."""
+    from oracle import cpu_oracle as O
+    from util import nl2
+    r = rng(sum(shape) + 3)
+    N, C, H, W = shape
+    x32 = (r.standard_normal(shape) * 1.5 - 0.2).astype(np.float32)
+    x32.ravel()[::17] = x32.ravel()[1]          # repeated values
+    dy32 = r.standard_normal(shape).astype(np.float32)
+    gamma = (1 + 0.3 * r.standard_normal(C)).astype(np.float32)
+    beta = (0.2 * r.standard_normal(C)).astype(np.float32)
+    gamma[0], beta[0] = 0.0, 0.0                # a channel whose output is exactly 0 everywhere: ReLU passes nothing
+    if C > 1:
+        gamma[1], beta[1] = 1e-6, 1e-8          # tiny outputs: underflow to zero in binary16
+    if kind == "f32":
+        xt, x, dyt, dy = singa.from_numpy(x32, dev), x32, singa.from_numpy(dy32, dev), dy32
+    else:
+        xt, x = _to(singa, dev, x32, kind)
+        dyt, dy = _to(singa, dev, dy32, kind)
+    gd, bd = singa.from_numpy(gamma, dev), singa.from_numpy(beta, dev)
+    h = singa.CudnnBatchNormHandle(0.9, xt)
+    y, mean, var = singa.GpuBatchNormForwardTraining(h, xt, gd, bd, None, None)
+    two = singa.GpuBatchNormBackward(h, singa.ReLUBackward(dyt, y), xt, gd, mean, var)
+    one = singa.GpuBatchNormReLUBackward(h, dyt, xt, gd, bd, mean, var)
+    for a, b, what in zip(one, two, ("dx", "dscale", "dbias")):
+        _same_bits(a.to_numpy(), b.to_numpy(), "fused vs separate " + what + " " + kind)
+    y_o, mean_o, invstd_o = O.bn_fwd_train(x, gamma, beta, np.zeros(C, np.float32), np.ones(C, np.float32), 0.9, 1e-5)
+    ynp = y.to_numpy()                          # the selection is made on the GPU's stored output
+    dx_o, ds_o, db_o = O.bn_bwd(O.relu_bwd(dy, ynp), x, gamma, mean.to_numpy(), var.to_numpy())
+    tol = 1e-3 if kind == "f32" else 1e-2
+    assert nl2(one[0].to_numpy(), dx_o) < tol
+    assert nl2(one[1].to_numpy(), ds_o) < 1e-3 and nl2(one[2].to_numpy(), db_o) < 1e-3
+
+
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("case", [
     (2, 3, 8, 8, (2, 2), (2, 2), (0, 0)),
