@@ -87,7 +87,7 @@ def main():
                     help="f16 / bf16: the mixed-precision tape (16-bit activations, gradients and conv weights, "
                          "fp32 BatchNorm statistics and master weights), e.g. --config resnet50 --batch 128")
     ap.add_argument("--no-fusion", action="store_true",
-                    help="run ReLU backward and BatchNorm backward as the two separate calls of the reference's tape")
+                    help="one call per op of the reference's tape (no ReLU+BatchNorm backward fusion, residual += as its own kernel)")
     ap.add_argument("--per-parameter-update", action="store_true",
                     help="update each parameter right after its gradient (one launch each) instead of one fused launch")
     args = ap.parse_args()
@@ -104,7 +104,7 @@ def main():
     dev = singa.create_hip_gpu_on(0)
     half = args.storage != "f32"
     hip = wl.HalfHipOps(dev, singa.kFloat16 if args.storage == "f16" else singa.kBFloat16) if half else wl.HipOps(dev)
-    hip.fuse_bn_relu = not args.no_fusion
+    hip.fuse_bn_relu = hip.fuse_dgrad_add = not args.no_fusion
     net = wl.build(args.config, hip, lr=0.05, momentum=0.9)
     x, labels = wl.make_inputs(args.config, args.batch)
     net.forward(hip.from_numpy(x), hip.from_numpy(labels))
@@ -166,7 +166,8 @@ def main():
         "config": {"workload": "%s backward+update, N=%d, 3x224x224, %s, SGD momentum 0.9" % (
                        args.config, args.batch, "fp32" if not half else args.storage + " storage / fp32 accumulate, statistics and master weights"),
                    "update": "fused multi-tensor" if fused else "per parameter",
-                   "tape": "ReLU backward folded into BatchNorm backward (conv-BN-ReLU)" if hip.fuse_bn_relu
+                   "tape": "ReLU backward folded into BatchNorm backward (conv-BN-ReLU), residual += folded into the data gradient"
+                           if hip.fuse_bn_relu
                            else "one call per reference op"},
         "roofline": roofline,
         "host_enqueue_ms_per_step": round(t_enqueued / args.steps * 1e3, 4),

@@ -253,6 +253,14 @@ SGH_API size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which);
  * dx[n,c,h,w] = sum_{k,r,s} dy[n,k,p,q] * W[k,c,r,s], h = p*stride - pad + r. */
 SGH_API int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx,
                                void *workspace, size_t ws_bytes, void *stream);
+/* dx += the data gradient: cudnnConvolutionBackwardData's beta = 1 (the reference passes beta = 0,
+ * convolution.cc:649-654, and sums gradients that fan in with a separate `+=`,
+ * python/singa/autograd.py:204).  Each element is computed exactly as above and then added to the
+ * value already in dx, so the result equals the separate call followed by `dx_old += result`.
+ * Covered by the shared-tile kernels (3x3, pad 1, stride 1, or stride 2 on even images, C >= 64,
+ * K a multiple of 16); SGH_EUNSUPPORTED otherwise, with dx untouched. */
+SGH_API int sgh_conv_dgrad_acc_f32(const sgh_conv_geom *g, const float *dy, const float *W,
+                                   float *dx, void *workspace, size_t ws_bytes, void *stream);
 /* GpuConvBackwardW (src/model/operation/convolution.cc:658-681; native algorithm
  * src/model/layer/convolution.cc:166-177 + Im2col :197-222):
  * dW[k,c,r,s] = sum_{n,p,q} dy[n,k,p,q] * x[n,c,p*stride-pad+r,q*stride-pad+s].

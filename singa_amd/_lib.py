@@ -96,6 +96,7 @@ SIGNATURES = {
     "sgh_conv_geom_init": (C.c_int, [C.POINTER(ConvGeom)] + [C.c_int] * 11),
     "sgh_conv_workspace_bytes": (sz, [C.POINTER(ConvGeom), C.c_int]),
     "sgh_conv_dgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
+    "sgh_conv_dgrad_acc_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_wgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_bgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp]),
     "sgh_conv_fwd_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
@@ -131,6 +132,7 @@ SIGNATURES = {
 }
 
 SGH_CONV_FWD, SGH_CONV_DGRAD, SGH_CONV_WGRAD = 0, 1, 2
+SGH_EUNSUPPORTED = -3
 
 
 class SingaHipError(RuntimeError):

@@ -54,8 +54,9 @@ bool sgh_dgrad3x3_supported(const sgh_conv_geom *g);
 size_t sgh_dgrad3x3_partial_bytes(const sgh_conv_geom *g);  // scratch for split-reduction partial images
 // `tag` names the profiling record; `bias` (may be NULL) is added per output channel -- the forward
 // convolution runs through this kernel as the data gradient of the channel-swapped problem.
+// `accumulate`: dx += result (the sum in the fixed order result-then-add of the separate "+=").
 int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, int KP, float *dx, float *partials,
-                     hipStream_t s, const char *tag, const float *bias);
+                     hipStream_t s, const char *tag, const float *bias, bool accumulate);
 
 // Stride-2 data gradient for at most four input channels and a large filter (the 7x7 stem),
 // dgrad_fewc.hip: direct 16-row MFMA kernel, W in its native [K][C][R][S] layout.

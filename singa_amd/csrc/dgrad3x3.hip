@@ -42,6 +42,7 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
 struct D3Args {
   const float *dy, *wt;   // wt: re-laid weights [tap][KP][C]
   const float *bias;      // per output channel, added when a tile is finished (NULL: none)
+  int accumulate;         // dx += result instead of dx = result (gradient fan-in folded into the store)
   float *dx;
   int N, C, H, W, K, KP;  // dx is N x C x H x W
   int P, Q;               // dy is N x K x P x Q (stride 1: P == H, Q == W; stride 2: H == 2P, W == 2Q)
@@ -263,8 +264,11 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
           if (c < a.C) {
             const float bb = a.bias ? a.bias[c] : 0.f;
             float *oc = o + size_t(c) * HW;
-            *reinterpret_cast<v2f *>(oc) = v2f{acc[0 * TM + i][v] + bb, acc[1 * TM + i][v] + bb};
-            *reinterpret_cast<v2f *>(oc + a.W) = v2f{acc[2 * TM + i][v] + bb, acc[3 * TM + i][v] + bb};
+            v2f r0 = v2f{acc[0 * TM + i][v] + bb, acc[1 * TM + i][v] + bb};
+            v2f r1 = v2f{acc[2 * TM + i][v] + bb, acc[3 * TM + i][v] + bb};
+            if (a.accumulate) r0 += *reinterpret_cast<const v2f *>(oc), r1 += *reinterpret_cast<const v2f *>(oc + a.W);
+            *reinterpret_cast<v2f *>(oc) = r0;
+            *reinterpret_cast<v2f *>(oc + a.W) = r1;
           }
         }
     } else {
@@ -274,7 +278,11 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int c = c0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * lhalf + (v & 3);
-          if (c < a.C) o[size_t(c) * HW] = a.bias ? acc[i][v] + a.bias[c] : acc[i][v];
+          if (c < a.C) {
+            float r = a.bias ? acc[i][v] + a.bias[c] : acc[i][v];
+            if (a.accumulate) r += o[size_t(c) * HW];
+            o[size_t(c) * HW] = r;
+          }
         }
     }
   }
@@ -322,7 +330,8 @@ __global__ __launch_bounds__(256) void k_dgrad3x3_fixup(D3Args a) {
   int pix = pix0 + col;
   int pn = pix / PQ, prem = pix - pn * PQ;
   if (!S2 && (PQ & 3) == 0 && pix + 3 < a.total_pix) {  // the four pixels lie in one image, 16-byte aligned
-    *reinterpret_cast<v4f *>(a.dx + (size_t(pn) * a.C + c) * HW + prem) = s[0] + bb;
+    v4f *o = reinterpret_cast<v4f *>(a.dx + (size_t(pn) * a.C + c) * HW + prem);
+    *o = a.accumulate ? *o + (s[0] + bb) : s[0] + bb;
     return;
   }
 #pragma unroll
@@ -331,10 +340,14 @@ __global__ __launch_bounds__(256) void k_dgrad3x3_fixup(D3Args a) {
     if (S2) {
       const int i = prem / a.Q, jj = prem - i * a.Q;
       float *o = a.dx + (size_t(pn) * a.C + c) * HW + (2 * i) * a.W + 2 * jj;
-      *reinterpret_cast<v2f *>(o) = v2f{s[0][j] + bb, s[NCLS > 1 ? 1 : 0][j] + bb};
-      *reinterpret_cast<v2f *>(o + a.W) = v2f{s[NCLS > 2 ? 2 : 0][j] + bb, s[NCLS > 3 ? 3 : 0][j] + bb};
+      v2f r0 = v2f{s[0][j] + bb, s[NCLS > 1 ? 1 : 0][j] + bb};
+      v2f r1 = v2f{s[NCLS > 2 ? 2 : 0][j] + bb, s[NCLS > 3 ? 3 : 0][j] + bb};
+      if (a.accumulate) r0 += *reinterpret_cast<const v2f *>(o), r1 += *reinterpret_cast<const v2f *>(o + a.W);
+      *reinterpret_cast<v2f *>(o) = r0;
+      *reinterpret_cast<v2f *>(o + a.W) = r1;
     } else {
-      a.dx[(size_t(pn) * a.C + c) * HW + prem] = s[0][j] + bb;
+      float *o = a.dx + (size_t(pn) * a.C + c) * HW + prem;
+      *o = a.accumulate ? *o + (s[0][j] + bb) : s[0][j] + bb;
     }
     if (++prem == PQ) prem = 0, ++pn;
   }
@@ -433,7 +446,7 @@ size_t sgh_dgrad3x3_partial_bytes(const sgh_conv_geom *g) {
 // `wt` holds the weights re-laid as [tap][KP][C] (KP = K rounded up to 16, zero rows beyond K);
 // `partials` is sgh_dgrad3x3_partial_bytes(g) bytes of scratch (may be NULL when that is 0).
 int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, int KP, float *dx, float *partials,
-                     hipStream_t s, const char *tag, const float *bias) {
+                     hipStream_t s, const char *tag, const float *bias, bool accumulate) {
   const D3Plan p = plan(g);
   if (!p.ok) return SGH_EUNSUPPORTED;
   if (p.sk_wgs > 0 && !partials) return SGH_EWORKSPACE;
@@ -441,6 +454,7 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   a.dy = dy;
   a.wt = wt;
   a.bias = bias;
+  a.accumulate = accumulate ? 1 : 0;
   a.dx = dx;
   a.N = g->N;
   a.C = g->C;

@@ -904,14 +904,15 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
   }
 }
 
-int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
-                       size_t ws_bytes, void *stream) {
+static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
+                      size_t ws_bytes, void *stream, bool accumulate) {
   if (!conv_ok(g) || !dy || !W || !dx) return SGH_EINVAL;
   const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_DGRAD);
   if (need && (!workspace || ws_bytes < need)) return SGH_EWORKSPACE;
   hipStream_t s = sgh_stream_of(stream);
   const int RS = g->R * g->S, KP = round_up(g->K, BK);
   const DgradPath path = dgrad_path(g);
+  if (accumulate && path != kDgradTile3x3) return SGH_EUNSUPPORTED;  // only the shared-tile kernels add into dx
   int rc = SGH_OK;
   sgh_prof_start("conv_dgrad_op", conv_flops(g), s);
 
@@ -965,7 +966,7 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
     float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) +
                                                 align256(size_t(RS) * KP * g->C * sizeof(float)) +
                                                 align256(sizeof(DgClsTable)));
-    rc = sgh_dgrad3x3_run(g, dy, Wt, KP, dx, partials, s, "conv_dgrad", nullptr);
+    rc = sgh_dgrad3x3_run(g, dy, Wt, KP, dx, partials, s, "conv_dgrad", nullptr, accumulate);
   } else if (path == kDgradClasses) {
     float *Wc = static_cast<float *>(workspace);
     const size_t wc_bytes = size_t(RS) * KP * g->C * sizeof(float);
@@ -1045,6 +1046,16 @@ int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, 
   return SGH_OK;
 }
 
+int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
+                       size_t ws_bytes, void *stream) {
+  return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, false);
+}
+
+int sgh_conv_dgrad_acc_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
+                           size_t ws_bytes, void *stream) {
+  return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, true);
+}
+
 int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, const float *bias, float *y,
                      void *workspace, size_t ws_bytes, void *stream) {
   if (!conv_ok(g) || !x || !W || !y) return SGH_EINVAL;
@@ -1063,7 +1074,7 @@ int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, con
     hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, CP, 2);
     float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) +
                                                 align256(size_t(RS) * CP * g->K * sizeof(float)));
-    const int rc3 = sgh_dgrad3x3_run(&gt, x, Wt, CP, y, partials, s, "conv_fwd", bias);
+    const int rc3 = sgh_dgrad3x3_run(&gt, x, Wt, CP, y, partials, s, "conv_fwd", bias, false);
     sgh_prof_stop(s);
     return rc3;
   }

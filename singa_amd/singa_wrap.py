@@ -520,6 +520,22 @@ def GpuConvForward(x, W, b, h):
     return y
 
 
+def GpuConvBackwardxAccumulate(dy, W, x, h, dx):
+    """``dx += GpuConvBackwardx(dy, W, x, h)`` in place, returning ``dx``: the gradient fan-in of a
+    residual connection (``+=``, python/singa/autograd.py:204) folded into the store of the data
+    gradient where the kernel supports it, otherwise the two separate steps."""
+    h._check_dy(dy)
+    _same(dx, x)
+    if dy.data_type() == kFloat32:
+        rc = _L().sgh_conv_dgrad_acc_f32(C.byref(h.geom), dy.ptr, W.ptr, dx.ptr, h.workspace.ptr,
+                                         h.workspace.MemSize(), dy.device().stream)
+        if rc != _lib.SGH_EUNSUPPORTED:
+            check(rc, "sgh_conv_dgrad_acc_f32")
+            return dx
+    dx += GpuConvBackwardx(dy, W, x, h)
+    return dx
+
+
 def GpuConvBackwardx(dy, W, x, h):
     h._check_dy(dy)
     dx = _like(x)

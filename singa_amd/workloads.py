@@ -117,6 +117,12 @@ class HipOps(object):
     def conv_bwd_w(self, dy, x, W, h):
         return singa.GpuConvBackwardW(dy, x, W, h)
 
+    # cross-op fusion the tape permits: the "+=" of a residual fan-in folded into the data gradient
+    fuse_dgrad_add = True
+
+    def conv_bwd_x_acc(self, dy, W, x, h, into):
+        return singa.GpuConvBackwardxAccumulate(dy, W, x, h, into)
+
     def conv_bwd_b(self, dy, b, h):
         return singa.GpuConvBackwardb(dy, b, h)
 
@@ -200,9 +206,15 @@ class Conv(_Layer):
         self.x = x
         return self.ops.conv_fwd(x, self.W, self.b, self.h)
 
-    def bwd(self, dy, grads):
+    def bwd(self, dy, grads, add_into=None):
+        """`add_into`: a gradient of this convolution's input that arrived earlier over another
+        branch; the data gradient is added into that tensor (ops implementations with
+        ``fuse_dgrad_add``), which is returned."""
         # _Conv2d.backward: dx is always computed, even for the network input (autograd.py:1695-1697)
-        dx = self.ops.conv_bwd_x(dy, self.W, self.x, self.h)
+        if add_into is not None:
+            dx = self.ops.conv_bwd_x_acc(dy, self.W, self.x, self.h, add_into)
+        else:
+            dx = self.ops.conv_bwd_x(dy, self.W, self.x, self.h)
         grads(self.name + ".W", self.W, self.ops.conv_bwd_w(dy, self.x, self.W, self.h))
         if self.b is not None:
             grads(self.name + ".b", self.b, self.ops.conv_bwd_b(dy, self.b, self.h))
@@ -354,8 +366,10 @@ class BasicBlock(_Layer):
             d_res = self.ds_conv.bwd(self.ds_bn.bwd(d_add, grads), grads)
         else:
             d_res = d_add
-        d_main = self.conv1.bwd(self.bn1.bwd_through_relu(self.relu1, self.conv2.bwd(self.bn2.bwd(d_add, grads), grads),
-                                                          grads), grads)
+        d = self.bn1.bwd_through_relu(self.relu1, self.conv2.bwd(self.bn2.bwd(d_add, grads), grads), grads)
+        if getattr(self.ops, "fuse_dgrad_add", False):
+            return self.conv1.bwd(d, grads, add_into=d_res)   # every other reader of d_res is done by now
+        d_main = self.conv1.bwd(d, grads)
         if d_res is d_add:
             # the first-arrived buffer is another op's input gradient: accumulate into the fresh one
             return self.ops.accumulate(d_main, d_res)
@@ -408,7 +422,10 @@ class Bottleneck(_Layer):
             d_res = d_add
         d = self.conv3.bwd(self.bn3.bwd(d_add, grads), grads)
         d = self.conv2.bwd(self.bn2.bwd_through_relu(self.relu2, d, grads), grads)
-        d_main = self.conv1.bwd(self.bn1.bwd_through_relu(self.relu1, d, grads), grads)
+        d = self.bn1.bwd_through_relu(self.relu1, d, grads)
+        if getattr(self.ops, "fuse_dgrad_add", False):
+            return self.conv1.bwd(d, grads, add_into=d_res)
+        d_main = self.conv1.bwd(d, grads)
         if d_res is d_add:
             return self.ops.accumulate(d_main, d_res)
         return self.ops.accumulate(d_res, d_main)

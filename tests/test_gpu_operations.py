@@ -126,6 +126,32 @@ def test_conv_wgrad_is_deterministic(singa, dev):
         assert_bit_equal(singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy(), a, "split-K reduction order")
 
 
+@pytest.mark.parametrize("n,c,hw,k,r,stride,pad", [
+    (40, 64, 56, 64, 3, 1, 1),    # shared remainder tiles: whole-tile stores and the fix-up pass both add
+    (16, 256, 14, 256, 3, 1, 1),  # every tile shared
+    (16, 64, 28, 128, 3, 2, 1),   # residue-class kernel
+    (3, 64, 9, 64, 3, 1, 1),      # odd image, tiles straddle images
+    (4, 64, 16, 128, 1, 2, 0),    # not covered by the accumulating kernels: the two-step fallback
+    (2, 8, 12, 16, 5, 1, 2),      # generic path: fallback
+])
+def test_conv_dgrad_accumulate(singa, dev, n, c, hw, k, r, stride, pad):
+    """dx += dgrad (the residual fan-in folded into the data gradient) equals the separate data
+    gradient followed by "+=" bit for bit, on the kernels that add in their store and on the
+    fallback alike."""
+    rg = rng(23)
+    p = (hw + 2 * pad - r) // stride + 1
+    x, dy = randn(rg, n, c, hw, hw), randn(rg, n, k, p, p)
+    w, base = randn(rg, k, c, r, r), randn(rg, n, c, hw, hw)
+    xd, wd, dyd = singa.from_numpy(x, dev), singa.from_numpy(w, dev), singa.from_numpy(dy, dev)
+    h = singa.CudnnConvHandle(xd, (r, r), (stride, stride), (pad, pad), c, k, False)
+    want = singa.from_numpy(base, dev)
+    want += singa.GpuConvBackwardx(dyd, wd, xd, h)
+    acc = singa.from_numpy(base, dev)
+    got = singa.GpuConvBackwardxAccumulate(dyd, wd, xd, h, acc)
+    assert got is acc
+    assert_bit_equal(got.to_numpy(), want.to_numpy(), "accumulating dgrad")
+
+
 @pytest.mark.parametrize("n,c,hw,k,stride", [
     (40, 64, 56, 64, 1),     # 980 tiles: three whole rounds of tiles plus a shared remainder
     (16, 256, 14, 256, 1),   # fewer tiles than CUs: every tile is shared between workgroups

@@ -135,3 +135,21 @@ def test_resnet50_bottleneck_16bit_step(dev, kind):
         worst = sorted(d.items(), key=lambda kv: -kv[1])[:4]
         print(what, "worst:", ", ".join("%s=%.2e" % kv for kv in worst))
         assert len(d) > 100 and worst[0][1] < tol
+
+
+def test_fused_tape_equals_reference_tape(dev):
+    """The tape with ReLU backward folded into BatchNorm backward and the residual "+=" folded into
+    the data gradient leaves bit-identical parameters and input gradient to the tape that makes
+    one call per reference op."""
+    x, labels = wl.make_inputs("resnet18_small", 2)
+    outs = []
+    for fuse in (False, True):
+        hip = wl.HipOps(dev)
+        hip.fuse_bn_relu = hip.fuse_dgrad_add = fuse
+        net = wl.build("resnet18_small", hip)
+        for _ in range(2):
+            net.forward(hip.from_numpy(x), hip.from_numpy(labels))
+            dx = net.backward_and_update()
+        outs.append([hip.to_numpy(dx)] + [hip.to_numpy(p) for _, p in net.params()])
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
