@@ -145,6 +145,15 @@ SGH_API int sgh_eltwise_mult_f32(const float *a, const float *b, int b_is_scalar
 /* Add<float, Lang> (Tensor::operator+=, src/core/tensor/tensor.cc:579-586): gradient fan-in
  * of python/singa/autograd.py:204.  out may alias a or b. */
 SGH_API int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream);
+/* The other elementwise tensor functions the autograd ops of these models call around the
+ * backward path (src/core/tensor/tensor_math_cpp.h): Sub :645-650, Div (tensor / tensor) :423-430,
+ * Add(tensor, scalar) :383-388, EltwiseMult(tensor, scalar) :432-437.  Div(tensor, scalar) is
+ * EltwiseMult by the fp32 reciprocal in the reference (tensor_math.h:149-153): callers pass 1/x to
+ * sgh_mult_scalar_f32.  out may alias an input. */
+SGH_API int sgh_sub_f32(const float *a, const float *b, float *out, size_t n, void *stream);
+SGH_API int sgh_div_f32(const float *a, const float *b, float *out, size_t n, void *stream);
+SGH_API int sgh_add_scalar_f32(const float *a, float x, float *out, size_t n, void *stream);
+SGH_API int sgh_mult_scalar_f32(const float *a, float x, float *out, size_t n, void *stream);
 
 /* -------------------------------------------------------------------------------------
  * 16-bit storage variants: IEEE binary16 ("f16", the reference's half_float::half / __half
@@ -309,6 +318,11 @@ SGH_API int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float
                                  float *running_mean, float *running_var, float factor, float eps,
                                  float *y, float *save_mean, float *save_invstd, int N, int C,
                                  int HW, void *workspace, size_t ws_bytes, void *stream);
+/* GpuBatchNormForwardInference (src/model/operation/batchnorm.cc:331-366):
+ * y = gamma * (x - running_mean) / sqrt(running_var + eps) + beta. */
+SGH_API int sgh_bn_fwd_infer_f32(const float *x, const float *gamma, const float *beta,
+                                 const float *running_mean, const float *running_var, float eps,
+                                 float *y, int N, int C, int HW, void *stream);
 /* GpuBatchNormBackward (src/model/operation/batchnorm.cc:368-404):
  * dbeta = sum dy, dgamma = sum dy*xhat, dx = gamma*invstd/M * (M*dy - dbeta - xhat*dgamma).
  * dbeta = sum dy etc. are summed in a fixed order: results are run-to-run identical. */
@@ -338,6 +352,12 @@ SGH_API int sgh_bn_fwd_train_bf16(const uint16_t *x, const float *gamma, const f
                                   float *running_mean, float *running_var, float factor, float eps,
                                   uint16_t *y, float *save_mean, float *save_invstd, int N, int C,
                                   int HW, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_fwd_infer_f16(const uint16_t *x, const float *gamma, const float *beta,
+                                 const float *running_mean, const float *running_var, float eps,
+                                 uint16_t *y, int N, int C, int HW, void *stream);
+SGH_API int sgh_bn_fwd_infer_bf16(const uint16_t *x, const float *gamma, const float *beta,
+                                  const float *running_mean, const float *running_var, float eps,
+                                  uint16_t *y, int N, int C, int HW, void *stream);
 SGH_API int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma,
                            const float *save_mean, const float *save_invstd, uint16_t *dx,
                            float *dgamma, float *dbeta, int N, int C, int HW, void *workspace,

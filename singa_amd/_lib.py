@@ -66,6 +66,13 @@ SIGNATURES = {
     "sgh_axpy_devalpha_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_eltwise_mult_f32": (C.c_int, [vp, vp, C.c_int, vp, sz, vp]),
     "sgh_add_f32": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_sub_f32": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_div_f32": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_add_scalar_f32": (C.c_int, [vp, C.c_float, vp, sz, vp]),
+    "sgh_mult_scalar_f32": (C.c_int, [vp, C.c_float, vp, sz, vp]),
+    "sgh_bn_fwd_infer_f32": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int, vp]),
+    "sgh_bn_fwd_infer_f16": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int, vp]),
+    "sgh_bn_fwd_infer_bf16": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int, vp]),
     "sgh_cast_f32_to_f16": (C.c_int, [vp, vp, sz, vp]),
     "sgh_cast_f16_to_f32": (C.c_int, [vp, vp, sz, vp]),
     "sgh_cast_f32_to_bf16": (C.c_int, [vp, vp, sz, vp]),

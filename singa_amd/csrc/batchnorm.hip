@@ -164,6 +164,28 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const typename S::elem 
       [&](size_t off) { S::st(y + off, bn_out(S::ld(x + off), mean, invstd, g, be)); });
 }
 
+// ---- forward, inference: normalise with the running statistics ------------------------------
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_bn_fwd_infer(const typename S::elem *__restrict__ x,
+                                                        const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                        const float *__restrict__ running_mean,
+                                                        const float *__restrict__ running_var, float eps,
+                                                        typename S::elem *__restrict__ y, BnShape s) {
+  const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
+  const float mean = running_mean[c];
+  const float invstd = float(1.0 / sqrt(double(running_var[c]) + double(eps)));
+  const float g = gamma[c], be = beta[c];
+  channel_range<kBlock, S>(
+      s, c, sp * s.per_split, (sp + 1) * s.per_split, x, nullptr,
+      [&](size_t off, const float *v, const float *) {
+        float r[S::VEC];
+#pragma unroll
+        for (int q = 0; q < S::VEC; ++q) r[q] = bn_out(v[q], mean, invstd, g, be);
+        S::store16(y + off, r);
+      },
+      [&](size_t off) { S::st(y + off, bn_out(S::ld(x + off), mean, invstd, g, be)); });
+}
+
 // ---- backward, pass 1: partial sum(dy) and sum(dy * xhat) ---------------------------------
 // RELU: dy is the gradient behind a ReLU that consumed this BatchNorm's output; the gradient that
 // reaches the BatchNorm is dy where the recomputed output is > 0 and 0 elsewhere (ReLUBackward's
@@ -294,6 +316,18 @@ int bn_fwd_train(const typename S::elem *x, const float *gamma, const float *bet
   return SGH_OK;
 }
 
+template <class S>
+int bn_fwd_infer(const typename S::elem *x, const float *gamma, const float *beta, const float *running_mean,
+                 const float *running_var, float eps, typename S::elem *y, int N, int C, int HW, void *stream) {
+  if (!shape_ok(N, C, HW) || !x || !gamma || !beta || !running_mean || !running_var || !y) return SGH_EINVAL;
+  if (!sgh_aligned16(x) || !sgh_aligned16(y)) return SGH_EINVAL;
+  const BnShape s = make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem)));
+  hipLaunchKernelGGL(k_bn_fwd_infer<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, gamma, beta,
+                     running_mean, running_var, eps, y, s);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
 // beta != NULL selects the fused ReLU + BatchNorm backward
 template <class S>
 int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *gamma, const float *beta,
@@ -369,6 +403,19 @@ int sgh_bn_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma, c
                     void *workspace, size_t ws_bytes, void *stream) {
   return bn_bwd<StBF16>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
                         stream);
+}
+
+int sgh_bn_fwd_infer_f32(const float *x, const float *gamma, const float *beta, const float *running_mean,
+                         const float *running_var, float eps, float *y, int N, int C, int HW, void *stream) {
+  return bn_fwd_infer<StF32>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);
+}
+int sgh_bn_fwd_infer_f16(const uint16_t *x, const float *gamma, const float *beta, const float *running_mean,
+                         const float *running_var, float eps, uint16_t *y, int N, int C, int HW, void *stream) {
+  return bn_fwd_infer<StF16>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);
+}
+int sgh_bn_fwd_infer_bf16(const uint16_t *x, const float *gamma, const float *beta, const float *running_mean,
+                          const float *running_var, float eps, uint16_t *y, int N, int C, int HW, void *stream) {
+  return bn_fwd_infer<StBF16>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);
 }
 
 int sgh_bn_relu_bwd_f32(const float *dy, const float *x, const float *gamma, const float *beta, const float *save_mean,

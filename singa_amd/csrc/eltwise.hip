@@ -117,6 +117,20 @@ struct AddOp {
 struct MulOp {
   __device__ __forceinline__ float operator()(float a, float b) const { return a * b; }
 };
+struct SubOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a - b; }
+};
+struct DivOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a / b; }
+};
+struct AddScalarOp {  // second operand unused
+  float s;
+  __device__ __forceinline__ float operator()(float a, float) const { return a + s; }
+};
+struct MulScalarOp {
+  float s;
+  __device__ __forceinline__ float operator()(float a, float) const { return a * s; }
+};
 struct AxpyOp {  // (x, y) -> y + alpha * x, two roundings
   float alpha;
   __device__ __forceinline__ float operator()(float x, float y) const {
@@ -469,6 +483,22 @@ int sgh_relu_fwd_f32(const float *x, float *y, size_t n, void *stream) {
 
 int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
   return launch_map2(a, b, out, n, AddOp{}, stream);
+}
+
+int sgh_sub_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
+  return launch_map2(a, b, out, n, SubOp{}, stream);
+}
+
+int sgh_div_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
+  return launch_map2(a, b, out, n, DivOp{}, stream);
+}
+
+int sgh_add_scalar_f32(const float *a, float x, float *out, size_t n, void *stream) {
+  return launch_map1(a, out, n, AddScalarOp{x}, stream);
+}
+
+int sgh_mult_scalar_f32(const float *a, float x, float *out, size_t n, void *stream) {
+  return launch_map1(a, out, n, MulScalarOp{x}, stream);
 }
 
 int sgh_eltwise_mult_f32(const float *a, const float *b, int b_is_scalar, float *out, size_t n, void *stream) {

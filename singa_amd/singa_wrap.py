@@ -435,6 +435,49 @@ def __add__(a, b):
     return out
 
 
+def _binary_f32(name, a, b):
+    _same(a, b)
+    if a.data_type() != kFloat32:
+        raise SingaHipError(name + " is an fp32 function")
+    out = _like(a)
+    check(getattr(_L(), name)(a.ptr, b.ptr, out.ptr, a.Size(), a.device().stream), name)
+    return out
+
+
+def _scalar_f32(name, a, x):
+    if a.data_type() != kFloat32:
+        raise SingaHipError(name + " is an fp32 function")
+    out = _like(a)
+    check(getattr(_L(), name)(a.ptr, float(x), out.ptr, a.Size(), a.device().stream), name)
+    return out
+
+
+def __sub__(a, b):
+    """``singa.__sub__`` (Sub, src/core/tensor/tensor_math_cpp.h:645-650)."""
+    return _binary_f32("sgh_sub_f32", a, b)
+
+
+def __div__(a, b):
+    """``singa.__div__`` (tensor / tensor, src/core/tensor/tensor_math_cpp.h:423-430)."""
+    return _binary_f32("sgh_div_f32", a, b)
+
+
+def AddFloat(t, x):
+    """``singa.AddFloat`` (tensor + scalar, src/core/tensor/tensor_math_cpp.h:383-388)."""
+    return _scalar_f32("sgh_add_scalar_f32", t, x)
+
+
+def MultFloat(t, x):
+    """``singa.MultFloat`` (tensor * scalar, src/core/tensor/tensor_math_cpp.h:432-437)."""
+    return _scalar_f32("sgh_mult_scalar_f32", t, x)
+
+
+def DivFloat(t, x):
+    """``singa.DivFloat``: the reference multiplies by the fp32 reciprocal
+    (include/singa/core/tensor.h Div -> src/core/tensor/tensor_math.h:149-153)."""
+    return _scalar_f32("sgh_mult_scalar_f32", t, np.float32(1.0) / np.float32(x))
+
+
 def Mult(A, B):
     """``singa.Mult(A, B)`` for 2-D tensors (src/core/tensor/tensor.cc:1633-1706): the transpose
     flags of the views select the GEMM variant, no data is moved."""
@@ -597,6 +640,15 @@ def GpuBatchNormForwardTraining(h, x, scale, bias, running_mean, running_var):
              h.factor, _BN_EPS, y.ptr, mean.ptr, var.ptr, h.batchsize, h.channels,
              h.height * h.width, h.workspace.ptr, h.workspace.MemSize(), x.device().stream), name)
     return [y, mean, var]
+
+
+def GpuBatchNormForwardInference(h, x, scale, bias, running_mean, running_var):
+    """``y`` normalised with the running statistics (src/model/operation/batchnorm.cc:331-366)."""
+    y = _like(x)
+    fn, name = _fn("bn_fwd_infer", x)
+    check(fn(x.ptr, scale.ptr, bias.ptr, running_mean.ptr, running_var.ptr, _BN_EPS, y.ptr, h.batchsize, h.channels,
+             h.height * h.width, x.device().stream), name)
+    return y
 
 
 def GpuBatchNormBackward(h, dy, x, scale, mean, var):

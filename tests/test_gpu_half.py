@@ -121,6 +121,39 @@ def test_batchnorm_16bit_storage(singa, dev, kind, shape):
 
 
 @pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 28, 28), (3, 7, 4, 2)])
+def test_batchnorm_inference(singa, dev, kind, shape):
+    """BatchNorm inference, y = gamma * (x - running_mean) / sqrt(running_var + 1e-5) + beta
+    (cudnnBatchNormalizationForwardInference with CUDNN_BN_MIN_EPSILON, batchnorm.cc:352-360),
+    against the formula in float64; and it reproduces the training-mode output when it is handed
+    that batch's own statistics."""
+    from util import nl2
+    r = rng(sum(shape) + 9)
+    N, C, H, W = shape
+    x32 = (r.standard_normal(shape) * 2 + 0.5).astype(np.float32)
+    gamma = (1 + 0.1 * r.standard_normal(C)).astype(np.float32)
+    beta = (0.1 * r.standard_normal(C)).astype(np.float32)
+    rm = (0.3 * r.standard_normal(C)).astype(np.float32)
+    rv = (0.5 + r.random(C)).astype(np.float32)
+    if kind == "f32":
+        xt, x = singa.from_numpy(x32, dev), x32
+    else:
+        xt, x = _to(singa, dev, x32, kind)
+    gd, bd = singa.from_numpy(gamma, dev), singa.from_numpy(beta, dev)
+    h = singa.CudnnBatchNormHandle(0.9, xt)
+    y = singa.GpuBatchNormForwardInference(h, xt, gd, bd, singa.from_numpy(rm, dev), singa.from_numpy(rv, dev))
+    assert y.data_type() == xt.data_type()
+    c = (1, C, 1, 1)
+    want = gamma.reshape(c).astype(np.float64) * (x.astype(np.float64) - rm.reshape(c)) / np.sqrt(
+        rv.reshape(c).astype(np.float64) + 1e-5) + beta.reshape(c)
+    assert nl2(y.to_numpy(), want) < (1e-6 if kind == "f32" else 1e-2)
+    yt, mean, invstd = singa.GpuBatchNormForwardTraining(h, xt, gd, bd, None, None)
+    var = 1.0 / invstd.to_numpy().astype(np.float64) ** 2 - 1e-5
+    y2 = singa.GpuBatchNormForwardInference(h, xt, gd, bd, mean, singa.from_numpy(var.astype(np.float32), dev))
+    assert nl2(y2.to_numpy(), yt.to_numpy()) < (1e-5 if kind == "f32" else 1e-2)
+
+
+@pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 28, 28), (16, 32, 8, 8), (3, 7, 4, 2),
                                    (32, 64, 56, 56)])
 def test_fused_relu_batchnorm_backward(singa, dev, kind, shape):

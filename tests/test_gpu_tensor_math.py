@@ -214,3 +214,18 @@ def test_pool_reuses_freed_blocks(singa, dev):
         t.SetFloatValue(1.0)
         del t
     assert dev.PoolStats()["driver_allocs"] - before <= 1
+
+
+@pytest.mark.parametrize("n", [1, 5, 1000, 4099, 1 << 20])
+def test_elementwise_functions_around_the_path(singa, dev, n):
+    """Sub, Div, Add/Mult/Div by a scalar: each is one IEEE operation per element, so NumPy's fp32
+    result is the reference result bit for bit (Div by a scalar multiplies by the fp32 reciprocal
+    as the reference does)."""
+    r = rng(n + 7)
+    a, b = randn(r, n), randn(r, n) + np.float32(3.0)
+    ad, bd = singa.from_numpy(a, dev), singa.from_numpy(b, dev)
+    assert_bit_equal(singa.__sub__(ad, bd).to_numpy(), a - b, "Sub")
+    assert_bit_equal(singa.__div__(ad, bd).to_numpy(), a / b, "Div")
+    assert_bit_equal(singa.AddFloat(ad, 1.25).to_numpy(), a + np.float32(1.25), "Add scalar")
+    assert_bit_equal(singa.MultFloat(ad, -0.3).to_numpy(), a * np.float32(-0.3), "Mult scalar")
+    assert_bit_equal(singa.DivFloat(ad, 64).to_numpy(), a * (np.float32(1.0) / np.float32(64)), "Div scalar")
