@@ -86,6 +86,10 @@ def main():
     ap.add_argument("--storage", default="f32", choices=["f32", "f16", "bf16"],
                     help="f16 / bf16: the mixed-precision tape (16-bit activations, gradients and conv weights, "
                          "fp32 BatchNorm statistics and master weights), e.g. --config resnet50 --batch 128")
+    ap.add_argument("--graph", action="store_true",
+                    help="record one step and replay it (graph mode, Device::EnableGraph / RunGraph) instead of "
+                         "enqueueing every launch of every step from the host; the step is GPU-bound, so this "
+                         "frees the host (0.94 -> 0.09 ms/step) without changing the throughput")
     ap.add_argument("--no-fusion", action="store_true",
                     help="one call per op of the reference's tape (no ReLU+BatchNorm backward fusion, residual += as its own kernel)")
     ap.add_argument("--per-parameter-update", action="store_true",
@@ -114,19 +118,35 @@ def main():
         dev.Sync()
         torch.cuda.synchronize()
 
-    for _ in range(args.warmup):
+    graph = args.graph
+    if graph:
+        # graph mode as the reference runs a compiled model (python/singa/model.py:70-90): the first
+        # iterations run eagerly, one is recorded, every later one replays the recording
+        for _ in range(2):
+            net.backward_and_update(fused_update=fused)
+        sync()
+        dev.EnableGraph(True)
         net.backward_and_update(fused_update=fused)
+        dev.EnableGraph(False)
+        step = dev.RunGraph
+    else:
+        def step():
+            net.backward_and_update(fused_update=fused)
+    for _ in range(args.warmup):
+        step()
     sync()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        net.backward_and_update(fused_update=fused)
+        step()
     t_enqueued = time.perf_counter() - t0   # host time to enqueue every launch of the timed steps
     sync()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     imgs_per_s = args.batch * args.steps / elapsed
 
-    # kernel-level pass: every conv / GEMM launch bracketed by HIP events on the device stream
+    if graph:
+        dev.ResetGraph()
+    # kernel-level pass (eager): every conv / GEMM launch bracketed by HIP events on the device stream
     prof_steps = max(1, min(args.steps, 5))
     lib.sgh_prof_enable(1)
     for _ in range(prof_steps):
@@ -166,6 +186,7 @@ def main():
         "config": {"workload": "%s backward+update, N=%d, 3x224x224, %s, SGD momentum 0.9" % (
                        args.config, args.batch, "fp32" if not half else args.storage + " storage / fp32 accumulate, statistics and master weights"),
                    "update": "fused multi-tensor" if fused else "per parameter",
+                   "launch": "one recorded step replayed (graph mode)" if graph else "eager, one launch per kernel",
                    "tape": "ReLU backward folded into BatchNorm backward (conv-BN-ReLU), residual += folded into the data gradient"
                            if hip.fuse_bn_relu
                            else "one call per reference op"},

@@ -70,6 +70,22 @@ SGH_API int sgh_malloc(sgh_device *dev, void **ptr, size_t bytes);
 SGH_API int sgh_free(sgh_device *dev, void *ptr);
 /* DeviceMemPool::GetMemUsage: bytes handed out, bytes cached in the pool, driver calls made. */
 SGH_API int sgh_pool_stats(sgh_device *dev, size_t *in_use, size_t *cached, size_t *driver_allocs);
+
+/* Record-and-replay of everything enqueued on the device's stream, the counterpart of the
+ * reference's graph mode (Device::EnableGraph / RunGraph / ResetGraph, include/singa/core/device.h
+ * :69-98, src/core/device/device.cc:55-82: operations are buffered instead of executed while the
+ * graph is enabled, then replayed every iteration).  Between sgh_graph_begin and sgh_graph_end the
+ * entry points record into a HIP graph instead of running; sgh_graph_launch replays the recording
+ * on the same stream.  While recording, nothing executes: sgh_device_sync and device-to-host copies
+ * return SGH_EUNSUPPORTED, host-to-device copies are performed immediately (outside the graph), and
+ * blocks freed to the pool stay reserved for the graph until sgh_graph_destroy.  The recording
+ * holds raw pointers: tensors that exist before sgh_graph_begin and are used inside must outlive
+ * the graph. */
+typedef struct sgh_graph sgh_graph;
+SGH_API int sgh_graph_begin(sgh_device *dev);
+SGH_API int sgh_graph_end(sgh_device *dev, sgh_graph **out);
+SGH_API int sgh_graph_launch(sgh_graph *g);
+SGH_API int sgh_graph_destroy(sgh_graph *g);
 /* Return every cached block to the driver. */
 SGH_API int sgh_pool_trim(sgh_device *dev);
 

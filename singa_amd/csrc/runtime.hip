@@ -5,6 +5,7 @@
 #include <mutex>
 #include <new>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "common.h"
@@ -12,11 +13,27 @@
 struct sgh_device {
   int id = 0;
   hipStream_t stream = nullptr;
+  hipStream_t side = nullptr;  // uploads that must happen while `stream` is recording
   std::mutex mu;
   // free blocks keyed by their (rounded) size; blocks in use keyed by address
   std::multimap<size_t, void *> free_blocks;
   std::unordered_map<void *, size_t> live;
   size_t in_use = 0, cached = 0, driver_allocs = 0;
+  // stream capture (sgh_graph_begin .. sgh_graph_end): blocks freed meanwhile are kept out of the
+  // pool, because the captured kernels will write to them on every replay
+  bool capturing = false;
+  std::vector<std::pair<void *, size_t>> held;
+  std::unordered_set<void *> born;        // blocks handed out while recording
+  std::vector<struct sgh_graph *> graphs;  // instantiated recordings of this device
+};
+
+struct sgh_graph {
+  sgh_device *dev = nullptr;
+  hipGraphExec_t exec = nullptr;
+  std::vector<std::pair<void *, size_t>> held;
+  // blocks handed out during the recording and still in use when it ended: when their owner
+  // frees them they join `held` instead of the pool, for the recorded kernels still write there
+  std::unordered_set<void *> born;
 };
 
 struct sgh_event {
@@ -120,7 +137,9 @@ int sgh_device_open(int gpu_id, sgh_device **out) {
   if (!d) return SGH_ENOMEM;
   d->id = gpu_id;
   hipError_t e = hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking);
+  if (e == hipSuccess) e = hipStreamCreateWithFlags(&d->side, hipStreamNonBlocking);
   if (e != hipSuccess) {
+    if (d->stream) (void)hipStreamDestroy(d->stream);
     delete d;
     return (int)e;
   }
@@ -145,6 +164,7 @@ int sgh_device_close(sgh_device *dev) {
   for (auto &kv : dev->free_blocks) (void)hipFree(kv.second);
   for (auto &kv : dev->live) (void)hipFree(kv.first);
   (void)hipStreamDestroy(dev->stream);
+  (void)hipStreamDestroy(dev->side);
   delete dev;
   return SGH_OK;
 }
@@ -153,7 +173,71 @@ void *sgh_device_stream(sgh_device *dev) { return dev ? reinterpret_cast<void *>
 
 int sgh_device_sync(sgh_device *dev) {
   if (!dev) return SGH_EINVAL;
+  if (dev->capturing) return SGH_EUNSUPPORTED;  // nothing runs while the stream records
   SGH_HIP_TRY(hipStreamSynchronize(dev->stream));
+  return SGH_OK;
+}
+
+int sgh_graph_begin(sgh_device *dev) {
+  if (!dev || dev->capturing) return SGH_EINVAL;
+  // relaxed mode: the pool may still call hipMalloc while the stream records
+  SGH_HIP_TRY(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeRelaxed));
+  dev->capturing = true;
+  return SGH_OK;
+}
+
+int sgh_graph_end(sgh_device *dev, sgh_graph **out) {
+  if (!dev || !out || !dev->capturing) return SGH_EINVAL;
+  dev->capturing = false;
+  hipGraph_t g = nullptr;
+  hipError_t e = hipStreamEndCapture(dev->stream, &g);
+  sgh_graph *gr = new (std::nothrow) sgh_graph();
+  if (e == hipSuccess && gr) e = hipGraphInstantiate(&gr->exec, g, nullptr, nullptr, 0);
+  if (g) (void)hipGraphDestroy(g);
+  std::lock_guard<std::mutex> lk(dev->mu);
+  if (e != hipSuccess || !gr) {  // the blocks go back to the pool: nothing will replay
+    for (auto &b : dev->held) {
+      dev->free_blocks.emplace(b.second, b.first);
+      dev->cached += b.second;
+    }
+    dev->held.clear();
+    dev->born.clear();
+    delete gr;
+    (void)hipGetLastError();
+    return e != hipSuccess ? (int)e : SGH_ENOMEM;
+  }
+  gr->dev = dev;
+  gr->held.swap(dev->held);
+  gr->born.swap(dev->born);
+  dev->graphs.push_back(gr);
+  *out = gr;
+  return SGH_OK;
+}
+
+int sgh_graph_launch(sgh_graph *g) {
+  if (!g || !g->exec || g->dev->capturing) return SGH_EINVAL;
+  SGH_HIP_TRY(hipGraphLaunch(g->exec, g->dev->stream));
+  return SGH_OK;
+}
+
+int sgh_graph_destroy(sgh_graph *g) {
+  if (!g) return SGH_EINVAL;
+  sgh_device *dev = g->dev;
+  (void)hipStreamSynchronize(dev->stream);
+  if (g->exec) (void)hipGraphExecDestroy(g->exec);
+  {
+    std::lock_guard<std::mutex> lk(dev->mu);
+    for (auto &b : g->held) {
+      dev->free_blocks.emplace(b.second, b.first);
+      dev->cached += b.second;
+    }
+    for (size_t i = 0; i < dev->graphs.size(); ++i)
+      if (dev->graphs[i] == g) {
+        dev->graphs.erase(dev->graphs.begin() + i);
+        break;
+      }
+  }
+  delete g;
   return SGH_OK;
 }
 
@@ -187,6 +271,7 @@ int sgh_malloc(sgh_device *dev, void **ptr, size_t bytes) {
   }
   dev->live.emplace(p, r);
   dev->in_use += r;
+  if (dev->capturing) dev->born.insert(p);
   *ptr = p;
   return SGH_OK;
 }
@@ -200,6 +285,19 @@ int sgh_free(sgh_device *dev, void *ptr) {
   const size_t r = it->second;
   dev->live.erase(it);
   dev->in_use -= r;
+  if (dev->capturing) {  // part of the graph being recorded: reserved until the graph is destroyed
+    dev->held.emplace_back(ptr, r);
+    dev->born.erase(ptr);
+    return SGH_OK;
+  }
+  for (sgh_graph *g : dev->graphs) {
+    auto b = g->born.find(ptr);
+    if (b != g->born.end()) {
+      g->born.erase(b);
+      g->held.emplace_back(ptr, r);
+      return SGH_OK;
+    }
+  }
   // Work already enqueued on the device stream may still read the block; the next owner's
   // work is enqueued behind it on the same stream, so immediate reuse is ordered correctly.
   dev->free_blocks.emplace(r, ptr);
@@ -222,6 +320,14 @@ int sgh_memcpy(sgh_device *dev, void *dst, const void *src, size_t bytes, int ki
   if (!dst || !src) return SGH_EINVAL;
   static const hipMemcpyKind kinds[4] = {hipMemcpyHostToHost, hipMemcpyHostToDevice,
                                          hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice};
+  if (dev->capturing && kind != 3) {
+    // a host copy cannot wait on a recording stream: an upload happens now, outside the graph
+    // (small tables the recorded kernels read); a download has nothing to read yet
+    if (kind == 2) return SGH_EUNSUPPORTED;
+    SGH_HIP_TRY(hipMemcpyAsync(dst, src, bytes, kinds[kind], dev->side));
+    SGH_HIP_TRY(hipStreamSynchronize(dev->side));
+    return SGH_OK;
+  }
   SGH_HIP_TRY(hipMemcpyAsync(dst, src, bytes, kinds[kind], dev->stream));
   if (kind != 3) SGH_HIP_TRY(hipStreamSynchronize(dev->stream));
   return SGH_OK;

@@ -96,13 +96,35 @@ class HipGPU(object):
         check(_L().sgh_pool_stats(self._h, C.byref(a), C.byref(c), C.byref(d)))
         return {"in_use": a.value, "cached": c.value, "driver_allocs": d.value}
 
-    # graph buffering is a property of SINGA's scheduler, not of this device
+    # Graph mode (include/singa/core/device.h:69-98): EnableGraph(True) .. EnableGraph(False)
+    # records what is enqueued on the stream instead of running it (the reference buffers the
+    # operations in its scheduler), RunGraph() replays the recording, ResetGraph() drops it.
+    _graph = None
+    _recording = False
+
     def graph_enabled(self):
-        return False
+        return self._recording
 
     def EnableGraph(self, flag):
-        if flag:
-            raise SingaHipError("graph buffering lives in SINGA's scheduler; not available here")
+        if flag and not self._recording:
+            self.ResetGraph()
+            check(_L().sgh_graph_begin(self._h), "sgh_graph_begin")
+            self._recording = True
+        elif not flag and self._recording:
+            g = C.c_void_p()
+            self._recording = False
+            check(_L().sgh_graph_end(self._h, C.byref(g)), "sgh_graph_end")
+            self._graph = g
+
+    def RunGraph(self, serial=False):
+        if self._graph is None:
+            raise SingaHipError("RunGraph without a recorded graph")
+        check(_L().sgh_graph_launch(self._graph), "sgh_graph_launch")
+
+    def ResetGraph(self):
+        if self._graph is not None:
+            check(_L().sgh_graph_destroy(self._graph), "sgh_graph_destroy")
+            self._graph = None
 
     def _malloc(self, nbytes):
         p = C.c_void_p()

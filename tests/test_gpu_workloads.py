@@ -153,3 +153,41 @@ def test_fused_tape_equals_reference_tape(dev):
         outs.append([hip.to_numpy(dx)] + [hip.to_numpy(p) for _, p in net.params()])
     for a, b in zip(*outs):
         assert np.array_equal(a, b)
+
+
+def test_graph_replay_of_the_step(dev):
+    """Graph mode (EnableGraph / RunGraph): one recorded backward+update step, replayed several
+    times with eager work and synchronisations in between, leaves after every replay exactly the
+    parameters of a network that ran the same number of eager steps."""
+    hip = wl.HipOps(dev)
+    x, labels = wl.make_inputs("resnet18_small", 2)
+    nets = []
+    for _ in range(2):
+        net = wl.build("resnet18_small", hip, lr=0.002)
+        net.forward(hip.from_numpy(x), hip.from_numpy(labels))
+        nets.append(net)
+    eager, replayed = nets
+    for _ in range(2):   # momentum buffers, kernel attributes and the pool are set up by eager steps
+        eager.backward_and_update(fused_update=True)
+        replayed.backward_and_update(fused_update=True)
+    dev.Sync()
+    before = [hip.to_numpy(p) for _, p in replayed.params()]
+    dev.EnableGraph(True)
+    assert dev.graph_enabled()
+    replayed.backward_and_update(fused_update=True)
+    dev.EnableGraph(False)
+    for a, (_, p) in zip(before, replayed.params()):
+        assert np.isfinite(a).all() and np.array_equal(a, hip.to_numpy(p)), "recording must not execute"
+    for i in range(4):
+        eager.backward_and_update(fused_update=True)
+        dev.RunGraph()
+        t = hip.from_numpy(np.full(100000, i, np.float32))   # eager work on the same stream and pool
+        t += t
+        assert np.array_equal(hip.to_numpy(t), np.full(100000, 2 * i, np.float32))
+        for (k, a), (_, b) in zip(eager.params(), replayed.params()):
+            assert np.array_equal(hip.to_numpy(a), hip.to_numpy(b)), (i, k)
+    dev.ResetGraph()
+    eager.backward_and_update(fused_update=True)   # the device is back in eager mode
+    replayed.backward_and_update(fused_update=True)
+    for (k, a), (_, b) in zip(eager.params(), replayed.params()):
+        assert np.array_equal(hip.to_numpy(a), hip.to_numpy(b)), k
