@@ -925,12 +925,15 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     DilateStore st{dx, g->C, g->H, g->W, g->P, g->Q, g->stride_h, g->stride_w, Ncols};
     const int chunks = (g->K + BK - 1) / BK;
     const long tiles128 = long((g->C + 127) / 128) * ((Ncols + 127) / 128);
-    if (g->C > 64 && tiles128 >= sgh_num_cus()) {
+    // (this GEMM has a short reduction and a large store: it wants many workgroups in flight, so the
+    // larger tiles are only taken when they still give two workgroups per CU)
+    const long need = long(sgh_num_cus()) * 2;
+    if (g->C > 64 && tiles128 >= need) {
       auto la = dense_loader<128, false>(W, 1, g->C, g->C, g->K);
       auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
       rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, DilateStore, false, false>(
           la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad", conv_flops(g));
-    } else if (long((g->C + 63) / 64) * ((Ncols + 127) / 128) >= sgh_num_cus()) {
+    } else if (long((g->C + 63) / 64) * ((Ncols + 127) / 128) >= need) {
       auto la = dense_loader<64, false>(W, 1, g->C, g->C, g->K);
       auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
       rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DilateStore, false, false>(
