@@ -23,8 +23,11 @@
 //     Stride 2 is handled by residue class: output pixels (2i+a, 2j+b) of one class form their own
 //     pixel space with a stride-1 gradient window, and only the taps of that class are visited.
 //
-// 256 threads = 2 x 2 wavefronts, workgroup tile 128 (or 64) x 128, reduction chunk 64, LDS and
-// register double buffering.
+// 512 threads = two groups of 2 x 2 wavefronts on a workgroup tile of 128 (or 64) x 128; both groups
+// tile the same outputs and take the first / second half of every 64-wide reduction chunk's MFMA
+// steps, their accumulators are added through LDS at the end.  With two workgroups per CU that
+// puts four wavefronts on every SIMD, so one wavefront's staging arithmetic and memory waits
+// overlap the others' matrix work.  LDS and register double buffering.
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -34,7 +37,7 @@
 
 namespace {
 
-constexpr int NT = 256, BN = 128, KC = 64, PITCH = KC + 8;  // PITCH in 16-bit elements
+constexpr int NT = 512, BN = 128, KC = 64, PITCH = KC + 8;  // PITCH in 16-bit elements
 constexpr int kOOB = int(0x80000000u);
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -88,22 +91,46 @@ __device__ __forceinline__ u32x4 load16b(const uint16_t *p) {  // 16 bytes at an
   return v;
 }
 
-// One reduction chunk (64 indices = four MFMA steps) of a wavefront's (TM*32) x 64 tile.
+// One wavefront group's half (two of the four MFMA steps) of a reduction chunk, on a wavefront's
+// (TM*32) x 64 tile.  `koff` = element offset of the half within the chunk (0 or 32) + 8 * (lane / 32).
+// acc[.][j] belongs to the 32-column block at B row brow + j * bstep: group 0 numbers its two blocks
+// 0, 1 and group 1 numbers them 1, 0, so that for both groups acc[.][0] is the block the group keeps
+// and acc[.][1] the one it hands over when the groups' sums are combined.
 template <int TM, bool BF16>
-__device__ __forceinline__ void mma_chunk(const uint16_t *As, const uint16_t *Bs, int arow, int brow, int lh,
-                                          f32x16 (&acc)[TM][2]) {
+__device__ __forceinline__ void mma_chunk(const uint16_t *As, const uint16_t *Bs, int arow, int brow, int bstep,
+                                          int koff, f32x16 (&acc)[TM][2]) {
 #pragma unroll
-  for (int j = 0; j < KC / 16; ++j) {
+  for (int j = 0; j < KC / 32; ++j) {
     u32x4 av[TM], bv[2];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) av[i] = *reinterpret_cast<const u32x4 *>(As + (arow + i * 32) * PITCH + (2 * j + lh) * 8);
+    for (int i = 0; i < TM; ++i) av[i] = *reinterpret_cast<const u32x4 *>(As + (arow + i * 32) * PITCH + koff + 16 * j);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) bv[i] = *reinterpret_cast<const u32x4 *>(Bs + (brow + i * 32) * PITCH + (2 * j + lh) * 8);
+    for (int i = 0; i < 2; ++i) bv[i] = *reinterpret_cast<const u32x4 *>(Bs + (brow + i * bstep) * PITCH + koff + 16 * j);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int jn = 0; jn < 2; ++jn) acc[i][jn] = mfma<BF16>(av[i], bv[jn], acc[i][jn]);
   }
+}
+
+// Sums the two wavefront groups' accumulators through LDS (after the last chunk; the tile buffers
+// are free then).  Every wavefront hands over acc[.][1] and adds what its partner hands over to
+// acc[.][0] (see mma_chunk for the numbering), so afterwards acc[.][0] is complete in both groups and
+// both take part in the store.
+template <int TM>
+__device__ __forceinline__ void combine_halves(float *lds, int half, int w4, int lane, f32x16 (&acc)[TM][2]) {
+  __syncthreads();
+  float *send = lds + ((half * 4 + w4) * (TM * 16)) * 64 + lane;
+  const float *recv = lds + (((half ^ 1) * 4 + w4) * (TM * 16)) * 64 + lane;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) send[(i * 16 + v) * 64] = acc[i][1][v];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][0][v] += recv[(i * 16 + v) * 64];
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -120,7 +147,7 @@ struct W16Args {
 };
 
 template <int BM, int STRIDE, bool BF16>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_wgrad16(W16Args a) {
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_wgrad16(W16Args a) {
   extern __shared__ __align__(16) uint16_t lds16[];
   constexpr int TM = BM / 64, ASLOTS = BM * 8 / NT, BSLOTS = BN * 8 / NT;
   uint16_t *const As0 = lds16, *const Bs0 = lds16 + BM * PITCH;
@@ -128,7 +155,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   // octet masks by valid element range: lut[lo * 9 + hi] keeps elements lo <= j < hi (branch-free
   // border handling: one LDS read and four ANDs per octet)
   u32x4 *const lut = reinterpret_cast<u32x4 *>(lds16 + 2 * (BM + BN) * PITCH);
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int half = wave >> 2, w4 = wave & 3, wm = w4 >> 1, wn = w4 & 1;
   const int l32 = lane & 31, lh = lane >> 5;
   // Workgroup w runs on XCD w % 8 (each XCD has its own L2).  All tiles of one split of the
   // reduction read the same dy rows, so a split's tiles are given to one XCD: split = 8 * (slot /
@@ -170,13 +198,13 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   int aoff[ASLOTS];
 #pragma unroll
   for (int i = 0; i < ASLOTS; ++i) {
-    const int k = m0 + rb + 32 * i;
-    aoff[i] = k < a.K ? k * PQ : -1;
+    const int k = m0 + rb + 64 * i;
+    aoff[i] = k < a.K && rb + 64 * i < BM ? k * PQ : -1;
   }
   int boff[BSLOTS], br[BSLOTS], bs[BSLOTS];
 #pragma unroll
   for (int i = 0; i < BSLOTS; ++i) {
-    const int col = n0 + rb + 32 * i;
+    const int col = n0 + rb + 64 * i;
     const int c = col / RS, tap = col - c * RS, r = tap / a.S;
     br[i] = r - a.pad_h;
     bs[i] = tap - r * a.S - a.pad_w;
@@ -250,7 +278,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   auto stage = [&](const Stage &g, uint16_t *As, uint16_t *Bs) {
     const u32x4 ma = lut[g.a_nv];
 #pragma unroll
-    for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 32 * i) * PITCH + oct * 8) = g.ra[i] & ma;
+    for (int i = 0; i < ASLOTS; ++i)
+      if (BM >= 128 || rb < BM) *reinterpret_cast<u32x4 *>(As + (rb + 64 * i) * PITCH + oct * 8) = g.ra[i] & ma;
 #pragma unroll
     for (int i = 0; i < BSLOTS; ++i) {
       u32x4 v = g.rbv[i][0];
@@ -262,7 +291,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         v[2] = __builtin_amdgcn_perm(v1[1], v1[0], 0x05040100u);
         v[3] = __builtin_amdgcn_perm(v1[3], v1[2], 0x05040100u);
       }
-      *reinterpret_cast<u32x4 *>(Bs + (rb + 32 * i) * PITCH + oct * 8) = v & lut[g.b_lohi[i]];
+      *reinterpret_cast<u32x4 *>(Bs + (rb + 64 * i) * PITCH + oct * 8) = v & lut[g.b_lohi[i]];
     }
   };
 
@@ -274,40 +303,21 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const int arow = wm * (TM * 32) + l32, brow = wn * 64 + l32;
+  const int arow = wm * (TM * 32) + l32, brow = wn * 64 + half * 32 + l32, bstep = half ? -32 : 32;
+  const int koff = half * 32 + lh * 8;
+  // Chunk c is computed from LDS buffer c & 1 while the loads of chunk c + 1 are in flight; they are
+  // written to the other buffer after the MFMA steps.
   auto run = [&](auto tails) {
-    if constexpr (STRIDE == 1) {
-      // Chunk c is computed from LDS buffer c & 1 while chunk c + 1 waits in registers (stage set
-      // (c + 1) & 1) and the loads of chunk c + 2 are issued: two chunks of memory latency are covered.
-      Stage g0, g1;
-      load(g0, tails);
-      stage(g0, As0, Bs0);
-      if (c_begin + 1 < c_end) load(g1, tails);
+    Stage g;
+    load(g, tails);
+    stage(g, As0, Bs0);
+    __syncthreads();
+    for (int c = c_begin; c < c_end; ++c) {
+      const bool cur1 = (c - c_begin) & 1, more = c + 1 < c_end;
+      if (more) load(g, tails);
+      mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, arow, brow, bstep, koff, acc);
+      if (more) stage(g, cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
       __syncthreads();
-      for (int c = c_begin; c < c_end; c += 2) {
-        if (c + 2 < c_end) load(g0, tails);
-        mma_chunk<TM, BF16>(As0, Bs0, arow, brow, lh, acc);
-        if (c + 1 >= c_end) break;
-        stage(g1, As1, Bs1);
-        __syncthreads();
-        if (c + 3 < c_end) load(g1, tails);
-        mma_chunk<TM, BF16>(As1, Bs1, arow, brow, lh, acc);
-        if (c + 2 < c_end) stage(g0, As0, Bs0);
-        __syncthreads();
-      }
-    } else {
-      // (stride 2 holds twice the x registers per chunk: one chunk in flight, or the kernel spills)
-      Stage g;
-      load(g, tails);
-      stage(g, As0, Bs0);
-      __syncthreads();
-      for (int c = c_begin; c < c_end; ++c) {
-        const bool cur1 = (c - c_begin) & 1, more = c + 1 < c_end;
-        if (more) load(g, tails);
-        mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, arow, brow, lh, acc);
-        if (more) stage(g, cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
-        __syncthreads();
-      }
     }
   };
   // Only the first chunk (x rows before the first image) and the chunks of the last two output
@@ -318,19 +328,18 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     else run(std::false_type{});
   }
 
+  combine_halves<TM>(reinterpret_cast<float *>(lds16), half, w4, lane, acc);
   float *out = a.partial + size_t(split) * a.K * a.CRS;
+  const int col = n0 + wn * 64 + half * 32 + l32;   // the block this group kept
+  if (col < a.CRS) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int jn = 0; jn < 2; ++jn) {
-      const int col = n0 + wn * 64 + jn * 32 + l32;
-      if (col >= a.CRS) continue;
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-        if (row < a.K) out[size_t(row) * a.CRS + col] = acc[i][jn][v];
+        if (row < a.K) out[size_t(row) * a.CRS + col] = acc[i][0][v];
       }
-    }
+  }
 }
 
 // dW = round16(sum over splits).  A workgroup takes EP consecutive elements; its 256 threads form
@@ -371,13 +380,13 @@ struct D16Args {
 constexpr unsigned kSelLo = 0x05040100u, kSelHi = 0x07060302u, kSelZero = 0x0c0c0c0cu;
 
 template <int BM, bool BF16>
-__global__ __launch_bounds__(NT) void k_dgrad16(D16Args a) {
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_dgrad16(D16Args a) {
   extern __shared__ __align__(16) uint16_t lds16[];
   constexpr int TM = BM / 64, ASLOTS = BM * 8 / NT;
   uint16_t *const As0 = lds16, *const Bs0 = lds16 + BM * PITCH;
   uint16_t *const As1 = lds16 + (BM + BN) * PITCH, *const Bs1 = As1 + BM * PITCH;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lh = lane >> 5;
+  const int half = wave >> 2, w4 = wave & 3, wm = w4 >> 1, wn = w4 & 1, l32 = lane & 31, lh = lane >> 5;
   // XCD-aware ids (workgroup w runs on XCD w % 8): the channel tiles of one pixel tile read the
   // same gradient pixels and share an XCD's L2.
   const int slot = int(blockIdx.x) >> 3, pt = (slot / a.mtiles) * 8 + (int(blockIdx.x) & 7);
@@ -394,7 +403,7 @@ __global__ __launch_bounds__(NT) void k_dgrad16(D16Args a) {
   const long pix0 = long(pt - a.cls_tile0[cls]) * BN;
   const rsrc_t rdy = make_rsrc(a.dy, a.dy_bytes);
 
-  // B loader: pixel pair pp of the tile, k octets kq and kq + 4 of the chunk
+  // B loader: pixel pair pp of the tile, k octet kq of the chunk (one per wavefront)
   const int pp = lane, kq = wave;
   const long pixA = pix0 + 2 * pp, pixB = pixA + 1;
   const int nA = int(pixA / HWc), remA = int(pixA - long(nA) * HWc), iA = remA / Wc, jA = remA - iA * Wc;
@@ -423,42 +432,34 @@ __global__ __launch_bounds__(NT) void k_dgrad16(D16Args a) {
 
   const int oct = t & 7, rb = t >> 3;
   u32x4 ra[ASLOTS];
-  unsigned rd[2][8];   // the pair's dword for 8 consecutive k
+  unsigned rd[8];      // the pair's dword for 8 consecutive k
   const rsrc_t rwt = make_rsrc(a.wt, a.wt_bytes);
-  const int woff = ((m0 + rb) * a.KP + oct * 8) * 2;
+  const int woff = ((m0 + rb) * a.KP + oct * 8) * 2;   // rb = t / 8 in 0..63
   auto load = [&](int tap, int kc) {
     const int wso = (tap * a.CP * a.KP + kc * KC) * 2;
 #pragma unroll
     for (int i = 0; i < ASLOTS; ++i)
-      ra[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rwt, woff + 32 * i * a.KP * 2, wso, 0));
+      ra[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rwt, woff + 64 * i * a.KP * 2, wso, 0));
+    const int kb = kc * KC + kq * 8;
+    if (kb < a.K) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int kb = kc * KC + (kq + 4 * i) * 8;
-      if (kb < a.K) {
+      for (int j = 0; j < 8; ++j) rd[j] = unsigned(__builtin_amdgcn_raw_buffer_load_b32(rdy, voff, (kb + j) * PQ * 2, 0));
+    } else {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          rd[i][j] = unsigned(__builtin_amdgcn_raw_buffer_load_b32(rdy, voff, (kb + j) * PQ * 2, 0));
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) rd[i][j] = 0u;
-      }
+      for (int j = 0; j < 8; ++j) rd[j] = 0u;
     }
   };
   auto stage = [&](uint16_t *As, uint16_t *Bs) {
 #pragma unroll
-    for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 32 * i) * PITCH + oct * 8) = ra[i];
+    for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 64 * i) * PITCH + oct * 8) = ra[i];
+    u32x4 vA, vB;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      u32x4 vA, vB;
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        vA[d] = __builtin_amdgcn_perm(rd[i][2 * d + 1], rd[i][2 * d], selA);
-        vB[d] = __builtin_amdgcn_perm(rd[i][2 * d + 1], rd[i][2 * d], selB);
-      }
-      *reinterpret_cast<u32x4 *>(Bs + (2 * pp) * PITCH + (kq + 4 * i) * 8) = vA;
-      *reinterpret_cast<u32x4 *>(Bs + (2 * pp + 1) * PITCH + (kq + 4 * i) * 8) = vB;
+    for (int d = 0; d < 4; ++d) {
+      vA[d] = __builtin_amdgcn_perm(rd[2 * d + 1], rd[2 * d], selA);
+      vB[d] = __builtin_amdgcn_perm(rd[2 * d + 1], rd[2 * d], selB);
     }
+    *reinterpret_cast<u32x4 *>(Bs + (2 * pp) * PITCH + kq * 8) = vA;
+    *reinterpret_cast<u32x4 *>(Bs + (2 * pp + 1) * PITCH + kq * 8) = vB;
   };
 
   f32x16 acc[TM][2];
@@ -487,7 +488,8 @@ __global__ __launch_bounds__(NT) void k_dgrad16(D16Args a) {
         if (newtap) set_tap(ti, tj);   // (the registers of the previous chunk were packed with the old selectors)
         load((r0 + st * ti) * a.S + s0 + st * tj, kc);
       }
-      mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, wm * (TM * 32) + l32, wn * 64 + l32, lh, acc);
+      mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, wm * (TM * 32) + l32, wn * 64 + half * 32 + l32,
+                          half ? -32 : 32, half * 32 + lh * 8, acc);
       if (!more) break;
       stage(cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
       __syncthreads();
@@ -496,21 +498,19 @@ __global__ __launch_bounds__(NT) void k_dgrad16(D16Args a) {
   }
 
   // epilogue: lane's pixel column, 16 channel rows per accumulator
+  combine_halves<TM>(reinterpret_cast<float *>(lds16), half, w4, lane, acc);
+  const long pix = pix0 + wn * 64 + half * 32 + l32;   // the block this group kept
+  if (pix >= cnt) return;
+  const int n = int(pix / HWc), rem = int(pix - long(n) * HWc), i_ = rem / Wc, j_ = rem - i_ * Wc;
+  if (j_ >= Wreal) return;
+  uint16_t *o = a.dx + (size_t(n) * a.C) * HW + (st * i_ + ca) * a.W + st * j_ + cb;
 #pragma unroll
-  for (int jn = 0; jn < 2; ++jn) {
-    const long pix = pix0 + wn * 64 + jn * 32 + l32;
-    if (pix >= cnt) continue;
-    const int n = int(pix / HWc), rem = int(pix - long(n) * HWc), i_ = rem / Wc, j_ = rem - i_ * Wc;
-    if (j_ >= Wreal) continue;
-    uint16_t *o = a.dx + (size_t(n) * a.C) * HW + (st * i_ + ca) * a.W + st * j_ + cb;
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int c = m0 + wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-        if (c < a.C) o[size_t(c) * HW] = round16<BF16>(acc[i][jn][v]);
-      }
-  }
+    for (int v = 0; v < 16; ++v) {
+      const int c = m0 + wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+      if (c < a.C) o[size_t(c) * HW] = round16<BF16>(acc[i][0][v]);
+    }
 }
 
 // wt[tap][c][k] (c < CP, k < KP; zero beyond C / K) from W[k][c][r][s]
