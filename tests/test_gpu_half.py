@@ -314,6 +314,46 @@ def test_conv_gradients_16bit_matrix_kernels(singa, dev, kind, case):
     _same_bits(singa.GpuConvBackwardW(dyt, xt, wt, h).to_numpy(), dw.to_numpy(), "wgrad run-to-run")
 
 
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", [
+    (128, 64, 56, 64, 3, 1, 1),      # ResNet-50 stage 1, 3x3
+    (128, 256, 56, 64, 1, 1, 0),     # bottleneck reduce
+    (128, 128, 56, 128, 3, 2, 1),    # stage transition, stride 2
+    (128, 1024, 14, 256, 1, 1, 0),   # plane of 196 pixels: 24.5 octets
+])
+def test_conv_gradients_16bit_full_size_properties(singa, dev, kind, shape):
+    """The 16-bit gradient kernels at the half-precision configuration's full batch (N = 128), too
+    large for the CPU oracle inside a test: adjointness <x, dgrad(dy)> = <W, wgrad(dy)> (both equal
+    <conv(x, W), dy>) on the stored values, the oracle on one image of the batch for dgrad, on a
+    2-image sub-batch for wgrad (additive over images), and exact linearity under scaling by 2
+    (wherever the result is a normal number of the storage type)."""
+    from oracle import cpu_oracle as O
+    from util import nl2
+    N, C, H, K, R, st, pd = shape
+    r = rng(sum(shape))
+    xt, x = _to(singa, dev, r.standard_normal((N, C, H, H)).astype(np.float32), kind)
+    wt, w = _to(singa, dev, (r.standard_normal((K, C, R, R)) * np.sqrt(2.0 / (C * R * R))).astype(np.float32), kind)
+    h = singa.CudnnConvHandle(xt, (R, R), (st, st), (pd, pd), C, K, False)
+    P = h.conv_height
+    dy32 = r.standard_normal((N, K, P, P)).astype(np.float32)
+    dyt, dy = _to(singa, dev, dy32, kind)
+    dx = singa.GpuConvBackwardx(dyt, wt, xt, h).to_numpy()
+    dw = singa.GpuConvBackwardW(dyt, xt, wt, h).to_numpy()
+    a = float((x.astype(np.float64) * dx).sum()), float((w.astype(np.float64) * dw).sum())
+    scale = float(np.sqrt((x.astype(np.float64) ** 2).sum() * (dx.astype(np.float64) ** 2).sum()))
+    assert abs(a[0] - a[1]) < 1e-3 * scale      # both sides carry one 16-bit rounding per element
+    dx5, _ = O.conv_bwd(dy[5:6], x[5:6], w, (st, st), (pd, pd), want_dw=False)
+    assert nl2(dx[5:6], dx5) < 1e-2
+    dys = dy.copy()
+    dys[2:] = 0
+    dw2 = singa.GpuConvBackwardW(_to(singa, dev, dys, kind)[0], xt, wt, h).to_numpy()
+    _, dw2_o = O.conv_bwd(dy[:2], x[:2], w, (st, st), (pd, pd), want_dx=False)
+    assert nl2(dw2, dw2_o) < 1e-2
+    dx2 = singa.GpuConvBackwardx(_to(singa, dev, dy * 2, kind)[0], wt, xt, h).to_numpy()
+    normal = np.abs(dx) >= 2.0 ** -13        # (binary16 subnormals have a coarser grid: 2x is not exact there)
+    _same_bits(dx2[normal], dx[normal] * 2, "dgrad linearity " + kind)
+
+
 def _sgd_ref(p, g, v, lr, mu, damp, wd, nesterov):
     """The four ops of SGD.apply in fp32, each product / sum rounded separately."""
     f = np.float32
