@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes the 40 conv dgrad/wgrad MFMA launches of one default step move (fetched + written), from the
 # rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, each scaled by what the same counter reads for
 # a streaming kernel of known size (ReLU forward: 1.998 and 1.000).  Valid for the default workload only.
-CONV_HBM_BYTES_PER_STEP = 5.56e9
+CONV_HBM_BYTES_PER_STEP = 6.71e9
 
 
 def collect_prof(lib):
@@ -163,7 +163,8 @@ def main():
     roofline = {
         "bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
         "frac": round(achieved / peak, 4),
-        "traffic": CONV_HBM_BYTES_PER_STEP if (args.config == "resnet18" and args.batch == 64) else None,
+        "traffic": CONV_HBM_BYTES_PER_STEP if (args.config == "resnet18" and args.batch == 64 and not half
+                                               and not args.no_fusion) else None,
         "traffic_unit": "HBM bytes per step over the same launches (PMC, calibrated)",
         "kernel": ("16-bit MFMA conv dgrad + wgrad kernels (k_dgrad16, k_wgrad16; fp32 kernels for the stem dgrad; %d launches/step)"
                    if half else
