@@ -161,8 +161,17 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   // Workgroup w runs on XCD w % 8 (each XCD has its own L2).  All tiles of one split of the
   // reduction read the same dy rows, so a split's tiles are given to one XCD: split = 8 * (slot /
   // tiles) + w % 8 with slot = w / 8.
-  const int slot = int(blockIdx.x) >> 3, tile = slot % a.tiles;
-  const int split = (slot / a.tiles) * 8 + (int(blockIdx.x) & 7);
+  // (only when the split count is a multiple of 8: otherwise some XCDs would get more splits than
+  // others, and the tiles are dealt round-robin instead)
+  int tile, split;
+  if ((a.splits & 7) == 0) {
+    const int slot = int(blockIdx.x) >> 3;
+    tile = slot % a.tiles;
+    split = (slot / a.tiles) * 8 + (int(blockIdx.x) & 7);
+  } else {
+    tile = int(blockIdx.x) % a.tiles;
+    split = int(blockIdx.x) / a.tiles;
+  }
   if (split >= a.splits) return;
   if (t < 81) lut[t] = mask_range(u32x4{~0u, ~0u, ~0u, ~0u}, t / 9, t % 9);
   __syncthreads();
@@ -566,7 +575,10 @@ W16Plan wplan(const sgh_conv_geom *g) {
     if (s < 1) s = 1;
     if (s > (p.chunks + 3) / 4) s = (p.chunks + 3) / 4;
     if (s < 1) s = 1;
-    const int cps = (p.chunks + s - 1) / s, s2 = (p.chunks + cps - 1) / cps;
+    if (s >= 8) s &= ~7;   // a multiple of 8 lets every XCD take whole splits (see the kernel)
+    const int cps = (p.chunks + s - 1) / s;
+    // (with 8 or more splits the count stays the multiple of 8; the last splits may then be short or empty)
+    const int s2 = s >= 8 ? s : (p.chunks + cps - 1) / cps;
     const long rounds = (long(tiles) * s2 + slots - 1) / slots, cost = rounds * (cps + 2);  // (+2: prologue, epilogue)
     if (best < 0 || cost < best) best = cost, p.cps = cps, p.splits = s2;
   }
@@ -615,7 +627,7 @@ int launch_w(const W16Args &a, const W16Plan &p, hipStream_t s) {
     if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
     attr = true;
   }
-  hipLaunchKernelGGL(kern, dim3(unsigned(p.mtiles * p.ntiles) * 8u * unsigned((p.splits + 7) / 8)), dim3(NT), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(unsigned(p.mtiles * p.ntiles) * unsigned(p.splits)), dim3(NT), lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
