@@ -112,7 +112,7 @@ def main():
     net = wl.build(args.config, hip, lr=0.05, momentum=0.9)
     x, labels = wl.make_inputs(args.config, args.batch)
     net.forward(hip.from_numpy(x), hip.from_numpy(labels))
-    fused = not args.per_parameter_update and not half   # (the single-launch update covers fp32 parameters)
+    fused = not args.per_parameter_update
 
     def sync():
         dev.Sync()

@@ -226,6 +226,22 @@ SGH_API int sgh_sgd_momentum_multi_f32(const sgh_sgd_item *table_dev, int count,
  * sgh_sgd_momentum_master_f16 / _bf16: mixed precision -- fp32 master weights and fp32 momentum
  *   are updated from the 16-bit gradient, and p_out receives the master rounded to 16 bits
  *   (the working copy the next forward pass reads).  No counterpart in the reference's opt.py. */
+/* sgh_sgd_momentum_multi_mixed: every parameter of a mixed-precision network in one launch (the
+ *   loop of Optimizer.call, python/singa/opt.py:107-111, over fp32 parameters and 16-bit parameters
+ *   with fp32 master copies alike).  An item with p16 == NULL is an fp32 parameter (g is float);
+ *   otherwise p is the fp32 master, g the 16-bit gradient (binary16, or bfloat16 when `bf16` is
+ *   set) and p16 the working copy that receives the updated master rounded once.  At most 2048
+ *   items.  Per element identical to the single-tensor entry points. */
+typedef struct sgh_sgd_mixed_item {
+  float *p;
+  const void *g;
+  float *v;
+  uint16_t *p16;
+  uint64_t n;
+} sgh_sgd_mixed_item;
+SGH_API int sgh_sgd_momentum_multi_mixed(const sgh_sgd_mixed_item *table_dev, int count,
+                                         size_t total_n, int bf16, float lr, float mu, float damp,
+                                         float wd, int nesterov, void *stream);
 SGH_API int sgh_sgd_momentum_f16(uint16_t *p, const uint16_t *g, uint16_t *v, size_t n, float lr,
                                  float mu, float damp, float wd, int nesterov, void *stream);
 SGH_API int sgh_sgd_momentum_bf16(uint16_t *p, const uint16_t *g, uint16_t *v, size_t n, float lr,

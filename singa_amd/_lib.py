@@ -33,6 +33,11 @@ class SgdItem(C.Structure):
     _fields_ = [("p", vp), ("g", vp), ("v", vp), ("n", C.c_uint64)]
 
 
+class SgdMixedItem(C.Structure):
+    """``sgh_sgd_mixed_item``"""
+    _fields_ = [("p", vp), ("g", vp), ("v", vp), ("p16", vp), ("n", C.c_uint64)]
+
+
 # name -> (restype, argtypes); every symbol the header declares
 SIGNATURES = {
     "sgh_error_string": (C.c_char_p, [C.c_int]),
@@ -70,6 +75,8 @@ SIGNATURES = {
     "sgh_axpy_devalpha_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_eltwise_mult_f32": (C.c_int, [vp, vp, C.c_int, vp, sz, vp]),
     "sgh_add_f32": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_sgd_momentum_multi_mixed": (C.c_int, [vp, C.c_int, sz, C.c_int, C.c_float, C.c_float, C.c_float, C.c_float,
+                                               C.c_int, vp]),
     "sgh_sub_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_div_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_add_scalar_f32": (C.c_int, [vp, C.c_float, vp, sz, vp]),

@@ -221,9 +221,73 @@ int sgd_h(uint16_t *p16, const uint16_t *g16, uint16_t *v16, float *p32, float *
   return SGH_OK;
 }
 
+// All parameters of a mixed-precision network in one launch: fp32 items (p, g, v fp32) and master
+// items (16-bit gradient, fp32 master p and momentum v, 16-bit working copy p16 refreshed) share a
+// table; a block takes chunks of kMixChunk elements, the chunk -> item lookup goes through an LDS
+// prefix table built once per block.  Per element the same sgd_one as the single-tensor kernels.
+constexpr int kMixChunk = kBlock * 8;
+constexpr int kMixTab = 2048;
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void k_sgd_multi_mixed(const sgh_sgd_mixed_item *__restrict__ table, int count,
+                                                           SgdHyper h, int nesterov) {
+  __shared__ unsigned pre[kMixTab + 1];  // pre[i] = chunks of items 0 .. i-1
+  for (int i = threadIdx.x; i < count; i += kBlock) pre[i + 1] = unsigned((table[i].n + kMixChunk - 1) / kMixChunk);
+  if (threadIdx.x == 0) pre[0] = 0;
+  __syncthreads();
+  if (threadIdx.x < 64) {  // wavefront 0: inclusive scan in tiles of 64 with a running carry
+    unsigned carry = 0;
+    for (int base = 0; base < count; base += 64) {
+      const int i = base + threadIdx.x;
+      unsigned v = i < count ? pre[i + 1] : 0u;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const unsigned u = __shfl_up(v, o, 64);
+        if (int(threadIdx.x) >= o) v += u;
+      }
+      v += carry;
+      if (i < count) pre[i + 1] = v;
+      carry = __shfl(v, 63, 64);
+    }
+  }
+  __syncthreads();
+  int it = 0;
+  for (unsigned chunk = blockIdx.x; chunk < pre[count]; chunk += gridDim.x) {
+    while (chunk >= pre[it + 1]) ++it;
+    const sgh_sgd_mixed_item item = table[it];
+    const bool has_v = h.mu != 0.f && item.v != nullptr;
+    const size_t base = size_t(chunk - pre[it]) * kMixChunk;
+    const size_t end = base + kMixChunk < item.n ? base + kMixChunk : size_t(item.n);
+    const float *g32 = static_cast<const float *>(item.g);
+    const u16 *g16 = static_cast<const u16 *>(item.g);
+    for (size_t i = base + threadIdx.x; i < end; i += kBlock) {
+      float pp = item.p[i];
+      float vv = has_v ? item.v[i] : 0.f;
+      sgd_one(pp, item.p16 ? T::load(g16[i]) : g32[i], vv, h, nesterov, has_v);
+      item.p[i] = pp;
+      if (has_v) item.v[i] = vv;
+      if (item.p16) item.p16[i] = T::store(pp);
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" {
+
+int sgh_sgd_momentum_multi_mixed(const sgh_sgd_mixed_item *table_dev, int count, size_t total_n, int bf16, float lr,
+                                 float mu, float damp, float wd, int nesterov, void *stream) {
+  if (count == 0) return SGH_OK;
+  if (!table_dev || count < 0 || count > kMixTab) return SGH_EINVAL;
+  size_t chunks = total_n / kMixChunk + size_t(count);  // upper bound on the sum of per-item chunk counts
+  const size_t cap = size_t(sgh_num_cus()) * 8;
+  if (chunks > cap) chunks = cap;
+  const SgdHyper h{lr, mu, damp, wd};
+  if (bf16) hipLaunchKernelGGL(k_sgd_multi_mixed<BF16>, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count, h, nesterov);
+  else hipLaunchKernelGGL(k_sgd_multi_mixed<F16>, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count, h, nesterov);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
 
 int sgh_sgd_momentum_f16(uint16_t *p, const uint16_t *g, uint16_t *v, size_t n, float lr, float mu, float damp,
                          float wd, int nesterov, void *stream) {

@@ -113,6 +113,46 @@ class SGD(object):
                                                     self.momentum, self.dampening, self.weight_decay,
                                                     int(self.nesterov), dev.stream), "sgh_sgd_momentum_multi_f32")
 
+    def apply_all_mixed(self, named_params_grads):
+        """``apply_all`` for a mixed-precision network: fp32 parameters and 16-bit parameters (updated
+        through fp32 master copies as in ``apply_master``) in ONE launch.  The 16-bit tensors must
+        all have the same type."""
+        items = list(named_params_grads)
+        if not items:
+            return
+        dev = items[0][1].device()
+        key = ("mixed",) + tuple((n, p.ptr, g.ptr) for n, p, g in items)
+        cached = self._tables.get(key)
+        if cached is None:
+            arr = (_lib.SgdMixedItem * len(items))()
+            total, half_type = 0, None
+            for i, (n, p, g) in enumerate(items):
+                assert p.shape() == g.shape(), ("shape mismatch", n)
+                if p.data_type() != g.data_type():
+                    raise singa.SingaHipError("parameter and gradient differ in data type")
+                if p.data_type() == singa.kFloat32:
+                    tgt, p16 = p, None
+                else:
+                    if half_type not in (None, p.data_type()):
+                        raise singa.SingaHipError("one 16-bit type per update")
+                    half_type = p.data_type()
+                    if n not in self.masters:
+                        self.masters[n] = p.AsType(singa.kFloat32)
+                    tgt, p16 = self.masters[n], p.ptr
+                v = self._moment(n, tgt) if self.momentum != 0 else None
+                arr[i].p, arr[i].g, arr[i].v, arr[i].p16, arr[i].n = tgt.ptr, g.ptr, (v.ptr if v is not None else None), p16, p.Size()
+                total += p.Size()
+            nbytes = C.sizeof(arr)
+            table = singa.Tensor(((nbytes + 3) // 4,), dev, singa.kInt)
+            check(_lib.lib().sgh_memcpy(dev._h, table.ptr, C.addressof(arr), nbytes, 1), "sgh_memcpy H2D")
+            if len(self._tables) >= 16:
+                self._tables.pop(next(iter(self._tables)))
+            cached = self._tables[key] = (table, total, int(half_type == singa.kBFloat16))
+        table, total, bf16 = cached
+        check(_lib.lib().sgh_sgd_momentum_multi_mixed(table.ptr, len(items), total, bf16, self.lr, self.momentum,
+                                                      self.dampening, self.weight_decay, int(self.nesterov),
+                                                      dev.stream), "sgh_sgd_momentum_multi_mixed")
+
     def step(self):
         self.step_counter += 1
 

@@ -150,6 +150,9 @@ class _MixedSGD(hip_opt.SGD):
             return self.apply_master(name, p, g)
         return super(_MixedSGD, self).apply(name, p, g)
 
+    def apply_all(self, named_params_grads):
+        return self.apply_all_mixed(named_params_grads)
+
 
 class HalfHipOps(HipOps):
     """Mixed precision as the reference trains in half (``layer.py:684-696`` casts the conv / linear

@@ -192,3 +192,25 @@ def test_graph_replay_of_the_step(dev):
     replayed.backward_and_update(fused_update=True)
     for (k, a), (_, b) in zip(eager.params(), replayed.params()):
         assert np.array_equal(hip.to_numpy(a), hip.to_numpy(b)), k
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+def test_mixed_precision_fused_update_equals_per_parameter_update(dev, kind):
+    """One launch over all parameters of the mixed-precision network (fp32 BatchNorm / classifier
+    parameters, 16-bit convolution weights with fp32 masters) leaves bit-identical parameters and
+    masters to the per-parameter updates."""
+    from singa_amd import singa_wrap as singa
+    dt = singa.kFloat16 if kind == "f16" else singa.kBFloat16
+    x, labels = wl.make_inputs("resnet50_small", 4)
+    outs = []
+    for fused in (False, True):
+        hip = wl.HalfHipOps(dev, dt)
+        net = wl.build("resnet50_small", hip, lr=0.01)
+        for _ in range(2):
+            net.forward(hip.from_numpy(x), hip.from_numpy(labels))
+            net.backward_and_update(fused_update=fused)
+        outs.append([hip.to_numpy(p) for _, p in net.params()] +
+                    [net.sgd.masters[k].to_numpy() for k in sorted(net.sgd.masters)])
+        assert len(net.sgd.masters) == 53
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
