@@ -64,6 +64,9 @@ bool sgh_dgrad_fewc_supported(const sgh_conv_geom *g);
 size_t sgh_dgrad_fewc_workspace_bytes(const sgh_conv_geom *g);
 int sgh_dgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
                        size_t ws_bytes, hipStream_t s);
+// the same kernel reading a 16-bit dy and writing a 16-bit dx (fp32 weights, slab and arithmetic)
+int sgh_dgrad_fewc_run16(const sgh_conv_geom *g, const uint16_t *dy, const float *W, uint16_t *dx, void *workspace,
+                         size_t ws_bytes, bool bf16, hipStream_t s);
 
 // Convolution gradients on 16-bit tensors with the 16-bit matrix instructions (conv16.hip).
 // *_workspace_bytes is 0 and the run functions return SGH_EUNSUPPORTED for geometries they do not

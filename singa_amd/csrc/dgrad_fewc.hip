@@ -20,6 +20,7 @@
 #include <stdlib.h>
 
 #include "common.h"
+#include "storage.h"
 
 namespace {
 
@@ -39,8 +40,9 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
 }
 
 struct DFArgs {
-  const float *dy, *aw;   // aw: A re-laid as [dp,dq (16)][K][16]
-  float *dx;
+  const void *dy;         // fp32, or 16-bit storage (template parameter S of the kernel)
+  const float *aw;        // A re-laid as [dp,dq (16)][K][16], always fp32
+  void *dx;
   int N, C, H, W, K, P, Q;
   int dp0, dq0;           // smallest row / column offset
 };
@@ -58,9 +60,12 @@ __global__ __launch_bounds__(256) void k_dgrad_fewc_weights(const float *__restr
   }
 }
 
-// QT: 16-column tiles per class row (Q <= 16 * QT)
-template <int QT>
+// QT: 16-column tiles per class row (Q <= 16 * QT); S: storage type of dy and dx (storage.h) -- the
+// slab in LDS, the weights and the arithmetic are fp32 in every case, a 16-bit dx is rounded once.
+template <int QT, class S>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_dgrad_fewc(DFArgs a) {
+  typedef typename S::elem elem;
+  constexpr int ES = int(sizeof(elem));
   constexpr int PITCH = QT * 16 + 8;                       // slab column of dy column q is q + 4
   constexpr int CHS0 = SROWS * PITCH;
   constexpr int CHS = CHS0 + ((16 - CHS0 % 32) + 32) % 32;  // = 16 mod 32: the four k of a B fragment hit disjoint banks
@@ -76,7 +81,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int i0 = blockIdx.x * TI, n = blockIdx.y;
   const int PQ = a.P * a.Q, HW = a.H * a.W, Q4 = a.Q >> 2;
-  const rsrc_t rdy = make_rsrc(a.dy + size_t(n) * a.K * PQ, unsigned(a.K) * PQ * 4u);
+  const rsrc_t rdy = make_rsrc(static_cast<const elem *>(a.dy) + size_t(n) * a.K * PQ, unsigned(a.K) * PQ * unsigned(ES));
   const rsrc_t ra = make_rsrc(a.aw, unsigned(ND * ND) * a.K * 16 * 4u);
 
   // pad columns and rows outside the image stay zero: only image columns are (re)written
@@ -90,12 +95,22 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const int f = e * NT + t, kc = f / (SROWS * Q4), rem = f - kc * (SROWS * Q4), sr = rem / Q4, c4 = rem - sr * Q4;
     const int p = i0 + a.dp0 + sr;
     const bool ok = kc < KC && unsigned(p) < unsigned(a.P);
-    sg[e] = ok ? ((kc * a.P + p) * a.Q + c4 * 4) * 4 : kOOB;
+    sg[e] = ok ? ((kc * a.P + p) * a.Q + c4 * 4) * ES : kOOB;
     sl[e] = kc < KC ? kc * CHS + sr * PITCH + 4 + c4 * 4 : -1;
   }
   const int ag = ((t >> 5) * a.K * 16 + (t & 31) * 4) * 4;   // A float4 index t: offset t / 32, (k, m) slice t % 32
   auto ldv = [&](rsrc_t r, int voff) -> v4f {
     return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
+  };
+  auto ld_dy = [&](int voff) -> v4f {   // four consecutive dy elements as floats
+    if constexpr (ES == 4) {
+      return ldv(rdy, voff);
+    } else {
+      typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+      const v2u w = __builtin_bit_cast(v2u, __builtin_amdgcn_raw_buffer_load_b64(rdy, voff, 0, 0));
+      const elem h[4] = {elem(w[0] & 0xffffu), elem(w[0] >> 16), elem(w[1] & 0xffffu), elem(w[1] >> 16)};
+      return v4f{S::ld(h), S::ld(h + 1), S::ld(h + 2), S::ld(h + 3)};
+    }
   };
 
   // ---- operand lane constants -------------------------------------------------------------------
@@ -112,7 +127,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   __syncthreads();  // zero fill done
 #pragma unroll
   for (int e = 0; e < SSLOTS; ++e) {
-    const v4f v = ldv(rdy, sg[e]);
+    const v4f v = ld_dy(sg[e]);
     if (sl[e] >= 0) *reinterpret_cast<v4f *>(dyS + sl[e]) = v;
   }
   *reinterpret_cast<v4f *>(aS + t * 4) = ldv(ra, ag);
@@ -126,7 +141,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const int k1 = (ch + 1) * KC;
     v4f ns[SSLOTS];
 #pragma unroll
-    for (int e = 0; e < SSLOTS; ++e) ns[e] = ldv(rdy, sg[e] + k1 * PQ * 4);
+    for (int e = 0; e < SSLOTS; ++e) ns[e] = ld_dy(sg[e] + k1 * PQ * ES);
     const v4f na = ldv(ra, ag + k1 * 16 * 4);
 
     float av[2], bv[2][QT];
@@ -156,13 +171,20 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   // epilogue: lane group lane / 16 is the channel, register v = a*2 + b the position in the 2x2 block
   const int c = lane >> 4, i = i0 + wave;
   if (c < a.C && i < a.P) {
-    float *o = a.dx + (size_t(n) * a.C + c) * HW + size_t(2 * i) * a.W;
+    elem *o = static_cast<elem *>(a.dx) + (size_t(n) * a.C + c) * HW + size_t(2 * i) * a.W;
 #pragma unroll
     for (int j = 0; j < QT; ++j) {
       const int q = j * 16 + (lane & 15);
       if (q < a.Q) {
-        *reinterpret_cast<v2f *>(o + 2 * q) = v2f{acc[j][0], acc[j][1]};
-        *reinterpret_cast<v2f *>(o + a.W + 2 * q) = v2f{acc[j][2], acc[j][3]};
+        if constexpr (ES == 4) {
+          *reinterpret_cast<v2f *>(o + 2 * q) = v2f{acc[j][0], acc[j][1]};
+          *reinterpret_cast<v2f *>(o + a.W + 2 * q) = v2f{acc[j][2], acc[j][3]};
+        } else {   // two 16-bit elements per 4-byte store (W is even: the pairs are aligned)
+          elem r0[2], r1[2];
+          S::st(r0, acc[j][0]), S::st(r0 + 1, acc[j][1]), S::st(r1, acc[j][2]), S::st(r1 + 1, acc[j][3]);
+          *reinterpret_cast<unsigned *>(o + 2 * q) = unsigned(r0[0]) | (unsigned(r0[1]) << 16);
+          *reinterpret_cast<unsigned *>(o + a.W + 2 * q) = unsigned(r1[0]) | (unsigned(r1[1]) << 16);
+        }
       }
     }
   }
@@ -211,9 +233,9 @@ inline DFPlan plan(const sgh_conv_geom *g) {
   return p;
 }
 
-template <int QT>
+template <int QT, class S>
 int launch(const DFArgs &a, const DFPlan &p, dim3 grid, hipStream_t s) {
-  auto kern = k_dgrad_fewc<QT>;
+  auto kern = k_dgrad_fewc<QT, S>;
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -233,8 +255,10 @@ size_t sgh_dgrad_fewc_workspace_bytes(const sgh_conv_geom *g) {
   return plan(g).ok ? size_t(ND * ND) * g->K * 16 * sizeof(float) : 0;
 }
 
-int sgh_dgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
-                       size_t ws_bytes, hipStream_t s) {
+// dy / dx in storage type S (fp32 weights W in every case)
+template <class S>
+static int dgrad_fewc_run(const sgh_conv_geom *g, const void *dy, const float *W, void *dx, void *workspace,
+                          size_t ws_bytes, hipStream_t s, const char *tag) {
   const DFPlan p = plan(g);
   if (!p.ok) return SGH_EUNSUPPORTED;
   if (!workspace || ws_bytes < sgh_dgrad_fewc_workspace_bytes(g)) return SGH_EWORKSPACE;
@@ -258,18 +282,29 @@ int sgh_dgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *W, 
   dim3 grid((g->P + TI - 1) / TI, g->N, 1);
   if (grid.y > 65535u) return SGH_EUNSUPPORTED;
   int rc = SGH_EUNSUPPORTED;
-  sgh_prof_start("conv_dgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S, s);
+  sgh_prof_start(tag, 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S, s);
   switch (p.qt) {
-    case 1: rc = launch<1>(a, p, grid, s); break;
-    case 2: rc = launch<2>(a, p, grid, s); break;
-    case 3: rc = launch<3>(a, p, grid, s); break;
-    case 4: rc = launch<4>(a, p, grid, s); break;
-    case 5: rc = launch<5>(a, p, grid, s); break;
-    case 6: rc = launch<6>(a, p, grid, s); break;
-    case 7: rc = launch<7>(a, p, grid, s); break;
-    case 8: rc = launch<8>(a, p, grid, s); break;
+    case 1: rc = launch<1, S>(a, p, grid, s); break;
+    case 2: rc = launch<2, S>(a, p, grid, s); break;
+    case 3: rc = launch<3, S>(a, p, grid, s); break;
+    case 4: rc = launch<4, S>(a, p, grid, s); break;
+    case 5: rc = launch<5, S>(a, p, grid, s); break;
+    case 6: rc = launch<6, S>(a, p, grid, s); break;
+    case 7: rc = launch<7, S>(a, p, grid, s); break;
+    case 8: rc = launch<8, S>(a, p, grid, s); break;
     default: break;
   }
   sgh_prof_stop(s);
   return rc;
+}
+
+int sgh_dgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
+                       size_t ws_bytes, hipStream_t s) {
+  return dgrad_fewc_run<StF32>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad");
+}
+
+int sgh_dgrad_fewc_run16(const sgh_conv_geom *g, const uint16_t *dy, const float *W, uint16_t *dx, void *workspace,
+                         size_t ws_bytes, bool bf16, hipStream_t s) {
+  return bf16 ? dgrad_fewc_run<StBF16>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad16")
+              : dgrad_fewc_run<StF16>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad16");
 }

@@ -1237,6 +1237,18 @@ int conv_half(const sgh_conv_geom *g, int which, const uint16_t *a, const uint16
                        : sgh_conv16_wgrad(g, a, b, out, workspace, ws_bytes, bf16, sgh_stream_of(stream));
     if (rc != SGH_EUNSUPPORTED) return rc;
   }
+  // the stem's data gradient (few input channels, large filter): the fp32 kernel reads the 16-bit
+  // gradient and writes the 16-bit result itself; only the small weight tensor is widened
+  if (which == SGH_CONV_DGRAD && sgh_dgrad_fewc_supported(g) && !getenv("SGH_CONV16_OFF")) {
+    const size_t w_elems = size_t(g->K) * g->C * g->R * g->S, w_bytes = align256(w_elems * 4);
+    if (!workspace || ws_bytes < w_bytes + sgh_dgrad_fewc_workspace_bytes(g)) return SGH_EWORKSPACE;
+    float *w32 = static_cast<float *>(workspace);
+    int rc = in(b, w32, w_elems, stream);
+    if (rc != SGH_OK) return rc;
+    rc = sgh_dgrad_fewc_run16(g, a, w32, out, static_cast<char *>(workspace) + w_bytes, ws_bytes - w_bytes,
+                              in == sgh_cast_bf16_to_f32, sgh_stream_of(stream));
+    if (rc != SGH_EUNSUPPORTED) return rc;
+  }
   const HalfPlan p = half_plan(g, which);
   if (!workspace || ws_bytes < p.total() + (bias ? align256(size_t(g->K) * 4) : 0)) return SGH_EWORKSPACE;
   char *w = static_cast<char *>(workspace);
