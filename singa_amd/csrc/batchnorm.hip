@@ -201,7 +201,7 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_partial(const typename S::ele
   const int c = blockIdx.x / s.S, sp = blockIdx.x % s.S;
   const float mean = save_mean[c], invstd = save_invstd[c];
   const float g = RELU ? gamma[c] : 0.f, be = RELU ? beta[c] : 0.f;
-  auto gate = [&](float d, float v) { return !RELU || S::stored(bn_out(v, mean, invstd, g, be)) > 0.f ? d : 0.f; };
+  auto gate = [&](float d, float v) { return !RELU || S::stored_positive(bn_out(v, mean, invstd, g, be)) ? d : 0.f; };
   // (the products are accumulated with explicit fused multiply-adds: the fused and the plain
   // instantiation then round identically whatever the compiler does around the gate)
   float a = 0.f, b = 0.f, b1 = 0.f;
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const typename S::elem 
   const float k = g * invstd;
   const float rM = float(1.0 / (double(s.N) * s.HW));
   const float c0 = db * rM, c1 = dg * rM;
-  auto gate = [&](float d, float v) { return !RELU || S::stored(bn_out(v, mean, invstd, g, be)) > 0.f ? d : 0.f; };
+  auto gate = [&](float d, float v) { return !RELU || S::stored_positive(bn_out(v, mean, invstd, g, be)) ? d : 0.f; };
   channel_range<kBlock, S>(
       s, c, sp * s.per_split, (sp + 1) * s.per_split, x, dy,
       [&](size_t off, const float *v, const float *d) {
@@ -363,8 +363,9 @@ extern "C" {
 size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
   if (!shape_ok(N, C, HW)) return 0;
   // one size for every storage type: the larger of the fp32 and the 16-bit split counts
-  const int s4 = make_shape(N, C, HW, 4, 4).S, s8 = make_shape(N, C, HW, 8, 2).S;
-  return size_t(C) * (s4 > s8 ? s4 : s8) * 2 * sizeof(float);
+  const int s4 = make_shape(N, C, HW, 4, 4).S, s8 = make_shape(N, C, HW, 8, 2).S, s4h = make_shape(N, C, HW, 4, 2).S;
+  const int smax = s4 > s8 ? (s4 > s4h ? s4 : s4h) : (s8 > s4h ? s8 : s4h);
+  return size_t(C) * smax * 2 * sizeof(float);
 }
 
 int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float *beta, float *running_mean,
@@ -376,12 +377,16 @@ int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float *beta, 
 int sgh_bn_fwd_train_f16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
                          float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
                          float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  if (HW % 8 != 0 && HW % 4 == 0) return bn_fwd_train<StF16x4>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C, HW,
+                             workspace, ws_bytes, stream);  // 8-byte vectors (e.g. 14 x 14 planes)
   return bn_fwd_train<StF16>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C, HW,
                              workspace, ws_bytes, stream);
 }
 int sgh_bn_fwd_train_bf16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
                           float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
                           float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  if (HW % 8 != 0 && HW % 4 == 0) return bn_fwd_train<StBF16x4>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C,
+                              HW, workspace, ws_bytes, stream);  // 8-byte vectors (e.g. 14 x 14 planes)
   return bn_fwd_train<StBF16>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C,
                               HW, workspace, ws_bytes, stream);
 }
@@ -395,12 +400,16 @@ int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const fl
 int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                    const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                    void *workspace, size_t ws_bytes, void *stream) {
+  if (HW % 8 != 0 && HW % 4 == 0) return bn_bwd<StF16x4>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                       stream);  // 8-byte vectors (e.g. 14 x 14 planes)
   return bn_bwd<StF16>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
                        stream);
 }
 int sgh_bn_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                     const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                     void *workspace, size_t ws_bytes, void *stream) {
+  if (HW % 8 != 0 && HW % 4 == 0) return bn_bwd<StBF16x4>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                        stream);  // 8-byte vectors (e.g. 14 x 14 planes)
   return bn_bwd<StBF16>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
                         stream);
 }
@@ -411,10 +420,12 @@ int sgh_bn_fwd_infer_f32(const float *x, const float *gamma, const float *beta, 
 }
 int sgh_bn_fwd_infer_f16(const uint16_t *x, const float *gamma, const float *beta, const float *running_mean,
                          const float *running_var, float eps, uint16_t *y, int N, int C, int HW, void *stream) {
+  if (HW % 8 != 0 && HW % 4 == 0) return bn_fwd_infer<StF16x4>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);  // 8-byte vectors (e.g. 14 x 14 planes)
   return bn_fwd_infer<StF16>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);
 }
 int sgh_bn_fwd_infer_bf16(const uint16_t *x, const float *gamma, const float *beta, const float *running_mean,
                           const float *running_var, float eps, uint16_t *y, int N, int C, int HW, void *stream) {
+  if (HW % 8 != 0 && HW % 4 == 0) return bn_fwd_infer<StBF16x4>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);  // 8-byte vectors (e.g. 14 x 14 planes)
   return bn_fwd_infer<StBF16>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);
 }
 
@@ -429,6 +440,8 @@ int sgh_bn_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamm
                         const float *save_mean, const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta,
                         int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   if (!beta) return SGH_EINVAL;
+  if (HW % 8 != 0 && HW % 4 == 0) return bn_bwd<StF16x4>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                       stream);  // 8-byte vectors (e.g. 14 x 14 planes)
   return bn_bwd<StF16>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
                        stream);
 }
@@ -436,6 +449,8 @@ int sgh_bn_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gam
                          const float *save_mean, const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta,
                          int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   if (!beta) return SGH_EINVAL;
+  if (HW % 8 != 0 && HW % 4 == 0) return bn_bwd<StBF16x4>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
+                        stream);  // 8-byte vectors (e.g. 14 x 14 planes)
   return bn_bwd<StBF16>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
                         stream);
 }

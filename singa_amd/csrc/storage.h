@@ -35,6 +35,7 @@ struct StF32 {
   static __device__ __forceinline__ float ld(const elem *p) { return *p; }
   static __device__ __forceinline__ void st(elem *p, float v) { *p = v; }
   static __device__ __forceinline__ float stored(float v) { return v; }  // the value a store keeps
+  static __device__ __forceinline__ bool stored_positive(float v) { return v > 0.f; }
   template <bool NT>
   static __device__ __forceinline__ void load16(const elem *p, float *out) {
     const sgh_v4f v = NT ? __builtin_nontemporal_load(reinterpret_cast<const sgh_v4f *>(p))
@@ -49,32 +50,42 @@ struct StF32 {
   }
 };
 
-template <float (*LD)(uint16_t), uint16_t (*ST)(float)>
+// TINY: the largest float that the store rounds to zero (half of the smallest subnormal of the
+// 16-bit type: a tie, and ties go to the even neighbour 0), so "the stored value is > 0" is v > TINY.
+// HALFVEC: the vector accesses move 8 bytes (4 elements) instead of 16, for tensors whose rows are
+// 8- but not 16-byte aligned (e.g. 14 x 14 planes).
+template <float (*LD)(uint16_t), uint16_t (*ST)(float), unsigned TINY_BITS, bool HALFVEC = false>
 struct St16 {
   typedef uint16_t elem;
-  static constexpr int VEC = 8;
+  static constexpr int VEC = HALFVEC ? 4 : 8;
   static __device__ __forceinline__ float ld(const elem *p) { return LD(*p); }
   static __device__ __forceinline__ void st(elem *p, float v) { *p = ST(v); }
   static __device__ __forceinline__ float stored(float v) { return LD(ST(v)); }  // the value a store keeps
+  static __device__ __forceinline__ bool stored_positive(float v) { return v > __builtin_bit_cast(float, TINY_BITS); }
   template <bool NT>
-  static __device__ __forceinline__ void load16(const elem *p, float *out) {
-    const sgh_v4u v = NT ? __builtin_nontemporal_load(reinterpret_cast<const sgh_v4u *>(p))
-                         : *reinterpret_cast<const sgh_v4u *>(p);
+  static __device__ __forceinline__ void load16(const elem *p, float *out) {   // one vector access: VEC elements
+    typedef unsigned int vec __attribute__((ext_vector_type(VEC / 2)));
+    const vec v = NT ? __builtin_nontemporal_load(reinterpret_cast<const vec *>(p)) : *reinterpret_cast<const vec *>(p);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < VEC / 2; ++j) {
       out[2 * j] = LD(uint16_t(v[j] & 0xffffu));
       out[2 * j + 1] = LD(uint16_t(v[j] >> 16));
     }
   }
   static __device__ __forceinline__ void store16(elem *p, const float *in) {
-    sgh_v4u r;
+    typedef unsigned int vec __attribute__((ext_vector_type(VEC / 2)));
+    vec r;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) r[j] = unsigned(ST(in[2 * j])) | (unsigned(ST(in[2 * j + 1])) << 16);
-    *reinterpret_cast<sgh_v4u *>(p) = r;
+    for (int j = 0; j < VEC / 2; ++j) r[j] = unsigned(ST(in[2 * j])) | (unsigned(ST(in[2 * j + 1])) << 16);
+    *reinterpret_cast<vec *>(p) = r;
   }
 };
 
-typedef St16<sgh_f16_to_f32, sgh_f32_to_f16> StF16;
-typedef St16<sgh_bf16_to_f32, sgh_f32_to_bf16> StBF16;
+// binary16: smallest subnormal 2^-24, so 2^-25 (0x33000000) and below store as 0;
+// bfloat16: smallest subnormal 2^-133, so 2^-134 (fp32 subnormal 0x00008000) and below store as 0
+typedef St16<sgh_f16_to_f32, sgh_f32_to_f16, 0x33000000u> StF16;
+typedef St16<sgh_bf16_to_f32, sgh_f32_to_bf16, 0x00008000u> StBF16;
+typedef St16<sgh_f16_to_f32, sgh_f32_to_f16, 0x33000000u, true> StF16x4;
+typedef St16<sgh_bf16_to_f32, sgh_f32_to_bf16, 0x00008000u, true> StBF16x4;
 
 #endif  // SINGA_AMD_CSRC_STORAGE_H_
