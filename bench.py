@@ -108,7 +108,7 @@ def main():
     dev = singa.create_hip_gpu_on(0)
     half = args.storage != "f32"
     hip = wl.HalfHipOps(dev, singa.kFloat16 if args.storage == "f16" else singa.kBFloat16) if half else wl.HipOps(dev)
-    hip.fuse_bn_relu = hip.fuse_dgrad_add = not args.no_fusion
+    hip.set_fusion(not args.no_fusion)
     net = wl.build(args.config, hip, lr=0.05, momentum=0.9)
     x, labels = wl.make_inputs(args.config, args.batch)
     net.forward(hip.from_numpy(x), hip.from_numpy(labels))
@@ -188,7 +188,8 @@ def main():
                        args.config, args.batch, "fp32" if not half else args.storage + " storage / fp32 accumulate, statistics and master weights"),
                    "update": "fused multi-tensor" if fused else "per parameter",
                    "launch": "one recorded step replayed (graph mode)" if graph else "eager, one launch per kernel",
-                   "tape": "ReLU backward folded into BatchNorm backward (conv-BN-ReLU), residual += folded into the data gradient"
+                   "tape": "ReLU backward folded into BatchNorm backward (conv-BN-ReLU), residual += folded into the "
+                           + ("data gradient" if hip.fuse_dgrad_add else "ReLU backward that reads the sum")
                            if hip.fuse_bn_relu
                            else "one call per reference op"},
         "roofline": roofline,

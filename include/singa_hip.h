@@ -187,6 +187,16 @@ SGH_API int sgh_cast_bf16_to_f32(const uint16_t *src, float *dst, size_t n, void
  * CPU rule dx = x > 0 ? dy : 0 (the CUDA half kernel alone passes the gradient at x == 0). */
 SGH_API int sgh_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream);
 SGH_API int sgh_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream);
+/* ReLU backward on a gradient that arrives as two summands: dx[i] = x[i] > 0 ? dy0[i] + dy1[i] : 0,
+ * the sum in fp32 and one rounding at the store -- bit-identical to the reference's two steps, the
+ * gradient fan-in `dy0 += dy1` of a residual connection (python/singa/autograd.py:204) followed by
+ * ReLUBackward (tensor_math.h:175-179), without storing the sum.  dx may alias dy0 or dy1. */
+SGH_API int sgh_relu_bwd_add_f32(const float *dy0, const float *dy1, const float *x, float *dx, size_t n,
+                                 void *stream);
+SGH_API int sgh_relu_bwd_add_f16(const uint16_t *dy0, const uint16_t *dy1, const uint16_t *x,
+                                 uint16_t *dx, size_t n, void *stream);
+SGH_API int sgh_relu_bwd_add_bf16(const uint16_t *dy0, const uint16_t *dy1, const uint16_t *x,
+                                  uint16_t *dx, size_t n, void *stream);
 /* Add / EltwiseMult<half, Lang>: tensor_math_cuda.h:345-362, math_kernel.cu:111-117, :353-359.
  * out may alias an input. */
 SGH_API int sgh_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream);
@@ -318,8 +328,11 @@ SGH_API int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float
 
 /* The three convolution passes on 16-bit tensors (x, W, y and their gradients all binary16 or
  * all bfloat16, as a reference handle built from a half input runs them:
- * src/model/operation/convolution.cc:444-572).  Arithmetic: the operands are widened to fp32 in
- * the workspace, the fp32 MFMA kernels accumulate in fp32, the result is rounded once.
+ * src/model/operation/convolution.cc:444-572).  Arithmetic: fp32 accumulation of exact 16-bit
+ * products, the result rounded once.  The two gradients run on the 16-bit matrix instructions
+ * (stride 1 or 2; data gradient: K a multiple of 8, C >= 16, Q >= 2), the stem's data gradient on
+ * the fp32 kernel reading and writing 16-bit tensors; other geometries and the forward pass widen
+ * the operands to fp32 in the workspace and use the fp32 kernels.
  * Workspace: sgh_conv_workspace_bytes_h(g, which) bytes. */
 SGH_API size_t sgh_conv_workspace_bytes_h(const sgh_conv_geom *g, int which);
 SGH_API int sgh_conv_dgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W,

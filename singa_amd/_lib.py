@@ -89,6 +89,9 @@ SIGNATURES = {
     "sgh_cast_f32_to_bf16": (C.c_int, [vp, vp, sz, vp]),
     "sgh_cast_bf16_to_f32": (C.c_int, [vp, vp, sz, vp]),
     "sgh_relu_bwd_f16": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_relu_bwd_add_f32": (C.c_int, [vp, vp, vp, vp, sz, vp]),
+    "sgh_relu_bwd_add_f16": (C.c_int, [vp, vp, vp, vp, sz, vp]),
+    "sgh_relu_bwd_add_bf16": (C.c_int, [vp, vp, vp, vp, sz, vp]),
     "sgh_relu_bwd_bf16": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_add_f16": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_add_bf16": (C.c_int, [vp, vp, vp, sz, vp]),

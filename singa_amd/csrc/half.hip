@@ -96,6 +96,61 @@ int launch_map2_h(const uint16_t *a, const uint16_t *b, uint16_t *o, size_t n, F
 struct ReluBwd {
   __device__ __forceinline__ float operator()(float dy, float x) const { return x > 0.f ? dy : 0.f; }
 };
+
+// dx = x > 0 ? dy0 + dy1 : 0: ReLU backward on a gradient that arrives as two summands (the two
+// branches of a residual block), so that the sum is never stored.  dx may alias dy0 or dy1.
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_relu_bwd_add(const typename S::elem *dy0, const typename S::elem *dy1,
+                                                         const typename S::elem *x, typename S::elem *dx, size_t n,
+                                                         int vec) {
+  constexpr int V = S::VEC;
+  if (vec) {
+    const size_t nvec = n / V;
+    const size_t step = size_t(gridDim.x) * (kBlock * kUnroll);
+    for (size_t base = size_t(blockIdx.x) * (kBlock * kUnroll); base < nvec; base += step) {
+      float a[kUnroll][V], b[kUnroll][V], g[kUnroll][V];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const size_t i = base + u * kBlock + threadIdx.x;
+        if (i < nvec) {
+          S::template load16<true>(dy0 + i * V, a[u]);
+          S::template load16<true>(dy1 + i * V, b[u]);
+          S::template load16<true>(x + i * V, g[u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const size_t i = base + u * kBlock + threadIdx.x;
+        if (i < nvec) {
+          float r[V];
+#pragma unroll
+          for (int j = 0; j < V; ++j) r[j] = g[u][j] > 0.f ? a[u][j] + b[u][j] : 0.f;
+          S::store16(dx + i * V, r);
+        }
+      }
+    }
+    if (blockIdx.x == 0) {
+      const size_t t = nvec * V + threadIdx.x;
+      if (t < n) S::st(dx + t, S::ld(x + t) > 0.f ? S::ld(dy0 + t) + S::ld(dy1 + t) : 0.f);
+    }
+  } else {
+    const size_t stride = size_t(gridDim.x) * kBlock;
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride)
+      S::st(dx + i, S::ld(x + i) > 0.f ? S::ld(dy0 + i) + S::ld(dy1 + i) : 0.f);
+  }
+}
+
+template <class S>
+int launch_relu_bwd_add(const typename S::elem *dy0, const typename S::elem *dy1, const typename S::elem *x,
+                        typename S::elem *dx, size_t n, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!dy0 || !dy1 || !x || !dx) return SGH_EINVAL;
+  const int vec = sgh_aligned16(dy0) && sgh_aligned16(dy1) && sgh_aligned16(x) && sgh_aligned16(dx);
+  hipLaunchKernelGGL(k_relu_bwd_add<S>, dim3(grid_for(vec ? n / S::VEC : n)), dim3(kBlock), 0, sgh_stream_of(stream),
+                     dy0, dy1, x, dx, n, vec);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
 struct AddOp {
   __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
 };
@@ -317,6 +372,17 @@ int sgh_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t
 }
 int sgh_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream) {
   return launch_map2_h<BF16>(dy, x, dx, n, ReluBwd{}, stream);
+}
+int sgh_relu_bwd_add_f32(const float *dy0, const float *dy1, const float *x, float *dx, size_t n, void *stream) {
+  return launch_relu_bwd_add<StF32>(dy0, dy1, x, dx, n, stream);
+}
+int sgh_relu_bwd_add_f16(const uint16_t *dy0, const uint16_t *dy1, const uint16_t *x, uint16_t *dx, size_t n,
+                         void *stream) {
+  return launch_relu_bwd_add<StF16>(dy0, dy1, x, dx, n, stream);
+}
+int sgh_relu_bwd_add_bf16(const uint16_t *dy0, const uint16_t *dy1, const uint16_t *x, uint16_t *dx, size_t n,
+                          void *stream) {
+  return launch_relu_bwd_add<StBF16>(dy0, dy1, x, dx, n, stream);
 }
 int sgh_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
   return launch_map2_h<F16>(a, b, out, n, AddOp{}, stream);

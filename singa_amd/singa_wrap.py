@@ -375,6 +375,18 @@ def ReLUBackward(dy, x):
     return dx
 
 
+def ReLUBackwardSum(dy0, dy1, x):
+    """``ReLUBackward(dy0 + dy1, x)`` without storing the sum: the fan-in ``+=`` of a residual
+    connection (python/singa/autograd.py:204) folded into the ReLU backward that reads it
+    (python/singa/autograd.py:432-439); bit-identical to the two steps."""
+    _same(dy0, x)
+    _same(dy1, x)
+    dx = _like(dy0)
+    fn, name = _fn("relu_bwd_add", dy0)
+    check(fn(dy0.ptr, dy1.ptr, x.ptr, dx.ptr, dy0.Size(), dy0.device().stream), name)
+    return dx
+
+
 def SoftMax(x):
     batch = x.shape(0) if x.nDim() == 2 else 1
     p = _like(x)
@@ -591,7 +603,7 @@ def GpuConvBackwardxAccumulate(dy, W, x, h, dx):
     gradient where the kernel supports it, otherwise the two separate steps."""
     h._check_dy(dy)
     _same(dx, x)
-    if dy.data_type() == kFloat32:
+    if dy.data_type() == kFloat32:   # (on 16-bit tensors the kernel's read-modify-write loses to the separate add)
         rc = _L().sgh_conv_dgrad_acc_f32(C.byref(h.geom), dy.ptr, W.ptr, dx.ptr, h.workspace.ptr,
                                          h.workspace.MemSize(), dy.device().stream)
         if rc != _lib.SGH_EUNSUPPORTED:

@@ -126,6 +126,20 @@ class HipOps(object):
     def conv_bwd_b(self, dy, b, h):
         return singa.GpuConvBackwardb(dy, b, h)
 
+    # cross-op fusion the tape permits: a residual block hands its input gradient on as two summands
+    # and the ReLU backward of the block before adds them while gating (HalfHipOps turns it on)
+    fuse_add_relu = False
+
+    def relu_bwd_add(self, dy0, dy1, x):
+        return singa.ReLUBackwardSum(dy0, dy1, x)
+
+    fusions = ("fuse_bn_relu", "fuse_dgrad_add")   # what set_fusion(True) turns on
+
+    def set_fusion(self, on):
+        """All of this implementation's cross-op fusions on, or the reference's op-per-op tape."""
+        for f in ("fuse_bn_relu", "fuse_dgrad_add", "fuse_add_relu"):
+            setattr(self, f, bool(on) and f in self.fusions)
+
     def accumulate(self, a, b):
         a += b
         return a
@@ -160,6 +174,12 @@ class HalfHipOps(HipOps):
     4-D tensors -- activations, their gradients and convolution weights -- are stored in `dtype`
     (binary16 or bfloat16), BatchNorm parameters / statistics and the classifier head stay fp32,
     16-bit weights are updated through fp32 master copies."""
+
+    # the residual "+=": folded into the next ReLU backward (the 16-bit data-gradient kernel's
+    # scattered 2-byte stores make a read-modify-write epilogue slower than the separate add)
+    fuse_dgrad_add = False
+    fuse_add_relu = True
+    fusions = ("fuse_bn_relu", "fuse_add_relu")
 
     def __init__(self, dev, dtype):
         HipOps.__init__(self, dev)
@@ -260,6 +280,19 @@ class BatchNorm(_Layer):
         return dx
 
 
+class _Sum:
+    """A gradient still in two summands (``a`` freshly computed and owned by the tape, ``b`` possibly
+    shared): what a residual block returns under ``fuse_add_relu``; consumed by the ReLU backward of
+    the block before, or summed by ``_summed`` for any other reader."""
+
+    def __init__(self, a, b):
+        self.a, self.b = a, b
+
+
+def _summed(ops, dy):
+    return ops.accumulate(dy.a, dy.b) if isinstance(dy, _Sum) else dy
+
+
 class ReLU(_Layer):
     def __init__(self, ops, name):
         self.ops, self.name = ops, name
@@ -269,6 +302,8 @@ class ReLU(_Layer):
         return self.ops.relu(x)
 
     def bwd(self, dy, grads):
+        if isinstance(dy, _Sum):
+            return self.ops.relu_bwd_add(dy.a, dy.b, self.x)
         return self.ops.relu_bwd(dy, self.x)
 
 
@@ -373,6 +408,8 @@ class BasicBlock(_Layer):
         if getattr(self.ops, "fuse_dgrad_add", False):
             return self.conv1.bwd(d, grads, add_into=d_res)   # every other reader of d_res is done by now
         d_main = self.conv1.bwd(d, grads)
+        if getattr(self.ops, "fuse_add_relu", False):
+            return _Sum(d_main, d_res)
         if d_res is d_add:
             # the first-arrived buffer is another op's input gradient: accumulate into the fresh one
             return self.ops.accumulate(d_main, d_res)
@@ -429,6 +466,8 @@ class Bottleneck(_Layer):
         if getattr(self.ops, "fuse_dgrad_add", False):
             return self.conv1.bwd(d, grads, add_into=d_res)
         d_main = self.conv1.bwd(d, grads)
+        if getattr(self.ops, "fuse_add_relu", False):
+            return _Sum(d_main, d_res)
         if d_res is d_add:
             return self.ops.accumulate(d_main, d_res)
         return self.ops.accumulate(d_res, d_main)
@@ -504,11 +543,14 @@ class Net(object):
         i = 0
         while i < len(rev):
             if isinstance(rev[i], ReLU) and i + 1 < len(rev) and isinstance(rev[i + 1], BatchNorm):
-                dy = rev[i + 1].bwd_through_relu(rev[i], dy, grads)   # the stem's conv -> BatchNorm -> ReLU
+                dy = rev[i + 1].bwd_through_relu(rev[i], _summed(ops, dy), grads)   # the stem's conv -> BatchNorm -> ReLU
                 i += 2
             else:
+                if not isinstance(rev[i], (BasicBlock, Bottleneck)):
+                    dy = _summed(ops, dy)
                 dy = rev[i].bwd(dy, grads)
                 i += 1
+        dy = _summed(ops, dy)
         if keep_grads:
             self.grad_log["input"] = dy
         if fused_update:

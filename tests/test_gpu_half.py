@@ -76,6 +76,11 @@ def test_relu_backward_add_mult_axpy(singa, dev, kind, n):
     xt, x = _to(singa, dev, _special(r, n), kind)
     # ReLU backward: a select, so exact; gradient 0 at x == 0 (and at -0.0, NaN)
     _same_bits(singa.ReLUBackward(dyt, xt).to_numpy(), np.where(x > 0, dy, np.float32(0)), "relu_bwd " + kind)
+    # ReLU backward of a gradient in two summands: the fp32 sum rounded once, then the select
+    d1t, d1 = _to(singa, dev, _special(r, n), kind)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = np.where(x > 0, _round(singa, dy + d1, kind), np.float32(0))
+    _same_bits(singa.ReLUBackwardSum(dyt, d1t, xt).to_numpy(), want, "relu_bwd_add " + kind)
     with np.errstate(invalid="ignore", over="ignore"):
         _same_bits(singa.__add__(dyt, xt).to_numpy(), _round(singa, dy + x, kind), "add " + kind)
         _same_bits(singa.EltwiseMult(dyt, xt).to_numpy(), _round(singa, dy * x, kind), "mult " + kind)
@@ -313,6 +318,11 @@ def test_conv_gradients_16bit_matrix_kernels(singa, dev, kind, case):
     print("16-bit gradients nl2: dx %.2e dw %.2e" % e)
     assert max(e) < 1e-2
     _same_bits(singa.GpuConvBackwardW(dyt, xt, wt, h).to_numpy(), dw.to_numpy(), "wgrad run-to-run")
+    # dx_old += dgrad on 16-bit tensors: the data gradient and a separate 16-bit add (two roundings)
+    oldt, old = _to(singa, dev, r.standard_normal((N, C, H, W)).astype(np.float32), kind)
+    got = singa.GpuConvBackwardxAccumulate(dyt, wt, xt, h, oldt)
+    assert got is oldt
+    _same_bits(got.to_numpy(), _round(singa, old + dx.to_numpy(), kind), "dx += dgrad")
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])

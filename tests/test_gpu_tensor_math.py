@@ -40,6 +40,21 @@ def test_relu_backward(singa, dev, n):
     assert_bit_equal(dx, O.relu_bwd(dy, x), "relu_bwd n=%d" % n)
 
 
+@pytest.mark.parametrize("n", [1, 5, 1024, 4099, 1 << 20])
+def test_relu_backward_of_two_summands(singa, dev, n):
+    """ReLUBackwardSum(dy0, dy1, x) = ReLUBackward(dy0 + dy1, x) bit for bit (oracle: the fp32 sum,
+    then the select), also through the scalar path of unaligned pointers."""
+    r = rng(n + 77)
+    x, d0, d1 = randn(r, n), randn(r, n), randn(r, n)
+    x[::5] = 0.0
+    want = O.relu_bwd(d0 + d1, x)
+    t = [singa.from_numpy(a, dev) for a in (d0, d1, x)]
+    assert_bit_equal(singa.ReLUBackwardSum(*t).to_numpy(), want, "relu_bwd_add n=%d" % n)
+    if n > 1:
+        views = [singa.from_device_pointer(a.ptr + 4, (n - 1,), dev, keepalive=a) for a in t]
+        assert_bit_equal(singa.ReLUBackwardSum(*views).to_numpy(), want[1:], "relu_bwd_add unaligned")
+
+
 def test_relu_backward_stage1_shape_and_unaligned(singa, dev):
     r = rng(99)
     shape = (8, 64, 56, 56)

@@ -138,16 +138,26 @@ def test_resnet50_bottleneck_16bit_step(dev, kind):
         assert len(d) > 100 and worst[0][1] < tol
 
 
-def test_fused_tape_equals_reference_tape(dev):
-    """The tape with ReLU backward folded into BatchNorm backward and the residual "+=" folded into
-    the data gradient leaves bit-identical parameters and input gradient to the tape that makes
+@pytest.mark.parametrize("config,kind", [("resnet18_small", "f32"), ("resnet18_small", "f32-sum-in-relu"),
+                                         ("resnet50_small", "f16"), ("resnet50_small", "bf16")])
+def test_fused_tape_equals_reference_tape(dev, config, kind):
+    """The tape with its cross-op fusions on -- ReLU backward folded into BatchNorm backward; the
+    residual "+=" folded into the data gradient (fp32) or into the ReLU backward that reads the sum
+    (16-bit storage) -- leaves bit-identical parameters and input gradient to the tape that makes
     one call per reference op."""
-    x, labels = wl.make_inputs("resnet18_small", 2)
+    from singa_amd import singa_wrap as singa
+    x, labels = wl.make_inputs(config, 2)
     outs = []
     for fuse in (False, True):
-        hip = wl.HipOps(dev)
-        hip.fuse_bn_relu = hip.fuse_dgrad_add = fuse
-        net = wl.build("resnet18_small", hip)
+        if kind.startswith("f32"):
+            hip = wl.HipOps(dev)
+            if kind == "f32-sum-in-relu":   # the 16-bit tape's choice of fusions on the fp32 ops
+                hip.fusions = wl.HalfHipOps.fusions
+        else:
+            hip = wl.HalfHipOps(dev, singa.kFloat16 if kind == "f16" else singa.kBFloat16)
+        hip.set_fusion(fuse)
+        assert hip.fuse_bn_relu == fuse and (hip.fuse_dgrad_add or hip.fuse_add_relu) == fuse
+        net = wl.build(config, hip)
         for _ in range(2):
             net.forward(hip.from_numpy(x), hip.from_numpy(labels))
             dx = net.backward_and_update()
