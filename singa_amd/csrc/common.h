@@ -76,6 +76,8 @@ int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
                      size_t ws_bytes, bool bf16, hipStream_t s);
 int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
                      size_t ws_bytes, bool bf16, hipStream_t s);
+int sgh_conv16_fwd(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
+                   void *workspace, size_t ws_bytes, bool bf16, hipStream_t s);
 
 // Sum across the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float sgh_wave_sum(float v) {

@@ -384,6 +384,7 @@ struct D16Args {
   int KP, CP, mtiles, ptiles;
   int cls_tile0[5];  // first pixel tile of each residue class (stride^2 classes), then the total
   unsigned dy_bytes, wt_bytes;
+  const uint16_t *bias;  // per output row (channel c), or null: the forward pass run as a data gradient
 };
 
 constexpr unsigned kSelLo = 0x05040100u, kSelHi = 0x07060302u, kSelZero = 0x0c0c0c0cu;
@@ -518,7 +519,11 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int c = m0 + wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-      if (c < a.C) o[size_t(c) * HW] = round16<BF16>(acc[i][0][v]);
+      if (c < a.C) {
+        float r = acc[i][0][v];
+        if (a.bias) r += BF16 ? sgh_bf16_to_f32(a.bias[c]) : sgh_f16_to_f32(a.bias[c]);
+        o[size_t(c) * HW] = round16<BF16>(r);
+      }
     }
 }
 
@@ -528,6 +533,15 @@ __global__ __launch_bounds__(256) void k_relayout16(const uint16_t *W, uint16_t 
   if (i >= n) return;
   const int k = int(i % KP), c = int((i / KP) % CP), tap = int(i / (size_t(KP) * CP));
   wt[i] = (k < K && c < C) ? W[(size_t(k) * C + c) * RS + tap] : uint16_t(0);
+}
+
+// the forward pass as a data gradient: wt[tap][ko][c] = W[ko][c][RS - 1 - tap] (ko < KOP, c < CRP; zero beyond)
+__global__ __launch_bounds__(256) void k_relayout16_fwd(const uint16_t *W, uint16_t *wt, int K, int C, int RS, int CRP,
+                                                        int KOP) {
+  const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x, n = size_t(RS) * KOP * CRP;
+  if (i >= n) return;
+  const int c = int(i % CRP), ko = int((i / CRP) % KOP), tap = int(i / (size_t(CRP) * KOP));
+  wt[i] = (ko < K && c < C) ? W[(size_t(ko) * C + c) * RS + (RS - 1 - tap)] : uint16_t(0);
 }
 
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
@@ -644,9 +658,28 @@ int launch_d(const D16Args &a, const D16Plan &p, hipStream_t s) {
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
+// A stride-1 forward convolution is the data gradient of the convolution with the channel roles
+// swapped, the taps reversed and pad' = R - 1 - pad: y[ko][p,q] = sum_{c,r',s'} W[ko][c][R-1-r'][S-1-s']
+// * x[c][p + pad' - r'][q + pad' - s'].  False when the geometry has no such twin.
+bool fwd_twin(const sgh_conv_geom *g, sgh_conv_geom *t) {
+  if (g->stride_h != 1 || g->stride_w != 1) return false;
+  if (g->pad_h > g->R - 1 || g->pad_w > g->S - 1) return false;
+  *t = *g;
+  t->C = g->K, t->K = g->C;
+  t->H = g->P, t->W = g->Q, t->P = g->H, t->Q = g->W;
+  t->pad_h = g->R - 1 - g->pad_h, t->pad_w = g->S - 1 - g->pad_w;
+  return true;
+}
+
 }  // namespace
 
 size_t sgh_conv16_workspace_bytes(const sgh_conv_geom *g, int which) {
+  if (which == SGH_CONV_FWD) {
+    sgh_conv_geom t;
+    if (!fwd_twin(g, &t)) return 0;
+    const D16Plan p = dplan(&t);
+    return p.ok ? align256(size_t(g->R) * g->S * p.CP * p.KP * sizeof(uint16_t)) : 0;
+  }
   if (which == SGH_CONV_WGRAD) {
     const W16Plan p = wplan(g);
     return p.ok ? align256(size_t(p.splits) * g->K * g->C * g->R * g->S * sizeof(float)) : 0;
@@ -695,18 +728,27 @@ int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
-int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
-                     size_t ws_bytes, bool bf16, hipStream_t s) {
+namespace {
+
+// `fwd_of`: null for the data gradient of g; otherwise g is the twin (see fwd_twin) of the forward
+// geometry *fwd_of, W is that convolution's weight tensor and `bias` its bias (or null)
+int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t *dy, const uint16_t *W,
+            const uint16_t *bias, uint16_t *dx, void *workspace, size_t ws_bytes, bool bf16, hipStream_t s) {
   const D16Plan p = dplan(g);
   if (!p.ok) return SGH_EUNSUPPORTED;
-  if (!workspace || ws_bytes < sgh_conv16_workspace_bytes(g, SGH_CONV_DGRAD)) return SGH_EWORKSPACE;
-  uint16_t *wt = static_cast<uint16_t *>(workspace);
   const int RS = g->R * g->S;
   const size_t nw = size_t(RS) * p.CP * p.KP;
-  hipLaunchKernelGGL(k_relayout16, dim3(unsigned((nw + 255) / 256)), dim3(256), 0, s, W, wt, g->K, g->C, RS, p.KP, p.CP);
+  if (!workspace || ws_bytes < align256(nw * sizeof(uint16_t))) return SGH_EWORKSPACE;
+  uint16_t *wt = static_cast<uint16_t *>(workspace);
+  if (fwd_of)
+    hipLaunchKernelGGL(k_relayout16_fwd, dim3(unsigned((nw + 255) / 256)), dim3(256), 0, s, W, wt, fwd_of->K, fwd_of->C,
+                       RS, p.KP, p.CP);
+  else
+    hipLaunchKernelGGL(k_relayout16, dim3(unsigned((nw + 255) / 256)), dim3(256), 0, s, W, wt, g->K, g->C, RS, p.KP,
+                       p.CP);
   if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
   D16Args a{};
-  a.dy = dy, a.wt = wt, a.dx = dx;
+  a.dy = dy, a.wt = wt, a.dx = dx, a.bias = bias;
   a.N = g->N, a.C = g->C, a.H = g->H, a.W = g->W, a.K = g->K, a.P = g->P, a.Q = g->Q, a.R = g->R, a.S = g->S;
   a.stride = g->stride_h, a.pad_h = g->pad_h, a.pad_w = g->pad_w;
   a.KP = p.KP, a.CP = p.CP, a.mtiles = p.mtiles, a.ptiles = p.tiles;
@@ -714,10 +756,24 @@ int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2);
   a.wt_bytes = unsigned(nw * 2);
   const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
-  sgh_prof_start("conv_dgrad16", flops, s);
+  sgh_prof_start(fwd_of ? "conv_fwd16" : "conv_dgrad16", flops, s);
   int rc;
   if (p.bm == 128) rc = bf16 ? launch_d<128, true>(a, p, s) : launch_d<128, false>(a, p, s);
   else rc = bf16 ? launch_d<64, true>(a, p, s) : launch_d<64, false>(a, p, s);
   sgh_prof_stop(s);
   return rc;
+}
+
+}  // namespace
+
+int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
+                     size_t ws_bytes, bool bf16, hipStream_t s) {
+  return run_d16(g, nullptr, dy, W, nullptr, dx, workspace, ws_bytes, bf16, s);
+}
+
+int sgh_conv16_fwd(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
+                   void *workspace, size_t ws_bytes, bool bf16, hipStream_t s) {
+  sgh_conv_geom t;
+  if (!fwd_twin(g, &t)) return SGH_EUNSUPPORTED;
+  return run_d16(&t, g, x, W, bias, y, workspace, ws_bytes, bf16, s);
 }

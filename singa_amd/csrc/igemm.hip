@@ -1228,13 +1228,14 @@ typedef int (*cast_out_fn)(const float *, uint16_t *, size_t, void *);
 int conv_half(const sgh_conv_geom *g, int which, const uint16_t *a, const uint16_t *b, const uint16_t *bias,
               uint16_t *out, void *workspace, size_t ws_bytes, void *stream, cast_in_fn in, cast_out_fn outc) {
   if (!conv_ok(g) || !a || !b || !out) return SGH_EINVAL;
-  // the gradients run on the 16-bit matrix instructions where conv16.hip covers the geometry;
-  // everything else (and the forward pass) computes in fp32 on widened copies
-  if (which != SGH_CONV_FWD && sgh_conv16_workspace_bytes(g, which) != 0 && !getenv("SGH_CONV16_OFF")) {
+  // the gradients and the stride-1 forward pass run on the 16-bit matrix instructions where
+  // conv16.hip covers the geometry; everything else computes in fp32 on widened copies
+  if (sgh_conv16_workspace_bytes(g, which) != 0 && !getenv("SGH_CONV16_OFF")) {
     const bool bf16 = in == sgh_cast_bf16_to_f32;
-    const int rc = which == SGH_CONV_DGRAD
-                       ? sgh_conv16_dgrad(g, a, b, out, workspace, ws_bytes, bf16, sgh_stream_of(stream))
-                       : sgh_conv16_wgrad(g, a, b, out, workspace, ws_bytes, bf16, sgh_stream_of(stream));
+    hipStream_t s = sgh_stream_of(stream);
+    const int rc = which == SGH_CONV_DGRAD   ? sgh_conv16_dgrad(g, a, b, out, workspace, ws_bytes, bf16, s)
+                   : which == SGH_CONV_WGRAD ? sgh_conv16_wgrad(g, a, b, out, workspace, ws_bytes, bf16, s)
+                                             : sgh_conv16_fwd(g, a, b, bias, out, workspace, ws_bytes, bf16, s);
     if (rc != SGH_EUNSUPPORTED) return rc;
   }
   // the stem's data gradient (few input channels, large filter): the fp32 kernel reads the 16-bit

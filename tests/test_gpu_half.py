@@ -318,6 +318,14 @@ def test_conv_gradients_16bit_matrix_kernels(singa, dev, kind, case):
     print("16-bit gradients nl2: dx %.2e dw %.2e" % e)
     assert max(e) < 1e-2
     _same_bits(singa.GpuConvBackwardW(dyt, xt, wt, h).to_numpy(), dw.to_numpy(), "wgrad run-to-run")
+    # the forward pass (stride 1: the data-gradient kernel on the channel-swapped, tap-reversed twin;
+    # stride 2: fp32 kernels on widened copies), with and without bias
+    bt, b = _to(singa, dev, r.standard_normal(K).astype(np.float32), kind)
+    hb = singa.CudnnConvHandle(xt, (R, S), stride, pad, C, K, True)
+    e = (nl2(singa.GpuConvForward(xt, wt, None, h).to_numpy(), O.conv_fwd(x, w, None, stride, pad)),
+         nl2(singa.GpuConvForward(xt, wt, bt, hb).to_numpy(), O.conv_fwd(x, w, b, stride, pad)))
+    print("16-bit forward nl2: %.2e, with bias %.2e" % e)
+    assert max(e) < 1e-2
     # dx_old += dgrad on 16-bit tensors: the data gradient and a separate 16-bit add (two roundings)
     oldt, old = _to(singa, dev, r.standard_normal((N, C, H, W)).astype(np.float32), kind)
     got = singa.GpuConvBackwardxAccumulate(dyt, wt, xt, h, oldt)
@@ -363,6 +371,13 @@ def test_conv_gradients_16bit_full_size_properties(singa, dev, kind, shape):
     dx2 = singa.GpuConvBackwardx(_to(singa, dev, dy * 2, kind)[0], wt, xt, h).to_numpy()
     normal = np.abs(dx) >= 2.0 ** -13        # (binary16 subnormals have a coarser grid: 2x is not exact there)
     _same_bits(dx2[normal], dx[normal] * 2, "dgrad linearity " + kind)
+    # the forward pass at the same size: <conv(x, W), dy> closes the adjointness triangle, and the
+    # oracle on one image of the batch
+    y = singa.GpuConvForward(xt, wt, None, h).to_numpy()
+    a_y = float((y.astype(np.float64) * dy).sum())
+    scale_y = float(np.sqrt((y.astype(np.float64) ** 2).sum() * (dy.astype(np.float64) ** 2).sum()))
+    assert abs(a_y - a[0]) < 1e-3 * max(scale, scale_y)
+    assert nl2(y[5:6], O.conv_fwd(x[5:6], w, None, (st, st), (pd, pd))) < 1e-2
 
 
 def _sgd_ref(p, g, v, lr, mu, damp, wd, nesterov):
