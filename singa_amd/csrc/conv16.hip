@@ -583,7 +583,10 @@ W16Plan wplan(const sgh_conv_geom *g) {
   // take the split count whose (rounds x chunks per split) is smallest, i.e. avoid a last round
   // that is mostly empty.  Every split gets at least 4 chunks.
   const int tiles = p.mtiles * p.ntiles, slots = 2 * sgh_num_cus();
-  long best = -1;
+  // the split reduction reads splits x |dW| fp32 partials at about 5 TB/s; one chunk of a round takes
+  // about 0.9 us -> its cost in chunk units per split
+  const double reduce_chunks_per_split = double(g->K) * g->C * g->R * g->S * 4.0 / 5.0e6 / 0.9;
+  double best = -1;
   for (int r = 1; r <= 4; ++r) {
     int s = slots * r / tiles;
     if (s < 1) s = 1;
@@ -593,7 +596,8 @@ W16Plan wplan(const sgh_conv_geom *g) {
     const int cps = (p.chunks + s - 1) / s;
     // (with 8 or more splits the count stays the multiple of 8; the last splits may then be short or empty)
     const int s2 = s >= 8 ? s : (p.chunks + cps - 1) / cps;
-    const long rounds = (long(tiles) * s2 + slots - 1) / slots, cost = rounds * (cps + 2);  // (+2: prologue, epilogue)
+    const long rounds = (long(tiles) * s2 + slots - 1) / slots;
+    const double cost = double(rounds * (cps + 2)) + s2 * reduce_chunks_per_split;  // (+2: prologue, epilogue)
     if (best < 0 || cost < best) best = cost, p.cps = cps, p.splits = s2;
   }
   p.ok = true;
