@@ -275,6 +275,163 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const typename S::elem 
       });
 }
 
+// ---- backward in one pass for small channels: one workgroup per channel keeps the channel's x and
+// dy (N * HW elements each, raw storage) in LDS between the reduction and the normalisation, so the
+// tensors are read once instead of twice and the two launches become one.  Same arithmetic per
+// element as the two-pass kernels; the reduction tree differs (one workgroup instead of S splits).
+constexpr int kResNT = 1024;
+constexpr size_t kResidentLdsMax = size_t(144) << 10;
+
+template <int BYTES>
+struct RawVec;
+template <>
+struct RawVec<16> {
+  typedef sgh_v4u type;
+};
+template <>
+struct RawVec<8> {
+  typedef unsigned int type __attribute__((ext_vector_type(2)));
+};
+
+inline size_t resident_half_bytes(int N, int HW, size_t esize) { return (size_t(N) * HW * esize + 15) & ~size_t(15); }
+
+template <class S, bool RELU>
+__global__ __launch_bounds__(kResNT) void k_bn_bwd_resident(const typename S::elem *__restrict__ dy,
+                                                           const typename S::elem *__restrict__ x,
+                                                           const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                           const float *__restrict__ save_mean,
+                                                           const float *__restrict__ save_invstd,
+                                                           typename S::elem *__restrict__ dx, float *__restrict__ dgamma,
+                                                           float *__restrict__ dbeta, BnShape s) {
+  typedef typename S::elem elem;
+  constexpr int V = S::VEC, NT = kResNT;
+  typedef typename RawVec<V * sizeof(elem)>::type raw;
+  extern __shared__ __align__(16) unsigned char resident[];
+  __shared__ float red[16];
+  const int c = blockIdx.x, M = s.N * s.HW, t = threadIdx.x;
+  elem *xs = reinterpret_cast<elem *>(resident);
+  elem *ds = reinterpret_cast<elem *>(resident + ((size_t(M) * sizeof(elem) + 15) & ~size_t(15)));
+  const float mean = save_mean[c], invstd = save_invstd[c];
+  const float g = gamma[c], be = RELU ? beta[c] : 0.f;
+  auto gate = [&](float d, float v) { return !RELU || S::stored_positive(bn_out(v, mean, invstd, g, be)) ? d : 0.f; };
+  const bool vec = s.HW % V == 0;
+  const int PV = vec ? s.HW / V : s.HW, TV = s.N * PV;   // vectors (or elements) per plane / per channel
+  // stage: four (eight) independent loads per tensor in flight per thread
+  if (vec) {
+    const raw *xg = reinterpret_cast<const raw *>(x), *dg_ = reinterpret_cast<const raw *>(dy);
+    for (int base = 0; base < TV; base += 4 * NT) {
+      raw xv[4], dv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int iv = base + u * NT + t;
+        if (iv < TV) {
+          const int n = iv / PV, r = iv - n * PV;
+          const size_t off = (size_t(n) * s.C + c) * PV + r;
+          xv[u] = xg[off], dv[u] = dg_[off];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int iv = base + u * NT + t;
+        if (iv < TV) reinterpret_cast<raw *>(xs)[iv] = xv[u], reinterpret_cast<raw *>(ds)[iv] = dv[u];
+      }
+    }
+  } else {
+    for (int base = 0; base < TV; base += 8 * NT) {
+      elem xv[8], dv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = base + u * NT + t;
+        if (i < TV) {
+          const int n = i / PV, r = i - n * PV;
+          const size_t off = (size_t(n) * s.C + c) * PV + r;
+          xv[u] = x[off], dv[u] = dy[off];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = base + u * NT + t;
+        if (i < TV) xs[i] = xv[u], ds[i] = dv[u];
+      }
+    }
+  }
+  __syncthreads();
+  // sum(dy) and sum(dy * xhat), products as explicit fused multiply-adds (as in the two-pass kernels)
+  float a = 0.f, b = 0.f, b1 = 0.f;
+  if (vec) {
+    for (int iv = t; iv < TV; iv += NT) {
+      float v[V], d[V];
+      S::template load16<false>(xs + size_t(iv) * V, v);
+      S::template load16<false>(ds + size_t(iv) * V, d);
+#pragma unroll
+      for (int q = 0; q < V; q += 4) {
+        const float d0 = gate(d[q], v[q]), d1 = gate(d[q + 1], v[q + 1]), d2 = gate(d[q + 2], v[q + 2]),
+                    d3 = gate(d[q + 3], v[q + 3]);
+        a += (d0 + d1) + (d2 + d3);
+        b = __builtin_fmaf(d0, (v[q] - mean) * invstd, b);
+        b1 = __builtin_fmaf(d1, (v[q + 1] - mean) * invstd, b1);
+        b = __builtin_fmaf(d2, (v[q + 2] - mean) * invstd, b);
+        b1 = __builtin_fmaf(d3, (v[q + 3] - mean) * invstd, b1);
+      }
+    }
+  } else {
+    for (int i = t; i < TV; i += NT) {
+      const float v = S::ld(xs + i), d = gate(S::ld(ds + i), v);
+      a += d;
+      b = __builtin_fmaf(d, (v - mean) * invstd, b);
+    }
+  }
+  b += b1;
+  const float db = sgh_block_sum(a, red), dg = sgh_block_sum(b, red);
+  if (t == 0) {
+    dbeta[c] = db;
+    dgamma[c] = dg;
+  }
+  const float k = g * invstd;
+  const float rM = float(1.0 / (double(s.N) * s.HW));
+  const float c0 = db * rM, c1 = dg * rM;
+  if (vec) {
+    for (int iv = t; iv < TV; iv += NT) {
+      const int n = iv / PV, r = iv - n * PV;
+      float v[V], d[V], o[V];
+      S::template load16<false>(xs + size_t(iv) * V, v);
+      S::template load16<false>(ds + size_t(iv) * V, d);
+#pragma unroll
+      for (int q = 0; q < V; ++q) o[q] = k * (gate(d[q], v[q]) - __builtin_fmaf((v[q] - mean) * invstd, c1, c0));
+      S::store16(dx + ((size_t(n) * s.C + c) * PV + r) * V, o);
+    }
+  } else {
+    for (int i = t; i < TV; i += NT) {
+      const int n = i / PV, r = i - n * PV;
+      const float v = S::ld(xs + i);
+      S::st(dx + (size_t(n) * s.C + c) * PV + r, k * (gate(S::ld(ds + i), v) - __builtin_fmaf((v - mean) * invstd, c1, c0)));
+    }
+  }
+}
+
+// the one-pass kernel pays when a channel fits in LDS and there is a workgroup for at least half the CUs
+inline bool resident_ok(int N, int C, int HW, size_t esize) {
+  return 2 * resident_half_bytes(N, HW, esize) <= kResidentLdsMax && C >= sgh_num_cus() / 2;
+}
+
+template <class S, bool RELU>
+int launch_resident(const typename S::elem *dy, const typename S::elem *x, const float *gamma, const float *beta,
+                    const float *save_mean, const float *save_invstd, typename S::elem *dx, float *dgamma, float *dbeta,
+                    const BnShape &s, hipStream_t st) {
+  auto kern = k_bn_bwd_resident<S, RELU>;
+  static bool attr = false;
+  if (!attr) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            int(kResidentLdsMax)) != hipSuccess)
+      return SGH_EUNSUPPORTED;
+    attr = true;
+  }
+  const size_t lds = 2 * resident_half_bytes(s.N, s.HW, sizeof(typename S::elem));
+  hipLaunchKernelGGL(kern, dim3(s.C), dim3(kResNT), lds, st, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta,
+                     s);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
 inline bool shape_ok(int N, int C, int HW) {
   return N > 0 && C > 0 && HW > 0 && size_t(N) * HW < 0x7fffffffu;
 }
@@ -341,6 +498,11 @@ int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *g
   float *part = static_cast<float *>(workspace);
   const dim3 grid(C * s.S), block(kBlock);
   hipStream_t st = sgh_stream_of(stream);
+  if (resident_ok(N, C, HW, sizeof(typename S::elem))) {
+    const int rc = beta ? launch_resident<S, true>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, s, st)
+                        : launch_resident<S, false>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, s, st);
+    if (rc != SGH_EUNSUPPORTED) return rc;
+  }
   if (beta) {
     hipLaunchKernelGGL((k_bn_bwd_partial<S, true>), grid, block, 0, st, dy, x, gamma, beta, save_mean, save_invstd, part, s);
     SGH_LAUNCH_CHECK();
