@@ -379,6 +379,7 @@ __global__ __launch_bounds__(256) void k_wgrad16_reduce(const float *__restrict_
 // ------------------------------------------------------------------------------------------------
 struct D16Args {
   const uint16_t *dy, *wt;  // wt: [tap][CP][KP], zero-filled padding
+  const uint16_t *dyT;      // pixel-major copy [n][p][q][k] of dy (PIXK kernels), else null
   uint16_t *dx;
   int N, C, H, W, K, P, Q, R, S, stride, pad_h, pad_w;
   int KP, CP, mtiles, ptiles;
@@ -389,10 +390,13 @@ struct D16Args {
 
 constexpr unsigned kSelLo = 0x05040100u, kSelHi = 0x07060302u, kSelZero = 0x0c0c0c0cu;
 
-template <int BM, bool BF16>
+// PIXK: the gradient is read from a pixel-major copy dyT[n][p][q][k] (k contiguous; made by
+// k_pixel_major16 when a layer has several taps): an octet of the B tile is then one aligned 16-byte
+// load at any tap offset, staged like the weights, instead of eight dword loads and a transposition.
+template <int BM, bool BF16, bool PIXK>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_dgrad16(D16Args a) {
   extern __shared__ __align__(16) uint16_t lds16[];
-  constexpr int TM = BM / 64, ASLOTS = BM * 8 / NT;
+  constexpr int TM = BM / 64, ASLOTS = BM * 8 / NT, BSLOTS = BN * 8 / NT;
   uint16_t *const As0 = lds16, *const Bs0 = lds16 + BM * PITCH;
   uint16_t *const As1 = lds16 + (BM + BN) * PITCH, *const Bs1 = As1 + BM * PITCH;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -411,14 +415,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   const int Hc = (a.H - ca + st - 1) / st, Wreal = (a.W - cb + st - 1) / st, Wc = (Wreal + 1) & ~1, HWc = Hc * Wc;
   const long cnt = long(a.N) * HWc;
   const long pix0 = long(pt - a.cls_tile0[cls]) * BN;
-  const rsrc_t rdy = make_rsrc(a.dy, a.dy_bytes);
+  const rsrc_t rdy = make_rsrc(PIXK ? a.dyT : a.dy, a.dy_bytes);
 
-  // B loader: pixel pair pp of the tile, k octet kq of the chunk (one per wavefront)
-  const int pp = lane, kq = wave;
-  const long pixA = pix0 + 2 * pp, pixB = pixA + 1;
-  const int nA = int(pixA / HWc), remA = int(pixA - long(nA) * HWc), iA = remA / Wc, jA = remA - iA * Wc;
-  int voff = kOOB;  // byte offset of the dword holding both pixels (kOOB: neither exists)
-  unsigned selA = kSelZero, selB = kSelZero;
   // The taps of this class are r = r0 + st * ti, s = s0 + st * tj (ti < nr, tj < ns): those with
   // (ca + pad_h - r) and (cb + pad_w - s) divisible by the stride; the gradient pixel of tap
   // (ti, tj) is (i + dr0 - ti, j + ds0 - tj).  (st is 1 or 2: shifts, no divisions.)
@@ -426,23 +424,53 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   const int r0 = (ca + a.pad_h) & sh, s0 = (cb + a.pad_w) & sh;
   const int nr = r0 < a.R ? (a.R - r0 + sh) >> sh : 0, ns = s0 < a.S ? (a.S - s0 + sh) >> sh : 0;
   const int dr0 = (ca + a.pad_h - r0) >> sh, ds0 = (cb + a.pad_w - s0) >> sh;
+
+  const int oct = t & 7, rb = t >> 3;   // staging roles: octet of the chunk, tile row (0..63)
+  // B loader, dword pairs: pixel pair pp of the tile, k octet kq of the chunk (one per wavefront)
+  const int pp = lane, kq = wave;
+  const long pixA = pix0 + 2 * pp, pixB = pixA + 1;
+  const int nA = int(pixA / HWc), remA = int(pixA - long(nA) * HWc), iA = remA / Wc, jA = remA - iA * Wc;
+  int voff = kOOB;  // byte offset of the dword holding both pixels (kOOB: neither exists)
+  unsigned selA = kSelZero, selB = kSelZero;
   const bool pixA_ok = pixA < cnt, pixB_ok = pixB < cnt && jA + 1 < Wreal;
+  // B loader, pixel-major copy: pixels rb and rb + 64 of the tile, octet `oct`
+  int bn_[BSLOTS], bi_[BSLOTS], bj_[BSLOTS], bvoff[BSLOTS];
+  if constexpr (PIXK) {
+#pragma unroll
+    for (int i = 0; i < BSLOTS; ++i) {
+      const long pix = pix0 + rb + 64 * i;
+      const bool live = pix < cnt;
+      const int n = live ? int(pix / HWc) : 0, rem = live ? int(pix - long(n) * HWc) : 0;
+      bn_[i] = n, bi_[i] = rem / Wc, bj_[i] = rem - bi_[i] * Wc;
+      if (!live || bj_[i] >= Wreal) bi_[i] = -0x10000;   // no tap of a dummy pixel lands inside the image
+      bvoff[i] = kOOB;
+    }
+  }
   auto set_tap = [&](int ti, int tj) {
-    const int p = iA + dr0 - ti, q0 = jA + ds0 - tj;
-    const bool row = unsigned(p) < unsigned(a.P);
-    const bool memA = row && unsigned(q0) < unsigned(a.Q), memB = row && unsigned(q0 + 1) < unsigned(a.Q);
-    const int base = ((nA * a.K) * a.P + p) * a.Q + q0;
-    // both pixels exist: their dword; only A: the dword before (A in the high half); only B: the
-    // dword after (B in the low half) -- the load never leaves the row
-    voff = memA ? (memB ? base * 2 : (base - 1) * 2) : (memB ? (base + 1) * 2 : kOOB);
-    selA = memA && pixA_ok ? (memB ? kSelLo : kSelHi) : kSelZero;
-    selB = memB && pixB_ok ? (memA ? kSelHi : kSelLo) : kSelZero;
+    if constexpr (PIXK) {
+#pragma unroll
+      for (int i = 0; i < BSLOTS; ++i) {
+        const int p = bi_[i] + dr0 - ti, q = bj_[i] + ds0 - tj;
+        const bool in = unsigned(p) < unsigned(a.P) && unsigned(q) < unsigned(a.Q);
+        bvoff[i] = in ? (((bn_[i] * a.P + p) * a.Q + q) * a.K + oct * 8) * 2 : kOOB;
+      }
+    } else {
+      const int p = iA + dr0 - ti, q0 = jA + ds0 - tj;
+      const bool row = unsigned(p) < unsigned(a.P);
+      const bool memA = row && unsigned(q0) < unsigned(a.Q), memB = row && unsigned(q0 + 1) < unsigned(a.Q);
+      const int base = ((nA * a.K) * a.P + p) * a.Q + q0;
+      // both pixels exist: their dword; only A: the dword before (A in the high half); only B: the
+      // dword after (B in the low half) -- the load never leaves the row
+      voff = memA ? (memB ? base * 2 : (base - 1) * 2) : (memB ? (base + 1) * 2 : kOOB);
+      selA = memA && pixA_ok ? (memB ? kSelLo : kSelHi) : kSelZero;
+      selB = memB && pixB_ok ? (memA ? kSelHi : kSelLo) : kSelZero;
+    }
   };
   const int nkc = a.KP / KC;
 
-  const int oct = t & 7, rb = t >> 3;
   u32x4 ra[ASLOTS];
-  unsigned rd[8];      // the pair's dword for 8 consecutive k
+  u32x4 rbv[BSLOTS];   // pixel-major copy: the octets of this thread's pixels
+  unsigned rd[8];      // dword pairs: the pair's dword for 8 consecutive k
   const rsrc_t rwt = make_rsrc(a.wt, a.wt_bytes);
   const int woff = ((m0 + rb) * a.KP + oct * 8) * 2;   // rb = t / 8 in 0..63
   auto load = [&](int tap, int kc) {
@@ -450,26 +478,38 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
     for (int i = 0; i < ASLOTS; ++i)
       ra[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rwt, woff + 64 * i * a.KP * 2, wso, 0));
-    const int kb = kc * KC + kq * 8;
-    if (kb < a.K) {
+    if constexpr (PIXK) {
+      const bool kin = kc * KC + oct * 8 < a.K;   // (K is a multiple of 8: an octet is inside or outside)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) rd[j] = unsigned(__builtin_amdgcn_raw_buffer_load_b32(rdy, voff, (kb + j) * PQ * 2, 0));
+      for (int i = 0; i < BSLOTS; ++i)
+        rbv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rdy, kin ? bvoff[i] : kOOB, kc * KC * 2, 0));
     } else {
+      const int kb = kc * KC + kq * 8;
+      if (kb < a.K) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) rd[j] = 0u;
+        for (int j = 0; j < 8; ++j) rd[j] = unsigned(__builtin_amdgcn_raw_buffer_load_b32(rdy, voff, (kb + j) * PQ * 2, 0));
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) rd[j] = 0u;
+      }
     }
   };
   auto stage = [&](uint16_t *As, uint16_t *Bs) {
 #pragma unroll
     for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 64 * i) * PITCH + oct * 8) = ra[i];
-    u32x4 vA, vB;
+    if constexpr (PIXK) {
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      vA[d] = __builtin_amdgcn_perm(rd[2 * d + 1], rd[2 * d], selA);
-      vB[d] = __builtin_amdgcn_perm(rd[2 * d + 1], rd[2 * d], selB);
+      for (int i = 0; i < BSLOTS; ++i) *reinterpret_cast<u32x4 *>(Bs + (rb + 64 * i) * PITCH + oct * 8) = rbv[i];
+    } else {
+      u32x4 vA, vB;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        vA[d] = __builtin_amdgcn_perm(rd[2 * d + 1], rd[2 * d], selA);
+        vB[d] = __builtin_amdgcn_perm(rd[2 * d + 1], rd[2 * d], selB);
+      }
+      *reinterpret_cast<u32x4 *>(Bs + (2 * pp) * PITCH + kq * 8) = vA;
+      *reinterpret_cast<u32x4 *>(Bs + (2 * pp + 1) * PITCH + kq * 8) = vB;
     }
-    *reinterpret_cast<u32x4 *>(Bs + (2 * pp) * PITCH + kq * 8) = vA;
-    *reinterpret_cast<u32x4 *>(Bs + (2 * pp + 1) * PITCH + kq * 8) = vB;
   };
 
   f32x16 acc[TM][2];
@@ -525,6 +565,43 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         o[size_t(c) * HW] = round16<BF16>(r);
       }
     }
+}
+
+// dst[n][pq][k] = src[n][k][pq]: the pixel-major copy of a gradient tensor that the multi-tap data
+// gradient reads (64 x 64 tiles through LDS; K is even).  PAIR: PQ is even, the source is read as dwords.
+template <bool PAIR>
+__global__ __launch_bounds__(256) void k_pixel_major16(const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, int K,
+                                                      int PQ) {
+  __shared__ __align__(4) uint16_t tile[64][66];   // [k][pq]
+  const int t = threadIdx.x, n = blockIdx.z, k0 = blockIdx.y * 64, q0 = blockIdx.x * 64;
+  const uint16_t *s = src + size_t(n) * K * PQ;
+  if constexpr (PAIR) {
+    const int c2 = t & 31;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int kr = (t >> 5) + 8 * i, k = k0 + kr, pq = q0 + 2 * c2;
+      unsigned v = 0u;
+      if (k < K && pq < PQ) v = *reinterpret_cast<const unsigned *>(s + size_t(k) * PQ + pq);
+      *reinterpret_cast<unsigned *>(&tile[kr][2 * c2]) = v;
+    }
+  } else {
+    const int c = t & 63;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int kr = (t >> 6) + 4 * i, k = k0 + kr, pq = q0 + c;
+      tile[kr][c] = (k < K && pq < PQ) ? s[size_t(k) * PQ + pq] : uint16_t(0);
+    }
+  }
+  __syncthreads();
+  const int kd = 2 * (t & 31);
+  if (k0 + kd >= K) return;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int pr = (t >> 5) + 8 * i, pq = q0 + pr;
+    if (pq < PQ)
+      *reinterpret_cast<unsigned *>(dst + (size_t(n) * PQ + pq) * K + k0 + kd) =
+          unsigned(tile[kd][pr]) | (unsigned(tile[kd + 1][pr]) << 16);
+  }
 }
 
 // wt[tap][c][k] (c < CP, k < KP; zero beyond C / K) from W[k][c][r][s]
@@ -606,8 +683,10 @@ W16Plan wplan(const sgh_conv_geom *g) {
 
 struct D16Plan {
   bool ok;
+  bool pixk;   // several taps: the kernel reads a pixel-major copy of the gradient (k_pixel_major16)
   int bm, mtiles, KP, CP, tiles;
   int cls_tile0[5];
+  size_t wt_bytes, dyT_bytes;   // workspace: re-laid weights, then the pixel-major copy
 };
 
 D16Plan dplan(const sgh_conv_geom *g) {
@@ -632,6 +711,12 @@ D16Plan dplan(const sgh_conv_geom *g) {
   p.KP = (g->K + KC - 1) / KC * KC;
   if (tiles * p.mtiles >= (long(1) << 30) || size_t(g->R) * g->S * p.CP * p.KP >= lim) return p;
   p.tiles = int(tiles);
+  // The copy pays where the dword-pair loads are at their worst: odd class widths (7 x 7 planes,
+  // stride 2 on 14 x 14), where every pair row carries a dummy pixel.  (Elsewhere the kernel gains
+  // 10-20 % from the aligned loads and the copy costs as much: measured at 56 x 56 .. 14 x 14.)
+  p.pixk = g->R * g->S > 1 && ((g->W + st - 1) / st) % 2 == 1;
+  p.wt_bytes = align256(size_t(g->R) * g->S * p.CP * p.KP * sizeof(uint16_t));
+  p.dyT_bytes = p.pixk ? align256(size_t(g->N) * g->K * g->P * g->Q * sizeof(uint16_t)) : 0;
   p.ok = true;
   return p;
 }
@@ -649,9 +734,9 @@ int launch_w(const W16Args &a, const W16Plan &p, hipStream_t s) {
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
-template <int BM, bool BF16>
+template <int BM, bool BF16, bool PIXK>
 int launch_d(const D16Args &a, const D16Plan &p, hipStream_t s) {
-  auto kern = k_dgrad16<BM, BF16>;
+  auto kern = k_dgrad16<BM, BF16, PIXK>;
   const size_t lds = BM == 128 ? kLds128 : kLds64;
   static bool attr = false;
   if (!attr) {
@@ -682,7 +767,7 @@ size_t sgh_conv16_workspace_bytes(const sgh_conv_geom *g, int which) {
     sgh_conv_geom t;
     if (!fwd_twin(g, &t)) return 0;
     const D16Plan p = dplan(&t);
-    return p.ok ? align256(size_t(g->R) * g->S * p.CP * p.KP * sizeof(uint16_t)) : 0;
+    return p.ok ? p.wt_bytes + p.dyT_bytes : 0;
   }
   if (which == SGH_CONV_WGRAD) {
     const W16Plan p = wplan(g);
@@ -690,7 +775,7 @@ size_t sgh_conv16_workspace_bytes(const sgh_conv_geom *g, int which) {
   }
   if (which == SGH_CONV_DGRAD) {
     const D16Plan p = dplan(g);
-    return p.ok ? align256(size_t(g->R) * g->S * p.CP * p.KP * sizeof(uint16_t)) : 0;
+    return p.ok ? p.wt_bytes + p.dyT_bytes : 0;
   }
   return 0;
 }
@@ -742,8 +827,16 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
   if (!p.ok) return SGH_EUNSUPPORTED;
   const int RS = g->R * g->S;
   const size_t nw = size_t(RS) * p.CP * p.KP;
-  if (!workspace || ws_bytes < align256(nw * sizeof(uint16_t))) return SGH_EWORKSPACE;
+  if (!workspace || ws_bytes < p.wt_bytes + p.dyT_bytes) return SGH_EWORKSPACE;
   uint16_t *wt = static_cast<uint16_t *>(workspace);
+  uint16_t *dyT = p.pixk ? reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + p.wt_bytes) : nullptr;
+  if (p.pixk) {
+    const int PQ = g->P * g->Q;
+    const dim3 grid(unsigned((PQ + 63) / 64), unsigned((g->K + 63) / 64), unsigned(g->N));
+    if (PQ % 2 == 0) hipLaunchKernelGGL(k_pixel_major16<true>, grid, dim3(256), 0, s, dy, dyT, g->K, PQ);
+    else hipLaunchKernelGGL(k_pixel_major16<false>, grid, dim3(256), 0, s, dy, dyT, g->K, PQ);
+    if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
+  }
   if (fwd_of)
     hipLaunchKernelGGL(k_relayout16_fwd, dim3(unsigned((nw + 255) / 256)), dim3(256), 0, s, W, wt, fwd_of->K, fwd_of->C,
                        RS, p.KP, p.CP);
@@ -752,7 +845,7 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
                        p.CP);
   if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
   D16Args a{};
-  a.dy = dy, a.wt = wt, a.dx = dx, a.bias = bias;
+  a.dy = dy, a.dyT = dyT, a.wt = wt, a.dx = dx, a.bias = bias;
   a.N = g->N, a.C = g->C, a.H = g->H, a.W = g->W, a.K = g->K, a.P = g->P, a.Q = g->Q, a.R = g->R, a.S = g->S;
   a.stride = g->stride_h, a.pad_h = g->pad_h, a.pad_w = g->pad_w;
   a.KP = p.KP, a.CP = p.CP, a.mtiles = p.mtiles, a.ptiles = p.tiles;
@@ -762,8 +855,13 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
   const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
   sgh_prof_start(fwd_of ? "conv_fwd16" : "conv_dgrad16", flops, s);
   int rc;
-  if (p.bm == 128) rc = bf16 ? launch_d<128, true>(a, p, s) : launch_d<128, false>(a, p, s);
-  else rc = bf16 ? launch_d<64, true>(a, p, s) : launch_d<64, false>(a, p, s);
+  if (p.pixk) {
+    if (p.bm == 128) rc = bf16 ? launch_d<128, true, true>(a, p, s) : launch_d<128, false, true>(a, p, s);
+    else rc = bf16 ? launch_d<64, true, true>(a, p, s) : launch_d<64, false, true>(a, p, s);
+  } else {
+    if (p.bm == 128) rc = bf16 ? launch_d<128, true, false>(a, p, s) : launch_d<128, false, false>(a, p, s);
+    else rc = bf16 ? launch_d<64, true, false>(a, p, s) : launch_d<64, false, false>(a, p, s);
+  }
   sgh_prof_stop(s);
   return rc;
 }
