@@ -16,7 +16,7 @@ def singa():
     return singa_wrap
 
 
-SIZES = [1, 7, 8, 9, 1000, 4096 + 3, 64 * 1024 + 5, 3 * 1000 * 1000 + 1]
+SIZES = [0, 1, 7, 8, 9, 1000, 4096 + 3, 64 * 1024 + 5, 3 * 1000 * 1000 + 1]
 
 
 def _special(r, n):
