@@ -530,6 +530,10 @@ size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
   return size_t(C) * smax * 2 * sizeof(float);
 }
 
+// 16-bit planes that are a multiple of 4 but not of 8 elements (14 x 14) use the 8-byte vector class
+#define SGH_BN_DISPATCH16(fn, F16X8, F16X4, ...) \
+  (HW % 8 != 0 && HW % 4 == 0 ? fn<F16X4>(__VA_ARGS__) : fn<F16X8>(__VA_ARGS__))
+
 int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float *beta, float *running_mean,
                          float *running_var, float factor, float eps, float *y, float *save_mean, float *save_invstd,
                          int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
@@ -539,18 +543,14 @@ int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float *beta, 
 int sgh_bn_fwd_train_f16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
                          float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
                          float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
-  if (HW % 8 != 0 && HW % 4 == 0) return bn_fwd_train<StF16x4>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C, HW,
-                             workspace, ws_bytes, stream);  // 8-byte vectors (e.g. 14 x 14 planes)
-  return bn_fwd_train<StF16>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C, HW,
-                             workspace, ws_bytes, stream);
+  return SGH_BN_DISPATCH16(bn_fwd_train, StF16, StF16x4, x, gamma, beta, running_mean, running_var, factor, eps, y,
+                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream);
 }
 int sgh_bn_fwd_train_bf16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
                           float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
                           float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
-  if (HW % 8 != 0 && HW % 4 == 0) return bn_fwd_train<StBF16x4>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C,
-                              HW, workspace, ws_bytes, stream);  // 8-byte vectors (e.g. 14 x 14 planes)
-  return bn_fwd_train<StBF16>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C,
-                              HW, workspace, ws_bytes, stream);
+  return SGH_BN_DISPATCH16(bn_fwd_train, StBF16, StBF16x4, x, gamma, beta, running_mean, running_var, factor, eps, y,
+                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream);
 }
 
 int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const float *save_mean,
@@ -562,18 +562,14 @@ int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const fl
 int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                    const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                    void *workspace, size_t ws_bytes, void *stream) {
-  if (HW % 8 != 0 && HW % 4 == 0) return bn_bwd<StF16x4>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
-                       stream);  // 8-byte vectors (e.g. 14 x 14 planes)
-  return bn_bwd<StF16>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
-                       stream);
+  return SGH_BN_DISPATCH16(bn_bwd, StF16, StF16x4, dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N,
+                           C, HW, workspace, ws_bytes, stream);
 }
 int sgh_bn_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                     const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                     void *workspace, size_t ws_bytes, void *stream) {
-  if (HW % 8 != 0 && HW % 4 == 0) return bn_bwd<StBF16x4>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
-                        stream);  // 8-byte vectors (e.g. 14 x 14 planes)
-  return bn_bwd<StBF16>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
-                        stream);
+  return SGH_BN_DISPATCH16(bn_bwd, StBF16, StBF16x4, dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N,
+                           C, HW, workspace, ws_bytes, stream);
 }
 
 int sgh_bn_fwd_infer_f32(const float *x, const float *gamma, const float *beta, const float *running_mean,
@@ -582,13 +578,13 @@ int sgh_bn_fwd_infer_f32(const float *x, const float *gamma, const float *beta, 
 }
 int sgh_bn_fwd_infer_f16(const uint16_t *x, const float *gamma, const float *beta, const float *running_mean,
                          const float *running_var, float eps, uint16_t *y, int N, int C, int HW, void *stream) {
-  if (HW % 8 != 0 && HW % 4 == 0) return bn_fwd_infer<StF16x4>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);  // 8-byte vectors (e.g. 14 x 14 planes)
-  return bn_fwd_infer<StF16>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);
+  return SGH_BN_DISPATCH16(bn_fwd_infer, StF16, StF16x4, x, gamma, beta, running_mean, running_var, eps, y, N, C, HW,
+                           stream);
 }
 int sgh_bn_fwd_infer_bf16(const uint16_t *x, const float *gamma, const float *beta, const float *running_mean,
                           const float *running_var, float eps, uint16_t *y, int N, int C, int HW, void *stream) {
-  if (HW % 8 != 0 && HW % 4 == 0) return bn_fwd_infer<StBF16x4>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);  // 8-byte vectors (e.g. 14 x 14 planes)
-  return bn_fwd_infer<StBF16>(x, gamma, beta, running_mean, running_var, eps, y, N, C, HW, stream);
+  return SGH_BN_DISPATCH16(bn_fwd_infer, StBF16, StBF16x4, x, gamma, beta, running_mean, running_var, eps, y, N, C, HW,
+                           stream);
 }
 
 int sgh_bn_relu_bwd_f32(const float *dy, const float *x, const float *gamma, const float *beta, const float *save_mean,
@@ -602,19 +598,16 @@ int sgh_bn_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamm
                         const float *save_mean, const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta,
                         int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   if (!beta) return SGH_EINVAL;
-  if (HW % 8 != 0 && HW % 4 == 0) return bn_bwd<StF16x4>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
-                       stream);  // 8-byte vectors (e.g. 14 x 14 planes)
-  return bn_bwd<StF16>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
-                       stream);
+  return SGH_BN_DISPATCH16(bn_bwd, StF16, StF16x4, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C,
+                           HW, workspace, ws_bytes, stream);
 }
 int sgh_bn_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *beta,
                          const float *save_mean, const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta,
                          int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   if (!beta) return SGH_EINVAL;
-  if (HW % 8 != 0 && HW % 4 == 0) return bn_bwd<StBF16x4>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
-                        stream);  // 8-byte vectors (e.g. 14 x 14 planes)
-  return bn_bwd<StBF16>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
-                        stream);
+  return SGH_BN_DISPATCH16(bn_bwd, StBF16, StBF16x4, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C,
+                           HW, workspace, ws_bytes, stream);
 }
+#undef SGH_BN_DISPATCH16
 
 }  // extern "C"
