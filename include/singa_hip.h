@@ -288,6 +288,8 @@ typedef struct sgh_conv_geom {
   int K, R, S;          /* weight [K, C, R, S]                    */
   int stride_h, stride_w, pad_h, pad_w;
   int P, Q;             /* output [N, K, P, Q]                    */
+  int weights_prelaid;  /* set by sgh_conv_dgrad_prepare_multi, cleared by the caller: the workspace
+                           already holds this layer's re-laid weights for the data gradient */
 } sgh_conv_geom;
 SGH_API int sgh_conv_geom_init(sgh_conv_geom *g, int N, int C, int H, int W, int K, int R, int S,
                                int stride_h, int stride_w, int pad_h, int pad_w);
@@ -312,6 +314,24 @@ SGH_API int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const fl
  * K a multiple of 16); SGH_EUNSUPPORTED otherwise, with dx untouched. */
 SGH_API int sgh_conv_dgrad_acc_f32(const sgh_conv_geom *g, const float *dy, const float *W,
                                    float *dx, void *workspace, size_t ws_bytes, void *stream);
+/* The data gradient re-lays the weight tensor in its workspace before the matrix kernel runs:
+ * a launch of a few microseconds per layer.  A caller that runs many data gradients while the
+ * weights do not change (a backward pass) can have all of them re-laid by ONE launch up front:
+ * sgh_conv_dgrad_prepare_multi writes each listed layer's workspace and sets g->weights_prelaid on
+ * the layers whose kernel takes such weights (fp32: dtype 0, binary16: 1, bfloat16: 2); the data
+ * gradient entry points (sgh_conv_dgrad_*, sgh_conv_dgrad_acc_f32) then skip their own re-layout.
+ * Between the prepare call and a layer's data gradient its workspace must not be used by another
+ * pass; the caller clears weights_prelaid once the weights change (after the update).  Results
+ * are bit-identical with and without.  No counterpart in the reference (cuDNN keeps its filter
+ * transforms to itself). */
+typedef struct sgh_conv_prepare_item {
+  sgh_conv_geom *g;
+  const void *W;
+  void *workspace;
+  size_t ws_bytes;
+} sgh_conv_prepare_item;
+SGH_API int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, int dtype,
+                                         void *stream);
 /* GpuConvBackwardW (src/model/operation/convolution.cc:658-681; native algorithm
  * src/model/layer/convolution.cc:166-177 + Im2col :197-222):
  * dW[k,c,r,s] = sum_{n,p,q} dy[n,k,p,q] * x[n,c,p*stride-pad+r,q*stride-pad+s].

@@ -18,7 +18,13 @@ sz = C.c_size_t
 class ConvGeom(C.Structure):
     """``sgh_conv_geom``"""
     _fields_ = [(n, C.c_int) for n in
-                ("N", "C", "H", "W", "K", "R", "S", "stride_h", "stride_w", "pad_h", "pad_w", "P", "Q")]
+                ("N", "C", "H", "W", "K", "R", "S", "stride_h", "stride_w", "pad_h", "pad_w", "P", "Q",
+                 "weights_prelaid")]
+
+
+class ConvPrepareItem(C.Structure):
+    """``sgh_conv_prepare_item``"""
+    _fields_ = [("g", C.POINTER(ConvGeom)), ("W", vp), ("workspace", vp), ("ws_bytes", C.c_size_t)]
 
 
 class PoolGeom(C.Structure):
@@ -122,6 +128,7 @@ SIGNATURES = {
     "sgh_conv_bgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp]),
     "sgh_conv_fwd_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
     "sgh_conv_workspace_bytes_h": (sz, [C.POINTER(ConvGeom), C.c_int]),
+    "sgh_conv_dgrad_prepare_multi": (C.c_int, [C.POINTER(ConvPrepareItem), C.c_int, C.c_int, vp]),
     "sgh_conv_dgrad_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_dgrad_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_wgrad_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),

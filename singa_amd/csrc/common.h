@@ -76,6 +76,10 @@ int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
                      size_t ws_bytes, bool bf16, hipStream_t s);
 int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
                      size_t ws_bytes, bool bf16, hipStream_t s);
+// Data-gradient weight re-layout of conv16.hip as a batch item: false when the geometry is not covered;
+// otherwise the destination layout [tap][CP][KP] (sgh_conv16_dgrad skips its re-layout when
+// g->weights_prelaid is set).
+bool sgh_conv16_dgrad_relayout_dims(const sgh_conv_geom *g, int *CP, int *KP);
 int sgh_conv16_fwd(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
                    void *workspace, size_t ws_bytes, bool bf16, hipStream_t s);
 

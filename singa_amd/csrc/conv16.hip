@@ -837,7 +837,9 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
     else hipLaunchKernelGGL(k_pixel_major16<false>, grid, dim3(256), 0, s, dy, dyT, g->K, PQ);
     if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
   }
-  if (fwd_of)
+  if (!fwd_of && g->weights_prelaid) {
+    // re-laid by sgh_conv_dgrad_prepare_multi
+  } else if (fwd_of)
     hipLaunchKernelGGL(k_relayout16_fwd, dim3(unsigned((nw + 255) / 256)), dim3(256), 0, s, W, wt, fwd_of->K, fwd_of->C,
                        RS, p.KP, p.CP);
   else
@@ -867,6 +869,13 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
 }
 
 }  // namespace
+
+bool sgh_conv16_dgrad_relayout_dims(const sgh_conv_geom *g, int *CP, int *KP) {
+  const D16Plan p = dplan(g);
+  if (!p.ok) return false;
+  *CP = p.CP, *KP = p.KP;
+  return true;
+}
 
 int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
                      size_t ws_bytes, bool bf16, hipStream_t s) {

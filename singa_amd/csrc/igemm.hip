@@ -874,6 +874,7 @@ int sgh_conv_geom_init(sgh_conv_geom *g, int N, int C, int H, int W, int K, int 
   // ConvHandle's integer division (reference: src/model/operation/convolution.cc:56-59)
   g->P = (H + 2 * pad_h - R) / stride_h + 1;
   g->Q = (W + 2 * pad_w - S) / stride_w + 1;
+  g->weights_prelaid = 0;
   return conv_ok(g) ? SGH_OK : SGH_EINVAL;
 }
 
@@ -965,7 +966,8 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     const long total = long(RS) * KP * g->C;
     long blocks = (total + NT - 1) / NT;
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
+    if (!g->weights_prelaid)
+      hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
     float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) +
                                                 align256(size_t(RS) * KP * g->C * sizeof(float)) +
                                                 align256(sizeof(DgClsTable)));
@@ -1035,7 +1037,8 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     const long total = long(RS) * KP * g->C;
     long blocks = (total + NT - 1) / NT;
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
+    if (!g->weights_prelaid)
+      hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
     const int M = g->C, Ncols = g->N * g->H * g->W, Ktot = RS * KP;
     NchwStore st{dx, nullptr, g->C, g->H * g->W, Ncols};
     auto la = dense_loader<128, false>(Wt, 1, g->C, M, Ktot);
@@ -1052,6 +1055,139 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
 int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
                        size_t ws_bytes, void *stream) {
   return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, false);
+}
+
+// ---- all data-gradient weight re-layouts of a backward pass in one launch ----------------------
+namespace {
+
+constexpr int kMaxRelayouts = 56;   // per launch: the table travels as a kernel argument
+
+struct RelayoutTable {
+  int count;
+  int block0[kMaxRelayouts + 1];   // first workgroup of each item, then the total
+  struct Item {
+    const void *W;
+    void *Wt;
+    int K, C, RS, A, B;   // destination [tap][A][B]: fp32 A = KP (k), B = C;  16-bit A = CP (c), B = KP (k)
+  } it[kMaxRelayouts];
+};
+
+constexpr int kRelayoutPerBlock = NT * 8, kRelayoutTile = 32, kRelayoutMaxTaps = 9;
+
+// One 32 (k) x 32 (c) x RS tile of a re-layout through LDS: the source rows W[k][c0 .. c0+31][taps] are
+// contiguous runs, the destination rows [tap][.][32 contiguous] are too.
+extern "C++" {
+template <class T>
+__device__ __forceinline__ void relayout_tile(const T *__restrict__ W, T *__restrict__ Wt, int K, int C, int RS, int A,
+                                              int B, bool k_fastest, int tile) {
+  __shared__ T lds[kRelayoutTile][kRelayoutTile * kRelayoutMaxTaps + 1];
+  // destination [tap][A][B]; k_fastest: (A, B) = (c, k), else (k, c)
+  const int kdim = k_fastest ? B : A, cdim = k_fastest ? A : B;
+  const int ctiles = (cdim + kRelayoutTile - 1) / kRelayoutTile;
+  const int k0 = (tile / ctiles) * kRelayoutTile, c0 = (tile % ctiles) * kRelayoutTile;
+  const int run = kRelayoutTile * RS, t = threadIdx.x;
+  const int cvalid = C - c0 < kRelayoutTile ? C - c0 : kRelayoutTile, rlen = cvalid > 0 ? cvalid * RS : 0;
+  for (int kk = t >> 6; kk < kRelayoutTile; kk += NT / 64) {   // a wavefront per source row
+    const int k = k0 + kk;
+    const T *src = W + (long(k) * C + c0) * RS;
+    for (int r = t & 63; r < run; r += 64) lds[kk][r] = (k < K && r < rlen) ? src[r] : T(0);
+  }
+  __syncthreads();
+  const int f = t & 31;   // position along the destination's contiguous dimension
+  for (int o = t >> 5; o < kRelayoutTile * RS; o += NT / 32) {
+    const int tap = o / kRelayoutTile, s_ = o - tap * kRelayoutTile;   // s_: position along the other tile dimension
+    const int kk = k_fastest ? f : s_, cc = k_fastest ? s_ : f;
+    const int k = k0 + kk, c = c0 + cc;
+    if (k < kdim && c < cdim) {
+      const long dst = k_fastest ? (long(tap) * A + c) * B + k : (long(tap) * A + k) * B + c;
+      Wt[dst] = lds[kk][cc * RS + tap];
+    }
+  }
+}
+}  // extern "C++"
+
+extern "C++" {
+// T = float: destination [tap][KP][C]; T = uint16_t: destination [tap][CP][KP] (see RelayoutTable)
+template <class T>
+__global__ __launch_bounds__(NT) void k_weight_relayout_multi(const RelayoutTable t) {
+  constexpr bool k_fastest = sizeof(T) == 2;
+  int lo = 0, hi = t.count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (int(blockIdx.x) >= t.block0[mid]) lo = mid;
+    else hi = mid - 1;
+  }
+  const int K = t.it[lo].K, C = t.it[lo].C, RS = t.it[lo].RS, A = t.it[lo].A, B = t.it[lo].B;
+  const int blk = int(blockIdx.x) - t.block0[lo];
+  const T *W = static_cast<const T *>(t.it[lo].W);
+  T *Wt = static_cast<T *>(t.it[lo].Wt);
+  if (RS <= kRelayoutMaxTaps) {
+    relayout_tile<T>(W, Wt, K, C, RS, A, B, k_fastest, blk);
+    return;
+  }
+  // large filters: element by element
+  const long total = long(RS) * A * B;
+  const long base = long(blk) * kRelayoutPerBlock + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const long i = base + u * NT;
+    if (i < total) {
+      const int f = int(i % B), s_ = int((i / B) % A), tap = int(i / (long(A) * B));
+      const int k = k_fastest ? f : s_, c = k_fastest ? s_ : f;
+      Wt[i] = (k < K && c < C) ? W[(long(k) * C + c) * RS + tap] : T(0);
+    }
+  }
+}
+}  // extern "C++"
+
+}  // namespace
+
+int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, int dtype, void *stream) {
+  if (count < 0 || (count > 0 && !items) || dtype < 0 || dtype > 2) return SGH_EINVAL;
+  hipStream_t s = sgh_stream_of(stream);
+  RelayoutTable t;
+  t.count = 0, t.block0[0] = 0;
+  sgh_conv_geom *batch[kMaxRelayouts];
+  auto flush = [&]() -> int {
+    if (t.count == 0) return SGH_OK;
+    if (dtype == 0) hipLaunchKernelGGL(k_weight_relayout_multi<float>, dim3(unsigned(t.block0[t.count])), dim3(NT), 0, s, t);
+    else hipLaunchKernelGGL(k_weight_relayout_multi<uint16_t>, dim3(unsigned(t.block0[t.count])), dim3(NT), 0, s, t);
+    if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
+    for (int i = 0; i < t.count; ++i) batch[i]->weights_prelaid = 1;
+    t.count = 0;
+    return SGH_OK;
+  };
+  for (int i = 0; i < count; ++i) {
+    sgh_conv_geom *g = items[i].g;
+    if (!g || !conv_ok(g) || !items[i].W) return SGH_EINVAL;
+    g->weights_prelaid = 0;
+    RelayoutTable::Item it{};
+    it.W = items[i].W, it.Wt = items[i].workspace, it.K = g->K, it.C = g->C, it.RS = g->R * g->S;
+    size_t need;
+    if (dtype == 0) {
+      const DgradPath path = dgrad_path(g);
+      if (path != kDgradTile3x3 && path != kDgradGather) continue;   // the other kernels read W as it is or re-lay it their own way
+      it.A = round_up(g->K, BK), it.B = g->C;
+      need = sgh_conv_workspace_bytes(g, SGH_CONV_DGRAD);
+    } else {
+      if (getenv("SGH_CONV16_OFF") || !sgh_conv16_dgrad_relayout_dims(g, &it.A, &it.B)) continue;
+      need = sgh_conv16_workspace_bytes(g, SGH_CONV_DGRAD);
+    }
+    if (!items[i].workspace || items[i].ws_bytes < need) return SGH_EWORKSPACE;
+    const long total = long(it.RS) * it.A * it.B;
+    const long blocks = it.RS <= kRelayoutMaxTaps
+                            ? long((it.A + kRelayoutTile - 1) / kRelayoutTile) * ((it.B + kRelayoutTile - 1) / kRelayoutTile)
+                            : (total + kRelayoutPerBlock - 1) / kRelayoutPerBlock;
+    if (t.count == kMaxRelayouts || long(t.block0[t.count]) + blocks >= (long(1) << 30)) {
+      const int rc = flush();
+      if (rc != SGH_OK) return rc;
+    }
+    t.it[t.count] = it;
+    batch[t.count] = g;
+    t.block0[t.count + 1] = t.block0[t.count] + int(blocks);
+    ++t.count;
+  }
+  return flush();
 }
 
 int sgh_conv_dgrad_acc_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,

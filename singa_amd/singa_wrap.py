@@ -632,6 +632,32 @@ def GpuConvBackwardW(dy, x, W, h):
     return dW
 
 
+def GpuConvPrepareBackward(weights_and_handles):
+    """Re-lays the weights of all listed convolutions for their data gradients in ONE launch (the
+    re-layout each ``GpuConvBackwardx`` otherwise launches for itself); `weights_and_handles`: pairs
+    ``(W, handle)``.  Valid until the weights change: call ``GpuConvBackwardDone`` with the same
+    handles after the backward pass, and run no other pass on a handle between this call and its
+    ``GpuConvBackwardx``.  Results are bit-identical with and without."""
+    pairs = list(weights_and_handles)
+    if not pairs:
+        return
+    W0 = pairs[0][0]
+    arr = (_lib.ConvPrepareItem * len(pairs))()
+    for i, (W, h) in enumerate(pairs):
+        if W.data_type() != W0.data_type():
+            raise SingaHipError("one weight type per GpuConvPrepareBackward call")
+        arr[i].g, arr[i].W = C.pointer(h.geom), W.ptr
+        arr[i].workspace, arr[i].ws_bytes = h.workspace.ptr, h.workspace.MemSize()
+    dtype = {kFloat32: 0, kFloat16: 1, kBFloat16: 2}[W0.data_type()]
+    check(_L().sgh_conv_dgrad_prepare_multi(arr, len(pairs), dtype, W0.device().stream), "sgh_conv_dgrad_prepare_multi")
+
+
+def GpuConvBackwardDone(handles):
+    """The weights are about to change: the next data gradients re-lay them again."""
+    for h in handles:
+        h.geom.weights_prelaid = 0
+
+
 def GpuConvBackwardb(dy, b, h):
     h._check_dy(dy)
     db = _like(b)

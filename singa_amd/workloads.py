@@ -133,11 +133,27 @@ class HipOps(object):
     def relu_bwd_add(self, dy0, dy1, x):
         return singa.ReLUBackwardSum(dy0, dy1, x)
 
-    fusions = ("fuse_bn_relu", "fuse_dgrad_add")   # what set_fusion(True) turns on
+    # batching the tape permits: the weights do not change during a backward pass, so the re-layouts
+    # that the data gradients need are done by one launch before the first backward op
+    batch_relayout = True
+
+    def prepare_backward(self, convs):
+        if self.batch_relayout:
+            by_type = {}
+            for c in convs:
+                if c.h is not None:
+                    by_type.setdefault(c.W.data_type(), []).append((c.W, c.h))
+            for pairs in by_type.values():
+                singa.GpuConvPrepareBackward(pairs)
+
+    def finish_backward(self, convs):
+        singa.GpuConvBackwardDone([c.h for c in convs if c.h is not None])
+
+    fusions = ("fuse_bn_relu", "fuse_dgrad_add", "batch_relayout")   # what set_fusion(True) turns on
 
     def set_fusion(self, on):
         """All of this implementation's cross-op fusions on, or the reference's op-per-op tape."""
-        for f in ("fuse_bn_relu", "fuse_dgrad_add", "fuse_add_relu"):
+        for f in ("fuse_bn_relu", "fuse_dgrad_add", "fuse_add_relu", "batch_relayout"):
             setattr(self, f, bool(on) and f in self.fusions)
 
     def accumulate(self, a, b):
@@ -179,7 +195,7 @@ class HalfHipOps(HipOps):
     # scattered 2-byte stores make a read-modify-write epilogue slower than the separate add)
     fuse_dgrad_add = False
     fuse_add_relu = True
-    fusions = ("fuse_bn_relu", "fuse_add_relu")
+    fusions = ("fuse_bn_relu", "fuse_add_relu", "batch_relayout")
 
     def __init__(self, dev, dtype):
         HipOps.__init__(self, dev)
@@ -500,6 +516,9 @@ class Net(object):
             items += l.param_items()
         return items
 
+    def convs(self):
+        return [l for l in self.leaf_layers() if isinstance(l, Conv)]
+
     SAVED = ("x", "y", "mean", "var")
 
     def adopt_saved_tensors(self, other):
@@ -536,6 +555,9 @@ class Net(object):
             else:
                 self.sgd.apply(name, p, g)
 
+        convs = self.convs() if hasattr(ops, "prepare_backward") else []
+        if convs:
+            ops.prepare_backward(convs)
         dy = ops.softmax_ce_bwd(self.p, self.t, self.batch)
         if keep_grads:
             self.grad_log["logits"] = dy
@@ -551,6 +573,8 @@ class Net(object):
                 dy = rev[i].bwd(dy, grads)
                 i += 1
         dy = _summed(ops, dy)
+        if convs:
+            ops.finish_backward(convs)
         if keep_grads:
             self.grad_log["input"] = dy
         if fused_update:

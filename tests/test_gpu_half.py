@@ -337,6 +337,30 @@ def test_conv_gradients_16bit_matrix_kernels(singa, dev, kind, case):
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
+def test_conv_dgrad_16bit_with_batched_weight_relayout(singa, dev, kind):
+    """GpuConvPrepareBackward on the seeded 16-bit geometries: one launch re-lays the weights of all
+    layers that the 16-bit matrix kernel covers, the data gradients that follow give the same bits."""
+    layers = []
+    for i, case in enumerate(_grad16_cases(24, 9090) + [(2, 3, 32, 32, 64, 7, 7, (2, 2), (3, 3)),
+                                                        (4, 512, 7, 7, 512, 3, 3, (1, 1), (1, 1))]):
+        N, C, H, W, K, R, S, stride, pad = case
+        r = rng(700 + i)
+        P, Q = (H + 2 * pad[0] - R) // stride[0] + 1, (W + 2 * pad[1] - S) // stride[1] + 1
+        xt, _ = _to(singa, dev, r.standard_normal((N, C, H, W)).astype(np.float32), kind)
+        wt, _ = _to(singa, dev, r.standard_normal((K, C, R, S)).astype(np.float32), kind)
+        dyt, _ = _to(singa, dev, r.standard_normal((N, K, P, Q)).astype(np.float32), kind)
+        h = singa.CudnnConvHandle(xt, (R, S), stride, pad, C, K, False)
+        layers.append((case, xt, wt, dyt, h, singa.GpuConvBackwardx(dyt, wt, xt, h).to_numpy()))
+    singa.GpuConvPrepareBackward([(l[2], l[4]) for l in layers])
+    prelaid = [l[4].geom.weights_prelaid for l in layers]
+    assert 0 in prelaid and prelaid.count(1) >= len(layers) // 2, prelaid
+    for case, xt, wt, dyt, h, want in layers:
+        _same_bits(singa.GpuConvBackwardx(dyt, wt, xt, h).to_numpy(), want, "prepared dgrad %r" % (case,))
+    singa.GpuConvBackwardDone([l[4] for l in layers])
+    assert not any(l[4].geom.weights_prelaid for l in layers)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("shape", [
     (128, 64, 56, 64, 3, 1, 1),      # ResNet-50 stage 1, 3x3
     (128, 256, 56, 64, 1, 1, 0),     # bottleneck reduce

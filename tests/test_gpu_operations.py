@@ -115,6 +115,37 @@ def test_conv_backward_vs_oracle(singa, dev, case):
     assert nl2(y, O.conv_fwd(x, w, b, stride, pad)) < TOL
 
 
+def test_conv_dgrad_with_batched_weight_relayout(singa, dev):
+    """GpuConvPrepareBackward re-lays the weights of all CONV_CASES layers in one launch; the data
+    gradients (plain and accumulating) that follow skip their own re-layout and must give the same
+    bits; layers whose kernel reads W as it is are left alone; GpuConvBackwardDone ends it."""
+    layers = []
+    for i, case in enumerate(CONV_CASES):
+        N, C, H, W, K, R, S, stride, pad, _ = case
+        r = rng(2000 + i)
+        P, Q = (H + 2 * pad[0] - R) // stride[0] + 1, (W + 2 * pad[1] - S) // stride[1] + 1
+        xd, wd = singa.from_numpy(randn(r, N, C, H, W), dev), singa.from_numpy(randn(r, K, C, R, S), dev)
+        dyd = singa.from_numpy(randn(r, N, K, P, Q), dev)
+        h = singa.CudnnConvHandle(xd, (R, S), stride, pad, C, K, False)
+        old = randn(r, N, C, H, W)
+        want = singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy()
+        want_acc = singa.GpuConvBackwardxAccumulate(dyd, wd, xd, h, singa.from_numpy(old, dev)).to_numpy()
+        layers.append((case, xd, wd, dyd, h, old, want, want_acc))
+    singa.GpuConvPrepareBackward([(l[2], l[4]) for l in layers])
+    prelaid = [l[4].geom.weights_prelaid for l in layers]
+    assert 0 in prelaid and prelaid.count(1) >= 6, prelaid
+    for case, xd, wd, dyd, h, old, want, want_acc in layers:
+        assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), want, "prepared dgrad %r" % (case,))
+    # a second use of the same prepared weights (the workspaces were not touched in between)
+    for case, xd, wd, dyd, h, old, want, want_acc in layers:
+        got = singa.GpuConvBackwardxAccumulate(dyd, wd, xd, h, singa.from_numpy(old, dev)).to_numpy()
+        assert_bit_equal(got, want_acc, "prepared accumulating dgrad %r" % (case,))
+    singa.GpuConvBackwardDone([l[4] for l in layers])
+    assert not any(l[4].geom.weights_prelaid for l in layers)
+    case, xd, wd, dyd, h, old, want, want_acc = layers[4]
+    assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), want, "after GpuConvBackwardDone")
+
+
 def test_conv_wgrad_is_deterministic(singa, dev):
     r = rng(4)
     x, dy = randn(r, 8, 64, 28, 28), randn(r, 8, 64, 28, 28)
