@@ -386,6 +386,8 @@ struct D16Args {
   int cls_tile0[5];  // first pixel tile of each residue class (stride^2 classes), then the total
   unsigned dy_bytes, wt_bytes;
   const uint16_t *bias;  // per output row (channel c), or null: the forward pass run as a data gradient
+  int dilate, out_W, out_HW;   // 1x1 stride 2: the kernel sees the stride-1 problem on the P x Q grid and its store
+                               // writes the 2 x 2 block (value, 0 / 0, 0) of the real out_HW image per pixel
 };
 
 constexpr unsigned kSelLo = 0x05040100u, kSelHi = 0x07060302u, kSelZero = 0x0c0c0c0cu;
@@ -553,6 +555,20 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   if (pix >= cnt) return;
   const int n = int(pix / HWc), rem = int(pix - long(n) * HWc), i_ = rem / Wc, j_ = rem - i_ * Wc;
   if (j_ >= Wreal) return;
+  if (a.dilate) {
+    uint16_t *o2 = a.dx + (size_t(n) * a.C) * a.out_HW + (2 * i_) * a.out_W + 2 * j_;   // (even: dword aligned)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int c = m0 + wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+        if (c < a.C) {
+          *reinterpret_cast<unsigned *>(o2 + size_t(c) * a.out_HW) = unsigned(round16<BF16>(acc[i][0][v]));
+          *reinterpret_cast<unsigned *>(o2 + size_t(c) * a.out_HW + a.out_W) = 0u;
+        }
+      }
+    return;
+  }
   uint16_t *o = a.dx + (size_t(n) * a.C) * HW + (st * i_ + ca) * a.W + st * j_ + cb;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -687,15 +703,26 @@ struct D16Plan {
   int bm, mtiles, KP, CP, tiles;
   int cls_tile0[5];
   size_t wt_bytes, dyT_bytes;   // workspace: re-laid weights, then the pixel-major copy
+  bool dilate;        // 1x1, stride 2, no padding, even image: see D16Args::dilate
+  sgh_conv_geom kg;   // the geometry the kernel sees (the stride-1 problem on the P x Q grid when `dilate`)
 };
 
-D16Plan dplan(const sgh_conv_geom *g) {
+D16Plan dplan(const sgh_conv_geom *real) {
   D16Plan p{};
-  const int st = g->stride_h;
-  if (g->stride_h != g->stride_w || (st != 1 && st != 2)) return p;
-  if (g->K % 8 != 0 || g->Q < 2 || g->C < 16) return p;  // (a 64-row tile is mostly empty below 16 channels)
+  if (real->stride_h != real->stride_w || (real->stride_h != 1 && real->stride_h != 2)) return p;
+  if (real->K % 8 != 0 || real->Q < 2 || real->C < 16) return p;  // (a 64-row tile is mostly empty below 16 channels)
   const size_t lim = size_t(1) << 30;  // byte offsets of dy stay below 2^31
-  if (size_t(g->N) * g->K * g->P * g->Q >= lim || size_t(g->N) * g->C * g->H * g->W >= 2 * lim) return p;
+  if (size_t(real->N) * real->K * real->P * real->Q >= lim || size_t(real->N) * real->C * real->H * real->W >= 2 * lim)
+    return p;
+  // 1x1 stride 2: three of the four residue classes receive no tap; instead of workgroups that only
+  // store zeros at every other position, the (0, 0) class is computed as a stride-1 problem and its
+  // store writes whole 2 x 2 blocks
+  p.kg = *real;
+  p.dilate = real->R == 1 && real->S == 1 && real->stride_h == 2 && real->pad_h == 0 && real->pad_w == 0 &&
+             real->H % 2 == 0 && real->W % 2 == 0;
+  if (p.dilate) p.kg.H = real->P, p.kg.W = real->Q, p.kg.stride_h = p.kg.stride_w = 1;
+  const sgh_conv_geom *g = &p.kg;
+  const int st = g->stride_h;
   long tiles = 0;
   for (int cls = 0; cls < st * st; ++cls) {
     const int ca = cls / st, cb = cls % st;
@@ -848,8 +875,10 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
   if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
   D16Args a{};
   a.dy = dy, a.dyT = dyT, a.wt = wt, a.dx = dx, a.bias = bias;
-  a.N = g->N, a.C = g->C, a.H = g->H, a.W = g->W, a.K = g->K, a.P = g->P, a.Q = g->Q, a.R = g->R, a.S = g->S;
-  a.stride = g->stride_h, a.pad_h = g->pad_h, a.pad_w = g->pad_w;
+  const sgh_conv_geom *kg = &p.kg;
+  a.N = kg->N, a.C = kg->C, a.H = kg->H, a.W = kg->W, a.K = kg->K, a.P = kg->P, a.Q = kg->Q, a.R = kg->R, a.S = kg->S;
+  a.stride = kg->stride_h, a.pad_h = kg->pad_h, a.pad_w = kg->pad_w;
+  a.dilate = p.dilate ? 1 : 0, a.out_W = g->W, a.out_HW = g->H * g->W;
   a.KP = p.KP, a.CP = p.CP, a.mtiles = p.mtiles, a.ptiles = p.tiles;
   for (int i = 0; i < 5; ++i) a.cls_tile0[i] = p.cls_tile0[i];
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2);
