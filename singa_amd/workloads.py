@@ -557,24 +557,26 @@ class Net(object):
 
         convs = self.convs() if hasattr(ops, "prepare_backward") else []
         if convs:
-            ops.prepare_backward(convs)
-        dy = ops.softmax_ce_bwd(self.p, self.t, self.batch)
-        if keep_grads:
-            self.grad_log["logits"] = dy
-        rev = list(reversed(self.layers))
-        i = 0
-        while i < len(rev):
-            if isinstance(rev[i], ReLU) and i + 1 < len(rev) and isinstance(rev[i + 1], BatchNorm):
-                dy = rev[i + 1].bwd_through_relu(rev[i], _summed(ops, dy), grads)   # the stem's conv -> BatchNorm -> ReLU
-                i += 2
-            else:
-                if not isinstance(rev[i], (BasicBlock, Bottleneck)):
-                    dy = _summed(ops, dy)
-                dy = rev[i].bwd(dy, grads)
-                i += 1
-        dy = _summed(ops, dy)
-        if convs:
-            ops.finish_backward(convs)
+            ops.prepare_backward(convs)   # (every layer's data gradient runs before that layer's weights change)
+        try:
+            dy = ops.softmax_ce_bwd(self.p, self.t, self.batch)
+            if keep_grads:
+                self.grad_log["logits"] = dy
+            rev = list(reversed(self.layers))
+            i = 0
+            while i < len(rev):
+                if isinstance(rev[i], ReLU) and i + 1 < len(rev) and isinstance(rev[i + 1], BatchNorm):
+                    dy = rev[i + 1].bwd_through_relu(rev[i], _summed(ops, dy), grads)   # the stem's conv -> BatchNorm -> ReLU
+                    i += 2
+                else:
+                    if not isinstance(rev[i], (BasicBlock, Bottleneck)):
+                        dy = _summed(ops, dy)
+                    dy = rev[i].bwd(dy, grads)
+                    i += 1
+            dy = _summed(ops, dy)
+        finally:
+            if convs:
+                ops.finish_backward(convs)
         if keep_grads:
             self.grad_log["input"] = dy
         if fused_update:
