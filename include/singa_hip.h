@@ -349,10 +349,10 @@ SGH_API int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float
 /* The three convolution passes on 16-bit tensors (x, W, y and their gradients all binary16 or
  * all bfloat16, as a reference handle built from a half input runs them:
  * src/model/operation/convolution.cc:444-572).  Arithmetic: fp32 accumulation of exact 16-bit
- * products, the result rounded once.  The two gradients run on the 16-bit matrix instructions
- * (stride 1 or 2; data gradient: K a multiple of 8, C >= 16, Q >= 2), the stem's data gradient on
- * the fp32 kernel reading and writing 16-bit tensors; other geometries and the forward pass widen
- * the operands to fp32 in the workspace and use the fp32 kernels.
+ * products, the result rounded once.  All three passes run on the 16-bit matrix instructions for
+ * stride 1 or 2 (data gradient: K a multiple of 8, C >= 16, Q >= 2; forward: C a multiple of 8,
+ * K >= 16, W >= 2), the stem's data gradient on the fp32 kernel reading and writing 16-bit
+ * tensors; other geometries widen the operands to fp32 in the workspace and use the fp32 kernels.
  * Workspace: sgh_conv_workspace_bytes_h(g, which) bytes. */
 SGH_API size_t sgh_conv_workspace_bytes_h(const sgh_conv_geom *g, int which);
 SGH_API int sgh_conv_dgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W,

@@ -386,6 +386,8 @@ struct D16Args {
   int cls_tile0[5];  // first pixel tile of each residue class (stride^2 classes), then the total
   unsigned dy_bytes, wt_bytes;
   const uint16_t *bias;  // per output row (channel c), or null: the forward pass run as a data gradient
+  int fs;   // step of the gradient pixel per output pixel: 1, or the stride of a forward pass run on this kernel
+            // (pixel-major loads only): tap (ti, tj) of output pixel (i, j) reads (fs * i + dr0 - ti, fs * j + ds0 - tj)
   int dilate, out_W, out_HW;   // 1x1 stride 2: the kernel sees the stride-1 problem on the P x Q grid and its store
                                // writes the 2 x 2 block (value, 0 / 0, 0) of the real out_HW image per pixel
 };
@@ -452,7 +454,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     if constexpr (PIXK) {
 #pragma unroll
       for (int i = 0; i < BSLOTS; ++i) {
-        const int p = bi_[i] + dr0 - ti, q = bj_[i] + ds0 - tj;
+        const int p = bi_[i] * a.fs + dr0 - ti, q = bj_[i] * a.fs + ds0 - tj;
         const bool in = unsigned(p) < unsigned(a.P) && unsigned(q) < unsigned(a.Q);
         bvoff[i] = in ? (((bn_[i] * a.P + p) * a.Q + q) * a.K + oct * 8) * 2 : kOOB;
       }
@@ -703,12 +705,14 @@ struct D16Plan {
   int bm, mtiles, KP, CP, tiles;
   int cls_tile0[5];
   size_t wt_bytes, dyT_bytes;   // workspace: re-laid weights, then the pixel-major copy
+  int fs;             // see D16Args::fs
   bool dilate;        // 1x1, stride 2, no padding, even image: see D16Args::dilate
   sgh_conv_geom kg;   // the geometry the kernel sees (the stride-1 problem on the P x Q grid when `dilate`)
 };
 
-D16Plan dplan(const sgh_conv_geom *real) {
+D16Plan dplan(const sgh_conv_geom *real, int fs = 1) {
   D16Plan p{};
+  p.fs = fs;
   if (real->stride_h != real->stride_w || (real->stride_h != 1 && real->stride_h != 2)) return p;
   if (real->K % 8 != 0 || real->Q < 2 || real->C < 16) return p;  // (a 64-row tile is mostly empty below 16 channels)
   const size_t lim = size_t(1) << 30;  // byte offsets of dy stay below 2^31
@@ -741,7 +745,7 @@ D16Plan dplan(const sgh_conv_geom *real) {
   // The copy pays where the dword-pair loads are at their worst: odd class widths (7 x 7 planes,
   // stride 2 on 14 x 14), where every pair row carries a dummy pixel.  (Elsewhere the kernel gains
   // 10-20 % from the aligned loads and the copy costs as much: measured at 56 x 56 .. 14 x 14.)
-  p.pixk = g->R * g->S > 1 && ((g->W + st - 1) / st) % 2 == 1;
+  p.pixk = fs > 1 || (g->R * g->S > 1 && ((g->W + st - 1) / st) % 2 == 1);
   p.wt_bytes = align256(size_t(g->R) * g->S * p.CP * p.KP * sizeof(uint16_t));
   p.dyT_bytes = p.pixk ? align256(size_t(g->N) * g->K * g->P * g->Q * sizeof(uint16_t)) : 0;
   p.ok = true;
@@ -777,10 +781,14 @@ int launch_d(const D16Args &a, const D16Plan &p, hipStream_t s) {
 // A stride-1 forward convolution is the data gradient of the convolution with the channel roles
 // swapped, the taps reversed and pad' = R - 1 - pad: y[ko][p,q] = sum_{c,r',s'} W[ko][c][R-1-r'][S-1-s']
 // * x[c][p + pad' - r'][q + pad' - s'].  False when the geometry has no such twin.
-bool fwd_twin(const sgh_conv_geom *g, sgh_conv_geom *t) {
-  if (g->stride_h != 1 || g->stride_w != 1) return false;
+bool fwd_twin(const sgh_conv_geom *g, sgh_conv_geom *t, int *fs) {
+  // stride 2: the same twin with the input pixel of tap (r', s') at (2p + pad' - r', 2q + pad' - s'), which
+  // the pixel-major loader reaches by stepping two gradient pixels per output pixel (D16Args::fs)
+  if (g->stride_h != g->stride_w || (g->stride_h != 1 && g->stride_h != 2)) return false;
   if (g->pad_h > g->R - 1 || g->pad_w > g->S - 1) return false;
+  *fs = g->stride_h;
   *t = *g;
+  t->stride_h = t->stride_w = 1;
   t->C = g->K, t->K = g->C;
   t->H = g->P, t->W = g->Q, t->P = g->H, t->Q = g->W;
   t->pad_h = g->R - 1 - g->pad_h, t->pad_w = g->S - 1 - g->pad_w;
@@ -792,8 +800,9 @@ bool fwd_twin(const sgh_conv_geom *g, sgh_conv_geom *t) {
 size_t sgh_conv16_workspace_bytes(const sgh_conv_geom *g, int which) {
   if (which == SGH_CONV_FWD) {
     sgh_conv_geom t;
-    if (!fwd_twin(g, &t)) return 0;
-    const D16Plan p = dplan(&t);
+    int fs;
+    if (!fwd_twin(g, &t, &fs)) return 0;
+    const D16Plan p = dplan(&t, fs);
     return p.ok ? p.wt_bytes + p.dyT_bytes : 0;
   }
   if (which == SGH_CONV_WGRAD) {
@@ -849,8 +858,8 @@ namespace {
 // `fwd_of`: null for the data gradient of g; otherwise g is the twin (see fwd_twin) of the forward
 // geometry *fwd_of, W is that convolution's weight tensor and `bias` its bias (or null)
 int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t *dy, const uint16_t *W,
-            const uint16_t *bias, uint16_t *dx, void *workspace, size_t ws_bytes, bool bf16, hipStream_t s) {
-  const D16Plan p = dplan(g);
+            const uint16_t *bias, uint16_t *dx, void *workspace, size_t ws_bytes, bool bf16, hipStream_t s, int fs = 1) {
+  const D16Plan p = dplan(g, fs);
   if (!p.ok) return SGH_EUNSUPPORTED;
   const int RS = g->R * g->S;
   const size_t nw = size_t(RS) * p.CP * p.KP;
@@ -879,6 +888,7 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
   a.N = kg->N, a.C = kg->C, a.H = kg->H, a.W = kg->W, a.K = kg->K, a.P = kg->P, a.Q = kg->Q, a.R = kg->R, a.S = kg->S;
   a.stride = kg->stride_h, a.pad_h = kg->pad_h, a.pad_w = kg->pad_w;
   a.dilate = p.dilate ? 1 : 0, a.out_W = g->W, a.out_HW = g->H * g->W;
+  a.fs = p.fs;
   a.KP = p.KP, a.CP = p.CP, a.mtiles = p.mtiles, a.ptiles = p.tiles;
   for (int i = 0; i < 5; ++i) a.cls_tile0[i] = p.cls_tile0[i];
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2);
@@ -914,6 +924,7 @@ int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
 int sgh_conv16_fwd(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
                    void *workspace, size_t ws_bytes, bool bf16, hipStream_t s) {
   sgh_conv_geom t;
-  if (!fwd_twin(g, &t)) return SGH_EUNSUPPORTED;
-  return run_d16(&t, g, x, W, bias, y, workspace, ws_bytes, bf16, s);
+  int fs;
+  if (!fwd_twin(g, &t, &fs)) return SGH_EUNSUPPORTED;
+  return run_d16(&t, g, x, W, bias, y, workspace, ws_bytes, bf16, s, fs);
 }

@@ -1364,7 +1364,7 @@ typedef int (*cast_out_fn)(const float *, uint16_t *, size_t, void *);
 int conv_half(const sgh_conv_geom *g, int which, const uint16_t *a, const uint16_t *b, const uint16_t *bias,
               uint16_t *out, void *workspace, size_t ws_bytes, void *stream, cast_in_fn in, cast_out_fn outc) {
   if (!conv_ok(g) || !a || !b || !out) return SGH_EINVAL;
-  // the gradients and the stride-1 forward pass run on the 16-bit matrix instructions where
+  // the gradients and the forward pass (strides 1 and 2) run on the 16-bit matrix instructions where
   // conv16.hip covers the geometry; everything else computes in fp32 on widened copies
   if (sgh_conv16_workspace_bytes(g, which) != 0 && !getenv("SGH_CONV16_OFF")) {
     const bool bf16 = in == sgh_cast_bf16_to_f32;
