@@ -65,6 +65,31 @@ def test_workspace_sizes():
     assert lib.sgh_bn_workspace_bytes(0, 64, 49) == 0
 
 
+def test_prepare_multi_argument_checks_and_geometry_flag():
+    lib = _lib.lib()
+    g = _lib.ConvGeom()
+    g.weights_prelaid = 7
+    assert lib.sgh_conv_geom_init(C.byref(g), 8, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1) == 0
+    assert g.weights_prelaid == 0                       # a fresh geometry never claims prepared weights
+    items = (_lib.ConvPrepareItem * 1)()
+    assert lib.sgh_conv_dgrad_prepare_multi(items, -1, 0, None) == -1
+    assert lib.sgh_conv_dgrad_prepare_multi(None, 1, 0, None) == -1
+    assert lib.sgh_conv_dgrad_prepare_multi(items, 1, 3, None) == -1      # unknown data type
+    assert lib.sgh_conv_dgrad_prepare_multi(items, 1, 0, None) == -1      # item without geometry / weights
+    assert lib.sgh_conv_dgrad_prepare_multi(items, 0, 0, None) == 0       # nothing to do
+
+
+def test_16bit_conv_workspace_covers_every_pass():
+    lib = _lib.lib()
+    g = _lib.ConvGeom()
+    for (Cc, H, K, R, s, p) in [(64, 56, 64, 3, 1, 1), (256, 56, 512, 1, 2, 0), (128, 56, 128, 3, 2, 1), (3, 224, 64, 7, 2, 3)]:
+        assert lib.sgh_conv_geom_init(C.byref(g), 4, Cc, H, H, K, R, R, s, s, p, p) == 0
+        for which in (_lib.SGH_CONV_FWD, _lib.SGH_CONV_DGRAD, _lib.SGH_CONV_WGRAD):
+            b = lib.sgh_conv_workspace_bytes_h(C.byref(g), which)
+            assert b > 0 and b % 256 == 0, (Cc, H, K, R, s, which, b)
+    assert lib.sgh_conv_workspace_bytes_h(C.byref(g), 3) == 0
+
+
 def test_pool_geometry():
     lib = _lib.lib()
     g = _lib.PoolGeom()
