@@ -92,6 +92,9 @@ def main():
                          "frees the host (0.94 -> 0.09 ms/step) without changing the throughput")
     ap.add_argument("--no-fusion", action="store_true",
                     help="one call per op of the reference's tape (no ReLU+BatchNorm backward fusion, residual += as its own kernel)")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="every kernel on the one device stream (weight gradients otherwise run on a second stream); "
+                         "the setting for kernel traces whose durations should be those of kernels running alone")
     ap.add_argument("--per-parameter-update", action="store_true",
                     help="update each parameter right after its gradient (one launch each) instead of one fused launch")
     args = ap.parse_args()
@@ -109,6 +112,8 @@ def main():
     half = args.storage != "f32"
     hip = wl.HalfHipOps(dev, singa.kFloat16 if args.storage == "f16" else singa.kBFloat16) if half else wl.HipOps(dev)
     hip.set_fusion(not args.no_fusion)
+    if args.no_overlap:
+        hip.overlap_wgrad = False
     net = wl.build(args.config, hip, lr=0.05, momentum=0.9)
     x, labels = wl.make_inputs(args.config, args.batch)
     net.forward(hip.from_numpy(x), hip.from_numpy(labels))
@@ -148,6 +153,7 @@ def main():
         dev.ResetGraph()
     # kernel-level pass (eager): every conv / GEMM launch bracketed by HIP events on the device stream
     prof_steps = max(1, min(args.steps, 5))
+    hip.overlap_wgrad = False   # one kernel at a time on the device, so that an event pair brackets that kernel alone
     lib.sgh_prof_enable(1)
     for _ in range(prof_steps):
         net.backward_and_update(fused_update=fused)
@@ -190,6 +196,8 @@ def main():
                    "launch": "one recorded step replayed (graph mode)" if graph else "eager, one launch per kernel",
                    "tape": "ReLU backward folded into BatchNorm backward (conv-BN-ReLU), residual += folded into the "
                            + ("data gradient" if hip.fuse_dgrad_add else "ReLU backward that reads the sum")
+                           + ", weight re-layouts in one launch"
+                           + (", weight gradients on a second stream" if not (args.no_overlap or graph) else "")
                            if hip.fuse_bn_relu
                            else "one call per reference op"},
         "roofline": roofline,

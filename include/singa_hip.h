@@ -60,7 +60,14 @@ SGH_API int sgh_device_open(int gpu_id, sgh_device **out);
 SGH_API int sgh_device_close(sgh_device *dev);
 /* The stream behind Device::Exec for this device (hipStream_t as void*). */
 SGH_API void *sgh_device_stream(sgh_device *dev);
-/* Device::Sync (src/core/device/cuda_gpu.cc:206-209): blocks until the stream is idle. */
+/* A second compute stream of the device (default priority, created on first use; NULL on failure),
+ * for work that is independent of what the main stream runs next -- a layer's weight gradient
+ * beside its data gradient.  No counterpart in the reference (CudaGPU has one stream).  Order it
+ * against the main stream with sgh_event_record / sgh_stream_wait_event, and keep every buffer it
+ * reads or writes alive until the main stream has waited for it: the pool hands freed blocks out
+ * again in the submission order of the MAIN stream only. */
+SGH_API void *sgh_device_aux_stream(sgh_device *dev);
+/* Device::Sync (src/core/device/cuda_gpu.cc:206-209): blocks until the device's streams are idle. */
 SGH_API int sgh_device_sync(sgh_device *dev);
 
 /* DeviceMemPool::Malloc / Free (include/singa/core/memory.h:41-45).  Size-bucketed cache:
@@ -101,6 +108,8 @@ typedef struct sgh_event sgh_event;
 SGH_API int sgh_event_create(sgh_event **ev);
 SGH_API int sgh_event_destroy(sgh_event *ev);
 SGH_API int sgh_event_record(sgh_event *ev, void *stream);
+/* Work enqueued on `stream` after this call starts only when what `ev` recorded has finished. */
+SGH_API int sgh_stream_wait_event(void *stream, sgh_event *ev);
 /* Blocks on `stop`, then returns stop - start in milliseconds. */
 SGH_API int sgh_event_elapsed_ms(sgh_event *start, sgh_event *stop, float *ms);
 

@@ -53,6 +53,7 @@ SIGNATURES = {
     "sgh_device_open": (C.c_int, [C.c_int, C.POINTER(vp)]),
     "sgh_device_close": (C.c_int, [vp]),
     "sgh_device_stream": (vp, [vp]),
+    "sgh_device_aux_stream": (vp, [vp]),
     "sgh_device_sync": (C.c_int, [vp]),
     "sgh_malloc": (C.c_int, [vp, C.POINTER(vp), sz]),
     "sgh_free": (C.c_int, [vp, vp]),
@@ -67,6 +68,7 @@ SIGNATURES = {
     "sgh_event_create": (C.c_int, [C.POINTER(vp)]),
     "sgh_event_destroy": (C.c_int, [vp]),
     "sgh_event_record": (C.c_int, [vp, vp]),
+    "sgh_stream_wait_event": (C.c_int, [vp, vp]),
     "sgh_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
     "sgh_prof_enable": (C.c_int, [C.c_int]),
     "sgh_prof_count": (C.c_int, [C.POINTER(C.c_int)]),

@@ -14,6 +14,7 @@ struct sgh_device {
   int id = 0;
   hipStream_t stream = nullptr;
   hipStream_t side = nullptr;  // uploads that must happen while `stream` is recording
+  hipStream_t aux = nullptr;   // second compute stream (sgh_device_aux_stream), created on first use
   std::mutex mu;
   // free blocks keyed by their (rounded) size; blocks in use keyed by address
   std::multimap<size_t, void *> free_blocks;
@@ -165,16 +166,39 @@ int sgh_device_close(sgh_device *dev) {
   for (auto &kv : dev->live) (void)hipFree(kv.first);
   (void)hipStreamDestroy(dev->stream);
   (void)hipStreamDestroy(dev->side);
+  if (dev->aux) {
+    (void)hipStreamSynchronize(dev->aux);
+    (void)hipStreamDestroy(dev->aux);
+  }
   delete dev;
   return SGH_OK;
 }
 
 void *sgh_device_stream(sgh_device *dev) { return dev ? reinterpret_cast<void *>(dev->stream) : nullptr; }
 
+void *sgh_device_aux_stream(sgh_device *dev) {
+  if (!dev) return nullptr;
+  if (!dev->aux) {
+    (void)hipSetDevice(dev->id);
+    if (hipStreamCreateWithFlags(&dev->aux, hipStreamNonBlocking) != hipSuccess) {   // (default priority)
+      (void)hipGetLastError();
+      dev->aux = nullptr;
+    }
+  }
+  return reinterpret_cast<void *>(dev->aux);
+}
+
+int sgh_stream_wait_event(void *stream, sgh_event *ev) {
+  if (!ev) return SGH_EINVAL;
+  SGH_HIP_TRY(hipStreamWaitEvent(sgh_stream_of(stream), ev->ev, 0));
+  return SGH_OK;
+}
+
 int sgh_device_sync(sgh_device *dev) {
   if (!dev) return SGH_EINVAL;
   if (dev->capturing) return SGH_EUNSUPPORTED;  // nothing runs while the stream records
   SGH_HIP_TRY(hipStreamSynchronize(dev->stream));
+  if (dev->aux) SGH_HIP_TRY(hipStreamSynchronize(dev->aux));
   return SGH_OK;
 }
 

@@ -86,6 +86,34 @@ class HipGPU(object):
     def Sync(self):
         check(_L().sgh_device_sync(self._h), "sgh_device_sync")
 
+    # A second compute stream for work that the main stream's next ops do not depend on.  Fork():
+    # what is enqueued on the auxiliary stream afterwards starts when everything enqueued on the main
+    # stream so far has finished; Join(): the main stream waits for the auxiliary one.  Tensors the
+    # auxiliary stream touches must be kept alive until Join() (the pool recycles in main-stream order).
+    _aux = None
+
+    def AuxStream(self):
+        if self._aux is None:
+            s = _L().sgh_device_aux_stream(self._h)
+            if not s:
+                raise SingaHipError("no auxiliary stream")
+            ev = [C.c_void_p(), C.c_void_p()]
+            for e in ev:
+                check(_L().sgh_event_create(C.byref(e)), "sgh_event_create")
+            self._aux, self._fork_ev, self._join_ev = s, ev[0], ev[1]
+        return self._aux
+
+    def Fork(self):
+        aux = self.AuxStream()
+        check(_L().sgh_event_record(self._fork_ev, self.stream), "sgh_event_record")
+        check(_L().sgh_stream_wait_event(aux, self._fork_ev), "sgh_stream_wait_event")
+        return aux
+
+    def Join(self):
+        if self._aux is not None:
+            check(_L().sgh_event_record(self._join_ev, self._aux), "sgh_event_record")
+            check(_L().sgh_stream_wait_event(self.stream, self._join_ev), "sgh_stream_wait_event")
+
     def GetAllocatedMem(self):
         a, c, d = C.c_size_t(), C.c_size_t(), C.c_size_t()
         check(_L().sgh_pool_stats(self._h, C.byref(a), C.byref(c), C.byref(d)))
@@ -577,6 +605,7 @@ class CudnnConvHandle(object):
             raise SingaHipError("workspace of %d bytes exceeds the limit" % need)
         self.workspace_count = need // 4
         self.workspace = Tensor((max(self.workspace_count, 1),), x.device(), kFloat32)
+        self.wgrad_workspace = None   # a second one, made when a weight gradient runs on the auxiliary stream
 
     def _check_x(self, x):
         if x.shape() != [self.batchsize, self.channels, self.height, self.width]:
@@ -622,13 +651,24 @@ def GpuConvBackwardx(dy, W, x, h):
     return dx
 
 
-def GpuConvBackwardW(dy, x, W, h):
+def GpuConvBackwardW(dy, x, W, h, stream=None):
+    """`stream`: None = the device's stream.  Another stream (``HipGPU.Fork()``) runs the weight
+    gradient beside whatever the main stream does next; it then works in a workspace of its own
+    (``h.wgrad_workspace``), and the caller keeps dy, x and the result alive until ``Join()``."""
     h._check_dy(dy)
     h._check_x(x)
     dW = _like(W)
     fn, name = _fn("conv_wgrad", dy)
-    check(fn(C.byref(h.geom), dy.ptr, x.ptr, dW.ptr, h.workspace.ptr, h.workspace.MemSize(),
-             dy.device().stream), name)
+    ws = h.workspace
+    if stream is not None:
+        if h.wgrad_workspace is None:
+            which = _lib.SGH_CONV_WGRAD
+            need = (_L().sgh_conv_workspace_bytes(C.byref(h.geom), which) if dy.data_type() == kFloat32
+                    else _L().sgh_conv_workspace_bytes_h(C.byref(h.geom), which))
+            h.wgrad_workspace = Tensor(((max(need, 4) + 3) // 4,), dy.device(), kFloat32)
+        ws = h.wgrad_workspace
+    check(fn(C.byref(h.geom), dy.ptr, x.ptr, dW.ptr, ws.ptr, ws.MemSize(),
+             dy.device().stream if stream is None else stream), name)
     return dW
 
 

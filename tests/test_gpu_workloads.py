@@ -158,9 +158,12 @@ def test_fused_tape_equals_reference_tape(dev, config, kind):
         hip.set_fusion(fuse)
         assert hip.fuse_bn_relu == fuse and (hip.fuse_dgrad_add or hip.fuse_add_relu) == fuse
         net = wl.build(config, hip)
+        assert hip.overlap_wgrad == fuse and hip.batch_relayout == fuse
         for _ in range(2):
             net.forward(hip.from_numpy(x), hip.from_numpy(labels))
-            dx = net.backward_and_update()
+            # the fused tape also updates all parameters in one launch at the end, which lets it run
+            # the weight gradients on the auxiliary stream
+            dx = net.backward_and_update(fused_update=fuse)
         outs.append([hip.to_numpy(dx)] + [hip.to_numpy(p) for _, p in net.params()])
     for a, b in zip(*outs):
         assert np.array_equal(a, b)
