@@ -68,7 +68,8 @@ def _L():
 # ------------------------------------------------------------------------------------ device
 
 class HipGPU(object):
-    """Counterpart of ``CudaGPU`` (include/singa/core/device.h:57-174): one stream, one pool."""
+    """Counterpart of ``CudaGPU`` (include/singa/core/device.h:57-174): one stream, one pool (and an
+    auxiliary stream for work the caller orders itself, see ``Fork``)."""
 
     def __init__(self, gpu_id=0):
         h = C.c_void_p()
