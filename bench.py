@@ -177,6 +177,8 @@ def main():
                    "fp32 MFMA conv dgrad + wgrad kernels (k_dgrad3x3, k_wgrad3x3, k_dgrad_fewc, k_wgrad_fewc, k_igemm; %d launches/step)")
                   % (launches // prof_steps),
         "flop_per_step": flop / prof_steps, "kernel_ms_per_step": round(ms / prof_steps, 4),
+        "timing": "HIP event pair around every launch in %d extra steps with all kernels on one stream "
+                  "(the timed steps run the weight gradients on a second stream)" % prof_steps,
     }
     for k, v in conv.items():
         roofline[k + "_tflops"] = round(v["flop"] / (v["ms"] * 1e-3) / 1e12, 3) if v["ms"] > 0 else 0.0
