@@ -169,6 +169,28 @@ def test_fused_tape_equals_reference_tape(dev, config, kind):
         assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("config,batch,kind", [("resnet18", 64, "f32"), ("resnet50", 32, "f16")])
+def test_two_stream_tape_at_full_size(dev, config, batch, kind):
+    """The weight gradients on the auxiliary stream at the benchmark's layer sizes, where the two
+    chains really run side by side for milliseconds: three steps leave bit-identical parameters and
+    input gradient to the same tape with every kernel on one stream."""
+    from singa_amd import singa_wrap as singa
+    x, labels = wl.make_inputs(config, batch)
+    outs = []
+    for overlap in (False, True):
+        hip = wl.HipOps(dev) if kind == "f32" else wl.HalfHipOps(dev, singa.kFloat16)
+        hip.overlap_wgrad = overlap
+        net = wl.build(config, hip, lr=0.01)
+        for _ in range(3):
+            net.forward(hip.from_numpy(x), hip.from_numpy(labels))
+            dx = net.backward_and_update(fused_update=True)
+        outs.append([hip.to_numpy(dx)] + [hip.to_numpy(p) for _, p in net.params()])
+        del net
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b, equal_nan=True)
+    assert all(np.isfinite(a).all() for a in outs[0][1:])
+
+
 def test_graph_replay_of_the_step(dev):
     """Graph mode (EnableGraph / RunGraph): one recorded backward+update step, replayed several
     times with eager work and synchronisations in between, leaves after every replay exactly the
