@@ -35,6 +35,7 @@ extern "C" {
 #define SGH_EUNSUPPORTED (-3)
 #define SGH_ELABEL (-4)     /* a class label was out of range (checked variant only) */
 #define SGH_ENOMEM (-5)
+#define SGH_ELIMIT (-6)     /* size beyond the fixed scratch of a non-allocating entry point */
 
 /* Human-readable text for a return code (static storage). */
 SGH_API const char *sgh_error_string(int rc);
@@ -404,6 +405,20 @@ SGH_API int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma,
                            const float *save_mean, const float *save_invstd, float *dx,
                            float *dgamma, float *dbeta, int N, int C, int HW, void *workspace,
                            size_t ws_bytes, void *stream);
+/* sgh_bn_bwd_f32 for callers that cannot allocate device memory and have no workspace to pass
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same kernels, same results bit for bit; the per-channel partial
+ * sums live in a buffer that is part of the library's code object (128 KiB on every GPU the
+ * library runs on, held until the process ends) instead of a workspace.  Limit: the number of
+ * (channel, split) partial sums -- C for C > 2048, below 2048 + C otherwise -- may not exceed 16384, i.e. C <= 16384;
+ * beyond that SGH_ELIMIT is returned and nothing is launched.  Calls no hipMalloc / hipFree.
+ * All calls on one GPU share the buffer: calls that overlap on one GPU (two streams, two threads)
+ * race; calls on one stream are ordered and safe.  Nothing in the buffer needs clearing between
+ * calls (every slot read is written earlier in the same call). */
+SGH_API int sgh_bn_bwd_noalloc_f32(const float *dy, const float *x, const float *gamma,
+                                   const float *save_mean, const float *save_invstd, float *dx,
+                                   float *dgamma, float *dbeta, int N, int C, int HW,
+                                   void *stream);
 /* ReLUBackward followed by GpuBatchNormBackward in one pass, for a ReLU whose input is this
  * BatchNorm's output (python/singa/autograd.py:432-439 then batchnorm.cc:368-404; the tape of
  * conv -> BatchNorm -> ReLU, examples/cnn/model/resnet.py:54-60).  `dy` is the gradient behind the

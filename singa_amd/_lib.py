@@ -143,6 +143,7 @@ SIGNATURES = {
     "sgh_bn_fwd_train_f32": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
                                        C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_bwd_f32": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_bwd_noalloc_f32": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
     "sgh_bn_fwd_train_f16": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
                                        C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_fwd_train_bf16": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
@@ -163,6 +164,7 @@ SIGNATURES = {
 
 SGH_CONV_FWD, SGH_CONV_DGRAD, SGH_CONV_WGRAD = 0, 1, 2
 SGH_EUNSUPPORTED = -3
+SGH_ELIMIT = -6
 
 
 class SingaHipError(RuntimeError):

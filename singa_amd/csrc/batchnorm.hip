@@ -7,8 +7,16 @@
 // range of the channel's (n, hw) index space with 16-byte loads where HW % 4 == 0.
 // Reductions are a fixed tree (lane partials -> wavefront shuffle -> LDS -> ordered sum over
 // the S partials), so results are run-to-run identical.
+#include <mutex>
+
 #include "common.h"
 #include "storage.h"
+
+// Partial sums of sgh_bn_bwd_noalloc_f32: device memory the library owns from load time on, so the
+// entry point has nothing to allocate.  In host code this name is only a handle for
+// hipGetSymbolAddress; kernels receive the address looked up per device (noalloc_scratch_of).
+constexpr int kNoAllocMaxPairs = 16384;  // (channel, split) pairs of two floats: 128 KiB per device
+static __device__ __align__(256) float scratch[kNoAllocMaxPairs * 2];
 
 namespace {
 
@@ -518,7 +526,32 @@ int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *g
   return SGH_OK;
 }
 
+// ---- device address of `scratch`, looked up once per device with that device current
+constexpr int kNoAllocMaxDevices = 64;
+float *g_noalloc_ptr[kNoAllocMaxDevices];
+std::mutex g_noalloc_mu;
+
+int noalloc_scratch_of_current_device(float **out) {
+  int dev = -1;
+  SGH_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kNoAllocMaxDevices) return SGH_EUNSUPPORTED;
+  std::lock_guard<std::mutex> lk(g_noalloc_mu);
+  if (!g_noalloc_ptr[dev]) {
+    void *p = nullptr;
+    SGH_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return SGH_EUNSUPPORTED;
+    g_noalloc_ptr[dev] = static_cast<float *>(p);
+  }
+  *out = g_noalloc_ptr[dev];
+  return SGH_OK;
+}
+
 }  // namespace
+
+int sgh_bn_noalloc_setup() {
+  float *p = nullptr;
+  return noalloc_scratch_of_current_device(&p);
+}
 
 extern "C" {
 
@@ -558,6 +591,18 @@ int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const fl
                    void *workspace, size_t ws_bytes, void *stream) {
   return bn_bwd<StF32>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, workspace, ws_bytes,
                        stream);
+}
+int sgh_bn_bwd_noalloc_f32(const float *dy, const float *x, const float *gamma, const float *save_mean,
+                           const float *save_invstd, float *dx, float *dgamma, float *dbeta, int N, int C, int HW,
+                           void *stream) {
+  if (!shape_ok(N, C, HW)) return SGH_EINVAL;
+  const size_t pairs = size_t(C) * make_shape(N, C, HW, StF32::VEC, int(sizeof(float))).S;
+  if (pairs > size_t(kNoAllocMaxPairs)) return SGH_ELIMIT;
+  float *part = nullptr;  // (every slot the second kernel reads is written by the first: nothing to clear)
+  const int rc = noalloc_scratch_of_current_device(&part);
+  if (rc != SGH_OK) return rc;
+  return bn_bwd<StF32>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, part,
+                       pairs * 2 * sizeof(float), stream);
 }
 int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                    const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,

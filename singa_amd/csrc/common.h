@@ -31,6 +31,11 @@ static inline bool sgh_aligned16(const void *p) { return (reinterpret_cast<uintp
 // Number of compute units of the current device (cached per process; one GPU per process).
 int sgh_num_cus();
 
+// Looks up, for the current device, the address of the library-owned partial-sum buffer of
+// sgh_bn_bwd_noalloc_f32 (batchnorm.hip).  sgh_device_open calls it so that the entry point's first
+// call on a device finds the address ready; the entry point repeats the lookup if it was not.
+int sgh_bn_noalloc_setup();
+
 // Kernel-level profiling hooks (no-ops unless sgh_prof_enable(1) was called).
 bool sgh_prof_on();
 void sgh_prof_start(const char *tag, double work, hipStream_t s);

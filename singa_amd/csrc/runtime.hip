@@ -113,6 +113,7 @@ const char *sgh_error_string(int rc) {
     case SGH_EUNSUPPORTED: return "unsupported configuration";
     case SGH_ELABEL: return "class label out of range";
     case SGH_ENOMEM: return "out of device memory";
+    case SGH_ELIMIT: return "size beyond the fixed scratch buffer of a non-allocating entry point";
     default: break;
   }
   if (rc > 0) return hipGetErrorString(static_cast<hipError_t>(rc));
@@ -143,6 +144,13 @@ int sgh_device_open(int gpu_id, sgh_device **out) {
     if (d->stream) (void)hipStreamDestroy(d->stream);
     delete d;
     return (int)e;
+  }
+  const int rc = sgh_bn_noalloc_setup();
+  if (rc != SGH_OK) {
+    (void)hipStreamDestroy(d->stream);
+    (void)hipStreamDestroy(d->side);
+    delete d;
+    return rc;
   }
   *out = d;
   return SGH_OK;
