@@ -101,7 +101,12 @@ SGH_API int sgh_pool_trim(sgh_device *dev);
  * (= core.proto CopyDirection, src/proto/core.proto:43-48).  D2H and H2D block until the
  * copy has completed so the host may touch the buffer when the call returns. */
 SGH_API int sgh_memcpy(sgh_device *dev, void *dst, const void *src, size_t bytes, int kind);
+/* Tensor::SetValue (src/core/tensor/tensor.cc:849-865, Set<DType, Lang>): every element = value.
+ * The 16-bit variants round `value` once to the storage type (nearest, ties to even) and write
+ * 2-byte elements; n counts elements. */
 SGH_API int sgh_memset_f32(float *dst, float value, size_t n, void *stream);
+SGH_API int sgh_memset_f16(uint16_t *dst, float value, size_t n, void *stream);
+SGH_API int sgh_memset_bf16(uint16_t *dst, float value, size_t n, void *stream);
 
 /* Per-op timing for Graph profiling (TimeProfilingDoExec / EvaluateTimeElapsed,
  * src/core/device/cuda_gpu.cc:117-169): event pairs on the device stream. */

@@ -61,6 +61,8 @@ SIGNATURES = {
     "sgh_pool_trim": (C.c_int, [vp]),
     "sgh_memcpy": (C.c_int, [vp, vp, vp, sz, C.c_int]),
     "sgh_memset_f32": (C.c_int, [vp, C.c_float, sz, vp]),
+    "sgh_memset_f16": (C.c_int, [vp, C.c_float, sz, vp]),
+    "sgh_memset_bf16": (C.c_int, [vp, C.c_float, sz, vp]),
     "sgh_graph_begin": (C.c_int, [vp]),
     "sgh_graph_end": (C.c_int, [vp, C.POINTER(vp)]),
     "sgh_graph_launch": (C.c_int, [vp]),

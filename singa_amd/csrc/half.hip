@@ -6,6 +6,8 @@
 //
 // Each thread moves 16 bytes (8 elements) per access; a workgroup streams contiguous 16 KB
 // chunks, as in the fp32 kernels.
+#include <string.h>
+
 #include "common.h"
 #include "storage.h"
 #include "sgd_math.h"
@@ -326,9 +328,64 @@ __global__ __launch_bounds__(kBlock) void k_sgd_multi_mixed(const sgh_sgd_mixed_
   }
 }
 
+// Tensor::SetValue on a 16-bit tensor: the value rounded once, written as pairs where aligned
+__global__ __launch_bounds__(kBlock) void k_fill16(u16 *dst, u16 bits, size_t n) {
+  const size_t stride = size_t(gridDim.x) * kBlock, t = size_t(blockIdx.x) * kBlock + threadIdx.x;
+  const size_t head = (reinterpret_cast<uintptr_t>(dst) & 2u) ? 1 : 0;   // elements before the first 4-byte boundary
+  if (t == 0 && head && n) dst[0] = bits;
+  if (n <= head) return;
+  unsigned *d2 = reinterpret_cast<unsigned *>(dst + head);
+  const size_t pairs = (n - head) >> 1;
+  const unsigned two = unsigned(bits) | (unsigned(bits) << 16);
+  for (size_t i = t; i < pairs; i += stride) d2[i] = two;
+  if (t == 0 && ((n - head) & 1)) dst[n - 1] = bits;
+}
+
+int fill16(uint16_t *dst, uint16_t bits, size_t n, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!dst || (reinterpret_cast<uintptr_t>(dst) & 1u)) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_fill16, dim3(grid_for((n + 1) >> 1)), dim3(kBlock), 0, sgh_stream_of(stream), dst, bits, n);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+// host-side rounding to nearest even, the same results as the device conversions of storage.h
+uint16_t host_f32_to_bf16(float f) {
+  unsigned u;
+  memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return uint16_t(u >> 16);
+}
+uint16_t host_f32_to_f16(float f) {
+  unsigned u;
+  memcpy(&u, &f, 4);
+  const unsigned sign = (u >> 16) & 0x8000u;
+  u &= 0x7fffffffu;
+  if (u > 0x7f800000u) return uint16_t(sign | 0x7e00u);   // NaN
+  if (u >= 0x38800000u) {                                  // normal in binary16 (or beyond its range)
+    u += 0xfffu + ((u >> 13) & 1u);
+    if (u >= 0x47800000u) return uint16_t(sign | 0x7c00u);  // rounds to infinity (|f| >= 65520)
+    return uint16_t(sign | ((u - 0x38000000u) >> 13));
+  }
+  // subnormal result: adding 0.5 puts the unit in the last place at 2^-24, the FPU rounds to even
+  float a;
+  memcpy(&a, &u, 4);
+  a += 0.5f;
+  memcpy(&u, &a, 4);
+  return uint16_t(sign | (u - 0x3f000000u));
+}
+
 }  // namespace
 
 extern "C" {
+
+int sgh_memset_f16(uint16_t *dst, float value, size_t n, void *stream) {
+  return fill16(dst, host_f32_to_f16(value), n, stream);
+}
+int sgh_memset_bf16(uint16_t *dst, float value, size_t n, void *stream) {
+  return fill16(dst, host_f32_to_bf16(value), n, stream);
+}
 
 int sgh_sgd_momentum_multi_mixed(const sgh_sgd_mixed_item *table_dev, int count, size_t total_n, int bf16, float lr,
                                  float mu, float damp, float wd, int nesterov, void *stream) {

@@ -315,7 +315,8 @@ class Tensor(object):
         return out.reshape(self._shape)
 
     def SetFloatValue(self, v):
-        check(_L().sgh_memset_f32(self.ptr, float(v), self.Size(), self._dev.stream), "sgh_memset_f32")
+        fn, name = _fn("memset", self)   # the fill of this tensor's element size (int tensors are not filled with floats)
+        check(fn(self.ptr, float(v), self.Size(), self._dev.stream), name)
 
     # --- arithmetic used by autograd / opt  (Tensor::operator+=, *=: src/core/tensor/tensor.cc:579-589)
     def __iadd__(self, other):
@@ -329,9 +330,15 @@ class Tensor(object):
             scalar = other.Size() == 1 and self.Size() != 1
             if not scalar:
                 _same(self, other)
+            if self._dtype != kFloat32 and not scalar:
+                fn, name = _fn("eltwise_mult", self)
+                check(fn(self.ptr, other.ptr, self.ptr, self.Size(), self._dev.stream), name)
+                return self
+            _need_f32("Tensor *=", self, other)
             check(_L().sgh_eltwise_mult_f32(self.ptr, other.ptr, int(scalar), self.ptr, self.Size(),
                                             self._dev.stream), "sgh_eltwise_mult_f32")
         else:
+            _need_f32("Tensor *= scalar", self)
             s = from_numpy(np.array([other], dtype=np.float32), self._dev)
             check(_L().sgh_eltwise_mult_f32(self.ptr, s.ptr, 1, self.ptr, self.Size(), self._dev.stream),
                   "sgh_eltwise_mult_f32")
@@ -340,6 +347,14 @@ class Tensor(object):
     def __itruediv__(self, d):
         # Div(tensor, scalar) multiplies by the fp32 reciprocal (src/core/tensor/tensor_math.h:149-153)
         return self.__imul__(float(np.float32(1.0) / np.float32(d)))
+
+
+def _need_f32(what, *tensors):
+    """The fp32-only entry points read their operands as floats: refuse anything else, as the
+    reference's TYPE_LANG_SWITCH does for a type it has no kernel for (tensor.cc:760-812)."""
+    for t in tensors:
+        if t is not None and t.data_type() != kFloat32:
+            raise SingaHipError("%s: float32 tensors only, got data type %r" % (what, t.data_type()))
 
 
 def _same(a, b):
@@ -390,6 +405,7 @@ def _like(t):
 
 
 def ReLU(x):
+    _need_f32("ReLU", x)
     y = _like(x)
     check(_L().sgh_relu_fwd_f32(x.ptr, y.ptr, x.Size(), x.device().stream), "sgh_relu_fwd_f32")
     return y
@@ -417,6 +433,7 @@ def ReLUBackwardSum(dy0, dy1, x):
 
 
 def SoftMax(x):
+    _need_f32("SoftMax", x)
     batch = x.shape(0) if x.nDim() == 2 else 1
     p = _like(x)
     check(_L().sgh_softmax_fwd_f32(x.ptr, p.ptr, batch, x.Size() // batch, x.device().stream),
@@ -427,6 +444,7 @@ def SoftMax(x):
 def _ce_dims(p, t):
     if p.nDim() > 2 or t.nDim() > 2:
         raise SingaHipError("cross entropy expects at most 2-D tensors")
+    _need_f32("cross entropy", p)
     if t.data_type() != kInt:
         raise SingaHipError("the target tensor must hold int32 (the reference reads it as int)")
     batch = p.shape(0) if p.nDim() == 2 else 1
@@ -467,6 +485,7 @@ def Axpy(alpha, x, y):
     if isinstance(alpha, Tensor):
         if alpha.Size() != 1:
             raise SingaHipError("Tensor alpha must have one element")
+        _need_f32("Axpy with a Tensor alpha", alpha, x, y)
         check(_L().sgh_axpy_devalpha_f32(alpha.ptr, x.ptr, y.ptr, x.Size(), x.device().stream),
               "sgh_axpy_devalpha_f32")
     else:
@@ -546,6 +565,7 @@ def Mult(A, B):
     flags of the views select the GEMM variant, no data is moved."""
     if A.nDim() != 2 or B.nDim() != 2 or A.shape(1) != B.shape(0):
         raise SingaHipError("Mult shape mismatch %s x %s" % (A.shape(), B.shape()))
+    _need_f32("Mult", A, B)
     M, K, N = A.shape(0), A.shape(1), B.shape(1)
     out = Tensor((M, N), A.device(), kFloat32)
     tA, tB = A.transpose(), B.transpose()
@@ -560,12 +580,14 @@ def Sum(t, axis):
     """``singa.Sum(t, 0)`` of a 2-D tensor: column sums (bias gradient of AddBias)."""
     if t.nDim() != 2 or axis != 0 or t.transpose():
         raise SingaHipError("only Sum(2-D tensor, 0) is on the backward path")
+    _need_f32("Sum", t)
     out = Tensor((t.shape(1),), t.device(), kFloat32)
     check(_L().sgh_sum_rows_f32(t.ptr, out.ptr, t.shape(0), t.shape(1), t.device().stream), "sgh_sum_rows_f32")
     return out
 
 
 def AddRow(v, m):
+    _need_f32("AddRow", v, m)
     check(_L().sgh_add_row_f32(v.ptr, m.ptr, m.shape(0), m.shape(1), m.device().stream), "sgh_add_row_f32")
 
 

@@ -104,3 +104,19 @@ def test_pool_geometry():
 def test_missing_library_fails_loudly(tmp_path):
     with pytest.raises(_lib.SingaHipError):
         _lib.load(str(tmp_path / "nope.so"))
+
+
+def test_fp32_only_wrappers_check_the_data_type_before_any_call():
+    """A 16-bit tensor handed to a function that only exists for float32 is refused on the host
+    (the kernel would read twice the tensor's bytes).  Needs no GPU: the check comes first."""
+    import pytest
+    from singa_amd import singa_wrap as singa
+
+    class _NoDevice(object):
+        stream = None
+
+    t = singa.from_device_pointer(0x1000, (4, 8), _NoDevice(), singa.kFloat16)
+    for call in (lambda: singa.ReLU(t), lambda: singa.SoftMax(t), lambda: singa.Mult(t, t.T()), lambda: singa.Sum(t, 0),
+                 lambda: singa.AddRow(t, t), lambda: t.__imul__(2.0)):
+        with pytest.raises(singa.SingaHipError, match="float32"):
+            call()

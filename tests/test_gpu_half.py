@@ -452,3 +452,39 @@ def test_sgd_on_16bit_gradients(singa, dev, kind, hyper):
         _same_bits(pt.to_numpy(), _round(singa, p, kind), "working copy " + kind)
         if mu != 0:
             _same_bits(sgd.moments["w"].to_numpy(), v, "master v " + kind)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+def test_set_value_on_16bit_tensors_stays_inside_the_tensor(singa, dev, kind):
+    """Tensor::SetValue on a 16-bit tensor writes 2-byte elements: the neighbours of the filled
+    range keep their contents (a float fill of the same element count would run over them), at
+    every alignment of the range and for odd lengths; the value is rounded once to the storage type."""
+    dt = singa.kFloat16 if kind == "f16" else singa.kBFloat16
+    values = [0.1, -3.0, 65520.0, 1e-7, 2.0 ** -25 * 1.5, 1.00390625]
+    for off, n, v in [(0, 1000, 0.1), (1, 1001, -3.0), (2, 7, 65520.0), (3, 1, 1e-7), (5, 64 * 1024 + 3, values[4]),
+                      (8, 0, 1.0), (7, 2, values[5])]:
+        total = off + n + 9
+        sentinel = np.full(total, 0x7B7B, np.uint16)
+        big = singa.Tensor((total,), dev, dt)
+        big.CopyHalfDataFromHostPtr(sentinel.view(np.float16) if kind == "f16" else sentinel)   # (raw payloads)
+        view = singa.from_device_pointer(big.ptr + 2 * off, (n,), dev, dt, keepalive=big)
+        view.SetFloatValue(v)
+        got = np.empty(total, np.uint16)
+        from singa_amd._lib import check, lib
+        check(lib().sgh_memcpy(dev._h, got.ctypes.data, big.ptr, got.nbytes, 2))
+        want = sentinel.copy()
+        if kind == "f16":
+            with np.errstate(over="ignore"):
+                want[off:off + n] = np.float32(v).astype(np.float16).view(np.uint16)
+        else:
+            want[off:off + n] = singa.float_to_bf16_bits(np.array([v], np.float32))[0]
+        assert np.array_equal(got, want), (kind, off, n, v)
+
+
+def test_fp32_only_functions_refuse_16bit_tensors(singa, dev):
+    t = singa.Tensor((4, 8), dev, singa.kFloat16)
+    t.SetFloatValue(1.0)
+    for call in (lambda: singa.ReLU(t), lambda: singa.SoftMax(t), lambda: singa.Mult(t, t.T()),
+                 lambda: singa.Sum(t, 0), lambda: t.__imul__(2.0)):
+        with pytest.raises(singa.SingaHipError):
+            call()

@@ -8,7 +8,10 @@ import numpy as np
 import pytest
 
 from oracle.ops import OracleOps
+from rounding_oracle import UNIT_ROUNDOFF, RoundingOracleOps, errors_against_truth, saved_inputs, store_fn
 from singa_amd import workloads as wl
+from torch_ref import TorchNet
+from util import nl2
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -82,60 +85,56 @@ def test_resnet18_full_batch_properties(dev):
     assert all(np.isfinite(v).all() for v in runs[0][1].values())
 
 
-class _RoundingOracleOps(OracleOps):
-    """The fp32 CPU oracle as a model of 16-bit storage: fp32 arithmetic, and every 4-D array
-    (inputs, convolution weights, activations, activation and weight gradients) rounded to the
-    storage type once, where the GPU path stores it."""
-
-    ROUNDED = ("from_numpy", "conv_fwd", "bn_fwd_train", "pool_fwd", "relu", "add", "relu_bwd", "pool_bwd", "bn_bwd",
-               "conv_bwd_x", "conv_bwd_w", "accumulate")
-
-    def __init__(self, kind):
-        self.kind = kind
-
-    def _round(self, a):
-        if isinstance(a, tuple):
-            return tuple(self._round(v) for v in a)
-        if not isinstance(a, np.ndarray) or a.ndim != 4 or a.dtype.kind != "f":
-            return a
-        from singa_amd import singa_wrap as singa
-        if self.kind == "f16":
-            with np.errstate(over="ignore"):
-                return a.astype(np.float16).astype(np.float32)
-        return singa.bf16_bits_to_float(singa.float_to_bf16_bits(a.astype(np.float32))).reshape(a.shape)
-
-    def __getattribute__(self, name):
-        attr = OracleOps.__getattribute__(self, name)
-        if name in _RoundingOracleOps.ROUNDED:
-            return lambda *args, **kw: self._round(attr(*args, **kw))
-        return attr
-
-
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 def test_resnet50_bottleneck_16bit_step(dev, kind):
     """The half-precision configuration on a narrow ResNet-50 (stages [3, 4, 6, 3], widths 16..128,
     64x64 images): 16-bit activations / gradients / convolution weights, fp32 BatchNorm statistics
-    and parameters, fp32 master weights.  The checker is the fp32 oracle with the same rounding
-    points (one rounding per stored tensor), so what remains is the summation order of the kernels
-    and the occasional last-place flip it causes; bound: the per-operation 1e-2 on every gradient
-    and updated parameter of the whole network in binary16; in bfloat16 a flip is 2^-8 and they
-    compound over the 53 layers a gradient crosses, 5e-2 there.  (BatchNorm's d-beta / d-gamma are sums over up to
-    4096 rounded gradients that largely cancel, which amplifies those flips: 3e-2 for them in
-    binary16, 2.5e-1 in bfloat16 with its 8-bit significand (the stem's d-beta, behind all 53 layers,
-    moves between 0.08 and 0.11 with the summation order of the convolution kernels); the kernels themselves are held to the
-    bit in test_gpu_half.py.)"""
+    and parameters, fp32 master weights.
+
+    Error model.  Truth is float64 arithmetic between the tape's rounding points (PyTorch autograd
+    on an independently written graph, one rounding per stored 16-bit tensor; tests/torch_ref.py) on
+    the same stored activations.  The GPU step and the fp32 CPU oracle that rounds at the same
+    points are each measured against it, per gradient and updated parameter, in the normalised L2
+    norm; the BatchNorm parameter gradients, sums of terms that largely cancel, are measured against
+    the sum of |terms|.  Asserted:
+      * the GPU's error is at most twice the oracle's plus one unit roundoff of the storage type
+        (2^-11 / 2^-8): the kernels add nothing beyond what fp32 accumulation order does;
+      * binary16: every tensor within the stated 1e-2;
+      * bfloat16: within 5e-2 -- the oracle itself is 2e-2 from the truth on the first stage's
+        weight gradients, last-place flips of stored bfloat16 gradients compounding over the 53
+        layers behind them (test_tape_vs_torch.py); the 1e-2 bar is held per operation
+        (test_gpu_half.py)."""
     from singa_amd import singa_wrap as singa
     dt = singa.kFloat16 if kind == "f16" else singa.kBFloat16
-    res = wl.run_parity_case("resnet50_small", dev, _RoundingOracleOps(kind), batch=4,
-                             hip_ops=wl.HalfHipOps(dev, dt))
-    bwd = {k: v for k, v in res["errors"].items() if ".grad." in k or ".param." in k}
-    sums = {k: v for k, v in bwd.items() if "bn" in k and (k.endswith(".bias") or k.endswith(".scale"))}
-    rest = {k: v for k, v in bwd.items() if k not in sums}
-    for what, d, tol in (("BN parameter gradients", sums, 3e-2 if kind == "f16" else 2.5e-1),
-                         ("all other tensors", rest, 1e-2 if kind == "f16" else 5e-2)):
-        worst = sorted(d.items(), key=lambda kv: -kv[1])[:4]
-        print(what, "worst:", ", ".join("%s=%.2e" % kv for kv in worst))
-        assert len(d) > 100 and worst[0][1] < tol
+    name, lr, mu = "resnet50_small", 0.05, 0.9
+    hip, orc = wl.HalfHipOps(dev, dt), RoundingOracleOps(kind)
+    gpu, cpu = wl.build(name, hip, lr=lr, momentum=mu), wl.build(name, orc, lr=lr, momentum=mu)
+    x, labels = wl.make_inputs(name, 4)
+    p0 = {k: np.array(p) for k, p in cpu.params()}
+    for k, p in gpu.params():
+        assert np.array_equal(hip.to_numpy(p), p0[k]), k          # both start from the same stored weights
+    losses = [np.asarray(n.ops.to_numpy(n.forward(n.ops.from_numpy(x), n.ops.from_numpy(labels)))) for n in (gpu, cpu)]
+    # (each side's own 53-layer forward pass: not what this test judges -- the 16-bit forward ops are held
+    # to 1e-2 one by one in test_gpu_half.py; here only a sanity bound, the numbers are printed)
+    print(kind, "own forward: loss nl2 %.2e, logits nl2 %.2e" % (nl2(losses[0], losses[1]),
+                                                                 nl2(hip.to_numpy(gpu.logits), cpu.logits)))
+    assert nl2(losses[0], losses[1]) < 1e-1
+    gpu.adopt_saved_tensors(cpu)
+    truth = TorchNet(name, p0, lr, mu, store=store_fn(kind), adopt=saved_inputs(cpu))
+    gpu.backward_and_update(keep_grads=True)
+    cpu.backward_and_update(keep_grads=True)
+    out = truth.step(orc.from_numpy(x), labels)
+    e_gpu = errors_against_truth({k: hip.to_numpy(v) for k, v in gpu.grad_log.items()},
+                                 {k: hip.to_numpy(p) for k, p in gpu.params()}, out, truth.bn_abs, lr)
+    e_cpu = errors_against_truth(cpu.grad_log, dict(cpu.params()), out, truth.bn_abs, lr)
+    assert set(e_gpu) == set(e_cpu) and len(e_gpu) > 300
+    u = UNIT_ROUNDOFF[kind]
+    ratio = sorted(((e_gpu[k] / (2 * e_cpu[k] + u), k) for k in e_gpu), reverse=True)
+    worst = sorted(e_gpu.items(), key=lambda kv: -kv[1])[:4]
+    print(kind, "GPU vs float64 model, worst:", ", ".join("%s=%.2e (oracle %.2e)" % (k, v, e_cpu[k]) for k, v in worst))
+    print(kind, "largest GPU error / (2 x oracle error + u):", ", ".join("%s=%.2f" % (k, r) for r, k in ratio[:4]))
+    assert ratio[0][0] <= 1.0, ratio[:4]
+    assert worst[0][1] < (1e-2 if kind == "f16" else 5e-2), worst
 
 
 @pytest.mark.parametrize("config,kind", [("resnet18_small", "f32"), ("resnet18_small", "f32-sum-in-relu"),
@@ -187,8 +186,8 @@ def test_two_stream_tape_at_full_size(dev, config, batch, kind):
         outs.append([hip.to_numpy(dx)] + [hip.to_numpy(p) for _, p in net.params()])
         del net
     for a, b in zip(*outs):
-        assert np.array_equal(a, b, equal_nan=True)
-    assert all(np.isfinite(a).all() for a in outs[0][1:])
+        assert np.array_equal(a, b)
+    assert all(np.isfinite(a).all() for a in outs[0])     # the input gradient included
 
 
 def test_graph_replay_of_the_step(dev):
