@@ -63,11 +63,23 @@ SGH_API int sgh_device_close(sgh_device *dev);
 SGH_API void *sgh_device_stream(sgh_device *dev);
 /* A second compute stream of the device (default priority, created on first use; NULL on failure),
  * for work that is independent of what the main stream runs next -- a layer's weight gradient
- * beside its data gradient.  No counterpart in the reference (CudaGPU has one stream).  Order it
- * against the main stream with sgh_event_record / sgh_stream_wait_event, and keep every buffer it
- * reads or writes alive until the main stream has waited for it: the pool hands freed blocks out
- * again in the submission order of the MAIN stream only. */
+ * beside its data gradient.  No counterpart in the reference (CudaGPU has one stream).
+ *   sgh_device_fork   work enqueued on the auxiliary stream after this call starts once everything
+ *                     enqueued on the main stream so far has finished; returns the stream.
+ *   sgh_device_join   work enqueued on the main stream after this call starts once everything
+ *                     enqueued on the auxiliary stream so far has finished.
+ *   sgh_block_used_on tells the pool that work on `stream` reads or writes the pool block `ptr`
+ *                     (a pointer sgh_malloc returned).  The pool recycles freed blocks in the
+ *                     submission order of the MAIN stream; a block marked as used on the auxiliary
+ *                     stream may be freed at any time (SINGA's Graph frees a block right after it
+ *                     enqueued the last consumer, src/core/scheduler/scheduler.cc:349-354) and is
+ *                     handed out again only after the next sgh_device_join / sgh_device_sync.
+ *                     A no-op for the main stream; SGH_EINVAL for a foreign stream or pointer.
+ * Memory that did not come from sgh_malloc is the caller's to keep alive until the join. */
 SGH_API void *sgh_device_aux_stream(sgh_device *dev);
+SGH_API int sgh_device_fork(sgh_device *dev, void **aux_stream);
+SGH_API int sgh_device_join(sgh_device *dev);
+SGH_API int sgh_block_used_on(sgh_device *dev, void *ptr, void *stream);
 /* Device::Sync (src/core/device/cuda_gpu.cc:206-209): blocks until the device's streams are idle. */
 SGH_API int sgh_device_sync(sgh_device *dev);
 
@@ -303,8 +315,14 @@ typedef struct sgh_conv_geom {
   int K, R, S;          /* weight [K, C, R, S]                    */
   int stride_h, stride_w, pad_h, pad_w;
   int P, Q;             /* output [N, K, P, Q]                    */
-  int weights_prelaid;  /* set by sgh_conv_dgrad_prepare_multi, cleared by the caller: the workspace
-                           already holds this layer's re-laid weights for the data gradient */
+  /* Owned by the library (sgh_conv_geom_init zeroes them, callers never write them): the note
+   * sgh_conv_dgrad_prepare_multi leaves for this layer's next data gradient -- which weight
+   * tensor was re-laid, into which workspace, and the library's weight epoch at that moment. */
+  int prelaid_dtype;
+  const void *prelaid_W;
+  const void *prelaid_ws;
+  size_t prelaid_ws_bytes;
+  unsigned long long prelaid_epoch;
 } sgh_conv_geom;
 SGH_API int sgh_conv_geom_init(sgh_conv_geom *g, int N, int C, int H, int W, int K, int R, int S,
                                int stride_h, int stride_w, int pad_h, int pad_w);
@@ -319,7 +337,7 @@ SGH_API size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which);
 /* GpuConvBackwardx (src/model/operation/convolution.cc:634-656; native algorithm
  * src/model/layer/convolution.cc:178-182 + Col2im :224-248):
  * dx[n,c,h,w] = sum_{k,r,s} dy[n,k,p,q] * W[k,c,r,s], h = p*stride - pad + r. */
-SGH_API int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx,
+SGH_API int sgh_conv_dgrad_f32(sgh_conv_geom *g, const float *dy, const float *W, float *dx,
                                void *workspace, size_t ws_bytes, void *stream);
 /* dx += the data gradient: cudnnConvolutionBackwardData's beta = 1 (the reference passes beta = 0,
  * convolution.cc:649-654, and sums gradients that fan in with a separate `+=`,
@@ -327,18 +345,25 @@ SGH_API int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const fl
  * value already in dx, so the result equals the separate call followed by `dx_old += result`.
  * Covered by the shared-tile kernels (3x3, pad 1, stride 1, or stride 2 on even images, C >= 64,
  * K a multiple of 16); SGH_EUNSUPPORTED otherwise, with dx untouched. */
-SGH_API int sgh_conv_dgrad_acc_f32(const sgh_conv_geom *g, const float *dy, const float *W,
+SGH_API int sgh_conv_dgrad_acc_f32(sgh_conv_geom *g, const float *dy, const float *W,
                                    float *dx, void *workspace, size_t ws_bytes, void *stream);
 /* The data gradient re-lays the weight tensor in its workspace before the matrix kernel runs:
  * a launch of a few microseconds per layer.  A caller that runs many data gradients while the
  * weights do not change (a backward pass) can have all of them re-laid by ONE launch up front:
- * sgh_conv_dgrad_prepare_multi writes each listed layer's workspace and sets g->weights_prelaid on
- * the layers whose kernel takes such weights (fp32: dtype 0, binary16: 1, bfloat16: 2); the data
- * gradient entry points (sgh_conv_dgrad_*, sgh_conv_dgrad_acc_f32) then skip their own re-layout.
- * Between the prepare call and a layer's data gradient its workspace must not be used by another
- * pass; the caller clears weights_prelaid once the weights change (after the update).  Results
- * are bit-identical with and without.  No counterpart in the reference (cuDNN keeps its filter
- * transforms to itself). */
+ * sgh_conv_dgrad_prepare_multi writes each listed layer's workspace (fp32: dtype 0, binary16: 1,
+ * bfloat16: 2) and leaves a note in the layer's geometry, for the layers whose kernel takes such
+ * weights.  The layer's next data gradient (sgh_conv_dgrad_*, sgh_conv_dgrad_acc_f32) skips its
+ * own re-layout if, and only if, the note still holds: same W pointer, same workspace, and no
+ * call since the prepare that may have changed a weight tensor -- every sgh_sgd_momentum_*,
+ * sgh_axpy_*, sgh_memset_* and host-to-device / device-to-device sgh_memcpy call advances the
+ * library's weight epoch, and so does sgh_conv_weights_changed(), which a caller that writes
+ * weights by other means (its own kernels, a cast into a weight tensor) calls.  Otherwise the data gradient re-lays the weights
+ * itself, as without a prepare.  A note is used once: the data gradient that reads it, and any
+ * forward pass or weight gradient of the same geometry whose workspace overlaps the prepared one,
+ * removes it.  The workspaces listed must be private to their layer from the prepare call to the
+ * layer's data gradient (a workspace shared between layers cannot hold two layers' weights).
+ * Results are bit-identical with and without.  No counterpart in the reference (cuDNN keeps its
+ * filter transforms to itself). */
 typedef struct sgh_conv_prepare_item {
   sgh_conv_geom *g;
   const void *W;
@@ -347,17 +372,18 @@ typedef struct sgh_conv_prepare_item {
 } sgh_conv_prepare_item;
 SGH_API int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, int dtype,
                                          void *stream);
+SGH_API void sgh_conv_weights_changed(void);
 /* GpuConvBackwardW (src/model/operation/convolution.cc:658-681; native algorithm
  * src/model/layer/convolution.cc:166-177 + Im2col :197-222):
  * dW[k,c,r,s] = sum_{n,p,q} dy[n,k,p,q] * x[n,c,p*stride-pad+r,q*stride-pad+s].
  * The split reduction is summed in a fixed order: results are run-to-run identical. */
-SGH_API int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, float *dW,
+SGH_API int sgh_conv_wgrad_f32(sgh_conv_geom *g, const float *dy, const float *x, float *dW,
                                void *workspace, size_t ws_bytes, void *stream);
 /* GpuConvBackwardb (src/model/operation/convolution.cc:684-702; native CPU :425-440):
  * db[k] = sum_{n,p,q} dy[n,k,p,q]. */
 SGH_API int sgh_conv_bgrad_f32(const sgh_conv_geom *g, const float *dy, float *db, void *stream);
 /* GpuConvForward (src/model/operation/convolution.cc:585-632); bias may be NULL. */
-SGH_API int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W,
+SGH_API int sgh_conv_fwd_f32(sgh_conv_geom *g, const float *x, const float *W,
                              const float *bias, float *y, void *workspace, size_t ws_bytes,
                              void *stream);
 
@@ -370,20 +396,20 @@ SGH_API int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float
  * tensors; other geometries widen the operands to fp32 in the workspace and use the fp32 kernels.
  * Workspace: sgh_conv_workspace_bytes_h(g, which) bytes. */
 SGH_API size_t sgh_conv_workspace_bytes_h(const sgh_conv_geom *g, int which);
-SGH_API int sgh_conv_dgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W,
+SGH_API int sgh_conv_dgrad_f16(sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W,
                                uint16_t *dx, void *workspace, size_t ws_bytes, void *stream);
-SGH_API int sgh_conv_dgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W,
+SGH_API int sgh_conv_dgrad_bf16(sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W,
                                 uint16_t *dx, void *workspace, size_t ws_bytes, void *stream);
-SGH_API int sgh_conv_wgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x,
+SGH_API int sgh_conv_wgrad_f16(sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x,
                                uint16_t *dW, void *workspace, size_t ws_bytes, void *stream);
-SGH_API int sgh_conv_wgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x,
+SGH_API int sgh_conv_wgrad_bf16(sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x,
                                 uint16_t *dW, void *workspace, size_t ws_bytes, void *stream);
 SGH_API int sgh_conv_bgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db, void *stream);
 SGH_API int sgh_conv_bgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db, void *stream);
-SGH_API int sgh_conv_fwd_f16(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W,
+SGH_API int sgh_conv_fwd_f16(sgh_conv_geom *g, const uint16_t *x, const uint16_t *W,
                              const uint16_t *bias, uint16_t *y, void *workspace, size_t ws_bytes,
                              void *stream);
-SGH_API int sgh_conv_fwd_bf16(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W,
+SGH_API int sgh_conv_fwd_bf16(sgh_conv_geom *g, const uint16_t *x, const uint16_t *W,
                               const uint16_t *bias, uint16_t *y, void *workspace, size_t ws_bytes,
                               void *stream);
 

@@ -19,7 +19,8 @@ class ConvGeom(C.Structure):
     """``sgh_conv_geom``"""
     _fields_ = [(n, C.c_int) for n in
                 ("N", "C", "H", "W", "K", "R", "S", "stride_h", "stride_w", "pad_h", "pad_w", "P", "Q",
-                 "weights_prelaid")]
+                 "prelaid_dtype")] + [("prelaid_W", C.c_void_p), ("prelaid_ws", C.c_void_p),
+                                      ("prelaid_ws_bytes", C.c_size_t), ("prelaid_epoch", C.c_ulonglong)]
 
 
 class ConvPrepareItem(C.Structure):
@@ -55,6 +56,9 @@ SIGNATURES = {
     "sgh_device_stream": (vp, [vp]),
     "sgh_device_aux_stream": (vp, [vp]),
     "sgh_device_sync": (C.c_int, [vp]),
+    "sgh_device_fork": (C.c_int, [vp, C.POINTER(vp)]),
+    "sgh_device_join": (C.c_int, [vp]),
+    "sgh_block_used_on": (C.c_int, [vp, vp, vp]),
     "sgh_malloc": (C.c_int, [vp, C.POINTER(vp), sz]),
     "sgh_free": (C.c_int, [vp, vp]),
     "sgh_pool_stats": (C.c_int, [vp, C.POINTER(sz), C.POINTER(sz), C.POINTER(sz)]),
@@ -133,6 +137,7 @@ SIGNATURES = {
     "sgh_conv_fwd_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
     "sgh_conv_workspace_bytes_h": (sz, [C.POINTER(ConvGeom), C.c_int]),
     "sgh_conv_dgrad_prepare_multi": (C.c_int, [C.POINTER(ConvPrepareItem), C.c_int, C.c_int, vp]),
+    "sgh_conv_weights_changed": (None, []),
     "sgh_conv_dgrad_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_dgrad_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_wgrad_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),

@@ -28,6 +28,16 @@ static inline hipStream_t sgh_stream_of(void *s) { return reinterpret_cast<hipSt
 
 static inline bool sgh_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// The library's environment switches (A/B measurements; none is needed in normal use), read ONCE,
+// when the first entry point asks: changing the environment later has no effect, so a geometry's
+// workspace size and kernel choice cannot change between two calls.
+struct sgh_env_switches {
+  bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off;
+  int dgrad_tile, wgrad_tile;   // -1: chosen from the geometry
+  int dgrad3x3_bm;              // 0: chosen from the geometry, else 64 or 128
+};
+const sgh_env_switches &sgh_env();
+
 // Number of compute units of the current device (cached per process; one GPU per process).
 int sgh_num_cus();
 
@@ -35,6 +45,18 @@ int sgh_num_cus();
 // sgh_bn_bwd_noalloc_f32 (batchnorm.hip).  sgh_device_open calls it so that the entry point's first
 // call on a device finds the address ready; the entry point repeats the lookup if it was not.
 int sgh_bn_noalloc_setup();
+
+// Weight epoch: a host-side counter that every entry point which may change a weight tensor advances
+// (optimizer updates, Axpy, fills, casts, copies to the device, sgh_conv_weights_changed).  The note that
+// sgh_conv_dgrad_prepare_multi leaves in a geometry is honoured only within the epoch it was written in.
+unsigned long long sgh_weights_epoch();
+void sgh_weights_epoch_bump();
+// True when the note in `g` covers a data gradient of storage type `dtype` (0 fp32, 1 binary16, 2 bfloat16)
+// reading weights `W` with workspace `workspace` now.
+bool sgh_prelaid_valid(const sgh_conv_geom *g, int dtype, const void *W, const void *workspace);
+void sgh_prelaid_clear(sgh_conv_geom *g);
+// Removes the note if [workspace, workspace + ws_bytes) overlaps the prepared workspace (a pass that writes there).
+void sgh_prelaid_clear_if_overlap(sgh_conv_geom *g, const void *workspace, size_t ws_bytes);
 
 // Kernel-level profiling hooks (no-ops unless sgh_prof_enable(1) was called).
 bool sgh_prof_on();
@@ -80,10 +102,10 @@ size_t sgh_conv16_workspace_bytes(const sgh_conv_geom *g, int which);
 int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x, uint16_t *dW, void *workspace,
                      size_t ws_bytes, bool bf16, hipStream_t s);
 int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
-                     size_t ws_bytes, bool bf16, hipStream_t s);
+                     size_t ws_bytes, bool bf16, hipStream_t s, bool prelaid);
 // Data-gradient weight re-layout of conv16.hip as a batch item: false when the geometry is not covered;
-// otherwise the destination layout [tap][CP][KP] (sgh_conv16_dgrad skips its re-layout when
-// g->weights_prelaid is set).
+// otherwise the destination layout [tap][CP][KP] (sgh_conv16_dgrad skips its re-layout when told that the
+// workspace already holds it).
 bool sgh_conv16_dgrad_relayout_dims(const sgh_conv_geom *g, int *CP, int *KP);
 int sgh_conv16_fwd(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
                    void *workspace, size_t ws_bytes, bool bf16, hipStream_t s);

@@ -858,7 +858,8 @@ namespace {
 // `fwd_of`: null for the data gradient of g; otherwise g is the twin (see fwd_twin) of the forward
 // geometry *fwd_of, W is that convolution's weight tensor and `bias` its bias (or null)
 int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t *dy, const uint16_t *W,
-            const uint16_t *bias, uint16_t *dx, void *workspace, size_t ws_bytes, bool bf16, hipStream_t s, int fs = 1) {
+            const uint16_t *bias, uint16_t *dx, void *workspace, size_t ws_bytes, bool bf16, hipStream_t s, int fs = 1,
+            bool prelaid = false) {
   const D16Plan p = dplan(g, fs);
   if (!p.ok) return SGH_EUNSUPPORTED;
   const int RS = g->R * g->S;
@@ -873,7 +874,7 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
     else hipLaunchKernelGGL(k_pixel_major16<false>, grid, dim3(256), 0, s, dy, dyT, g->K, PQ);
     if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
   }
-  if (!fwd_of && g->weights_prelaid) {
+  if (!fwd_of && prelaid) {
     // re-laid by sgh_conv_dgrad_prepare_multi
   } else if (fwd_of)
     hipLaunchKernelGGL(k_relayout16_fwd, dim3(unsigned((nw + 255) / 256)), dim3(256), 0, s, W, wt, fwd_of->K, fwd_of->C,
@@ -917,8 +918,8 @@ bool sgh_conv16_dgrad_relayout_dims(const sgh_conv_geom *g, int *CP, int *KP) {
 }
 
 int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
-                     size_t ws_bytes, bool bf16, hipStream_t s) {
-  return run_d16(g, nullptr, dy, W, nullptr, dx, workspace, ws_bytes, bf16, s);
+                     size_t ws_bytes, bool bf16, hipStream_t s, bool prelaid) {
+  return run_d16(g, nullptr, dy, W, nullptr, dx, workspace, ws_bytes, bf16, s, 1, prelaid);
 }
 
 int sgh_conv16_fwd(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,

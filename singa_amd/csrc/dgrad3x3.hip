@@ -369,7 +369,7 @@ inline D3Plan plan(const sgh_conv_geom *g) {
   if (g->stride_h != 1 && !p.s2) return p;
   if (p.s2 && (g->H != 2 * g->P || g->W != 2 * g->Q)) return p;  // even image: four residue classes of equal size
   if (g->C < 64 || g->C % 4 != 0 || g->K % KC != 0 || g->Q < 2) return p;
-  if (getenv("SGH_DGRAD3X3_OFF")) return p;
+  if (sgh_env().dgrad3x3_off) return p;
   // slab columns: stride 1 has a halo column on both sides, stride 2 one zero column on the right
   const int cols = p.s2 ? g->Q + 1 : g->Q + 2;
   if (cols > 64) return p;
@@ -390,7 +390,7 @@ inline D3Plan plan(const sgh_conv_geom *g) {
     else if (p.logp == 5) p.vr = 16;
     else p.vr = need <= 16 ? 16 : 32;
     p.bm = (g->C % 128 == 0 || g->C > 192) ? 128 : 64;
-    if (const char *e = getenv("SGH_DGRAD3X3_BM")) p.bm = atoi(e) == 64 ? 64 : 128;
+    if (sgh_env().dgrad3x3_bm) p.bm = sgh_env().dgrad3x3_bm;
   }
   if (need > p.vr) return p;
   const size_t chs = size_t(p.vr) * (1u << p.logp);

@@ -215,7 +215,7 @@ inline bool offset_range(int R, int pad, int *d0, int *cnt) {
 inline DFPlan plan(const sgh_conv_geom *g) {
   DFPlan p{};
   p.ok = false;
-  if (getenv("SGH_DGRAD_FEWC_OFF")) return p;
+  if (sgh_env().dgrad_fewc_off) return p;
   if (g->stride_h != 2 || g->stride_w != 2 || g->C > 4) return p;
   if (g->H != 2 * g->P || g->W != 2 * g->Q) return p;          // even image: 2x2 output blocks tile it exactly
   if (g->K % KC != 0 || g->Q % 4 != 0 || g->Q > 128 || g->Q < 4) return p;

@@ -509,15 +509,18 @@ int sgh_eltwise_mult_f32(const float *a, const float *b, int b_is_scalar, float 
 }
 
 int sgh_axpy_f32(float alpha, const float *x, float *y, size_t n, void *stream) {
+  sgh_weights_epoch_bump();
   return launch_map2(x, y, y, n, AxpyOp{alpha}, stream);
 }
 
 int sgh_axpy_devalpha_f32(const float *alpha_dev, const float *x, float *y, size_t n, void *stream) {
+  sgh_weights_epoch_bump();
   if (n != 0 && !alpha_dev) return SGH_EINVAL;
   return launch_map2(x, y, y, n, AxpyDevOp{alpha_dev}, stream);
 }
 
 int sgh_memset_f32(float *dst, float value, size_t n, void *stream) {
+  sgh_weights_epoch_bump();
   if (n == 0) return SGH_OK;
   if (!dst) return SGH_EINVAL;
   hipLaunchKernelGGL(k_fill, dim3(grid_for(n)), dim3(kBlock), 0, sgh_stream_of(stream), dst, value, n);
@@ -544,11 +547,13 @@ static int sgd_launch(float *p, const float *g, float *v, size_t n, SgdHyper h, 
 
 int sgh_sgd_momentum_f32(float *p, const float *g, float *v, size_t n, float lr, float mu, float damp, float wd,
                          int nesterov, void *stream) {
+  sgh_weights_epoch_bump();
   return sgd_launch(p, g, v, n, SgdHyper{lr, mu, damp, wd}, nullptr, nesterov, mu != 0.f, stream);
 }
 
 int sgh_sgd_momentum_devhyper_f32(float *p, const float *g, float *v, size_t n, const float *hyper_dev, int nesterov,
                                   void *stream) {
+  sgh_weights_epoch_bump();
   if (!hyper_dev) return SGH_EINVAL;
   // mu lives on the device: a NULL v is only legal if mu turns out to be 0, which the kernel checks
   return sgd_launch(p, g, v, n, SgdHyper{0, 0, 0, 0}, hyper_dev, nesterov, false, stream);
@@ -556,6 +561,7 @@ int sgh_sgd_momentum_devhyper_f32(float *p, const float *g, float *v, size_t n, 
 
 int sgh_sgd_momentum_multi_f32(const sgh_sgd_item *table_dev, int count, size_t total_n, float lr, float mu, float damp,
                                float wd, int nesterov, void *stream) {
+  sgh_weights_epoch_bump();
   if (count == 0 || total_n == 0) return SGH_OK;
   if (!table_dev || count < 0) return SGH_EINVAL;
   size_t chunks = total_n / kChunk + size_t(count);  // upper bound on sum of per-item chunk counts

@@ -381,14 +381,17 @@ uint16_t host_f32_to_f16(float f) {
 extern "C" {
 
 int sgh_memset_f16(uint16_t *dst, float value, size_t n, void *stream) {
+  sgh_weights_epoch_bump();
   return fill16(dst, host_f32_to_f16(value), n, stream);
 }
 int sgh_memset_bf16(uint16_t *dst, float value, size_t n, void *stream) {
+  sgh_weights_epoch_bump();
   return fill16(dst, host_f32_to_bf16(value), n, stream);
 }
 
 int sgh_sgd_momentum_multi_mixed(const sgh_sgd_mixed_item *table_dev, int count, size_t total_n, int bf16, float lr,
                                  float mu, float damp, float wd, int nesterov, void *stream) {
+  sgh_weights_epoch_bump();
   if (count == 0) return SGH_OK;
   if (!table_dev || count < 0 || count > kMixTab) return SGH_EINVAL;
   size_t chunks = total_n / kMixChunk + size_t(count);  // upper bound on the sum of per-item chunk counts
@@ -403,18 +406,22 @@ int sgh_sgd_momentum_multi_mixed(const sgh_sgd_mixed_item *table_dev, int count,
 
 int sgh_sgd_momentum_f16(uint16_t *p, const uint16_t *g, uint16_t *v, size_t n, float lr, float mu, float damp,
                          float wd, int nesterov, void *stream) {
+  sgh_weights_epoch_bump();
   return sgd_h<F16, false>(p, g, v, nullptr, nullptr, n, lr, mu, damp, wd, nesterov, stream);
 }
 int sgh_sgd_momentum_bf16(uint16_t *p, const uint16_t *g, uint16_t *v, size_t n, float lr, float mu, float damp,
                           float wd, int nesterov, void *stream) {
+  sgh_weights_epoch_bump();
   return sgd_h<BF16, false>(p, g, v, nullptr, nullptr, n, lr, mu, damp, wd, nesterov, stream);
 }
 int sgh_sgd_momentum_master_f16(float *p_master, const uint16_t *g, float *v, uint16_t *p_out, size_t n, float lr,
                                 float mu, float damp, float wd, int nesterov, void *stream) {
+  sgh_weights_epoch_bump();
   return sgd_h<F16, true>(p_out, g, nullptr, p_master, v, n, lr, mu, damp, wd, nesterov, stream);
 }
 int sgh_sgd_momentum_master_bf16(float *p_master, const uint16_t *g, float *v, uint16_t *p_out, size_t n, float lr,
                                  float mu, float damp, float wd, int nesterov, void *stream) {
+  sgh_weights_epoch_bump();
   return sgd_h<BF16, true>(p_out, g, nullptr, p_master, v, n, lr, mu, damp, wd, nesterov, stream);
 }
 
@@ -454,9 +461,11 @@ int sgh_eltwise_mult_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, s
   return launch_map2_h<BF16>(a, b, out, n, MulOp{}, stream);
 }
 int sgh_axpy_f16(float alpha, const uint16_t *x, uint16_t *y, size_t n, void *stream) {
+  sgh_weights_epoch_bump();
   return launch_map2_h<F16>(x, y, y, n, AxpyOp{alpha}, stream);
 }
 int sgh_axpy_bf16(float alpha, const uint16_t *x, uint16_t *y, size_t n, void *stream) {
+  sgh_weights_epoch_bump();
   return launch_map2_h<BF16>(x, y, y, n, AxpyOp{alpha}, stream);
 }
 

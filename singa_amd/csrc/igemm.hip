@@ -737,13 +737,10 @@ inline WgradPlan plan_wgrad(const sgh_conv_geom *g) {
   // 576 = 64 channels x 9 taps is exactly three 192-wide tiles (a 128- or 256-wide tile would
   // spend 10 % / 25 % of its MFMAs on padding columns)
   if (p.bm == 64 && CRS % 192 == 0 && CRS % 256 != 0) p.bn = 192;
-  if (const char *e = getenv("SGH_WGRAD_TILE")) {
-    const int v = atoi(e);
+  if (sgh_env().wgrad_tile >= 0) {
     static const int bm[6] = {128, 64, 128, 64, 64, 64}, bn[6] = {128, 128, 64, 64, 256, 192};
-    if (v >= 0 && v <= 5) {
-      p.bm = bm[v];
-      p.bn = bn[v];
-    }
+    p.bm = bm[sgh_env().wgrad_tile];
+    p.bn = bn[sgh_env().wgrad_tile];
   }
   const long tiles = long((g->K + p.bm - 1) / p.bm) * ((CRS + p.bn - 1) / p.bn);
   const long G = long(g->N) * g->P * g->Q;
@@ -802,11 +799,8 @@ inline int gemm_pick(int M, int N, int K, float alpha, const float *A, long a_rs
 // problem takes the smallest tile.  An environment variable (value 0..3) overrides the choice,
 // the counterpart of the reference's CUDNN_CONV_ALG switch
 // (reference: src/model/operation/convolution.cc:453-457).
-inline int pick_tile(const char *env, int M, int N, int z) {
-  if (const char *e = getenv(env)) {
-    const int v = atoi(e);
-    if (v >= 0 && v <= 3) return v;
-  }
+inline int pick_tile(int forced, int M, int N, int z) {
+  if (forced >= 0) return forced;
   static const int bm[4] = {128, 64, 128, 64}, bn[4] = {128, 128, 64, 64};
   const long want = 2L * sgh_num_cus();
   for (int i = 0; i < 4; ++i) {
@@ -826,7 +820,7 @@ inline DgradPath dgrad_path(const sgh_conv_geom *g) {
   // at most four input channels, stride 2, large filter (the stem): direct 16-row MFMA kernel
   if (sgh_dgrad_fewc_supported(g)) return kDgradFewC;
   // 1x1 without padding: a plain GEMM over the output pixels whose store dilates by the stride
-  if (RS == 1 && g->pad_h == 0 && g->pad_w == 0 && g->C >= 32 && !getenv("SGH_DGRAD_POINTWISE_OFF"))
+  if (RS == 1 && g->pad_h == 0 && g->pad_w == 0 && g->C >= 32 && !sgh_env().dgrad_pointwise_off)
     return kDgradPointwise;
   // few input channels: the C x pixels output tile would waste most of a 64-row MFMA tile, so run
   // the dense GEMM dcol = W^T * dy (CRS rows) and fold the columns back with a gather
@@ -874,7 +868,7 @@ int sgh_conv_geom_init(sgh_conv_geom *g, int N, int C, int H, int W, int K, int 
   // ConvHandle's integer division (reference: src/model/operation/convolution.cc:56-59)
   g->P = (H + 2 * pad_h - R) / stride_h + 1;
   g->Q = (W + 2 * pad_w - S) / stride_w + 1;
-  g->weights_prelaid = 0;
+  sgh_prelaid_clear(g);
   return conv_ok(g) ? SGH_OK : SGH_EINVAL;
 }
 
@@ -905,8 +899,9 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
   }
 }
 
+// `prelaid`: the workspace already holds this layer's re-laid weights (sgh_conv_dgrad_prepare_multi)
 static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
-                      size_t ws_bytes, void *stream, bool accumulate) {
+                      size_t ws_bytes, void *stream, bool accumulate, bool prelaid) {
   if (!conv_ok(g) || !dy || !W || !dx) return SGH_EINVAL;
   const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_DGRAD);
   if (need && (!workspace || ws_bytes < need)) return SGH_EWORKSPACE;
@@ -966,7 +961,7 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     const long total = long(RS) * KP * g->C;
     long blocks = (total + NT - 1) / NT;
     if (blocks > 4096) blocks = 4096;
-    if (!g->weights_prelaid)
+    if (!prelaid)
       hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
     float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) +
                                                 align256(size_t(RS) * KP * g->C * sizeof(float)) +
@@ -1014,7 +1009,7 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     }
     const int M = g->C;
     DgradStore st{dx, to_g(g), tab_dev};
-    const int tile = pick_tile("SGH_DGRAD_TILE", M, max_cols, ncls);
+    const int tile = pick_tile(sgh_env().dgrad_tile, M, max_cols, ncls);
 #define SGH_DGRAD_CASE(BM_, BN_)                                                                              \
   {                                                                                                           \
     DgradWLoader<BM_> la{Wc, g->C, KP, tab_dev, unsigned(wc_bytes), 0, 0, 0, 0};                              \
@@ -1037,7 +1032,7 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     const long total = long(RS) * KP * g->C;
     long blocks = (total + NT - 1) / NT;
     if (blocks > 4096) blocks = 4096;
-    if (!g->weights_prelaid)
+    if (!prelaid)
       hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, KP, 1);
     const int M = g->C, Ncols = g->N * g->H * g->W, Ktot = RS * KP;
     NchwStore st{dx, nullptr, g->C, g->H * g->W, Ncols};
@@ -1052,10 +1047,21 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
   return SGH_OK;
 }
 
-int sgh_conv_dgrad_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
-                       size_t ws_bytes, void *stream) {
-  return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, false);
+// The note of a prepare call is read once: whether it held or not, this pass leaves none behind.
+static bool take_prelaid(sgh_conv_geom *g, int dtype, const void *W, const void *workspace) {
+  if (!g) return false;
+  const bool ok = sgh_prelaid_valid(g, dtype, W, workspace);
+  sgh_prelaid_clear(g);
+  return ok;
 }
+
+int sgh_conv_dgrad_f32(sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
+                       size_t ws_bytes, void *stream) {
+  const bool prelaid = take_prelaid(g, 0, W, workspace);
+  return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, false, prelaid);
+}
+
+void sgh_conv_weights_changed(void) { sgh_weights_epoch_bump(); }
 
 // ---- all data-gradient weight re-layouts of a backward pass in one launch ----------------------
 namespace {
@@ -1148,19 +1154,24 @@ int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, 
   RelayoutTable t;
   t.count = 0, t.block0[0] = 0;
   sgh_conv_geom *batch[kMaxRelayouts];
+  size_t batch_bytes[kMaxRelayouts];
   auto flush = [&]() -> int {
     if (t.count == 0) return SGH_OK;
     if (dtype == 0) hipLaunchKernelGGL(k_weight_relayout_multi<float>, dim3(unsigned(t.block0[t.count])), dim3(NT), 0, s, t);
     else hipLaunchKernelGGL(k_weight_relayout_multi<uint16_t>, dim3(unsigned(t.block0[t.count])), dim3(NT), 0, s, t);
     if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
-    for (int i = 0; i < t.count; ++i) batch[i]->weights_prelaid = 1;
+    for (int i = 0; i < t.count; ++i) {
+      sgh_conv_geom *g = batch[i];
+      g->prelaid_dtype = dtype, g->prelaid_W = t.it[i].W, g->prelaid_ws = t.it[i].Wt;
+      g->prelaid_ws_bytes = batch_bytes[i], g->prelaid_epoch = sgh_weights_epoch();
+    }
     t.count = 0;
     return SGH_OK;
   };
   for (int i = 0; i < count; ++i) {
     sgh_conv_geom *g = items[i].g;
     if (!g || !conv_ok(g) || !items[i].W) return SGH_EINVAL;
-    g->weights_prelaid = 0;
+    sgh_prelaid_clear(g);
     RelayoutTable::Item it{};
     it.W = items[i].W, it.Wt = items[i].workspace, it.K = g->K, it.C = g->C, it.RS = g->R * g->S;
     size_t need;
@@ -1170,7 +1181,7 @@ int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, 
       it.A = round_up(g->K, BK), it.B = g->C;
       need = sgh_conv_workspace_bytes(g, SGH_CONV_DGRAD);
     } else {
-      if (getenv("SGH_CONV16_OFF") || !sgh_conv16_dgrad_relayout_dims(g, &it.A, &it.B)) continue;
+      if (sgh_env().conv16_off || !sgh_conv16_dgrad_relayout_dims(g, &it.A, &it.B)) continue;
       need = sgh_conv16_workspace_bytes(g, SGH_CONV_DGRAD);
     }
     if (!items[i].workspace || items[i].ws_bytes < need) return SGH_EWORKSPACE;
@@ -1184,20 +1195,24 @@ int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, 
     }
     t.it[t.count] = it;
     batch[t.count] = g;
+    batch_bytes[t.count] = items[i].ws_bytes;
     t.block0[t.count + 1] = t.block0[t.count] + int(blocks);
     ++t.count;
   }
   return flush();
 }
 
-int sgh_conv_dgrad_acc_f32(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
+int sgh_conv_dgrad_acc_f32(sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
                            size_t ws_bytes, void *stream) {
-  return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, true);
+  if (g && conv_ok(g) && dgrad_path(g) != kDgradTile3x3) return SGH_EUNSUPPORTED;   // (the note stays for the fallback call)
+  const bool prelaid = take_prelaid(g, 0, W, workspace);
+  return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, true, prelaid);
 }
 
-int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, const float *bias, float *y,
+int sgh_conv_fwd_f32(sgh_conv_geom *g, const float *x, const float *W, const float *bias, float *y,
                      void *workspace, size_t ws_bytes, void *stream) {
   if (!conv_ok(g) || !x || !W || !y) return SGH_EINVAL;
+  sgh_prelaid_clear_if_overlap(g, workspace, ws_bytes);
   const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_FWD);
   if (!workspace || ws_bytes < need) return SGH_EWORKSPACE;
   hipStream_t s = sgh_stream_of(stream);
@@ -1243,9 +1258,10 @@ int sgh_conv_fwd_f32(const sgh_conv_geom *g, const float *x, const float *W, con
   return SGH_OK;
 }
 
-int sgh_conv_wgrad_f32(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
+int sgh_conv_wgrad_f32(sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
                        size_t ws_bytes, void *stream) {
   if (!conv_ok(g) || !dy || !x || !dW) return SGH_EINVAL;
+  sgh_prelaid_clear_if_overlap(g, workspace, ws_bytes);
   if (sgh_wgrad3x3_workspace_bytes(g)) {  // 3x3, stride 1 or 2: shared-input-tile kernel
     sgh_prof_start("conv_wgrad_op", conv_flops(g), sgh_stream_of(stream));
     const int rc3 = sgh_wgrad3x3_run(g, dy, x, dW, workspace, ws_bytes, sgh_stream_of(stream));
@@ -1361,22 +1377,25 @@ typedef int (*cast_in_fn)(const uint16_t *, float *, size_t, void *);
 typedef int (*cast_out_fn)(const float *, uint16_t *, size_t, void *);
 
 // which: SGH_CONV_*; (a, b) are the pass's two tensor inputs in the order of its fp32 entry point
-int conv_half(const sgh_conv_geom *g, int which, const uint16_t *a, const uint16_t *b, const uint16_t *bias,
+int conv_half(sgh_conv_geom *g, int which, const uint16_t *a, const uint16_t *b, const uint16_t *bias,
               uint16_t *out, void *workspace, size_t ws_bytes, void *stream, cast_in_fn in, cast_out_fn outc) {
   if (!conv_ok(g) || !a || !b || !out) return SGH_EINVAL;
+  bool prelaid = false;
+  if (which == SGH_CONV_DGRAD) prelaid = take_prelaid(g, in == sgh_cast_bf16_to_f32 ? 2 : 1, b, workspace);
+  else sgh_prelaid_clear_if_overlap(g, workspace, ws_bytes);
   // the gradients and the forward pass (strides 1 and 2) run on the 16-bit matrix instructions where
   // conv16.hip covers the geometry; everything else computes in fp32 on widened copies
-  if (sgh_conv16_workspace_bytes(g, which) != 0 && !getenv("SGH_CONV16_OFF")) {
+  if (sgh_conv16_workspace_bytes(g, which) != 0 && !sgh_env().conv16_off) {
     const bool bf16 = in == sgh_cast_bf16_to_f32;
     hipStream_t s = sgh_stream_of(stream);
-    const int rc = which == SGH_CONV_DGRAD   ? sgh_conv16_dgrad(g, a, b, out, workspace, ws_bytes, bf16, s)
+    const int rc = which == SGH_CONV_DGRAD   ? sgh_conv16_dgrad(g, a, b, out, workspace, ws_bytes, bf16, s, prelaid)
                    : which == SGH_CONV_WGRAD ? sgh_conv16_wgrad(g, a, b, out, workspace, ws_bytes, bf16, s)
                                              : sgh_conv16_fwd(g, a, b, bias, out, workspace, ws_bytes, bf16, s);
     if (rc != SGH_EUNSUPPORTED) return rc;
   }
   // the stem's data gradient (few input channels, large filter): the fp32 kernel reads the 16-bit
   // gradient and writes the 16-bit result itself; only the small weight tensor is widened
-  if (which == SGH_CONV_DGRAD && sgh_dgrad_fewc_supported(g) && !getenv("SGH_CONV16_OFF")) {
+  if (which == SGH_CONV_DGRAD && sgh_dgrad_fewc_supported(g) && !sgh_env().conv16_off) {
     const size_t w_elems = size_t(g->K) * g->C * g->R * g->S, w_bytes = align256(w_elems * 4);
     if (!workspace || ws_bytes < w_bytes + sgh_dgrad_fewc_workspace_bytes(g)) return SGH_EWORKSPACE;
     float *w32 = static_cast<float *>(workspace);
@@ -1432,32 +1451,32 @@ size_t sgh_conv_workspace_bytes_h(const sgh_conv_geom *g, int which) {
   return wide > native ? wide : native;
 }
 
-int sgh_conv_dgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
+int sgh_conv_dgrad_f16(sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
                        size_t ws_bytes, void *stream) {
   return conv_half(g, SGH_CONV_DGRAD, dy, W, nullptr, dx, workspace, ws_bytes, stream, sgh_cast_f16_to_f32,
                    sgh_cast_f32_to_f16);
 }
-int sgh_conv_dgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
+int sgh_conv_dgrad_bf16(sgh_conv_geom *g, const uint16_t *dy, const uint16_t *W, uint16_t *dx, void *workspace,
                         size_t ws_bytes, void *stream) {
   return conv_half(g, SGH_CONV_DGRAD, dy, W, nullptr, dx, workspace, ws_bytes, stream, sgh_cast_bf16_to_f32,
                    sgh_cast_f32_to_bf16);
 }
-int sgh_conv_wgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x, uint16_t *dW, void *workspace,
+int sgh_conv_wgrad_f16(sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x, uint16_t *dW, void *workspace,
                        size_t ws_bytes, void *stream) {
   return conv_half(g, SGH_CONV_WGRAD, dy, x, nullptr, dW, workspace, ws_bytes, stream, sgh_cast_f16_to_f32,
                    sgh_cast_f32_to_f16);
 }
-int sgh_conv_wgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x, uint16_t *dW, void *workspace,
+int sgh_conv_wgrad_bf16(sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x, uint16_t *dW, void *workspace,
                         size_t ws_bytes, void *stream) {
   return conv_half(g, SGH_CONV_WGRAD, dy, x, nullptr, dW, workspace, ws_bytes, stream, sgh_cast_bf16_to_f32,
                    sgh_cast_f32_to_bf16);
 }
-int sgh_conv_fwd_f16(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
+int sgh_conv_fwd_f16(sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
                      void *workspace, size_t ws_bytes, void *stream) {
   return conv_half(g, SGH_CONV_FWD, x, W, bias, y, workspace, ws_bytes, stream, sgh_cast_f16_to_f32,
                    sgh_cast_f32_to_f16);
 }
-int sgh_conv_fwd_bf16(const sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
+int sgh_conv_fwd_bf16(sgh_conv_geom *g, const uint16_t *x, const uint16_t *W, const uint16_t *bias, uint16_t *y,
                       void *workspace, size_t ws_bytes, void *stream) {
   return conv_half(g, SGH_CONV_FWD, x, W, bias, y, workspace, ws_bytes, stream, sgh_cast_bf16_to_f32,
                    sgh_cast_f32_to_bf16);

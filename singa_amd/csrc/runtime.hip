@@ -1,6 +1,9 @@
 // Device runtime behind the C ABI: one stream + one caching memory pool per opened device.
 // Mirrors what SINGA's CudaGPU + DeviceMemPool give the Tensor layer
 // (reference: src/core/device/cuda_gpu.cc:56-209, src/core/memory/memory.cc:32-118).
+#include <stdlib.h>
+
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <new>
@@ -15,6 +18,11 @@ struct sgh_device {
   hipStream_t stream = nullptr;
   hipStream_t side = nullptr;  // uploads that must happen while `stream` is recording
   hipStream_t aux = nullptr;   // second compute stream (sgh_device_aux_stream), created on first use
+  hipEvent_t fork_ev = nullptr, join_ev = nullptr;
+  // blocks that work on the auxiliary stream uses (sgh_block_used_on): when freed they wait in
+  // `pending` until the main stream has been ordered behind the auxiliary one (join / sync)
+  std::unordered_set<void *> on_aux;
+  std::vector<std::pair<void *, size_t>> pending;
   std::mutex mu;
   // free blocks keyed by their (rounded) size; blocks in use keyed by address
   std::multimap<size_t, void *> free_blocks;
@@ -52,6 +60,51 @@ int sgh_num_cus() {
   else
     g_num_cus = 256;
   return g_num_cus;
+}
+
+const sgh_env_switches &sgh_env() {
+  static const sgh_env_switches e = [] {
+    auto on = [](const char *n) { return getenv(n) != nullptr; };
+    auto num = [](const char *n, int lo, int hi) {
+      const char *v = getenv(n);
+      if (!v) return -1;
+      const int x = atoi(v);
+      return x >= lo && x <= hi ? x : -1;
+    };
+    sgh_env_switches s{};
+    s.dgrad3x3_off = on("SGH_DGRAD3X3_OFF"), s.wgrad3x3_off = on("SGH_WGRAD3X3_OFF");
+    s.dgrad_fewc_off = on("SGH_DGRAD_FEWC_OFF"), s.wgrad_fewc_off = on("SGH_WGRAD_FEWC_OFF");
+    s.dgrad_pointwise_off = on("SGH_DGRAD_POINTWISE_OFF"), s.conv16_off = on("SGH_CONV16_OFF");
+    s.dgrad_tile = num("SGH_DGRAD_TILE", 0, 3), s.wgrad_tile = num("SGH_WGRAD_TILE", 0, 5);
+    const char *bm = getenv("SGH_DGRAD3X3_BM");
+    s.dgrad3x3_bm = bm ? (atoi(bm) == 64 ? 64 : 128) : 0;
+    return s;
+  }();
+  return e;
+}
+
+// ---- weight epoch and the prepared-weights note of a convolution geometry
+static std::atomic<unsigned long long> g_weights_epoch{1};
+
+unsigned long long sgh_weights_epoch() { return g_weights_epoch.load(std::memory_order_relaxed); }
+void sgh_weights_epoch_bump() { g_weights_epoch.fetch_add(1, std::memory_order_relaxed); }
+
+bool sgh_prelaid_valid(const sgh_conv_geom *g, int dtype, const void *W, const void *workspace) {
+  return g->prelaid_W != nullptr && g->prelaid_W == W && g->prelaid_ws == workspace && g->prelaid_dtype == dtype &&
+         g->prelaid_epoch == sgh_weights_epoch();
+}
+
+void sgh_prelaid_clear(sgh_conv_geom *g) {
+  g->prelaid_dtype = 0;
+  g->prelaid_W = g->prelaid_ws = nullptr;
+  g->prelaid_ws_bytes = 0;
+  g->prelaid_epoch = 0;
+}
+
+void sgh_prelaid_clear_if_overlap(sgh_conv_geom *g, const void *workspace, size_t ws_bytes) {
+  if (!g->prelaid_W || !workspace) return;
+  const char *a = static_cast<const char *>(workspace), *b = static_cast<const char *>(g->prelaid_ws);
+  if (a < b + g->prelaid_ws_bytes && b < a + ws_bytes) sgh_prelaid_clear(g);
 }
 
 // ---- kernel-level profiling records
@@ -156,10 +209,28 @@ int sgh_device_open(int gpu_id, sgh_device **out) {
   return SGH_OK;
 }
 
+// (dev->mu held) the main stream is ordered behind everything enqueued on the auxiliary stream so far:
+// blocks that waited for that may be handed out again
+static void release_pending(sgh_device *dev) {
+  for (auto &b : dev->pending) {
+    dev->free_blocks.emplace(b.second, b.first);
+    dev->cached += b.second;
+  }
+  dev->pending.clear();
+}
+
+// (dev->mu held) nothing is running on either stream afterwards
+static hipError_t quiesce(sgh_device *dev) {
+  hipError_t e = hipStreamSynchronize(dev->stream);
+  if (e == hipSuccess && dev->aux) e = hipStreamSynchronize(dev->aux);
+  if (e == hipSuccess) release_pending(dev);
+  return e;
+}
+
 int sgh_pool_trim(sgh_device *dev) {
   if (!dev) return SGH_EINVAL;
   std::lock_guard<std::mutex> lk(dev->mu);
-  SGH_HIP_TRY(hipStreamSynchronize(dev->stream));
+  SGH_HIP_TRY(quiesce(dev));
   for (auto &kv : dev->free_blocks) (void)hipFree(kv.second);
   dev->free_blocks.clear();
   dev->cached = 0;
@@ -169,15 +240,15 @@ int sgh_pool_trim(sgh_device *dev) {
 int sgh_device_close(sgh_device *dev) {
   if (!dev) return SGH_EINVAL;
   (void)hipSetDevice(dev->id);
-  (void)hipStreamSynchronize(dev->stream);
+  (void)quiesce(dev);   // both streams idle before any memory or stream goes away
   for (auto &kv : dev->free_blocks) (void)hipFree(kv.second);
   for (auto &kv : dev->live) (void)hipFree(kv.first);
+  for (auto &b : dev->pending) (void)hipFree(b.first);
   (void)hipStreamDestroy(dev->stream);
   (void)hipStreamDestroy(dev->side);
-  if (dev->aux) {
-    (void)hipStreamSynchronize(dev->aux);
-    (void)hipStreamDestroy(dev->aux);
-  }
+  if (dev->aux) (void)hipStreamDestroy(dev->aux);
+  if (dev->fork_ev) (void)hipEventDestroy(dev->fork_ev);
+  if (dev->join_ev) (void)hipEventDestroy(dev->join_ev);
   delete dev;
   return SGH_OK;
 }
@@ -196,6 +267,41 @@ void *sgh_device_aux_stream(sgh_device *dev) {
   return reinterpret_cast<void *>(dev->aux);
 }
 
+int sgh_device_fork(sgh_device *dev, void **aux_stream) {
+  if (!dev || !aux_stream) return SGH_EINVAL;
+  if (dev->capturing) return SGH_EUNSUPPORTED;
+  void *aux = sgh_device_aux_stream(dev);
+  if (!aux) return SGH_ENOMEM;
+  if (!dev->fork_ev) {
+    SGH_HIP_TRY(hipEventCreateWithFlags(&dev->fork_ev, hipEventDisableTiming));
+    SGH_HIP_TRY(hipEventCreateWithFlags(&dev->join_ev, hipEventDisableTiming));
+  }
+  SGH_HIP_TRY(hipEventRecord(dev->fork_ev, dev->stream));
+  SGH_HIP_TRY(hipStreamWaitEvent(dev->aux, dev->fork_ev, 0));
+  *aux_stream = aux;
+  return SGH_OK;
+}
+
+int sgh_device_join(sgh_device *dev) {
+  if (!dev) return SGH_EINVAL;
+  if (!dev->aux || !dev->join_ev) return SGH_OK;   // never forked
+  if (dev->capturing) return SGH_EUNSUPPORTED;
+  SGH_HIP_TRY(hipEventRecord(dev->join_ev, dev->aux));
+  SGH_HIP_TRY(hipStreamWaitEvent(dev->stream, dev->join_ev, 0));
+  std::lock_guard<std::mutex> lk(dev->mu);
+  release_pending(dev);
+  return SGH_OK;
+}
+
+int sgh_block_used_on(sgh_device *dev, void *ptr, void *stream) {
+  if (!dev || !ptr) return SGH_EINVAL;
+  std::lock_guard<std::mutex> lk(dev->mu);
+  if (dev->live.find(ptr) == dev->live.end()) return SGH_EINVAL;
+  if (dev->aux && stream == reinterpret_cast<void *>(dev->aux)) dev->on_aux.insert(ptr);
+  else if (stream != reinterpret_cast<void *>(dev->stream)) return SGH_EINVAL;   // not a stream of this device
+  return SGH_OK;
+}
+
 int sgh_stream_wait_event(void *stream, sgh_event *ev) {
   if (!ev) return SGH_EINVAL;
   SGH_HIP_TRY(hipStreamWaitEvent(sgh_stream_of(stream), ev->ev, 0));
@@ -205,8 +311,8 @@ int sgh_stream_wait_event(void *stream, sgh_event *ev) {
 int sgh_device_sync(sgh_device *dev) {
   if (!dev) return SGH_EINVAL;
   if (dev->capturing) return SGH_EUNSUPPORTED;  // nothing runs while the stream records
-  SGH_HIP_TRY(hipStreamSynchronize(dev->stream));
-  if (dev->aux) SGH_HIP_TRY(hipStreamSynchronize(dev->aux));
+  std::lock_guard<std::mutex> lk(dev->mu);
+  SGH_HIP_TRY(quiesce(dev));
   return SGH_OK;
 }
 
@@ -286,10 +392,10 @@ int sgh_malloc(sgh_device *dev, void **ptr, size_t bytes) {
     dev->cached -= r;
   } else {
     hipError_t e = hipMalloc(&p, r);
-    if (e == hipErrorOutOfMemory && !dev->free_blocks.empty()) {
+    if (e == hipErrorOutOfMemory && !(dev->free_blocks.empty() && dev->pending.empty())) {
       // give the cache back to the driver once and retry
       (void)hipGetLastError();
-      (void)hipStreamSynchronize(dev->stream);
+      (void)quiesce(dev);
       for (auto &kv : dev->free_blocks) (void)hipFree(kv.second);
       dev->free_blocks.clear();
       dev->cached = 0;
@@ -317,6 +423,7 @@ int sgh_free(sgh_device *dev, void *ptr) {
   const size_t r = it->second;
   dev->live.erase(it);
   dev->in_use -= r;
+  const bool aux_use = dev->on_aux.erase(ptr) != 0;
   if (dev->capturing) {  // part of the graph being recorded: reserved until the graph is destroyed
     dev->held.emplace_back(ptr, r);
     dev->born.erase(ptr);
@@ -329,6 +436,11 @@ int sgh_free(sgh_device *dev, void *ptr) {
       g->held.emplace_back(ptr, r);
       return SGH_OK;
     }
+  }
+  if (aux_use) {
+    // work on the auxiliary stream may still touch the block: it waits for the next join / sync
+    dev->pending.emplace_back(ptr, r);
+    return SGH_OK;
   }
   // Work already enqueued on the device stream may still read the block; the next owner's
   // work is enqueued behind it on the same stream, so immediate reuse is ordered correctly.
@@ -350,6 +462,7 @@ int sgh_memcpy(sgh_device *dev, void *dst, const void *src, size_t bytes, int ki
   if (!dev || kind < 0 || kind > 3) return SGH_EINVAL;
   if (bytes == 0) return SGH_OK;
   if (!dst || !src) return SGH_EINVAL;
+  if (kind == 1 || kind == 3) sgh_weights_epoch_bump();   // the destination may be a weight tensor
   static const hipMemcpyKind kinds[4] = {hipMemcpyHostToHost, hipMemcpyHostToDevice,
                                          hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice};
   if (dev->capturing && kind != 3) {

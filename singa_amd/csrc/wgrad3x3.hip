@@ -345,7 +345,7 @@ inline W3Plan plan(const sgh_conv_geom *g) {
   const int st = g->stride_h;
   if (g->pad_h > 2 || g->pad_w > 2) return p;
   if (g->W + 2 > 64 || g->Q < 2 || g->Q > 64 || g->C < 32 || g->K < 64) return p;
-  if (getenv("SGH_WGRAD3X3_OFF")) return p;
+  if (sgh_env().wgrad3x3_off) return p;
   // instantiated slabs, stride 1: pitch 64 x 3 rows (RU 1), pitch 32 x 4 rows (RU 2), pitch 16 x 6 rows
   // (RU 4), pitch 16 x 9 rows (RU 7: a whole 7x7 plane); stride 2: pitch 64 x 5 rows (RU 2), pitch 32 x 9
   // rows (RU 4), pitch 16 x 15 rows (RU 7)

@@ -278,7 +278,7 @@ struct WFPlan {
 inline WFPlan plan(const sgh_conv_geom *g) {
   WFPlan p{};
   p.ok = false;
-  if (getenv("SGH_WGRAD_FEWC_OFF")) return p;
+  if (sgh_env().wgrad_fewc_off) return p;
   if (g->stride_h != g->stride_w || (g->stride_h != 1 && g->stride_h != 2)) return p;
   const int CRS = g->C * g->R * g->S;
   if (CRS > NTL * 32 || CRS <= 64) return p;            // narrower problems fit the generic 64-wide tile

@@ -89,8 +89,9 @@ class HipGPU(object):
 
     # A second compute stream for work that the main stream's next ops do not depend on.  Fork():
     # what is enqueued on the auxiliary stream afterwards starts when everything enqueued on the main
-    # stream so far has finished; Join(): the main stream waits for the auxiliary one.  Tensors the
-    # auxiliary stream touches must be kept alive until Join() (the pool recycles in main-stream order).
+    # stream so far has finished; Join(): the main stream waits for the auxiliary one.  Tensors handed
+    # to work on the auxiliary stream are announced with UsedOn(): they may then be dropped at any
+    # time, the pool hands their memory out again only after the Join().
     _aux = None
 
     def AuxStream(self):
@@ -98,22 +99,22 @@ class HipGPU(object):
             s = _L().sgh_device_aux_stream(self._h)
             if not s:
                 raise SingaHipError("no auxiliary stream")
-            ev = [C.c_void_p(), C.c_void_p()]
-            for e in ev:
-                check(_L().sgh_event_create(C.byref(e)), "sgh_event_create")
-            self._aux, self._fork_ev, self._join_ev = s, ev[0], ev[1]
+            self._aux = s
         return self._aux
 
     def Fork(self):
-        aux = self.AuxStream()
-        check(_L().sgh_event_record(self._fork_ev, self.stream), "sgh_event_record")
-        check(_L().sgh_stream_wait_event(aux, self._fork_ev), "sgh_stream_wait_event")
-        return aux
+        aux = C.c_void_p()
+        check(_L().sgh_device_fork(self._h, C.byref(aux)), "sgh_device_fork")
+        self._aux = aux.value
+        return self._aux
 
     def Join(self):
-        if self._aux is not None:
-            check(_L().sgh_event_record(self._join_ev, self._aux), "sgh_event_record")
-            check(_L().sgh_stream_wait_event(self.stream, self._join_ev), "sgh_stream_wait_event")
+        check(_L().sgh_device_join(self._h), "sgh_device_join")
+
+    def UsedOn(self, stream, *tensors):
+        for t in tensors:
+            if t._block.owned:    # (memory the pool does not own is the caller's to keep alive)
+                check(_L().sgh_block_used_on(self._h, t.ptr, stream), "sgh_block_used_on")
 
     def GetAllocatedMem(self):
         a, c, d = C.c_size_t(), C.c_size_t(), C.c_size_t()
@@ -677,7 +678,8 @@ def GpuConvBackwardx(dy, W, x, h):
 def GpuConvBackwardW(dy, x, W, h, stream=None):
     """`stream`: None = the device's stream.  Another stream (``HipGPU.Fork()``) runs the weight
     gradient beside whatever the main stream does next; it then works in a workspace of its own
-    (``h.wgrad_workspace``), and the caller keeps dy, x and the result alive until ``Join()``."""
+    (``h.wgrad_workspace``); dy, x, the result and that workspace are announced to the pool
+    (``HipGPU.UsedOn``), so the caller may drop them whenever it likes."""
     h._check_dy(dy)
     h._check_x(x)
     dW = _like(W)
@@ -690,6 +692,7 @@ def GpuConvBackwardW(dy, x, W, h, stream=None):
                     else _L().sgh_conv_workspace_bytes_h(C.byref(h.geom), which))
             h.wgrad_workspace = Tensor(((max(need, 4) + 3) // 4,), dy.device(), kFloat32)
         ws = h.wgrad_workspace
+        dy.device().UsedOn(stream, dy, x, dW, ws)
     check(fn(C.byref(h.geom), dy.ptr, x.ptr, dW.ptr, ws.ptr, ws.MemSize(),
              dy.device().stream if stream is None else stream), name)
     return dW
@@ -698,9 +701,10 @@ def GpuConvBackwardW(dy, x, W, h, stream=None):
 def GpuConvPrepareBackward(weights_and_handles):
     """Re-lays the weights of all listed convolutions for their data gradients in ONE launch (the
     re-layout each ``GpuConvBackwardx`` otherwise launches for itself); `weights_and_handles`: pairs
-    ``(W, handle)``.  Valid until the weights change: call ``GpuConvBackwardDone`` with the same
-    handles after the backward pass, and run no other pass on a handle between this call and its
-    ``GpuConvBackwardx``.  Results are bit-identical with and without."""
+    ``(W, handle)``.  Each handle's next ``GpuConvBackwardx`` uses the prepared weights if nothing
+    that may change a weight tensor (an update, Axpy, a fill, an upload) was called in between and no
+    other pass wrote the handle's workspace; otherwise it re-lays them itself.  Results are
+    bit-identical with and without."""
     pairs = list(weights_and_handles)
     if not pairs:
         return
@@ -715,10 +719,10 @@ def GpuConvPrepareBackward(weights_and_handles):
     check(_L().sgh_conv_dgrad_prepare_multi(arr, len(pairs), dtype, W0.device().stream), "sgh_conv_dgrad_prepare_multi")
 
 
-def GpuConvBackwardDone(handles):
-    """The weights are about to change: the next data gradients re-lay them again."""
-    for h in handles:
-        h.geom.weights_prelaid = 0
+def ConvWeightsChanged():
+    """For a caller that writes weight tensors by means this library cannot see: prepared weights
+    (``GpuConvPrepareBackward``) are not used after this call."""
+    _L().sgh_conv_weights_changed()
 
 
 def GpuConvBackwardb(dy, b, h):

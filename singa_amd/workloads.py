@@ -119,14 +119,12 @@ class HipOps(object):
     # gradients / BatchNorm / ReLU backward ops (matrix-bound work beside bandwidth-bound work)
     overlap_wgrad = True
     _aux = None          # the auxiliary stream while a backward pass is under way
-    _aux_keep = None     # tensors it still uses
 
     def conv_bwd_w(self, dy, x, W, h):
         if self._aux is not None:
             self._aux = self.dev.Fork()    # (everything enqueued so far, i.e. the producer of dy, comes first)
-            dW = singa.GpuConvBackwardW(dy, x, W, h, stream=self._aux)
-            self._aux_keep += [dy, x, dW]
-            return dW
+            # (the tensors it touches are announced to the pool there: nothing is kept alive here)
+            return singa.GpuConvBackwardW(dy, x, W, h, stream=self._aux)
         return singa.GpuConvBackwardW(dy, x, W, h)
 
     # cross-op fusion the tape permits: the "+=" of a residual fan-in folded into the data gradient
@@ -154,7 +152,7 @@ class HipOps(object):
         # (not while a graph is being recorded: a recording with a branch per layer replays slower than
         # the plain chain, 6.4 against 5.9 ms for ResNet-18)
         if self.overlap_wgrad and update_at_end and not self.dev.graph_enabled():
-            self._aux, self._aux_keep = self.dev.AuxStream(), []
+            self._aux = self.dev.AuxStream()
         if self.batch_relayout:
             by_type = {}
             for c in convs:
@@ -166,8 +164,7 @@ class HipOps(object):
     def finish_backward(self, convs):
         if self._aux is not None:
             self.dev.Join()    # the update (and any reader of a weight gradient) comes after the last of them
-            self._aux = self._aux_keep = None
-        singa.GpuConvBackwardDone([c.h for c in convs if c.h is not None])
+            self._aux = None
 
     fusions = ("fuse_bn_relu", "fuse_dgrad_add", "batch_relayout", "overlap_wgrad")   # what set_fusion(True) turns on
 

@@ -352,12 +352,18 @@ def test_conv_dgrad_16bit_with_batched_weight_relayout(singa, dev, kind):
         h = singa.CudnnConvHandle(xt, (R, S), stride, pad, C, K, False)
         layers.append((case, xt, wt, dyt, h, singa.GpuConvBackwardx(dyt, wt, xt, h).to_numpy()))
     singa.GpuConvPrepareBackward([(l[2], l[4]) for l in layers])
-    prelaid = [l[4].geom.weights_prelaid for l in layers]
-    assert 0 in prelaid and prelaid.count(1) >= len(layers) // 2, prelaid
+    prelaid = [bool(l[4].geom.prelaid_W) for l in layers]
+    assert False in prelaid and prelaid.count(True) >= len(layers) // 2, prelaid
     for case, xt, wt, dyt, h, want in layers:
         _same_bits(singa.GpuConvBackwardx(dyt, wt, xt, h).to_numpy(), want, "prepared dgrad %r" % (case,))
-    singa.GpuConvBackwardDone([l[4] for l in layers])
-    assert not any(l[4].geom.weights_prelaid for l in layers)
+    assert not any(l[4].geom.prelaid_W for l in layers)     # each note was used once
+    # prepared, then the weights change (an update of the 16-bit tensor): the current weights are used
+    case, xt, wt, dyt, h, want = layers[prelaid.index(True)]
+    singa.GpuConvPrepareBackward([(wt, h)])
+    singa.Axpy(0.5, wt, wt)
+    fresh_h = singa.CudnnConvHandle(xt, (case[5], case[6]), case[7], case[8], case[1], case[4], False)
+    _same_bits(singa.GpuConvBackwardx(dyt, wt, xt, h).to_numpy(), singa.GpuConvBackwardx(dyt, wt, xt, fresh_h).to_numpy(),
+               "prepared dgrad after the weights changed")
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])

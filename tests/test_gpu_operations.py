@@ -118,7 +118,7 @@ def test_conv_backward_vs_oracle(singa, dev, case):
 def test_conv_dgrad_with_batched_weight_relayout(singa, dev):
     """GpuConvPrepareBackward re-lays the weights of all CONV_CASES layers in one launch; the data
     gradients (plain and accumulating) that follow skip their own re-layout and must give the same
-    bits; layers whose kernel reads W as it is are left alone; GpuConvBackwardDone ends it."""
+    bits; layers whose kernel reads W as it is are left alone; a prepared layer's note is used once."""
     layers = []
     for i, case in enumerate(CONV_CASES):
         N, C, H, W, K, R, S, stride, pad, _ = case
@@ -132,18 +132,59 @@ def test_conv_dgrad_with_batched_weight_relayout(singa, dev):
         want_acc = singa.GpuConvBackwardxAccumulate(dyd, wd, xd, h, singa.from_numpy(old, dev)).to_numpy()
         layers.append((case, xd, wd, dyd, h, old, want, want_acc))
     singa.GpuConvPrepareBackward([(l[2], l[4]) for l in layers])
-    prelaid = [l[4].geom.weights_prelaid for l in layers]
-    assert 0 in prelaid and prelaid.count(1) >= 6, prelaid
+    prelaid = [bool(l[4].geom.prelaid_W) for l in layers]
+    assert False in prelaid and prelaid.count(True) >= 6, prelaid
     for case, xd, wd, dyd, h, old, want, want_acc in layers:
         assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), want, "prepared dgrad %r" % (case,))
-    # a second use of the same prepared weights (the workspaces were not touched in between)
+        assert not h.geom.prelaid_W            # a note is used once
+    singa.GpuConvPrepareBackward([(l[2], l[4]) for l in layers])
     for case, xd, wd, dyd, h, old, want, want_acc in layers:
         got = singa.GpuConvBackwardxAccumulate(dyd, wd, xd, h, singa.from_numpy(old, dev)).to_numpy()
         assert_bit_equal(got, want_acc, "prepared accumulating dgrad %r" % (case,))
-    singa.GpuConvBackwardDone([l[4] for l in layers])
-    assert not any(l[4].geom.weights_prelaid for l in layers)
-    case, xd, wd, dyd, h, old, want, want_acc = layers[4]
-    assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), want, "after GpuConvBackwardDone")
+        assert not h.geom.prelaid_W
+
+
+def test_prepared_weights_are_never_stale(singa, dev):
+    """What a caller can do wrong after GpuConvPrepareBackward, and still gets the gradient of the
+    CURRENT weights: (1) the weights change before the data gradient (an optimizer update, an upload
+    into the tensor, the caller's own write announced by ConvWeightsChanged); (2) another pass of
+    the same handle overwrites the workspace; (3) a different weight tensor is handed in."""
+    from singa_amd import opt
+    N, C, H, W, K = 2, 64, 14, 14, 64
+    r = rng(77)
+    x, w, w2, dy = randn(r, N, C, H, W), randn(r, K, C, 3, 3), randn(r, K, C, 3, 3), randn(r, N, K, H, W)
+    xd, dyd = singa.from_numpy(x, dev), singa.from_numpy(dy, dev)
+    h = singa.CudnnConvHandle(xd, (3, 3), (1, 1), (1, 1), C, K, False)
+    ref_h = singa.CudnnConvHandle(xd, (3, 3), (1, 1), (1, 1), C, K, False)
+
+    def fresh(wt):
+        return singa.GpuConvBackwardx(dyd, wt, xd, ref_h).to_numpy()
+
+    # (1a) an optimizer update between prepare and data gradient
+    wd = singa.from_numpy(w, dev)
+    singa.GpuConvPrepareBackward([(wd, h)])
+    assert h.geom.prelaid_W == wd.ptr
+    sgd = opt.SGD(lr=0.1, momentum=0.9)
+    sgd.apply("w", wd, singa.from_numpy(w2, dev))
+    assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), fresh(wd), "after an update")
+    # (1b) new values uploaded into the same tensor
+    singa.GpuConvPrepareBackward([(wd, h)])
+    wd.CopyFloatDataFromHostPtr(w2)
+    assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), fresh(wd), "after an upload")
+    # (1c) the caller's own write, announced
+    singa.GpuConvPrepareBackward([(wd, h)])
+    other = singa.from_numpy(w, dev)
+    singa.ConvWeightsChanged()
+    assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), fresh(wd), "after ConvWeightsChanged")
+    # (2) the weight gradient / the forward pass of the same handle ran on the prepared workspace
+    for other_pass in (lambda: singa.GpuConvBackwardW(dyd, xd, wd, h), lambda: singa.GpuConvForward(xd, wd, None, h)):
+        singa.GpuConvPrepareBackward([(wd, h)])
+        other_pass()
+        assert not h.geom.prelaid_W
+        assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), fresh(wd), "after another pass")
+    # (3) prepared for one weight tensor, called with another
+    singa.GpuConvPrepareBackward([(wd, h)])
+    assert_bit_equal(singa.GpuConvBackwardx(dyd, other, xd, h).to_numpy(), fresh(other), "another weight tensor")
 
 
 def test_conv_wgrad_is_deterministic(singa, dev):

@@ -231,6 +231,50 @@ def test_pool_reuses_freed_blocks(singa, dev):
     assert dev.PoolStats()["driver_allocs"] - before <= 1
 
 
+def test_pool_keeps_blocks_of_the_auxiliary_stream_until_the_join(singa, dev):
+    """A block that work on the auxiliary stream uses may be freed right after that work was enqueued
+    (SINGA's Graph does so): the pool hands it out again only once the main stream has been ordered
+    behind the auxiliary one (Join / Sync), never to main-stream work that could overtake it."""
+    from singa_amd._lib import lib
+    n = (1 << 18) + 4096
+    dev.Sync()
+
+    def grab(k):     # k live tensors of the size class (whatever the pool has cached comes out first)
+        return [singa.Tensor((n,), dev) for _ in range(k)]
+
+    aux = dev.Fork()
+    a = singa.Tensor((n,), dev)
+    pa = a.ptr
+    dev.UsedOn(aux, a)
+    assert lib().sgh_memset_f32(pa, 3.0, n, aux) == 0      # work on the auxiliary stream writes the block
+    cached0 = dev.PoolStats()["cached"]
+    del a                                                  # freed while that work may still be running
+    assert dev.PoolStats()["cached"] == cached0            # not back in the pool
+    held = grab(12)
+    assert pa not in [t.ptr for t in held]                 # and not handed to anyone
+    held[0].SetFloatValue(7.0)
+    cached1 = dev.PoolStats()["cached"]
+    dev.Join()
+    assert dev.PoolStats()["cached"] - cached1 >= 4 * n    # back in the pool after the join
+    more = grab(64)
+    assert pa in [t.ptr for t in more]                     # and handed out again
+    assert (held[0].to_numpy() == 7.0).all()
+    c = [t for t in more if t.ptr == pa][0]
+    del more, held
+    # marks are for this device's own blocks and streams only
+    assert lib().sgh_block_used_on(dev._h, pa + 64, aux) == -1
+    assert lib().sgh_block_used_on(dev._h, pa, 0xdead0) == -1
+    assert lib().sgh_block_used_on(dev._h, pa, dev.stream) == 0
+    # without a join, Sync releases what waited
+    dev.Fork()
+    dev.UsedOn(aux, c)
+    del c
+    held = grab(80)
+    assert pa not in [t.ptr for t in held]
+    dev.Sync()
+    assert pa in [t.ptr for t in grab(8)]
+
+
 @pytest.mark.parametrize("n", [1, 5, 1000, 4099, 1 << 20])
 def test_elementwise_functions_around_the_path(singa, dev, n):
     """Sub, Div, Add/Mult/Div by a scalar: each is one IEEE operation per element, so NumPy's fp32
