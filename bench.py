@@ -7,11 +7,17 @@ reference's examples/cnn/model/resnet.py.  One "step" = loss-gradient seed -> la
 updated (every backward kernel in tape order plus the update of all 62 parameter tensors), on
 synthetic seeded inputs whose forward activations are already resident in HBM.
 
-Prints ONE JSON line: the whole-job images/s plus
+Prints ONE JSON line: the whole-job images/s (mean over the timed steps; median and minimum of the
+per-step HIP event times as extra keys) plus
   roofline     -- the dominant kernel family (fp32 MFMA conv dgrad + wgrad kernels):
                   algorithmic FLOPs / measured kernel time (HIP events on the kernels' stream),
-                  against the MI355X fp32 matrix peak;
-  cpu_baseline -- the CPU oracle replaying the same tape on the host cores, on a bounded sample.
+                  against the MI355X fp32 matrix peak; `traffic` = HBM bytes per step of the same
+                  launches, read from the rocprofv3 counter summary under profiles/ when that
+                  summary was taken on the kernels this run launched (null otherwise);
+  hbm_kernels  -- the bandwidth-bound kernel families: algorithmic bytes / measured time against
+                  the HBM3E peak;
+  cpu_baseline -- the CPU oracle replaying the same tape on the host cores, on a bounded sample
+                  (all host threads at the benchmark's batch, and one thread on a few images).
 """
 import argparse
 import ctypes as C
@@ -27,50 +33,90 @@ if ROOT not in sys.path:
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_16BIT_MFMA_TFLOPS = 2500.0   # dense fp16 / bf16 matrix peak
 PEAK_HBM_GBS = 8000.0
-# HBM bytes the 40 conv dgrad/wgrad MFMA launches of one default step move (fetched + written), from the
-# rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, each scaled by what the same counter reads for
-# a streaming kernel of known size (ReLU forward: 1.998 and 1.000).  Valid for the default workload only.
-CONV_HBM_BYTES_PER_STEP = 6.71e9
+# HBM bytes the conv dgrad/wgrad MFMA launches of one step move (fetched + written) come from two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE), summarised in this file together with the
+# workload and the kernels the figure covers; it is quoted only for a run that launched exactly those kernels.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "conv_grad_kernels_hbm_traffic_pmc.txt")
 
 
 def collect_prof(lib):
+    """{class: {"launches", "ms", "work", "kernels": set}} from the library's per-launch event pairs;
+    a record's tag is "class" or "class/kernel"."""
     n = C.c_int()
     lib.sgh_prof_count(C.byref(n))
     out = {}
-    buf = C.create_string_buffer(32)
+    buf = C.create_string_buffer(64)
     for i in range(n.value):
         ms, work = C.c_float(), C.c_double()
-        rc = lib.sgh_prof_get(i, buf, 32, C.byref(ms), C.byref(work))
+        rc = lib.sgh_prof_get(i, buf, 64, C.byref(ms), C.byref(work))
         if rc != 0:
             raise RuntimeError("sgh_prof_get rc=%d" % rc)
-        d = out.setdefault(buf.value.decode(), {"launches": 0, "ms": 0.0, "flop": 0.0})
+        cls, _, kern = buf.value.decode().partition("/")
+        d = out.setdefault(cls, {"launches": 0, "ms": 0.0, "work": 0.0, "kernels": set()})
         d["launches"] += 1
         d["ms"] += ms.value
-        d["flop"] += work.value
+        d["work"] += work.value
+        if kern:
+            d["kernels"].add(kern)
     return out
 
 
-def cpu_baseline(config, sample_batch, budget_s):
+def traffic_from_profile(workload, kernels):
+    """HBM bytes per step from the committed counter summary, or None when the summary is missing, was
+    taken on another workload, or covers a different set of kernels than this run launched."""
+    try:
+        fields = {}
+        for line in open(TRAFFIC_PROFILE):
+            if line.startswith("#@ "):
+                k, _, v = line[3:].partition(":")
+                fields[k.strip()] = v.strip()
+        if fields.get("workload") != workload:
+            return None
+        if set(fields.get("kernels", "").split()) != set(kernels):
+            return None
+        return float(fields["traffic_bytes_per_step"])
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def cpu_baseline(config, sample_batch, budget_s, single_thread_batch):
     """The CPU oracle (a restatement of SINGA's CppCPU algorithms) replaying the same tape on the
-    host cores: whole steps at `sample_batch` until about `budget_s` seconds have been spent."""
+    host cores: whole steps at `sample_batch` until about `budget_s` seconds have been spent, then
+    one step on `single_thread_batch` images with one thread (the reference's per-image loop is
+    serial, and so is its tensor math without a threaded BLAS)."""
     from oracle import cpu_oracle as O
     from oracle.ops import OracleOps
     from singa_amd import workloads as wl
-    ops = OracleOps()
-    net = wl.build(config, ops)
-    x, labels = wl.make_inputs(config, sample_batch)
-    net.forward(ops.from_numpy(x), ops.from_numpy(labels))
-    steps, t0 = 0, time.perf_counter()
-    while True:
-        net.backward_and_update()
-        steps += 1
-        dt = time.perf_counter() - t0
-        if dt >= budget_s or steps >= 50:
-            break
-    return {"value": round(sample_batch * steps / dt, 3), "unit": "imgs/s", "cores": O.get_threads(), "kind": "port",
-            "sample": "%d %s backward+update step(s) at batch %d on the same seeded inputs, %.1f s of CPU time "
-                      "(OpenMP over the SGEMM rows / channels; the per-image loop is serial like the reference's)"
-                      % (steps, config, sample_batch, dt)}
+
+    def run(batch, budget, max_steps):
+        ops = OracleOps()
+        net = wl.build(config, ops)
+        x, labels = wl.make_inputs(config, batch)
+        net.forward(ops.from_numpy(x), ops.from_numpy(labels))
+        steps, t0 = 0, time.perf_counter()
+        while True:
+            net.backward_and_update()
+            steps += 1
+            dt = time.perf_counter() - t0
+            if dt >= budget or steps >= max_steps:
+                return steps, dt
+
+    threads = O.get_threads()
+    steps, dt = run(sample_batch, budget_s, 50)
+    out = {"value": round(sample_batch * steps / dt, 3), "unit": "imgs/s", "cores": threads, "kind": "port",
+           "sgemm": "the oracle's own blocked SGEMM loops (no BLAS library in this image)",
+           "sample": "%d %s backward+update step(s) at batch %d on the same seeded inputs, %.1f s of CPU time "
+                     "(OpenMP over the SGEMM rows / channels; the per-image loop is serial like the reference's)"
+                     % (steps, config, sample_batch, dt)}
+    if single_thread_batch > 0:
+        O.set_threads(1)
+        try:
+            s1, d1 = run(single_thread_batch, 0.0, 1)
+        finally:
+            O.set_threads(threads)
+        out["single_thread"] = {"value": round(single_thread_batch * s1 / d1, 3), "unit": "imgs/s", "cores": 1,
+                                "sample": "1 step at batch %d, %.1f s" % (single_thread_batch, d1)}
+    return out
 
 
 def main():
@@ -80,8 +126,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--config", default="resnet18")
-    ap.add_argument("--cpu-sample-batch", type=int, default=32)
+    ap.add_argument("--cpu-sample-batch", type=int, default=0, help="0: the benchmark's batch")
     ap.add_argument("--cpu-budget-s", type=float, default=10.0)
+    ap.add_argument("--cpu-single-thread-batch", type=int, default=4, help="images of the one-thread CPU sample (0: skip)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--storage", default="f32", choices=["f32", "f16", "bf16"],
                     help="f16 / bf16: the mixed-precision tape (16-bit activations, gradients and conv weights, "
@@ -102,7 +149,6 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
 
-    import torch  # device synchronisation only; no torch op is on the measured path
     from singa_amd import _lib
     from singa_amd import singa_wrap as singa
     from singa_amd import workloads as wl
@@ -119,9 +165,7 @@ def main():
     net.forward(hip.from_numpy(x), hip.from_numpy(labels))
     fused = not args.per_parameter_update
 
-    def sync():
-        dev.Sync()
-        torch.cuda.synchronize()
+    sync = dev.Sync   # waits for both streams of the device
 
     graph = args.graph
     if graph:
@@ -139,15 +183,32 @@ def main():
             net.backward_and_update(fused_update=fused)
     for _ in range(args.warmup):
         step()
+    # one event on the main stream at every step boundary (a step ends with the join and the update there)
+    evs = []
+    for _ in range(args.steps + 1):
+        e = C.c_void_p()
+        _lib.check(lib.sgh_event_create(C.byref(e)), "sgh_event_create")
+        evs.append(e)
     sync()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for i in range(args.steps):
+        _lib.check(lib.sgh_event_record(evs[i], dev.stream))
         step()
+    _lib.check(lib.sgh_event_record(evs[args.steps], dev.stream))
     t_enqueued = time.perf_counter() - t0   # host time to enqueue every launch of the timed steps
     sync()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     imgs_per_s = args.batch * args.steps / elapsed
+    step_ms = []
+    for i in range(args.steps):
+        ms = C.c_float()
+        _lib.check(lib.sgh_event_elapsed_ms(evs[i], evs[i + 1], C.byref(ms)))
+        step_ms.append(ms.value)
+    for e in evs:
+        lib.sgh_event_destroy(e)
+    step_ms.sort()
+    median_ms = step_ms[len(step_ms) // 2] if len(step_ms) % 2 else 0.5 * (step_ms[len(step_ms) // 2 - 1] + step_ms[len(step_ms) // 2])
 
     if graph:
         dev.ResetGraph()
@@ -161,36 +222,48 @@ def main():
     prof = collect_prof(lib)
     lib.sgh_prof_enable(0)
     conv = {k: prof[k] for k in ("conv_dgrad", "conv_wgrad", "conv_dgrad16", "conv_wgrad16") if k in prof}
-    flop = sum(v["flop"] for v in conv.values())
+    flop = sum(v["work"] for v in conv.values())
     ms = sum(v["ms"] for v in conv.values())
     launches = sum(v["launches"] for v in conv.values())
+    kernels = sorted(set().union(*[v["kernels"] for v in conv.values()])) if conv else []
     achieved = flop / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
     peak = PEAK_16BIT_MFMA_TFLOPS if half else PEAK_FP32_MFMA_TFLOPS
+    workload_key = "%s N=%d %s%s" % (args.config, args.batch, args.storage, " no-fusion" if args.no_fusion else "")
     roofline = {
         "bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
         "frac": round(achieved / peak, 4),
-        "traffic": CONV_HBM_BYTES_PER_STEP if (args.config == "resnet18" and args.batch == 64 and not half
-                                               and not args.no_fusion) else None,
-        "traffic_unit": "HBM bytes per step over the same launches (PMC, calibrated)",
-        "kernel": ("16-bit MFMA conv dgrad + wgrad kernels (k_dgrad16, k_wgrad16; fp32 kernels for the stem dgrad; %d launches/step)"
-                   if half else
-                   "fp32 MFMA conv dgrad + wgrad kernels (k_dgrad3x3, k_wgrad3x3, k_dgrad_fewc, k_wgrad_fewc, k_igemm; %d launches/step)")
-                  % (launches // prof_steps),
+        "traffic": traffic_from_profile(workload_key, kernels),
+        "traffic_unit": "HBM bytes per step over the same launches (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a "
+                        "streaming kernel; from profiles/%s, null when that summary covers other kernels or another workload)"
+                        % os.path.basename(TRAFFIC_PROFILE),
+        "kernel": "%s MFMA conv dgrad + wgrad kernels (%s; %d launches/step)"
+                  % ("16-bit" if half else "fp32", ", ".join(kernels), launches // prof_steps),
         "flop_per_step": flop / prof_steps, "kernel_ms_per_step": round(ms / prof_steps, 4),
         "timing": "HIP event pair around every launch in %d extra steps with all kernels on one stream "
                   "(the timed steps run the weight gradients on a second stream)" % prof_steps,
     }
     for k, v in conv.items():
-        roofline[k + "_tflops"] = round(v["flop"] / (v["ms"] * 1e-3) / 1e12, 3) if v["ms"] > 0 else 0.0
+        roofline[k + "_tflops"] = round(v["work"] / (v["ms"] * 1e-3) / 1e12, 3) if v["ms"] > 0 else 0.0
     # whole entry points (weight re-layout, split-K reduction and column gather kernels included)
     ops_ms = sum(prof[k]["ms"] for k in ("conv_dgrad_op", "conv_wgrad_op") if k in prof)
     roofline["entry_points_ms_per_step"] = round(ops_ms / prof_steps, 4)
+
+    # the bandwidth-bound families: algorithmic bytes (minimal tensor traffic) / time between the event pair
+    hbm = {}
+    for k in ("bn_relu_bwd", "bn_bwd", "relu_bwd", "relu_bwd_add", "add", "pool_bwd", "sgd"):
+        if k in prof and prof[k]["ms"] > 0:
+            v = prof[k]
+            gbs = v["work"] / (v["ms"] * 1e-3) / 1e9
+            hbm[k] = {"launches_per_step": v["launches"] // prof_steps, "bytes_per_step": v["work"] / prof_steps,
+                      "ms_per_step": round(v["ms"] / prof_steps, 4), "GB/s": round(gbs, 1),
+                      "frac": round(gbs / PEAK_HBM_GBS, 4)}
 
     out = {
         "metric": "backward+update imgs/sec, ResNet-18 N=64 fp32" if (args.config == "resnet18" and not half and args.batch == 64)
                   else "backward+update imgs/sec, %s N=%d %s" % (args.config, args.batch, args.storage),
         "value": round(imgs_per_s, 2), "unit": "imgs/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_median": round(median_ms, 4), "ms_per_step_min": round(step_ms[0], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.storage, "data": "synthetic",
         "config": {"workload": "%s backward+update, N=%d, 3x224x224, %s, SGD momentum 0.9" % (
                        args.config, args.batch, "fp32" if not half else args.storage + " storage / fp32 accumulate, statistics and master weights"),
@@ -203,10 +276,13 @@ def main():
                            if hip.fuse_bn_relu
                            else "one call per reference op"},
         "roofline": roofline,
+        "hbm_kernels": {"peak_GB/s": PEAK_HBM_GBS, "bytes": "algorithmic (every tensor of the op once)",
+                        "timing": "HIP event pair around each entry point, same extra steps as the roofline", **hbm},
         "host_enqueue_ms_per_step": round(t_enqueued / args.steps * 1e3, 4),
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args.config, args.cpu_sample_batch, args.cpu_budget_s)
+        out["cpu_baseline"] = cpu_baseline(args.config, args.cpu_sample_batch or args.batch, args.cpu_budget_s,
+                                           args.cpu_single_thread_batch)
     print(json.dumps(out))
 
 

@@ -506,6 +506,8 @@ int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *g
   float *part = static_cast<float *>(workspace);
   const dim3 grid(C * s.S), block(kBlock);
   hipStream_t st = sgh_stream_of(stream);
+  // algorithmic bytes: x and dy in, dx out (the fused form covers the ReLU backward as well)
+  sgh_prof_scope prof(beta ? "bn_relu_bwd/k_bn_bwd" : "bn_bwd/k_bn_bwd", 3.0 * N * C * HW * sizeof(typename S::elem), st);
   if (resident_ok(N, C, HW, sizeof(typename S::elem))) {
     const int rc = beta ? launch_resident<S, true>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, s, st)
                         : launch_resident<S, false>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, s, st);

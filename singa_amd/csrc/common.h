@@ -62,6 +62,19 @@ void sgh_prelaid_clear_if_overlap(sgh_conv_geom *g, const void *workspace, size_
 bool sgh_prof_on();
 void sgh_prof_start(const char *tag, double work, hipStream_t s);
 void sgh_prof_stop(hipStream_t s);
+// Record for the enclosing scope: `tag` is "class" or "class/kernel", `work` the algorithmic FLOPs or bytes.
+struct sgh_prof_scope {
+  hipStream_t s;
+  bool on;
+  sgh_prof_scope(const char *tag, double work, hipStream_t s_) : s(s_), on(sgh_prof_on()) {
+    if (on) sgh_prof_start(tag, work, s);
+  }
+  ~sgh_prof_scope() {
+    if (on) sgh_prof_stop(s);
+  }
+  sgh_prof_scope(const sgh_prof_scope &) = delete;
+  sgh_prof_scope &operator=(const sgh_prof_scope &) = delete;
+};
 
 // 3x3 (stride 1 or 2) weight gradient with a shared LDS input tile (wgrad3x3.hip).  *_run returns
 // SGH_EUNSUPPORTED for geometries it does not cover; *_workspace_bytes is 0 for those.

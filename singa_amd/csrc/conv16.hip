@@ -829,7 +829,7 @@ int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
   a.chunks = p.chunks, a.chunks_per_split = p.cps;
   a.dy_elems = long(g->N) * g->K * g->P * g->Q, a.x_elems = long(g->N) * g->C * g->H * g->W;
   const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
-  sgh_prof_start("conv_wgrad16", flops, s);
+  sgh_prof_start("conv_wgrad16/k_wgrad16", flops, s);
   int rc;
   if (p.bm == 128) {
     if (p.stride == 1) rc = bf16 ? launch_w<128, 1, true>(a, p, s) : launch_w<128, 1, false>(a, p, s);
@@ -895,7 +895,7 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2);
   a.wt_bytes = unsigned(nw * 2);
   const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
-  sgh_prof_start(fwd_of ? "conv_fwd16" : "conv_dgrad16", flops, s);
+  sgh_prof_start(fwd_of ? "conv_fwd16/k_dgrad16" : "conv_dgrad16/k_dgrad16", flops, s);
   int rc;
   if (p.pixk) {
     if (p.bm == 128) rc = bf16 ? launch_d<128, true, true>(a, p, s) : launch_d<128, false, true>(a, p, s);

@@ -300,11 +300,11 @@ static int dgrad_fewc_run(const sgh_conv_geom *g, const void *dy, const float *W
 
 int sgh_dgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
                        size_t ws_bytes, hipStream_t s) {
-  return dgrad_fewc_run<StF32>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad");
+  return dgrad_fewc_run<StF32>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad/k_dgrad_fewc");
 }
 
 int sgh_dgrad_fewc_run16(const sgh_conv_geom *g, const uint16_t *dy, const float *W, uint16_t *dx, void *workspace,
                          size_t ws_bytes, bool bf16, hipStream_t s) {
-  return bf16 ? dgrad_fewc_run<StBF16>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad16")
-              : dgrad_fewc_run<StF16>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad16");
+  return bf16 ? dgrad_fewc_run<StBF16>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad16/k_dgrad_fewc")
+              : dgrad_fewc_run<StF16>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad16/k_dgrad_fewc");
 }

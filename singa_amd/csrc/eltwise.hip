@@ -474,6 +474,7 @@ __global__ __launch_bounds__(kBlock) void k_add_row(const float *__restrict__ v,
 extern "C" {
 
 int sgh_relu_bwd_f32(const float *dy, const float *x, float *dx, size_t n, void *stream) {
+  sgh_prof_scope prof("relu_bwd/k_map2_1<ReluBwd>", 3.0 * n * sizeof(float), sgh_stream_of(stream));
   return launch_map2(dy, x, dx, n, ReluBwd{}, stream);
 }
 
@@ -482,6 +483,7 @@ int sgh_relu_fwd_f32(const float *x, float *y, size_t n, void *stream) {
 }
 
 int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
+  sgh_prof_scope prof("add/k_map2_1<AddOp>", 3.0 * n * sizeof(float), sgh_stream_of(stream));
   return launch_map2(a, b, out, n, AddOp{}, stream);
 }
 
@@ -567,6 +569,7 @@ int sgh_sgd_momentum_multi_f32(const sgh_sgd_item *table_dev, int count, size_t 
   size_t chunks = total_n / kChunk + size_t(count);  // upper bound on sum of per-item chunk counts
   const size_t cap = size_t(sgh_num_cus()) * 8;
   if (chunks > cap) chunks = cap;
+  sgh_prof_scope prof("sgd/k_sgd_multi", 20.0 * total_n, sgh_stream_of(stream));   // p, g, v in; p, v out
   hipLaunchKernelGGL(k_sgd_multi, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count,
                      SgdHyper{lr, mu, damp, wd}, nesterov);
   SGH_LAUNCH_CHECK();

@@ -398,6 +398,8 @@ int sgh_sgd_momentum_multi_mixed(const sgh_sgd_mixed_item *table_dev, int count,
   const size_t cap = size_t(sgh_num_cus()) * 8;
   if (chunks > cap) chunks = cap;
   const SgdHyper h{lr, mu, damp, wd};
+  // fp32 items: p, g, v in, p, v out; 16-bit items: p, v (4) + g (2) in, p, v (4) + p16 (2) out: 20 bytes either way
+  sgh_prof_scope prof("sgd/k_sgd_multi_mixed", 20.0 * total_n, sgh_stream_of(stream));
   if (bf16) hipLaunchKernelGGL(k_sgd_multi_mixed<BF16>, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count, h, nesterov);
   else hipLaunchKernelGGL(k_sgd_multi_mixed<F16>, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count, h, nesterov);
   SGH_LAUNCH_CHECK();
@@ -432,26 +434,33 @@ int sgh_cast_f32_to_bf16(const float *src, uint16_t *dst, size_t n, void *stream
 int sgh_cast_bf16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream) { return cast_from16<BF16>(src, dst, n, stream); }
 
 int sgh_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream) {
+  sgh_prof_scope prof("relu_bwd/k_map2_h<ReluBwd>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<F16>(dy, x, dx, n, ReluBwd{}, stream);
 }
 int sgh_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream) {
+  sgh_prof_scope prof("relu_bwd/k_map2_h<ReluBwd>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<BF16>(dy, x, dx, n, ReluBwd{}, stream);
 }
 int sgh_relu_bwd_add_f32(const float *dy0, const float *dy1, const float *x, float *dx, size_t n, void *stream) {
+  sgh_prof_scope prof("relu_bwd_add/k_relu_bwd_add", 4.0 * n * 4, sgh_stream_of(stream));
   return launch_relu_bwd_add<StF32>(dy0, dy1, x, dx, n, stream);
 }
 int sgh_relu_bwd_add_f16(const uint16_t *dy0, const uint16_t *dy1, const uint16_t *x, uint16_t *dx, size_t n,
                          void *stream) {
+  sgh_prof_scope prof("relu_bwd_add/k_relu_bwd_add", 4.0 * n * 2, sgh_stream_of(stream));
   return launch_relu_bwd_add<StF16>(dy0, dy1, x, dx, n, stream);
 }
 int sgh_relu_bwd_add_bf16(const uint16_t *dy0, const uint16_t *dy1, const uint16_t *x, uint16_t *dx, size_t n,
                           void *stream) {
+  sgh_prof_scope prof("relu_bwd_add/k_relu_bwd_add", 4.0 * n * 2, sgh_stream_of(stream));
   return launch_relu_bwd_add<StBF16>(dy0, dy1, x, dx, n, stream);
 }
 int sgh_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  sgh_prof_scope prof("add/k_map2_h<AddOp>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<F16>(a, b, out, n, AddOp{}, stream);
 }
 int sgh_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  sgh_prof_scope prof("add/k_map2_h<AddOp>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<BF16>(a, b, out, n, AddOp{}, stream);
 }
 int sgh_eltwise_mult_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {

@@ -928,17 +928,17 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
       auto la = dense_loader<128, false>(W, 1, g->C, g->C, g->K);
       auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
       rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, DilateStore, false, false>(
-          la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad", conv_flops(g));
+          la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad/k_igemm", conv_flops(g));
     } else if (long((g->C + 63) / 64) * ((Ncols + 127) / 128) >= need) {
       auto la = dense_loader<64, false>(W, 1, g->C, g->C, g->K);
       auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
       rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DilateStore, false, false>(
-          la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad", conv_flops(g));
+          la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad/k_igemm", conv_flops(g));
     } else {
       auto la = dense_loader<64, false>(W, 1, g->C, g->C, g->K);
       auto lb = gather_loader<64, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
       rc = launch_igemm<64, 64, DenseLoader<64, false>, PixelGatherLoader<64, false>, DilateStore, false, false>(
-          la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad", conv_flops(g));
+          la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad/k_igemm", conv_flops(g));
     }
   } else if (path == kDgradColumns) {
     float *dcol = static_cast<float *>(workspace);
@@ -948,7 +948,7 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
     DenseStore st{dcol, long(Ncols), CRS, Ncols, 1.f, 0.f};
     rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DenseStore, false, false>(
-        la, lb, st, CRS, Ncols, g->K, 1, (g->K + BK - 1) / BK, s, "conv_dgrad", conv_flops(g));
+        la, lb, st, CRS, Ncols, g->K, 1, (g->K + BK - 1) / BK, s, "conv_dgrad/k_igemm", conv_flops(g));
     if (rc == SGH_OK) {
       const long total = long(g->N) * g->C * g->H * (long((g->W + g->stride_w - 1) / g->stride_w) * g->stride_w);
       long blocks = (total + NT - 1) / NT;
@@ -966,7 +966,7 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) +
                                                 align256(size_t(RS) * KP * g->C * sizeof(float)) +
                                                 align256(sizeof(DgClsTable)));
-    rc = sgh_dgrad3x3_run(g, dy, Wt, KP, dx, partials, s, "conv_dgrad", nullptr, accumulate);
+    rc = sgh_dgrad3x3_run(g, dy, Wt, KP, dx, partials, s, "conv_dgrad/k_dgrad3x3", nullptr, accumulate);
   } else if (path == kDgradClasses) {
     float *Wc = static_cast<float *>(workspace);
     const size_t wc_bytes = size_t(RS) * KP * g->C * sizeof(float);
@@ -1020,7 +1020,7 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     lb.tab = tab_dev;                                                                                         \
     lb.bytes = bytes_of(size_t(g->N) * g->K * g->P * g->Q);                                                   \
     rc = launch_igemm<BM_, BN_, DgradWLoader<BM_>, DgradDyLoader<BN_>, DgradStore, false, false, true>(       \
-        la, lb, st, M, max_cols, 0, ncls, 0, s, "conv_dgrad", conv_flops(g));                                 \
+        la, lb, st, M, max_cols, 0, ncls, 0, s, "conv_dgrad/k_igemm", conv_flops(g));                                 \
   }
     if (tile == 0) SGH_DGRAD_CASE(128, 128)
     else if (tile == 1) SGH_DGRAD_CASE(64, 128)
@@ -1039,7 +1039,7 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     auto la = dense_loader<128, false>(Wt, 1, g->C, M, Ktot);
     auto lb = gather_loader<128, true>(dy, to_g(g), KP, g->K, g->P, g->Q, Ncols);
     rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, true>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, Ktot / BK, s, "conv_dgrad", conv_flops(g));
+        la, lb, st, M, Ncols, Ktot, 1, Ktot / BK, s, "conv_dgrad/k_igemm", conv_flops(g));
   }
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
@@ -1228,7 +1228,7 @@ int sgh_conv_fwd_f32(sgh_conv_geom *g, const float *x, const float *W, const flo
     hipLaunchKernelGGL(k_weight_relayout, dim3(int(blocks)), dim3(NT), 0, s, W, Wt, g->K, g->C, RS, CP, 2);
     float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) +
                                                 align256(size_t(RS) * CP * g->K * sizeof(float)));
-    const int rc3 = sgh_dgrad3x3_run(&gt, x, Wt, CP, y, partials, s, "conv_fwd", bias, false);
+    const int rc3 = sgh_dgrad3x3_run(&gt, x, Wt, CP, y, partials, s, "conv_fwd/k_dgrad3x3", bias, false);
     sgh_prof_stop(s);
     return rc3;
   }
@@ -1246,11 +1246,11 @@ int sgh_conv_fwd_f32(sgh_conv_geom *g, const float *x, const float *W, const flo
   if (M > 64) {
     auto la = dense_loader<128, false>(Wt, 1, g->K, M, Ktot);
     rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd", conv_flops(g));
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd/k_igemm", conv_flops(g));
   } else {
     auto la = dense_loader<64, false>(Wt, 1, g->K, M, Ktot);
     rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
-        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd", conv_flops(g));
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd/k_igemm", conv_flops(g));
   }
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
@@ -1293,7 +1293,7 @@ int sgh_conv_wgrad_f32(sgh_conv_geom *g, const float *dy, const float *x, float 
     lb.CRS = CRS;                                                                                                  \
     lb.bytes = bytes_of(size_t(g->N) * g->C * g->H * g->W);                                                        \
     rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true, false, WGM_>(       \
-        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s, "conv_wgrad", conv_flops(g));              \
+        la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s, "conv_wgrad/k_igemm", conv_flops(g));              \
   }
   if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128, 2)
   else if (p.bm == 64 && p.bn == 256) SGH_WGRAD_CASE(64, 256, 1)

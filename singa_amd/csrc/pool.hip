@@ -348,6 +348,11 @@ int pool_bwd(const sgh_pool_geom *g, const typename S::elem *dy, const typename 
   if (!geom_ok(g) || !dy || !dx) return SGH_EINVAL;
   if (g->is_max && !x) return SGH_EINVAL;
   const size_t total = size_t(g->N) * g->C * g->H * g->W;
+  // algorithmic bytes: dy and (max pooling) x in, dx out
+  sgh_prof_scope prof(g->is_max ? "pool_bwd/k_pool_max_bwd" : "pool_bwd/k_pool_avg_bwd",
+                      double(sizeof(typename S::elem)) *
+                          (double(total) * (g->is_max ? 2 : 1) + double(g->N) * g->C * g->P * g->Q),
+                      sgh_stream_of(stream));
   if (g->is_max) {
     // band height: about 12 KB of x rows per workgroup (measured optimum: enough workgroups per CU to
     // overlap one's staging with another's scans), bands of equal height

@@ -433,7 +433,7 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
   a.units_per_split = p.units_per_split;
   dim3 grid((g->K + p.bm - 1) / p.bm, (g->C + p.bc - 1) / p.bc, p.splits);
   int rc = SGH_EUNSUPPORTED;
-  sgh_prof_start("conv_wgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
+  sgh_prof_start("conv_wgrad/k_wgrad3x3", 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
 #define W3_CASE(BM_, BC_, LOGP_, ROWS_) \
   if (p.bm == BM_ && p.bc == BC_ && p.logp == LOGP_ && p.rows == ROWS_) rc = launch<BM_, BC_, LOGP_, ROWS_>(a, p, grid, s);
   W3_CASE(128, 32, 6, 3)

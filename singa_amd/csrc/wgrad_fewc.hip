@@ -352,7 +352,7 @@ int sgh_wgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *x, 
   a.total_units = p.total_units;
   a.units_per_split = p.units_per_split;
   dim3 grid((g->K + BM - 1) / BM, 1, p.splits);
-  sgh_prof_start("conv_wgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S, s);
+  sgh_prof_start("conv_wgrad/k_wgrad_fewc", 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S, s);
   const int rc = g->stride_h == 1 ? launch<1>(a, p, grid, s) : launch<2>(a, p, grid, s);
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
