@@ -439,10 +439,12 @@ SGH_API int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma,
 /* sgh_bn_bwd_f32 for callers that cannot allocate device memory and have no workspace to pass
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  Same kernels, same results bit for bit; the per-channel partial
- * sums live in a buffer that is part of the library's code object (128 KiB on every GPU the
- * library runs on, held until the process ends) instead of a workspace.  Limit: the number of
- * (channel, split) partial sums -- C for C > 2048, below 2048 + C otherwise -- may not exceed 16384, i.e. C <= 16384;
- * beyond that SGH_ELIMIT is returned and nothing is launched.  Calls no hipMalloc / hipFree.
+ * sums live in a buffer that is part of the library's code object (256 KiB on every GPU the
+ * library runs on, held until the process ends) instead of a workspace.  Limit: the partial sums
+ * of the shape must fit in those 256 KiB -- sgh_bn_workspace_bytes(N, C, HW) <= 262144 is
+ * sufficient (8 bytes per channel and split of the two-pass kernels, 16 per channel and slice of
+ * the one-pass kernel; every ResNet layer up to batch 128 fits) -- else SGH_ELIMIT is returned
+ * and nothing is launched.  Calls no hipMalloc / hipFree.
  * All calls on one GPU share the buffer: calls that overlap on one GPU (two streams, two threads)
  * race; calls on one stream are ordered and safe.  Nothing in the buffer needs clearing between
  * calls (every slot read is written earlier in the same call). */

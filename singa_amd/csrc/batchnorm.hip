@@ -7,7 +7,9 @@
 // range of the channel's (n, hw) index space with 16-byte loads where HW % 4 == 0.
 // Reductions are a fixed tree (lane partials -> wavefront shuffle -> LDS -> ordered sum over
 // the S partials), so results are run-to-run identical.
+#include <atomic>
 #include <mutex>
+#include <random>
 
 #include "common.h"
 #include "storage.h"
@@ -15,7 +17,7 @@
 // Partial sums of sgh_bn_bwd_noalloc_f32: device memory the library owns from load time on, so the
 // entry point has nothing to allocate.  In host code this name is only a handle for
 // hipGetSymbolAddress; kernels receive the address looked up per device (noalloc_scratch_of).
-constexpr int kNoAllocMaxPairs = 16384;  // (channel, split) pairs of two floats: 128 KiB per device
+constexpr int kNoAllocMaxPairs = 32768;  // partial sums: 256 KiB per device
 static __device__ __align__(256) float scratch[kNoAllocMaxPairs * 2];
 
 namespace {
@@ -417,6 +419,226 @@ __global__ __launch_bounds__(kResNT) void k_bn_bwd_resident(const typename S::el
   }
 }
 
+// ---- backward in one pass for planes of whole vectors: a channel is cut into G consecutive slices, one
+// workgroup per slice keeps its slice of x and dy IN REGISTERS (raw storage, up to chip_nv() vectors per
+// tensor and thread) from the reduction to the normalisation.  The G workgroups of a channel exchange their
+// partial sums through the workspace.  Each publishes (sum dy, sum dy * xhat) as two 64-bit words that carry
+// their own validity: the float in the upper half, half of a 64-bit ticket -- a number unique to the call --
+// in the lower half, written with relaxed device-scope atomic stores (no fence: a word is either the old
+// one or the new one).  Each then polls the 2 G words of its channel until all carry the ticket and adds the
+// G partials in slice order, so every workgroup of the channel obtains the same bits.  Having read them, a
+// A launch carries two tickets.  A workgroup first looks at what its own words hold: if that is the first
+// ticket it publishes under the second one, otherwise under the first -- so a recorded launch, which
+// carries the same two tickets into every replay, alternates between them (all words of a channel are
+// rewritten by every execution, so they agree on which one is next), and no word ever has to be cleared.
+// Only the G workgroups of one channel have to be on the chip together (G <= kChipMaxG, far below the number
+// of CUs); their ids are consecutive, workgroups are dispatched in id order, and a waiting workgroup waits
+// only for its own channel's slices, so the oldest unfinished channel always has all its slices dispatched
+// and finishes.  The wait is bounded all the same: after `spin_limit` polls a workgroup gives up and the
+// channel's outputs become NaN.
+// x and dy are read once and dx written once: 3 tensor passes instead of 5.
+constexpr int kChipMaxG = 128, kChipSpinLimit = 1 << 20;
+// vectors per tensor and thread: 8 (64 registers of raw data), 5 for 16-byte vectors of 16-bit elements,
+// whose eight conversions per vector need more registers beside the data
+template <class S>
+constexpr int chip_nv() { return (sizeof(typename S::elem) == 2 && S::VEC == 8) ? 5 : 8; }
+
+struct ChipSlot {   // one per (channel, slice): {bits(a) : ticket low half}, {bits(b) : ticket high half}
+  unsigned long long wa, wb;
+};
+inline size_t chip_workspace_bytes(int C, int G) { return size_t(C) * size_t(G) * sizeof(ChipSlot); }
+
+struct ChipPlan {
+  bool ok;
+  int G, vpg, nt;   // slices per channel, vectors per slice, threads per workgroup
+};
+
+template <class S>
+inline ChipPlan chip_plan(int N, int C, int HW) {
+  ChipPlan p{false, 0, 0, 0};
+  if (HW % S::VEC != 0) return p;
+  const long TV = long(N) * (HW / S::VEC);                       // vectors per channel
+  // 512 threads (two workgroups per CU: one loads while the other waits or stores) unless that cuts the
+  // channel into more slices than one wavefront can poll
+  p.nt = 512;
+  long G = (TV + long(p.nt) * chip_nv<S>() - 1) / (long(p.nt) * chip_nv<S>());
+  if (G > kChipMaxG) {
+    p.nt = 1024;
+    G = (TV + long(p.nt) * chip_nv<S>() - 1) / (long(p.nt) * chip_nv<S>());
+  }
+  // few channels: thinner slices, so that there are two workgroups for every CU (at least one wavefront of vectors each)
+  const long want = (2L * sgh_num_cus() + C - 1) / C;
+  if (G < want) G = want;
+  // whole rounds: as many slices as still fit into the rounds of (2 workgroups x CUs) that this many need
+  const long slots = 2L * sgh_num_cus(), rounds = (long(C) * G + slots - 1) / slots;
+  long fill = rounds * slots / C;
+  if (fill > kChipMaxG) fill = kChipMaxG;
+  if (fill > G) G = fill;
+  while (G > 1 && (TV + G - 1) / G < 64) --G;
+  if (G > kChipMaxG || G < 1) return p;
+  p.vpg = int((TV + G - 1) / G);
+  p.G = int((TV + p.vpg - 1) / p.vpg);
+  p.ok = long(C) * p.G < 0x7fffffffL;
+  return p;
+}
+
+template <class S, bool RELU, int NT>
+__global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem *__restrict__ dy,
+                                                          const typename S::elem *__restrict__ x,
+                                                          const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                          const float *__restrict__ save_mean,
+                                                          const float *__restrict__ save_invstd,
+                                                          typename S::elem *__restrict__ dx, float *__restrict__ dgamma,
+                                                          float *__restrict__ dbeta, unsigned long long *__restrict__ ws,
+                                                          BnShape s, int G, int vpg, unsigned long long ticket1,
+                                                          unsigned long long ticket2, int spin_limit) {
+  typedef typename S::elem elem;
+  constexpr int V = S::VEC, NV = chip_nv<S>();
+  typedef typename RawVec<V * sizeof(elem)>::type raw;
+  __shared__ float red[16];
+  __shared__ float part_a[kChipMaxG], part_b[kChipMaxG];
+  __shared__ int gave_up;
+  __shared__ unsigned long long ticket_s;
+  const int c = blockIdx.x / G, g = blockIdx.x - c * G, t = threadIdx.x;
+  unsigned long long *words = ws + size_t(c) * 2 * size_t(G);   // the channel's G slots
+  if (G > 1 && t == 0) {
+    const unsigned long long wa = __hip_atomic_load(words + 2 * g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long wb = __hip_atomic_load(words + 2 * g + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ticket_s = (unsigned(wa) == unsigned(ticket1) && unsigned(wb) == unsigned(ticket1 >> 32)) ? ticket2 : ticket1;
+    gave_up = 0;
+  }
+  const int PV = s.HW / V, TV = s.N * PV;
+  const int lo = g * vpg, hi = min(lo + vpg, TV);
+  const float mean = save_mean[c], invstd = save_invstd[c];
+  const float gm = gamma[c], be = RELU ? beta[c] : 0.f;
+  auto gate = [&](float d, float v) { return !RELU || S::stored_positive(bn_out(v, mean, invstd, gm, be)) ? d : 0.f; };
+  const raw *xg = reinterpret_cast<const raw *>(x), *dg_ = reinterpret_cast<const raw *>(dy);
+  raw xv[NV], dv[NV];
+  // every load of the slice is issued before the first value is used
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int iv = lo + i * NT + t;
+    if (iv < hi) {
+      const int n = iv / PV, r = iv - n * PV;
+      const size_t off = (size_t(n) * s.C + c) * PV + r;
+      xv[i] = __builtin_nontemporal_load(xg + off);
+      dv[i] = __builtin_nontemporal_load(dg_ + off);
+    }
+  }
+  float a = 0.f, b = 0.f, b1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (lo + i * NT + t < hi) {
+      float v[V], d[V];
+      S::template load16<false>(reinterpret_cast<const elem *>(&xv[i]), v);
+      S::template load16<false>(reinterpret_cast<const elem *>(&dv[i]), d);
+#pragma unroll
+      for (int q = 0; q < V; q += 4) {
+        const float d0 = gate(d[q], v[q]), d1 = gate(d[q + 1], v[q + 1]), d2 = gate(d[q + 2], v[q + 2]),
+                    d3 = gate(d[q + 3], v[q + 3]);
+        a += (d0 + d1) + (d2 + d3);
+        b = __builtin_fmaf(d0, (v[q] - mean) * invstd, b);
+        b1 = __builtin_fmaf(d1, (v[q + 1] - mean) * invstd, b1);
+        b = __builtin_fmaf(d2, (v[q + 2] - mean) * invstd, b);
+        b1 = __builtin_fmaf(d3, (v[q + 3] - mean) * invstd, b1);
+      }
+    }
+  }
+  b += b1;
+  float db = sgh_block_sum(a, red), dg = sgh_block_sum(b, red);
+  if (G > 1) {
+    // (the block sums above contain barriers: ticket_s and gave_up are visible to every thread)
+    const unsigned long long ticket = ticket_s;
+    const unsigned lo32 = unsigned(ticket), hi32 = unsigned(ticket >> 32);   // (both halves are nonzero)
+    if (t == 0) {
+      __hip_atomic_store(words + 2 * g, (static_cast<unsigned long long>(__float_as_uint(db)) << 32) | lo32,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(words + 2 * g + 1, (static_cast<unsigned long long>(__float_as_uint(dg)) << 32) | hi32,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (t < G) {   // one lane per slice of the channel polls that slice's words (the second one until it is
+                   // there, then the first one: one load per poll)
+      unsigned long long wa = 0, wb = 0;
+      int spins = 0;
+      bool have_b = false;
+      for (;;) {
+        if (!have_b) {
+          wb = __hip_atomic_load(words + 2 * t + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          have_b = unsigned(wb) == hi32;
+        }
+        if (have_b) {
+          wa = __hip_atomic_load(words + 2 * t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (unsigned(wa) == lo32) break;
+        }
+        if (++spins >= spin_limit) {
+          gave_up = 1;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(32);
+      }
+      part_a[t] = __uint_as_float(unsigned(wa >> 32));
+      part_b[t] = __uint_as_float(unsigned(wb >> 32));
+    }
+    __syncthreads();
+    // the same G numbers in the same order in every workgroup of the channel
+    db = 0.f, dg = 0.f;
+    for (int i = 0; i < G; ++i) db += part_a[i], dg += part_b[i];
+    if (gave_up) db = dg = __builtin_nanf("");
+  }
+  if (g == 0 && t == 0) {
+    dbeta[c] = db;
+    dgamma[c] = dg;
+  }
+  const float k = gm * invstd;
+  const float rM = float(1.0 / (double(s.N) * s.HW));
+  const float c0 = db * rM, c1 = dg * rM;
+  raw *og = reinterpret_cast<raw *>(dx);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int iv = lo + i * NT + t;
+    if (iv < hi) {
+      const int n = iv / PV, r = iv - n * PV;
+      float v[V], d[V], o[V];
+      S::template load16<false>(reinterpret_cast<const elem *>(&xv[i]), v);
+      S::template load16<false>(reinterpret_cast<const elem *>(&dv[i]), d);
+#pragma unroll
+      for (int q = 0; q < V; ++q) o[q] = k * (gate(d[q], v[q]) - __builtin_fmaf((v[q] - mean) * invstd, c1, c0));
+      raw ov;
+      S::store16(reinterpret_cast<elem *>(&ov), o);
+      og[(size_t(n) * s.C + c) * PV + r] = ov;
+    }
+  }
+}
+
+// tickets: a random 64-bit start (so that whatever an uninitialised workspace holds is not the next
+// ticket, up to a chance of 2^-64 per slot) and one step per call
+inline unsigned long long next_ticket() {
+  static std::atomic<unsigned long long> t{[] {
+    std::random_device rd;
+    return (static_cast<unsigned long long>(rd()) << 32) ^ rd() ^ 0x9e3779b97f4a7c15ull;
+  }()};
+  unsigned long long v;
+  do v = t.fetch_add(0x9e3779b97f4a7c15ull | 1ull, std::memory_order_relaxed);
+  while (unsigned(v) == 0 || unsigned(v >> 32) == 0);   // a zeroed word must never look valid
+  return v;
+}
+
+template <class S, bool RELU>
+int launch_onchip(const typename S::elem *dy, const typename S::elem *x, const float *gamma, const float *beta,
+                  const float *save_mean, const float *save_invstd, typename S::elem *dx, float *dgamma, float *dbeta,
+                  void *workspace, const BnShape &s, const ChipPlan &p, hipStream_t st) {
+  unsigned long long *ws = static_cast<unsigned long long *>(workspace);
+  const dim3 grid(unsigned(s.C) * p.G);
+  const unsigned long long t1 = next_ticket(), t2 = next_ticket();
+  if (p.nt == 512)
+    hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean, save_invstd,
+                       dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit);
+  else
+    hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 1024>), grid, dim3(1024), 0, st, dy, x, gamma, beta, save_mean,
+                       save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
 // the one-pass kernel pays when a channel fits in LDS and there is a workgroup for at least half the CUs
 inline bool resident_ok(int N, int C, int HW, size_t esize) {
   return 2 * resident_half_bytes(N, HW, esize) <= kResidentLdsMax && C >= sgh_num_cus() / 2;
@@ -493,6 +715,16 @@ int bn_fwd_infer(const typename S::elem *x, const float *gamma, const float *bet
   return SGH_OK;
 }
 
+// bytes of workspace the backward pass of storage class S needs: the partial sums of the two-pass
+// kernels or the slots of the one-pass kernel, whichever the shape takes
+template <class S>
+inline size_t bwd_workspace_need(int N, int C, int HW) {
+  const size_t two_pass = size_t(C) * make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem))).S * 2 * sizeof(float);
+  const ChipPlan cp = chip_plan<S>(N, C, HW);
+  const size_t chip = cp.ok ? chip_workspace_bytes(C, cp.G) : 0;
+  return two_pass > chip ? two_pass : chip;
+}
+
 // beta != NULL selects the fused ReLU + BatchNorm backward
 template <class S>
 int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *gamma, const float *beta,
@@ -502,12 +734,21 @@ int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *g
     return SGH_EINVAL;
   if (!sgh_aligned16(x) || !sgh_aligned16(dy) || !sgh_aligned16(dx)) return SGH_EINVAL;
   const BnShape s = make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem)));
-  if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
+  if (!workspace || ws_bytes < bwd_workspace_need<S>(N, C, HW)) return SGH_EWORKSPACE;
   float *part = static_cast<float *>(workspace);
   const dim3 grid(C * s.S), block(kBlock);
   hipStream_t st = sgh_stream_of(stream);
   // algorithmic bytes: x and dy in, dx out (the fused form covers the ReLU backward as well)
   sgh_prof_scope prof(beta ? "bn_relu_bwd/k_bn_bwd" : "bn_bwd/k_bn_bwd", 3.0 * N * C * HW * sizeof(typename S::elem), st);
+  const ChipPlan cp = chip_plan<S>(N, C, HW);
+  // (channels of at most 4096 vectors that fit in LDS are a little faster through the LDS-resident kernel below:
+  // 13.4 against 14.9 us at 64 x 256 x 14 x 14 fp32)
+  const bool small_resident = resident_ok(N, C, HW, sizeof(typename S::elem)) && long(N) * (HW / S::VEC) <= 4096;
+  if (cp.ok && !small_resident && !sgh_env().bn_onchip_off) {
+    if (!sgh_aligned16(workspace)) return SGH_EINVAL;
+    return beta ? launch_onchip<S, true>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, workspace, s, cp, st)
+                : launch_onchip<S, false>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, workspace, s, cp, st);
+  }
   if (resident_ok(N, C, HW, sizeof(typename S::elem))) {
     const int rc = beta ? launch_resident<S, true>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, s, st)
                         : launch_resident<S, false>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, s, st);
@@ -562,7 +803,11 @@ size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
   // one size for every storage type: the larger of the fp32 and the 16-bit split counts
   const int s4 = make_shape(N, C, HW, 4, 4).S, s8 = make_shape(N, C, HW, 8, 2).S, s4h = make_shape(N, C, HW, 4, 2).S;
   const int smax = s4 > s8 ? (s4 > s4h ? s4 : s4h) : (s8 > s4h ? s8 : s4h);
-  return size_t(C) * smax * 2 * sizeof(float);
+  size_t need = size_t(C) * smax * 2 * sizeof(float);   // (the forward pass and the two-pass backward)
+  const size_t b[3] = {bwd_workspace_need<StF32>(N, C, HW), bwd_workspace_need<StF16>(N, C, HW),
+                       bwd_workspace_need<StF16x4>(N, C, HW)};
+  for (size_t v : b) need = v > need ? v : need;
+  return need;
 }
 
 // 16-bit planes that are a multiple of 4 but not of 8 elements (14 x 14) use the 8-byte vector class
@@ -598,13 +843,12 @@ int sgh_bn_bwd_noalloc_f32(const float *dy, const float *x, const float *gamma, 
                            const float *save_invstd, float *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                            void *stream) {
   if (!shape_ok(N, C, HW)) return SGH_EINVAL;
-  const size_t pairs = size_t(C) * make_shape(N, C, HW, StF32::VEC, int(sizeof(float))).S;
-  if (pairs > size_t(kNoAllocMaxPairs)) return SGH_ELIMIT;
+  const size_t need = bwd_workspace_need<StF32>(N, C, HW);
+  if (need > sizeof(float) * 2 * size_t(kNoAllocMaxPairs)) return SGH_ELIMIT;
   float *part = nullptr;  // (every slot the second kernel reads is written by the first: nothing to clear)
   const int rc = noalloc_scratch_of_current_device(&part);
   if (rc != SGH_OK) return rc;
-  return bn_bwd<StF32>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, part,
-                       pairs * 2 * sizeof(float), stream);
+  return bn_bwd<StF32>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, part, need, stream);
 }
 int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                    const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,

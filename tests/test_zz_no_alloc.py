@@ -45,17 +45,19 @@ def _case(singa, dev, shape, seed):
 
 def test_no_alloc_bn_bwd_two_calls_in_a_row(dev):
     from singa_amd import singa_wrap as singa
-    # split channels (two-pass kernels, partial sums through the library's buffer), then a smaller
-    # input with fewer channels and fewer splits, then an odd plane (scalar path)
+    # channels cut into slices (one-pass kernel, partial sums and tickets through the library's buffer),
+    # then a smaller input with fewer channels and slices, then an odd plane (two-pass kernels, scalar path),
+    # then the first shape again over what the others left in the buffer
     _case(singa, dev, (8, 48, 28, 28), 1)
     _case(singa, dev, (4, 16, 12, 12), 2)
     _case(singa, dev, (3, 5, 7, 5), 3)
+    _case(singa, dev, (8, 48, 28, 28), 4)
 
 
 def test_no_alloc_bn_bwd_rejects_sizes_beyond_its_buffer(dev):
     from singa_amd import singa_wrap as singa
     from singa_amd._lib import SGH_ELIMIT, lib
-    C = 20000
+    C = 40000      # 8 bytes of partial sums per channel: beyond the 256 KiB the library holds
     t = singa.Tensor((1, C, 1, 1), dev)
     t.SetFloatValue(0.0)
     v = singa.Tensor((C,), dev)
