@@ -379,6 +379,16 @@ SGH_API void sgh_conv_weights_changed(void);
  * The split reduction is summed in a fixed order: results are run-to-run identical. */
 SGH_API int sgh_conv_wgrad_f32(sgh_conv_geom *g, const float *dy, const float *x, float *dW,
                                void *workspace, size_t ws_bytes, void *stream);
+/* GpuConvBackwardW and GpuConvBackwardb of one layer in one call (the reference makes two cuDNN
+ * calls, src/model/operation/convolution.cc:658-702, both reading dy).  Where the generic
+ * implicit-GEMM kernel runs the weight gradient and its last column tile has a spare column
+ * (C*R*S not a multiple of the tile width), db is computed by the same matrix instructions as one
+ * more column of the x operand -- a column of ones -- so dy is read once; other geometries run
+ * the reduction of sgh_conv_bgrad_f32 behind the weight gradient.  Either way db agrees with
+ * sgh_conv_bgrad_f32 to rounding (different summation order).  Workspace as for the weight
+ * gradient. */
+SGH_API int sgh_conv_wgrad_bias_f32(sgh_conv_geom *g, const float *dy, const float *x, float *dW,
+                                    float *db, void *workspace, size_t ws_bytes, void *stream);
 /* GpuConvBackwardb (src/model/operation/convolution.cc:684-702; native CPU :425-440):
  * db[k] = sum_{n,p,q} dy[n,k,p,q]. */
 SGH_API int sgh_conv_bgrad_f32(const sgh_conv_geom *g, const float *dy, float *db, void *stream);

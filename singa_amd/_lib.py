@@ -133,6 +133,7 @@ SIGNATURES = {
     "sgh_conv_dgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_dgrad_acc_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_wgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
+    "sgh_conv_wgrad_bias_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
     "sgh_conv_bgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp]),
     "sgh_conv_fwd_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
     "sgh_conv_workspace_bytes_h": (sz, [C.POINTER(ConvGeom), C.c_int]),

@@ -211,11 +211,17 @@ struct WgradXLoader {
   int off[ROWS * BK / NT];
   short dr[ROWS * BK / NT], ds[ROWS * BK / NT];
   int h0_, w0_, base_, ok_;
+  // Column `ones_col` (CRS when the bias gradient rides along, else -1) is a column of ones over the
+  // valid pixels: its dot product with a dy row is that row's sum, i.e. db[k], from the same MFMAs.
+  int ones_col;
+  unsigned ones_mask;   // staged rows of this thread that are that column
   __device__ __forceinline__ void init(int tile_col0, int t) {
     const int RS = g.R * g.S;
+    ones_mask = 0u;
 #pragma unroll
     for (int e = 0; e < M::E; ++e) {
       const int j = tile_col0 + M::row0(t) + e * M::ROW_STEP;
+      if (j == ones_col) ones_mask |= 1u << e;
       if (j < CRS) {
         const int c = j / RS, rs = j - c * RS, fr = rs / g.S, fs = rs - fr * g.S;
         dr[e] = short(fr - g.ph);
@@ -242,7 +248,8 @@ struct WgradXLoader {
     const int h = h0_ + dr[e], w = w0_ + ds[e];
     // unsigned compares fold the two-sided range checks
     const int v = ok_ & int(unsigned(h) < unsigned(g.H)) & int(unsigned(w) < unsigned(g.W));
-    return buf_ld(make_rsrc(x, bytes), base_ + off[e], v);
+    const float xv = buf_ld(make_rsrc(x, bytes), base_ + off[e], v);
+    return (ones_mask >> e) & 1u ? (ok_ ? 1.f : 0.f) : xv;
   }
 };
 
@@ -403,11 +410,13 @@ struct DilateStore {
   }
 };
 
-struct SplitStore {  // partial[split][m * N + n]
+struct SplitStore {  // partial[split][m * N + n]; column N, if wanted, goes to bpart[split][m]
   float *part;
   int M, N;
+  float *bpart;
   __device__ __forceinline__ void operator()(int m, int n, float v) const {
     if (m < M && n < N) part[long(blockIdx.z) * M * N + long(m) * N + n] = v;
+    else if (bpart && m < M && n == N) bpart[long(blockIdx.z) * M + m] = v;
   }
 };
 
@@ -893,7 +902,8 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
       const size_t fewc = sgh_wgrad_fewc_workspace_bytes(g);
       if (fewc) return fewc;
       const WgradPlan p = plan_wgrad(g);
-      return p.splits > 1 ? size_t(p.splits) * g->K * g->C * RS * sizeof(float) : 0;
+      // split partials of dW, then those of the bias gradient that may ride along (sgh_conv_wgrad_bias_f32)
+      return p.splits > 1 ? align256(size_t(p.splits) * g->K * g->C * RS * sizeof(float)) + size_t(p.splits) * g->K * sizeof(float) : 0;
     }
     default: return 0;
   }
@@ -1258,21 +1268,30 @@ int sgh_conv_fwd_f32(sgh_conv_geom *g, const float *x, const float *W, const flo
   return SGH_OK;
 }
 
-int sgh_conv_wgrad_f32(sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
-                       size_t ws_bytes, void *stream) {
+static int bgrad_launch(const sgh_conv_geom *g, const float *dy, float *db, hipStream_t s) {
+  hipLaunchKernelGGL(k_conv_bgrad<StF32>, dim3(g->K), dim3(NT), 0, s, dy, db, g->N, g->K, g->P * g->Q);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+// `db` (may be null): the bias gradient as well.  In the generic kernel it rides along as one more column
+// of the x operand (a column of ones) whenever the last column tile has a spare column; the shared-tile
+// and few-channel kernels are followed by the reduction kernel of sgh_conv_bgrad_f32.
+static int conv_wgrad(sgh_conv_geom *g, const float *dy, const float *x, float *dW, float *db, void *workspace,
+                      size_t ws_bytes, void *stream) {
   if (!conv_ok(g) || !dy || !x || !dW) return SGH_EINVAL;
   sgh_prelaid_clear_if_overlap(g, workspace, ws_bytes);
   if (sgh_wgrad3x3_workspace_bytes(g)) {  // 3x3, stride 1 or 2: shared-input-tile kernel
     sgh_prof_start("conv_wgrad_op", conv_flops(g), sgh_stream_of(stream));
     const int rc3 = sgh_wgrad3x3_run(g, dy, x, dW, workspace, ws_bytes, sgh_stream_of(stream));
     sgh_prof_stop(sgh_stream_of(stream));
-    return rc3;
+    return rc3 == SGH_OK && db ? bgrad_launch(g, dy, db, sgh_stream_of(stream)) : rc3;
   }
   if (sgh_wgrad_fewc_workspace_bytes(g)) {  // few input channels, large filter (the stem)
     sgh_prof_start("conv_wgrad_op", conv_flops(g), sgh_stream_of(stream));
     const int rcf = sgh_wgrad_fewc_run(g, dy, x, dW, workspace, ws_bytes, sgh_stream_of(stream));
     sgh_prof_stop(sgh_stream_of(stream));
-    return rcf;
+    return rcf == SGH_OK && db ? bgrad_launch(g, dy, db, sgh_stream_of(stream)) : rcf;
   }
   const WgradPlan p = plan_wgrad(g);
   const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_WGRAD);
@@ -1281,7 +1300,12 @@ int sgh_conv_wgrad_f32(sgh_conv_geom *g, const float *dy, const float *x, float 
   const int CRS = g->C * g->R * g->S, PQ = g->P * g->Q;
   const long G = long(g->N) * PQ;
   float *part = p.splits > 1 ? static_cast<float *>(workspace) : dW;
-  SplitStore st{part, g->K, CRS};
+  const bool ride = db && CRS % p.bn != 0;   // a spare column in the last column tile
+  float *bpart = !ride ? nullptr
+                 : p.splits > 1 ? reinterpret_cast<float *>(static_cast<char *>(workspace) +
+                                                            align256(size_t(p.splits) * g->K * CRS * sizeof(float)))
+                                : db;
+  SplitStore st{part, g->K, CRS, bpart};
   int rc;
   sgh_prof_start("conv_wgrad_op", conv_flops(g), s);
 #define SGH_WGRAD_CASE(BM_, BN_, WGM_)                                                                             \
@@ -1291,6 +1315,7 @@ int sgh_conv_wgrad_f32(sgh_conv_geom *g, const float *dy, const float *x, float 
     lb.x = x;                                                                                                      \
     lb.g = to_g(g);                                                                                                \
     lb.CRS = CRS;                                                                                                  \
+    lb.ones_col = ride ? CRS : -1;                                                                                 \
     lb.bytes = bytes_of(size_t(g->N) * g->C * g->H * g->W);                                                        \
     rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true, false, WGM_>(       \
         la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s, "conv_wgrad/k_igemm", conv_flops(g));              \
@@ -1311,12 +1336,25 @@ int sgh_conv_wgrad_f32(sgh_conv_geom *g, const float *dy, const float *x, float 
       if (blocks > 2048) blocks = 2048;
       hipLaunchKernelGGL(k_split_reduce, dim3(int(blocks)), dim3(NT), 0, s, part, dW, n, p.splits);
     }
+    if (ride) hipLaunchKernelGGL(k_split_reduce, dim3((g->K + NT - 1) / NT), dim3(NT), 0, s, bpart, db, long(g->K), p.splits);
   }
   sgh_prof_stop(s);
   if (rc != SGH_OK) return rc;
   SGH_LAUNCH_CHECK();
-  return SGH_OK;
+  return db && !ride ? bgrad_launch(g, dy, db, s) : SGH_OK;
 }
+
+int sgh_conv_wgrad_f32(sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace,
+                       size_t ws_bytes, void *stream) {
+  return conv_wgrad(g, dy, x, dW, nullptr, workspace, ws_bytes, stream);
+}
+
+int sgh_conv_wgrad_bias_f32(sgh_conv_geom *g, const float *dy, const float *x, float *dW, float *db, void *workspace,
+                            size_t ws_bytes, void *stream) {
+  if (!db) return SGH_EINVAL;
+  return conv_wgrad(g, dy, x, dW, db, workspace, ws_bytes, stream);
+}
+
 
 int sgh_conv_bgrad_f32(const sgh_conv_geom *g, const float *dy, float *db, void *stream) {
   if (!conv_ok(g) || !dy || !db) return SGH_EINVAL;

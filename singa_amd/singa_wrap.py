@@ -698,6 +698,21 @@ def GpuConvBackwardW(dy, x, W, h, stream=None):
     return dW
 
 
+def GpuConvBackwardWb(dy, x, W, b, h):
+    """``GpuConvBackwardW`` and ``GpuConvBackwardb`` of one layer in one call: ``(dW, db)``.  Where the
+    generic kernel computes the weight gradient the bias gradient rides along in its matrix
+    instructions and dy is read once (fp32 tensors; other types make the two calls)."""
+    if dy.data_type() != kFloat32:
+        return GpuConvBackwardW(dy, x, W, h), GpuConvBackwardb(dy, b, h)
+    h._check_dy(dy)
+    h._check_x(x)
+    dW, db = _like(W), _like(b)
+    ws = h.workspace
+    check(_L().sgh_conv_wgrad_bias_f32(C.byref(h.geom), dy.ptr, x.ptr, dW.ptr, db.ptr, ws.ptr, ws.MemSize(),
+                                       dy.device().stream), "sgh_conv_wgrad_bias_f32")
+    return dW, db
+
+
 def GpuConvPrepareBackward(weights_and_handles):
     """Re-lays the weights of all listed convolutions for their data gradients in ONE launch (the
     re-layout each ``GpuConvBackwardx`` otherwise launches for itself); `weights_and_handles`: pairs

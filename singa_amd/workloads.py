@@ -136,6 +136,12 @@ class HipOps(object):
     def conv_bwd_b(self, dy, b, h):
         return singa.GpuConvBackwardb(dy, b, h)
 
+    # cross-op fusion the tape permits: a layer's bias gradient computed with its weight gradient
+    fuse_wgrad_bias = True
+
+    def conv_bwd_wb(self, dy, x, W, b, h):
+        return singa.GpuConvBackwardWb(dy, x, W, b, h)
+
     # cross-op fusion the tape permits: a residual block hands its input gradient on as two summands
     # and the ReLU backward of the block before adds them while gating (HalfHipOps turns it on)
     fuse_add_relu = False
@@ -166,11 +172,11 @@ class HipOps(object):
             self.dev.Join()    # the update (and any reader of a weight gradient) comes after the last of them
             self._aux = None
 
-    fusions = ("fuse_bn_relu", "fuse_dgrad_add", "batch_relayout", "overlap_wgrad")   # what set_fusion(True) turns on
+    fusions = ("fuse_bn_relu", "fuse_dgrad_add", "fuse_wgrad_bias", "batch_relayout", "overlap_wgrad")   # what set_fusion(True) turns on
 
     def set_fusion(self, on):
         """All of this implementation's cross-op fusions on, or the reference's op-per-op tape."""
-        for f in ("fuse_bn_relu", "fuse_dgrad_add", "fuse_add_relu", "batch_relayout", "overlap_wgrad"):
+        for f in ("fuse_bn_relu", "fuse_dgrad_add", "fuse_add_relu", "fuse_wgrad_bias", "batch_relayout", "overlap_wgrad"):
             setattr(self, f, bool(on) and f in self.fusions)
 
     def accumulate(self, a, b):
@@ -212,7 +218,7 @@ class HalfHipOps(HipOps):
     # scattered 2-byte stores make a read-modify-write epilogue slower than the separate add)
     fuse_dgrad_add = False
     fuse_add_relu = True
-    fusions = ("fuse_bn_relu", "fuse_add_relu", "batch_relayout", "overlap_wgrad")
+    fusions = ("fuse_bn_relu", "fuse_add_relu", "fuse_wgrad_bias", "batch_relayout", "overlap_wgrad")
 
     def __init__(self, dev, dtype):
         HipOps.__init__(self, dev)
@@ -269,6 +275,7 @@ class Conv(_Layer):
         # A weight gradient that goes to the auxiliary stream is enqueued first, so that it starts beside
         # this layer's data gradient instead of behind it (it has a workspace of its own there).
         early = getattr(self.ops, "_aux", None) is not None
+        db = None
         if early:
             dW = self.ops.conv_bwd_w(dy, self.x, self.W, self.h)
         # _Conv2d.backward: dx is always computed, even for the network input (autograd.py:1695-1697)
@@ -277,10 +284,13 @@ class Conv(_Layer):
         else:
             dx = self.ops.conv_bwd_x(dy, self.W, self.x, self.h)
         if not early:
-            dW = self.ops.conv_bwd_w(dy, self.x, self.W, self.h)
+            if self.b is not None and getattr(self.ops, "fuse_wgrad_bias", False):
+                dW, db = self.ops.conv_bwd_wb(dy, self.x, self.W, self.b, self.h)
+            else:
+                dW = self.ops.conv_bwd_w(dy, self.x, self.W, self.h)
         grads(self.name + ".W", self.W, dW)
         if self.b is not None:
-            grads(self.name + ".b", self.b, self.ops.conv_bwd_b(dy, self.b, self.h))
+            grads(self.name + ".b", self.b, db if db is not None else self.ops.conv_bwd_b(dy, self.b, self.h))
         return dx
 
 

@@ -115,6 +115,31 @@ def test_conv_backward_vs_oracle(singa, dev, case):
     assert nl2(y, O.conv_fwd(x, w, b, stride, pad)) < TOL
 
 
+@pytest.mark.parametrize("case", [c for c in CONV_CASES if c[-1]] + [
+    (4, 32, 16, 16, 64, 5, 5, (1, 1), (2, 2), True),      # generic kernel, split reduction: db rides along as a column of ones
+    (1, 20, 6, 6, 40, 5, 5, (1, 1), (2, 2), True),        # ... without a split (one chunk range): written straight to db
+    (2, 32, 9, 9, 16, 2, 2, (1, 1), (0, 0), True),        # C*R*S = 128, a whole number of column tiles: the reduction kernel instead
+])
+def test_conv_weight_and_bias_gradient_in_one_call(singa, dev, case):
+    """GpuConvBackwardWb: dW bit-identical to GpuConvBackwardW (same kernel, the extra column changes no
+    other sum), db within the reduction bar of the CPU oracle and of GpuConvBackwardb."""
+    N, C, H, W, K, R, S, stride, pad, _ = case
+    r = rng(abs(hash(case)) % 2**31 + 5)
+    x, w, b = randn(r, N, C, H, W), randn(r, K, C, R, S), randn(r, K)
+    P, Q = (H + 2 * pad[0] - R) // stride[0] + 1, (W + 2 * pad[1] - S) // stride[1] + 1
+    dy = (randn(r, N, K, P, Q) + 0.25).astype(np.float32)    # (a mean, so that db is not a sum that cancels)
+    xd, wd, bd, dyd = (singa.from_numpy(a, dev) for a in (x, w, b, dy))
+    h = singa.CudnnConvHandle(xd, (R, S), stride, pad, C, K, True)
+    dW, db = singa.GpuConvBackwardWb(dyd, xd, wd, bd, h)
+    assert_bit_equal(dW.to_numpy(), singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy(), "dW")
+    want = O.conv_bgrad(dy)
+    e = (nl2(db.to_numpy(), want), nl2(db.to_numpy(), singa.GpuConvBackwardb(dyd, bd, h).to_numpy()))
+    print("db nl2 vs oracle %.2e, vs the separate kernel %.2e" % e)
+    assert max(e) < TOL
+    dW2, db2 = singa.GpuConvBackwardWb(dyd, xd, wd, bd, h)     # run-to-run identical
+    assert_bit_equal(db2.to_numpy(), db.to_numpy(), "db again")
+
+
 def test_conv_dgrad_with_batched_weight_relayout(singa, dev):
     """GpuConvPrepareBackward re-lays the weights of all CONV_CASES layers in one launch; the data
     gradients (plain and accumulating) that follow skip their own re-layout and must give the same
