@@ -172,6 +172,41 @@ SGH_API int sgh_softmax_fwd_f32(const float *x, float *p, size_t batch, size_t d
 SGH_API int sgh_cross_entropy_fwd_f32(const float *p, const int32_t *t, float *loss, size_t batch,
                                       size_t dim, int int_target, void *stream);
 
+/* Transform<float, Lang> (src/core/tensor/tensor_math_cpp.h:685-689, CUDA tensor_math_cuda.h:284-300):
+ * the dense row-major copy of a strided view -- transposed, sliced or broadcast (stride 0, as
+ * Tensor::Broadcast makes them, src/core/tensor/tensor.cc:481-503).  Element i of `out`, in
+ * row-major order of `shape`, is in[sum_d index_d * strides[d]] (strides in elements, innermost
+ * dimension last, at most SGH_MAX_DIMS dimensions) -- the walk of next_offset,
+ * tensor_math_cpp.h:126-138.  What the reference's CUDA EltwiseMult / Add do first with an operand
+ * that is not dense (tensor_math_cuda.h:300-362). */
+#define SGH_MAX_DIMS 8
+SGH_API int sgh_transform_f32(const float *in, float *out, int ndim, const size_t *shape,
+                              const int64_t *strides, void *stream);
+/* RowMax<float, Lang> (tensor_math_cpp.h:1122-1140): out[r] = max(0, max_c in[r][c]) for a dense
+ * nrow x ncol matrix -- the CPU function seeds the maximum with 0 (the CUDA kernel with the row's
+ * first element, math_kernel.cu:493); the CPU path is the one results are compared with. */
+SGH_API int sgh_row_max_f32(const float *in, float *out, size_t nrow, size_t ncol, void *stream);
+/* Dot<float, Lang> with a Tensor result (tensor_math_cpp.h:839-849, cublasSdot in device pointer
+ * mode tensor_math_cuda.h:1084-1092) and Sum<float, Lang> over all elements (tensor_math_cpp.h:
+ * 655-663): *out = sum a[i] * b[i] / sum a[i], `out` in device memory.  Summed in an order that
+ * depends on n only: run-to-run identical.  workspace: sgh_reduce_workspace_bytes() bytes. */
+SGH_API size_t sgh_reduce_workspace_bytes(void);
+SGH_API int sgh_dot_f32(const float *a, const float *b, size_t n, float *out, void *workspace,
+                        size_t ws_bytes, void *stream);
+SGH_API int sgh_sum_all_f32(const float *a, size_t n, float *out, void *workspace, size_t ws_bytes,
+                            void *stream);
+/* Uniform<float, Lang> / Gaussian<float, Lang> (tensor_math_cpp.h:712-740; cuRAND in
+ * tensor_math_cuda.h:950-1000).  The reference draws from the device's generator state
+ * (Device::SetRandSeed); here element i of a fill is a pure function of (seed, offset + i): the
+ * (offset + i)-th output of splitmix64 seeded with `seed` gives a double in [0, 1), a Gaussian
+ * takes two of them (offset + 2i, offset + 2i + 1) through Box-Muller in double precision.  The
+ * caller advances `offset` by n (2n) per fill to continue the stream.  The reference's streams
+ * (std::mt19937, cuRAND) are not reproduced: no test of the reference depends on their values. */
+SGH_API int sgh_uniform_f32(float low, float high, float *out, size_t n, uint64_t seed,
+                            uint64_t offset, void *stream);
+SGH_API int sgh_gaussian_f32(float mean, float std, float *out, size_t n, uint64_t seed,
+                             uint64_t offset, void *stream);
+
 /* Axpy<float, Lang>, scalar and Tensor-alpha overloads: tensor_math.h:393-402;
  * CPU tensor_math_cpp.h:788-823; CUDA tensor_math_cuda.h:1031-1072 (device pointer mode).
  * y += alpha * x. */

@@ -287,3 +287,63 @@ def sum_rows(m):
     out, po = _out((m.shape[1],))
     lib().oracle_sum_rows(pm, po, C.c_int(m.shape[0]), C.c_int(m.shape[1]))
     return out
+
+
+# ---- the remaining tensor functions (Transform, RowMax, Dot, Sum) and the seeded input generator
+
+def transform(a, shape, strides):
+    """Dense row-major copy of the view (shape, strides in elements) of the flat array `a`."""
+    a, pa = _f(a)
+    shape = [int(s) for s in shape]
+    out, po = _out(shape)
+    sh = (C.c_size_t * len(shape))(*shape)
+    st = (C.c_long * len(shape))(*[int(s) for s in strides])
+    lib().oracle_transform(pa, po, C.c_int(len(shape)), sh, st)
+    return out
+
+
+def row_max(m):
+    m, pm = _f(m)
+    out, po = _out((m.shape[0],))
+    lib().oracle_row_max(pm, po, C.c_size_t(m.shape[0]), C.c_size_t(m.shape[1]))
+    return out
+
+
+def dot(a, b):
+    a, pa = _f(a)
+    b, pb = _f(b)
+    fn = lib().oracle_dot
+    fn.restype = C.c_float
+    return float(fn(pa, pb, C.c_size_t(a.size)))
+
+
+def sum_all(a):
+    a, pa = _f(a)
+    fn = lib().oracle_sum_all
+    fn.restype = C.c_float
+    return float(fn(pa, C.c_size_t(a.size)))
+
+
+def rng_raw(seed, k):
+    fn = lib().oracle_rng_raw
+    fn.restype = C.c_uint64
+    return int(fn(C.c_uint64(seed), C.c_uint64(k)))
+
+
+def rng_uniform(seed, n, low=0.0, high=1.0, offset=0):
+    out, po = _out((n,))
+    lib().oracle_rng_uniform(C.c_uint64(seed), C.c_uint64(offset), C.c_double(low), C.c_double(high), po, C.c_size_t(n))
+    return out
+
+
+def rng_normal(seed, n, mean=0.0, std=1.0, offset=0):
+    out, po = _out((n,))
+    lib().oracle_rng_normal(C.c_uint64(seed), C.c_uint64(offset), C.c_double(mean), C.c_double(std), po, C.c_size_t(n))
+    return out
+
+
+def rng_integers(seed, n, hi, offset=0):
+    out = np.empty(n, dtype=np.int32)
+    lib().oracle_rng_integers(C.c_uint64(seed), C.c_uint64(offset), C.c_uint64(hi), out.ctypes.data_as(C.c_void_p),
+                              C.c_size_t(n))
+    return out

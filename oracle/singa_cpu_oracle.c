@@ -615,3 +615,84 @@ ORACLE_API void oracle_sum_rows(const float *m, float *out, int rows, int cols) 
   for (int i = 0; i < rows; ++i)
     for (int j = 0; j < cols; ++j) out[j] += m[(size_t)i * cols + j];
 }
+
+/* ------------------------------------------------------------- the remaining tensor functions */
+
+/* Transform<float, lang::Cpp>, src/core/tensor/tensor_math_cpp.h:685-689 = traverse_unary with the
+ * identity over a view that is not dense: the offset walk of next_offset, :126-138 (the last
+ * dimension moves first; `stride` in elements, 0 for a broadcast dimension).
+ * Pinned by: NumPy's as_strided / broadcast_to / transpose on random views. */
+ORACLE_API void oracle_transform(const float *in, float *out, int ndim, const size_t *shape,
+                                 const long *stride) {
+  size_t n = 1;
+  for (int d = 0; d < ndim; ++d) n *= shape[d];
+  size_t index[16] = {0};
+  long offset = 0;
+  for (size_t i = 0; i < n; ++i) {
+    out[i] = in[offset];
+    for (int k = ndim - 1; k >= 0; --k) {
+      if (index[k] + 1 < shape[k]) {
+        offset += stride[k];
+        index[k] += 1;
+        break;
+      }
+      index[k] = 0;
+      offset -= stride[k] * (long)(shape[k] - 1);
+    }
+  }
+}
+
+/* RowMax<float, lang::Cpp>, tensor_math_cpp.h:1122-1140: the running maximum starts at 0, not at
+ * the row's first element.  Pinned by: numpy.maximum(0, x.max(axis=1)) incl. all-negative rows. */
+ORACLE_API void oracle_row_max(const float *in, float *out, size_t nrow, size_t ncol) {
+  for (size_t r = 0; r < nrow; ++r) {
+    float maxval = 0;
+    for (size_t c = 0; c < ncol; ++c) maxval = in[r * ncol + c] > maxval ? in[r * ncol + c] : maxval;
+    out[r] = maxval;
+  }
+}
+
+/* Dot<float, lang::Cpp>, tensor_math_cpp.h:827-849: cblas_sdot (OpenBLAS, not vendored: its
+ * summation order is not reproduced; the published definition sum_i x[i] * y[i] is, accumulated
+ * in order).  Sum<float, lang::Cpp>, :655-663: a sequential float sum.
+ * Pinned by: float64 NumPy within |error| <= 1e-6 * sum |terms|. */
+ORACLE_API NO_CONTRACT float oracle_dot(const float *a, const float *b, size_t n) {
+  float s = 0.f;
+  for (size_t i = 0; i < n; ++i) s += a[i] * b[i];
+  return s;
+}
+ORACLE_API float oracle_sum_all(const float *a, size_t n) {
+  float s = 0.f;
+  for (size_t i = 0; i < n; ++i) s += a[i];
+  return s;
+}
+
+/* ------------------------------------------------------------- seeded synthetic inputs
+ * A counter-based generator, so that the benchmark's inputs do not depend on any library's random
+ * stream: the k-th output of splitmix64 seeded with `seed` is mix(seed + (k + 1) * golden).
+ * uniform: (out >> 11) * 2^-53 in [0, 1); normal: Box-Muller in double on outputs 2i and 2i + 1,
+ * rounded to float once; integers: out % hi.  The Python twin is singa_amd/rng.py; the test-suite
+ * holds the two to each other and to known splitmix64 outputs.  (Not a restatement of the
+ * reference: SINGA draws from std::mt19937, tensor_math_cpp.h:712-740, whose streams no reference
+ * test depends on.) */
+static uint64_t splitmix64_at(uint64_t seed, uint64_t k) {
+  uint64_t z = seed + (k + 1u) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+ORACLE_API uint64_t oracle_rng_raw(uint64_t seed, uint64_t k) { return splitmix64_at(seed, k); }
+ORACLE_API void oracle_rng_uniform(uint64_t seed, uint64_t offset, double low, double high, float *out, size_t n) {
+  for (size_t i = 0; i < n; ++i)
+    out[i] = (float)(low + (double)(splitmix64_at(seed, offset + i) >> 11) * 0x1.0p-53 * (high - low));
+}
+ORACLE_API void oracle_rng_normal(uint64_t seed, uint64_t offset, double mean, double std, float *out, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    const double u1 = (double)(splitmix64_at(seed, offset + 2 * i) >> 11) * 0x1.0p-53;
+    const double u2 = (double)(splitmix64_at(seed, offset + 2 * i + 1) >> 11) * 0x1.0p-53;
+    out[i] = (float)(mean + std * (sqrt(-2.0 * log(1.0 - u1)) * cos(6.283185307179586476925286766559 * u2)));
+  }
+}
+ORACLE_API void oracle_rng_integers(uint64_t seed, uint64_t offset, uint64_t hi, int *out, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = (int)(splitmix64_at(seed, offset + i) % hi);
+}

@@ -85,6 +85,13 @@ SIGNATURES = {
     "sgh_softmax_ce_label_errors": (C.c_int, [vp, C.POINTER(C.c_int)]),
     "sgh_softmax_fwd_f32": (C.c_int, [vp, vp, sz, sz, vp]),
     "sgh_cross_entropy_fwd_f32": (C.c_int, [vp, vp, vp, sz, sz, C.c_int, vp]),
+    "sgh_transform_f32": (C.c_int, [vp, vp, C.c_int, C.POINTER(C.c_size_t), C.POINTER(C.c_int64), vp]),
+    "sgh_row_max_f32": (C.c_int, [vp, vp, sz, sz, vp]),
+    "sgh_reduce_workspace_bytes": (sz, []),
+    "sgh_dot_f32": (C.c_int, [vp, vp, sz, vp, vp, sz, vp]),
+    "sgh_sum_all_f32": (C.c_int, [vp, sz, vp, vp, sz, vp]),
+    "sgh_uniform_f32": (C.c_int, [C.c_float, C.c_float, vp, sz, C.c_uint64, C.c_uint64, vp]),
+    "sgh_gaussian_f32": (C.c_int, [C.c_float, C.c_float, vp, sz, C.c_uint64, C.c_uint64, vp]),
     "sgh_axpy_f32": (C.c_int, [C.c_float, vp, vp, sz, vp]),
     "sgh_axpy_devalpha_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_eltwise_mult_f32": (C.c_int, [vp, vp, C.c_int, vp, sz, vp]),

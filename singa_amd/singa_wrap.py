@@ -87,6 +87,25 @@ class HipGPU(object):
     def Sync(self):
         check(_L().sgh_device_sync(self._h), "sgh_device_sync")
 
+    # Device::SetRandSeed (include/singa/core/device.h:64): the state behind Uniform / Gaussian is a seed
+    # and a count of outputs consumed; a fill of n elements takes the next n (Gaussian: 2n) outputs
+    _rand_seed, _rand_offset = 0, 0
+
+    def SetRandSeed(self, seed):
+        self._rand_seed, self._rand_offset = int(seed) & 0xFFFFFFFFFFFFFFFF, 0
+
+    def _take_random(self, count):
+        off = self._rand_offset
+        self._rand_offset += int(count)
+        return self._rand_seed, off
+
+    _reduce_ws = None
+
+    def reduce_workspace(self):
+        if self._reduce_ws is None:
+            self._reduce_ws = Tensor((_L().sgh_reduce_workspace_bytes() // 4,), self, kFloat32)
+        return self._reduce_ws
+
     # A second compute stream for work that the main stream's next ops do not depend on.  Fork():
     # what is enqueued on the auxiliary stream afterwards starts when everything enqueued on the main
     # stream so far has finished; Join(): the main stream waits for the auxiliary one.  Tensors handed
@@ -358,6 +377,101 @@ def _need_f32(what, *tensors):
             raise SingaHipError("%s: float32 tensors only, got data type %r" % (what, t.data_type()))
 
 
+def Transform(t):
+    """``singa.Transform``: the dense copy of a view (here: a transposed 2-D view; dense tensors are
+    returned as they are)."""
+    if not t.transpose():
+        return t
+    _need_f32("Transform", t)
+    rows, cols = t.shape()
+    out = Tensor((rows, cols), t.device(), kFloat32)
+    shape = (C.c_size_t * 2)(rows, cols)
+    strides = (C.c_int64 * 2)(1, rows)       # element (i, j) of the view is element (j, i) of the stored matrix
+    check(_L().sgh_transform_f32(t.ptr, out.ptr, 2, shape, strides, t.device().stream), "sgh_transform_f32")
+    return out
+
+
+def Broadcast(t, shape):
+    """``Tensor::Broadcast`` (src/core/tensor/tensor.cc:481-503) made dense: NumPy's broadcasting
+    rules, trailing dimensions aligned, stride 0 along every broadcast dimension."""
+    _need_f32("Broadcast", t)
+    t = Transform(t)
+    shape = tuple(int(v) for v in shape)
+    src = (1,) * (len(shape) - t.nDim()) + tuple(t.shape())
+    if len(src) != len(shape) or any(a != b and a != 1 for a, b in zip(src, shape)):
+        raise SingaHipError("cannot broadcast %s to %s" % (t.shape(), list(shape)))
+    if len(shape) > 8:
+        raise SingaHipError("at most 8 dimensions")
+    strides, acc = [], 1
+    for a in reversed(src):
+        strides.append(acc)
+        acc *= a
+    strides = [0 if a == 1 and b != 1 else st for a, b, st in zip(src, shape, reversed(strides))]
+    out = Tensor(shape, t.device(), kFloat32)
+    check(_L().sgh_transform_f32(t.ptr, out.ptr, len(shape), (C.c_size_t * len(shape))(*shape),
+                                 (C.c_int64 * len(shape))(*strides), t.device().stream), "sgh_transform_f32")
+    return out
+
+
+def _dense_pair(a, b):
+    """Operands of an elementwise function as two dense tensors of one shape: what the reference's GPU
+    path does with views that are not dense (Transform first, tensor_math_cuda.h:300-362)."""
+    a, b = Transform(a), Transform(b)
+    if a.shape() == b.shape():
+        return a, b
+    sa, sb = a.shape(), b.shape()
+    n = max(len(sa), len(sb))
+    pa, pb = [1] * (n - len(sa)) + sa, [1] * (n - len(sb)) + sb
+    if any(x != y and x != 1 and y != 1 for x, y in zip(pa, pb)):
+        raise SingaHipError("shapes %s and %s do not broadcast" % (sa, sb))
+    shape = [max(x, y) for x, y in zip(pa, pb)]
+    return (a if sa == shape else Broadcast(a, shape)), (b if sb == shape else Broadcast(b, shape))
+
+
+def RowMax(t):
+    """``singa.RowMax``: per row max(0, max over the row) (the CPU rule, tensor_math_cpp.h:1122-1140)."""
+    _need_f32("RowMax", t)
+    t = Transform(t)
+    if t.nDim() != 2:
+        raise SingaHipError("RowMax expects a matrix")
+    out = Tensor((t.shape(0),), t.device(), kFloat32)
+    check(_L().sgh_row_max_f32(t.ptr, out.ptr, t.shape(0), t.shape(1), t.device().stream), "sgh_row_max_f32")
+    return out
+
+
+def Dot(a, b):
+    """``singa.Dot(a, b)`` with a Tensor result: a 1-element tensor on the device."""
+    _need_f32("Dot", a, b)
+    if a.Size() != b.Size() or a.transpose() or b.transpose():
+        raise SingaHipError("Dot expects two dense tensors of one size")
+    out, ws = Tensor((1,), a.device(), kFloat32), a.device().reduce_workspace()
+    check(_L().sgh_dot_f32(a.ptr, b.ptr, a.Size(), out.ptr, ws.ptr, ws.MemSize(), a.device().stream), "sgh_dot_f32")
+    return out
+
+
+def SumAll(t):
+    """``singa.SumAll(t)``: the sum of all elements as a Python float (blocks until it is there)."""
+    _need_f32("SumAll", t)
+    out, ws = Tensor((1,), t.device(), kFloat32), t.device().reduce_workspace()
+    check(_L().sgh_sum_all_f32(t.ptr, t.Size(), out.ptr, ws.ptr, ws.MemSize(), t.device().stream), "sgh_sum_all_f32")
+    return float(out.to_numpy()[0])
+
+
+def Uniform(low, high, t):
+    """``singa.Uniform(low, high, t)``: fills `t` from the device's generator state (``SetRandSeed``)."""
+    _need_f32("Uniform", t)
+    seed, off = t.device()._take_random(t.Size())
+    check(_L().sgh_uniform_f32(float(low), float(high), t.ptr, t.Size(), seed, off, t.device().stream), "sgh_uniform_f32")
+
+
+def Gaussian(mean, std, t):
+    """``singa.Gaussian(mean, std, t)``."""
+    _need_f32("Gaussian", t)
+    seed, off = t.device()._take_random(2 * t.Size())
+    check(_L().sgh_gaussian_f32(float(mean), float(std), t.ptr, t.Size(), seed, off, t.device().stream),
+          "sgh_gaussian_f32")
+
+
 def _same(a, b):
     if a.Size() != b.Size() or a.data_type() != b.data_type():
         raise SingaHipError("shape/type mismatch: %s vs %s" % (a.shape(), b.shape()))
@@ -495,8 +609,10 @@ def Axpy(alpha, x, y):
 
 
 def EltwiseMult(a, b, out=None):
-    out = _like(a) if out is None else out
     scalar = b.Size() == 1 and a.Size() != 1
+    if not scalar and a.data_type() == kFloat32 and (a.shape() != b.shape() or a.transpose() or b.transpose()):
+        a, b = _dense_pair(a, b)     # broadcast / transposed operands
+    out = _like(a) if out is None else out
     if not scalar:
         _same(a, b)
     if a.data_type() != kFloat32:
@@ -511,6 +627,8 @@ def EltwiseMult(a, b, out=None):
 
 
 def __add__(a, b):
+    if a.data_type() == kFloat32 and (a.shape() != b.shape() or a.transpose() or b.transpose()):
+        a, b = _dense_pair(a, b)     # broadcast / transposed operands
     _same(a, b)
     out = _like(a)
     fn, name = _fn("add", a)

@@ -18,6 +18,7 @@ description (conv5x5-32 p2, ReLU, maxpool2, conv5x5-64 p2, ReLU, maxpool2, Linea
 import numpy as np
 
 from . import opt as hip_opt
+from . import rng
 from . import singa_wrap as singa
 
 
@@ -708,25 +709,28 @@ CONFIGS = {
 }
 
 SEED_BASE = 0x5167A000
-# per-configuration seed offsets (fixed numbers, so that adding a configuration leaves the inputs of
-# the others unchanged)
-_SEED_INDEX = {"cnn": 0, "mlp": 1, "resnet18": 2, "resnet18_small": 3, "smoke_cnn": 4, "resnet50": 5,
-               "resnet50_small": 6}
+# Seeds: SEED_BASE + 256 * configuration + tensor index; tensor 0 is the input batch, 1 the labels, 2.. the
+# weight tensors in the order the builder creates them.  The generator is counter-based (singa_amd/rng.py:
+# splitmix64 -> Box-Muller), so the bytes do not depend on a library's random stream and a smaller batch is
+# a prefix of a larger one.  (Fixed numbers: adding a configuration leaves the inputs of the others unchanged.)
+_CONFIG_INDEX = {"mlp": 1, "conv": 2, "cnn": 3, "resnet18": 4, "resnet50": 5, "resnet18_small": 6, "smoke_cnn": 7,
+                 "resnet50_small": 8}
 
 
 def make_inputs(name, batch=None):
     builder, kw, xshape, classes, default_batch = CONFIGS[name]
     batch = batch or default_batch
-    r = np.random.default_rng(SEED_BASE + 17 * (_SEED_INDEX[name] + 1) + batch)
-    x = r.standard_normal((batch,) + xshape).astype(np.float32)
-    labels = r.integers(0, classes, size=batch).astype(np.int32)
+    base = SEED_BASE + 256 * _CONFIG_INDEX[name]
+    x = rng.normal(base + 0, (batch,) + xshape)
+    labels = rng.integers(base + 1, (batch,), classes)
     return x, labels
 
 
 def build(name, ops, lr=0.05, momentum=0.9):
     builder, kw, _, _, _ = CONFIGS[name]
-    wr = np.random.default_rng(SEED_BASE + 1000 + _SEED_INDEX[name])
-    return builder(ops, wr, lr=lr, momentum=momentum, **kw)
+    stream = rng.Stream(SEED_BASE + 256 * _CONFIG_INDEX[name])
+    stream.index = 2
+    return builder(ops, stream, lr=lr, momentum=momentum, **kw)
 
 
 def resnet18_flops(batch=64):

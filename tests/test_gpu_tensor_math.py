@@ -288,3 +288,77 @@ def test_elementwise_functions_around_the_path(singa, dev, n):
     assert_bit_equal(singa.AddFloat(ad, 1.25).to_numpy(), a + np.float32(1.25), "Add scalar")
     assert_bit_equal(singa.MultFloat(ad, -0.3).to_numpy(), a * np.float32(-0.3), "Mult scalar")
     assert_bit_equal(singa.DivFloat(ad, 64).to_numpy(), a * (np.float32(1.0) / np.float32(64)), "Div scalar")
+
+
+# ---- the remaining Tensor functions: Transform / Broadcast, RowMax, Dot, SumAll, Uniform, Gaussian
+
+def test_transform_and_broadcast(singa, dev):
+    r = rng(31)
+    m = randn(r, 37, 53)
+    t = singa.from_numpy(m, dev)
+    assert_bit_equal(singa.Transform(t.T()).to_numpy(), m.T.copy(), "transposed view made dense")
+    assert singa.Transform(t) is t
+    for src, shape in [((53,), (37, 53)), ((37, 1), (37, 53)), ((1,), (5, 4, 3)), ((4, 1, 3), (2, 4, 6, 3)),
+                       ((2, 1, 1, 1, 3, 1, 1, 2), (2, 3, 2, 2, 3, 2, 2, 2))]:
+        a = randn(r, *src)
+        want = np.broadcast_to(a, shape)
+        assert_bit_equal(singa.Broadcast(singa.from_numpy(a, dev), shape).to_numpy(), want, "broadcast %r -> %r" % (src, shape))
+        assert_bit_equal(O.transform(a.ravel(), shape, [0 if s == 0 else s // 4 for s in want.strides]), want)
+    with pytest.raises(singa.SingaHipError):
+        singa.Broadcast(t, (37, 54))
+
+
+def test_eltwise_ops_on_broadcast_and_transposed_operands(singa, dev):
+    """Tensor *= / + with operands that are not dense: NumPy's result, as in the reference
+    (src/core/tensor/tensor.cc:481-503 Broadcast, then the dense op)."""
+    r = rng(32)
+    a, row, col = randn(r, 12, 33), randn(r, 33), randn(r, 12, 1)
+    ad, rowd, cold = (singa.from_numpy(v, dev) for v in (a, row, col))
+    assert_bit_equal(singa.EltwiseMult(ad, rowd).to_numpy(), a * row, "matrix * row")
+    assert_bit_equal(singa.__add__(cold, ad).to_numpy(), col + a, "column + matrix")
+    b = randn(r, 33, 12)
+    assert_bit_equal(singa.EltwiseMult(ad, singa.from_numpy(b, dev).T()).to_numpy(), a * b.T, "matrix * transposed view")
+    assert_bit_equal(singa.__add__(rowd, cold).to_numpy(), row + col, "outer sum of a row and a column")
+    with pytest.raises(singa.SingaHipError):
+        singa.__add__(ad, singa.from_numpy(randn(r, 12, 32), dev))
+
+
+def test_row_max_dot_and_sum(singa, dev):
+    r = rng(33)
+    for rows, cols in [(1, 1), (3, 7), (128, 1000), (17, 4097)]:
+        m = randn(r, rows, cols)
+        m[0] = -np.abs(m[0]) - 1          # an all-negative row: the maximum starts at 0
+        assert_bit_equal(singa.RowMax(singa.from_numpy(m, dev)).to_numpy(), O.row_max(m), "row max")
+    for n in (1, 100, 4096, 4097, 1 << 20, 5 * (1 << 20) + 3):
+        a, b = randn(r, n), randn(r, n)
+        ad, bd = singa.from_numpy(a, dev), singa.from_numpy(b, dev)
+        scale = float(np.abs(a.astype(np.float64) * b).sum())
+        got = float(singa.Dot(ad, bd).to_numpy()[0])
+        assert abs(got - float(a.astype(np.float64) @ b.astype(np.float64))) <= 1e-6 * scale + 1e-12
+        assert abs(got - O.dot(a, b)) <= 1e-5 * scale + 1e-12          # the CPU function sums in another order
+        assert got == float(singa.Dot(ad, bd).to_numpy()[0])           # run-to-run identical
+        s = singa.SumAll(ad)
+        assert abs(s - float(a.astype(np.float64).sum())) <= 1e-6 * float(np.abs(a).sum()) + 1e-12
+        assert abs(s - O.sum_all(a)) <= 1e-5 * float(np.abs(a).sum()) + 1e-12
+
+
+def test_uniform_and_gaussian_fills(singa, dev):
+    """The device fills against the CPU twin of the same counter-based generator: uniform numbers
+    bit for bit, Gaussian ones to the last place of the device's double-precision log / cos."""
+    from singa_amd import rng as host
+    dev.SetRandSeed(0x5167A123)
+    n = 100003
+    t = singa.Tensor((n,), dev)
+    singa.Uniform(-2.0, 3.0, t)
+    assert_bit_equal(t.to_numpy(), O.rng_uniform(0x5167A123, n, -2.0, 3.0), "uniform")
+    singa.Uniform(0.0, 1.0, t)                                  # the stream continues where the last fill ended
+    assert_bit_equal(t.to_numpy(), host.uniform(0x5167A123, (n,), offset=n), "uniform, continued")
+    singa.Gaussian(0.5, 2.0, t)
+    want = O.rng_normal(0x5167A123, n, 0.5, 2.0, offset=2 * n)
+    got = t.to_numpy()
+    assert int((got.view(np.uint32) != want.view(np.uint32)).sum()) <= n // 1000
+    assert float(np.abs(got - want).max()) <= 1e-6 * 8
+    dev.SetRandSeed(0x5167A123)                                 # the same seed replays the stream
+    u = singa.Tensor((10,), dev)
+    singa.Uniform(-2.0, 3.0, u)
+    assert_bit_equal(u.to_numpy(), O.rng_uniform(0x5167A123, 10, -2.0, 3.0))

@@ -233,3 +233,57 @@ def test_elementwise_definitions():
     assert np.array_equal(y, b + np.float32(0.3) * a)
     assert np.array_equal(O.sum_rows(a[:1000].reshape(10, 100)),
                           np.add.reduce(a[:1000].reshape(10, 100), axis=0, dtype=np.float32))
+
+
+# ---- the remaining tensor functions and the seeded generator
+
+def test_transform_walks_a_view_like_numpy():
+    r = np.random.default_rng(3)
+    a = r.standard_normal(4 * 5 * 6).astype(np.float32)
+    cube = a.reshape(4, 5, 6)
+    # transposed, sliced with a step, broadcast (stride 0), and all at once
+    for view in (cube.transpose(2, 0, 1), cube[:, ::2, 1:5], np.broadcast_to(cube[:, :1, :], (4, 7, 6)),
+                 np.broadcast_to(cube.transpose(1, 2, 0)[None, :, ::3, :], (3, 5, 2, 4)), cube[1:2, 2, 3:4]):
+        strides = [s // 4 for s in view.strides]
+        base = (view.__array_interface__["data"][0] - a.__array_interface__["data"][0]) // 4
+        got = O.transform(a[base:], view.shape, strides)
+        assert np.array_equal(got, np.ascontiguousarray(view))
+
+
+def test_row_max_starts_from_zero():
+    m = np.array([[-3.0, -1.0, -2.0], [0.5, 4.0, -7.0], [0.0, 0.0, 0.0]], np.float32)
+    assert np.array_equal(O.row_max(m), np.array([0.0, 4.0, 0.0], np.float32))   # not -1: the maximum starts at 0
+    r = np.random.default_rng(5).standard_normal((37, 101)).astype(np.float32)
+    assert np.array_equal(O.row_max(r), np.maximum(0, r.max(axis=1)))
+
+
+def test_dot_and_sum_against_float64():
+    r = np.random.default_rng(6)
+    for n in (1, 17, 4096, 100003):
+        a, b = r.standard_normal(n).astype(np.float32), r.standard_normal(n).astype(np.float32)
+        assert abs(O.dot(a, b) - float(a.astype(np.float64) @ b.astype(np.float64))) <= 1e-6 * float(np.abs(a * b).sum()) + 1e-12
+        assert abs(O.sum_all(a) - float(a.astype(np.float64).sum())) <= 1e-6 * float(np.abs(a).sum()) + 1e-12
+    assert O.dot(np.zeros(0, np.float32), np.zeros(0, np.float32)) == 0.0
+
+
+def test_seeded_generator_twins_and_known_answers():
+    """splitmix64's published first outputs for seed 0 and for seed 1234567 (the reference C
+    program by its author prints them), the C and NumPy twins agreeing bit for bit, and the
+    moments of the derived distributions."""
+    from singa_amd import rng
+    assert [O.rng_raw(0, k) for k in range(3)] == [0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4, 0x06C45D188009454F]
+    assert [O.rng_raw(1234567, k) for k in range(3)] == [6457827717110365317, 3203168211198807973, 9817491932198370423]
+    ks = np.arange(1000, dtype=np.uint64)
+    assert [int(v) for v in rng.raw(99, ks)] == [O.rng_raw(99, int(k)) for k in ks]
+    assert int(rng.raw(0xFFFFFFFFFFFFFFFF, 5)) == O.rng_raw(0xFFFFFFFFFFFFFFFF, 5)      # wrap-around of the state
+    n = 200000
+    z_c, z_py = O.rng_normal(0x5167A400, n), rng.normal(0x5167A400, (n,))
+    assert (z_c.view(np.uint32) != z_py.view(np.uint32)).sum() <= 2      # libm vs NumPy: a last-place flip at most, rarely
+    assert abs(z_py.mean()) < 0.01 and abs(z_py.std() - 1) < 0.01 and abs((z_py ** 4).mean() - 3) < 0.1
+    assert np.array_equal(z_py[:1000], rng.normal(0x5167A400, (1000,)))  # a smaller tensor is a prefix
+    assert np.array_equal(rng.normal(7, (10,), offset=2 * 5)[:5], rng.normal(7, (15,))[5:10])   # offsets continue a stream
+    u = rng.uniform(5, (n,), -1.0, 3.0)
+    assert np.array_equal(u, O.rng_uniform(5, n, -1.0, 3.0)) and u.min() >= -1 and u.max() < 3 and abs(u.mean() - 1) < 0.02
+    k = rng.integers(11, (n,), 1000)
+    assert np.array_equal(k, O.rng_integers(11, n, 1000)) and k.min() == 0 and k.max() == 999
+    assert abs(np.bincount(k, minlength=1000).std() - np.sqrt(n / 1000)) < 3
