@@ -207,6 +207,11 @@ SGH_API int sgh_uniform_f32(float low, float high, float *out, size_t n, uint64_
 SGH_API int sgh_gaussian_f32(float mean, float std, float *out, size_t n, uint64_t seed,
                              uint64_t offset, void *stream);
 
+/* Clamp<float, Lang> (src/core/tensor/tensor_math_cpp.h:398-410; autograd.clip): out = min(max(x, low), high).
+ * With the two casts above it is the single-GPU part of DistOpt.backward_and_update_half
+ * (python/singa/opt.py:867-920): gradients optionally clipped, then sent through half precision. */
+SGH_API int sgh_clamp_f32(float low, float high, const float *x, float *out, size_t n, void *stream);
+
 /* Axpy<float, Lang>, scalar and Tensor-alpha overloads: tensor_math.h:393-402;
  * CPU tensor_math_cpp.h:788-823; CUDA tensor_math_cuda.h:1031-1072 (device pointer mode).
  * y += alpha * x. */

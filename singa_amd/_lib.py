@@ -92,6 +92,7 @@ SIGNATURES = {
     "sgh_sum_all_f32": (C.c_int, [vp, sz, vp, vp, sz, vp]),
     "sgh_uniform_f32": (C.c_int, [C.c_float, C.c_float, vp, sz, C.c_uint64, C.c_uint64, vp]),
     "sgh_gaussian_f32": (C.c_int, [C.c_float, C.c_float, vp, sz, C.c_uint64, C.c_uint64, vp]),
+    "sgh_clamp_f32": (C.c_int, [C.c_float, C.c_float, vp, vp, sz, vp]),
     "sgh_axpy_f32": (C.c_int, [C.c_float, vp, vp, sz, vp]),
     "sgh_axpy_devalpha_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_eltwise_mult_f32": (C.c_int, [vp, vp, C.c_int, vp, sz, vp]),

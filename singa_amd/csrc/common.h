@@ -32,8 +32,8 @@ static inline bool sgh_aligned16(const void *p) { return (reinterpret_cast<uintp
 // when the first entry point asks: changing the environment later has no effect, so a geometry's
 // workspace size and kernel choice cannot change between two calls.
 struct sgh_env_switches {
-  bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off, bn_onchip_off;
-  int dgrad_tile, wgrad_tile;   // -1: chosen from the geometry
+  bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off, bn_onchip_off, pw_dgrad_off;
+  int dgrad_tile, wgrad_tile, pw_tile;   // -1: chosen from the geometry
   int dgrad3x3_bm;              // 0: chosen from the geometry, else 64 or 128
 };
 const sgh_env_switches &sgh_env();
@@ -107,6 +107,11 @@ int sgh_dgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *W, 
 // the same kernel reading a 16-bit dy and writing a 16-bit dx (fp32 weights, slab and arithmetic)
 int sgh_dgrad_fewc_run16(const sgh_conv_geom *g, const uint16_t *dy, const float *W, uint16_t *dx, void *workspace,
                          size_t ws_bytes, bool bf16, hipStream_t s);
+
+// Data gradient of 1x1 convolutions without padding, fed from global memory without LDS (pointwise.hip):
+// K a multiple of 32, at least 32 input channels, equal strides.
+bool sgh_pw_dgrad_supported(const sgh_conv_geom *g);
+int sgh_pw_dgrad_run(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, hipStream_t s);
 
 // Convolution gradients on 16-bit tensors with the 16-bit matrix instructions (conv16.hip).
 // *_workspace_bytes is 0 and the run functions return SGH_EUNSUPPORTED for geometries they do not

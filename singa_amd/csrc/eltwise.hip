@@ -114,6 +114,10 @@ struct ReluFwd {  // second operand unused
 struct AddOp {
   __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
 };
+struct ClampOp {  // second operand unused; NaN passes through, as in the CPU function's two comparisons
+  float lo, hi;
+  __device__ __forceinline__ float operator()(float x, float) const { return x < lo ? lo : (x > hi ? hi : x); }
+};
 struct MulOp {
   __device__ __forceinline__ float operator()(float a, float b) const { return a * b; }
 };
@@ -480,6 +484,10 @@ int sgh_relu_bwd_f32(const float *dy, const float *x, float *dx, size_t n, void 
 
 int sgh_relu_fwd_f32(const float *x, float *y, size_t n, void *stream) {
   return launch_map1(x, y, n, ReluFwd{}, stream);
+}
+
+int sgh_clamp_f32(float low, float high, const float *x, float *out, size_t n, void *stream) {
+  return launch_map1(x, out, n, ClampOp{low, high}, stream);
 }
 
 int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream) {

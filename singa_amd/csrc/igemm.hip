@@ -427,7 +427,7 @@ struct SplitStore {  // partial[split][m * N + n]; column N, if wanted, goes to 
 // and whether this tile lies outside the class).
 // ------------------------------------------------------------------------------------------
 template <int BM, int BN, class LA, class LB, class ST, bool A_KCONTIG, bool B_KCONTIG, bool ZCLASS = false,
-          int WGM = 2>
+          int WGM = 2, int PF = 1>
 __global__ __launch_bounds__(NT) void k_igemm(LA la, LB lb, ST st, int Ktotal, int chunks_per_split) {
   // the four wavefronts form a WGM x WGN grid over the tile
   constexpr int WGN = 4 / WGM;
@@ -461,63 +461,84 @@ __global__ __launch_bounds__(NT) void k_igemm(LA la, LB lb, ST st, int Ktotal, i
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  float ra[EA], rb[EB];
+  // PF chunks of loads are in flight in registers (set c % PF holds chunk c until it is written to LDS): a
+  // chunk of a small tile holds far fewer MFMA cycles than a load takes to return, so one chunk ahead leaves
+  // the loop waiting for memory; the loop is unrolled PF times so that the sets are addressed statically.
+  float ra[PF][EA], rb[PF][EB];
   if (k_begin < k_end) {
-    la.prepare(m0, k_begin, k_end, t);
-    lb.prepare(n0, k_begin, k_end, t);
 #pragma unroll
-    for (int e = 0; e < EA; ++e) ra[e] = la.get(e);
+    for (int d = 0; d < PF; ++d) {
+      la.prepare(m0, k_begin + d * BK, k_end, t);
+      lb.prepare(n0, k_begin + d * BK, k_end, t);
 #pragma unroll
-    for (int e = 0; e < EB; ++e) rb[e] = lb.get(e);
-    stage_store<BM, A_KCONTIG>(As[0], ra, t);
-    stage_store<BN, B_KCONTIG>(Bs[0], rb, t);
+      for (int e = 0; e < EA; ++e) ra[d][e] = la.get(e);
+#pragma unroll
+      for (int e = 0; e < EB; ++e) rb[d][e] = lb.get(e);
+    }
+    stage_store<BM, A_KCONTIG>(As[0], ra[0], t);
+    stage_store<BN, B_KCONTIG>(Bs[0], rb[0], t);
   }
   __syncthreads();
 
   int cur = 0;
-  for (int k0 = k_begin; k0 < k_end; k0 += BK) {
-    // the next chunk is always fetched: past the end every loader yields zeros (or, for the
-    // gather loaders, values that are never stored), which keeps this loop free of branches
-    la.prepare(m0, k0 + BK, k_end, t);
-    lb.prepare(n0, k0 + BK, k_end, t);
+  for (int kb = k_begin; kb < k_end; kb += PF * BK) {
+#pragma unroll
+    for (int d = 0; d < PF; ++d) {
+      const int k0 = kb + d * BK;
+      if (k0 >= k_end) break;
+      // chunk k0 / BK + PF is always fetched into the set this chunk has just left: past the end every loader
+      // yields zeros (or, for the gather loaders, values that are never stored), which keeps this loop free
+      // of branches
+      la.prepare(m0, k0 + PF * BK, k_end, t);
+      lb.prepare(n0, k0 + PF * BK, k_end, t);
 
-    const float *as = As[cur] + (lane >> 5) * PA + wm * WM + (lane & 31);
-    const float *bs = Bs[cur] + (lane >> 5) * PB + wn * WN + (lane & 31);
-    float a[2][TM], b[2][TN];
+      const float *as = As[cur] + (lane >> 5) * PA + wm * WM + (lane & 31);
+      const float *bs = Bs[cur] + (lane >> 5) * PB + wn * WN + (lane & 31);
+      float a[2][TM], b[2][TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) a[0][i] = as[i * 32];
+      for (int i = 0; i < TM; ++i) a[0][i] = as[i * 32];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) b[0][j] = bs[j * 32];
+      for (int j = 0; j < TN; ++j) b[0][j] = bs[j * 32];
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      const int cb = s & 1, nb = cb ^ 1;
-      if (s + 1 < KSTEPS) {
+      for (int s = 0; s < KSTEPS; ++s) {
+        const int cb = s & 1, nb = cb ^ 1;
+        if (s + 1 < KSTEPS) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) a[nb][i] = as[(2 * s + 2) * PA + i * 32];
+          for (int i = 0; i < TM; ++i) a[nb][i] = as[(2 * s + 2) * PA + i * 32];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) b[nb][j] = bs[(2 * s + 2) * PB + j * 32];
-      }
-      __builtin_amdgcn_sched_barrier(0);  // operand prefetch stays ahead of this k-step's MFMAs
+          for (int j = 0; j < TN; ++j) b[nb][j] = bs[(2 * s + 2) * PB + j * 32];
+        }
+        __builtin_amdgcn_sched_barrier(0);  // operand prefetch stays ahead of this k-step's MFMAs
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cb][i], b[cb][j], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);  // this k-step's share of the next chunk's global loads
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cb][i], b[cb][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);  // this k-step's share of the global loads
+        if (PF == 1) {
 #pragma unroll
-      for (int q = 0; q < ET; ++q) {
-        if (q * KSTEPS / ET == s) {
-          if (q < EA) ra[q] = la.get(q);
-          else rb[q - EA] = lb.get(q - EA);
+          for (int q = 0; q < ET; ++q) {
+            if (q * KSTEPS / ET == s) {
+              if (q < EA) ra[d][q] = la.get(q);
+              else rb[d][q - EA] = lb.get(q - EA);
+            }
+          }
         }
       }
+      if (k0 + BK < k_end) {
+        // the next chunk's registers go to LDS before its set is reloaded (with one set, it was reloaded above)
+        stage_store<BM, A_KCONTIG>(As[cur ^ 1], ra[(d + 1) % PF], t);
+        stage_store<BN, B_KCONTIG>(Bs[cur ^ 1], rb[(d + 1) % PF], t);
+      }
+      if (PF > 1) {
+#pragma unroll
+        for (int e = 0; e < EA; ++e) ra[d][e] = la.get(e);
+#pragma unroll
+        for (int e = 0; e < EB; ++e) rb[d][e] = lb.get(e);
+      }
+      __syncthreads();
+      cur ^= 1;
     }
-    if (k0 + BK < k_end) {
-      stage_store<BM, A_KCONTIG>(As[cur ^ 1], ra, t);
-      stage_store<BN, B_KCONTIG>(Bs[cur ^ 1], rb, t);
-    }
-    __syncthreads();
-    cur ^= 1;
   }
 
 #pragma unroll
@@ -765,13 +786,13 @@ inline WgradPlan plan_wgrad(const sgh_conv_geom *g) {
   return p;
 }
 
-template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc, bool ZCLASS = false, int WGM = 2>
+template <int BM, int BN, class LA, class LB, class ST, bool AK, bool BKc, bool ZCLASS = false, int WGM = 2, int PF = 1>
 inline int launch_igemm(const LA &la, const LB &lb, const ST &st, int M, int N, int Ktotal, int splits,
                         int chunks_per_split, hipStream_t stream, const char *tag = nullptr, double flops = 0) {
   dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
   if (grid.y > 65535u || grid.z > 65535u) return SGH_EUNSUPPORTED;
   if (tag) sgh_prof_start(tag, flops, stream);  // kernel-level record: this launch only
-  hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc, ZCLASS, WGM>), grid, dim3(NT), 0, stream, la, lb, st,
+  hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc, ZCLASS, WGM, PF>), grid, dim3(NT), 0, stream, la, lb, st,
                      Ktotal, chunks_per_split);
   if (tag) sgh_prof_stop(stream);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
@@ -790,8 +811,8 @@ inline int gemm_tile(int M, int N, int K, float alpha, const float *A, long a_rs
   auto lb = dense_loader<BN, BKc>(B, b_rs, b_ks, N, K);
   DenseStore st{C, ldc, M, N, alpha, beta};
   const int chunks = (K + BK - 1) / BK;
-  return launch_igemm<BM, BN, DenseLoader<BM, AK>, DenseLoader<BN, BKc>, DenseStore, AK, BKc>(la, lb, st, M, N, K, 1,
-                                                                                               chunks, stream);
+  return launch_igemm<BM, BN, DenseLoader<BM, AK>, DenseLoader<BN, BKc>, DenseStore, AK, BKc, false, 2, (BM * BN <= 64 * 64 ? 4 : 2)>(
+      la, lb, st, M, N, K, 1, chunks, stream);
 }
 
 template <bool AK, bool BKc>
@@ -924,6 +945,8 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
 
   if (path == kDgradFewC) {
     rc = sgh_dgrad_fewc_run(g, dy, W, dx, workspace, ws_bytes, s);
+  } else if (path == kDgradPointwise && sgh_pw_dgrad_supported(g) && !sgh_env().pw_dgrad_off) {
+    rc = sgh_pw_dgrad_run(g, dy, W, dx, s);
   } else if (path == kDgradPointwise) {
     // dx block (img, m, p, q) = sum_k W[k][m] * dy[img][k][p][q]: A(m, k) = W[k * C + m] in its native layout
     const int Ncols = g->N * g->P * g->Q;
@@ -937,17 +960,17 @@ static int conv_dgrad(const sgh_conv_geom *g, const float *dy, const float *W, f
     if (g->C > 64 && tiles128 >= need) {
       auto la = dense_loader<128, false>(W, 1, g->C, g->C, g->K);
       auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
-      rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, DilateStore, false, false>(
+      rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, DilateStore, false, false, false, 2, 2>(
           la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad/k_igemm", conv_flops(g));
     } else if (long((g->C + 63) / 64) * ((Ncols + 127) / 128) >= need) {
       auto la = dense_loader<64, false>(W, 1, g->C, g->C, g->K);
       auto lb = gather_loader<128, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
-      rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DilateStore, false, false>(
+      rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, DilateStore, false, false, false, 2, 4>(
           la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad/k_igemm", conv_flops(g));
     } else {
       auto la = dense_loader<64, false>(W, 1, g->C, g->C, g->K);
       auto lb = gather_loader<64, false>(dy, fake, KP, g->K, g->P, g->Q, Ncols);
-      rc = launch_igemm<64, 64, DenseLoader<64, false>, PixelGatherLoader<64, false>, DilateStore, false, false>(
+      rc = launch_igemm<64, 64, DenseLoader<64, false>, PixelGatherLoader<64, false>, DilateStore, false, false, false, 2, 4>(
           la, lb, st, g->C, Ncols, g->K, 1, chunks, s, "conv_dgrad/k_igemm", conv_flops(g));
     }
   } else if (path == kDgradColumns) {
@@ -1308,7 +1331,7 @@ static int conv_wgrad(sgh_conv_geom *g, const float *dy, const float *x, float *
   SplitStore st{part, g->K, CRS, bpart};
   int rc;
   sgh_prof_start("conv_wgrad_op", conv_flops(g), s);
-#define SGH_WGRAD_CASE(BM_, BN_, WGM_)                                                                             \
+#define SGH_WGRAD_CASE(BM_, BN_, WGM_, PF_)                                                                          \
   {                                                                                                                \
     WgradDyLoader<BM_> la{dy, g->K, PQ, int(G), bytes_of(size_t(G) * g->K), 0, 0, 0};                              \
     WgradXLoader<BN_> lb;                                                                                          \
@@ -1317,15 +1340,16 @@ static int conv_wgrad(sgh_conv_geom *g, const float *dy, const float *x, float *
     lb.CRS = CRS;                                                                                                  \
     lb.ones_col = ride ? CRS : -1;                                                                                 \
     lb.bytes = bytes_of(size_t(g->N) * g->C * g->H * g->W);                                                        \
-    rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true, false, WGM_>(       \
+    rc = launch_igemm<BM_, BN_, WgradDyLoader<BM_>, WgradXLoader<BN_>, SplitStore, true, true, false, WGM_, PF_>(  \
         la, lb, st, g->K, CRS, int(G), p.splits, p.chunks_per_split, s, "conv_wgrad/k_igemm", conv_flops(g));              \
   }
-  if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128, 2)
-  else if (p.bm == 64 && p.bn == 256) SGH_WGRAD_CASE(64, 256, 1)
-  else if (p.bm == 64 && p.bn == 192) SGH_WGRAD_CASE(64, 192, 2)
-  else if (p.bm == 64 && p.bn == 128) SGH_WGRAD_CASE(64, 128, 2)
-  else if (p.bm == 128 && p.bn == 64) SGH_WGRAD_CASE(128, 64, 2)
-  else SGH_WGRAD_CASE(64, 64, 2)
+  // (chunks in flight: see k_igemm; the smaller the tile, the fewer MFMA cycles a chunk holds)
+  if (p.bm == 128 && p.bn == 128) SGH_WGRAD_CASE(128, 128, 2, 2)
+  else if (p.bm == 64 && p.bn == 256) SGH_WGRAD_CASE(64, 256, 1, 2)
+  else if (p.bm == 64 && p.bn == 192) SGH_WGRAD_CASE(64, 192, 2, 2)
+  else if (p.bm == 64 && p.bn == 128) SGH_WGRAD_CASE(64, 128, 2, 3)
+  else if (p.bm == 128 && p.bn == 64) SGH_WGRAD_CASE(128, 64, 2, 3)
+  else SGH_WGRAD_CASE(64, 64, 2, 4)
 #undef SGH_WGRAD_CASE
   if (rc == SGH_OK && p.splits > 1) {
     const long n = long(g->K) * CRS;

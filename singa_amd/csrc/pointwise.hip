@@ -1,0 +1,169 @@
+// Data gradient of 1x1 convolutions without padding (fp32): dx[n][c][s*p][s*q] = sum_k W[k][c] * dy[n][k][p][q],
+// the other positions of each s x s block zero -- the downsample convolutions of a residual network
+// (reference call: GpuConvBackwardx, src/model/operation/convolution.cc:634-656).
+//
+// The reduction index k is the strided one in both operands while channels (W rows) and pixels (dy rows)
+// are contiguous, which is exactly the operand shape of v_mfma_f32_32x32x2_f32: lane (i = lane % 32,
+// h = lane / 32) supplies A[i][h] and B[h][i].  So a wavefront feeds its matrix instructions straight from
+// global memory -- lane (i, h) loads W[2 j + h][c0 + i] and dy[..][2 j + h][col0 + i], 128 contiguous bytes per
+// half wavefront -- with no LDS, no barrier and two adds of address arithmetic per step.  The generic
+// implicit-GEMM kernel spent 23 vector and 13 scalar instructions per matrix instruction on these layers
+// (staging arithmetic of its general loaders) and ran them at 27 TFLOP/s whatever their size; they are
+// bandwidth kernels: 0.8 GFLOP against 13 - 77 MB of tensors.
+//
+// One wavefront owns (32 * TM) channels x 32 consecutive pixels of the flattened (n, p, q) index; the four
+// wavefronts of a workgroup take the channel tiles of one pixel tile first (they read the same gradient
+// pixels).  Every lane owns one pixel column for the whole kernel, so (n, p, q) is computed once.
+#include "common.h"
+
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int kOOB = int(0x80000000u);
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, int(bytes), 0x00020000);
+}
+
+struct PwArgs {
+  const float *W, *dy;
+  float *dx;
+  int N, C, K, H, Wd, P, Q, s;   // stride s in both directions
+  int ncols, mtiles, ctiles;     // N * P * Q; channel tiles of 32 * TM; pixel tiles of 32 * TN
+  unsigned w_bytes, dy_bytes;
+};
+
+template <int TM, int TN>
+__global__ __launch_bounds__(256) void k_pw_dgrad(PwArgs a) {
+  const int lane = threadIdx.x & 63, i32 = lane & 31, h = lane >> 5;
+  const int wave = int(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int ct = wave / a.mtiles, mt = wave - ct * a.mtiles;
+  if (ct >= a.ctiles) return;
+  const int PQ = a.P * a.Q;
+  const int m0 = mt * (32 * TM);
+  const rsrc_t rw = make_rsrc(a.W, a.w_bytes), rdy = make_rsrc(a.dy, a.dy_bytes);
+  // byte offsets of this lane's first elements (k = h); a k step of 2 adds 2 * C / 2 * PQ elements
+  int woff[TM], doff[TN], img[TN], rem[TN];
+  bool col_ok[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) woff[i] = m0 + 32 * i + i32 < a.C ? (h * a.C + m0 + 32 * i + i32) * 4 : kOOB;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = (ct * TN + j) * 32 + i32;
+    col_ok[j] = col < a.ncols;
+    img[j] = col_ok[j] ? col / PQ : 0, rem[j] = col_ok[j] ? col - img[j] * PQ : 0;
+    doff[j] = col_ok[j] ? ((img[j] * a.K + h) * PQ + rem[j]) * 4 : kOOB;
+  }
+  const int wstep = 2 * a.C * 4, dstep = 2 * PQ * 4;
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // Batches of U matrix steps; the loads of batch j + 2 are issued before the matrix instructions of batch j
+  // (three register sets, the loop unrolled three times so that they are addressed statically): a batch holds
+  // U * 64 cycles of matrix work, a load takes longer than that to come back from HBM.
+  constexpr int U = 16 / (TM * TN > 2 ? 2 : 1), SETS = 3;   // (K is a multiple of 2 * U)
+  float av[SETS][TM][U], bv[SETS][TN][U];
+  auto load = [&](int set, int batch) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        av[set][i][u] =
+            __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rw, woff[i], (batch * U + u) * wstep, 0));
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bv[set][j][u] =
+            __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rdy, doff[j], (batch * U + u) * dstep, 0));
+    }
+  };
+  auto mma = [&](int set) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[set][i][u], bv[set][j][u], acc[i][j], 0, 0, 0);
+  };
+  const int nb = a.K / (2 * U);
+  load(0, 0);
+  if (nb > 1) load(1, 1);
+  for (int b = 0; b < nb; b += SETS) {
+#pragma unroll
+    for (int i = 0; i < SETS; ++i) {
+      if (b + i < nb) {
+        if (b + i + 2 < nb) load((i + 2) % SETS, b + i + 2);
+        mma(i);
+      }
+    }
+  }
+
+  const size_t plane = size_t(a.H) * a.Wd;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    if (!col_ok[j]) continue;
+    const int p = rem[j] / a.Q, q = rem[j] - p * a.Q;
+    float *base = a.dx + (size_t(img[j]) * a.C) * plane + size_t(a.s * p) * a.Wd + a.s * q;
+    // the s x s block of this pixel: the value at its origin, zeros elsewhere; the last block of a row / column
+    // also covers what lies beyond s * Q (s * P), and stops at the image border
+    const int he = p == a.P - 1 ? a.H - p * a.s : a.s, we = q == a.Q - 1 ? a.Wd - q * a.s : a.s;
+    const bool pair = a.s == 2 && he == 2 && we == 2 && (a.Wd & 1) == 0 && (reinterpret_cast<uintptr_t>(a.dx) & 7u) == 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
+        if (m >= a.C) continue;
+        float *o = base + size_t(m) * plane;
+        if (a.s == 1) {
+          *o = acc[i][j][v];
+        } else if (pair) {
+          *reinterpret_cast<v2f *>(o) = v2f{acc[i][j][v], 0.f};
+          *reinterpret_cast<v2f *>(o + a.Wd) = v2f{0.f, 0.f};
+        } else {
+          for (int r = 0; r < he; ++r)
+            for (int c = 0; c < we; ++c) o[r * a.Wd + c] = (r == 0 && c == 0) ? acc[i][j][v] : 0.f;
+        }
+      }
+  }
+}
+
+}  // namespace
+
+bool sgh_pw_dgrad_supported(const sgh_conv_geom *g) {
+  if (g->R != 1 || g->S != 1 || g->pad_h != 0 || g->pad_w != 0 || g->stride_h != g->stride_w) return false;
+  if (g->K % 32 != 0 || g->C < 32) return false;
+  const size_t lim = size_t(1) << 29;   // byte offsets stay below 2^31
+  return size_t(g->N) * g->K * g->P * g->Q < lim && size_t(g->K) * g->C < lim;
+}
+
+int sgh_pw_dgrad_run(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, hipStream_t s) {
+  if (!sgh_pw_dgrad_supported(g)) return SGH_EUNSUPPORTED;
+  PwArgs a{};
+  a.W = W, a.dy = dy, a.dx = dx;
+  a.N = g->N, a.C = g->C, a.K = g->K, a.H = g->H, a.Wd = g->W, a.P = g->P, a.Q = g->Q, a.s = g->stride_h;
+  a.ncols = g->N * g->P * g->Q;
+  a.w_bytes = unsigned(size_t(g->K) * g->C * 4), a.dy_bytes = unsigned(size_t(a.ncols) * g->K * 4);
+  // wavefront tiles of 64 x 64 (half the operand loads per matrix instruction) while that still gives every
+  // SIMD a wavefront, else 32 x 32
+  const int force = sgh_env().pw_tile;
+  const long waves64 = long((g->C + 63) / 64) * ((a.ncols + 63) / 64);
+  const bool big = force > 0 ? force == 2 : (g->C >= 64 && waves64 >= 3L * sgh_num_cus());
+  a.mtiles = big ? (g->C + 63) / 64 : (g->C + 31) / 32;
+  a.ctiles = big ? (a.ncols + 63) / 64 : (a.ncols + 31) / 32;
+  const long waves = long(a.mtiles) * a.ctiles;
+  const unsigned blocks = unsigned((waves + 3) / 4);
+  sgh_prof_start("conv_dgrad/k_pw_dgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C, s);
+  if (big) hipLaunchKernelGGL((k_pw_dgrad<2, 2>), dim3(blocks), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((k_pw_dgrad<1, 1>), dim3(blocks), dim3(256), 0, s, a);
+  sgh_prof_stop(s);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}

@@ -153,6 +153,18 @@ class SGD(object):
                                                       self.dampening, self.weight_decay, int(self.nesterov),
                                                       dev.stream), "sgh_sgd_momentum_multi_mixed")
 
+    def through_half(self, g, clipping=False, clip_value=100, dtype=None):
+        """What ``DistOpt.backward_and_update_half`` (python/singa/opt.py:867-920) does to a gradient on
+        one GPU: optional clipping to [-clip_value, clip_value] (``autograd.clip``), then the trip through
+        half precision that the gradient takes on its way through the communicator
+        (``cuda::float2half`` / ``half2float``, src/io/communicator.cc:369-466).  The exchange between
+        GPUs itself is not part of this library."""
+        if g.data_type() != singa.kFloat32:
+            raise singa.SingaHipError("backward_and_update_half is defined for float32 gradients")
+        if clipping:
+            g = singa.Clamp(-clip_value, clip_value, g)
+        return g.AsType(dtype if dtype is not None else singa.kFloat16).AsType(singa.kFloat32)
+
     def step(self):
         self.step_counter += 1
 

@@ -428,6 +428,14 @@ def _dense_pair(a, b):
     return (a if sa == shape else Broadcast(a, shape)), (b if sb == shape else Broadcast(b, shape))
 
 
+def Clamp(low, high, t):
+    """``singa.Clamp`` (autograd.clip): a new tensor with min(max(t, low), high)."""
+    _need_f32("Clamp", t)
+    out = _like(t)
+    check(_L().sgh_clamp_f32(float(low), float(high), t.ptr, out.ptr, t.Size(), t.device().stream), "sgh_clamp_f32")
+    return out
+
+
 def RowMax(t):
     """``singa.RowMax``: per row max(0, max over the row) (the CPU rule, tensor_math_cpp.h:1122-1140)."""
     _need_f32("RowMax", t)

@@ -90,6 +90,8 @@ CONV_CASES = [
     (2, 2, 24, 24, 40, 7, 7, (1, 1), (3, 3), False),      # few-channel large-filter path at stride 1
     (2, 4, 24, 24, 16, 5, 5, (2, 2), (2, 2), False),      # direct few-channel dgrad: 5x5 (three offsets per dimension), C = 4
     (2, 1, 16, 16, 8, 7, 7, (2, 2), (3, 3), True),        # direct few-channel dgrad: one channel
+    (32, 96, 57, 57, 32, 1, 1, (2, 2), (0, 0), False),    # 1x1 stride 2, 64 x 64 wavefront tiles: ragged channel tile, odd image
+    (2, 48, 11, 11, 64, 1, 1, (3, 3), (0, 0), False),     # 1x1 stride 3 on the matrix-instruction-from-global-memory kernel
 ]
 
 
@@ -275,6 +277,7 @@ def test_conv_dgrad_is_deterministic(singa, dev, n, c, hw, k, stride):
     (64, 3, 224, 64, 7, 2, 3),     # ResNet stem: few-channel wgrad / direct dgrad kernels
     (64, 64, 56, 128, 3, 2, 1),    # stage transition: residue-class shared-tile dgrad, stride-2 slab wgrad
     (64, 256, 14, 512, 1, 2, 0),   # downsample: pointwise dgrad with dilating store
+    (64, 64, 56, 128, 1, 2, 0),    # first downsample: 64 x 64 wavefront tiles
 ])
 def test_conv_full_size_properties(singa, dev, shape):
     """Convolutions at the benchmark's full batch are too large for the CPU oracle inside a test,

@@ -362,3 +362,20 @@ def test_uniform_and_gaussian_fills(singa, dev):
     u = singa.Tensor((10,), dev)
     singa.Uniform(-2.0, 3.0, u)
     assert_bit_equal(u.to_numpy(), O.rng_uniform(0x5167A123, 10, -2.0, 3.0))
+
+
+def test_clamp_and_the_half_precision_trip_of_a_gradient(singa, dev):
+    from singa_amd import opt
+    r = rng(34)
+    g = (randn(r, 100003) * 60).astype(np.float32)
+    g[:4] = [np.nan, np.inf, -np.inf, 100.0]
+    gd = singa.from_numpy(g, dev)
+    got = singa.Clamp(-100.0, 100.0, gd).to_numpy()
+    want = np.where(g < -100, -100, np.where(g > 100, 100, g)).astype(np.float32)
+    assert np.array_equal(got[1:], want[1:]) and np.isnan(got[0])
+    sgd = opt.SGD(lr=0.1)
+    out = sgd.through_half(gd, clipping=True, clip_value=100).to_numpy()
+    with np.errstate(invalid="ignore"):
+        assert np.array_equal(out[1:], want[1:].astype(np.float16).astype(np.float32))
+    big = singa.from_numpy(np.array([70000.0, -1e-9, 3.0], np.float32), dev)
+    assert np.array_equal(sgd.through_half(big).to_numpy(), np.array([np.inf, -0.0, 3.0], np.float32))   # no clipping: overflow
