@@ -207,6 +207,11 @@ def main():
         step_ms.append(ms.value)
     for e in evs:
         lib.sgh_event_destroy(e)
+    # one more step enqueued into empty queues: what the host needs when nothing makes it wait
+    t1 = time.perf_counter()
+    step()
+    t_idle_enqueue = time.perf_counter() - t1
+    sync()
     step_ms.sort()
     median_ms = step_ms[len(step_ms) // 2] if len(step_ms) % 2 else 0.5 * (step_ms[len(step_ms) // 2 - 1] + step_ms[len(step_ms) // 2])
 
@@ -279,6 +284,7 @@ def main():
         "hbm_kernels": {"peak_GB/s": PEAK_HBM_GBS, "bytes": "algorithmic (every tensor of the op once)",
                         "timing": "HIP event pair around each entry point, same extra steps as the roofline", **hbm},
         "host_enqueue_ms_per_step": round(t_enqueued / args.steps * 1e3, 4),
+        "host_enqueue_ms_idle_queue": round(t_idle_enqueue * 1e3, 4),
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.config, args.cpu_sample_batch or args.batch, args.cpu_budget_s,

@@ -113,6 +113,13 @@ SGH_API int sgh_pool_trim(sgh_device *dev);
  * (= core.proto CopyDirection, src/proto/core.proto:43-48).  D2H and H2D block until the
  * copy has completed so the host may touch the buffer when the call returns. */
 SGH_API int sgh_memcpy(sgh_device *dev, void *dst, const void *src, size_t bytes, int kind);
+/* Host-to-device copy that does not wait (no counterpart in the reference, whose CopyDataFromHostPtr
+ * blocks): `src` is copied to pinned staging memory before the call returns, so the caller may reuse
+ * it at once; the copy to `dst` is enqueued on the device's stream in order with the kernels there.
+ * For the small tables a step uploads (pointer tables of the multi-tensor update) -- a blocking copy
+ * would drain the stream once per step.  Up to 64 KiB; larger copies and copies while the stream is
+ * being recorded behave like sgh_memcpy(kind 1). */
+SGH_API int sgh_upload_async(sgh_device *dev, void *dst, const void *src, size_t bytes);
 /* Tensor::SetValue (src/core/tensor/tensor.cc:849-865, Set<DType, Lang>): every element = value.
  * The 16-bit variants round `value` once to the storage type (nearest, ties to even) and write
  * 2-byte elements; n counts elements. */

@@ -64,6 +64,7 @@ SIGNATURES = {
     "sgh_pool_stats": (C.c_int, [vp, C.POINTER(sz), C.POINTER(sz), C.POINTER(sz)]),
     "sgh_pool_trim": (C.c_int, [vp]),
     "sgh_memcpy": (C.c_int, [vp, vp, vp, sz, C.c_int]),
+    "sgh_upload_async": (C.c_int, [vp, vp, vp, sz]),
     "sgh_memset_f32": (C.c_int, [vp, C.c_float, sz, vp]),
     "sgh_memset_f16": (C.c_int, [vp, C.c_float, sz, vp]),
     "sgh_memset_bf16": (C.c_int, [vp, C.c_float, sz, vp]),

@@ -11,6 +11,8 @@
 #include <unordered_set>
 #include <vector>
 
+#include <string.h>
+
 #include "common.h"
 
 struct sgh_device {
@@ -34,6 +36,12 @@ struct sgh_device {
   std::vector<std::pair<void *, size_t>> held;
   std::unordered_set<void *> born;        // blocks handed out while recording
   std::vector<struct sgh_graph *> graphs;  // instantiated recordings of this device
+  // sgh_upload_async: ring of pinned staging slots; a slot is reused once its copy has run
+  static constexpr int kUploadSlots = 8;
+  static constexpr size_t kUploadSlotBytes = 64 * 1024;
+  char *upload_host = nullptr;   // kUploadSlots * kUploadSlotBytes of pinned memory, allocated on first use
+  hipEvent_t upload_done[kUploadSlots] = {};
+  int upload_next = 0;
 };
 
 struct sgh_graph {
@@ -251,6 +259,9 @@ int sgh_device_close(sgh_device *dev) {
   if (dev->aux) (void)hipStreamDestroy(dev->aux);
   if (dev->fork_ev) (void)hipEventDestroy(dev->fork_ev);
   if (dev->join_ev) (void)hipEventDestroy(dev->join_ev);
+  for (hipEvent_t e : dev->upload_done)
+    if (e) (void)hipEventDestroy(e);
+  if (dev->upload_host) (void)hipHostFree(dev->upload_host);
   delete dev;
   return SGH_OK;
 }
@@ -457,6 +468,29 @@ int sgh_pool_stats(sgh_device *dev, size_t *in_use, size_t *cached, size_t *driv
   if (in_use) *in_use = dev->in_use;
   if (cached) *cached = dev->cached;
   if (driver_allocs) *driver_allocs = dev->driver_allocs;
+  return SGH_OK;
+}
+
+int sgh_upload_async(sgh_device *dev, void *dst, const void *src, size_t bytes) {
+  if (!dev) return SGH_EINVAL;
+  if (bytes == 0) return SGH_OK;
+  if (!dst || !src) return SGH_EINVAL;
+  if (dev->capturing || bytes > sgh_device::kUploadSlotBytes) return sgh_memcpy(dev, dst, src, bytes, 1);
+  sgh_weights_epoch_bump();   // the destination may be a weight tensor
+  std::lock_guard<std::mutex> lk(dev->mu);
+  if (!dev->upload_host) {
+    void *h = nullptr;
+    SGH_HIP_TRY(hipHostMalloc(&h, sgh_device::kUploadSlots * sgh_device::kUploadSlotBytes, hipHostMallocDefault));
+    dev->upload_host = static_cast<char *>(h);
+  }
+  const int slot = dev->upload_next;
+  dev->upload_next = (slot + 1) % sgh_device::kUploadSlots;
+  if (!dev->upload_done[slot]) SGH_HIP_TRY(hipEventCreateWithFlags(&dev->upload_done[slot], hipEventDisableTiming));
+  else SGH_HIP_TRY(hipEventSynchronize(dev->upload_done[slot]));   // the copy issued kUploadSlots uploads ago
+  char *stage = dev->upload_host + size_t(slot) * sgh_device::kUploadSlotBytes;
+  memcpy(stage, src, bytes);
+  SGH_HIP_TRY(hipMemcpyAsync(dst, stage, bytes, hipMemcpyHostToDevice, dev->stream));
+  SGH_HIP_TRY(hipEventRecord(dev->upload_done[slot], dev->stream));
   return SGH_OK;
 }
 

@@ -83,8 +83,9 @@ class SGD(object):
         """Update every (name, p, g) triple with ONE kernel launch.  The pointer table is built
         once per distinct set of buffers and kept on the device; the memory pool hands the
         gradient buffers out in a short cycle of address sets, so a few tables are cached and a
-        steady-state step uploads nothing (an upload is a blocking copy that would drain the
-        stream at the end of every step)."""
+        steady-state step usually uploads nothing; when the set is new (with weight gradients on
+        the auxiliary stream the cycle of address sets is long) the table goes up through
+        ``sgh_upload_async``, which does not drain the stream."""
         items = list(named_params_grads)
         if not items:
             return
@@ -104,7 +105,7 @@ class SGD(object):
                 total += p.Size()
             nbytes = C.sizeof(arr)
             table = singa.Tensor(((nbytes + 3) // 4,), dev, singa.kInt)
-            check(_lib.lib().sgh_memcpy(dev._h, table.ptr, C.addressof(arr), nbytes, 1), "sgh_memcpy H2D")
+            check(_lib.lib().sgh_upload_async(dev._h, table.ptr, C.addressof(arr), nbytes), "sgh_upload_async")
             self._table, self._table_key, self._table_total = table, key, total
             if len(self._tables) >= 16:
                 self._tables.pop(next(iter(self._tables)))
@@ -144,7 +145,7 @@ class SGD(object):
                 total += p.Size()
             nbytes = C.sizeof(arr)
             table = singa.Tensor(((nbytes + 3) // 4,), dev, singa.kInt)
-            check(_lib.lib().sgh_memcpy(dev._h, table.ptr, C.addressof(arr), nbytes, 1), "sgh_memcpy H2D")
+            check(_lib.lib().sgh_upload_async(dev._h, table.ptr, C.addressof(arr), nbytes), "sgh_upload_async")
             if len(self._tables) >= 16:
                 self._tables.pop(next(iter(self._tables)))
             cached = self._tables[key] = (table, total, int(half_type == singa.kBFloat16))

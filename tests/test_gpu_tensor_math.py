@@ -231,6 +231,30 @@ def test_pool_reuses_freed_blocks(singa, dev):
     assert dev.PoolStats()["driver_allocs"] - before <= 1
 
 
+def test_upload_without_waiting(singa, dev):
+    """sgh_upload_async: the host buffer may be overwritten as soon as the call returns, copies land
+    in stream order (more uploads than staging slots in a row), oversize copies take the blocking path."""
+    import ctypes as C
+    from singa_amd import _lib
+    lib = _lib.lib()
+    host = np.zeros(3000, np.float32)
+    tensors = []
+    for i in range(20):
+        host[:] = np.arange(3000, dtype=np.float32) + 1000 * i
+        t = singa.Tensor((3000,), dev)
+        _lib.check(lib.sgh_upload_async(dev._h, t.ptr, host.ctypes.data, host.nbytes), "sgh_upload_async")
+        tensors.append(t)
+    host[:] = -1
+    for i, t in enumerate(tensors):
+        assert_bit_equal(t.to_numpy(), np.arange(3000, dtype=np.float32) + 1000 * i, "upload %d" % i)
+    big = np.arange(40000, dtype=np.float32)   # 160 KB: beyond a staging slot
+    t = singa.Tensor((40000,), dev)
+    _lib.check(lib.sgh_upload_async(dev._h, t.ptr, big.ctypes.data, big.nbytes), "sgh_upload_async")
+    assert_bit_equal(t.to_numpy(), big, "large upload")
+    assert lib.sgh_upload_async(dev._h, None, big.ctypes.data, 16) == -1
+    assert lib.sgh_upload_async(dev._h, t.ptr, big.ctypes.data, 0) == 0
+
+
 def test_pool_keeps_blocks_of_the_auxiliary_stream_until_the_join(singa, dev):
     """A block that work on the auxiliary stream uses may be freed right after that work was enqueued
     (SINGA's Graph does so): the pool hands it out again only once the main stream has been ordered
