@@ -318,7 +318,10 @@ __global__ __launch_bounds__(kResNT) void k_bn_bwd_resident(const typename S::el
   typedef typename RawVec<V * sizeof(elem)>::type raw;
   extern __shared__ __align__(16) unsigned char resident[];
   __shared__ float red[16];
-  const int c = blockIdx.x, M = s.N * s.HW, t = threadIdx.x;
+  // workgroup w runs on XCD w % 8: each XCD takes a run of consecutive channels, whose planes share cache
+  // lines when a plane is not a whole number of lines (49 or 196 elements), so a line is fetched into one L2
+  const int c = int(blockIdx.x & 7) * int(gridDim.x >> 3) + int(blockIdx.x >> 3), M = s.N * s.HW, t = threadIdx.x;
+  if (c >= s.C) return;
   elem *xs = reinterpret_cast<elem *>(resident);
   elem *ds = reinterpret_cast<elem *>(resident + ((size_t(M) * sizeof(elem) + 15) & ~size_t(15)));
   const float mean = save_mean[c], invstd = save_invstd[c];
@@ -491,7 +494,7 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
                                                           typename S::elem *__restrict__ dx, float *__restrict__ dgamma,
                                                           float *__restrict__ dbeta, unsigned long long *__restrict__ ws,
                                                           BnShape s, int G, int vpg, unsigned long long ticket1,
-                                                          unsigned long long ticket2, int spin_limit) {
+                                                          unsigned long long ticket2, int spin_limit, int xcd_runs) {
   typedef typename S::elem elem;
   constexpr int V = S::VEC, NV = chip_nv<S>();
   typedef typename RawVec<V * sizeof(elem)>::type raw;
@@ -499,7 +502,12 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
   __shared__ float part_a[kChipMaxG], part_b[kChipMaxG];
   __shared__ int gave_up;
   __shared__ unsigned long long ticket_s;
-  const int c = blockIdx.x / G, g = blockIdx.x - c * G, t = threadIdx.x;
+  // Channels of few slices: each XCD (workgroup w runs on XCD w % 8) takes a run of consecutive channels, see
+  // k_bn_bwd_resident; gridDim.x is then 8 * (channels per XCD) * G.  The slices of a channel stay G
+  // consecutive workgroups of their XCD, so the oldest unfinished channel of an XCD still completes.
+  const int unit = xcd_runs ? int(blockIdx.x & 7) * int(gridDim.x >> 3) + int(blockIdx.x >> 3) : int(blockIdx.x);
+  const int c = unit / G, g = unit - c * G, t = threadIdx.x;
+  if (c >= s.C) return;
   unsigned long long *words = ws + size_t(c) * 2 * size_t(G);   // the channel's G slots
   if (G > 1 && t == 0) {
     const unsigned long long wa = __hip_atomic_load(words + 2 * g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -574,7 +582,7 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
           gave_up = 1;
           break;
         }
-        __builtin_amdgcn_s_sleep(32);
+        __builtin_amdgcn_s_sleep(4);
       }
       part_a[t] = __uint_as_float(unsigned(wa >> 32));
       part_b[t] = __uint_as_float(unsigned(wb >> 32));
@@ -628,14 +636,16 @@ int launch_onchip(const typename S::elem *dy, const typename S::elem *x, const f
                   const float *save_mean, const float *save_invstd, typename S::elem *dx, float *dgamma, float *dbeta,
                   void *workspace, const BnShape &s, const ChipPlan &p, hipStream_t st) {
   unsigned long long *ws = static_cast<unsigned long long *>(workspace);
-  const dim3 grid(unsigned(s.C) * p.G);
+  // (a run of channels per XCD needs the G workgroups of a channel resident on one XCD's 32 CUs together)
+  const int xcd_runs = p.G <= 16 && s.C >= 8 ? 1 : 0;
+  const dim3 grid(xcd_runs ? unsigned((s.C + 7) / 8) * 8u * p.G : unsigned(s.C) * p.G);
   const unsigned long long t1 = next_ticket(), t2 = next_ticket();
   if (p.nt == 512)
     hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean, save_invstd,
-                       dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit);
+                       dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
   else
     hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 1024>), grid, dim3(1024), 0, st, dy, x, gamma, beta, save_mean,
-                       save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit);
+                       save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -657,7 +667,7 @@ int launch_resident(const typename S::elem *dy, const typename S::elem *x, const
     attr = true;
   }
   const size_t lds = 2 * resident_half_bytes(s.N, s.HW, sizeof(typename S::elem));
-  hipLaunchKernelGGL(kern, dim3(s.C), dim3(kResNT), lds, st, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta,
+  hipLaunchKernelGGL(kern, dim3((s.C + 7) / 8 * 8), dim3(kResNT), lds, st, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta,
                      s);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }

@@ -250,6 +250,134 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_bwd_tiled(const typename S:
   }
 }
 
+// Max-pool backward for the residual networks' pooling layer: 3 x 3 windows, stride 2, padding 1, even H and W.
+// The dx block (rows 2i, 2i+1; columns 2j, 2j+1) can only receive from windows (i, j), (i, j+1), (i+1, j),
+// (i+1, j+1), and only at fixed positions of those windows, so instead of tables of arg-max positions and
+// dy values in LDS (the general kernel above: 67 vector instructions per dx element, which bound it) a lane
+// walks down one window column with everything in registers:
+//   * window p shares its top row with window p - 1's bottom row: the per-row first maximum (strict '>',
+//     left to right) is computed once per x row, and three of them combine top to bottom -- the same winner
+//     as the row-major scan of the CPU loop;
+//   * the winner is kept as a code 3 * dh + dw; the right-hand neighbour's code and dy come from lane + 1;
+//   * a block's four elements add the dy of the windows whose code names them, in ascending (p, q) order
+//     starting from +0.0, exactly the additions of the general kernel.
+// A workgroup owns kStripRows block rows per wavefront of one plane; x rows are staged in LDS as stored, behind
+// an element and (for the first band) a row of -inf, so no position needs a bounds check.
+constexpr int kStripRows = 7;   // block rows per wavefront (a wavefront also computes the window row below them)
+constexpr float kLowest = -3.402823466e38f;
+
+struct RowBest {
+  float m;
+  int k;   // column within the window (0..2), 64 = none
+};
+
+template <class S>
+__device__ __forceinline__ RowBest row_best(const typename S::elem *row) {   // row -> the window's middle element of one x row
+  typedef typename S::elem elem;
+  float a, b, c;
+  if constexpr (sizeof(elem) == 4) {
+    a = row[-1];
+    const float2 bc = *reinterpret_cast<const float2 *>(row);
+    b = bc.x, c = bc.y;
+  } else {
+    const unsigned pr = *reinterpret_cast<const unsigned *>(row);
+    const elem lo = elem(pr & 0xffffu), hi = elem(pr >> 16);
+    a = S::ld(row - 1), b = S::ld(&lo), c = S::ld(&hi);
+  }
+  RowBest r{kLowest, 64};
+  if (a > r.m) r.m = a, r.k = 0;
+  if (b > r.m) r.m = b, r.k = 1;
+  if (c > r.m) r.m = c, r.k = 2;
+  return r;
+}
+
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_pool_max_bwd_3x3s2(const typename S::elem *__restrict__ dy,
+                                                               const typename S::elem *__restrict__ x,
+                                                               typename S::elem *__restrict__ dx, int H, int W, int bands) {
+  typedef typename S::elem elem;
+  constexpr int V = S::VEC;
+  typedef sgh_v4u raw;   // 16 bytes: V elements
+  // x rows as stored: element (r, w) at (r - r_lo) * pitch + V + w (rows start on 16-byte boundaries), the element
+  // before a row and the row above the image hold -inf, which no comparison selects
+  extern __shared__ __align__(16) unsigned char xs_raw[];
+  elem *xs = reinterpret_cast<elem *>(xs_raw);
+  const int P = H >> 1, Q = W >> 1, pitch = W + V;
+  const int plane = blockIdx.x / bands, band = blockIdx.x - plane * bands;
+  const int i0 = band * (4 * kStripRows), i1 = min(i0 + 4 * kStripRows, P);   // block rows (= window rows) of the band
+  const int r_lo = 2 * i0 - 1, r_hi = min(2 * i1 + 1, H - 1), rr0 = max(r_lo, 0);
+  const elem *xb = x + size_t(plane) * H * W;
+  const elem *db = dy + size_t(plane) * P * Q;
+  elem *ob = dx + size_t(plane) * H * W;
+  const int vpr = W / V;   // 16-byte (8-byte) vectors per row
+  for (int i = threadIdx.x; i < (r_hi - rr0 + 1) * vpr; i += kBlock) {
+    const int r = i / vpr, c = (i - r * vpr) * V;
+    *reinterpret_cast<raw *>(xs + (rr0 - r_lo + r) * pitch + V + c) =
+        __builtin_nontemporal_load(reinterpret_cast<const raw *>(xb + size_t(rr0 + r) * W + c));
+  }
+  for (int r = threadIdx.x; r <= r_hi - r_lo; r += kBlock) S::st(xs + r * pitch + V - 1, -__builtin_inff());
+  if (r_lo < 0)
+    for (int c = threadIdx.x; c < pitch; c += kBlock) S::st(xs + c, -__builtin_inff());
+  __syncthreads();
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ia = i0 + wave * kStripRows, ib = min(ia + kStripRows, i1);   // this wavefront's block rows [ia, ib)
+  if (ia >= ib) return;
+  for (int q0 = 0; q0 < Q; q0 += 63) {   // lanes 0..62 produce blocks, lane 63 only hands its window to lane 62
+    const int q = q0 + lane;
+    const bool col = q < Q;
+    const int qc = col ? q : Q - 1;   // (a lane without a window reads a valid address and discards it)
+    float dyr[kStripRows + 1];
+#pragma unroll
+    for (int k = 0; k <= kStripRows; ++k) {
+      const int p = ia + k;
+      dyr[k] = (p <= ib && p < P && col) ? S::ld(db + p * Q + q) : 0.f;
+    }
+    const elem *xq = xs + (2 * ia - r_lo) * pitch + V + 2 * qc;   // element (2 ia, 2 q)
+    RowBest top = row_best<S>(xq - pitch);
+    int code_p = 64, ncode_p = 64;
+    float dy_p = 0.f, ndy_p = 0.f;
+#pragma unroll
+    for (int k = 0; k <= kStripRows; ++k) {
+      const int p = ia + k;
+      if (p > ib) break;
+      int code = 64;
+      if (p < P) {
+        const RowBest mid = row_best<S>(xq + (2 * k) * pitch), bot = row_best<S>(xq + (2 * k + 1) * pitch);
+        float best = top.m;
+        code = top.k;
+        if (mid.m > best) best = mid.m, code = 3 + mid.k;
+        if (bot.m > best) code = 6 + bot.k;
+        if (!col) code = 64;
+        top = bot;
+      }
+      const float dyv = dyr[k];
+      const int ncode = __shfl_down(code, 1);
+      const float ndy = __shfl_down(dyv, 1);
+      if (k > 0 && lane < 63 && col) {
+        // block row p - 1: windows (p-1, q), (p-1, q+1), (p, q), (p, q+1) in that order
+        const float o00 = 0.f + (code_p == 4 ? dy_p : 0.f);
+        const float o01 = (0.f + (code_p == 5 ? dy_p : 0.f)) + (ncode_p == 3 ? ndy_p : 0.f);
+        const float o10 = (0.f + (code_p == 7 ? dy_p : 0.f)) + (code == 1 ? dyv : 0.f);
+        const float o11 = (((0.f + (code_p == 8 ? dy_p : 0.f)) + (ncode_p == 6 ? ndy_p : 0.f)) + (code == 2 ? dyv : 0.f)) +
+                          (ncode == 0 ? ndy : 0.f);
+        elem *o = ob + size_t(2 * (p - 1)) * W + 2 * q;
+        if constexpr (sizeof(elem) == 4) {
+          typedef float v2f __attribute__((ext_vector_type(2)));
+          __builtin_nontemporal_store(v2f{o00, o01}, reinterpret_cast<v2f *>(o));
+          __builtin_nontemporal_store(v2f{o10, o11}, reinterpret_cast<v2f *>(o + W));
+        } else {
+          elem t0[2], t1[2];
+          S::st(t0, o00), S::st(t0 + 1, o01), S::st(t1, o10), S::st(t1 + 1, o11);
+          *reinterpret_cast<unsigned *>(o) = unsigned(t0[0]) | (unsigned(t0[1]) << 16);
+          *reinterpret_cast<unsigned *>(o + W) = unsigned(t1[0]) | (unsigned(t1[1]) << 16);
+        }
+      }
+      code_p = code, ncode_p = ncode, dy_p = dyv, ndy_p = ndy;
+    }
+  }
+}
+
 __device__ __forceinline__ int window_count(const PoolG g, int p, int q, int *hs_, int *he_, int *ws_, int *we_) {
   int hs = p * g.sh - g.ph, ws = q * g.sw - g.pw;
   const int he = min(hs + g.kh, g.H), we = min(ws + g.kw, g.W);
@@ -353,7 +481,15 @@ int pool_bwd(const sgh_pool_geom *g, const typename S::elem *dy, const typename 
                       double(sizeof(typename S::elem)) *
                           (double(total) * (g->is_max ? 2 : 1) + double(g->N) * g->C * g->P * g->Q),
                       sgh_stream_of(stream));
-  if (g->is_max) {
+  if (g->is_max && g->kernel_h == 3 && g->kernel_w == 3 && g->stride_h == 2 && g->stride_w == 2 && g->pad_h == 1 &&
+      g->pad_w == 1 && g->H % 2 == 0 && g->W % S::VEC == 0 && g->W <= 256 &&
+      size_t(g->N) * g->C * ((g->H / 2 + 4 * kStripRows - 1) / (4 * kStripRows)) < 0x7fffffffu && sgh_aligned16(x) &&
+      sgh_aligned16(dx)) {
+    const int bands = (g->H / 2 + 4 * kStripRows - 1) / (4 * kStripRows);
+    const size_t lds = size_t(8 * kStripRows + 3) * (g->W + S::VEC) * sizeof(typename S::elem);   // <= 61 KB
+    hipLaunchKernelGGL(k_pool_max_bwd_3x3s2<S>, dim3(unsigned(size_t(g->N) * g->C * bands)), dim3(kBlock), lds,
+                       sgh_stream_of(stream), dy, x, dx, g->H, g->W, bands);
+  } else if (g->is_max) {
     // band height: about 12 KB of x rows per workgroup (measured optimum: enough workgroups per CU to
     // overlap one's staging with another's scans), bands of equal height
     int TH = 3072 / g->W - g->kernel_h;

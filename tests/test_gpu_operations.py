@@ -336,6 +336,9 @@ POOL_CASES = [
     (1, 2, 7, 5, (3, 2), (1, 2), (1, 0)),
     (2, 2, 6, 6, (2, 2), (3, 3), (0, 0)),        # stride > kernel: inputs outside every window
     (4, 512, 7, 7, (7, 7), (1, 1), (0, 0)),      # ResNet global pool geometry
+    (3, 5, 12, 8, (3, 3), (2, 2), (1, 1)),       # window-column kernel: one partial wavefront strip
+    (2, 3, 60, 16, (3, 3), (2, 2), (1, 1)),      # ... two bands (28 + 2 block rows)
+    (1, 2, 6, 256, (3, 3), (2, 2), (1, 1)),      # ... 128 window columns: three column groups of 63
 ]
 
 
@@ -376,6 +379,19 @@ def test_max_pool_bit_exact(singa, dev, case, ties):
     assert_bit_equal(y.to_numpy(), y_o, "max-pool forward")
     dx = singa.GpuPoolingBackward(h, singa.from_numpy(dy, dev), xd, y).to_numpy()
     assert_bit_equal(dx, O.pool_max_bwd(dy, mask, x.shape), "max-pool routing")
+
+
+def test_max_pool_backward_keeps_the_sign_of_zero_sums(singa, dev):
+    """A dx element that receives only -0.0 gradients is +0.0 on the CPU (its sum starts at +0.0)."""
+    r = rng(5)
+    x = randn(r, 2, 3, 16, 16)
+    y_o, mask = O.pool_max_fwd(x, (3, 3), (2, 2), (1, 1))
+    dy = np.where(r.random(y_o.shape) < 0.5, np.float32(-0.0), randn(r, *y_o.shape)).astype(np.float32)
+    xd = singa.from_numpy(x, dev)
+    h = singa.CudnnPoolingHandle(xd, (3, 3), (2, 2), (1, 1), True)
+    y = singa.GpuPoolingForward(h, xd)
+    dx = singa.GpuPoolingBackward(h, singa.from_numpy(dy, dev), xd, y).to_numpy()
+    assert_bit_equal(dx, O.pool_max_bwd(dy, mask, x.shape), "max-pool routing with -0.0 gradients")
 
 
 @pytest.mark.parametrize("case", POOL_CASES)
