@@ -388,6 +388,7 @@ struct D16Args {
   const uint16_t *bias;  // per output row (channel c), or null: the forward pass run as a data gradient
   int fs;   // step of the gradient pixel per output pixel: 1, or the stride of a forward pass run on this kernel
             // (pixel-major loads only): tap (ti, tj) of output pixel (i, j) reads (fs * i + dr0 - ti, fs * j + ds0 - tj)
+  int rowstore;   // the tile leaves as contiguous rows (stride 1, even width, planes of whole 8-byte groups, dx 16-byte aligned)
   int dilate, out_W, out_HW;   // 1x1 stride 2: the kernel sees the stride-1 problem on the P x Q grid and its store
                                // writes the 2 x 2 block (value, 0 / 0, 0) of the real out_HW image per pixel
 };
@@ -553,6 +554,46 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 
   // epilogue: lane's pixel column, 16 channel rows per accumulator
   combine_halves<TM>(reinterpret_cast<float *>(lds16), half, w4, lane, acc);
+  if (a.rowstore) {
+    // Stride 1 on an even width with planes that are whole 8-byte groups: the tile is 128 consecutive pixels of
+    // dx, so it goes through LDS as [channel][pixel] and leaves in 8- or 16-byte pieces of contiguous rows (a
+    // wavefront's own layout, one pixel per lane and 2 bytes per store, kept the vector memory path busy
+    // longer than the whole reduction on the layers with large outputs).
+    constexpr int OP = BN + 8;
+    uint16_t *ot = lds16;
+    __syncthreads();   // the exchange above has been read
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+        float r = acc[i][0][v];
+        if (a.bias && m0 + row < a.C) r += BF16 ? sgh_bf16_to_f32(a.bias[m0 + row]) : sgh_f16_to_f32(a.bias[m0 + row]);
+        ot[row * OP + wn * 64 + half * 32 + l32] = round16<BF16>(r);
+      }
+    __syncthreads();
+    if ((HW & 7) == 0) {
+      const int g = t & 15;
+      const long p8 = pix0 + 8 * g;
+      if (p8 < cnt) {
+        const int n = int(p8 / HW), rem = int(p8 - long(n) * HW);
+        uint16_t *o = a.dx + (size_t(n) * a.C + m0) * HW + rem;
+        for (int row = t >> 4; row < BM && m0 + row < a.C; row += NT / 16)
+          *reinterpret_cast<u32x4 *>(o + size_t(row) * HW) = *reinterpret_cast<const u32x4 *>(ot + row * OP + 8 * g);
+      }
+    } else {
+      typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+      const int g = t & 31;
+      const long p4 = pix0 + 4 * g;
+      if (p4 < cnt) {
+        const int n = int(p4 / HW), rem = int(p4 - long(n) * HW);
+        uint16_t *o = a.dx + (size_t(n) * a.C + m0) * HW + rem;
+        for (int row = t >> 5; row < BM && m0 + row < a.C; row += NT / 32)
+          *reinterpret_cast<u32x2 *>(o + size_t(row) * HW) = *reinterpret_cast<const u32x2 *>(ot + row * OP + 4 * g);
+      }
+    }
+    return;
+  }
   const long pix = pix0 + wn * 64 + half * 32 + l32;   // the block this group kept
   if (pix >= cnt) return;
   const int n = int(pix / HWc), rem = int(pix - long(n) * HWc), i_ = rem / Wc, j_ = rem - i_ * Wc;
@@ -890,6 +931,8 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
   a.stride = kg->stride_h, a.pad_h = kg->pad_h, a.pad_w = kg->pad_w;
   a.dilate = p.dilate ? 1 : 0, a.out_W = g->W, a.out_HW = g->H * g->W;
   a.fs = p.fs;
+  a.rowstore = (!p.dilate && kg->stride_h == 1 && kg->W % 2 == 0 && (kg->H * kg->W) % 4 == 0 &&
+                (reinterpret_cast<uintptr_t>(dx) & 15u) == 0) ? 1 : 0;
   a.KP = p.KP, a.CP = p.CP, a.mtiles = p.mtiles, a.ptiles = p.tiles;
   for (int i = 0; i < 5; ++i) a.cls_tile0[i] = p.cls_tile0[i];
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2);
