@@ -32,7 +32,7 @@ static inline bool sgh_aligned16(const void *p) { return (reinterpret_cast<uintp
 // when the first entry point asks: changing the environment later has no effect, so a geometry's
 // workspace size and kernel choice cannot change between two calls.
 struct sgh_env_switches {
-  bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off, bn_onchip_off, pw_dgrad_off;
+  bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off, bn_onchip_off, pw_dgrad_off, pw_wgrad_off;
   int dgrad_tile, wgrad_tile, pw_tile;   // -1: chosen from the geometry
   int dgrad3x3_bm;              // 0: chosen from the geometry, else 64 or 128
 };
@@ -110,6 +110,9 @@ int sgh_dgrad_fewc_run16(const sgh_conv_geom *g, const uint16_t *dy, const float
 
 // Data gradient of 1x1 convolutions without padding, fed from global memory without LDS (pointwise.hip):
 // K a multiple of 32, at least 32 input channels, equal strides.
+size_t sgh_pw_wgrad_workspace_bytes(const sgh_conv_geom *g);   // 0: not a layer of the pointwise weight-gradient kernel
+int sgh_pw_wgrad_run(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace, size_t ws_bytes,
+                     hipStream_t s);
 bool sgh_pw_dgrad_supported(const sgh_conv_geom *g);
 int sgh_pw_dgrad_run(const sgh_conv_geom *g, const float *dy, const float *W, float *dx, hipStream_t s);
 

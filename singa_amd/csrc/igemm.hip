@@ -922,6 +922,8 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
       if (tiled) return tiled;
       const size_t fewc = sgh_wgrad_fewc_workspace_bytes(g);
       if (fewc) return fewc;
+      const size_t pw = sgh_env().pw_wgrad_off ? 0 : sgh_pw_wgrad_workspace_bytes(g);
+      if (pw) return pw;
       const WgradPlan p = plan_wgrad(g);
       // split partials of dW, then those of the bias gradient that may ride along (sgh_conv_wgrad_bias_f32)
       return p.splits > 1 ? align256(size_t(p.splits) * g->K * g->C * RS * sizeof(float)) + size_t(p.splits) * g->K * sizeof(float) : 0;
@@ -1315,6 +1317,12 @@ static int conv_wgrad(sgh_conv_geom *g, const float *dy, const float *x, float *
     const int rcf = sgh_wgrad_fewc_run(g, dy, x, dW, workspace, ws_bytes, sgh_stream_of(stream));
     sgh_prof_stop(sgh_stream_of(stream));
     return rcf == SGH_OK && db ? bgrad_launch(g, dy, db, sgh_stream_of(stream)) : rcf;
+  }
+  if (!sgh_env().pw_wgrad_off && sgh_pw_wgrad_workspace_bytes(g)) {  // 1x1 strided (the downsample layers)
+    sgh_prof_start("conv_wgrad_op", conv_flops(g), sgh_stream_of(stream));
+    const int rcp = sgh_pw_wgrad_run(g, dy, x, dW, workspace, ws_bytes, sgh_stream_of(stream));
+    sgh_prof_stop(sgh_stream_of(stream));
+    return rcp == SGH_OK && db ? bgrad_launch(g, dy, db, sgh_stream_of(stream)) : rcp;
   }
   const WgradPlan p = plan_wgrad(g);
   const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_WGRAD);

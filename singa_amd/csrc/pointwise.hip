@@ -136,6 +136,163 @@ __global__ __launch_bounds__(256) void k_pw_dgrad(PwArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Weight gradient of the same layers: dW[k][c] = sum_{n,p,q} dy[n][k][p][q] * x[n][c][s*p][s*q].
+//
+// The reduction runs over pixels, which are contiguous in dy and every s-th element of every s-th row in x.
+// A unit of the reduction is one output row (n, p): Q pixels.  Per unit a workgroup (4 wavefronts, tile
+// 128 k x 64 c) stages dyS[k][q] and xS[c][q] in LDS -- every staging address is a thread constant plus a
+// scalar term of the unit (no division and no predicate per element: what the generic implicit-GEMM loaders
+// spend their time on for these layers) -- and multiplies with v_mfma_f32_32x32x2_f32, lane (i, h) reading
+// element (row i, pixel 2 t + h) of each operand (row pitch odd: conflict-free).  The loads of the next unit
+// are in flight while the current one is multiplied.  The units are split over workgroups; partial sums
+// [split][K][C] are added in ascending split order by k_pw_wgrad_reduce (16 z-lanes in a fixed order), so the
+// result is run-to-run identical.
+struct PwWArgs {
+  const float *dy, *x;
+  float *part;
+  int N, C, K, H, Wd, P, Q, s;
+  int mtiles, ntiles, units, ups;   // units = N * P rows, `ups` of them per split
+  unsigned dy_bytes, x_bytes;
+};
+
+template <int QC>   // the number of pixels per row Q, known at compile time (divisions by it become multiplications)
+__global__ __launch_bounds__(256) void k_pw_wgrad(PwWArgs a) {
+  constexpr int BM = 128, BN = 64, Q = QC, DS = (BM * Q + 255) / 256, XS = (BN * Q + 255) / 256;
+  constexpr int QP = (Q + 1) | 1;               // odd, and a zero column behind an odd number of pixels
+  constexpr int STEPS = (Q + 1) / 2;
+  extern __shared__ float lds[];
+  float *dyS0 = lds, *xS0 = lds + BM * QP, *dyS1 = lds + (BM + BN) * QP, *xS1 = dyS1 + BM * QP;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, i32 = lane & 31, h = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tile = int(blockIdx.x) % (a.mtiles * a.ntiles), split = int(blockIdx.x) / (a.mtiles * a.ntiles);
+  const int k0 = (tile / a.ntiles) * BM, c0 = (tile % a.ntiles) * BN;
+  const int u0 = split * a.ups, u1 = min(u0 + a.ups, a.units);
+  const int PQ = a.P * Q, HW = a.H * a.Wd;
+  const rsrc_t rdy = make_rsrc(a.dy, a.dy_bytes), rx = make_rsrc(a.x, a.x_bytes);
+  // the columns behind the pixels stay zero (nothing else is read before it is written)
+  for (int i = t; i < 2 * (BM + BN); i += 256)
+#pragma unroll
+    for (int q = Q; q < QP; ++q) lds[i * QP + q] = 0.f;
+
+  int dvo[DS], dlo[DS], xvo[XS], xlo[XS];
+#pragma unroll
+  for (int i = 0; i < DS; ++i) {
+    const int e = i * 256 + t, k = e / Q, q = e - k * Q;
+    const bool ok = k < BM && k0 + k < a.K;
+    dvo[i] = ok ? ((k0 + k) * PQ + q) * 4 : kOOB;
+    dlo[i] = k < BM ? k * QP + q : -1;
+  }
+#pragma unroll
+  for (int i = 0; i < XS; ++i) {
+    const int e = i * 256 + t, c = e / Q, q = e - c * Q;
+    const bool ok = c < BN && c0 + c < a.C;
+    xvo[i] = ok ? ((c0 + c) * HW + a.s * q) * 4 : kOOB;
+    xlo[i] = c < BN ? c * QP + q : -1;
+  }
+  // two register sets: the loads of unit u + 2 are issued before unit u is multiplied
+  float dr[2][DS], xr[2][XS];
+  auto load = [&](int set, int u) {
+    const bool live = u < u1;
+    const int n = live ? u / a.P : 0, p = live ? u - n * a.P : 0;
+    const int dso = (n * a.K * PQ + p * Q) * 4, xso = (n * a.C * HW + a.s * p * a.Wd) * 4;
+#pragma unroll
+    for (int i = 0; i < DS; ++i)
+      dr[set][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rdy, live ? dvo[i] : kOOB, dso, 0));
+#pragma unroll
+    for (int i = 0; i < XS; ++i)
+      xr[set][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rx, live ? xvo[i] : kOOB, xso, 0));
+  };
+  auto stage = [&](int set, float *dS, float *xS) {
+#pragma unroll
+    for (int i = 0; i < DS; ++i)
+      if (dlo[i] >= 0) dS[dlo[i]] = dr[set][i];
+#pragma unroll
+    for (int i = 0; i < XS; ++i)
+      if (xlo[i] >= 0) xS[xlo[i]] = xr[set][i];
+  };
+  v16f acc0, acc1;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc0[v] = 0.f, acc1[v] = 0.f;
+  const int ao = (wm * 64 + i32) * QP + h, bo = (wn * 32 + i32) * QP + h;
+  auto mma = [&](const float *dS, const float *xS) {
+    float a0[STEPS], a1[STEPS], b[STEPS];
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) a0[st] = dS[ao + 2 * st], a1[st] = dS[ao + 32 * QP + 2 * st], b[st] = xS[bo + 2 * st];
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[st], b[st], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[st], b[st], acc1, 0, 0, 0);
+    }
+  };
+  load(0, u0);
+  load(1, u0 + 1);
+  __syncthreads();   // (the zero columns)
+  for (int u = u0; u < u1; u += 2) {
+    stage(0, dyS0, xS0);
+    __syncthreads();
+    load(0, u + 2);
+    mma(dyS0, xS0);
+    if (u + 1 >= u1) break;
+    stage(1, dyS1, xS1);
+    __syncthreads();
+    load(1, u + 3);
+    mma(dyS1, xS1);
+  }
+  float *out = a.part + size_t(split) * a.K * a.C;
+  const int c = c0 + wn * 32 + i32;
+  if (c < a.C) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int m = k0 + wm * 64 + 8 * (v >> 2) + 4 * h + (v & 3);
+      if (m < a.K) out[size_t(m) * a.C + c] = acc0[v];
+      if (m + 32 < a.K) out[size_t(m + 32) * a.C + c] = acc1[v];
+    }
+  }
+}
+
+// out[i] = sum over splits of part[z][i], z ascending within each of 16 z-lanes, the lanes added in lane order
+__global__ __launch_bounds__(256) void k_pw_wgrad_reduce(const float *__restrict__ part, float *__restrict__ out, long n,
+                                                        int splits) {
+  __shared__ float lanes[16][17];
+  const int e = threadIdx.x & 15, zl = threadIdx.x >> 4;
+  const long i = long(blockIdx.x) * 16 + e;
+  float s = 0.f;
+  if (i < n)
+    for (int z = zl; z < splits; z += 16) s += part[long(z) * n + i];
+  lanes[zl][e] = s;
+  __syncthreads();
+  if (threadIdx.x < 16 && i < n) {
+    float r = lanes[0][e];
+#pragma unroll
+    for (int l = 1; l < 16; ++l) r += lanes[l][e];
+    out[i] = r;
+  }
+}
+
+struct PwWPlan {
+  bool ok;
+  int mtiles, ntiles, units, ups, splits;
+};
+
+PwWPlan pw_wgrad_plan(const sgh_conv_geom *g) {
+  PwWPlan p{};
+  if (g->R != 1 || g->S != 1 || g->pad_h != 0 || g->pad_w != 0 || g->stride_h != g->stride_w || g->stride_h < 2) return p;
+  if ((g->Q != 28 && g->Q != 14 && g->Q != 7) || g->K < 32 || g->C < 32) return p;   // (the rows of the residual networks)
+  const size_t lim = size_t(1) << 29;   // byte offsets stay below 2^31
+  if (size_t(g->N) * g->K * g->P * g->Q >= lim || size_t(g->N) * g->C * g->H * g->W >= lim) return p;
+  p.mtiles = (g->K + 127) / 128, p.ntiles = (g->C + 63) / 64;
+  p.units = g->N * g->P;
+  // about two workgroups per CU; at least four rows per workgroup so that the pipeline has something to overlap
+  int splits = 2 * sgh_num_cus() / (p.mtiles * p.ntiles);
+  if (splits < 1) splits = 1;
+  if (splits > p.units / 4) splits = p.units / 4 > 0 ? p.units / 4 : 1;
+  p.ups = (p.units + splits - 1) / splits;
+  p.splits = (p.units + p.ups - 1) / p.ups;
+  p.ok = true;
+  return p;
+}
+
 }  // namespace
 
 bool sgh_pw_dgrad_supported(const sgh_conv_geom *g) {
@@ -165,5 +322,34 @@ int sgh_pw_dgrad_run(const sgh_conv_geom *g, const float *dy, const float *W, fl
   if (big) hipLaunchKernelGGL((k_pw_dgrad<2, 2>), dim3(blocks), dim3(256), 0, s, a);
   else hipLaunchKernelGGL((k_pw_dgrad<1, 1>), dim3(blocks), dim3(256), 0, s, a);
   sgh_prof_stop(s);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
+size_t sgh_pw_wgrad_workspace_bytes(const sgh_conv_geom *g) {
+  const PwWPlan p = pw_wgrad_plan(g);
+  return p.ok ? size_t(p.splits) * g->K * g->C * sizeof(float) : 0;
+}
+
+int sgh_pw_wgrad_run(const sgh_conv_geom *g, const float *dy, const float *x, float *dW, void *workspace, size_t ws_bytes,
+                     hipStream_t s) {
+  const PwWPlan p = pw_wgrad_plan(g);
+  if (!p.ok) return SGH_EUNSUPPORTED;
+  if (!workspace || ws_bytes < sgh_pw_wgrad_workspace_bytes(g)) return SGH_EWORKSPACE;
+  PwWArgs a{};
+  a.dy = dy, a.x = x, a.part = static_cast<float *>(workspace);
+  a.N = g->N, a.C = g->C, a.K = g->K, a.H = g->H, a.Wd = g->W, a.P = g->P, a.Q = g->Q, a.s = g->stride_h;
+  a.mtiles = p.mtiles, a.ntiles = p.ntiles, a.units = p.units, a.ups = p.ups;
+  a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 4), a.x_bytes = unsigned(size_t(g->N) * g->C * g->H * g->W * 4);
+  const int QP = (g->Q + 1) | 1;
+  const size_t lds = size_t(2) * (128 + 64) * QP * sizeof(float);
+  const dim3 grid(unsigned(p.mtiles * p.ntiles * p.splits));
+  sgh_prof_start("conv_wgrad/k_pw_wgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C, s);
+  if (g->Q == 7) hipLaunchKernelGGL(k_pw_wgrad<7>, grid, dim3(256), lds, s, a);
+  else if (g->Q == 14) hipLaunchKernelGGL(k_pw_wgrad<14>, grid, dim3(256), lds, s, a);
+  else hipLaunchKernelGGL(k_pw_wgrad<28>, grid, dim3(256), lds, s, a);
+  sgh_prof_stop(s);
+  if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
+  const long n = long(g->K) * g->C;
+  hipLaunchKernelGGL(k_pw_wgrad_reduce, dim3(unsigned((n + 15) / 16)), dim3(256), 0, s, a.part, dW, n, p.splits);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }

@@ -92,6 +92,9 @@ CONV_CASES = [
     (2, 1, 16, 16, 8, 7, 7, (2, 2), (3, 3), True),        # direct few-channel dgrad: one channel
     (32, 96, 57, 57, 32, 1, 1, (2, 2), (0, 0), False),    # 1x1 stride 2, 64 x 64 wavefront tiles: ragged channel tile, odd image
     (2, 48, 11, 11, 64, 1, 1, (3, 3), (0, 0), False),     # 1x1 stride 3 on the matrix-instruction-from-global-memory kernel
+    (3, 40, 28, 28, 96, 1, 1, (2, 2), (0, 0), True),      # 1x1 stride 2, rows of 14: pointwise weight gradient, ragged tiles
+    (2, 64, 56, 56, 130, 1, 1, (2, 2), (0, 0), False),    # ... rows of 28, a second (nearly empty) row tile
+    (5, 33, 14, 14, 160, 1, 1, (2, 2), (0, 0), False),    # ... rows of 7 (odd: zero column behind the pixels)
 ]
 
 
