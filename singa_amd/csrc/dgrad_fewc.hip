@@ -190,6 +190,145 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same data gradient on 16-bit tensors with the 16-bit matrix instruction
+// (v_mfma_f32_16x16x32_{f16,bf16}: M = 16 rows (c, a, b), N = 16 block columns j, 32 reduction indices per
+// instruction, fp32 accumulation).  The reduction is ordered (offset (dp, dq), k) with k fastest, so one
+// instruction consumes 32 channels k of one offset and a lane supplies eight consecutive k of its pixel:
+// the gradient slab sits in LDS pixel-major, slab[row][col][k] (80-byte pitch: the 64 lanes of a fragment
+// read spread evenly over the banks), transposed once per 32 channels while it is staged (dword = two
+// pixels of one k; eight k and two v_perm give two 16-byte octets) and then read by all 16 offsets.  The
+// weight fragments A[off][m][k] come straight from global memory (32 KB per layer, cache resident), all 16
+// of a chunk before its first matrix instruction.  One wavefront per class row, four rows per workgroup,
+// two workgroups per CU.  Every fragment read is 1 KB of LDS for 16 cycles of matrix work, so the kernel is
+// bound by LDS bandwidth, at several times the fp32 instruction's rate.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int TI16 = 4, SR16 = TI16 + ND - 1, KC16 = 32, KP16 = KC16 + 8;
+
+struct DF16Args {
+  const uint16_t *dy;
+  const uint16_t *aw;     // A re-laid as [dp,dq (16)][m (16)][KA], 16-bit, KA = K rounded up to 32
+  uint16_t *dx;
+  int N, C, H, W, K, KA, P, Q;
+  int dp0, dq0;
+};
+
+// aw[(off * 16 + m) * KA + k], m = c*4 + a*2 + b; W holds the 16-bit weights widened to fp32 (exact)
+template <bool BF16>
+__global__ __launch_bounds__(256) void k_dgrad_fewc16_weights(const float *__restrict__ W, uint16_t *__restrict__ aw, int K,
+                                                             int KA, int C, int R, int S, int ph, int pw, int dp0,
+                                                             int dq0) {
+  const int total = ND * ND * 16 * KA;
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+    const int k = i % KA, m = (i / KA) & 15, off = i / (KA * 16);
+    const int c = m >> 2, a = (m >> 1) & 1, b = m & 1;
+    const int r = a + ph - 2 * (dp0 + off / ND), s = b + pw - 2 * (dq0 + off % ND);
+    const bool ok = k < K && c < C && unsigned(r) < unsigned(R) && unsigned(s) < unsigned(S);
+    const float v = ok ? W[((long(k) * C + c) * R + r) * S + s] : 0.f;
+    aw[i] = BF16 ? sgh_f32_to_bf16(v) : sgh_f32_to_f16(v);
+  }
+}
+
+template <int QT, bool BF16>
+__global__ __launch_bounds__(256) void k_dgrad_fewc16(DF16Args a) {
+  constexpr int COLS = QT * 16 + 8;                      // slab column of dy column q is q + 4
+  constexpr int UN = (SR16 * QT * 8 * 4 + 255) / 256;    // staging units per thread (upper bound): (row, pixel pair, k octet)
+  extern __shared__ __align__(16) uint16_t slab[];       // [SR16][COLS][KP16]
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int i0 = blockIdx.x * TI16, n = blockIdx.y;
+  const int PQ = a.P * a.Q, HW = a.H * a.W, Q2 = a.Q >> 1, npair = SR16 * Q2;
+  const rsrc_t rdy = make_rsrc(a.dy + size_t(n) * a.K * PQ, unsigned(a.K) * PQ * 2u);
+  const rsrc_t raw = make_rsrc(a.aw, unsigned(ND * ND * 16) * a.KA * 2u);
+
+  // rows outside the image and the pad columns stay zero: only image pixels are (re)written
+  for (int i = t; i < SR16 * COLS * KP16 / 8; i += 256) reinterpret_cast<u32x4 *>(slab)[i] = u32x4{0u, 0u, 0u, 0u};
+
+  int sg[UN], sl[UN];
+#pragma unroll
+  for (int e = 0; e < UN; ++e) {
+    const int u = e * 256 + t, ko = u / npair, pr = u - ko * npair, sr = pr / Q2, pp = pr - sr * Q2;
+    const int p = i0 + a.dp0 + sr;
+    const bool ok = ko < 4 && unsigned(p) < unsigned(a.P);
+    sg[e] = ok ? ((ko * 8 * a.P + p) * a.Q + 2 * pp) * 2 : kOOB;
+    sl[e] = ok ? (sr * COLS + 2 * pp + 4) * KP16 + ko * 8 : -1;
+  }
+  const int m = lane & 15, g = lane >> 4;
+  const int aoff = (m * a.KA + 8 * g) * 2;                                   // + off * 16 * KA * 2 + chunk
+  const int boff = (wave * COLS + m + 4 + a.dq0) * KP16 + 8 * g;             // + (dpi * COLS + j * 16 + dqi) * KP16
+
+  v4f acc[QT];
+#pragma unroll
+  for (int i = 0; i < QT; ++i) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  const int nchunks = a.KA / KC16;
+  for (int ch = 0; ch < nchunks; ++ch) {
+    const int k0 = ch * KC16;
+    u32x4 af[ND * ND];
+#pragma unroll
+    for (int o = 0; o < ND * ND; ++o)
+      af[o] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(raw, aoff + o * 16 * a.KA * 2, k0 * 2, 0));
+    unsigned rd[UN][8];
+#pragma unroll
+    for (int e = 0; e < UN; ++e)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        rd[e][j] = unsigned(__builtin_amdgcn_raw_buffer_load_b32(rdy, sg[e], (k0 + j) * PQ * 2, 0));
+    __syncthreads();   // the zero fill / every wavefront has finished reading the previous chunk
+#pragma unroll
+    for (int e = 0; e < UN; ++e) {
+      if (sl[e] < 0) continue;
+      u32x4 vA, vB;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        vA[d] = __builtin_amdgcn_perm(rd[e][2 * d + 1], rd[e][2 * d], 0x05040100u);
+        vB[d] = __builtin_amdgcn_perm(rd[e][2 * d + 1], rd[e][2 * d], 0x07060302u);
+      }
+      *reinterpret_cast<u32x4 *>(slab + sl[e]) = vA;
+      *reinterpret_cast<u32x4 *>(slab + sl[e] + KP16) = vB;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int o = 0; o < ND * ND; ++o) {
+      const int dpi = o / ND, dqi = o % ND;
+      u32x4 bf[QT];
+#pragma unroll
+      for (int j = 0; j < QT; ++j)
+        bf[j] = *reinterpret_cast<const u32x4 *>(slab + boff + (dpi * COLS + j * 16 + dqi) * KP16);
+#pragma unroll
+      for (int j = 0; j < QT; ++j) {
+        if constexpr (BF16)
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af[o]), __builtin_bit_cast(bf16x8, bf[j]),
+                                                           acc[j], 0, 0, 0);
+        else
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[o]), __builtin_bit_cast(f16x8, bf[j]),
+                                                          acc[j], 0, 0, 0);
+      }
+    }
+  }
+
+  // epilogue: lane group lane / 16 is the channel, register v = a*2 + b the position in the 2x2 block
+  const int c = lane >> 4, i = i0 + wave;
+  if (c < a.C && i < a.P) {
+    uint16_t *o = a.dx + (size_t(n) * a.C + c) * HW + size_t(2 * i) * a.W;
+#pragma unroll
+    for (int j = 0; j < QT; ++j) {
+      const int q = j * 16 + (lane & 15);
+      if (q < a.Q) {
+        const unsigned r00 = BF16 ? sgh_f32_to_bf16(acc[j][0]) : sgh_f32_to_f16(acc[j][0]);
+        const unsigned r01 = BF16 ? sgh_f32_to_bf16(acc[j][1]) : sgh_f32_to_f16(acc[j][1]);
+        const unsigned r10 = BF16 ? sgh_f32_to_bf16(acc[j][2]) : sgh_f32_to_f16(acc[j][2]);
+        const unsigned r11 = BF16 ? sgh_f32_to_bf16(acc[j][3]) : sgh_f32_to_f16(acc[j][3]);
+        *reinterpret_cast<unsigned *>(o + 2 * q) = r00 | (r01 << 16);
+        *reinterpret_cast<unsigned *>(o + a.W + 2 * q) = r10 | (r11 << 16);
+      }
+    }
+  }
+}
+
 struct DFPlan {
   bool ok;
   int qt, dp0, dq0;
@@ -303,8 +442,66 @@ int sgh_dgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *W, 
   return dgrad_fewc_run<StF32>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad/k_dgrad_fewc");
 }
 
+namespace {
+
+template <int QT, bool BF16>
+int launch16(const DF16Args &a, size_t lds, dim3 grid, hipStream_t s) {
+  auto kern = k_dgrad_fewc16<QT, BF16>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            160 * 1024) != hipSuccess)
+      return SGH_EUNSUPPORTED;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
+template <bool BF16>
+int dgrad_fewc16_mfma(const sgh_conv_geom *g, const DFPlan &p, const uint16_t *dy, const float *W, uint16_t *dx,
+                      void *workspace, hipStream_t s) {
+  const int KA = (g->K + KC16 - 1) / KC16 * KC16;
+  uint16_t *aw = static_cast<uint16_t *>(workspace);   // (half the bytes of the fp32 table the workspace is sized for)
+  const int total = ND * ND * 16 * KA;
+  hipLaunchKernelGGL(k_dgrad_fewc16_weights<BF16>, dim3((total + 255) / 256), dim3(256), 0, s, W, aw, g->K, KA, g->C, g->R,
+                     g->S, g->pad_h, g->pad_w, p.dp0, p.dq0);
+  DF16Args a{};
+  a.dy = dy, a.aw = aw, a.dx = dx;
+  a.N = g->N, a.C = g->C, a.H = g->H, a.W = g->W, a.K = g->K, a.KA = KA, a.P = g->P, a.Q = g->Q;
+  a.dp0 = p.dp0, a.dq0 = p.dq0;
+  const dim3 grid((g->P + TI16 - 1) / TI16, g->N, 1);
+  const size_t lds = size_t(SR16) * (p.qt * 16 + 8) * KP16 * sizeof(uint16_t);
+  int rc = SGH_EUNSUPPORTED;
+  sgh_prof_start("conv_dgrad16/k_dgrad_fewc16", 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S, s);
+  switch (p.qt) {
+    case 1: rc = launch16<1, BF16>(a, lds, grid, s); break;
+    case 2: rc = launch16<2, BF16>(a, lds, grid, s); break;
+    case 3: rc = launch16<3, BF16>(a, lds, grid, s); break;
+    case 4: rc = launch16<4, BF16>(a, lds, grid, s); break;
+    case 5: rc = launch16<5, BF16>(a, lds, grid, s); break;
+    case 6: rc = launch16<6, BF16>(a, lds, grid, s); break;
+    case 7: rc = launch16<7, BF16>(a, lds, grid, s); break;
+    case 8: rc = launch16<8, BF16>(a, lds, grid, s); break;
+    default: break;
+  }
+  sgh_prof_stop(s);
+  return rc;
+}
+
+}  // namespace
+
 int sgh_dgrad_fewc_run16(const sgh_conv_geom *g, const uint16_t *dy, const float *W, uint16_t *dx, void *workspace,
                          size_t ws_bytes, bool bf16, hipStream_t s) {
+  {
+    // the 16-bit matrix instruction: K in whole chunks of 32, even Q (pixel pairs), offsets of the slab
+    const DFPlan p = plan(g);
+    if (p.ok && g->K % KC16 == 0 && g->Q % 2 == 0 && g->N <= 65535 && !sgh_env().dgrad_fewc16_off) {
+      if (!workspace || ws_bytes < sgh_dgrad_fewc_workspace_bytes(g)) return SGH_EWORKSPACE;
+      return bf16 ? dgrad_fewc16_mfma<true>(g, p, dy, W, dx, workspace, s)
+                  : dgrad_fewc16_mfma<false>(g, p, dy, W, dx, workspace, s);
+    }
+  }
   return bf16 ? dgrad_fewc_run<StBF16>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad16/k_dgrad_fewc")
               : dgrad_fewc_run<StF16>(g, dy, W, dx, workspace, ws_bytes, s, "conv_dgrad16/k_dgrad_fewc");
 }

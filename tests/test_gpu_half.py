@@ -301,6 +301,9 @@ def _grad16_cases(count, seed):
     (3, 64, 7, 7, 256, 1, 1, (1, 1), (0, 0)),       # odd plane: single-pixel gradient loads
     (2, 128, 28, 28, 256, 1, 1, (2, 2), (0, 0)),    # downsample
     (1, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3)),       # stem
+    (2, 3, 224, 224, 64, 7, 7, (2, 2), (3, 3)),     # stem at full image size: seven column tiles per class row
+    (2, 4, 40, 40, 96, 7, 7, (2, 2), (3, 3)),       # stem-like: four channels, three chunks of 32 gradient channels, a partial row band
+    (2, 1, 24, 24, 32, 5, 5, (2, 2), (2, 2)),       # stem-like: one channel, 5x5 (three offsets per dimension)
 ])
 def test_conv_gradients_16bit_matrix_kernels(singa, dev, kind, case):
     """dgrad / wgrad on the 16-bit MFMA kernels against the fp32 CPU oracle on the same stored

@@ -276,7 +276,7 @@ def test_conv_dgrad_is_deterministic(singa, dev, n, c, hw, k, stride):
 
 
 @pytest.mark.parametrize("shape", [
-    (64, 64, 56, 64, 3, 1, 1),     # BASELINE single-conv configuration
+    (64, 64, 56, 64, 3, 1, 1),     # the single-convolution benchmark configuration
     (64, 3, 224, 64, 7, 2, 3),     # ResNet stem: few-channel wgrad / direct dgrad kernels
     (64, 64, 56, 128, 3, 2, 1),    # stage transition: residue-class shared-tile dgrad, stride-2 slab wgrad
     (64, 256, 14, 512, 1, 2, 0),   # downsample: pointwise dgrad with dilating store
