@@ -680,6 +680,275 @@ __global__ __launch_bounds__(256) void k_relayout16_fwd(const uint16_t *W, uint1
   wt[i] = (ko < K && c < C) ? W[(size_t(ko) * C + c) * RS + (RS - 1 - tap)] : uint16_t(0);
 }
 
+// ------------------------------------------------------------------------------------------------
+// data gradient of 3x3 / stride 1 / padding 1 layers: gradient slab shared by the nine taps
+// ------------------------------------------------------------------------------------------------
+// The pixels of all images are laid on one line with ONE zero position behind every row and one
+// zero row behind every image: position g = (n * (H + 1) + h) * (W + 1) + w.  The neighbour (h + dr,
+// w + ds) of a pixel is then g + dr * (W + 1) + ds for every pixel, border or not -- what falls off
+// an image lands on a zero position -- so a tap is a constant shift of the whole tile.  A workgroup
+// takes MT consecutive positions x BMC channels.  Per 64 gradient channels it stages the positions
+// [m0 - W - 2, m0 + MT + W + 2) ONCE as a pixel-major slab in LDS and all nine taps read their B
+// fragments from it at their shift; only the 16 KB weight tile of a (tap, chunk) pair is streamed.
+// That is a ninth of the gradient loads of the tap-by-tap kernel above and 9 x 4 matrix steps per
+// slab instead of 4.
+//   Staging: a thread owns EV (8 or 4) consecutive pixels of the NCHW tensor and 8 consecutive k: it
+// loads the 8 rows with 16- (8-) byte loads, transposes the 8 x EV block in registers (v_perm_b32) and
+// writes one 16-byte octet per pixel to that pixel's slab row (planes are whole groups of EV pixels, so
+// a group never straddles two images; it may straddle two rows, where the slab row skips the zero
+// position).  Zero positions are written once, at the start.  (2-byte loads, one per element, kept the
+// vector memory path busy for 10 us per slab: 47 cycles per wavefront instruction.)
+//   Pipeline: the nine tap steps of a chunk are unrolled.  The loads of the next chunk's block are
+// issued in steps 0-3 and written in steps 7-8; the weight tile of step s + 2 is loaded in step s into
+// one of two register sets and written to LDS at the end of step s + 1 (a tile loaded and written within
+// one step left every wavefront waiting 500 ns for L2 at the end of the step).  Every load is issued
+// unconditionally (out-of-range ones through an offset beyond the buffer, which reads zero) so that the
+// waits can count loads instead of draining them.
+// 512 threads: two groups of four wavefronts tile the same outputs and take the first / second half of
+// the matrix steps of every weight tile (summed through LDS at the end, as above); a wavefront holds
+// TC x TP accumulator blocks (channels x positions).
+struct S16Args {
+  const uint16_t *dy, *wt;  // wt: [tap][CP][KP]
+  uint16_t *dx;
+  const uint16_t *bias;
+  int N, C, H, W, K, KP, CP, mtiles, ptiles;
+  int Wp, HpWp, SP;   // W + 1, (H + 1) * (W + 1), slab entries MT + 2 * Wp + 2
+  int G;              // positions in all: N * HpWp
+  unsigned dy_bytes, wt_bytes;
+};
+
+template <int EV> struct SlabVec;
+template <> struct SlabVec<8> {
+  typedef u32x4 type;
+  static __device__ __forceinline__ type load(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+  }
+};
+template <> struct SlabVec<4> {
+  typedef unsigned int type __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ type load(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(type, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+  }
+};
+
+// MULTI: more than one chunk of 64 gradient channels (two slab buffers; the next chunk's block in flight)
+template <int TC, int TP, int WC, int WP, int EV, bool MULTI, bool BF16>
+__global__ __launch_bounds__(NT) void k_dgrad16_slab(S16Args a) {
+  // SPLIT: two groups of four wavefronts share the outputs and split every tile's matrix steps; otherwise the
+  // eight wavefronts tile the outputs and each takes all four steps
+  constexpr bool SPLIT = WC * WP == 4;
+  constexpr int KS = SPLIT ? 2 : 4;
+  static_assert((WC * WP == 4 && TP % 2 == 0) || WC * WP == 8, "four wavefronts per group (each keeps half of the position blocks), or eight tiles");
+  constexpr int BMC = WC * TC * 32, MT = WP * TP * 32, WSLOTS = BMC * 8 / NT;
+  constexpr int NB = EV == 8 ? 1 : 2;   // blocks (8 k x EV pixels) per thread and chunk
+  typedef typename SlabVec<EV>::type ev_t;
+  extern __shared__ __align__(16) uint16_t lds16[];
+  const int SPR = a.SP + 1;   // slab rows: the entries and a sink for octets that belong to no entry
+  uint16_t *const slab0 = lds16, *const slab1 = slab0 + (MULTI ? SPR * PITCH : 0);
+  uint16_t *const wts0 = slab1 + SPR * PITCH, *const wts1 = wts0 + BMC * PITCH;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int half = SPLIT ? wave >> 2 : 0, w4 = SPLIT ? wave & 3 : wave, wc = w4 / WP, wp = w4 % WP, l32 = lane & 31, lh = lane >> 5;
+  // workgroup w runs on XCD w % 8: the channel tiles of one position tile share an XCD's L2
+  const int slot = int(blockIdx.x) >> 3, pt = (slot / a.mtiles) * 8 + (int(blockIdx.x) & 7);
+  if (pt >= a.ptiles) return;
+  const int c0 = (slot % a.mtiles) * BMC, m0 = pt * MT, HW = a.H * a.W;
+  const rsrc_t rdy = make_rsrc(a.dy, a.dy_bytes), rwt = make_rsrc(a.wt, a.wt_bytes);
+
+  // This thread's pixel group: number gi among the groups of EV pixels (in tensor order, all images on one
+  // line) from the one that holds the first pixel of the slab; its blocks are k octets ko[j] of a chunk.
+  const int g_lo = m0 - a.Wp - 1;
+  int voff = kOOB, row0 = a.SP, wrapat = EV, wrapinc = 0;
+  {
+    int n, h, w;
+    {
+      const int gs = g_lo > 0 ? g_lo : 0;
+      n = gs / a.HpWp;
+      const int rem = gs - n * a.HpWp;
+      h = rem / a.Wp, w = rem - h * a.Wp;
+      if (h == a.H) h = 0, w = 0, ++n;   // (a zero row: on to the next image)
+      else if (w == a.W) {               // (a zero position: on to the next row)
+        w = 0;
+        if (++h == a.H) h = 0, ++n;
+      }
+    }
+    const long f_lo = long(n) * HW + h * a.W + w;
+    const long f0 = (f_lo / EV + (NB == 1 ? lane : (t & 127))) * EV;
+    if (f0 < long(a.N) * HW) {
+      const int n0 = int(f0 / HW), pix = int(f0 - long(n0) * HW), h0 = pix / a.W, w0 = pix - h0 * a.W;
+      row0 = n0 * a.HpWp + h0 * a.Wp + w0 - g_lo;
+      wrapat = a.W - w0;
+      wrapinc = 1 + (h0 + 1 == a.H ? a.Wp : 0);
+      const int last = row0 + EV - 1 + (EV - 1 >= wrapat ? wrapinc : 0);
+      if (last >= 0 && row0 < a.SP) voff = (n0 * a.K * HW + pix) * 2;
+    }
+  }
+  int ko[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) ko[j] = NB == 1 ? wave : (t >> 7) + 4 * j;
+
+  ev_t blk[NB][8];       // the block(s) in flight: row kk = EV pixels of gradient channel 8 * ko + kk
+  u32x4 ra[2][WSLOTS];   // two weight tiles in flight
+  const int oct = t & 7, rb = t >> 3;
+  const int woff = ((c0 + rb) * a.KP + oct * 8) * 2;
+  const int nkc = a.KP / KC, nsteps = 9 * nkc;
+
+  auto load_rows = [&](int kc, int kk0, int count) {   // rows kk0 .. kk0 + count - 1 of the blocks of chunk kc
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int kb = kc * KC + ko[j] * 8;
+      const int vo = kc < nkc && kb < a.K ? voff : kOOB;   // (K is a multiple of 8)
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk)
+        if (kk >= kk0 && kk < kk0 + count) blk[j][kk] = SlabVec<EV>::load(rdy, vo, (kb + kk) * HW * 2);
+    }
+  };
+  auto stage_pixels = [&](uint16_t *slab, int p0, int count) {   // pixels p0 .. p0 + count - 1 of the blocks
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int p = 0; p < EV; ++p)
+        if (p >= p0 && p < p0 + count) {
+          u32x4 v;
+#pragma unroll
+          for (int d = 0; d < 4; ++d)
+            v[d] = __builtin_amdgcn_perm(blk[j][2 * d + 1][p >> 1], blk[j][2 * d][p >> 1], (p & 1) ? kSelHi : kSelLo);
+          int row = row0 + p + (p >= wrapat ? wrapinc : 0);
+          row = unsigned(row) < unsigned(a.SP) ? row : a.SP;
+          *reinterpret_cast<u32x4 *>(slab + row * PITCH + ko[j] * 8) = v;
+        }
+  };
+  auto load_w = [&](int step, u32x4 (&r)[WSLOTS]) {
+    const int kc = step / 9, tap = step - 9 * kc;
+    const int wso = (tap * a.CP * a.KP + kc * KC) * 2;
+    const int vo = step < nsteps ? woff : kOOB;
+#pragma unroll
+    for (int i = 0; i < WSLOTS; ++i)
+      r[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rwt, vo + 64 * i * a.KP * 2, wso, 0));
+  };
+  auto stage_w = [&](uint16_t *wts, const u32x4 (&r)[WSLOTS]) {
+#pragma unroll
+    for (int i = 0; i < WSLOTS; ++i) *reinterpret_cast<u32x4 *>(wts + (rb + 64 * i) * PITCH + oct * 8) = r[i];
+  };
+
+  // prologue: the first chunk's block and the first two weight tiles on their way, the slabs zeroed meanwhile
+  load_rows(0, 0, 8);
+  load_w(0, ra[0]);
+  load_w(1, ra[1]);
+  {
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    const int n16 = (MULTI ? 2 : 1) * SPR * PITCH / 8;
+    for (int i = t; i < n16; i += NT) reinterpret_cast<u32x4 *>(slab0)[i] = z;
+  }
+  f32x16 acc[TC][TP];
+#pragma unroll
+  for (int i = 0; i < TC; ++i)
+#pragma unroll
+    for (int j = 0; j < TP; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  __syncthreads();
+  stage_pixels(slab0, 0, EV);
+  stage_w(wts0, ra[0]);
+  __syncthreads();
+
+  const int arow = (wc * TC * 32 + l32) * PITCH + half * 32 + lh * 8;
+  const int brow = (wp * TP * 32 + l32 + a.Wp + 1) * PITCH + half * 32 + lh * 8;
+  // step = 9 * kc + tap; PAR = step & 1 names the weight tile buffer in LDS that the step reads and the
+  // register set that it loads
+  auto step = [&](int kc, auto tapc, auto parc) {
+    constexpr int TAP = decltype(tapc)::value, PAR = decltype(parc)::value, R_ = TAP / 3, S_ = TAP % 3;
+    const uint16_t *const slab = (MULTI && (kc & 1)) ? slab1 : slab0;
+    uint16_t *const slab_next = (MULTI && (kc & 1)) ? slab0 : slab1;
+    load_w(9 * kc + TAP + 2, ra[PAR]);
+    if (MULTI && TAP < 4) load_rows(kc + 1, 2 * TAP, 2);
+    const uint16_t *As = (PAR ? wts1 : wts0) + arow;
+    const uint16_t *Bs = slab + brow + ((1 - R_) * a.Wp + (1 - S_)) * PITCH;
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+      u32x4 av[TC], bv[TP];
+#pragma unroll
+      for (int i = 0; i < TC; ++i) av[i] = *reinterpret_cast<const u32x4 *>(As + i * 32 * PITCH + 16 * j);
+#pragma unroll
+      for (int i = 0; i < TP; ++i) bv[i] = *reinterpret_cast<const u32x4 *>(Bs + i * 32 * PITCH + 16 * j);
+#pragma unroll
+      for (int i = 0; i < TC; ++i)
+#pragma unroll
+        for (int jp = 0; jp < TP; ++jp) acc[i][jp] = mfma<BF16>(av[i], bv[jp], acc[i][jp]);
+    }
+    stage_w(PAR ? wts0 : wts1, ra[PAR ^ 1]);   // the tile of step + 1, loaded during step - 1
+    if (MULTI && TAP == 7) stage_pixels(slab_next, 0, EV / 2);
+    if (MULTI && TAP == 8) stage_pixels(slab_next, EV / 2, EV / 2);
+    __syncthreads();
+  };
+  auto chunk = [&](int kc, auto parc) {
+    constexpr int P = decltype(parc)::value;
+    typedef std::integral_constant<int, P> P0;
+    typedef std::integral_constant<int, P ^ 1> P1;
+    step(kc, std::integral_constant<int, 0>{}, P0{});
+    step(kc, std::integral_constant<int, 1>{}, P1{});
+    step(kc, std::integral_constant<int, 2>{}, P0{});
+    step(kc, std::integral_constant<int, 3>{}, P1{});
+    step(kc, std::integral_constant<int, 4>{}, P0{});
+    step(kc, std::integral_constant<int, 5>{}, P1{});
+    step(kc, std::integral_constant<int, 6>{}, P0{});
+    step(kc, std::integral_constant<int, 7>{}, P1{});
+    step(kc, std::integral_constant<int, 8>{}, P0{});
+  };
+  for (int kc = 0; kc < nkc; kc += 2) {
+    chunk(kc, std::integral_constant<int, 0>{});
+    if (!MULTI || kc + 1 >= nkc) break;
+    chunk(kc + 1, std::integral_constant<int, 1>{});
+  }
+
+  // SPLIT: the two groups' sums meet in LDS, one channel block at a time: a wavefront hands over the position
+  // blocks of the other group's half and adds what its partner hands over to the blocks it keeps.
+  constexpr int TH = SPLIT ? TP / 2 : TP;
+  if constexpr (SPLIT) {
+    float *const xl = reinterpret_cast<float *>(lds16);
+    float *send = xl + ((half * 4 + w4) * (TH * 16)) * 64 + lane;
+    const float *recv = xl + (((half ^ 1) * 4 + w4) * (TH * 16)) * 64 + lane;
+#pragma unroll
+    for (int i = 0; i < TC; ++i) {
+      if (i) __syncthreads();
+#pragma unroll
+      for (int j = 0; j < TH; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) send[(j * 16 + v) * 64] = half ? acc[i][j][v] : acc[i][TH + j][v];
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < TH; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          if (half) acc[i][TH + j][v] += recv[(j * 16 + v) * 64];
+          else acc[i][j][v] += recv[(j * 16 + v) * 64];
+        }
+    }
+  }
+  // store: a lane owns one position per kept block, 16 channels per accumulator.  (Measured against this: the tile
+  // taken through LDS as [channel][pixel in tensor order] and written in 16-byte groups, with and without
+  // non-temporal stores -- 3 to 10 us slower per layer; the workgroups of a round reach their stores together
+  // and the burst is bound by the write path either way.)
+#pragma unroll
+  for (int j = 0; j < TH; ++j) {
+    const int g = m0 + (wp * TP + half * TH + j) * 32 + l32;
+    if (g >= a.G) continue;
+    const int n = g / a.HpWp, rem = g - n * a.HpWp, h = rem / a.Wp, w = rem - h * a.Wp;
+    if (h >= a.H || w >= a.W) continue;
+    uint16_t *o = a.dx + (size_t(n) * a.C) * HW + h * a.W + w;
+#pragma unroll
+    for (int i = 0; i < TC; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int c = c0 + (wc * TC + i) * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+        if (c < a.C) {
+          float r = (SPLIT && half) ? acc[i][TP - TH + j][v] : acc[i][j][v];
+          if (a.bias) r += BF16 ? sgh_bf16_to_f32(a.bias[c]) : sgh_f16_to_f32(a.bias[c]);
+          o[size_t(c) * HW] = round16<BF16>(r);
+        }
+      }
+  }
+}
+
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
 constexpr size_t kLutBytes = 81 * 16;  // wgrad: octet mask table behind the tiles
@@ -747,6 +1016,9 @@ struct D16Plan {
   int cls_tile0[5];
   size_t wt_bytes, dyT_bytes;   // workspace: re-laid weights, then the pixel-major copy
   int fs;             // see D16Args::fs
+  int slab;           // k_dgrad16_slab: 0 no, else the tile: 1 = 64 channels x 256 positions, 2 = 128 x 256, 3 = 128 x 128
+  int slab_sp;        // slab entries
+  int slab_ev;        // pixels per staging group: 8 or 4
   bool dilate;        // 1x1, stride 2, no padding, even image: see D16Args::dilate
   sgh_conv_geom kg;   // the geometry the kernel sees (the stride-1 problem on the P x Q grid when `dilate`)
 };
@@ -776,6 +1048,31 @@ D16Plan dplan(const sgh_conv_geom *real, int fs = 1) {
     tiles += (long(g->N) * Hc * Wc + BN - 1) / BN;
   }
   for (int cls = st * st; cls < 5; ++cls) p.cls_tile0[cls] = int(tiles);
+  // 3x3 / stride 1 / padding 1 on planes of whole 4- or 8-pixel groups: the slab kernel, when its slab fits beside
+  // the weight tiles in the 160 KB of LDS and a thread per pixel group (two per group of 4) covers it
+  if (fs == 1 && g->R == 3 && g->S == 3 && st == 1 && g->pad_h == 1 && g->pad_w == 1 && !sgh_env().slab16_off &&
+      (g->H * g->W) % 4 == 0 && g->W >= 8) {
+    const long G = long(g->N) * (g->H + 1) * (g->W + 1);
+    const int ev = (g->H * g->W) % 8 == 0 ? 8 : 4;
+    const int bmc = g->C <= 64 ? 64 : 128, mt_c = (g->C + bmc - 1) / bmc;
+    const int KP = (g->K + KC - 1) / KC * KC;
+    int mt = 256;
+    if (bmc == 128 && ((G + 255) / 256) * mt_c < sgh_num_cus() * 3 / 4) mt = 128;
+    for (; mt >= (bmc == 128 ? 128 : 256); mt /= 2) {
+      const int sp = mt + 2 * (g->W + 1) + 2;
+      const size_t lds = (size_t(KP > KC ? 2 : 1) * (sp + 1) + 2 * bmc) * PITCH * 2;
+      if (G + 1024 >= (long(1) << 31) || sp / ev + 3 > (ev == 8 ? 64 : 128) || lds > size_t(160) * 1024) continue;
+      p.slab = bmc == 64 ? 1 : (mt == 256 ? 2 : 3);
+      p.slab_sp = sp, p.slab_ev = ev;
+      p.bm = bmc, p.mtiles = mt_c, p.CP = mt_c * bmc, p.KP = KP;
+      p.tiles = int((G + mt - 1) / mt);
+      p.pixk = false;
+      p.wt_bytes = align256(size_t(9) * p.CP * p.KP * sizeof(uint16_t));
+      p.dyT_bytes = 0;
+      p.ok = true;
+      return p;
+    }
+  }
   // 64-row channel tiles when 128-row ones would leave CUs without a workgroup
   p.bm = (g->C <= 64 || tiles * ((g->C + 127) / 128) < sgh_num_cus() * 5 / 4) ? 64 : 128;
   p.mtiles = (g->C + p.bm - 1) / p.bm;
@@ -817,6 +1114,31 @@ int launch_d(const D16Args &a, const D16Plan &p, hipStream_t s) {
   }
   hipLaunchKernelGGL(kern, dim3(unsigned((p.tiles + 7) / 8) * 8u * unsigned(p.mtiles)), dim3(NT), lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
+template <int TC, int TP, int WC, int WP, int EV, bool MULTI, bool BF16>
+int launch_slab2(const S16Args &a, const D16Plan &p, hipStream_t s) {
+  auto kern = k_dgrad16_slab<TC, TP, WC, WP, EV, MULTI, BF16>;
+  constexpr int BMC = WC * TC * 32;
+  const size_t lds = (size_t(MULTI ? 2 : 1) * (p.slab_sp + 1) + 2 * BMC) * PITCH * 2;
+  static size_t allowed = 0;
+  if (lds > allowed) {
+    if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
+    allowed = lds;
+  }
+  hipLaunchKernelGGL(kern, dim3(unsigned((p.tiles + 7) / 8) * 8u * unsigned(p.mtiles)), dim3(NT), lds, s, a);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+}
+
+template <int TC, int TP, int WC, int WP>
+int launch_slab(const S16Args &a, const D16Plan &p, bool bf16, hipStream_t s) {
+  const bool multi = a.KP > KC;
+  if (p.slab_ev == 8) {
+    if (multi) return bf16 ? launch_slab2<TC, TP, WC, WP, 8, true, true>(a, p, s) : launch_slab2<TC, TP, WC, WP, 8, true, false>(a, p, s);
+    return bf16 ? launch_slab2<TC, TP, WC, WP, 8, false, true>(a, p, s) : launch_slab2<TC, TP, WC, WP, 8, false, false>(a, p, s);
+  }
+  if (multi) return bf16 ? launch_slab2<TC, TP, WC, WP, 4, true, true>(a, p, s) : launch_slab2<TC, TP, WC, WP, 4, true, false>(a, p, s);
+  return bf16 ? launch_slab2<TC, TP, WC, WP, 4, false, true>(a, p, s) : launch_slab2<TC, TP, WC, WP, 4, false, false>(a, p, s);
 }
 
 // A stride-1 forward convolution is the data gradient of the convolution with the channel roles
@@ -924,6 +1246,22 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
     hipLaunchKernelGGL(k_relayout16, dim3(unsigned((nw + 255) / 256)), dim3(256), 0, s, W, wt, g->K, g->C, RS, p.KP,
                        p.CP);
   if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
+  if (p.slab) {
+    S16Args b{};
+    b.dy = dy, b.wt = wt, b.dx = dx, b.bias = bias;
+    b.N = g->N, b.C = g->C, b.H = g->H, b.W = g->W, b.K = g->K, b.KP = p.KP, b.CP = p.CP;
+    b.mtiles = p.mtiles, b.ptiles = p.tiles;
+    b.Wp = g->W + 1, b.HpWp = (g->H + 1) * (g->W + 1), b.SP = p.slab_sp, b.G = g->N * b.HpWp;
+    b.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2), b.wt_bytes = unsigned(nw * 2);
+    const double fl = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * 9;
+    sgh_prof_start(fwd_of ? "conv_fwd16/k_dgrad16_slab" : "conv_dgrad16/k_dgrad16_slab", fl, s);
+    int rc;
+    if (p.slab == 1) rc = launch_slab<2, 2, 1, 4>(b, p, bf16, s);
+    else if (p.slab == 2) rc = launch_slab<2, 2, 2, 4>(b, p, bf16, s);
+    else rc = launch_slab<2, 2, 2, 2>(b, p, bf16, s);
+    sgh_prof_stop(s);
+    return rc;
+  }
   D16Args a{};
   a.dy = dy, a.dyT = dyT, a.wt = wt, a.dx = dx, a.bias = bias;
   const sgh_conv_geom *kg = &p.kg;

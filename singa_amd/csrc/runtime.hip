@@ -85,6 +85,7 @@ const sgh_env_switches &sgh_env() {
     s.dgrad_pointwise_off = on("SGH_DGRAD_POINTWISE_OFF"), s.conv16_off = on("SGH_CONV16_OFF");
     s.bn_onchip_off = on("SGH_BN_ONCHIP_OFF"), s.pw_dgrad_off = on("SGH_PW_DGRAD_OFF");
     s.pw_wgrad_off = on("SGH_PW_WGRAD_OFF"), s.dgrad_fewc16_off = on("SGH_DGRAD_FEWC16_OFF");
+    s.slab16_off = on("SGH_SLAB16_OFF");
     s.dgrad_tile = num("SGH_DGRAD_TILE", 0, 3), s.wgrad_tile = num("SGH_WGRAD_TILE", 0, 5);
     s.pw_tile = num("SGH_PW_TILE", 1, 2);
     const char *bm = getenv("SGH_DGRAD3X3_BM");

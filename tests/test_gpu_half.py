@@ -304,6 +304,13 @@ def _grad16_cases(count, seed):
     (2, 3, 224, 224, 64, 7, 7, (2, 2), (3, 3)),     # stem at full image size: seven column tiles per class row
     (2, 4, 40, 40, 96, 7, 7, (2, 2), (3, 3)),       # stem-like: four channels, three chunks of 32 gradient channels, a partial row band
     (2, 1, 24, 24, 32, 5, 5, (2, 2), (2, 2)),       # stem-like: one channel, 5x5 (three offsets per dimension)
+    # 3x3 / stride 1 / padding 1 on the slab kernel (gradient slab shared by the nine taps):
+    (3, 136, 12, 8, 136, 3, 3, (1, 1), (1, 1)),     # three chunks of gradient channels (the last partial), two channel tiles, 8-pixel groups
+    (9, 256, 14, 14, 256, 3, 3, (1, 1), (1, 1)),    # planes of 196 pixels: 4-pixel groups, tiles that span images
+    (5, 40, 30, 32, 72, 3, 3, (1, 1), (1, 1)),      # rows longer than a pixel group, two chunks, channel tile mostly empty
+    (40, 128, 28, 28, 72, 3, 3, (1, 1), (1, 1)),    # many tiles of 256 positions across 40 images
+    (2, 64, 10, 10, 64, 3, 3, (1, 1), (1, 1)),      # one chunk: the single-slab variant, groups of 4
+    (1, 65, 16, 56, 64, 3, 3, (1, 1), (1, 1)),      # widest rows of the residual networks, 65 channels
 ])
 def test_conv_gradients_16bit_matrix_kernels(singa, dev, kind, case):
     """dgrad / wgrad on the 16-bit MFMA kernels against the fp32 CPU oracle on the same stored
