@@ -362,6 +362,7 @@ typedef struct sgh_conv_geom {
   int K, R, S;          /* weight [K, C, R, S]                    */
   int stride_h, stride_w, pad_h, pad_w;
   int P, Q;             /* output [N, K, P, Q]                    */
+  int groups;           /* 1, or the group count: weight [K, C / groups, R, S] (sgh_conv_geom_init_grouped) */
   /* Owned by the library (sgh_conv_geom_init zeroes them, callers never write them): the note
    * sgh_conv_dgrad_prepare_multi leaves for this layer's next data gradient -- which weight
    * tensor was re-laid, into which workspace, and the library's weight epoch at that moment. */
@@ -373,6 +374,15 @@ typedef struct sgh_conv_geom {
 } sgh_conv_geom;
 SGH_API int sgh_conv_geom_init(sgh_conv_geom *g, int N, int C, int H, int W, int K, int R, int S,
                                int stride_h, int stride_w, int pad_h, int pad_w);
+/* The handle of a grouped convolution (CudnnConvHandle's `groups` argument,
+ * src/model/operation/convolution.cc:446-461 and :486-495: cudnnSetConvolutionGroupCount, filter descriptor
+ * [K, C / groups, R, S]; python/singa/layer.py:668-718 and the depthwise layer of SeparableConv2d, :780-795).
+ * C and K must be multiples of `groups`.  Group i convolves input channels [i C/groups, (i+1) C/groups) with
+ * filters [i K/groups, (i+1) K/groups).  Every convolution entry point below takes such a geometry: each group
+ * runs as a dense convolution on slices gathered in the workspace (sgh_conv_workspace_bytes[_h] account for
+ * them); sgh_conv_dgrad_acc_f32 returns SGH_EUNSUPPORTED and sgh_conv_dgrad_prepare_multi skips it. */
+SGH_API int sgh_conv_geom_init_grouped(sgh_conv_geom *g, int N, int C, int H, int W, int K, int R, int S,
+                                       int stride_h, int stride_w, int pad_h, int pad_w, int groups);
 
 #define SGH_CONV_FWD 0
 #define SGH_CONV_DGRAD 1

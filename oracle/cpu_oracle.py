@@ -189,6 +189,31 @@ def conv_bwd(dy, x, Wt, stride, pad, want_dx=True, want_dw=True):
     return dx, dw
 
 
+def conv_fwd_grouped(x, Wt, b, stride, pad, groups):
+    """Grouped convolution as its definition: group i convolves input channels [i C/G, (i+1) C/G) with filters
+    [i K/G, (i+1) K/G) of the [K, C/G, R, S] weight tensor (the reference runs it through
+    cudnnSetConvolutionGroupCount, src/model/operation/convolution.cc:486-490, and has no CPU path for it:
+    python/singa/layer.py:668-669).  Each group is one call of the dense convolution above."""
+    x = np.asarray(x, np.float32)
+    Wt = np.asarray(Wt, np.float32)
+    Cg, Kg = x.shape[1] // groups, Wt.shape[0] // groups
+    assert Cg * groups == x.shape[1] and Kg * groups == Wt.shape[0] and Wt.shape[1] == Cg
+    return np.concatenate([conv_fwd(x[:, i * Cg:(i + 1) * Cg], Wt[i * Kg:(i + 1) * Kg],
+                                    None if b is None else b[i * Kg:(i + 1) * Kg], stride, pad)
+                           for i in range(groups)], axis=1)
+
+
+def conv_bwd_grouped(dy, x, Wt, stride, pad, groups):
+    """(dx, dW) of the grouped convolution: the dense gradients of each group on its channel slices."""
+    dy = np.asarray(dy, np.float32)
+    x = np.asarray(x, np.float32)
+    Wt = np.asarray(Wt, np.float32)
+    Cg, Kg = x.shape[1] // groups, Wt.shape[0] // groups
+    parts = [conv_bwd(dy[:, i * Kg:(i + 1) * Kg], x[:, i * Cg:(i + 1) * Cg], Wt[i * Kg:(i + 1) * Kg], stride, pad)
+             for i in range(groups)]
+    return np.concatenate([p[0] for p in parts], axis=1), np.concatenate([p[1] for p in parts], axis=0)
+
+
 def conv_bgrad(dy):
     dy, pdy = _f(dy)
     N, K = dy.shape[:2]

@@ -18,7 +18,7 @@ sz = C.c_size_t
 class ConvGeom(C.Structure):
     """``sgh_conv_geom``"""
     _fields_ = [(n, C.c_int) for n in
-                ("N", "C", "H", "W", "K", "R", "S", "stride_h", "stride_w", "pad_h", "pad_w", "P", "Q",
+                ("N", "C", "H", "W", "K", "R", "S", "stride_h", "stride_w", "pad_h", "pad_w", "P", "Q", "groups",
                  "prelaid_dtype")] + [("prelaid_W", C.c_void_p), ("prelaid_ws", C.c_void_p),
                                       ("prelaid_ws_bytes", C.c_size_t), ("prelaid_epoch", C.c_ulonglong)]
 
@@ -138,6 +138,7 @@ SIGNATURES = {
     "sgh_sum_rows_f32": (C.c_int, [vp, vp, C.c_int, C.c_int, vp]),
     "sgh_add_row_f32": (C.c_int, [vp, vp, C.c_int, C.c_int, vp]),
     "sgh_conv_geom_init": (C.c_int, [C.POINTER(ConvGeom)] + [C.c_int] * 11),
+    "sgh_conv_geom_init_grouped": (C.c_int, [C.POINTER(ConvGeom)] + [C.c_int] * 12),
     "sgh_conv_workspace_bytes": (sz, [C.POINTER(ConvGeom), C.c_int]),
     "sgh_conv_dgrad_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_dgrad_acc_f32": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),

@@ -708,6 +708,7 @@ inline bool conv_ok(const sgh_conv_geom *g) {
     return false;
   if (g->P != (g->H + 2 * g->pad_h - g->R) / g->stride_h + 1) return false;
   if (g->Q != (g->W + 2 * g->pad_w - g->S) / g->stride_w + 1) return false;
+  if (g->groups < 1 || g->C % g->groups != 0 || g->K % g->groups != 0) return false;
   if (g->pad_h > 16000 || g->pad_w > 16000 || g->R > 16000 || g->S > 16000) return false;
   // every tensor is addressed with 32-bit byte offsets inside the kernels
   const size_t lim = kMaxOperandBytes / sizeof(float);
@@ -875,6 +876,72 @@ inline bool fwd_as_dgrad(const sgh_conv_geom *g, sgh_conv_geom *gt) {
 
 }  // namespace
 
+// ---- grouped convolution (cudnnSetConvolutionGroupCount in the reference, src/model/operation/convolution.cc
+// :486-490): group i convolves input channels [i C/G, (i+1) C/G) with filters [i K/G, (i+1) K/G) of the
+// [K, C/G, R, S] weight tensor.  Each group runs as a dense convolution of its own: its channel slices are
+// gathered into dense tensors in the workspace (strided device-to-device copies, one row per image), the
+// ordinary entry point runs on the sub-geometry, and the result is scattered back; a group's weight gradient
+// is a dense block of dW and needs no copy.  Workspace: [x slice | y slice | workspace of the sub-geometry].
+namespace {
+
+struct GroupPlan {
+  sgh_conv_geom sg;          // one group's geometry
+  size_t xe, ye, we;         // elements of a group's x / y slice per image, and of its weights
+  size_t x_bytes, y_bytes;   // the gathered slices
+};
+
+GroupPlan group_plan(const sgh_conv_geom *g, size_t elem) {
+  GroupPlan p{};
+  p.sg = *g;
+  p.sg.C = g->C / g->groups, p.sg.K = g->K / g->groups, p.sg.groups = 1;
+  sgh_prelaid_clear(&p.sg);
+  p.xe = size_t(p.sg.C) * g->H * g->W, p.ye = size_t(p.sg.K) * g->P * g->Q;
+  p.we = size_t(p.sg.K) * p.sg.C * g->R * g->S;
+  p.x_bytes = align256(p.xe * g->N * elem), p.y_bytes = align256(p.ye * g->N * elem);
+  return p;
+}
+
+// `sub(sg, which, a, b, bias, out, workspace, ws_bytes)` runs one dense pass; T is the element type.
+template <typename T, typename Sub>
+int conv_grouped(const sgh_conv_geom *g, int which, const T *a, const T *b, const T *bias, T *out, void *workspace,
+                 size_t ws_bytes, size_t sub_ws, hipStream_t s, Sub sub) {
+  if (!conv_ok(g) || !a || !b || !out) return SGH_EINVAL;
+  GroupPlan p = group_plan(g, sizeof(T));
+  if (!workspace || ws_bytes < p.x_bytes + p.y_bytes + sub_ws) return SGH_EWORKSPACE;
+  char *w = static_cast<char *>(workspace);
+  T *xg = reinterpret_cast<T *>(w), *yg = reinterpret_cast<T *>(w + p.x_bytes);
+  void *inner = w + p.x_bytes + p.y_bytes;
+  const size_t xfull = size_t(g->C) * g->H * g->W, yfull = size_t(g->K) * g->P * g->Q;
+  auto gather = [&](T *dst, const T *src, size_t per, size_t full, int gi) {
+    return hipMemcpy2DAsync(dst, per * sizeof(T), src + gi * per, full * sizeof(T), per * sizeof(T), size_t(g->N),
+                            hipMemcpyDeviceToDevice, s);
+  };
+  auto scatter = [&](T *dst, const T *src, size_t per, size_t full, int gi) {
+    return hipMemcpy2DAsync(dst + gi * per, full * sizeof(T), src, per * sizeof(T), per * sizeof(T), size_t(g->N),
+                            hipMemcpyDeviceToDevice, s);
+  };
+  for (int gi = 0; gi < g->groups; ++gi) {
+    int rc;
+    if (which == SGH_CONV_FWD) {           // a = x, b = W, out = y
+      SGH_HIP_TRY(gather(xg, a, p.xe, xfull, gi));
+      rc = sub(&p.sg, which, xg, b + gi * p.we, bias ? bias + gi * p.sg.K : nullptr, yg, inner, sub_ws);
+      if (rc == SGH_OK) SGH_HIP_TRY(scatter(out, yg, p.ye, yfull, gi));
+    } else if (which == SGH_CONV_DGRAD) {  // a = dy, b = W, out = dx
+      SGH_HIP_TRY(gather(yg, a, p.ye, yfull, gi));
+      rc = sub(&p.sg, which, yg, b + gi * p.we, nullptr, xg, inner, sub_ws);
+      if (rc == SGH_OK) SGH_HIP_TRY(scatter(out, xg, p.xe, xfull, gi));
+    } else {                               // a = dy, b = x, out = dW
+      SGH_HIP_TRY(gather(yg, a, p.ye, yfull, gi));
+      SGH_HIP_TRY(gather(xg, b, p.xe, xfull, gi));
+      rc = sub(&p.sg, which, yg, xg, nullptr, out + gi * p.we, inner, sub_ws);
+    }
+    if (rc != SGH_OK) return rc;
+  }
+  return SGH_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 int sgh_conv_geom_init(sgh_conv_geom *g, int N, int C, int H, int W, int K, int R, int S, int stride_h, int stride_w,
@@ -898,12 +965,49 @@ int sgh_conv_geom_init(sgh_conv_geom *g, int N, int C, int H, int W, int K, int 
   // ConvHandle's integer division (reference: src/model/operation/convolution.cc:56-59)
   g->P = (H + 2 * pad_h - R) / stride_h + 1;
   g->Q = (W + 2 * pad_w - S) / stride_w + 1;
+  g->groups = 1;
   sgh_prelaid_clear(g);
   return conv_ok(g) ? SGH_OK : SGH_EINVAL;
 }
 
+int sgh_conv_geom_init_grouped(sgh_conv_geom *g, int N, int C, int H, int W, int K, int R, int S, int stride_h,
+                               int stride_w, int pad_h, int pad_w, int groups) {
+  if (groups < 1 || C <= 0 || K <= 0 || C % groups != 0 || K % groups != 0) return SGH_EINVAL;
+  const int rc = sgh_conv_geom_init(g, N, C, H, W, K, R, S, stride_h, stride_w, pad_h, pad_w);
+  if (rc != SGH_OK) return rc;
+  g->groups = groups;
+  return SGH_OK;
+}
+
+namespace {
+
+int conv_dense_f32(sgh_conv_geom *sg, int which, const float *a, const float *b, const float *bias, float *out,
+                   void *ws, size_t ws_bytes, void *stream) {
+  if (which == SGH_CONV_FWD) return sgh_conv_fwd_f32(sg, a, b, bias, out, ws, ws_bytes, stream);
+  if (which == SGH_CONV_DGRAD) return sgh_conv_dgrad_f32(sg, a, b, out, ws, ws_bytes, stream);
+  return sgh_conv_wgrad_f32(sg, a, b, out, ws, ws_bytes, stream);
+}
+
+int conv_grouped_f32(const sgh_conv_geom *g, int which, const float *a, const float *b, const float *bias, float *out,
+                     void *workspace, size_t ws_bytes, void *stream) {
+  GroupPlan p = group_plan(g, sizeof(float));
+  const size_t sub_ws = sgh_conv_workspace_bytes(&p.sg, which);
+  return conv_grouped<float>(g, which, a, b, bias, out, workspace, ws_bytes, sub_ws, sgh_stream_of(stream),
+                             [&](sgh_conv_geom *sg, int wh, const float *a_, const float *b_, const float *bias_,
+                                 float *out_, void *ws, size_t wsb) {
+                               return conv_dense_f32(sg, wh, a_, b_, bias_, out_, ws, wsb, stream);
+                             });
+}
+
+}  // namespace
+
 size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
   if (!conv_ok(g)) return 0;
+  if (g->groups > 1) {
+    if (which < 0 || which > 2) return 0;
+    const GroupPlan p = group_plan(g, sizeof(float));
+    return p.x_bytes + p.y_bytes + sgh_conv_workspace_bytes(&p.sg, which);
+  }
   const size_t RS = size_t(g->R) * g->S;
   switch (which) {
     case SGH_CONV_FWD: {
@@ -1092,6 +1196,8 @@ static bool take_prelaid(sgh_conv_geom *g, int dtype, const void *W, const void 
 
 int sgh_conv_dgrad_f32(sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
                        size_t ws_bytes, void *stream) {
+  if (g && conv_ok(g) && g->groups > 1)
+    return conv_grouped_f32(g, SGH_CONV_DGRAD, dy, W, nullptr, dx, workspace, ws_bytes, stream);
   const bool prelaid = take_prelaid(g, 0, W, workspace);
   return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, false, prelaid);
 }
@@ -1207,6 +1313,7 @@ int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, 
     sgh_conv_geom *g = items[i].g;
     if (!g || !conv_ok(g) || !items[i].W) return SGH_EINVAL;
     sgh_prelaid_clear(g);
+    if (g->groups > 1) continue;   // (a grouped layer re-lays each group's weights when its data gradient runs)
     RelayoutTable::Item it{};
     it.W = items[i].W, it.Wt = items[i].workspace, it.K = g->K, it.C = g->C, it.RS = g->R * g->S;
     size_t need;
@@ -1239,7 +1346,7 @@ int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, 
 
 int sgh_conv_dgrad_acc_f32(sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
                            size_t ws_bytes, void *stream) {
-  if (g && conv_ok(g) && dgrad_path(g) != kDgradTile3x3) return SGH_EUNSUPPORTED;   // (the note stays for the fallback call)
+  if (g && conv_ok(g) && (g->groups > 1 || dgrad_path(g) != kDgradTile3x3)) return SGH_EUNSUPPORTED;   // (the note stays for the fallback call)
   const bool prelaid = take_prelaid(g, 0, W, workspace);
   return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, true, prelaid);
 }
@@ -1247,6 +1354,7 @@ int sgh_conv_dgrad_acc_f32(sgh_conv_geom *g, const float *dy, const float *W, fl
 int sgh_conv_fwd_f32(sgh_conv_geom *g, const float *x, const float *W, const float *bias, float *y,
                      void *workspace, size_t ws_bytes, void *stream) {
   if (!conv_ok(g) || !x || !W || !y) return SGH_EINVAL;
+  if (g->groups > 1) return conv_grouped_f32(g, SGH_CONV_FWD, x, W, bias, y, workspace, ws_bytes, stream);
   sgh_prelaid_clear_if_overlap(g, workspace, ws_bytes);
   const size_t need = sgh_conv_workspace_bytes(g, SGH_CONV_FWD);
   if (!workspace || ws_bytes < need) return SGH_EWORKSPACE;
@@ -1305,6 +1413,10 @@ static int bgrad_launch(const sgh_conv_geom *g, const float *dy, float *db, hipS
 static int conv_wgrad(sgh_conv_geom *g, const float *dy, const float *x, float *dW, float *db, void *workspace,
                       size_t ws_bytes, void *stream) {
   if (!conv_ok(g) || !dy || !x || !dW) return SGH_EINVAL;
+  if (g->groups > 1) {   // (the bias gradient does not depend on the grouping)
+    const int rc = conv_grouped_f32(g, SGH_CONV_WGRAD, dy, x, nullptr, dW, workspace, ws_bytes, stream);
+    return rc == SGH_OK && db ? bgrad_launch(g, dy, db, sgh_stream_of(stream)) : rc;
+  }
   sgh_prelaid_clear_if_overlap(g, workspace, ws_bytes);
   if (sgh_wgrad3x3_workspace_bytes(g)) {  // 3x3, stride 1 or 2: shared-input-tile kernel
     sgh_prof_start("conv_wgrad_op", conv_flops(g), sgh_stream_of(stream));
@@ -1450,6 +1562,15 @@ typedef int (*cast_out_fn)(const float *, uint16_t *, size_t, void *);
 int conv_half(sgh_conv_geom *g, int which, const uint16_t *a, const uint16_t *b, const uint16_t *bias,
               uint16_t *out, void *workspace, size_t ws_bytes, void *stream, cast_in_fn in, cast_out_fn outc) {
   if (!conv_ok(g) || !a || !b || !out) return SGH_EINVAL;
+  if (g->groups > 1) {
+    GroupPlan p = group_plan(g, sizeof(uint16_t));
+    const size_t sub_ws = sgh_conv_workspace_bytes_h(&p.sg, which);
+    return conv_grouped<uint16_t>(g, which, a, b, bias, out, workspace, ws_bytes, sub_ws, sgh_stream_of(stream),
+                                  [&](sgh_conv_geom *sg, int wh, const uint16_t *a_, const uint16_t *b_,
+                                      const uint16_t *bias_, uint16_t *out_, void *ws, size_t wsb) {
+                                    return conv_half(sg, wh, a_, b_, bias_, out_, ws, wsb, stream, in, outc);
+                                  });
+  }
   bool prelaid = false;
   if (which == SGH_CONV_DGRAD) prelaid = take_prelaid(g, in == sgh_cast_bf16_to_f32 ? 2 : 1, b, workspace);
   else sgh_prelaid_clear_if_overlap(g, workspace, ws_bytes);
@@ -1516,6 +1637,10 @@ int sgh_conv_bgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db
 
 size_t sgh_conv_workspace_bytes_h(const sgh_conv_geom *g, int which) {
   if (!conv_ok(g) || which < 0 || which > 2) return 0;
+  if (g->groups > 1) {
+    const GroupPlan p = group_plan(g, sizeof(uint16_t));
+    return p.x_bytes + p.y_bytes + sgh_conv_workspace_bytes_h(&p.sg, which);
+  }
   const size_t wide = half_plan(g, which).total() + (which == SGH_CONV_FWD ? align256(size_t(g->K) * 4) : 0);
   const size_t native = sgh_conv16_workspace_bytes(g, which);
   return wide > native ? wide : native;

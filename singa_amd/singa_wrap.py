@@ -727,8 +727,9 @@ class CudnnConvHandle(object):
 
     def __init__(self, x, kernel_size, stride, padding, in_channels, out_channels, bias, groups=1,
                  workspace_byte_limit=1024 * 1024 * 1024, prefer="fastest"):
-        if groups != 1:
-            raise SingaHipError("grouped convolution is not on the backward path built here")
+        groups = int(groups)
+        if groups < 1 or in_channels % groups != 0 or out_channels % groups != 0:
+            raise SingaHipError("channels and filters must be multiples of the group count")
         if x.nDim() != 4 or x.shape(1) != in_channels:
             raise SingaHipError("the number of input channels mismatched.")
         self.kernel_h, self.kernel_w = int(kernel_size[0]), int(kernel_size[1])
@@ -739,10 +740,11 @@ class CudnnConvHandle(object):
         self.bias_term = bool(bias)
         self.batchsize, _, self.height, self.width = x.shape()
         self.geom = _lib.ConvGeom()
-        check(_L().sgh_conv_geom_init(C.byref(self.geom), self.batchsize, self.channels, self.height,
-                                      self.width, self.num_filters, self.kernel_h, self.kernel_w,
-                                      self.stride_h, self.stride_w, self.pad_h, self.pad_w),
-              "sgh_conv_geom_init")
+        check(_L().sgh_conv_geom_init_grouped(C.byref(self.geom), self.batchsize, self.channels, self.height,
+                                              self.width, self.num_filters, self.kernel_h, self.kernel_w,
+                                              self.stride_h, self.stride_w, self.pad_h, self.pad_w, groups),
+              "sgh_conv_geom_init_grouped")
+        self.channels_per_filter = self.channels // groups   # (convolution.cc:461)
         self.conv_height, self.conv_width = self.geom.P, self.geom.Q
         self.col_height = self.channels * self.kernel_h * self.kernel_w
         self.col_width = self.conv_height * self.conv_width

@@ -50,6 +50,26 @@ def test_conv_geometry_follows_reference_integer_division():
     assert lib.sgh_conv_geom_init(None, 1, 3, 8, 8, 4, 3, 3, 1, 1, 0, 0) == -1
 
 
+def test_grouped_conv_geometry():
+    """sgh_conv_geom_init_grouped: channel and filter counts must be multiples of the group count; the workspace
+    of a grouped layer holds one group's slices of x and y next to the sub-geometry's own workspace."""
+    lib = _lib.lib()
+    g, d = _lib.ConvGeom(), _lib.ConvGeom()
+    assert lib.sgh_conv_geom_init(C.byref(d), 4, 16, 14, 14, 32, 3, 3, 1, 1, 1, 1) == 0 and d.groups == 1
+    assert lib.sgh_conv_geom_init_grouped(C.byref(g), 4, 64, 14, 14, 128, 3, 3, 1, 1, 1, 1, 4) == 0
+    assert (g.groups, g.C, g.K, g.P, g.Q) == (4, 64, 128, 14, 14)
+    for bad in (0, -1, 3, 5, 128):
+        assert lib.sgh_conv_geom_init_grouped(C.byref(g), 4, 64, 14, 14, 128, 3, 3, 1, 1, 1, 1, bad) == -1
+    assert lib.sgh_conv_geom_init_grouped(C.byref(g), 4, 64, 14, 14, 128, 3, 3, 1, 1, 1, 1, 4) == 0
+    for which in (_lib.SGH_CONV_FWD, _lib.SGH_CONV_DGRAD, _lib.SGH_CONV_WGRAD):
+        slices = 4 * 16 * 14 * 14 + 4 * 32 * 14 * 14
+        for fn, es in ((lib.sgh_conv_workspace_bytes, 4), (lib.sgh_conv_workspace_bytes_h, 2)):
+            got, sub = fn(C.byref(g), which), fn(C.byref(d), which)
+            assert slices * es + sub <= got <= slices * es + sub + 512
+    g.groups = 3     # a geometry whose fields were edited by hand is refused
+    assert lib.sgh_conv_workspace_bytes(C.byref(g), 0) == 0
+
+
 def test_workspace_sizes():
     lib = _lib.lib()
     g = _lib.ConvGeom()

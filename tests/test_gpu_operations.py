@@ -120,6 +120,52 @@ def test_conv_backward_vs_oracle(singa, dev, case):
     assert nl2(y, O.conv_fwd(x, w, b, stride, pad)) < TOL
 
 
+@pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", [
+    (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), 2, True),      # two groups of a shared-tile layer
+    (3, 32, 9, 11, 48, 3, 3, (2, 2), (1, 1), 4, False),      # stride 2, ragged image, 8 -> 12 channels per group
+    (2, 24, 12, 12, 24, 3, 3, (1, 1), (1, 1), 24, True),     # depthwise (the first half of SeparableConv2d)
+    (4, 16, 8, 8, 40, 1, 1, (1, 1), (0, 0), 8, False),       # pointwise, 2 -> 5 channels per group
+    (1, 6, 7, 5, 9, 5, 3, (2, 1), (2, 1), 3, True),          # generic path
+])
+def test_grouped_conv_vs_oracle(singa, dev, kind, case):
+    """Grouped convolution (CudnnConvHandle's `groups`): forward, data, weight and bias gradient against the
+    per-group oracle, fp32 at the reduction bar and on 16-bit tensors (stored values, 1e-2)."""
+    N, C, H, W, K, R, S, stride, pad, G, bias = case
+    r = rng(sum(case[:7]) + 31 * G)
+    dt = {"f32": singa.kFloat32, "f16": singa.kFloat16, "bf16": singa.kBFloat16}[kind]
+    tol = TOL if kind == "f32" else 1e-2
+
+    def to(a):
+        t = singa.from_numpy(a.astype(np.float32), dev)
+        if kind != "f32":
+            t = t.AsType(dt)
+        return t, (t.AsType(singa.kFloat32) if kind != "f32" else t).to_numpy()
+    xt, x = to(randn(r, N, C, H, W))
+    wt, w = to(randn(r, K, C // G, R, S) * np.sqrt(2.0 * G / (C * R * S)))
+    bt, b = to(randn(r, K)) if bias else (None, None)
+    h = singa.CudnnConvHandle(xt, (R, S), stride, pad, C, K, bias, G)
+    assert h.group == G and h.channels_per_filter == C // G
+    y = singa.GpuConvForward(xt, wt, bt, h)
+    y_o = O.conv_fwd_grouped(x, w, b, stride, pad, G)
+    assert y.shape() == list(y_o.shape) and nl2(y.to_numpy(), y_o) < tol
+    dyt, dy = to(randn(r, *y_o.shape))
+    dx_o, dw_o = O.conv_bwd_grouped(dy, x, w, stride, pad, G)
+    dx = singa.GpuConvBackwardx(dyt, wt, xt, h)
+    dw = singa.GpuConvBackwardW(dyt, xt, wt, h)
+    e = nl2(dx.to_numpy(), dx_o), nl2(dw.to_numpy(), dw_o)
+    print("grouped conv %s: dx %.2e dw %.2e" % (kind, e[0], e[1]))
+    assert dw.shape() == [K, C // G, R, S] and max(e) < tol
+    if bias:
+        assert nl2(singa.GpuConvBackwardb(dyt, bt, h).to_numpy(), O.conv_bgrad(dy)) < tol
+        if kind == "f32":
+            dW2, db2 = singa.GpuConvBackwardWb(dyt, xt, wt, bt, h)
+            assert_bit_equal(dW2.to_numpy(), dw.to_numpy(), "grouped dW with bias")
+            assert nl2(db2.to_numpy(), O.conv_bgrad(dy)) < tol
+    # the tensors outside the slices stay untouched: a second call gives the same bits
+    assert_bit_equal(singa.GpuConvBackwardx(dyt, wt, xt, h).to_numpy(), dx.to_numpy(), "grouped dx again")
+
+
 @pytest.mark.parametrize("case", [c for c in CONV_CASES if c[-1]] + [
     (4, 32, 16, 16, 64, 5, 5, (1, 1), (2, 2), True),      # generic kernel, split reduction: db rides along as a column of ones
     (1, 20, 6, 6, 40, 5, 5, (1, 1), (2, 2), True),        # ... without a split (one chunk range): written straight to db

@@ -63,6 +63,28 @@ def test_conv_against_brute_force_and_adjoints(case):
     np.testing.assert_allclose(O.conv_bgrad(dy), dy.astype(np.float64).sum(axis=(0, 2, 3)), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("case", [(2, 4, 6, 5, 6, 3, 3, (1, 1), (1, 1), 2), (3, 6, 7, 7, 6, 3, 3, (2, 2), (1, 1), 6),
+                                  (2, 8, 5, 6, 4, 1, 1, (1, 1), (0, 0), 4), (1, 6, 9, 8, 9, 5, 3, (2, 1), (2, 1), 3)])
+def test_grouped_conv_against_torch(case):
+    """The grouped convolution of the oracle (per-group calls of the dense functions) against an independent
+    implementation: torch's conv2d with `groups` in float64 and its autograd."""
+    import torch
+    N, C, H, W, K, R, S, stride, pad, G = case
+    r = np.random.default_rng(sum(case[:7]) + G)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = r.standard_normal((K, C // G, R, S)).astype(np.float32)
+    b = r.standard_normal(K).astype(np.float32)
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    tw = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    ty = torch.nn.functional.conv2d(tx, tw, torch.tensor(b, dtype=torch.float64), stride, pad, 1, G)
+    y = O.conv_fwd_grouped(x, w, b, stride, pad, G)
+    assert y.shape == tuple(ty.shape) and nl2(y, ty.detach().numpy()) < 1e-6
+    dy = r.standard_normal(y.shape).astype(np.float32)
+    ty.backward(torch.tensor(dy, dtype=torch.float64))
+    dx, dw = O.conv_bwd_grouped(dy, x, w, stride, pad, G)
+    assert nl2(dx, tx.grad.numpy()) < 1e-6 and nl2(dw, tw.grad.numpy()) < 1e-6
+
+
 def test_im2col_matches_definition():
     r = rng(3)
     im = randn(r, 2, 5, 4)
