@@ -441,10 +441,20 @@ __global__ __launch_bounds__(kResNT) void k_bn_bwd_resident(const typename S::el
 // channel's outputs become NaN.
 // x and dy are read once and dx written once: 3 tensor passes instead of 5.
 constexpr int kChipMaxG = 128, kChipSpinLimit = 1 << 20;
+#ifndef BN_CHIP_NL_ON
+#define BN_CHIP_NL_ON 1
+#endif
 // vectors per tensor and thread: 8 (64 registers of raw data), 5 for 16-byte vectors of 16-bit elements,
 // whose eight conversions per vector need more registers beside the data
 template <class S>
 constexpr int chip_nv() { return (sizeof(typename S::elem) == 2 && S::VEC == 8) ? 5 : 8; }
+// 16-byte vectors of 16-bit elements: four more vectors per tensor and thread wait in LDS, which the kernel does
+// not use otherwise (2 tensors x 4 x 512 threads x 16 bytes = 64 KB: still two workgroups per CU).  They are
+// loaded straight into LDS (buffer_load ... lds: no destination registers while in flight), every thread reads
+// back only what it loaded itself.  What a CU streams is (bytes resident) / (lifetime of a workgroup): the five
+// register vectors alone left these shapes at 3.2-4.0 TB/s against 4.3-4.7 for fp32 with its eight.
+template <class S>
+constexpr int chip_nl() { return BN_CHIP_NL_ON && sizeof(typename S::elem) == 2 && S::VEC == 8 ? 4 : 0; }
 
 struct ChipSlot {   // one per (channel, slice): {bits(a) : ticket low half}, {bits(b) : ticket high half}
   unsigned long long wa, wb;
@@ -454,21 +464,30 @@ inline size_t chip_workspace_bytes(int C, int G) { return size_t(C) * size_t(G) 
 struct ChipPlan {
   bool ok;
   int G, vpg, nt;   // slices per channel, vectors per slice, threads per workgroup
+  int nl;           // vectors per tensor and thread kept in LDS (0: registers only)
 };
 
 template <class S>
 inline ChipPlan chip_plan(int N, int C, int HW) {
-  ChipPlan p{false, 0, 0, 0};
+  ChipPlan p{false, 0, 0, 0, 0};
   if (HW % S::VEC != 0) return p;
   const long TV = long(N) * (HW / S::VEC);                       // vectors per channel
   // 512 threads (two workgroups per CU: one loads while the other waits or stores) unless that cuts the
   // channel into more slices than one wavefront can poll
   p.nt = 512;
-  long G = (TV + long(p.nt) * chip_nv<S>() - 1) / (long(p.nt) * chip_nv<S>());
+  // (the vectors in LDS only with 512 threads, and only for tensors up to 128 MB: measured at N = 128, fused with
+  // the ReLU gate, C64 56x56 47.5 -> 40.2 us, C128 28x28 23.9 -> 21.5, C512 28x28 83.9 -> 79.4, C128 56x56 83.7 ->
+  // 80.0, but the 205 MB tensors C256 56x56 153.8 -> 166.1 and C64 112x112 168.6 -> 174.8, with or without the
+  // non-temporal hint that the register loads carry)
+  const bool lds_ok = chip_nl<S>() > 0 && size_t(N) * C * HW * sizeof(typename S::elem) <= (size_t(128) << 20);
+  int per_thread = chip_nv<S>() + (lds_ok ? chip_nl<S>() : 0);
+  long G = (TV + long(p.nt) * per_thread - 1) / (long(p.nt) * per_thread);
   if (G > kChipMaxG) {
     p.nt = 1024;
-    G = (TV + long(p.nt) * chip_nv<S>() - 1) / (long(p.nt) * chip_nv<S>());
+    per_thread = chip_nv<S>();
+    G = (TV + long(p.nt) * per_thread - 1) / (long(p.nt) * per_thread);
   }
+  p.nl = p.nt == 512 && lds_ok ? chip_nl<S>() : 0;
   // few channels: thinner slices, so that there are two workgroups for every CU (at least one wavefront of vectors each)
   const long want = (2L * sgh_num_cus() + C - 1) / C;
   if (G < want) G = want;
@@ -485,7 +504,7 @@ inline ChipPlan chip_plan(int N, int C, int HW) {
   return p;
 }
 
-template <class S, bool RELU, int NT>
+template <class S, bool RELU, int NT, int NL = 0>
 __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem *__restrict__ dy,
                                                           const typename S::elem *__restrict__ x,
                                                           const float *__restrict__ gamma, const float *__restrict__ beta,
@@ -522,10 +541,32 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
   auto gate = [&](float d, float v) { return !RELU || S::stored_positive(bn_out(v, mean, invstd, gm, be)) ? d : 0.f; };
   const raw *xg = reinterpret_cast<const raw *>(x), *dg_ = reinterpret_cast<const raw *>(dy);
   raw xv[NV], dv[NV];
+  // vectors 0 .. NL-1 of a thread go to LDS: slot j of tensor z at ((z * NL + j) * NT + t) * 16 bytes.  A
+  // wavefront's instruction writes 64 consecutive slots (LDS address = wavefront-uniform base + 16 * lane).
+  extern __shared__ __align__(16) unsigned char chip_lds[];
+  if constexpr (NL > 0) {
+    typedef __amdgpu_buffer_rsrc_t rsrc_t;
+    const unsigned bytes = unsigned(size_t(s.N) * s.C * s.HW * sizeof(elem));
+    const rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(x), 0, int(bytes), 0x00020000);
+    const rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(dy), 0, int(bytes), 0x00020000);
+    const int wbase = __builtin_amdgcn_readfirstlane(t & ~63);
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+      const int iv = lo + j * NT + t;
+      int voff = int(0x80000000u);   // (beyond the buffer: the slot reads as zero and is never used)
+      if (iv < hi) {
+        const int n = iv / PV, r = iv - n * PV;
+        voff = int((unsigned(n) * unsigned(s.C) + unsigned(c)) * unsigned(PV) + unsigned(r)) * 16;
+      }
+      typedef unsigned char __attribute__((address_space(3))) * lds_ptr;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(chip_lds + size_t((0 * NL + j) * NT + wbase) * 16), 16, voff, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr)(chip_lds + size_t((1 * NL + j) * NT + wbase) * 16), 16, voff, 0, 0, 0);
+    }
+  }
   // every load of the slice is issued before the first value is used
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    const int iv = lo + i * NT + t;
+    const int iv = lo + (NL + i) * NT + t;
     if (iv < hi) {
       const int n = iv / PV, r = iv - n * PV;
       const size_t off = (size_t(n) * s.C + c) * PV + r;
@@ -534,24 +575,38 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     }
   }
   float a = 0.f, b = 0.f, b1 = 0.f;
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    if (lo + i * NT + t < hi) {
-      float v[V], d[V];
-      S::template load16<false>(reinterpret_cast<const elem *>(&xv[i]), v);
-      S::template load16<false>(reinterpret_cast<const elem *>(&dv[i]), d);
-#pragma unroll
-      for (int q = 0; q < V; q += 4) {
-        const float d0 = gate(d[q], v[q]), d1 = gate(d[q + 1], v[q + 1]), d2 = gate(d[q + 2], v[q + 2]),
-                    d3 = gate(d[q + 3], v[q + 3]);
-        a += (d0 + d1) + (d2 + d3);
-        b = __builtin_fmaf(d0, (v[q] - mean) * invstd, b);
-        b1 = __builtin_fmaf(d1, (v[q + 1] - mean) * invstd, b1);
-        b = __builtin_fmaf(d2, (v[q + 2] - mean) * invstd, b);
-        b1 = __builtin_fmaf(d3, (v[q + 3] - mean) * invstd, b1);
-      }
-    }
+  // (a macro, not a lambda: with the vectors passed to a lambda the register arrays went to scratch memory)
+#define BN_CHIP_ACCUMULATE(XR, DR)                                                                            \
+  {                                                                                                           \
+    float v[V], d[V];                                                                                         \
+    S::template load16<false>(reinterpret_cast<const elem *>(&(XR)), v);                                      \
+    S::template load16<false>(reinterpret_cast<const elem *>(&(DR)), d);                                      \
+    _Pragma("unroll") for (int q = 0; q < V; q += 4) {                                                        \
+      const float d0 = gate(d[q], v[q]), d1 = gate(d[q + 1], v[q + 1]), d2 = gate(d[q + 2], v[q + 2]),        \
+                  d3 = gate(d[q + 3], v[q + 3]);                                                              \
+      a += (d0 + d1) + (d2 + d3);                                                                             \
+      b = __builtin_fmaf(d0, (v[q] - mean) * invstd, b);                                                      \
+      b1 = __builtin_fmaf(d1, (v[q + 1] - mean) * invstd, b1);                                                \
+      b = __builtin_fmaf(d2, (v[q + 2] - mean) * invstd, b);                                                  \
+      b1 = __builtin_fmaf(d3, (v[q + 3] - mean) * invstd, b1);                                                \
+    }                                                                                                         \
   }
+  if constexpr (NL > 0) {
+    // the loads into LDS are the oldest: wait for everything (the compiler does not count them for LDS reads)
+    __builtin_amdgcn_s_waitcnt(0);
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int j = 0; j < NL; ++j)
+      if (lo + j * NT + t < hi) {
+        const raw xl = *reinterpret_cast<const raw *>(chip_lds + size_t((0 * NL + j) * NT + t) * 16);
+        const raw dl = *reinterpret_cast<const raw *>(chip_lds + size_t((1 * NL + j) * NT + t) * 16);
+        BN_CHIP_ACCUMULATE(xl, dl)
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+    if (lo + (NL + i) * NT + t < hi) BN_CHIP_ACCUMULATE(xv[i], dv[i])
+#undef BN_CHIP_ACCUMULATE
   b += b1;
   float db = sgh_block_sum(a, red), dg = sgh_block_sum(b, red);
   if (G > 1) {
@@ -601,21 +656,35 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
   const float rM = float(1.0 / (double(s.N) * s.HW));
   const float c0 = db * rM, c1 = dg * rM;
   raw *og = reinterpret_cast<raw *>(dx);
+#define BN_CHIP_FINISH(IV, XR, DR)                                                                            \
+  {                                                                                                           \
+    const int n = (IV) / PV, r = (IV) - n * PV;                                                               \
+    float v[V], d[V], o[V];                                                                                   \
+    S::template load16<false>(reinterpret_cast<const elem *>(&(XR)), v);                                      \
+    S::template load16<false>(reinterpret_cast<const elem *>(&(DR)), d);                                      \
+    _Pragma("unroll") for (int q = 0; q < V; ++q)                                                             \
+        o[q] = k * (gate(d[q], v[q]) - __builtin_fmaf((v[q] - mean) * invstd, c1, c0));                       \
+    raw ov;                                                                                                   \
+    S::store16(reinterpret_cast<elem *>(&ov), o);                                                             \
+    og[(size_t(n) * s.C + c) * PV + r] = ov;                                                                  \
+  }
+  if constexpr (NL > 0) {
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int iv = lo + i * NT + t;
-    if (iv < hi) {
-      const int n = iv / PV, r = iv - n * PV;
-      float v[V], d[V], o[V];
-      S::template load16<false>(reinterpret_cast<const elem *>(&xv[i]), v);
-      S::template load16<false>(reinterpret_cast<const elem *>(&dv[i]), d);
-#pragma unroll
-      for (int q = 0; q < V; ++q) o[q] = k * (gate(d[q], v[q]) - __builtin_fmaf((v[q] - mean) * invstd, c1, c0));
-      raw ov;
-      S::store16(reinterpret_cast<elem *>(&ov), o);
-      og[(size_t(n) * s.C + c) * PV + r] = ov;
+    for (int j = 0; j < NL; ++j) {
+      const int iv = lo + j * NT + t;
+      if (iv < hi) {
+        const raw xl = *reinterpret_cast<const raw *>(chip_lds + size_t((0 * NL + j) * NT + t) * 16);
+        const raw dl = *reinterpret_cast<const raw *>(chip_lds + size_t((1 * NL + j) * NT + t) * 16);
+        BN_CHIP_FINISH(iv, xl, dl)
+      }
     }
   }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int iv = lo + (NL + i) * NT + t;
+    if (iv < hi) BN_CHIP_FINISH(iv, xv[i], dv[i])
+  }
+#undef BN_CHIP_FINISH
 }
 
 // tickets: a random 64-bit start (so that whatever an uninitialised workspace holds is not the next
@@ -640,6 +709,23 @@ int launch_onchip(const typename S::elem *dy, const typename S::elem *x, const f
   const int xcd_runs = p.G <= 16 && s.C >= 8 ? 1 : 0;
   const dim3 grid(xcd_runs ? unsigned((s.C + 7) / 8) * 8u * p.G : unsigned(s.C) * p.G);
   const unsigned long long t1 = next_ticket(), t2 = next_ticket();
+  if constexpr (chip_nl<S>() > 0) {
+    if (p.nl > 0) {
+      constexpr int NL = chip_nl<S>();
+      auto kern = k_bn_bwd_onchip<S, RELU, 512, NL>;
+      constexpr int lds = 2 * NL * 512 * 16;
+      static bool attr = false;
+      if (!attr) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
+            hipSuccess)
+          return SGH_EUNSUPPORTED;
+        attr = true;
+      }
+      hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, ws,
+                         s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
+      return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+    }
+  }
   if (p.nt == 512)
     hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean, save_invstd,
                        dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
