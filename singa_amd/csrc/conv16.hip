@@ -692,7 +692,8 @@ __global__ __launch_bounds__(256) void k_relayout16_fwd(const uint16_t *W, uint1
 // fragments from it at their shift; only the 16 KB weight tile of a (tap, chunk) pair is streamed.
 // That is a ninth of the gradient loads of the tap-by-tap kernel above and 9 x 4 matrix steps per
 // slab instead of 4.
-//   Staging: a thread owns EV (8 or 4) consecutive pixels of the NCHW tensor and 8 consecutive k: it
+//   Staging: a thread owns EV (8 or 4) consecutive pixels of the NCHW tensor and 8 consecutive k (the lanes that
+// share a pixel group take different k octets): it
 // loads the 8 rows with 16- (8-) byte loads, transposes the 8 x EV block in registers (v_perm_b32) and
 // writes one 16-byte octet per pixel to that pixel's slab row (planes are whole groups of EV pixels, so
 // a group never straddles two images; it may straddle two rows, where the slab row skips the zero
@@ -741,6 +742,7 @@ __global__ __launch_bounds__(NT) void k_dgrad16_slab(S16Args a) {
   static_assert((WC * WP == 4 && TP % 2 == 0) || WC * WP == 8, "four wavefronts per group (each keeps half of the position blocks), or eight tiles");
   constexpr int BMC = WC * TC * 32, MT = WP * TP * 32, WSLOTS = BMC * 8 / NT;
   constexpr int NB = EV == 8 ? 1 : 2;   // blocks (8 k x EV pixels) per thread and chunk
+  constexpr int KOL = 8 / NB;           // lanes per pixel group
   typedef typename SlabVec<EV>::type ev_t;
   extern __shared__ __align__(16) uint16_t lds16[];
   const int SPR = a.SP + 1;   // slab rows: the entries and a sink for octets that belong to no entry
@@ -772,7 +774,7 @@ __global__ __launch_bounds__(NT) void k_dgrad16_slab(S16Args a) {
       }
     }
     const long f_lo = long(n) * HW + h * a.W + w;
-    const long f0 = (f_lo / EV + (NB == 1 ? lane : (t & 127))) * EV;
+    const long f0 = (f_lo / EV + wave * (8 * NB) + lane / KOL) * EV;
     if (f0 < long(a.N) * HW) {
       const int n0 = int(f0 / HW), pix = int(f0 - long(n0) * HW), h0 = pix / a.W, w0 = pix - h0 * a.W;
       row0 = n0 * a.HpWp + h0 * a.Wp + w0 - g_lo;
@@ -782,9 +784,12 @@ __global__ __launch_bounds__(NT) void k_dgrad16_slab(S16Args a) {
       if (last >= 0 && row0 < a.SP) voff = (n0 * a.K * HW + pix) * 2;
     }
   }
+  // k octets of this thread's blocks.  The KOL lanes that share a pixel group take different octets, so that a
+  // wavefront's LDS write covers whole slab rows (128 or 64 contiguous bytes per row, 4-way bank conflicts; with
+  // one octet per wavefront and a row per lane, rows EV apart fell on 2 of the 16 bank groups: 32-way).
   int ko[NB];
 #pragma unroll
-  for (int j = 0; j < NB; ++j) ko[j] = NB == 1 ? wave : (t >> 7) + 4 * j;
+  for (int j = 0; j < NB; ++j) ko[j] = lane % KOL + KOL * j;
 
   ev_t blk[NB][8];       // the block(s) in flight: row kk = EV pixels of gradient channel 8 * ko + kk
   u32x4 ra[2][WSLOTS];   // two weight tiles in flight
@@ -796,10 +801,10 @@ __global__ __launch_bounds__(NT) void k_dgrad16_slab(S16Args a) {
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
       const int kb = kc * KC + ko[j] * 8;
-      const int vo = kc < nkc && kb < a.K ? voff : kOOB;   // (K is a multiple of 8)
+      const int vo = (kc < nkc && kb < a.K ? voff : kOOB) + ko[j] * 8 * HW * 2;   // (K is a multiple of 8)
 #pragma unroll
       for (int kk = 0; kk < 8; ++kk)
-        if (kk >= kk0 && kk < kk0 + count) blk[j][kk] = SlabVec<EV>::load(rdy, vo, (kb + kk) * HW * 2);
+        if (kk >= kk0 && kk < kk0 + count) blk[j][kk] = SlabVec<EV>::load(rdy, vo, (kc * KC + kk) * HW * 2);
     }
   };
   auto stage_pixels = [&](uint16_t *slab, int p0, int count) {   // pixels p0 .. p0 + count - 1 of the blocks
