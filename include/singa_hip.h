@@ -471,6 +471,14 @@ SGH_API int sgh_conv_wgrad_f16(sgh_conv_geom *g, const uint16_t *dy, const uint1
                                uint16_t *dW, void *workspace, size_t ws_bytes, void *stream);
 SGH_API int sgh_conv_wgrad_bf16(sgh_conv_geom *g, const uint16_t *dy, const uint16_t *x,
                                 uint16_t *dW, void *workspace, size_t ws_bytes, void *stream);
+/* How sgh_conv_wgrad_{f16,bf16} split their reduction.  -1 (the default): by the stream of the call -- on a
+ * device's auxiliary stream (sgh_device_aux_stream) the launch shares the chip with the main stream's kernels
+ * and the split is planned for one workgroup per CU (half the fp32 partials to write and sum), elsewhere for
+ * two; 1: always the shared-chip plan, 0: never.  The plans sum the fp32 partials in different orders, so
+ * results of different plans differ in the last place of the 16-bit result; each plan is run-to-run
+ * identical.  Process-wide; meant for measurements and for comparing a two-stream tape bit by bit with a
+ * one-stream one.  No counterpart in the reference (cuDNN chooses its algorithms by itself). */
+SGH_API void sgh_conv_wgrad16_split_mode(int mode);
 SGH_API int sgh_conv_bgrad_f16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db, void *stream);
 SGH_API int sgh_conv_bgrad_bf16(const sgh_conv_geom *g, const uint16_t *dy, uint16_t *db, void *stream);
 SGH_API int sgh_conv_fwd_f16(sgh_conv_geom *g, const uint16_t *x, const uint16_t *W,

@@ -153,6 +153,7 @@ SIGNATURES = {
     "sgh_conv_dgrad_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_wgrad_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
     "sgh_conv_wgrad_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, sz, vp]),
+    "sgh_conv_wgrad16_split_mode": (None, [C.c_int]),
     "sgh_conv_bgrad_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp]),
     "sgh_conv_bgrad_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp]),
     "sgh_conv_fwd_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),

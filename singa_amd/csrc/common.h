@@ -41,6 +41,10 @@ const sgh_env_switches &sgh_env();
 // Number of compute units of the current device (cached per process; one GPU per process).
 int sgh_num_cus();
 
+// True when `s` is the auxiliary stream of an open device (sgh_device_aux_stream): work launched there runs
+// beside the main stream's kernels and shares the chip with them.
+bool sgh_stream_is_aux(hipStream_t s);
+
 // Looks up, for the current device, the address of the library-owned partial-sum buffer of
 // sgh_bn_bwd_noalloc_f32 (batchnorm.hip).  sgh_device_open calls it so that the entry point's first
 // call on a device finds the address ready; the entry point repeats the lookup if it was not.

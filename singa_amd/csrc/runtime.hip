@@ -15,6 +15,20 @@
 
 #include "common.h"
 
+// The auxiliary streams of all open devices: a kernel entry point that is handed one of them knows that its
+// launch shares the chip with the main stream's work (sgh_stream_is_aux).
+static std::mutex g_aux_mu;
+static std::vector<hipStream_t> g_aux_streams;
+
+bool sgh_stream_is_aux(hipStream_t s) {
+  if (!s) return false;
+  std::lock_guard<std::mutex> lock(g_aux_mu);
+  for (hipStream_t a : g_aux_streams)
+    if (a == s) return true;
+  return false;
+}
+
+
 struct sgh_device {
   int id = 0;
   hipStream_t stream = nullptr;
@@ -258,7 +272,17 @@ int sgh_device_close(sgh_device *dev) {
   for (auto &b : dev->pending) (void)hipFree(b.first);
   (void)hipStreamDestroy(dev->stream);
   (void)hipStreamDestroy(dev->side);
-  if (dev->aux) (void)hipStreamDestroy(dev->aux);
+  if (dev->aux) {
+    {
+      std::lock_guard<std::mutex> lock(g_aux_mu);
+      for (size_t i = 0; i < g_aux_streams.size(); ++i)
+        if (g_aux_streams[i] == dev->aux) {
+          g_aux_streams.erase(g_aux_streams.begin() + long(i));
+          break;
+        }
+    }
+    (void)hipStreamDestroy(dev->aux);
+  }
   if (dev->fork_ev) (void)hipEventDestroy(dev->fork_ev);
   if (dev->join_ev) (void)hipEventDestroy(dev->join_ev);
   for (hipEvent_t e : dev->upload_done)
@@ -277,6 +301,9 @@ void *sgh_device_aux_stream(sgh_device *dev) {
     if (hipStreamCreateWithFlags(&dev->aux, hipStreamNonBlocking) != hipSuccess) {   // (default priority)
       (void)hipGetLastError();
       dev->aux = nullptr;
+    } else {
+      std::lock_guard<std::mutex> lock(g_aux_mu);
+      g_aux_streams.push_back(dev->aux);
     }
   }
   return reinterpret_cast<void *>(dev->aux);
