@@ -226,6 +226,7 @@ def main():
     sync()
     prof = collect_prof(lib)
     lib.sgh_prof_enable(0)
+    lib.sgh_prof_clear()
     conv = {k: prof[k] for k in ("conv_dgrad", "conv_wgrad", "conv_dgrad16", "conv_wgrad16") if k in prof}
     flop = sum(v["work"] for v in conv.values())
     ms = sum(v["ms"] for v in conv.values())

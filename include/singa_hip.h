@@ -147,6 +147,9 @@ SGH_API int sgh_event_elapsed_ms(sgh_event *start, sgh_event *stop, float *ms);
  * a dense GEMM.  Records nest.  sgh_prof_enable(1) clears old records.
  * sgh_prof_get waits for record i to finish and returns its tag, duration and work. */
 SGH_API int sgh_prof_enable(int on);
+/* Drops the records taken so far and destroys their events (sgh_prof_enable(1) does the same before it starts;
+ * this is for a caller that has read what it wanted and does not profile again).  Profiling must be off. */
+SGH_API int sgh_prof_clear(void);
 SGH_API int sgh_prof_count(int *n);
 SGH_API int sgh_prof_get(int i, char *tag, size_t tag_len, float *ms, double *work);
 

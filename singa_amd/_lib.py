@@ -78,6 +78,7 @@ SIGNATURES = {
     "sgh_stream_wait_event": (C.c_int, [vp, vp]),
     "sgh_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
     "sgh_prof_enable": (C.c_int, [C.c_int]),
+    "sgh_prof_clear": (C.c_int, []),
     "sgh_prof_count": (C.c_int, [C.POINTER(C.c_int)]),
     "sgh_prof_get": (C.c_int, [C.c_int, C.c_char_p, sz, C.POINTER(C.c_float), C.POINTER(C.c_double)]),
     "sgh_relu_bwd_f32": (C.c_int, [vp, vp, vp, sz, vp]),

@@ -549,6 +549,12 @@ int sgh_prof_enable(int on) {
   return SGH_OK;
 }
 
+int sgh_prof_clear(void) {
+  if (g_prof_on) return SGH_EINVAL;   // (records are still being taken)
+  prof_clear();
+  return SGH_OK;
+}
+
 int sgh_prof_count(int *n) {
   if (!n) return SGH_EINVAL;
   *n = int(g_prof.size());

@@ -231,6 +231,38 @@ def test_pool_reuses_freed_blocks(singa, dev):
     assert dev.PoolStats()["driver_allocs"] - before <= 1
 
 
+def test_profiling_records_and_their_release(singa, dev):
+    """sgh_prof_enable / count / get / clear: a bracketed launch leaves a record with its tag, a positive
+    duration and its work; records outlive sgh_prof_enable(0) until sgh_prof_clear drops them; clearing
+    while records are still being taken is refused."""
+    import ctypes as C
+    from singa_amd import _lib
+    lib = _lib.lib()
+    m = 5000
+    x = singa.Tensor((m,), dev); x.SetFloatValue(1.0)
+    dy = singa.Tensor((m,), dev); dy.SetFloatValue(2.0)
+    n = C.c_int(-1)
+    assert lib.sgh_prof_enable(1) == 0
+    assert lib.sgh_prof_count(C.byref(n)) == 0 and n.value == 0
+    dx = singa.ReLUBackward(dy, x)
+    dev.Sync()
+    assert lib.sgh_prof_clear() == -1                       # still enabled
+    assert lib.sgh_prof_count(C.byref(n)) == 0 and n.value >= 1
+    taken = n.value
+    buf = C.create_string_buffer(64)
+    ms, work = C.c_float(), C.c_double()
+    assert lib.sgh_prof_get(0, buf, 64, C.byref(ms), C.byref(work)) == 0
+    assert buf.value.decode().startswith("relu_bwd/") and ms.value > 0
+    assert work.value == 3.0 * m * 4
+    assert lib.sgh_prof_get(taken, buf, 64, C.byref(ms), C.byref(work)) == -1
+    assert lib.sgh_prof_enable(0) == 0
+    assert lib.sgh_prof_count(C.byref(n)) == 0 and n.value == taken   # kept for the reader
+    assert lib.sgh_prof_clear() == 0
+    assert lib.sgh_prof_count(C.byref(n)) == 0 and n.value == 0
+    assert lib.sgh_prof_clear() == 0                        # idempotent
+    assert (dx.to_numpy() == 2.0).all()
+
+
 def test_upload_without_waiting(singa, dev):
     """sgh_upload_async: the host buffer may be overwritten as soon as the call returns, copies land
     in stream order (more uploads than staging slots in a row), oversize copies take the blocking path."""
