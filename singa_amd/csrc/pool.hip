@@ -434,6 +434,36 @@ __global__ __launch_bounds__(kBlock) void k_pool_avg_bwd(const typename S::elem 
   }
 }
 
+// One window that is the whole plane (global average pooling): every element of a plane receives
+// dy[plane] / (H * W), the same arithmetic as the kernel above, written in whole vectors.
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_pool_avg_bwd_global(const typename S::elem *__restrict__ dy,
+                                                               typename S::elem *__restrict__ dx, int HW, size_t total) {
+  constexpr int V = S::VEC;
+  const size_t stride = size_t(gridDim.x) * kBlock, tid = size_t(blockIdx.x) * kBlock + threadIdx.x;
+  const size_t nvec = total / V;
+  const float cnt = float(HW);
+  for (size_t iv = tid; iv < nvec; iv += stride) {
+    const size_t i0 = iv * V;
+    size_t plane = i0 / size_t(HW);
+    int r = int(i0 - plane * size_t(HW));
+    float gv = 0.f + S::ld(dy + plane) / cnt;
+    float o[V];
+#pragma unroll
+    for (int q = 0; q < V; ++q) {
+      if (r == HW) {
+        r = 0;
+        ++plane;
+        gv = 0.f + S::ld(dy + plane) / cnt;
+      }
+      o[q] = gv;
+      ++r;
+    }
+    S::store16(dx + i0, o);
+  }
+  for (size_t i = nvec * V + tid; i < total; i += stride) S::st(dx + i, 0.f + S::ld(dy + i / size_t(HW)) / cnt);
+}
+
 inline int grid_for(size_t n) {
   size_t blocks = (n + kBlock - 1) / kBlock;
   const size_t cap = size_t(sgh_num_cus()) * 32;
@@ -516,7 +546,11 @@ int pool_bwd(const sgh_pool_geom *g, const typename S::elem *dy, const typename 
       hipLaunchKernelGGL(k_pool_max_bwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
                          to_g(g), total);
     }
-  } else
+  } else if (g->P == 1 && g->Q == 1 && g->pad_h == 0 && g->pad_w == 0 && g->kernel_h >= g->H && g->kernel_w >= g->W &&
+             sgh_aligned16(dx))
+    hipLaunchKernelGGL(k_pool_avg_bwd_global<S>, dim3(grid_for((total + S::VEC - 1) / S::VEC)), dim3(kBlock), 0,
+                       sgh_stream_of(stream), dy, dx, g->H * g->W, total);
+  else
     hipLaunchKernelGGL(k_pool_avg_bwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, dx, to_g(g),
                        total);
   SGH_LAUNCH_CHECK();

@@ -209,6 +209,8 @@ def test_fused_relu_batchnorm_backward(singa, dev, kind, shape):
     (2, 16, 112, 112, (3, 3), (2, 2), (1, 1)),   # ResNet stem max-pool geometry (tiled kernel, 16-byte staging)
     (1, 2, 7, 5, (3, 2), (1, 2), (1, 0)),
     (3, 8, 14, 14, (3, 3), (1, 1), (1, 1)),
+    (3, 40, 7, 7, (7, 7), (1, 1), (0, 0)),       # ResNet global pool geometry (whole-vector average backward)
+    (1, 3, 5, 3, (5, 3), (1, 1), (0, 0)),        # ... planes of 15 elements: vectors across planes, scalar tail
 ])
 def test_pooling_16bit_storage(singa, dev, kind, case):
     """Max pooling on 16-bit tensors routes the gradient like the CPU algorithm on the stored

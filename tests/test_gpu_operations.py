@@ -385,6 +385,7 @@ POOL_CASES = [
     (1, 2, 7, 5, (3, 2), (1, 2), (1, 0)),
     (2, 2, 6, 6, (2, 2), (3, 3), (0, 0)),        # stride > kernel: inputs outside every window
     (4, 512, 7, 7, (7, 7), (1, 1), (0, 0)),      # ResNet global pool geometry
+    (1, 3, 5, 3, (5, 3), (1, 1), (0, 0)),        # global pool, planes of 15: vectors across planes and a scalar tail
     (3, 5, 12, 8, (3, 3), (2, 2), (1, 1)),       # window-column kernel: one partial wavefront strip
     (2, 3, 60, 16, (3, 3), (2, 2), (1, 1)),      # ... two bands (28 + 2 block rows)
     (1, 2, 6, 256, (3, 3), (2, 2), (1, 1)),      # ... 128 window columns: three column groups of 63
