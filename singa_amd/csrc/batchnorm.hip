@@ -465,13 +465,17 @@ struct ChipPlan {
   bool ok;
   int G, vpg, nt;   // slices per channel, vectors per slice, threads per workgroup
   int nl;           // vectors per tensor and thread kept in LDS (0: registers only)
+  bool ragged;      // planes that are not whole vectors (7 x 7): see RAGGED in k_bn_bwd_onchip
 };
 
 template <class S>
 inline ChipPlan chip_plan(int N, int C, int HW) {
-  ChipPlan p{false, 0, 0, 0, 0};
-  if (HW % S::VEC != 0) return p;
-  const long TV = long(N) * (HW / S::VEC);                       // vectors per channel
+  ChipPlan p{false, 0, 0, 0, 0, false};
+  p.ragged = HW % S::VEC != 0;
+  if (p.ragged && (S::VEC * sizeof(typename S::elem) != 16 || HW < S::VEC || sgh_env().bn_ragged_off ||
+                   size_t(N) * C * HW * sizeof(typename S::elem) >= (size_t(1) << 31)))
+    return p;
+  const long TV = long(N) * ((HW + S::VEC - 1) / S::VEC);        // vectors per channel
   // 512 threads (two workgroups per CU: one loads while the other waits or stores) unless that cuts the
   // channel into more slices than one wavefront can poll
   p.nt = 512;
@@ -479,7 +483,7 @@ inline ChipPlan chip_plan(int N, int C, int HW) {
   // the ReLU gate, C64 56x56 47.5 -> 40.2 us, C128 28x28 23.9 -> 21.5, C512 28x28 83.9 -> 79.4, C128 56x56 83.7 ->
   // 80.0, but the 205 MB tensors C256 56x56 153.8 -> 166.1 and C64 112x112 168.6 -> 174.8, with or without the
   // non-temporal hint that the register loads carry)
-  const bool lds_ok = chip_nl<S>() > 0 && size_t(N) * C * HW * sizeof(typename S::elem) <= (size_t(128) << 20);
+  const bool lds_ok = chip_nl<S>() > 0 && !p.ragged && size_t(N) * C * HW * sizeof(typename S::elem) <= (size_t(128) << 20);
   int per_thread = chip_nv<S>() + (lds_ok ? chip_nl<S>() : 0);
   long G = (TV + long(p.nt) * per_thread - 1) / (long(p.nt) * per_thread);
   if (G > kChipMaxG) {
@@ -500,11 +504,15 @@ inline ChipPlan chip_plan(int N, int C, int HW) {
   if (G > kChipMaxG || G < 1) return p;
   p.vpg = int((TV + G - 1) / G);
   p.G = int((TV + p.vpg - 1) / p.vpg);
-  p.ok = long(C) * p.G < 0x7fffffffL;
+  p.ok = long(C) * p.G < 0x7fffffffL && !(p.ragged && p.nt != 512);
   return p;
 }
 
-template <class S, bool RELU, int NT, int NL = 0>
+// RAGGED: planes that are not whole vectors.  A plane of HW elements is covered by ceil(HW / V) pieces of 16 bytes
+// at 2- or 4-byte alignment (buffer loads and stores take any); the last piece starts at HW - V, i.e. overlaps
+// the one before it instead of running into the next plane: its first V - HW % V elements are left out of the
+// sums, and its store rewrites them with the values the piece before it stores (same inputs, same expression).
+template <class S, bool RELU, int NT, int NL = 0, bool RAGGED = false>
 __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem *__restrict__ dy,
                                                           const typename S::elem *__restrict__ x,
                                                           const float *__restrict__ gamma, const float *__restrict__ beta,
@@ -534,12 +542,23 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     ticket_s = (unsigned(wa) == unsigned(ticket1) && unsigned(wb) == unsigned(ticket1 >> 32)) ? ticket2 : ticket1;
     gave_up = 0;
   }
-  const int PV = s.HW / V, TV = s.N * PV;
+  static_assert(!RAGGED || (NL == 0 && V * sizeof(elem) == 16), "ragged planes: 16-byte pieces in registers");
+  const int PV = RAGGED ? (s.HW + V - 1) / V : s.HW / V, TV = s.N * PV;
+  const int tail_skip = RAGGED && s.HW % V ? V - s.HW % V : 0;   // elements of a plane's last piece that are not its own
   const int lo = g * vpg, hi = min(lo + vpg, TV);
   const float mean = save_mean[c], invstd = save_invstd[c];
   const float gm = gamma[c], be = RELU ? beta[c] : 0.f;
   auto gate = [&](float d, float v) { return !RELU || S::stored_positive(bn_out(v, mean, invstd, gm, be)) ? d : 0.f; };
   const raw *xg = reinterpret_cast<const raw *>(x), *dg_ = reinterpret_cast<const raw *>(dy);
+  const int tensor_bytes = RAGGED ? int(size_t(s.N) * s.C * s.HW * sizeof(elem)) : 0;
+  const __amdgpu_buffer_rsrc_t rxb = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(x), 0, tensor_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rdb = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(dy), 0, tensor_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rob = __builtin_amdgcn_make_buffer_rsrc(dx, 0, tensor_bytes, 0x00020000);
+  // byte offset of piece r of plane (n, c)
+  auto piece = [&](int n, int r) {
+    return int(((unsigned(n) * unsigned(s.C) + unsigned(c)) * unsigned(s.HW) + unsigned(r == PV - 1 ? s.HW - V : r * V)) *
+               unsigned(sizeof(elem)));
+  };
   raw xv[NV], dv[NV];
   // vectors 0 .. NL-1 of a thread go to LDS: slot j of tensor z at ((z * NL + j) * NT + t) * 16 bytes.  A
   // wavefront's instruction writes 64 consecutive slots (LDS address = wavefront-uniform base + 16 * lane).
@@ -569,18 +588,26 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     const int iv = lo + (NL + i) * NT + t;
     if (iv < hi) {
       const int n = iv / PV, r = iv - n * PV;
-      const size_t off = (size_t(n) * s.C + c) * PV + r;
-      xv[i] = __builtin_nontemporal_load(xg + off);
-      dv[i] = __builtin_nontemporal_load(dg_ + off);
+      if constexpr (RAGGED) {
+        xv[i] = __builtin_bit_cast(raw, __builtin_amdgcn_raw_buffer_load_b128(rxb, piece(n, r), 0, 0));
+        dv[i] = __builtin_bit_cast(raw, __builtin_amdgcn_raw_buffer_load_b128(rdb, piece(n, r), 0, 0));
+      } else {
+        const size_t off = (size_t(n) * s.C + c) * PV + r;
+        xv[i] = __builtin_nontemporal_load(xg + off);
+        dv[i] = __builtin_nontemporal_load(dg_ + off);
+      }
     }
   }
   float a = 0.f, b = 0.f, b1 = 0.f;
   // (a macro, not a lambda: with the vectors passed to a lambda the register arrays went to scratch memory)
-#define BN_CHIP_ACCUMULATE(XR, DR)                                                                            \
+#define BN_CHIP_ACCUMULATE(XR, DR, SKIP)                                                                      \
   {                                                                                                           \
     float v[V], d[V];                                                                                         \
     S::template load16<false>(reinterpret_cast<const elem *>(&(XR)), v);                                      \
     S::template load16<false>(reinterpret_cast<const elem *>(&(DR)), d);                                      \
+    if constexpr (RAGGED) {                                                                                   \
+      _Pragma("unroll") for (int q = 0; q < V; ++q) d[q] = q < (SKIP) ? 0.f : d[q];                           \
+    }                                                                                                         \
     _Pragma("unroll") for (int q = 0; q < V; q += 4) {                                                        \
       const float d0 = gate(d[q], v[q]), d1 = gate(d[q + 1], v[q + 1]), d2 = gate(d[q + 2], v[q + 2]),        \
                   d3 = gate(d[q + 3], v[q + 3]);                                                              \
@@ -600,12 +627,14 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
       if (lo + j * NT + t < hi) {
         const raw xl = *reinterpret_cast<const raw *>(chip_lds + size_t((0 * NL + j) * NT + t) * 16);
         const raw dl = *reinterpret_cast<const raw *>(chip_lds + size_t((1 * NL + j) * NT + t) * 16);
-        BN_CHIP_ACCUMULATE(xl, dl)
+        BN_CHIP_ACCUMULATE(xl, dl, 0)
       }
   }
 #pragma unroll
-  for (int i = 0; i < NV; ++i)
-    if (lo + (NL + i) * NT + t < hi) BN_CHIP_ACCUMULATE(xv[i], dv[i])
+  for (int i = 0; i < NV; ++i) {
+    const int iv = lo + (NL + i) * NT + t;
+    if (iv < hi) BN_CHIP_ACCUMULATE(xv[i], dv[i], (iv % PV == PV - 1 ? tail_skip : 0))
+  }
 #undef BN_CHIP_ACCUMULATE
   b += b1;
   float db = sgh_block_sum(a, red), dg = sgh_block_sum(b, red);
@@ -666,7 +695,10 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
         o[q] = k * (gate(d[q], v[q]) - __builtin_fmaf((v[q] - mean) * invstd, c1, c0));                       \
     raw ov;                                                                                                   \
     S::store16(reinterpret_cast<elem *>(&ov), o);                                                             \
-    og[(size_t(n) * s.C + c) * PV + r] = ov;                                                                  \
+    if constexpr (RAGGED)                                                                                     \
+      __builtin_amdgcn_raw_buffer_store_b128(ov, rob, piece(n, r), 0, 0);                                     \
+    else                                                                                                      \
+      og[(size_t(n) * s.C + c) * PV + r] = ov;                                                                \
   }
   if constexpr (NL > 0) {
 #pragma unroll
@@ -726,6 +758,14 @@ int launch_onchip(const typename S::elem *dy, const typename S::elem *x, const f
       return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
     }
   }
+  if constexpr (S::VEC * sizeof(typename S::elem) == 16) {
+    if (p.ragged) {
+      hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512, 0, true>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean,
+                         save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
+      return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+    }
+  }
+  if (p.ragged) return SGH_EUNSUPPORTED;
   if (p.nt == 512)
     hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean, save_invstd,
                        dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
@@ -839,7 +879,11 @@ int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *g
   const ChipPlan cp = chip_plan<S>(N, C, HW);
   // (channels of at most 4096 vectors that fit in LDS are a little faster through the LDS-resident kernel below:
   // 13.4 against 14.9 us at 64 x 256 x 14 x 14 fp32)
-  const bool small_resident = resident_ok(N, C, HW, sizeof(typename S::elem)) && long(N) * (HW / S::VEC) <= 4096;
+  // (ragged planes of few elements -- 7 x 7 -- as well, unless the channels need more than two rounds of its
+  // one workgroup per channel: f16 128 x 512 x 7 x 7 13.3 us there, 13.9 here, but 128 x 2048 x 7 x 7 42.6 against
+  // 23.7 -- the LDS-resident kernel moves single elements)
+  const bool small_resident = resident_ok(N, C, HW, sizeof(typename S::elem)) &&
+                              (cp.ragged ? HW <= 64 && C <= 2 * sgh_num_cus() : long(N) * (HW / S::VEC) <= 4096);
   if (cp.ok && !small_resident && !sgh_env().bn_onchip_off) {
     if (!sgh_aligned16(workspace)) return SGH_EINVAL;
     return beta ? launch_onchip<S, true>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, workspace, s, cp, st)
@@ -909,6 +953,10 @@ size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
 // 16-bit planes that are a multiple of 4 but not of 8 elements (14 x 14) use the 8-byte vector class
 #define SGH_BN_DISPATCH16(fn, F16X8, F16X4, ...) \
   (HW % 8 != 0 && HW % 4 == 0 ? fn<F16X4>(__VA_ARGS__) : fn<F16X8>(__VA_ARGS__))
+// (the backward pass takes such planes in 16-byte pieces, the last one overlapping -- RAGGED in k_bn_bwd_onchip:
+// 128 x 1024 x 14 x 14 47.4 -> 41.4 us, fused with the ReLU gate 52.2 -> 44.9)
+#define SGH_BN_DISPATCH16_BWD(fn, F16X8, F16X4, ...) \
+  (HW % 8 != 0 && HW % 4 == 0 && sgh_env().bn_ragged_off ? fn<F16X4>(__VA_ARGS__) : fn<F16X8>(__VA_ARGS__))
 
 int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float *beta, float *running_mean,
                          float *running_var, float factor, float eps, float *y, float *save_mean, float *save_invstd,
@@ -949,13 +997,13 @@ int sgh_bn_bwd_noalloc_f32(const float *dy, const float *x, const float *gamma, 
 int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                    const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                    void *workspace, size_t ws_bytes, void *stream) {
-  return SGH_BN_DISPATCH16(bn_bwd, StF16, StF16x4, dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N,
+  return SGH_BN_DISPATCH16_BWD(bn_bwd, StF16, StF16x4, dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N,
                            C, HW, workspace, ws_bytes, stream);
 }
 int sgh_bn_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                     const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                     void *workspace, size_t ws_bytes, void *stream) {
-  return SGH_BN_DISPATCH16(bn_bwd, StBF16, StBF16x4, dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N,
+  return SGH_BN_DISPATCH16_BWD(bn_bwd, StBF16, StBF16x4, dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N,
                            C, HW, workspace, ws_bytes, stream);
 }
 
@@ -985,16 +1033,17 @@ int sgh_bn_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamm
                         const float *save_mean, const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta,
                         int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   if (!beta) return SGH_EINVAL;
-  return SGH_BN_DISPATCH16(bn_bwd, StF16, StF16x4, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C,
+  return SGH_BN_DISPATCH16_BWD(bn_bwd, StF16, StF16x4, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C,
                            HW, workspace, ws_bytes, stream);
 }
 int sgh_bn_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *beta,
                          const float *save_mean, const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta,
                          int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   if (!beta) return SGH_EINVAL;
-  return SGH_BN_DISPATCH16(bn_bwd, StBF16, StBF16x4, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C,
+  return SGH_BN_DISPATCH16_BWD(bn_bwd, StBF16, StBF16x4, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, N, C,
                            HW, workspace, ws_bytes, stream);
 }
 #undef SGH_BN_DISPATCH16
+#undef SGH_BN_DISPATCH16_BWD
 
 }  // extern "C"

@@ -98,7 +98,8 @@ def test_relu_backward_add_mult_axpy(singa, dev, kind, n):
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 28, 28), (16, 32, 8, 8), (3, 7, 4, 2),
                                    (16, 24, 14, 14), (2, 8, 6, 6),    # these two: planes of 8-byte vectors
-                                   (8, 128, 14, 14), (16, 256, 7, 7), (4, 130, 5, 6), (32, 128, 8, 8)])  # one-pass backward
+                                   (8, 128, 14, 14), (16, 256, 7, 7), (4, 130, 5, 6), (32, 128, 8, 8),   # one-pass backward
+                                   (128, 8, 7, 7), (96, 16, 5, 5)])    # ... ragged planes, a channel in several slices
 def test_batchnorm_16bit_storage(singa, dev, kind, shape):
     """BN forward-training / backward on 16-bit activations with fp32 parameters and statistics:
     the fp32 CPU oracle on the same (already rounded) inputs, outputs compared at the 16-bit
@@ -164,7 +165,8 @@ def test_batchnorm_inference(singa, dev, kind, shape):
 @pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 28, 28), (16, 32, 8, 8), (3, 7, 4, 2),
                                    (32, 64, 56, 56), (16, 24, 14, 14), (2, 8, 6, 6),
                                    # the one-pass backward (a channel fits in LDS, >= 128 channels)
-                                   (8, 128, 14, 14), (16, 256, 7, 7), (4, 130, 5, 6), (32, 128, 8, 8), (128, 256, 14, 14)])
+                                   (8, 128, 14, 14), (16, 256, 7, 7), (4, 130, 5, 6), (32, 128, 8, 8), (128, 256, 14, 14),
+                                   (128, 8, 7, 7), (96, 16, 5, 5)])
 def test_fused_relu_batchnorm_backward(singa, dev, kind, shape):
     """The fused ReLU + BatchNorm backward equals ReLUBackward followed by GpuBatchNormBackward on
     the forward's own output BIT FOR BIT (the recomputed output selects the same elements as the

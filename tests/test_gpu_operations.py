@@ -488,7 +488,9 @@ def test_bn_reference_vectors(singa, dev, golden):
 @pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 56, 56), (64, 512, 7, 7), (16, 128, 28, 28),
                                    (2, 64, 112, 112), (32, 10),
                                    # a channel fits in LDS and there are >= 128 of them: the one-pass backward
-                                   (8, 128, 14, 14), (16, 256, 7, 7), (4, 130, 5, 6), (64, 256, 14, 14), (3, 300, 1, 1)])
+                                   (8, 128, 14, 14), (16, 256, 7, 7), (4, 130, 5, 6), (64, 256, 14, 14), (3, 300, 1, 1),
+                                   # planes that are not whole vectors, a channel in several slices
+                                   (128, 8, 7, 7), (96, 16, 5, 5)])
 def test_bn_vs_oracle(singa, dev, shape):
     r = rng(sum(shape))
     x = (randn(r, *shape) * 2 + 0.5).astype(np.float32)
