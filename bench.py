@@ -142,6 +142,9 @@ def main():
     ap.add_argument("--no-overlap", action="store_true",
                     help="every kernel on the one device stream (weight gradients otherwise run on a second stream); "
                          "the setting for kernel traces whose durations should be those of kernels running alone")
+    ap.add_argument("--with-forward", action="store_true",
+                    help="time whole training steps -- forward pass, backward pass and update, inputs resident on the "
+                         "device -- instead of the backward pass and update alone (the metric's name says so)")
     ap.add_argument("--per-parameter-update", action="store_true",
                     help="update each parameter right after its gradient (one launch each) instead of one fused launch")
     args = ap.parse_args()
@@ -162,8 +165,12 @@ def main():
         hip.overlap_wgrad = False
     net = wl.build(args.config, hip, lr=0.05, momentum=0.9)
     x, labels = wl.make_inputs(args.config, args.batch)
-    net.forward(hip.from_numpy(x), hip.from_numpy(labels))
+    x_dev, labels_dev = hip.from_numpy(x), hip.from_numpy(labels)
+    net.forward(x_dev, labels_dev)
     fused = not args.per_parameter_update
+    if args.with_forward and args.graph:
+        print("bench.py: --with-forward times the eager tape (drop --graph)", file=sys.stderr)
+        sys.exit(2)
 
     sync = dev.Sync   # waits for both streams of the device
 
@@ -180,6 +187,8 @@ def main():
         step = dev.RunGraph
     else:
         def step():
+            if args.with_forward:
+                net.forward(x_dev, labels_dev)
             net.backward_and_update(fused_update=fused)
     for _ in range(args.warmup):
         step()
@@ -265,14 +274,15 @@ def main():
                       "frac": round(gbs / PEAK_HBM_GBS, 4)}
 
     out = {
-        "metric": "backward+update imgs/sec, ResNet-18 N=64 fp32" if (args.config == "resnet18" and not half and args.batch == 64)
+        "metric": "forward+backward+update imgs/sec, %s N=%d %s" % (args.config, args.batch, args.storage) if args.with_forward
+                  else "backward+update imgs/sec, ResNet-18 N=64 fp32" if (args.config == "resnet18" and not half and args.batch == 64)
                   else "backward+update imgs/sec, %s N=%d %s" % (args.config, args.batch, args.storage),
         "value": round(imgs_per_s, 2), "unit": "imgs/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "ms_per_step_median": round(median_ms, 4), "ms_per_step_min": round(step_ms[0], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.storage, "data": "synthetic",
-        "config": {"workload": "%s backward+update, N=%d, 3x224x224, %s, SGD momentum 0.9" % (
-                       args.config, args.batch, "fp32" if not half else args.storage + " storage / fp32 accumulate, statistics and master weights"),
+        "config": {"workload": "%s %sbackward+update, N=%d, 3x224x224, %s, SGD momentum 0.9" % (
+                       args.config, "forward+" if args.with_forward else "", args.batch, "fp32" if not half else args.storage + " storage / fp32 accumulate, statistics and master weights"),
                    "update": "fused multi-tensor" if fused else "per parameter",
                    "launch": "one recorded step replayed (graph mode)" if graph else "eager, one launch per kernel",
                    "tape": "ReLU backward folded into BatchNorm backward (conv-BN-ReLU), residual += folded into the "

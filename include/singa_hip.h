@@ -238,6 +238,14 @@ SGH_API int sgh_eltwise_mult_f32(const float *a, const float *b, int b_is_scalar
 /* Add<float, Lang> (Tensor::operator+=, src/core/tensor/tensor.cc:579-586): gradient fan-in
  * of python/singa/autograd.py:204.  out may alias a or b. */
 SGH_API int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream);
+/* Add followed by ReLU in one pass: the forward of a residual block's end, relu(out + identity)
+ * (examples/cnn/model/resnet.py:74-77, :112-115; python/singa/autograd.py add :1026-1040 then ReLU :421-430).
+ * Stores what the two calls store (the sum rounded to the storage type, then the selection); the ReLU's
+ * backward may gate on this output instead of the sum: both are positive at the same elements.
+ * out may alias a or b. */
+SGH_API int sgh_add_relu_f32(const float *a, const float *b, float *out, size_t n, void *stream);
+SGH_API int sgh_add_relu_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream);
+SGH_API int sgh_add_relu_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream);
 /* The other elementwise tensor functions the autograd ops of these models call around the
  * backward path (src/core/tensor/tensor_math_cpp.h): Sub :645-650, Div (tensor / tensor) :423-430,
  * Add(tensor, scalar) :383-388, EltwiseMult(tensor, scalar) :432-437.  Div(tensor, scalar) is
@@ -502,6 +510,22 @@ SGH_API int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float
                                  float *running_mean, float *running_var, float factor, float eps,
                                  float *y, float *save_mean, float *save_invstd, int N, int C,
                                  int HW, void *workspace, size_t ws_bytes, void *stream);
+/* GpuBatchNormForwardTraining followed by ReLU in one call (conv -> BatchNorm -> ReLU,
+ * examples/cnn/model/resnet.py:54-60; batchnorm.cc:287-329 then tensor_math_cpp.h:585-589): same statistics,
+ * y holds relu(BatchNorm(x)) -- the bits the two calls store -- so the ReLU's pass over y disappears.
+ * sgh_bn_relu_bwd_* is its backward (it recomputes the gate from x).  *_f16 / *_bf16 below likewise. */
+SGH_API int sgh_bn_relu_fwd_train_f32(const float *x, const float *gamma, const float *beta,
+                                      float *running_mean, float *running_var, float factor, float eps,
+                                      float *y, float *save_mean, float *save_invstd, int N, int C,
+                                      int HW, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_relu_fwd_train_f16(const uint16_t *x, const float *gamma, const float *beta,
+                                      float *running_mean, float *running_var, float factor, float eps,
+                                      uint16_t *y, float *save_mean, float *save_invstd, int N, int C,
+                                      int HW, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_relu_fwd_train_bf16(const uint16_t *x, const float *gamma, const float *beta,
+                                       float *running_mean, float *running_var, float factor, float eps,
+                                       uint16_t *y, float *save_mean, float *save_invstd, int N, int C,
+                                       int HW, void *workspace, size_t ws_bytes, void *stream);
 /* GpuBatchNormForwardInference (src/model/operation/batchnorm.cc:331-366):
  * y = gamma * (x - running_mean) / sqrt(running_var + eps) + beta. */
 SGH_API int sgh_bn_fwd_infer_f32(const float *x, const float *gamma, const float *beta,

@@ -99,6 +99,9 @@ SIGNATURES = {
     "sgh_axpy_devalpha_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_eltwise_mult_f32": (C.c_int, [vp, vp, C.c_int, vp, sz, vp]),
     "sgh_add_f32": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_add_relu_f32": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_add_relu_f16": (C.c_int, [vp, vp, vp, sz, vp]),
+    "sgh_add_relu_bf16": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_sgd_momentum_multi_mixed": (C.c_int, [vp, C.c_int, sz, C.c_int, C.c_float, C.c_float, C.c_float, C.c_float,
                                                C.c_int, vp]),
     "sgh_sub_f32": (C.c_int, [vp, vp, vp, sz, vp]),
@@ -161,6 +164,12 @@ SIGNATURES = {
     "sgh_conv_fwd_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
     "sgh_bn_workspace_bytes": (sz, [C.c_int, C.c_int, C.c_int]),
     "sgh_bn_fwd_train_f32": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
+                                       C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_relu_fwd_train_f32": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
+                                       C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_relu_fwd_train_f16": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
+                                       C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_relu_fwd_train_bf16": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
                                        C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_bwd_f32": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_bwd_noalloc_f32": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),

@@ -99,6 +99,14 @@ __device__ __forceinline__ void channel_range(const BnShape s, int c, int lo, in
 __device__ __forceinline__ float bn_out(float v, float mean, float invstd, float g, float be) {
   return __builtin_fmaf(g, (v - mean) * invstd, be);
 }
+// The same value as an fp32 number the compiler cannot look behind: a binary16 store right behind the fmaf
+// otherwise becomes one instruction that rounds the exact product-sum to 16 bits once, and a store with
+// anything in between (the ReLU selection) rounds twice -- one unit in the last place apart now and then.
+__device__ __forceinline__ float bn_out_rounded(float v, float mean, float invstd, float g, float be) {
+  float r = bn_out(v, mean, invstd, g, be);
+  asm volatile("" : "+v"(r));
+  return r;
+}
 
 // ---- forward, pass 1: per (c, split) partial sum and sum of squares about a pivot ---------
 // The pivot (the channel's first element) keeps the single-pass variance well conditioned.
@@ -133,7 +141,15 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_partial(const typename S::ele
 }
 
 // ---- forward, pass 2: finish statistics (every workgroup redoes the tiny S-sum), normalise --
+// RELU: the ReLU that consumes this BatchNorm's output folded in -- what the two separate calls store, bit for bit
+// (fp32: y >= 0 ? y : 0 as the ReLU kernel; 16-bit: the stored value where it is positive, else 0)
 template <class S>
+__device__ __forceinline__ float bn_relu_value(float y) {
+  if constexpr (sizeof(typename S::elem) == 4) return y >= 0.f ? y : 0.f;
+  else return S::stored_positive(y) ? y : 0.f;
+}
+
+template <class S, bool RELU>
 __global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const typename S::elem *__restrict__ x,
                                                         const float *__restrict__ gamma, const float *__restrict__ beta,
                                                         const float *__restrict__ part, float *__restrict__ running_mean,
@@ -168,10 +184,16 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const typename S::elem 
       [&](size_t off, const float *v, const float *) {
         float r[S::VEC];
 #pragma unroll
-        for (int q = 0; q < S::VEC; ++q) r[q] = bn_out(v[q], mean, invstd, g, be);
+        for (int q = 0; q < S::VEC; ++q) {
+          r[q] = bn_out_rounded(v[q], mean, invstd, g, be);
+          if (RELU) r[q] = bn_relu_value<S>(r[q]);
+        }
         S::store16(y + off, r);
       },
-      [&](size_t off) { S::st(y + off, bn_out(S::ld(x + off), mean, invstd, g, be)); });
+      [&](size_t off) {
+        const float r = bn_out_rounded(S::ld(x + off), mean, invstd, g, be);
+        S::st(y + off, RELU ? bn_relu_value<S>(r) : r);
+      });
 }
 
 // ---- forward, inference: normalise with the running statistics ------------------------------
@@ -190,10 +212,10 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_infer(const typename S::elem 
       [&](size_t off, const float *v, const float *) {
         float r[S::VEC];
 #pragma unroll
-        for (int q = 0; q < S::VEC; ++q) r[q] = bn_out(v[q], mean, invstd, g, be);
+        for (int q = 0; q < S::VEC; ++q) r[q] = bn_out_rounded(v[q], mean, invstd, g, be);
         S::store16(y + off, r);
       },
-      [&](size_t off) { S::st(y + off, bn_out(S::ld(x + off), mean, invstd, g, be)); });
+      [&](size_t off) { S::st(y + off, bn_out_rounded(S::ld(x + off), mean, invstd, g, be)); });
 }
 
 // ---- backward, pass 1: partial sum(dy) and sum(dy * xhat) ---------------------------------
@@ -825,7 +847,7 @@ inline BnShape make_shape(int N, int C, int HW, int vec, int esize) {
 template <class S>
 int bn_fwd_train(const typename S::elem *x, const float *gamma, const float *beta, float *running_mean,
                  float *running_var, float factor, float eps, typename S::elem *y, float *save_mean, float *save_invstd,
-                 int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+                 int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream, bool relu = false) {
   if (!shape_ok(N, C, HW) || !x || !gamma || !beta || !y || !save_mean || !save_invstd) return SGH_EINVAL;
   const BnShape s = make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem)));
   if (!sgh_aligned16(x) || !sgh_aligned16(y)) return SGH_EINVAL;
@@ -833,8 +855,12 @@ int bn_fwd_train(const typename S::elem *x, const float *gamma, const float *bet
   float *scratch = static_cast<float *>(workspace);
   hipLaunchKernelGGL(k_bn_fwd_partial<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, scratch, s);
   SGH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_bn_fwd_apply<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, gamma, beta, scratch,
-                     running_mean, running_var, factor, eps, y, save_mean, save_invstd, s);
+  if (relu)
+    hipLaunchKernelGGL((k_bn_fwd_apply<S, true>), dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, gamma, beta,
+                       scratch, running_mean, running_var, factor, eps, y, save_mean, save_invstd, s);
+  else
+    hipLaunchKernelGGL((k_bn_fwd_apply<S, false>), dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, gamma, beta,
+                       scratch, running_mean, running_var, factor, eps, y, save_mean, save_invstd, s);
   SGH_LAUNCH_CHECK();
   return SGH_OK;
 }
@@ -975,6 +1001,25 @@ int sgh_bn_fwd_train_bf16(const uint16_t *x, const float *gamma, const float *be
                           float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   return SGH_BN_DISPATCH16(bn_fwd_train, StBF16, StBF16x4, x, gamma, beta, running_mean, running_var, factor, eps, y,
                            save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream);
+}
+
+int sgh_bn_relu_fwd_train_f32(const float *x, const float *gamma, const float *beta, float *running_mean,
+                              float *running_var, float factor, float eps, float *y, float *save_mean,
+                              float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  return bn_fwd_train<StF32>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C, HW,
+                             workspace, ws_bytes, stream, true);
+}
+int sgh_bn_relu_fwd_train_f16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
+                              float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
+                              float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  return SGH_BN_DISPATCH16(bn_fwd_train, StF16, StF16x4, x, gamma, beta, running_mean, running_var, factor, eps, y,
+                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream, true);
+}
+int sgh_bn_relu_fwd_train_bf16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
+                               float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
+                               float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+  return SGH_BN_DISPATCH16(bn_fwd_train, StBF16, StBF16x4, x, gamma, beta, running_mean, running_var, factor, eps, y,
+                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream, true);
 }
 
 int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const float *save_mean,

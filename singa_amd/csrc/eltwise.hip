@@ -114,6 +114,12 @@ struct ReluFwd {  // second operand unused
 struct AddOp {
   __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
 };
+struct AddReluOp {  // ReluFwd of the sum
+  __device__ __forceinline__ float operator()(float a, float b) const {
+    const float s = a + b;
+    return s >= 0.f ? s : 0.f;
+  }
+};
 struct ClampOp {  // second operand unused; NaN passes through, as in the CPU function's two comparisons
   float lo, hi;
   __device__ __forceinline__ float operator()(float x, float) const { return x < lo ? lo : (x > hi ? hi : x); }
@@ -493,6 +499,10 @@ int sgh_clamp_f32(float low, float high, const float *x, float *out, size_t n, v
 int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
   sgh_prof_scope prof("add/k_map2_1<AddOp>", 3.0 * n * sizeof(float), sgh_stream_of(stream));
   return launch_map2(a, b, out, n, AddOp{}, stream);
+}
+
+int sgh_add_relu_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
+  return launch_map2(a, b, out, n, AddReluOp{}, stream);
 }
 
 int sgh_sub_f32(const float *a, const float *b, float *out, size_t n, void *stream) {

@@ -156,6 +156,13 @@ int launch_relu_bwd_add(const typename S::elem *dy0, const typename S::elem *dy1
 struct AddOp {
   __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
 };
+template <class T>
+struct AddReluOp {  // the stored sum where it is positive, else 0: Add followed by the 16-bit ReLU
+  __device__ __forceinline__ float operator()(float a, float b) const {
+    const float s = T::load(T::store(a + b));
+    return s > 0.f ? s : 0.f;
+  }
+};
 struct MulOp {
   __device__ __forceinline__ float operator()(float a, float b) const { return a * b; }
 };
@@ -462,6 +469,12 @@ int sgh_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, v
 int sgh_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
   sgh_prof_scope prof("add/k_map2_h<AddOp>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<BF16>(a, b, out, n, AddOp{}, stream);
+}
+int sgh_add_relu_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  return launch_map2_h<F16>(a, b, out, n, AddReluOp<F16>{}, stream);
+}
+int sgh_add_relu_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  return launch_map2_h<BF16>(a, b, out, n, AddReluOp<BF16>{}, stream);
 }
 int sgh_eltwise_mult_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
   return launch_map2_h<F16>(a, b, out, n, MulOp{}, stream);

@@ -644,6 +644,16 @@ def __add__(a, b):
     return out
 
 
+def AddReLU(a, b):
+    """``relu(a + b)`` in one pass, the end of a residual block's forward (examples/cnn/model/resnet.py:74-77):
+    the bits ``ReLU(a + b)`` stores."""
+    _same(a, b)
+    out = _like(a)
+    fn, name = _fn("add_relu", a)
+    check(fn(a.ptr, b.ptr, out.ptr, a.Size(), a.device().stream), name)
+    return out
+
+
 def _binary_f32(name, a, b):
     _same(a, b)
     if a.data_type() != kFloat32:
@@ -904,6 +914,21 @@ def GpuBatchNormForwardTraining(h, x, scale, bias, running_mean, running_var):
     mean = Tensor((h.channels,), x.device(), kFloat32)
     var = Tensor((h.channels,), x.device(), kFloat32)
     fn, name = _fn("bn_fwd_train", x)  # 16-bit activations keep fp32 scale / bias / statistics
+    check(fn(x.ptr, scale.ptr, bias.ptr,
+             running_mean.ptr if running_mean is not None else None,
+             running_var.ptr if running_var is not None else None,
+             h.factor, _BN_EPS, y.ptr, mean.ptr, var.ptr, h.batchsize, h.channels,
+             h.height * h.width, h.workspace.ptr, h.workspace.MemSize(), x.device().stream), name)
+    return [y, mean, var]
+
+
+def GpuBatchNormReLUForwardTraining(h, x, scale, bias, running_mean, running_var):
+    """``GpuBatchNormForwardTraining`` with the ReLU that follows folded in: ``[relu(y), mean, var]``, the bits
+    ``ReLU(GpuBatchNormForwardTraining(...)[0])`` stores (conv -> BatchNorm -> ReLU, examples/cnn/model/resnet.py:54-60)."""
+    y = _like(x)
+    mean = Tensor((h.channels,), x.device(), kFloat32)
+    var = Tensor((h.channels,), x.device(), kFloat32)
+    fn, name = _fn("bn_relu_fwd_train", x)
     check(fn(x.ptr, scale.ptr, bias.ptr,
              running_mean.ptr if running_mean is not None else None,
              running_var.ptr if running_var is not None else None,

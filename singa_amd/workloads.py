@@ -64,6 +64,16 @@ class HipOps(object):
     def bn_fwd_train(self, h, x, g, b, rm, rv):
         return singa.GpuBatchNormForwardTraining(h, x, g, b, rm, rv)
 
+    # cross-op fusion of the forward pass: the ReLU behind a BatchNorm, or behind the sum that ends a residual
+    # block, applied by the kernel that produces its input (the same bits, one tensor pass less each)
+    fuse_forward = True
+
+    def bn_relu_fwd_train(self, h, x, g, b, rm, rv):
+        return singa.GpuBatchNormReLUForwardTraining(h, x, g, b, rm, rv)
+
+    def add_relu(self, a, b):
+        return singa.AddReLU(a, b)
+
     def pool_fwd(self, h, x):
         return singa.GpuPoolingForward(h, x)
 
@@ -173,11 +183,12 @@ class HipOps(object):
             self.dev.Join()    # the update (and any reader of a weight gradient) comes after the last of them
             self._aux = None
 
-    fusions = ("fuse_bn_relu", "fuse_dgrad_add", "fuse_wgrad_bias", "batch_relayout", "overlap_wgrad")   # what set_fusion(True) turns on
+    fusions = ("fuse_bn_relu", "fuse_dgrad_add", "fuse_wgrad_bias", "batch_relayout", "overlap_wgrad", "fuse_forward")   # what set_fusion(True) turns on
 
     def set_fusion(self, on):
         """All of this implementation's cross-op fusions on, or the reference's op-per-op tape."""
-        for f in ("fuse_bn_relu", "fuse_dgrad_add", "fuse_add_relu", "fuse_wgrad_bias", "batch_relayout", "overlap_wgrad"):
+        for f in ("fuse_bn_relu", "fuse_dgrad_add", "fuse_add_relu", "fuse_wgrad_bias", "batch_relayout", "overlap_wgrad",
+                  "fuse_forward"):
             setattr(self, f, bool(on) and f in self.fusions)
 
     def accumulate(self, a, b):
@@ -219,7 +230,7 @@ class HalfHipOps(HipOps):
     # scattered 2-byte stores make a read-modify-write epilogue slower than the separate add)
     fuse_dgrad_add = False
     fuse_add_relu = True
-    fusions = ("fuse_bn_relu", "fuse_add_relu", "fuse_wgrad_bias", "batch_relayout", "overlap_wgrad")
+    fusions = ("fuse_bn_relu", "fuse_add_relu", "fuse_wgrad_bias", "batch_relayout", "overlap_wgrad", "fuse_forward")
 
     def __init__(self, dev, dtype):
         HipOps.__init__(self, dev)
@@ -314,6 +325,19 @@ class BatchNorm(_Layer):
         self.x = x
         return y
 
+    def fwd_through_relu(self, relu, x):
+        """Forward of ``relu(self(x))``, as one fused call where the ops implementation offers it.  The ReLU then
+        keeps its output for its backward: positive exactly where its input was."""
+        if not getattr(self.ops, "fuse_forward", False):
+            return relu.fwd(self.fwd(x))
+        if self.h is None:
+            self.h = self.ops.bn_handle(self.momentum, x)
+        y, self.mean, self.var = self.ops.bn_relu_fwd_train(self.h, x, self.scale, self.bias, self.running_mean,
+                                                            self.running_var)
+        self.x = x
+        relu.x = y
+        return y
+
     def bwd(self, dy, grads):
         dx, ds, db = self.ops.bn_bwd(self.h, dy, self.x, self.scale, self.mean, self.var)
         grads(self.name + ".scale", self.scale, ds)
@@ -351,6 +375,14 @@ class ReLU(_Layer):
     def fwd(self, x):
         self.x = x
         return self.ops.relu(x)
+
+    def fwd_of_sum(self, a, b):
+        """Forward of ``relu(a + b)`` (the end of a residual block), in one pass where the ops implementation
+        offers it; the output is kept for the backward as in BatchNorm.fwd_through_relu."""
+        if not getattr(self.ops, "fuse_forward", False):
+            return self.fwd(self.ops.add(a, b))
+        self.x = self.ops.add_relu(a, b)
+        return self.x
 
     def bwd(self, dy, grads):
         if isinstance(dy, _Sum):
@@ -442,11 +474,11 @@ class BasicBlock(_Layer):
         return ls
 
     def fwd(self, x):
-        out = self.bn2.fwd(self.conv2.fwd(self.relu1.fwd(self.bn1.fwd(self.conv1.fwd(x)))))
+        out = self.bn2.fwd(self.conv2.fwd(self.bn1.fwd_through_relu(self.relu1, self.conv1.fwd(x))))
         residual = x
         if self.ds_conv is not None:
             residual = self.ds_bn.fwd(self.ds_conv.fwd(x))
-        return self.relu2.fwd(self.ops.add(out, residual))
+        return self.relu2.fwd_of_sum(out, residual)
 
     def bwd(self, dy, grads):
         d_add = self.relu2.bwd(dy, grads)
@@ -497,13 +529,13 @@ class Bottleneck(_Layer):
         return ls
 
     def fwd(self, x):
-        out = self.relu1.fwd(self.bn1.fwd(self.conv1.fwd(x)))
-        out = self.relu2.fwd(self.bn2.fwd(self.conv2.fwd(out)))
+        out = self.bn1.fwd_through_relu(self.relu1, self.conv1.fwd(x))
+        out = self.bn2.fwd_through_relu(self.relu2, self.conv2.fwd(out))
         out = self.bn3.fwd(self.conv3.fwd(out))
         residual = x
         if self.ds_conv is not None:
             residual = self.ds_bn.fwd(self.ds_conv.fwd(x))
-        return self.relu3.fwd(self.ops.add(out, residual))
+        return self.relu3.fwd_of_sum(out, residual)
 
     def bwd(self, dy, grads):
         d_add = self.relu3.bwd(dy, grads)
@@ -569,8 +601,15 @@ class Net(object):
     def forward(self, x, labels):
         """Runs the forward pass, keeps what the backward needs, returns the mean loss tensor data."""
         self.batch = self.ops.shape(x)[0]
-        for l in self.layers:
-            x = l.fwd(x)
+        i = 0
+        while i < len(self.layers):
+            l = self.layers[i]
+            if isinstance(l, BatchNorm) and i + 1 < len(self.layers) and isinstance(self.layers[i + 1], ReLU):
+                x = l.fwd_through_relu(self.layers[i + 1], x)   # the stem's conv -> BatchNorm -> ReLU
+                i += 2
+            else:
+                x = l.fwd(x)
+                i += 1
         self.logits = x
         self.p = self.ops.softmax(x)
         self.t = labels

@@ -204,6 +204,55 @@ def test_fused_relu_batchnorm_backward(singa, dev, kind, shape):
     assert nl2(one[1].to_numpy(), ds_o) < 1e-3 and nl2(one[2].to_numpy(), db_o) < 1e-3
 
 
+@pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", [(4, 3, 5, 6), (8, 64, 28, 28), (16, 24, 14, 14), (16, 256, 7, 7), (3, 7, 4, 2),
+                                   (2, 5, 7, 7)])
+def test_fused_forward_calls(singa, dev, kind, shape):
+    """The forward fusions store the bits of the separate calls: GpuBatchNormReLUForwardTraining =
+    ReLU(GpuBatchNormForwardTraining(...)) with the same saved and running statistics, AddReLU(a, b) =
+    ReLU(a + b) (zeros, negative zeros of the sum and 16-bit underflow included); and a ReLU backward gated on
+    the fused output equals the one gated on the ReLU's input."""
+    r = rng(sum(shape) + 11)
+    N, C, H, W = shape
+    x32 = (r.standard_normal(shape) * 1.5 - 0.2).astype(np.float32)
+    a32 = r.standard_normal(shape).astype(np.float32)
+    a32.ravel()[::5] = -x32.ravel()[::5]        # sums that are exactly zero
+    a32.ravel()[1::7] = 0.0
+    dy32 = r.standard_normal(shape).astype(np.float32)
+    gamma = (1 + 0.3 * r.standard_normal(C)).astype(np.float32)
+    beta = (0.2 * r.standard_normal(C)).astype(np.float32)
+    gamma[0], beta[0] = 0.0, 0.0                # outputs exactly 0
+    if C > 1:
+        gamma[1], beta[1] = 1e-6, 1e-8          # tiny outputs: underflow to zero in binary16
+    if kind == "f32":
+        xt, at, dyt = (singa.from_numpy(v, dev) for v in (x32, a32, dy32))
+        relu = singa.ReLU
+    else:
+        xt, at, dyt = (_to(singa, dev, v, kind)[0] for v in (x32, a32, dy32))
+        relu = lambda t: singa.ReLUBackward(t, t)   # the 16-bit tape's ReLU: t > 0 ? t : 0
+    gd, bd = singa.from_numpy(gamma, dev), singa.from_numpy(beta, dev)
+    stats = lambda: (singa.from_numpy(np.full(C, 0.25, np.float32), dev), singa.from_numpy(np.full(C, 2.0, np.float32), dev))
+    h = singa.CudnnBatchNormHandle(0.9, xt)
+    rm1, rv1 = stats()
+    y, mean, var = singa.GpuBatchNormForwardTraining(h, xt, gd, bd, rm1, rv1)
+    rm2, rv2 = stats()
+    yr, mean2, var2 = singa.GpuBatchNormReLUForwardTraining(h, xt, gd, bd, rm2, rv2)
+    _same_bits(yr.to_numpy(), relu(y).to_numpy(), "BatchNorm + ReLU forward " + kind)
+    for got, want, what in ((mean2, mean, "mean"), (var2, var, "invstd"), (rm2, rm1, "running mean"), (rv2, rv1, "running var")):
+        _same_bits(got.to_numpy(), want.to_numpy(), what + " " + kind)
+    _same_bits(singa.ReLUBackward(dyt, yr).to_numpy(), singa.ReLUBackward(dyt, y).to_numpy(), "ReLU backward gated on the output " + kind)
+    s = singa.__add__(xt, at)
+    sr = singa.AddReLU(xt, at)
+    _same_bits(sr.to_numpy(), relu(s).to_numpy(), "Add + ReLU forward " + kind)
+    _same_bits(singa.ReLUBackward(dyt, sr).to_numpy(), singa.ReLUBackward(dyt, s).to_numpy(), "ReLU backward gated on the sum's output " + kind)
+    # unaligned operands take the scalar path
+    n = xt.Size() - 1
+    dt = {"f32": singa.kFloat32, "f16": singa.kFloat16, "bf16": singa.kBFloat16}[kind]
+    views = [singa.from_device_pointer(t.ptr + (4 if kind == "f32" else 2), (n,), dev, dtype=dt, keepalive=t)
+             for t in (xt, at)]
+    _same_bits(singa.AddReLU(*views).to_numpy(), sr.to_numpy().ravel()[1:], "Add + ReLU, unaligned " + kind)
+
+
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("case", [
     (2, 3, 8, 8, (2, 2), (2, 2), (0, 0)),
