@@ -1576,6 +1576,11 @@ int conv_half(sgh_conv_geom *g, int which, const uint16_t *a, const uint16_t *b,
   else sgh_prelaid_clear_if_overlap(g, workspace, ws_bytes);
   // the gradients and the forward pass (strides 1 and 2) run on the 16-bit matrix instructions where
   // conv16.hip covers the geometry; everything else computes in fp32 on widened copies
+  if (which == SGH_CONV_FWD && !sgh_env().conv16_off && !sgh_env().fwd_fewc16_off) {   // the stem
+    const int rc = sgh_fwd_fewc16_run(g, a, b, bias, out, workspace, ws_bytes, in == sgh_cast_bf16_to_f32,
+                                      sgh_stream_of(stream));
+    if (rc != SGH_EUNSUPPORTED) return rc;
+  }
   if (sgh_conv16_workspace_bytes(g, which) != 0 && !sgh_env().conv16_off) {
     const bool bf16 = in == sgh_cast_bf16_to_f32;
     hipStream_t s = sgh_stream_of(stream);
@@ -1642,7 +1647,8 @@ size_t sgh_conv_workspace_bytes_h(const sgh_conv_geom *g, int which) {
     return p.x_bytes + p.y_bytes + sgh_conv_workspace_bytes_h(&p.sg, which);
   }
   const size_t wide = half_plan(g, which).total() + (which == SGH_CONV_FWD ? align256(size_t(g->K) * 4) : 0);
-  const size_t native = sgh_conv16_workspace_bytes(g, which);
+  size_t native = sgh_conv16_workspace_bytes(g, which);
+  if (which == SGH_CONV_FWD && sgh_fwd_fewc16_workspace_bytes(g) > native) native = sgh_fwd_fewc16_workspace_bytes(g);
   return wide > native ? wide : native;
 }
 

@@ -324,6 +324,32 @@ def test_conv_16bit_storage(singa, dev, kind, case):
         assert nl2(db.to_numpy(), O.conv_bgrad(dy)) < 1e-2
 
 
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("case", [
+    # N, C, H = W, bias: the stem's forward kernel (7 x 7, stride 2, padding 3, 64 filters) at its four widths
+    (3, 3, 32, True), (2, 1, 64, False), (2, 2, 128, True), (1, 3, 224, False),
+])
+def test_stem_forward_16bit(singa, dev, kind, case):
+    """Forward convolution of the stem geometry on 16-bit tensors against the fp32 oracle on the same stored
+    inputs (1e-2 normalised L2 as for every 16-bit convolution; the rounding of the result alone is about 3e-4
+    for binary16 and 2e-3 for bfloat16, and the bound asserted here is 4e-3), borders included: every output
+    row and column whose window reaches outside the image is compared on its own."""
+    from oracle import cpu_oracle as O
+    from util import nl2
+    N, C, H, bias = case
+    r = rng(H + 7 * C)
+    xt, x = _to(singa, dev, r.standard_normal((N, C, H, H)).astype(np.float32), kind)
+    wt, w = _to(singa, dev, (r.standard_normal((64, C, 7, 7)) * np.sqrt(2.0 / (C * 49))).astype(np.float32), kind)
+    bt, b = _to(singa, dev, r.standard_normal(64).astype(np.float32), kind) if bias else (None, None)
+    h = singa.CudnnConvHandle(xt, (7, 7), (2, 2), (3, 3), C, 64, bias)
+    y = singa.GpuConvForward(xt, wt, bt, h).to_numpy()
+    want = O.conv_fwd(x, w, b, (2, 2), (3, 3))
+    assert y.shape == want.shape == (N, 64, H // 2, H // 2)
+    assert nl2(y, want) < 4e-3
+    for sl in (np.s_[:, :, :2, :], np.s_[:, :, -2:, :], np.s_[:, :, :, :2], np.s_[:, :, :, -2:]):
+        assert nl2(y[sl], want[sl]) < 4e-3
+
+
 def _grad16_cases(count, seed):
     """Seeded geometries for the 16-bit matrix-instruction gradient kernels: output rows of 1..3
     octets with partly empty last octets, odd and even widths (paired and single-pixel gradient
