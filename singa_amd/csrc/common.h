@@ -32,7 +32,7 @@ static inline bool sgh_aligned16(const void *p) { return (reinterpret_cast<uintp
 // when the first entry point asks: changing the environment later has no effect, so a geometry's
 // workspace size and kernel choice cannot change between two calls.
 struct sgh_env_switches {
-  bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off, bn_onchip_off, pw_dgrad_off, pw_wgrad_off, dgrad_fewc16_off, slab16_off, bn_ragged_off, fwd_fewc16_off;
+  bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off, bn_onchip_off, pw_dgrad_off, pw_wgrad_off, dgrad_fewc16_off, slab16_off, bn_ragged_off, fwd_fewc_off;
   int dgrad_tile, wgrad_tile, pw_tile;   // -1: chosen from the geometry
   int dgrad3x3_bm;              // 0: chosen from the geometry, else 64 or 128
 };
@@ -132,6 +132,12 @@ int sgh_conv16_dgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
 // otherwise the destination layout [tap][CP][KP] (sgh_conv16_dgrad skips its re-layout when told that the
 // workspace already holds it).
 bool sgh_conv16_dgrad_relayout_dims(const sgh_conv_geom *g, int *CP, int *KP);
+// The stem's forward convolution in fp32 (7 x 7, stride 2, padding 3, up to 3 input channels, 64 filters):
+// fwd_fewc.hip.  SGH_EUNSUPPORTED for every other geometry.
+bool sgh_fwd_fewc_supported(const sgh_conv_geom *g);
+size_t sgh_fwd_fewc_workspace_bytes(const sgh_conv_geom *g);
+int sgh_fwd_fewc_run(const sgh_conv_geom *g, const float *x, const float *W, const float *bias, float *y, void *workspace,
+                     size_t ws_bytes, hipStream_t s);
 // The stem's forward convolution on 16-bit tensors (7 x 7, stride 2, padding 3, up to 3 input channels, 64 filters):
 // fwd_fewc16.hip.  SGH_EUNSUPPORTED for every other geometry.
 bool sgh_fwd_fewc16_supported(const sgh_conv_geom *g);

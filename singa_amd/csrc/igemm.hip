@@ -1013,7 +1013,8 @@ size_t sgh_conv_workspace_bytes(const sgh_conv_geom *g, int which) {
     case SGH_CONV_FWD: {
       sgh_conv_geom gt;
       const size_t wt = RS * round_up(g->C, BK) * g->K * sizeof(float);
-      return fwd_as_dgrad(g, &gt) ? align256(wt) + sgh_dgrad3x3_partial_bytes(&gt) : wt;
+      const size_t need = fwd_as_dgrad(g, &gt) ? align256(wt) + sgh_dgrad3x3_partial_bytes(&gt) : wt;
+      return need > sgh_fwd_fewc_workspace_bytes(g) ? need : sgh_fwd_fewc_workspace_bytes(g);
     }
     case SGH_CONV_DGRAD:
       if (dgrad_path(g) == kDgradFewC) return sgh_dgrad_fewc_workspace_bytes(g);
@@ -1362,6 +1363,13 @@ int sgh_conv_fwd_f32(sgh_conv_geom *g, const float *x, const float *W, const flo
   float *Wt = static_cast<float *>(workspace);
   const int RS = g->R * g->S, CP = round_up(g->C, BK);
   sgh_prof_start("conv_fwd_op", conv_flops(g), s);
+  if (!sgh_env().fwd_fewc_off) {   // the stem
+    const int rcf = sgh_fwd_fewc_run(g, x, W, bias, y, workspace, ws_bytes, s);
+    if (rcf != SGH_EUNSUPPORTED) {
+      sgh_prof_stop(s);
+      return rcf;
+    }
+  }
   sgh_conv_geom gt;
   if (fwd_as_dgrad(g, &gt)) {
     // 3x3 stride 1 pad 1: the shared-tile kernel on the channel-swapped problem with reversed taps
@@ -1576,7 +1584,7 @@ int conv_half(sgh_conv_geom *g, int which, const uint16_t *a, const uint16_t *b,
   else sgh_prelaid_clear_if_overlap(g, workspace, ws_bytes);
   // the gradients and the forward pass (strides 1 and 2) run on the 16-bit matrix instructions where
   // conv16.hip covers the geometry; everything else computes in fp32 on widened copies
-  if (which == SGH_CONV_FWD && !sgh_env().conv16_off && !sgh_env().fwd_fewc16_off) {   // the stem
+  if (which == SGH_CONV_FWD && !sgh_env().conv16_off && !sgh_env().fwd_fewc_off) {   // the stem
     const int rc = sgh_fwd_fewc16_run(g, a, b, bias, out, workspace, ws_bytes, in == sgh_cast_bf16_to_f32,
                                       sgh_stream_of(stream));
     if (rc != SGH_EUNSUPPORTED) return rc;

@@ -459,6 +459,38 @@ def test_avg_pool_bit_exact(singa, dev, case):
     assert_bit_equal(dx, O.pool_avg_bwd(dy, x.shape, kernel, stride, pad, include_pad=False), "avg-pool backward")
 
 
+@pytest.mark.parametrize("case", [
+    # N, C, H = W, bias: the stem's forward kernel (7 x 7, stride 2, padding 3, 64 filters) at its four widths
+    (3, 3, 32, True), (2, 1, 64, False), (2, 2, 128, True), (1, 3, 224, False),
+])
+def test_stem_forward_fp32(singa, dev, case):
+    """Forward convolution of the stem geometry against the CPU oracle (1e-3 normalised L2 as for every fp32
+    convolution; asserted here: 1e-5), the border rows and columns on their own, and an infinity next to a
+    window staying out of it."""
+    N, C, H, bias = case
+    r = rng(H + 7 * C)
+    x = randn(r, N, C, H, H)
+    w = (randn(r, 64, C, 7, 7) * np.sqrt(2.0 / (C * 49))).astype(np.float32)
+    b = randn(r, 64) if bias else None
+    xd, wd = singa.from_numpy(x, dev), singa.from_numpy(w, dev)
+    bd = singa.from_numpy(b, dev) if bias else None
+    h = singa.CudnnConvHandle(xd, (7, 7), (2, 2), (3, 3), C, 64, bias)
+    y = singa.GpuConvForward(xd, wd, bd, h).to_numpy()
+    want = O.conv_fwd(x, w, b, (2, 2), (3, 3))
+    assert y.shape == want.shape == (N, 64, H // 2, H // 2)
+    assert nl2(y, want) < 1e-5
+    for sl in (np.s_[:, :, :2, :], np.s_[:, :, -2:, :], np.s_[:, :, :, :2], np.s_[:, :, :, -2:]):
+        assert nl2(y[sl], want[sl]) < 1e-5
+    # window (p, q) covers rows 2 p - 3 .. 2 p + 3 and columns 2 q - 3 .. 2 q + 3: an infinity at (9, 12) belongs to
+    # the windows p = 3..6, q = 5..7 and to no other (column 12 is the one in front of window q = 8)
+    x2 = x.copy()
+    x2[0, 0, 9, 12] = np.inf
+    y2 = singa.GpuConvForward(singa.from_numpy(x2, dev), wd, bd, h).to_numpy()
+    hit = np.zeros(y2.shape, bool)
+    hit[0, :, 3:7, 5:8] = True
+    assert not np.isfinite(y2[hit]).any() and np.isfinite(y2[~hit]).all()
+
+
 # ---------------------------------------------------------------------------------- batch norm
 
 def test_bn_reference_vectors(singa, dev, golden):
