@@ -741,6 +741,164 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
 #undef BN_CHIP_FINISH
 }
 
+// ---- forward (training) in one pass, the same way: a slice of x stays in registers (more vectors than in the
+// backward kernel, there is only one tensor) from the sums to the normalisation, the G workgroups of a channel
+// exchange (sum (x - pivot), sum (x - pivot)^2) through the tagged words described above and finish the
+// statistics in double precision in slice order, like k_bn_fwd_apply does over its splits.  x is read once and
+// y written once: 2 tensor passes instead of 3.
+// vectors per thread: what stays clear of register spills beside the double-precision statistics
+template <class S>
+constexpr int chip_fwd_nv() { return sizeof(typename S::elem) == 4 ? 12 : (S::VEC == 8 ? 8 : 12); }
+
+template <class S>
+inline ChipPlan chip_fwd_plan(int N, int C, int HW) {
+  ChipPlan p{false, 0, 0, 512, 0, false};
+  if (HW % S::VEC != 0) return p;
+  const long TV = long(N) * (HW / S::VEC);
+  const long per_wg = 512L * chip_fwd_nv<S>();
+  long G = (TV + per_wg - 1) / per_wg;
+  const long want = (2L * sgh_num_cus() + C - 1) / C;   // few channels: thinner slices, two workgroups for every CU
+  if (G < want) G = want;
+  const long slots = 2L * sgh_num_cus(), rounds = (long(C) * G + slots - 1) / slots;
+  long fill = rounds * slots / C;                       // whole rounds
+  if (fill > kChipMaxG) fill = kChipMaxG;
+  if (fill > G) G = fill;
+  while (G > 1 && (TV + G - 1) / G < 64) --G;
+  if (G > kChipMaxG || G < 1) return p;
+  p.vpg = int((TV + G - 1) / G);
+  p.G = int((TV + p.vpg - 1) / p.vpg);
+  p.ok = long(C) * p.G < 0x7fffffffL;
+  return p;
+}
+
+template <class S, bool RELU>
+__global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem *__restrict__ x,
+                                                           const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                           float *__restrict__ running_mean, float *__restrict__ running_var,
+                                                           float factor, float eps, typename S::elem *__restrict__ y,
+                                                           float *__restrict__ save_mean, float *__restrict__ save_invstd,
+                                                           unsigned long long *__restrict__ ws, BnShape s, int G, int vpg,
+                                                           unsigned long long ticket1, unsigned long long ticket2,
+                                                           int spin_limit, int xcd_runs) {
+  typedef typename S::elem elem;
+  constexpr int V = S::VEC, NV = chip_fwd_nv<S>(), NT = 512;
+  typedef typename RawVec<V * sizeof(elem)>::type raw;
+  __shared__ float red[16];
+  __shared__ float part_a[kChipMaxG], part_b[kChipMaxG];
+  __shared__ int gave_up;
+  __shared__ unsigned long long ticket_s;
+  const int unit = xcd_runs ? int(blockIdx.x & 7) * int(gridDim.x >> 3) + int(blockIdx.x >> 3) : int(blockIdx.x);
+  const int c = unit / G, g = unit - c * G, t = threadIdx.x;
+  if (c >= s.C) return;
+  unsigned long long *words = ws + size_t(c) * 2 * size_t(G);   // the channel's G slots
+  if (G > 1 && t == 0) {
+    const unsigned long long wa = __hip_atomic_load(words + 2 * g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long wb = __hip_atomic_load(words + 2 * g + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ticket_s = (unsigned(wa) == unsigned(ticket1) && unsigned(wb) == unsigned(ticket1 >> 32)) ? ticket2 : ticket1;
+    gave_up = 0;
+  }
+  const int PV = s.HW / V, TV = s.N * PV;
+  const int lo = g * vpg, hi = min(lo + vpg, TV);
+  const float pivot = S::ld(x + size_t(c) * s.HW);
+  const raw *xg = reinterpret_cast<const raw *>(x);
+  raw xv[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int iv = lo + i * NT + t;
+    if (iv < hi) {
+      const int n = iv / PV, r = iv - n * PV;
+      xv[i] = __builtin_nontemporal_load(xg + (size_t(n) * s.C + c) * PV + r);
+    }
+  }
+  float a = 0.f, b = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+    if (lo + i * NT + t < hi) {
+      float v[V];
+      S::template load16<false>(reinterpret_cast<const elem *>(&xv[i]), v);
+#pragma unroll
+      for (int q = 0; q < V; q += 4) {
+        const float d0 = v[q] - pivot, d1 = v[q + 1] - pivot, d2 = v[q + 2] - pivot, d3 = v[q + 3] - pivot;
+        a += (d0 + d1) + (d2 + d3);
+        b += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+      }
+    }
+  a = sgh_block_sum(a, red);
+  b = sgh_block_sum(b, red);
+  double A = a, B = b;
+  if (G > 1) {
+    // (the block sums above contain barriers: ticket_s and gave_up are visible to every thread)
+    const unsigned long long ticket = ticket_s;
+    const unsigned lo32 = unsigned(ticket), hi32 = unsigned(ticket >> 32);   // (both halves are nonzero)
+    if (t == 0) {
+      __hip_atomic_store(words + 2 * g, (static_cast<unsigned long long>(__float_as_uint(a)) << 32) | lo32,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(words + 2 * g + 1, (static_cast<unsigned long long>(__float_as_uint(b)) << 32) | hi32,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (t < G) {   // one lane per slice of the channel polls that slice's words
+      unsigned long long wa = 0, wb = 0;
+      int spins = 0;
+      bool have_b = false;
+      for (;;) {
+        if (!have_b) {
+          wb = __hip_atomic_load(words + 2 * t + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          have_b = unsigned(wb) == hi32;
+        }
+        if (have_b) {
+          wa = __hip_atomic_load(words + 2 * t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (unsigned(wa) == lo32) break;
+        }
+        if (++spins >= spin_limit) {
+          gave_up = 1;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+      part_a[t] = __uint_as_float(unsigned(wa >> 32));
+      part_b[t] = __uint_as_float(unsigned(wb >> 32));
+    }
+    __syncthreads();
+    A = 0, B = 0;
+    for (int i = 0; i < G; ++i) A += part_a[i], B += part_b[i];   // the same numbers in the same order in every slice
+  }
+  const double M = double(s.N) * s.HW;
+  const double dm = A / M;
+  double var = B / M - dm * dm;
+  if (var < 0) var = 0;
+  float mean = float(double(pivot) + dm);
+  const float invstd = float(1.0 / sqrt(var + double(eps)));
+  if (G > 1 && gave_up) mean = __builtin_nanf("");
+  if (g == 0 && t == 0) {
+    save_mean[c] = mean;
+    save_invstd[c] = invstd;
+    if (running_mean) running_mean[c] = (1.f - factor) * running_mean[c] + factor * mean;
+    if (running_var) {
+      const double unb = M > 1 ? var * M / (M - 1) : var;
+      running_var[c] = (1.f - factor) * running_var[c] + factor * float(unb);
+    }
+  }
+  const float gm = gamma[c], be = beta[c];
+  raw *og = reinterpret_cast<raw *>(y);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int iv = lo + i * NT + t;
+    if (iv < hi) {
+      const int n = iv / PV, r = iv - n * PV;
+      float v[V], o[V];
+      S::template load16<false>(reinterpret_cast<const elem *>(&xv[i]), v);
+#pragma unroll
+      for (int q = 0; q < V; ++q) {
+        o[q] = bn_out_rounded(v[q], mean, invstd, gm, be);
+        if (RELU) o[q] = bn_relu_value<S>(o[q]);
+      }
+      raw ov;
+      S::store16(reinterpret_cast<elem *>(&ov), o);
+      og[(size_t(n) * s.C + c) * PV + r] = ov;
+    }
+  }
+}
+
 // tickets: a random 64-bit start (so that whatever an uninitialised workspace holds is not the next
 // ticket, up to a chance of 2^-64 per slot) and one step per call
 inline unsigned long long next_ticket() {
@@ -752,6 +910,19 @@ inline unsigned long long next_ticket() {
   do v = t.fetch_add(0x9e3779b97f4a7c15ull | 1ull, std::memory_order_relaxed);
   while (unsigned(v) == 0 || unsigned(v >> 32) == 0);   // a zeroed word must never look valid
   return v;
+}
+
+template <class S, bool RELU>
+int launch_fwd_onchip(const typename S::elem *x, const float *gamma, const float *beta, float *running_mean,
+                      float *running_var, float factor, float eps, typename S::elem *y, float *save_mean,
+                      float *save_invstd, void *workspace, const BnShape &s, const ChipPlan &p, hipStream_t st) {
+  const int xcd_runs = p.G <= 16 && s.C >= 8 ? 1 : 0;
+  const dim3 grid(xcd_runs ? unsigned((s.C + 7) / 8) * 8u * p.G : unsigned(s.C) * p.G);
+  const unsigned long long t1 = next_ticket(), t2 = next_ticket();
+  hipLaunchKernelGGL((k_bn_fwd_onchip<S, RELU>), grid, dim3(512), 0, st, x, gamma, beta, running_mean, running_var, factor,
+                     eps, y, save_mean, save_invstd, static_cast<unsigned long long *>(workspace), s, p.G, p.vpg, t1, t2,
+                     kChipSpinLimit, xcd_runs);
+  return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
 template <class S, bool RELU>
@@ -852,6 +1023,13 @@ int bn_fwd_train(const typename S::elem *x, const float *gamma, const float *bet
   const BnShape s = make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem)));
   if (!sgh_aligned16(x) || !sgh_aligned16(y)) return SGH_EINVAL;
   if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
+  const ChipPlan fp = chip_fwd_plan<S>(N, C, HW);
+  if (fp.ok && !sgh_env().bn_onchip_off && !sgh_env().bn_fwd_onchip_off && sgh_aligned16(workspace) &&
+      ws_bytes >= chip_workspace_bytes(C, fp.G))
+    return relu ? launch_fwd_onchip<S, true>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean,
+                                             save_invstd, workspace, s, fp, sgh_stream_of(stream))
+                : launch_fwd_onchip<S, false>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean,
+                                              save_invstd, workspace, s, fp, sgh_stream_of(stream));
   float *scratch = static_cast<float *>(workspace);
   hipLaunchKernelGGL(k_bn_fwd_partial<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, scratch, s);
   SGH_LAUNCH_CHECK();
@@ -973,6 +1151,9 @@ size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
   const size_t b[3] = {bwd_workspace_need<StF32>(N, C, HW), bwd_workspace_need<StF16>(N, C, HW),
                        bwd_workspace_need<StF16x4>(N, C, HW)};
   for (size_t v : b) need = v > need ? v : need;
+  const ChipPlan f[3] = {chip_fwd_plan<StF32>(N, C, HW), chip_fwd_plan<StF16>(N, C, HW), chip_fwd_plan<StF16x4>(N, C, HW)};
+  for (const ChipPlan &p : f)
+    if (p.ok && chip_workspace_bytes(C, p.G) > need) need = chip_workspace_bytes(C, p.G);
   return need;
 }
 

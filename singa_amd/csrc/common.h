@@ -32,7 +32,7 @@ static inline bool sgh_aligned16(const void *p) { return (reinterpret_cast<uintp
 // when the first entry point asks: changing the environment later has no effect, so a geometry's
 // workspace size and kernel choice cannot change between two calls.
 struct sgh_env_switches {
-  bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off, bn_onchip_off, pw_dgrad_off, pw_wgrad_off, dgrad_fewc16_off, slab16_off, bn_ragged_off, fwd_fewc_off;
+  bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off, bn_onchip_off, pw_dgrad_off, pw_wgrad_off, dgrad_fewc16_off, slab16_off, bn_ragged_off, fwd_fewc_off, bn_fwd_onchip_off;
   int dgrad_tile, wgrad_tile, pw_tile;   // -1: chosen from the geometry
   int dgrad3x3_bm;              // 0: chosen from the geometry, else 64 or 128
 };

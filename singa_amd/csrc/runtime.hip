@@ -97,7 +97,7 @@ const sgh_env_switches &sgh_env() {
     s.dgrad3x3_off = on("SGH_DGRAD3X3_OFF"), s.wgrad3x3_off = on("SGH_WGRAD3X3_OFF");
     s.dgrad_fewc_off = on("SGH_DGRAD_FEWC_OFF"), s.wgrad_fewc_off = on("SGH_WGRAD_FEWC_OFF");
     s.dgrad_pointwise_off = on("SGH_DGRAD_POINTWISE_OFF"), s.conv16_off = on("SGH_CONV16_OFF");
-    s.bn_ragged_off = on("SGH_BN_RAGGED_OFF"), s.fwd_fewc_off = on("SGH_FWD_FEWC_OFF"), s.bn_onchip_off = on("SGH_BN_ONCHIP_OFF"), s.pw_dgrad_off = on("SGH_PW_DGRAD_OFF");
+    s.bn_ragged_off = on("SGH_BN_RAGGED_OFF"), s.fwd_fewc_off = on("SGH_FWD_FEWC_OFF"), s.bn_fwd_onchip_off = on("SGH_BN_FWD_ONCHIP_OFF"), s.bn_onchip_off = on("SGH_BN_ONCHIP_OFF"), s.pw_dgrad_off = on("SGH_PW_DGRAD_OFF");
     s.pw_wgrad_off = on("SGH_PW_WGRAD_OFF"), s.dgrad_fewc16_off = on("SGH_DGRAD_FEWC16_OFF");
     s.slab16_off = on("SGH_SLAB16_OFF");
     s.dgrad_tile = num("SGH_DGRAD_TILE", 0, 3), s.wgrad_tile = num("SGH_WGRAD_TILE", 0, 5);
