@@ -52,6 +52,44 @@ __global__ __launch_bounds__(kBlock) void k_pool_max_fwd(const typename S::elem 
   }
 }
 
+// The residual networks' pooling layer (3 x 3, stride 2, padding 1, even image, Q a multiple of the vector
+// length): a thread produces one vector of outputs from two vectors and one element of each of its three input
+// rows, comparing in the order of window_argmax (rows top to bottom, columns left to right, strict '>').
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_pool_max_fwd_3x3s2(const typename S::elem *__restrict__ x,
+                                                              typename S::elem *__restrict__ y, int H, int W, size_t nvec) {
+  constexpr int V = S::VEC;
+  const int P = H >> 1, Q = W >> 1, QV = Q / V;
+  const float none = -__builtin_inff();   // (never greater than anything: a position outside the image)
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  for (size_t iv = size_t(blockIdx.x) * kBlock + threadIdx.x; iv < nvec; iv += stride) {
+    const size_t pr = iv / QV;              // plane * P + p
+    const int qv = int(iv - pr * QV), q = qv * V;
+    const size_t plane = pr / P;
+    const int p = int(pr - plane * P);
+    const typename S::elem *xb = x + plane * size_t(H) * W;
+    float best[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) best[j] = -3.402823466e38f;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      const int h = 2 * p - 1 + r;
+      if (h < 0) continue;                  // (h <= H - 1 always: H is even)
+      const typename S::elem *row = xb + size_t(h) * W + 2 * q;
+      float e[2 * V + 1];
+      e[0] = q > 0 ? S::ld(row - 1) : none;
+      S::template load16<false>(row, e + 1);
+      S::template load16<false>(row + V, e + 1 + V);
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+#pragma unroll
+        for (int c = 0; c < 3; ++c)
+          if (e[2 * j + c] > best[j]) best[j] = e[2 * j + c];
+    }
+    S::store16(y + (pr * size_t(Q)) + q, best);
+  }
+}
+
 template <class S>
 __global__ __launch_bounds__(kBlock) void k_pool_max_bwd(const typename S::elem *__restrict__ dy,
                                                         const typename S::elem *__restrict__ x,
@@ -489,7 +527,11 @@ template <class S>
 int pool_fwd(const sgh_pool_geom *g, const typename S::elem *x, typename S::elem *y, void *stream) {
   if (!geom_ok(g) || !x || !y) return SGH_EINVAL;
   const size_t total = size_t(g->N) * g->C * g->P * g->Q;
-  if (g->is_max)
+  if (g->is_max && g->kernel_h == 3 && g->kernel_w == 3 && g->stride_h == 2 && g->stride_w == 2 && g->pad_h == 1 &&
+      g->pad_w == 1 && g->H % 2 == 0 && g->W % 2 == 0 && g->Q % S::VEC == 0 && sgh_aligned16(x) && sgh_aligned16(y))
+    hipLaunchKernelGGL(k_pool_max_fwd_3x3s2<S>, dim3(grid_for(total / S::VEC)), dim3(kBlock), 0, sgh_stream_of(stream), x, y,
+                       g->H, g->W, total / S::VEC);
+  else if (g->is_max)
     hipLaunchKernelGGL(k_pool_max_fwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), x, y, to_g(g),
                        total);
   else
