@@ -1392,15 +1392,25 @@ int sgh_conv_fwd_f32(sgh_conv_geom *g, const float *x, const float *W, const flo
   const int M = g->K, Ncols = g->N * g->P * g->Q, Ktot = RS * CP;
   const int chunks = Ktot / BK;
   NchwStore st{y, bias, g->K, g->P * g->Q, Ncols};
-  auto lb = gather_loader<128, false>(x, to_g(g), CP, g->C, g->H, g->W, Ncols);
   int rc;
-  if (M > 64) {
+  // the largest tile that still gives every CU a workgroup (the late, small layers: 98 tiles of 128 x 128 at
+  // 512 filters on 7 x 7 planes, N = 64)
+  const long cus = sgh_num_cus();
+  const long t128 = long((M + 127) / 128) * ((Ncols + 127) / 128), t64x128 = long((M + 63) / 64) * ((Ncols + 127) / 128);
+  if (M > 64 && t128 >= cus) {
     auto la = dense_loader<128, false>(Wt, 1, g->K, M, Ktot);
+    auto lb = gather_loader<128, false>(x, to_g(g), CP, g->C, g->H, g->W, Ncols);
     rc = launch_igemm<128, 128, DenseLoader<128, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
+        la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd/k_igemm", conv_flops(g));
+  } else if (M <= 64 || t64x128 >= cus) {
+    auto la = dense_loader<64, false>(Wt, 1, g->K, M, Ktot);
+    auto lb = gather_loader<128, false>(x, to_g(g), CP, g->C, g->H, g->W, Ncols);
+    rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
         la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd/k_igemm", conv_flops(g));
   } else {
     auto la = dense_loader<64, false>(Wt, 1, g->K, M, Ktot);
-    rc = launch_igemm<64, 128, DenseLoader<64, false>, PixelGatherLoader<128, false>, NchwStore, false, false>(
+    auto lb = gather_loader<64, false>(x, to_g(g), CP, g->C, g->H, g->W, Ncols);
+    rc = launch_igemm<64, 64, DenseLoader<64, false>, PixelGatherLoader<64, false>, NchwStore, false, false, false, 2, 4>(
         la, lb, st, M, Ncols, Ktot, 1, chunks, s, "conv_fwd/k_igemm", conv_flops(g));
   }
   sgh_prof_stop(s);
