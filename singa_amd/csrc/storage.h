@@ -23,10 +23,10 @@ __device__ __forceinline__ uint16_t sgh_f32_to_f16(float f) {
 }
 __device__ __forceinline__ float sgh_bf16_to_f32(uint16_t b) { return __builtin_bit_cast(float, unsigned(b) << 16); }
 __device__ __forceinline__ uint16_t sgh_f32_to_bf16(float f) {
-  unsigned u = __builtin_bit_cast(unsigned, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40u);  // NaN stays a (quiet) NaN
-  u += 0x7fffu + ((u >> 16) & 1u);                                          // round to nearest even
-  return uint16_t(u >> 16);
+  const __bf16 h = __bf16(f);  // v_cvt_pk_bf16_f32: round to nearest even, NaN stays a (quiet) NaN
+  uint16_t b;
+  __builtin_memcpy(&b, &h, 2);
+  return b;
 }
 
 struct StF32 {
