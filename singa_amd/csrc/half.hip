@@ -23,11 +23,13 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 struct F16 {
   static __device__ __forceinline__ float load(u16 b) { return sgh_f16_to_f32(b); }
   static __device__ __forceinline__ u16 store(float f) { return sgh_f32_to_f16(f); }
+  static __device__ __forceinline__ unsigned pack2(float lo, float hi) { return sgh_pack2_f16(lo, hi); }
 };
 
 struct BF16 {
   static __device__ __forceinline__ float load(u16 b) { return sgh_bf16_to_f32(b); }
   static __device__ __forceinline__ u16 store(float f) { return sgh_f32_to_bf16(f); }
+  static __device__ __forceinline__ unsigned pack2(float lo, float hi) { return sgh_pack2_bf16(lo, hi); }
 };
 
 inline int grid_for(size_t nvec) {
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(kBlock) void k_map2_h(const u16 *a, const u16 *b, u
           for (int j = 0; j < 4; ++j) {
             const float lo = f(T::load(u16(va[u][j] & 0xffffu)), T::load(u16(vb[u][j] & 0xffffu)));
             const float hi = f(T::load(u16(va[u][j] >> 16)), T::load(u16(vb[u][j] >> 16)));
-            r[j] = unsigned(T::store(lo)) | (unsigned(T::store(hi)) << 16);
+            r[j] = T::pack2(lo, hi);
           }
           o4[i] = r;
         }
@@ -187,10 +189,10 @@ __global__ __launch_bounds__(kBlock) void k_cast_to16(const float *__restrict__ 
     for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += stride) {
       const float4 x0 = s4[2 * i], x1 = s4[2 * i + 1];
       v4u r;
-      r[0] = unsigned(T::store(x0.x)) | (unsigned(T::store(x0.y)) << 16);
-      r[1] = unsigned(T::store(x0.z)) | (unsigned(T::store(x0.w)) << 16);
-      r[2] = unsigned(T::store(x1.x)) | (unsigned(T::store(x1.y)) << 16);
-      r[3] = unsigned(T::store(x1.z)) | (unsigned(T::store(x1.w)) << 16);
+      r[0] = T::pack2(x0.x, x0.y);
+      r[1] = T::pack2(x0.z, x0.w);
+      r[2] = T::pack2(x1.x, x1.y);
+      r[3] = T::pack2(x1.z, x1.w);
       d4[i] = r;
     }
     if (blockIdx.x == 0) {

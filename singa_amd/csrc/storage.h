@@ -29,6 +29,20 @@ __device__ __forceinline__ uint16_t sgh_f32_to_bf16(float f) {
   return b;
 }
 
+// two results rounded and packed into a dword (low half first) by one instruction: v_cvt_pk_f16_f32 /
+// v_cvt_pk_bf16_f32, the same roundings as the single conversions above
+typedef float sgh_v2f __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned sgh_pack2_f16(float lo, float hi) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  const h2 h = __builtin_convertvector(sgh_v2f{lo, hi}, h2);
+  return __builtin_bit_cast(unsigned, h);
+}
+__device__ __forceinline__ unsigned sgh_pack2_bf16(float lo, float hi) {
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  const b2 h = __builtin_convertvector(sgh_v2f{lo, hi}, b2);
+  return __builtin_bit_cast(unsigned, h);
+}
+
 struct StF32 {
   typedef float elem;
   static constexpr int VEC = 4;
@@ -76,7 +90,11 @@ struct St16 {
     typedef unsigned int vec __attribute__((ext_vector_type(VEC / 2)));
     vec r;
 #pragma unroll
-    for (int j = 0; j < VEC / 2; ++j) r[j] = unsigned(ST(in[2 * j])) | (unsigned(ST(in[2 * j + 1])) << 16);
+    for (int j = 0; j < VEC / 2; ++j) {
+      if constexpr (ST == sgh_f32_to_f16) r[j] = sgh_pack2_f16(in[2 * j], in[2 * j + 1]);
+      else if constexpr (ST == sgh_f32_to_bf16) r[j] = sgh_pack2_bf16(in[2 * j], in[2 * j + 1]);
+      else r[j] = unsigned(ST(in[2 * j])) | (unsigned(ST(in[2 * j + 1])) << 16);
+    }
     *reinterpret_cast<vec *>(p) = r;
   }
 };
