@@ -134,11 +134,9 @@ __global__ __launch_bounds__(kNT) void k_fwd_fewc16(FwArgs a) {
     uint16_t *row = a.y + ((size_t(n) * kFilters + k) * a.P + p) * a.Q + 4 * g;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      uint16_t h[4];
-#pragma unroll
-      for (int v = 0; v < 4; ++v) h[v] = BF16 ? sgh_f32_to_bf16(acc[b][m][v] + bb) : sgh_f32_to_f16(acc[b][m][v] + bb);
-      *reinterpret_cast<u32x2 *>(row + 16 * b) =
-          u32x2{unsigned(h[0]) | (unsigned(h[1]) << 16), unsigned(h[2]) | (unsigned(h[3]) << 16)};
+      const f32x4 r = acc[b][m] + bb;
+      *reinterpret_cast<u32x2 *>(row + 16 * b) = BF16 ? u32x2{sgh_pack2_bf16(r[0], r[1]), sgh_pack2_bf16(r[2], r[3])}
+                                                      : u32x2{sgh_pack2_f16(r[0], r[1]), sgh_pack2_f16(r[2], r[3])};
     }
   }
 }
@@ -148,9 +146,10 @@ int launch(const FwArgs &a, hipStream_t s) {
   auto kern = k_fwd_fewc16<NB, BF16>;
   const size_t lds = (size_t(kFilters) * kWPitch + size_t(a.C) * kRowsIn * (32 * NB + 8)) * sizeof(uint16_t);
   static bool attr = false;
-  if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) !=
-        hipSuccess)
+  if (!attr) {   // (once, for the largest case: three channels)
+    const size_t lds_max = (size_t(kFilters) * kWPitch + size_t(3) * kRowsIn * (32 * NB + 8)) * sizeof(uint16_t);
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            int(lds_max)) != hipSuccess)
       return SGH_EUNSUPPORTED;
     attr = true;
   }
