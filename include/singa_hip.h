@@ -526,6 +526,23 @@ SGH_API int sgh_bn_relu_fwd_train_bf16(const uint16_t *x, const float *gamma, co
                                        float *running_mean, float *running_var, float factor, float eps,
                                        uint16_t *y, float *save_mean, float *save_invstd, int N, int C,
                                        int HW, void *workspace, size_t ws_bytes, void *stream);
+/* The same with the sum that ends a residual block in between: y = relu(BatchNorm(x) + z), the forward of
+ * relu(bn(conv(..)) + identity) (examples/cnn/model/resnet.py:70-77, :108-115) in one call -- the bits that
+ * GpuBatchNormForwardTraining, the tensor addition (autograd.py add) and ReLU store one after the other (BatchNorm
+ * output and sum each rounded to the storage type).  The BatchNorm's own output is not kept: its backward needs
+ * x only, the ReLU's backward gates on y.  z has the shape and type of x. */
+SGH_API int sgh_bn_add_relu_fwd_train_f32(const float *x, const float *z, const float *gamma, const float *beta,
+                                          float *running_mean, float *running_var, float factor, float eps,
+                                          float *y, float *save_mean, float *save_invstd, int N, int C,
+                                          int HW, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_add_relu_fwd_train_f16(const uint16_t *x, const uint16_t *z, const float *gamma, const float *beta,
+                                          float *running_mean, float *running_var, float factor, float eps,
+                                          uint16_t *y, float *save_mean, float *save_invstd, int N, int C,
+                                          int HW, void *workspace, size_t ws_bytes, void *stream);
+SGH_API int sgh_bn_add_relu_fwd_train_bf16(const uint16_t *x, const uint16_t *z, const float *gamma, const float *beta,
+                                           float *running_mean, float *running_var, float factor, float eps,
+                                           uint16_t *y, float *save_mean, float *save_invstd, int N, int C,
+                                           int HW, void *workspace, size_t ws_bytes, void *stream);
 /* GpuBatchNormForwardInference (src/model/operation/batchnorm.cc:331-366):
  * y = gamma * (x - running_mean) / sqrt(running_var + eps) + beta. */
 SGH_API int sgh_bn_fwd_infer_f32(const float *x, const float *gamma, const float *beta,

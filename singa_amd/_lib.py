@@ -167,6 +167,12 @@ SIGNATURES = {
                                        C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_relu_fwd_train_f32": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
                                        C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_add_relu_fwd_train_f32": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
+                                       C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_add_relu_fwd_train_f16": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
+                                       C.c_int, C.c_int, vp, sz, vp]),
+    "sgh_bn_add_relu_fwd_train_bf16": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
+                                       C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_relu_fwd_train_f16": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
                                        C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_relu_fwd_train_bf16": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,

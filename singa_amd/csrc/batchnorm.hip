@@ -149,8 +149,22 @@ __device__ __forceinline__ float bn_relu_value(float y) {
   else return S::stored_positive(y) ? y : 0.f;
 }
 
-template <class S, bool RELU>
+// ACT: what is stored -- 0: y; 1: relu(y); 2: relu(y + z) for a second tensor z (the end of a residual block), with
+// the roundings of the separate calls: y to the storage type, the sum to the storage type, then the selection
+template <class S, int ACT>
+__device__ __forceinline__ float bn_fwd_value(float y, float z) {
+  if constexpr (ACT == 0) return y;
+  else if constexpr (ACT == 1) return bn_relu_value<S>(y);
+  else {
+    const float sum = S::stored(S::stored(y) + z);
+    if constexpr (sizeof(typename S::elem) == 4) return sum >= 0.f ? sum : 0.f;
+    else return sum > 0.f ? sum : 0.f;
+  }
+}
+
+template <class S, int ACT>
 __global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const typename S::elem *__restrict__ x,
+                                                        const typename S::elem *__restrict__ z,
                                                         const float *__restrict__ gamma, const float *__restrict__ beta,
                                                         const float *__restrict__ part, float *__restrict__ running_mean,
                                                         float *__restrict__ running_var, float factor, float eps,
@@ -180,19 +194,17 @@ __global__ __launch_bounds__(kBlock) void k_bn_fwd_apply(const typename S::elem 
   }
   const float g = gamma[c], be = beta[c];
   channel_range<kBlock, S>(
-      s, c, sp * s.per_split, (sp + 1) * s.per_split, x, nullptr,
-      [&](size_t off, const float *v, const float *) {
+      s, c, sp * s.per_split, (sp + 1) * s.per_split, x, ACT == 2 ? z : nullptr,
+      [&](size_t off, const float *v, const float *zv) {
         float r[S::VEC];
 #pragma unroll
-        for (int q = 0; q < S::VEC; ++q) {
-          r[q] = bn_out_rounded(v[q], mean, invstd, g, be);
-          if (RELU) r[q] = bn_relu_value<S>(r[q]);
-        }
+        for (int q = 0; q < S::VEC; ++q)
+          r[q] = bn_fwd_value<S, ACT>(bn_out_rounded(v[q], mean, invstd, g, be), ACT == 2 ? zv[q] : 0.f);
         S::store16(y + off, r);
       },
       [&](size_t off) {
         const float r = bn_out_rounded(S::ld(x + off), mean, invstd, g, be);
-        S::st(y + off, RELU ? bn_relu_value<S>(r) : r);
+        S::st(y + off, bn_fwd_value<S, ACT>(r, ACT == 2 ? S::ld(z + off) : 0.f));
       });
 }
 
@@ -747,15 +759,19 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
 // statistics in double precision in slice order, like k_bn_fwd_apply does over its splits.  x is read once and
 // y written once: 2 tensor passes instead of 3.
 // vectors per thread: what stays clear of register spills beside the double-precision statistics
+// (with a second tensor -- `two`, ACT == 2 in the kernel -- as many vectors of z wait in registers from before the
+// exchange, so fewer of each)
 template <class S>
-constexpr int chip_fwd_nv() { return sizeof(typename S::elem) == 4 ? 12 : (S::VEC == 8 ? 8 : 12); }
+constexpr int chip_fwd_nv(bool two) {
+  return two ? (sizeof(typename S::elem) == 4 ? 7 : (S::VEC == 8 ? 5 : 7)) : (sizeof(typename S::elem) == 4 ? 12 : (S::VEC == 8 ? 8 : 12));
+}
 
 template <class S>
-inline ChipPlan chip_fwd_plan(int N, int C, int HW) {
+inline ChipPlan chip_fwd_plan(int N, int C, int HW, bool two) {
   ChipPlan p{false, 0, 0, 512, 0, false};
   if (HW % S::VEC != 0) return p;
   const long TV = long(N) * (HW / S::VEC);
-  const long per_wg = 512L * chip_fwd_nv<S>();
+  const long per_wg = 512L * chip_fwd_nv<S>(two);
   long G = (TV + per_wg - 1) / per_wg;
   const long want = (2L * sgh_num_cus() + C - 1) / C;   // few channels: thinner slices, two workgroups for every CU
   if (G < want) G = want;
@@ -771,8 +787,9 @@ inline ChipPlan chip_fwd_plan(int N, int C, int HW) {
   return p;
 }
 
-template <class S, bool RELU>
+template <class S, int ACT>
 __global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem *__restrict__ x,
+                                                           const typename S::elem *__restrict__ z,
                                                            const float *__restrict__ gamma, const float *__restrict__ beta,
                                                            float *__restrict__ running_mean, float *__restrict__ running_var,
                                                            float factor, float eps, typename S::elem *__restrict__ y,
@@ -781,7 +798,7 @@ __global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem
                                                            unsigned long long ticket1, unsigned long long ticket2,
                                                            int spin_limit, int xcd_runs) {
   typedef typename S::elem elem;
-  constexpr int V = S::VEC, NV = chip_fwd_nv<S>(), NT = 512;
+  constexpr int V = S::VEC, NV = chip_fwd_nv<S>(ACT == 2), NT = 512;
   typedef typename RawVec<V * sizeof(elem)>::type raw;
   __shared__ float red[16];
   __shared__ float part_a[kChipMaxG], part_b[kChipMaxG];
@@ -823,6 +840,19 @@ __global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem
         b += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
       }
     }
+  // the second tensor's slice is requested now and arrives during the block sums and the exchange
+  raw zr[ACT == 2 ? NV : 1];
+  if constexpr (ACT == 2) {
+    const raw *zg = reinterpret_cast<const raw *>(z);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int iv = lo + i * NT + t;
+      if (iv < hi) {
+        const int n = iv / PV, r = iv - n * PV;
+        zr[i] = __builtin_nontemporal_load(zg + (size_t(n) * s.C + c) * PV + r);
+      }
+    }
+  }
   a = sgh_block_sum(a, red);
   b = sgh_block_sum(b, red);
   double A = a, B = b;
@@ -885,13 +915,12 @@ __global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem
     const int iv = lo + i * NT + t;
     if (iv < hi) {
       const int n = iv / PV, r = iv - n * PV;
-      float v[V], o[V];
+      float v[V], o[V], zv[V];
       S::template load16<false>(reinterpret_cast<const elem *>(&xv[i]), v);
+      if constexpr (ACT == 2) S::template load16<false>(reinterpret_cast<const elem *>(&zr[i]), zv);
 #pragma unroll
-      for (int q = 0; q < V; ++q) {
-        o[q] = bn_out_rounded(v[q], mean, invstd, gm, be);
-        if (RELU) o[q] = bn_relu_value<S>(o[q]);
-      }
+      for (int q = 0; q < V; ++q)
+        o[q] = bn_fwd_value<S, ACT>(bn_out_rounded(v[q], mean, invstd, gm, be), ACT == 2 ? zv[q] : 0.f);
       raw ov;
       S::store16(reinterpret_cast<elem *>(&ov), o);
       og[(size_t(n) * s.C + c) * PV + r] = ov;
@@ -912,14 +941,15 @@ inline unsigned long long next_ticket() {
   return v;
 }
 
-template <class S, bool RELU>
-int launch_fwd_onchip(const typename S::elem *x, const float *gamma, const float *beta, float *running_mean,
+template <class S, int ACT>
+int launch_fwd_onchip(const typename S::elem *x, const typename S::elem *z, const float *gamma, const float *beta,
+                      float *running_mean,
                       float *running_var, float factor, float eps, typename S::elem *y, float *save_mean,
                       float *save_invstd, void *workspace, const BnShape &s, const ChipPlan &p, hipStream_t st) {
   const int xcd_runs = p.G <= 16 && s.C >= 8 ? 1 : 0;
   const dim3 grid(xcd_runs ? unsigned((s.C + 7) / 8) * 8u * p.G : unsigned(s.C) * p.G);
   const unsigned long long t1 = next_ticket(), t2 = next_ticket();
-  hipLaunchKernelGGL((k_bn_fwd_onchip<S, RELU>), grid, dim3(512), 0, st, x, gamma, beta, running_mean, running_var, factor,
+  hipLaunchKernelGGL((k_bn_fwd_onchip<S, ACT>), grid, dim3(512), 0, st, x, z, gamma, beta, running_mean, running_var, factor,
                      eps, y, save_mean, save_invstd, static_cast<unsigned long long *>(workspace), s, p.G, p.vpg, t1, t2,
                      kChipSpinLimit, xcd_runs);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
@@ -1015,32 +1045,47 @@ inline BnShape make_shape(int N, int C, int HW, int vec, int esize) {
   return s;
 }
 
-template <class S>
-int bn_fwd_train(const typename S::elem *x, const float *gamma, const float *beta, float *running_mean,
-                 float *running_var, float factor, float eps, typename S::elem *y, float *save_mean, float *save_invstd,
-                 int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream, bool relu = false) {
+template <class S, int ACT>
+int bn_fwd_train_act(const typename S::elem *x, const typename S::elem *z, const float *gamma, const float *beta,
+                     float *running_mean, float *running_var, float factor, float eps, typename S::elem *y,
+                     float *save_mean, float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes,
+                     void *stream) {
   if (!shape_ok(N, C, HW) || !x || !gamma || !beta || !y || !save_mean || !save_invstd) return SGH_EINVAL;
+  if (ACT == 2 && (!z || !sgh_aligned16(z))) return SGH_EINVAL;
   const BnShape s = make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem)));
   if (!sgh_aligned16(x) || !sgh_aligned16(y)) return SGH_EINVAL;
   if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
-  const ChipPlan fp = chip_fwd_plan<S>(N, C, HW);
+  const ChipPlan fp = chip_fwd_plan<S>(N, C, HW, ACT == 2);
   if (fp.ok && !sgh_env().bn_onchip_off && !sgh_env().bn_fwd_onchip_off && sgh_aligned16(workspace) &&
       ws_bytes >= chip_workspace_bytes(C, fp.G))
-    return relu ? launch_fwd_onchip<S, true>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean,
-                                             save_invstd, workspace, s, fp, sgh_stream_of(stream))
-                : launch_fwd_onchip<S, false>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean,
-                                              save_invstd, workspace, s, fp, sgh_stream_of(stream));
+    return launch_fwd_onchip<S, ACT>(x, z, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd,
+                                     workspace, s, fp, sgh_stream_of(stream));
   float *scratch = static_cast<float *>(workspace);
   hipLaunchKernelGGL(k_bn_fwd_partial<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, scratch, s);
   SGH_LAUNCH_CHECK();
-  if (relu)
-    hipLaunchKernelGGL((k_bn_fwd_apply<S, true>), dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, gamma, beta,
-                       scratch, running_mean, running_var, factor, eps, y, save_mean, save_invstd, s);
-  else
-    hipLaunchKernelGGL((k_bn_fwd_apply<S, false>), dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, gamma, beta,
-                       scratch, running_mean, running_var, factor, eps, y, save_mean, save_invstd, s);
+  hipLaunchKernelGGL((k_bn_fwd_apply<S, ACT>), dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, z, gamma, beta,
+                     scratch, running_mean, running_var, factor, eps, y, save_mean, save_invstd, s);
   SGH_LAUNCH_CHECK();
   return SGH_OK;
+}
+
+// (act: 0 = BatchNorm alone, 1 = + ReLU, 2 = + the second tensor z, then ReLU)
+template <class S>
+int bn_fwd_train(const typename S::elem *x, const float *gamma, const float *beta, float *running_mean,
+                 float *running_var, float factor, float eps, typename S::elem *y, float *save_mean, float *save_invstd,
+                 int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream, int act = 0,
+                 const typename S::elem *z = nullptr) {
+  switch (act) {
+    case 0:
+      return bn_fwd_train_act<S, 0>(x, nullptr, gamma, beta, running_mean, running_var, factor, eps, y, save_mean,
+                                    save_invstd, N, C, HW, workspace, ws_bytes, stream);
+    case 1:
+      return bn_fwd_train_act<S, 1>(x, nullptr, gamma, beta, running_mean, running_var, factor, eps, y, save_mean,
+                                    save_invstd, N, C, HW, workspace, ws_bytes, stream);
+    default:
+      return bn_fwd_train_act<S, 2>(x, z, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd,
+                                    N, C, HW, workspace, ws_bytes, stream);
+  }
 }
 
 template <class S>
@@ -1151,7 +1196,9 @@ size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
   const size_t b[3] = {bwd_workspace_need<StF32>(N, C, HW), bwd_workspace_need<StF16>(N, C, HW),
                        bwd_workspace_need<StF16x4>(N, C, HW)};
   for (size_t v : b) need = v > need ? v : need;
-  const ChipPlan f[3] = {chip_fwd_plan<StF32>(N, C, HW), chip_fwd_plan<StF16>(N, C, HW), chip_fwd_plan<StF16x4>(N, C, HW)};
+  const ChipPlan f[6] = {chip_fwd_plan<StF32>(N, C, HW, false), chip_fwd_plan<StF16>(N, C, HW, false),
+                         chip_fwd_plan<StF16x4>(N, C, HW, false), chip_fwd_plan<StF32>(N, C, HW, true),
+                         chip_fwd_plan<StF16>(N, C, HW, true), chip_fwd_plan<StF16x4>(N, C, HW, true)};
   for (const ChipPlan &p : f)
     if (p.ok && chip_workspace_bytes(C, p.G) > need) need = chip_workspace_bytes(C, p.G);
   return need;
@@ -1188,19 +1235,40 @@ int sgh_bn_relu_fwd_train_f32(const float *x, const float *gamma, const float *b
                               float *running_var, float factor, float eps, float *y, float *save_mean,
                               float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   return bn_fwd_train<StF32>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C, HW,
-                             workspace, ws_bytes, stream, true);
+                             workspace, ws_bytes, stream, 1);
 }
 int sgh_bn_relu_fwd_train_f16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
                               float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
                               float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   return SGH_BN_DISPATCH16(bn_fwd_train, StF16, StF16x4, x, gamma, beta, running_mean, running_var, factor, eps, y,
-                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream, true);
+                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream, 1);
 }
 int sgh_bn_relu_fwd_train_bf16(const uint16_t *x, const float *gamma, const float *beta, float *running_mean,
                                float *running_var, float factor, float eps, uint16_t *y, float *save_mean,
                                float *save_invstd, int N, int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
   return SGH_BN_DISPATCH16(bn_fwd_train, StBF16, StBF16x4, x, gamma, beta, running_mean, running_var, factor, eps, y,
-                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream, true);
+                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream, 1);
+}
+int sgh_bn_add_relu_fwd_train_f32(const float *x, const float *z, const float *gamma, const float *beta,
+                                  float *running_mean, float *running_var, float factor, float eps, float *y,
+                                  float *save_mean, float *save_invstd, int N, int C, int HW, void *workspace,
+                                  size_t ws_bytes, void *stream) {
+  return bn_fwd_train<StF32>(x, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd, N, C, HW,
+                             workspace, ws_bytes, stream, 2, z);
+}
+int sgh_bn_add_relu_fwd_train_f16(const uint16_t *x, const uint16_t *z, const float *gamma, const float *beta,
+                                  float *running_mean, float *running_var, float factor, float eps, uint16_t *y,
+                                  float *save_mean, float *save_invstd, int N, int C, int HW, void *workspace,
+                                  size_t ws_bytes, void *stream) {
+  return SGH_BN_DISPATCH16(bn_fwd_train, StF16, StF16x4, x, gamma, beta, running_mean, running_var, factor, eps, y,
+                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream, 2, z);
+}
+int sgh_bn_add_relu_fwd_train_bf16(const uint16_t *x, const uint16_t *z, const float *gamma, const float *beta,
+                                   float *running_mean, float *running_var, float factor, float eps, uint16_t *y,
+                                   float *save_mean, float *save_invstd, int N, int C, int HW, void *workspace,
+                                   size_t ws_bytes, void *stream) {
+  return SGH_BN_DISPATCH16(bn_fwd_train, StBF16, StBF16x4, x, gamma, beta, running_mean, running_var, factor, eps, y,
+                           save_mean, save_invstd, N, C, HW, workspace, ws_bytes, stream, 2, z);
 }
 
 int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const float *save_mean,

@@ -937,6 +937,22 @@ def GpuBatchNormReLUForwardTraining(h, x, scale, bias, running_mean, running_var
     return [y, mean, var]
 
 
+def GpuBatchNormAddReLUForwardTraining(h, x, z, scale, bias, running_mean, running_var):
+    """``[relu(BatchNorm(x) + z), mean, var]``: the forward of ``relu(bn(..) + identity)`` at the end of a residual block
+    (examples/cnn/model/resnet.py:70-77) in one call, the bits the three separate calls store."""
+    _same(x, z)
+    y = _like(x)
+    mean = Tensor((h.channels,), x.device(), kFloat32)
+    var = Tensor((h.channels,), x.device(), kFloat32)
+    fn, name = _fn("bn_add_relu_fwd_train", x)
+    check(fn(x.ptr, z.ptr, scale.ptr, bias.ptr,
+             running_mean.ptr if running_mean is not None else None,
+             running_var.ptr if running_var is not None else None,
+             h.factor, _BN_EPS, y.ptr, mean.ptr, var.ptr, h.batchsize, h.channels,
+             h.height * h.width, h.workspace.ptr, h.workspace.MemSize(), x.device().stream), name)
+    return [y, mean, var]
+
+
 def GpuBatchNormForwardInference(h, x, scale, bias, running_mean, running_var):
     """``y`` normalised with the running statistics (src/model/operation/batchnorm.cc:331-366)."""
     y = _like(x)

@@ -74,6 +74,9 @@ class HipOps(object):
     def add_relu(self, a, b):
         return singa.AddReLU(a, b)
 
+    def bn_add_relu_fwd_train(self, h, x, z, g, b, rm, rv):
+        return singa.GpuBatchNormAddReLUForwardTraining(h, x, z, g, b, rm, rv)
+
     def pool_fwd(self, h, x):
         return singa.GpuPoolingForward(h, x)
 
@@ -338,6 +341,19 @@ class BatchNorm(_Layer):
         relu.x = y
         return y
 
+    def fwd_add_relu(self, relu, x, residual):
+        """Forward of ``relu(self(x) + residual)``, the end of a residual block, as one fused call where the ops
+        implementation offers it (this layer's own output is then never stored: its backward needs x only)."""
+        if not getattr(self.ops, "fuse_forward", False):
+            return relu.fwd_of_sum(self.fwd(x), residual)
+        if self.h is None:
+            self.h = self.ops.bn_handle(self.momentum, x)
+        y, self.mean, self.var = self.ops.bn_add_relu_fwd_train(self.h, x, residual, self.scale, self.bias,
+                                                                self.running_mean, self.running_var)
+        self.x = x
+        relu.x = y
+        return y
+
     def bwd(self, dy, grads):
         dx, ds, db = self.ops.bn_bwd(self.h, dy, self.x, self.scale, self.mean, self.var)
         grads(self.name + ".scale", self.scale, ds)
@@ -474,11 +490,11 @@ class BasicBlock(_Layer):
         return ls
 
     def fwd(self, x):
-        out = self.bn2.fwd(self.conv2.fwd(self.bn1.fwd_through_relu(self.relu1, self.conv1.fwd(x))))
+        out = self.conv2.fwd(self.bn1.fwd_through_relu(self.relu1, self.conv1.fwd(x)))
         residual = x
         if self.ds_conv is not None:
             residual = self.ds_bn.fwd(self.ds_conv.fwd(x))
-        return self.relu2.fwd_of_sum(out, residual)
+        return self.bn2.fwd_add_relu(self.relu2, out, residual)
 
     def bwd(self, dy, grads):
         d_add = self.relu2.bwd(dy, grads)
@@ -531,11 +547,11 @@ class Bottleneck(_Layer):
     def fwd(self, x):
         out = self.bn1.fwd_through_relu(self.relu1, self.conv1.fwd(x))
         out = self.bn2.fwd_through_relu(self.relu2, self.conv2.fwd(out))
-        out = self.bn3.fwd(self.conv3.fwd(out))
+        out = self.conv3.fwd(out)
         residual = x
         if self.ds_conv is not None:
             residual = self.ds_bn.fwd(self.ds_conv.fwd(x))
-        return self.relu3.fwd_of_sum(out, residual)
+        return self.bn3.fwd_add_relu(self.relu3, out, residual)
 
     def bwd(self, dy, grads):
         d_add = self.relu3.bwd(dy, grads)

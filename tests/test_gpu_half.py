@@ -241,6 +241,11 @@ def test_fused_forward_calls(singa, dev, kind, shape):
     for got, want, what in ((mean2, mean, "mean"), (var2, var, "invstd"), (rm2, rm1, "running mean"), (rv2, rv1, "running var")):
         _same_bits(got.to_numpy(), want.to_numpy(), what + " " + kind)
     _same_bits(singa.ReLUBackward(dyt, yr).to_numpy(), singa.ReLUBackward(dyt, y).to_numpy(), "ReLU backward gated on the output " + kind)
+    rm3, rv3 = stats()
+    ysr, mean3, var3 = singa.GpuBatchNormAddReLUForwardTraining(h, xt, at, gd, bd, rm3, rv3)
+    _same_bits(ysr.to_numpy(), relu(singa.__add__(y, at)).to_numpy(), "BatchNorm + Add + ReLU forward " + kind)
+    for got, want, what in ((mean3, mean, "mean"), (var3, var, "invstd"), (rm3, rm1, "running mean"), (rv3, rv1, "running var")):
+        _same_bits(got.to_numpy(), want.to_numpy(), what + " (with the sum) " + kind)
     s = singa.__add__(xt, at)
     sr = singa.AddReLU(xt, at)
     _same_bits(sr.to_numpy(), relu(s).to_numpy(), "Add + ReLU forward " + kind)
