@@ -446,6 +446,33 @@ __global__ __launch_bounds__(kBlock) void k_pool_avg_fwd(const typename S::elem 
   }
 }
 
+// One window that is the whole plane, planes of at most 64 elements (global average pooling, 7 x 7): a workgroup
+// stages its 256 consecutive planes -- one contiguous run of memory -- in LDS with whole-vector loads and a thread
+// sums one plane in the order of the loop above.
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_pool_avg_fwd_global(const typename S::elem *__restrict__ x,
+                                                               typename S::elem *__restrict__ y, int HW, size_t planes) {
+  constexpr int V = S::VEC;
+  extern __shared__ float xs_f[];   // kBlock * HW
+  const size_t plane0 = size_t(blockIdx.x) * kBlock;
+  const int np = int(planes - plane0 < size_t(kBlock) ? planes - plane0 : size_t(kBlock)), n = np * HW, t = threadIdx.x;
+  const typename S::elem *base = x + plane0 * size_t(HW);
+  const int nvec = n / V;
+  for (int v = t; v < nvec; v += kBlock) {
+    float e[V];
+    S::template load16<false>(base + v * V, e);
+#pragma unroll
+    for (int q = 0; q < V; ++q) xs_f[v * V + q] = e[q];
+  }
+  for (int i = nvec * V + t; i < n; i += kBlock) xs_f[i] = S::ld(base + i);
+  __syncthreads();
+  if (t < np) {
+    float s = 0.f;
+    for (int j = 0; j < HW; ++j) s += xs_f[t * HW + j];
+    S::st(y + plane0 + t, s / float(HW));
+  }
+}
+
 template <class S>
 __global__ __launch_bounds__(kBlock) void k_pool_avg_bwd(const typename S::elem *__restrict__ dy,
                                                         typename S::elem *__restrict__ dx, PoolG g, size_t total) {
@@ -534,6 +561,10 @@ int pool_fwd(const sgh_pool_geom *g, const typename S::elem *x, typename S::elem
   else if (g->is_max)
     hipLaunchKernelGGL(k_pool_max_fwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), x, y, to_g(g),
                        total);
+  else if (g->P == 1 && g->Q == 1 && g->pad_h == 0 && g->pad_w == 0 && g->kernel_h >= g->H && g->kernel_w >= g->W &&
+           g->H * g->W <= 64 && sgh_aligned16(x) && (total + kBlock - 1) / kBlock < 0x7fffffffu)
+    hipLaunchKernelGGL(k_pool_avg_fwd_global<S>, dim3(unsigned((total + kBlock - 1) / kBlock)), dim3(kBlock),
+                       size_t(kBlock) * g->H * g->W * sizeof(float), sgh_stream_of(stream), x, y, g->H * g->W, total);
   else
     hipLaunchKernelGGL(k_pool_avg_fwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), x, y, to_g(g),
                        total);
