@@ -504,7 +504,9 @@ SGH_API int sgh_conv_fwd_bf16(sgh_conv_geom *g, const uint16_t *x, const uint16_
  * running = (1-factor)*running + factor*batch (unbiased variance), saves (mean, invstd) with
  * invstd = 1/sqrt(var + eps) in the slots Python calls (mean, var)
  * (python/singa/autograd.py:1777-1781).  running_* may be NULL.
- * workspace (both passes): sgh_bn_workspace_bytes(N, C, HW) bytes of per-channel partial sums. */
+ * workspace (both passes): sgh_bn_workspace_bytes(N, C, HW) bytes of per-channel partial sums; the
+ * one-pass forward kernels keep their exchange words in a part of it that no other kernel writes, so
+ * recorded forward and backward launches that share a workspace replay in any order. */
 SGH_API size_t sgh_bn_workspace_bytes(int N, int C, int HW);
 SGH_API int sgh_bn_fwd_train_f32(const float *x, const float *gamma, const float *beta,
                                  float *running_mean, float *running_var, float factor, float eps,

@@ -1045,6 +1045,28 @@ inline BnShape make_shape(int N, int C, int HW, int vec, int esize) {
   return s;
 }
 
+// bytes of workspace the backward pass of storage class S needs: the partial sums of the two-pass
+// kernels or the slots of the one-pass kernel, whichever the shape takes
+template <class S>
+inline size_t bwd_workspace_need(int N, int C, int HW) {
+  const size_t two_pass = size_t(C) * make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem))).S * 2 * sizeof(float);
+  const ChipPlan cp = chip_plan<S>(N, C, HW);
+  const size_t chip = cp.ok ? chip_workspace_bytes(C, cp.G) : 0;
+  return two_pass > chip ? two_pass : chip;
+}
+
+// the part of a workspace that the two-pass kernels and the backward pass of every storage type use, a multiple
+// of 256 bytes (one size for every storage type: the largest of the fp32 and the 16-bit needs)
+inline size_t shared_workspace_bytes(int N, int C, int HW) {
+  const int s4 = make_shape(N, C, HW, 4, 4).S, s8 = make_shape(N, C, HW, 8, 2).S, s4h = make_shape(N, C, HW, 4, 2).S;
+  const int smax = s4 > s8 ? (s4 > s4h ? s4 : s4h) : (s8 > s4h ? s8 : s4h);
+  size_t need = size_t(C) * smax * 2 * sizeof(float);   // (the two-pass forward and backward)
+  const size_t b[3] = {bwd_workspace_need<StF32>(N, C, HW), bwd_workspace_need<StF16>(N, C, HW),
+                       bwd_workspace_need<StF16x4>(N, C, HW)};
+  for (size_t v : b) need = v > need ? v : need;
+  return (need + 255) & ~size_t(255);
+}
+
 template <class S, int ACT>
 int bn_fwd_train_act(const typename S::elem *x, const typename S::elem *z, const float *gamma, const float *beta,
                      float *running_mean, float *running_var, float factor, float eps, typename S::elem *y,
@@ -1056,10 +1078,14 @@ int bn_fwd_train_act(const typename S::elem *x, const typename S::elem *z, const
   if (!sgh_aligned16(x) || !sgh_aligned16(y)) return SGH_EINVAL;
   if (!workspace || ws_bytes < size_t(C) * s.S * 2 * sizeof(float)) return SGH_EWORKSPACE;
   const ChipPlan fp = chip_fwd_plan<S>(N, C, HW, ACT == 2);
+  // the one-pass kernel's words lie behind everything the backward pass and the two-pass kernels write: a
+  // recorded launch tells which of its two tickets is next from what its own words hold, so no other kernel
+  // may write some of a channel's words between two replays
+  const size_t slots_at = shared_workspace_bytes(N, C, HW);
   if (fp.ok && !sgh_env().bn_onchip_off && !sgh_env().bn_fwd_onchip_off && sgh_aligned16(workspace) &&
-      ws_bytes >= chip_workspace_bytes(C, fp.G))
+      ws_bytes >= slots_at + chip_workspace_bytes(C, fp.G))
     return launch_fwd_onchip<S, ACT>(x, z, gamma, beta, running_mean, running_var, factor, eps, y, save_mean, save_invstd,
-                                     workspace, s, fp, sgh_stream_of(stream));
+                                     static_cast<char *>(workspace) + slots_at, s, fp, sgh_stream_of(stream));
   float *scratch = static_cast<float *>(workspace);
   hipLaunchKernelGGL(k_bn_fwd_partial<S>, dim3(C * s.S), dim3(kBlock), 0, sgh_stream_of(stream), x, scratch, s);
   SGH_LAUNCH_CHECK();
@@ -1098,16 +1124,6 @@ int bn_fwd_infer(const typename S::elem *x, const float *gamma, const float *bet
                      running_mean, running_var, eps, y, s);
   SGH_LAUNCH_CHECK();
   return SGH_OK;
-}
-
-// bytes of workspace the backward pass of storage class S needs: the partial sums of the two-pass
-// kernels or the slots of the one-pass kernel, whichever the shape takes
-template <class S>
-inline size_t bwd_workspace_need(int N, int C, int HW) {
-  const size_t two_pass = size_t(C) * make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem))).S * 2 * sizeof(float);
-  const ChipPlan cp = chip_plan<S>(N, C, HW);
-  const size_t chip = cp.ok ? chip_workspace_bytes(C, cp.G) : 0;
-  return two_pass > chip ? two_pass : chip;
 }
 
 // beta != NULL selects the fused ReLU + BatchNorm backward
@@ -1189,19 +1205,14 @@ extern "C" {
 
 size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
   if (!shape_ok(N, C, HW)) return 0;
-  // one size for every storage type: the larger of the fp32 and the 16-bit split counts
-  const int s4 = make_shape(N, C, HW, 4, 4).S, s8 = make_shape(N, C, HW, 8, 2).S, s4h = make_shape(N, C, HW, 4, 2).S;
-  const int smax = s4 > s8 ? (s4 > s4h ? s4 : s4h) : (s8 > s4h ? s8 : s4h);
-  size_t need = size_t(C) * smax * 2 * sizeof(float);   // (the forward pass and the two-pass backward)
-  const size_t b[3] = {bwd_workspace_need<StF32>(N, C, HW), bwd_workspace_need<StF16>(N, C, HW),
-                       bwd_workspace_need<StF16x4>(N, C, HW)};
-  for (size_t v : b) need = v > need ? v : need;
+  // the shared part, then the words of the one-pass forward kernel
+  size_t fwd = 0;
   const ChipPlan f[6] = {chip_fwd_plan<StF32>(N, C, HW, false), chip_fwd_plan<StF16>(N, C, HW, false),
                          chip_fwd_plan<StF16x4>(N, C, HW, false), chip_fwd_plan<StF32>(N, C, HW, true),
                          chip_fwd_plan<StF16>(N, C, HW, true), chip_fwd_plan<StF16x4>(N, C, HW, true)};
   for (const ChipPlan &p : f)
-    if (p.ok && chip_workspace_bytes(C, p.G) > need) need = chip_workspace_bytes(C, p.G);
-  return need;
+    if (p.ok && chip_workspace_bytes(C, p.G) > fwd) fwd = chip_workspace_bytes(C, p.G);
+  return shared_workspace_bytes(N, C, HW) + fwd;
 }
 
 // 16-bit planes that are a multiple of 4 but not of 8 elements (14 x 14) use the 8-byte vector class

@@ -258,6 +258,46 @@ def test_fused_forward_calls(singa, dev, kind, shape):
     _same_bits(singa.AddReLU(*views).to_numpy(), sr.to_numpy().ravel()[1:], "Add + ReLU, unaligned " + kind)
 
 
+@pytest.mark.parametrize("kind,shape", [("f16", (64, 256, 56, 56)), ("f32", (32, 96, 28, 28))])
+def test_recorded_batchnorm_forward_between_eager_backward_passes(singa, dev, kind, shape):
+    """A recorded BatchNorm + Add + ReLU forward (graph mode) is replayed with eager backward passes on the same
+    handle -- the same workspace -- in between: every replay stores the bits of the eager forward call.  (The
+    one-pass forward kernel cuts a channel into other slices than the backward kernel; each keeps its exchange
+    words in a part of the workspace that the other never writes.)"""
+    r = rng(sum(shape) + 5)
+    N, C, H, W = shape
+    x32, z32, dy32 = (r.standard_normal(shape).astype(np.float32) for _ in range(3))
+    if kind == "f32":
+        xt, zt, dyt = (singa.from_numpy(v, dev) for v in (x32, z32, dy32))
+    else:
+        xt, zt, dyt = (_to(singa, dev, v, kind)[0] for v in (x32, z32, dy32))
+    gd = singa.from_numpy((1 + 0.3 * r.standard_normal(C)).astype(np.float32), dev)
+    bd = singa.from_numpy((0.2 * r.standard_normal(C)).astype(np.float32), dev)
+    rm, rv = singa.from_numpy(np.zeros(C, np.float32), dev), singa.from_numpy(np.ones(C, np.float32), dev)
+    h = singa.CudnnBatchNormHandle(0.9, xt)
+    for _ in range(2):   # (the pool holds the blocks the recorded call will take)
+        want, mean, var = singa.GpuBatchNormAddReLUForwardTraining(h, xt, zt, gd, bd, rm, rv)
+        singa.GpuBatchNormBackward(h, dyt, xt, gd, mean, var)
+    want_bits, want_mean = want.to_numpy(), mean.to_numpy()
+    assert np.isfinite(want_bits.astype(np.float32)).all()
+    del want
+    dev.Sync()
+    dev.EnableGraph(True)
+    y, mean_g, var_g = singa.GpuBatchNormAddReLUForwardTraining(h, xt, zt, gd, bd, rm, rv)
+    dev.EnableGraph(False)
+    try:
+        for i in range(5):
+            y.SetFloatValue(0.0)
+            dev.RunGraph()
+            _same_bits(y.to_numpy(), want_bits, "replay %d of the recorded forward, %s" % (i, kind))
+            _same_bits(mean_g.to_numpy(), want_mean, "saved mean of replay %d" % i)
+            if i != 2:   # (also two replays in a row)
+                dx, _, _ = singa.GpuBatchNormBackward(h, dyt, xt, gd, mean, var)
+                assert np.isfinite(dx.to_numpy().astype(np.float32)).all()
+    finally:
+        dev.ResetGraph()
+
+
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("case", [
     (2, 3, 8, 8, (2, 2), (2, 2), (0, 0)),
