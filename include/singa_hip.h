@@ -567,8 +567,9 @@ SGH_API int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma,
  * the one-pass kernel; every ResNet layer up to batch 128 fits) -- else SGH_ELIMIT is returned
  * and nothing is launched.  Calls no hipMalloc / hipFree.
  * All calls on one GPU share the buffer: calls that overlap on one GPU (two streams, two threads)
- * race; calls on one stream are ordered and safe.  Nothing in the buffer needs clearing between
- * calls (every slot read is written earlier in the same call). */
+ * race; calls on one stream are ordered and safe, recorded calls of several shapes replayed in a
+ * graph included.  The caller clears nothing: what a call reads it has written itself (the one-pass
+ * kernel's exchange words are zeroed by a small kernel of the same call). */
 SGH_API int sgh_bn_bwd_noalloc_f32(const float *dy, const float *x, const float *gamma,
                                    const float *save_mean, const float *save_invstd, float *dx,
                                    float *dgamma, float *dbeta, int N, int C, int HW,

@@ -1179,6 +1179,12 @@ constexpr int kNoAllocMaxDevices = 64;
 float *g_noalloc_ptr[kNoAllocMaxDevices];
 std::mutex g_noalloc_mu;
 
+// the exchange words of the one-pass kernel in the shared buffer, zeroed (no ticket has a zero half)
+__global__ __launch_bounds__(256) void k_bn_clear_words(unsigned long long *__restrict__ w, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) w[i] = 0ull;
+}
+
 int noalloc_scratch_of_current_device(float **out) {
   int dev = -1;
   SGH_HIP_TRY(hipGetDevice(&dev));
@@ -1294,9 +1300,21 @@ int sgh_bn_bwd_noalloc_f32(const float *dy, const float *x, const float *gamma, 
   if (!shape_ok(N, C, HW)) return SGH_EINVAL;
   const size_t need = bwd_workspace_need<StF32>(N, C, HW);
   if (need > sizeof(float) * 2 * size_t(kNoAllocMaxPairs)) return SGH_ELIMIT;
-  float *part = nullptr;  // (every slot the second kernel reads is written by the first: nothing to clear)
+  float *part = nullptr;
   const int rc = noalloc_scratch_of_current_device(&part);
   if (rc != SGH_OK) return rc;
+  // The two-pass kernels read only what the same call wrote.  The one-pass kernel tells from what its words
+  // hold which of its two tickets a replay of a recorded launch publishes under, and that needs every word of a
+  // channel in the same state: here calls of other shapes write the same buffer in between, some words of a
+  // channel and not others, so its words are cleared first (by a kernel: a recorded call replays it too) and
+  // every execution publishes under its first ticket.
+  const ChipPlan cp = chip_plan<StF32>(N, C, HW);
+  if (cp.ok && cp.G > 1) {
+    const int words = int(chip_workspace_bytes(C, cp.G) / sizeof(unsigned long long));
+    hipLaunchKernelGGL(k_bn_clear_words, dim3((words + 255) / 256), dim3(256), 0, sgh_stream_of(stream),
+                       reinterpret_cast<unsigned long long *>(part), words);
+    SGH_LAUNCH_CHECK();
+  }
   return bn_bwd<StF32>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, part, need, stream);
 }
 int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,

@@ -54,6 +54,51 @@ def test_no_alloc_bn_bwd_two_calls_in_a_row(dev):
     _case(singa, dev, (8, 48, 28, 28), 4)
 
 
+def test_no_alloc_bn_bwd_recorded_calls_of_two_shapes(dev):
+    """The callers this entry point is for record it into graphs: two recorded calls of different shapes share
+    the library's buffer (the second overwrites some of the first one's exchange words and not others); every
+    replay stores the bits of the eager calls."""
+    from singa_amd import singa_wrap as singa
+    from singa_amd._lib import check, lib
+    shapes = [(8, 48, 28, 28), (16, 20, 20, 20)]
+    cases = []
+    for k, shape in enumerate(shapes):
+        r = rng(40 + k)
+        N, C, H, W = shape
+        x = (randn(r, *shape) * 1.5 - 0.3).astype(np.float32)
+        host = [randn(r, *shape), x, (randn(r, C) * 0.2 + 1).astype(np.float32), x.mean(axis=(0, 2, 3)).astype(np.float32),
+                (1.0 / np.sqrt(x.var(axis=(0, 2, 3)) + 1e-5)).astype(np.float32)]
+        ins = [singa.from_numpy(a, dev) for a in host]
+        outs = [singa.Tensor(shape, dev), singa.Tensor((C,), dev), singa.Tensor((C,), dev)]
+        cases.append((shape, ins, outs))
+
+    def call_all():
+        for (N, C, H, W), ins, outs in cases:
+            check(lib().sgh_bn_bwd_noalloc_f32(*[t.ptr for t in ins], *[t.ptr for t in outs], N, C, H * W, dev.stream),
+                  "sgh_bn_bwd_noalloc_f32")
+
+    print("sgh_bn_bwd_noalloc_f32 recorded, shapes", shapes, flush=True)
+    call_all()
+    want = [[t.to_numpy() for t in outs] for _, _, outs in cases]
+    dev.Sync()
+    dev.EnableGraph(True)
+    call_all()
+    dev.EnableGraph(False)
+    try:
+        for i in range(4):
+            for _, _, outs in cases:
+                for t in outs:
+                    t.SetFloatValue(-77.0)
+            dev.RunGraph()
+            if i == 1:
+                call_all()   # eager calls between replays
+            for (shape, _, outs), w in zip(cases, want):
+                for t, a, what in zip(outs, w, ("dx", "dgamma", "dbeta")):
+                    assert_bit_equal(t.to_numpy(), a, "%s of %r, replay %d" % (what, shape, i))
+    finally:
+        dev.ResetGraph()
+
+
 def test_no_alloc_bn_bwd_rejects_sizes_beyond_its_buffer(dev):
     from singa_amd import singa_wrap as singa
     from singa_amd._lib import SGH_ELIMIT, lib
