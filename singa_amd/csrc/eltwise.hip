@@ -468,8 +468,19 @@ __global__ __launch_bounds__(kBlock) void k_sum_rows(const float *__restrict__ m
                                                     int cols) {
   const int j = blockIdx.x * kBlock + threadIdx.x;
   if (j >= cols) return;
+  // (32 loads in flight per thread; the additions stay in row order.  The loop of one load per addition waited
+  // for each load in turn: 31 us for 128 x 1000)
+  constexpr int U = 32;
   float s = 0.f;
-  for (int i = 0; i < rows; ++i) s += m[size_t(i) * cols + j];
+  int i = 0;
+  for (; i + U <= rows; i += U) {
+    float v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = m[size_t(i + u) * cols + j];
+#pragma unroll
+    for (int u = 0; u < U; ++u) s += v[u];
+  }
+  for (; i < rows; ++i) s += m[size_t(i) * cols + j];
   out[j] = s;
 }
 

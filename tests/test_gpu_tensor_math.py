@@ -220,6 +220,10 @@ def test_linear_backward_gemms(singa, dev, M, N, K):
     assert tt.shape() == [N, K]
     db = singa.Sum(dyd, 0).to_numpy()
     assert max_rel_err(db, O.sum_rows(dy), floor=1e-3) < 1e-5
+    in_row_order = np.zeros(K, np.float32)
+    for row in dy:          # the kernel adds the rows in ascending order, one fp32 addition each
+        in_row_order += row
+    assert_bit_equal(db, in_row_order, "column sums in row order")
 
 
 def test_pool_reuses_freed_blocks(singa, dev):
