@@ -816,6 +816,83 @@ inline int gemm_tile(int M, int N, int K, float alpha, const float *A, long a_rs
       la, lb, st, M, N, K, 1, chunks, stream);
 }
 
+// ---- C = alpha * A * B^T + beta * C with few output tiles and a long reduction (the data gradient of a
+// classifier: batch x features, reduced over the classes) ------------------------------------------------
+// Both operands have the reduction index contiguous -- the operand shape of v_mfma_f32_32x32x2_f32, whose lane
+// (i, h) supplies A[i][h] and B[h][i] -- so the wavefronts feed the matrix instructions straight from global
+// memory with 16-byte loads: lane (i, h) takes the reduction indices 8 j + 4 h + (0..3) of row i of each
+// operand, which the four instructions of group j consume as the pairs (8 j + u, 8 j + 4 + u).  A workgroup
+// owns a 32 x 32 tile of C; its four wavefronts each take a quarter of the reduction and the four partial
+// tiles are added in wavefront order through LDS, so results are run-to-run identical.  The tiled kernel
+// runs such a problem on 16 workgroups that walk the whole reduction one 16-index chunk at a time
+// (128 x 512 x 1000: 33.8 us).
+extern "C++" {
+__global__ __launch_bounds__(256) void k_gemm_kk(const float *__restrict__ A, long lda, const float *__restrict__ B,
+                                                 long ldb, float *__restrict__ C, long ldc, int M, int N, int K, int kq,
+                                                 float alpha, float beta) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  typedef float f32x16 __attribute__((ext_vector_type(16)));
+  __shared__ float part[4][32 * 32];
+  const int t = threadIdx.x, wave = t >> 6, lane = t & 63, i = lane & 31, h = lane >> 5;
+  const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+  const int kb = wave * kq, ke = kb + kq < K ? kb + kq : K;   // (kq is a multiple of 8)
+  const bool am = m0 + i < M, bn = n0 + i < N;
+  const float *ap = A + size_t(am ? m0 + i : 0) * lda + 4 * h;
+  const float *bp = B + size_t(bn ? n0 + i : 0) * ldb + 4 * h;
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  constexpr int U = 4;   // groups of eight reduction indices requested before the first is used
+  int k = kb;
+  for (; k + 8 * U <= ke; k += 8 * U) {
+    f32x4 a[U], b[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      a[u] = *reinterpret_cast<const f32x4 *>(ap + k + 8 * u);
+      b[u] = *reinterpret_cast<const f32x4 *>(bp + k + 8 * u);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!am) a[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (!bn) b[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][e], b[u][e], acc, 0, 0, 0);
+    }
+  }
+  for (; k < ke; k += 8) {   // the last groups, element by element
+    f32x4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (k + 4 * h + e < ke) {
+        if (am) a[e] = ap[k + e];
+        if (bn) b[e] = bp[k + e];
+      }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc, 0, 0, 0);
+  }
+  // lane (i, h) holds column i, rows 8 (v / 4) + 4 h + v % 4
+#pragma unroll
+  for (int v = 0; v < 16; ++v) part[wave][(8 * (v >> 2) + 4 * h + (v & 3)) * 32 + i] = acc[v];
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int e = t + 256 * r, row = e >> 5, col = e & 31;
+    const float v = ((part[0][e] + part[1][e]) + part[2][e]) + part[3][e];
+    if (m0 + row < M && n0 + col < N) {
+      float *p = C + size_t(m0 + row) * ldc + n0 + col;
+      *p = beta == 0.f ? alpha * v : alpha * v + beta * *p;
+    }
+  }
+}
+}  // extern "C++"
+
+// (used when the 64 x 64 tiles of the tiled kernel would leave more than half of the CUs without a workgroup)
+inline bool gemm_kk_ok(int M, int N, int K, const float *A, long lda, const float *B, long ldb) {
+  const long tiles64 = long((M + 63) / 64) * ((N + 63) / 64);
+  return K >= 256 && tiles64 * 2 <= sgh_num_cus() && lda % 4 == 0 && ldb % 4 == 0 && sgh_aligned16(A) && sgh_aligned16(B) &&
+         (N + 31) / 32 <= 65535 && (M + 31) / 32 <= 65535;
+}
+
 template <bool AK, bool BKc>
 inline int gemm_pick(int M, int N, int K, float alpha, const float *A, long a_rs, long a_ks, const float *B, long b_rs,
                      long b_ks, float beta, float *C, int ldc, hipStream_t stream) {
@@ -1542,7 +1619,12 @@ int sgh_gemm_f32(int transA, int transB, int M, int N, int K, float alpha, const
   const long b_rs = transB ? ldb : 1, b_ks = transB ? 1 : ldb;  // B(k, n) addressed as (n, k)
   int rc;
   sgh_prof_start("gemm", 2.0 * M * N * K, s);
-  if (!transA && transB) rc = gemm_pick<true, true>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
+  if (!transA && transB && gemm_kk_ok(M, N, K, A, lda, B, ldb)) {
+    const int kq = ((K + 3) / 4 + 7) / 8 * 8;
+    hipLaunchKernelGGL(k_gemm_kk, dim3(unsigned((N + 31) / 32), unsigned((M + 31) / 32)), dim3(256), 0, s, A, long(lda), B,
+                       long(ldb), C, long(ldc), M, N, K, kq, alpha, beta);
+    rc = hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+  } else if (!transA && transB) rc = gemm_pick<true, true>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
   else if (!transA && !transB) rc = gemm_pick<true, false>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
   else if (transA && transB) rc = gemm_pick<false, true>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);
   else rc = gemm_pick<false, false>(M, N, K, alpha, A, a_rs, a_ks, B, b_rs, b_ks, beta, C, ldc, s);

@@ -204,7 +204,7 @@ def test_sgd_multi_tensor_matches_per_tensor(singa, dev):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 784, 1000), (128, 1000, 10), (64, 512, 1000), (1, 1, 1), (65, 129, 33),
-                                   (300, 260, 515)])
+                                   (300, 260, 515), (70, 90, 516), (128, 2048, 1000), (33, 31, 256)])
 def test_linear_backward_gemms(singa, dev, M, N, K):
     """Matmul.backward: dx = dy * W^T, dW = x^T * dy (python/singa/autograd.py:613-623)."""
     r = rng(M + N + K)
@@ -224,6 +224,28 @@ def test_linear_backward_gemms(singa, dev, M, N, K):
     for row in dy:          # the kernel adds the rows in ascending order, one fp32 addition each
         in_row_order += row
     assert_bit_equal(db, in_row_order, "column sums in row order")
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 512, 1000), (70, 90, 516), (5, 40, 300), (128, 96, 64)])
+def test_gemm_alpha_beta_with_contiguous_reductions(singa, dev, M, N, K):
+    """sgh_gemm_f32 as C = alpha * A * B^T + beta * C (cublasSgemm's contract, src/core/tensor/tensor_math_cuda.h:
+    GEMM): few output tiles with a long reduction run on the kernel that splits the reduction over a workgroup's
+    wavefronts; checked against float64, with beta = 0 not reading C (NaN in it), and run twice for identical bits."""
+    from singa_amd._lib import check, lib
+    r = rng(M * 3 + N * 5 + K)
+    a, b, c = randn(r, M, K), randn(r, N, K), randn(r, M, N)
+    ad, bd = singa.from_numpy(a, dev), singa.from_numpy(b, dev)
+    want = a.astype(np.float64) @ b.astype(np.float64).T
+    outs = []
+    for alpha, beta in ((1.0, 0.0), (0.5, -2.0), (1.0, 0.0)):
+        c0 = np.full((M, N), np.nan, np.float32) if beta == 0.0 else c
+        cd = singa.from_numpy(c0, dev)
+        check(lib().sgh_gemm_f32(0, 1, M, N, K, alpha, ad.ptr, K, bd.ptr, K, beta, cd.ptr, N, dev.stream), "sgh_gemm_f32")
+        got = cd.to_numpy()
+        ref = alpha * want + (beta * c.astype(np.float64) if beta != 0.0 else 0.0)
+        assert nl2(got, ref.astype(np.float32)) < 1e-5, (alpha, beta)
+        outs.append(got)
+    assert_bit_equal(outs[0], outs[2], "two runs")
 
 
 def test_pool_reuses_freed_blocks(singa, dev):
