@@ -363,8 +363,19 @@ __global__ __launch_bounds__(256) void k_wgrad16_reduce(const float *__restrict_
   const int e = threadIdx.x % EP, zl = threadIdx.x / EP;
   const size_t i = size_t(blockIdx.x) * EP + e;
   float s = 0.f;
-  if (i < n)
-    for (int z = zl; z < splits; z += ZL) s += partial[size_t(z) * n + i];
+  if (i < n) {
+    // (eight loads in flight, added in the same ascending order: one load per addition waited for each in turn)
+    constexpr int U = 8;
+    int z = zl;
+    for (; z + (U - 1) * ZL < splits; z += U * ZL) {
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = partial[size_t(z + u * ZL) * n + i];
+#pragma unroll
+      for (int u = 0; u < U; ++u) s += v[u];
+    }
+    for (; z < splits; z += ZL) s += partial[size_t(z) * n + i];
+  }
   lanes[zl][e] = s;
   __syncthreads();
   if (zl == 0 && i < n) {

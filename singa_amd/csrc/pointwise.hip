@@ -258,8 +258,17 @@ __global__ __launch_bounds__(256) void k_pw_wgrad_reduce(const float *__restrict
   const int e = threadIdx.x & 15, zl = threadIdx.x >> 4;
   const long i = long(blockIdx.x) * 16 + e;
   float s = 0.f;
-  if (i < n)
-    for (int z = zl; z < splits; z += 16) s += part[long(z) * n + i];
+  if (i < n) {   // (four loads in flight, added in the same ascending order)
+    int z = zl;
+    for (; z + 48 < splits; z += 64) {
+      float v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = part[long(z + 16 * u) * n + i];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) s += v[u];
+    }
+    for (; z < splits; z += 16) s += part[long(z) * n + i];
+  }
   lanes[zl][e] = s;
   __syncthreads();
   if (threadIdx.x < 16 && i < n) {
