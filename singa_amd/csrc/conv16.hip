@@ -485,44 +485,55 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   };
   const int nkc = a.KP / KC;
 
-  u32x4 ra[ASLOTS];
-  u32x4 rbv[BSLOTS];   // pixel-major copy: the octets of this thread's pixels
-  unsigned rd[8];      // dword pairs: the pair's dword for 8 consecutive k
+  // Two register sets: the chunk after next is requested before the next one is written to LDS, so a request has
+  // two chunks of matrix work to arrive in (one chunk is 0.1 us of a wavefront's matrix work against a memory
+  // latency of about 1 us: with one set the reduction loop ran at the speed of the loads).
+  // (the 128-row tile has 64 accumulator registers and no room for a second set within the 128 registers of four
+  // wavefronts per SIMD: it keeps one set)
+  constexpr int NSETS = BM == 64 ? 2 : 1;
+  u32x4 ra[NSETS][ASLOTS];
+  u32x4 rbv[NSETS][BSLOTS];   // pixel-major copy: the octets of this thread's pixels
+  unsigned rd[NSETS][8];      // dword pairs: the pair's dword for 8 consecutive k
+  unsigned sel_a[NSETS], sel_b[NSETS];   // the selectors of the tap a set was requested for
   const rsrc_t rwt = make_rsrc(a.wt, a.wt_bytes);
   const int woff = ((m0 + rb) * a.KP + oct * 8) * 2;   // rb = t / 8 in 0..63
-  auto load = [&](int tap, int kc) {
+  // (`live` false: a request beyond the last chunk.  It issues the same loads at out-of-range offsets, which
+  // return zeros without touching memory: the number of loads between a request and its use is then the same on
+  // every path, so the wait in front of the use can leave the newer request in flight.  A request inside a
+  // branch made every such wait a wait for all loads.)
+  auto load = [&](auto SET, int tap, int kc, bool live) {
+    constexpr int S = decltype(SET)::value;
     const int wso = (tap * a.CP * a.KP + kc * KC) * 2;
+    const int wv = live ? woff : kOOB;
 #pragma unroll
     for (int i = 0; i < ASLOTS; ++i)
-      ra[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rwt, woff + 64 * i * a.KP * 2, wso, 0));
+      ra[S][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rwt, wv + 64 * i * a.KP * 2, wso, 0));
     if constexpr (PIXK) {
-      const bool kin = kc * KC + oct * 8 < a.K;   // (K is a multiple of 8: an octet is inside or outside)
+      const bool kin = live && kc * KC + oct * 8 < a.K;   // (K is a multiple of 8: an octet is inside or outside)
 #pragma unroll
       for (int i = 0; i < BSLOTS; ++i)
-        rbv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rdy, kin ? bvoff[i] : kOOB, kc * KC * 2, 0));
+        rbv[S][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rdy, kin ? bvoff[i] : kOOB, kc * KC * 2, 0));
     } else {
+      sel_a[S] = selA, sel_b[S] = selB;
       const int kb = kc * KC + kq * 8;
-      if (kb < a.K) {
+      const int dv = live && kb < a.K ? voff : kOOB;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) rd[j] = unsigned(__builtin_amdgcn_raw_buffer_load_b32(rdy, voff, (kb + j) * PQ * 2, 0));
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) rd[j] = 0u;
-      }
+      for (int j = 0; j < 8; ++j) rd[S][j] = unsigned(__builtin_amdgcn_raw_buffer_load_b32(rdy, dv, (kb + j) * PQ * 2, 0));
     }
   };
-  auto stage = [&](uint16_t *As, uint16_t *Bs) {
+  auto stage = [&](auto SET, uint16_t *As, uint16_t *Bs) {
+    constexpr int S = decltype(SET)::value;
 #pragma unroll
-    for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 64 * i) * PITCH + oct * 8) = ra[i];
+    for (int i = 0; i < ASLOTS; ++i) *reinterpret_cast<u32x4 *>(As + (rb + 64 * i) * PITCH + oct * 8) = ra[S][i];
     if constexpr (PIXK) {
 #pragma unroll
-      for (int i = 0; i < BSLOTS; ++i) *reinterpret_cast<u32x4 *>(Bs + (rb + 64 * i) * PITCH + oct * 8) = rbv[i];
+      for (int i = 0; i < BSLOTS; ++i) *reinterpret_cast<u32x4 *>(Bs + (rb + 64 * i) * PITCH + oct * 8) = rbv[S][i];
     } else {
       u32x4 vA, vB;
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
-        vA[d] = __builtin_amdgcn_perm(rd[2 * d + 1], rd[2 * d], selA);
-        vB[d] = __builtin_amdgcn_perm(rd[2 * d + 1], rd[2 * d], selB);
+        vA[d] = __builtin_amdgcn_perm(rd[S][2 * d + 1], rd[S][2 * d], sel_a[S]);
+        vB[d] = __builtin_amdgcn_perm(rd[S][2 * d + 1], rd[S][2 * d], sel_b[S]);
       }
       *reinterpret_cast<u32x4 *>(Bs + (2 * pp) * PITCH + kq * 8) = vA;
       *reinterpret_cast<u32x4 *>(Bs + (2 * pp + 1) * PITCH + kq * 8) = vB;
@@ -538,29 +549,52 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   if (nr > 0 && ns > 0) {
-    int ti = 0, tj = 0, kc = 0;
-    set_tap(ti, tj);
-    load((r0 + st * ti) * a.S + s0 + st * tj, kc);
-    stage(As0, Bs0);
-    __syncthreads();
-    bool cur1 = false;
-    while (true) {
-      bool newtap = false;
-      if (++kc == nkc) {
-        kc = 0, newtap = true;
+    typedef std::integral_constant<int, 0> Set0;
+    typedef std::integral_constant<int, NSETS - 1> Set1;
+    const int total = nr * ns * nkc;   // chunks: taps in (ti, tj) order, the k chunks of a tap in turn
+    int ti = 0, tj = 0, kc = 0;        // the next chunk to request
+    auto request = [&](auto SET) {
+      const bool live = ti < nr;
+      if (live && kc == 0) set_tap(ti, tj);
+      load(SET, live ? (r0 + st * ti) * a.S + s0 + st * tj : 0, live ? kc : 0, live);
+      if (live && ++kc == nkc) {
+        kc = 0;
         if (++tj == ns) tj = 0, ++ti;
       }
-      const bool more = ti < nr;
-      if (more) {
-        if (newtap) set_tap(ti, tj);   // (the registers of the previous chunk were packed with the old selectors)
-        load((r0 + st * ti) * a.S + s0 + st * tj, kc);
-      }
-      mma_chunk<TM, BF16>(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0, wm * (TM * 32) + l32, wn * 64 + half * 32 + l32,
-                          half ? -32 : 32, half * 32 + lh * 8, acc);
-      if (!more) break;
-      stage(cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
+    };
+    auto mma = [&](const uint16_t *As, const uint16_t *Bs) {
+      mma_chunk<TM, BF16>(As, Bs, wm * (TM * 32) + l32, wn * 64 + half * 32 + l32, half ? -32 : 32, half * 32 + lh * 8, acc);
+    };
+    request(Set0{});
+    if constexpr (NSETS == 2) {
+      request(Set1{});
+      stage(Set0{}, As0, Bs0);
       __syncthreads();
-      cur1 = !cur1;
+      for (int c = 0;; c += 2) {
+        // chunk c is in LDS buffer 0, chunk c + 1 on its way into register set 1
+        request(Set0{});
+        mma(As0, Bs0);
+        if (c + 1 >= total) break;
+        stage(Set1{}, As1, Bs1);
+        __syncthreads();
+        request(Set1{});
+        mma(As1, Bs1);
+        if (c + 2 >= total) break;
+        stage(Set0{}, As0, Bs0);
+        __syncthreads();
+      }
+    } else {
+      stage(Set0{}, As0, Bs0);
+      __syncthreads();
+      bool cur1 = false;
+      for (int c = 0;; ++c) {
+        request(Set0{});
+        mma(cur1 ? As1 : As0, cur1 ? Bs1 : Bs0);
+        if (c + 1 >= total) break;
+        stage(Set0{}, cur1 ? As0 : As1, cur1 ? Bs0 : Bs1);
+        __syncthreads();
+        cur1 = !cur1;
+      }
     }
   }
 
