@@ -160,8 +160,12 @@ SGH_API int sgh_prof_get(int i, char *tag, size_t tag_len, float *ms, double *wo
 /* ReLUBackward<float, Lang>: tensor_math.h:175-179; CPU tensor_math_cpp.h:446-451;
  * CUDA math_kernel.cu:253-261.  dx[i] = x[i] > 0 ? dy[i] : 0 (x = the ReLU input). */
 SGH_API int sgh_relu_bwd_f32(const float *dy, const float *x, float *dx, size_t n, void *stream);
-/* ReLU<float, Lang>: tensor_math_cpp.h:585-589 (needed to produce the backward's inputs). */
+/* ReLU<float, Lang>: tensor_math_cpp.h:585-589 (needed to produce the backward's inputs); on half
+ * tensors ReLU<half, Lang>, src/core/tensor/math_kernel.cu:242-251 (16-bit variants: y = x > 0 ? x : 0
+ * on the stored values, exact). */
 SGH_API int sgh_relu_fwd_f32(const float *x, float *y, size_t n, void *stream);
+SGH_API int sgh_relu_fwd_f16(const uint16_t *x, uint16_t *y, size_t n, void *stream);
+SGH_API int sgh_relu_fwd_bf16(const uint16_t *x, uint16_t *y, size_t n, void *stream);
 
 /* SoftmaxCrossEntropyBwd<float, Lang>: tensor_math.h:475-480; CPU tensor_math_cpp.h:1090-1119;
  * CUDA math_kernel.cu:564-611; host wrapper src/core/tensor/tensor.cc:1717-1758.
@@ -174,6 +178,15 @@ SGH_API int sgh_relu_fwd_f32(const float *x, float *y, size_t n, void *stream);
  * flag readable with sgh_softmax_ce_label_errors (the CPU reference aborts on negatives). */
 SGH_API int sgh_softmax_ce_bwd_f32(const float *p, const int32_t *t, float *grad, size_t batch,
                                    size_t dim, int int_target, float scale, void *stream);
+/* SoftmaxCrossEntropyBwd<half, Lang> (src/core/tensor/math_kernel.cu:588-611; a layer of a half
+ * model casts its inputs to the layer's type, python/singa/layer.py:171-185, so the loss of a pure
+ * half model arrives here).  p and grad are 16-bit, t stays int32; the subtraction (and the row sum
+ * of an array target, the division, the scale) are fp32 on the widened values, one rounding at the
+ * store.  Label handling and the error flag are those of the fp32 entry point. */
+SGH_API int sgh_softmax_ce_bwd_f16(const uint16_t *p, const int32_t *t, uint16_t *grad, size_t batch,
+                                   size_t dim, int int_target, float scale, void *stream);
+SGH_API int sgh_softmax_ce_bwd_bf16(const uint16_t *p, const int32_t *t, uint16_t *grad, size_t batch,
+                                    size_t dim, int int_target, float scale, void *stream);
 /* Number of out-of-range labels seen since the last call (synchronises the stream). */
 SGH_API int sgh_softmax_ce_label_errors(void *stream, int *count);
 /* SoftMax<float, Lang> (rows) and ComputeCrossEntropy<float, Lang>: forward helpers,
@@ -192,10 +205,16 @@ SGH_API int sgh_cross_entropy_fwd_f32(const float *p, const int32_t *t, float *l
 #define SGH_MAX_DIMS 8
 SGH_API int sgh_transform_f32(const float *in, float *out, int ndim, const size_t *shape,
                               const int64_t *strides, void *stream);
-/* RowMax<float, Lang> (tensor_math_cpp.h:1122-1140): out[r] = max(0, max_c in[r][c]) for a dense
- * nrow x ncol matrix -- the CPU function seeds the maximum with 0 (the CUDA kernel with the row's
- * first element, math_kernel.cu:493); the CPU path is the one results are compared with. */
+/* RowMax<float, Lang> for a dense nrow x ncol matrix.  The reference's two backends differ on rows
+ * without a positive element: its accelerator kernel seeds the maximum with the row's first element
+ * and returns the true maximum (src/core/tensor/math_kernel.cu:488-499, called from
+ * tensor_math_cuda.h:1493-1507), its CPU function seeds it with 0 (tensor_math_cpp.h:1122-1140).
+ *   sgh_row_max_f32             out[r] = max_c in[r][c]            (the accelerator rule: this
+ *                                library replaces that path)
+ *   sgh_row_max_zero_seeded_f32 out[r] = max(0, max_c in[r][c])    (the CPU rule, for comparisons
+ *                                with the CPU path bit for bit) */
 SGH_API int sgh_row_max_f32(const float *in, float *out, size_t nrow, size_t ncol, void *stream);
+SGH_API int sgh_row_max_zero_seeded_f32(const float *in, float *out, size_t nrow, size_t ncol, void *stream);
 /* Dot<float, Lang> with a Tensor result (tensor_math_cpp.h:839-849, cublasSdot in device pointer
  * mode tensor_math_cuda.h:1084-1092) and Sum<float, Lang> over all elements (tensor_math_cpp.h:
  * 655-663): *out = sum a[i] * b[i] / sum a[i], `out` in device memory.  Summed in an order that
@@ -268,6 +287,12 @@ SGH_API int sgh_cast_f32_to_f16(const float *src, uint16_t *dst, size_t n, void 
 SGH_API int sgh_cast_f16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream);
 SGH_API int sgh_cast_f32_to_bf16(const float *src, uint16_t *dst, size_t n, void *stream);
 SGH_API int sgh_cast_bf16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream);
+/* CastCopy<float, int, Lang> / CastCopy<int, float, Lang> (tensor_math_cuda.h:177-191,
+ * src/core/tensor/math_kernel.cu:280-292: `(int)src[i]` and `(float)src[i]`).  float -> int truncates
+ * toward zero; values outside the int32 range saturate to INT32_MIN / INT32_MAX and NaN gives 0 (what
+ * the conversion instruction does; C leaves both undefined).  int -> float rounds to nearest even. */
+SGH_API int sgh_cast_f32_to_i32(const float *src, int32_t *dst, size_t n, void *stream);
+SGH_API int sgh_cast_i32_to_f32(const int32_t *src, float *dst, size_t n, void *stream);
 /* ReLUBackward<half, Lang>: tensor_math_cuda.h:665-674, math_kernel.cu:261-271.  Follows the
  * CPU rule dx = x > 0 ? dy : 0 (the CUDA half kernel alone passes the gradient at x == 0). */
 SGH_API int sgh_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream);
@@ -355,6 +380,16 @@ SGH_API int sgh_sgd_momentum_master_bf16(float *p_master, const uint16_t *g, flo
 SGH_API int sgh_gemm_f32(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                          int lda, const float *B, int ldb, float beta, float *C, int ldc,
                          void *stream);
+/* GEMM<half, Lang> (cublasHgemm in the reference, src/core/tensor/tensor_math_cuda.h:1163-1187): the
+ * Linear layers of a half model.  A, B, C are binary16 (bfloat16); products of the stored values are
+ * accumulated in fp32 on the 16-bit matrix instructions (v_mfma_f32_32x32x16), alpha and beta apply in
+ * fp32, C is rounded once.  Same argument meaning as sgh_gemm_f32.  Run-to-run identical. */
+SGH_API int sgh_gemm_f16(int transA, int transB, int M, int N, int K, float alpha, const uint16_t *A,
+                         int lda, const uint16_t *B, int ldb, float beta, uint16_t *C, int ldc,
+                         void *stream);
+SGH_API int sgh_gemm_bf16(int transA, int transB, int M, int N, int K, float alpha, const uint16_t *A,
+                          int lda, const uint16_t *B, int ldb, float beta, uint16_t *C, int ldc,
+                          void *stream);
 /* SumRows<float, Lang> (Sum(dy, 0), src/core/tensor/tensor.cc:1523-1538): out[j] = sum_i m[i][j].
  * Bias gradient of AddBias.backward (python/singa/autograd.py:696-709). */
 SGH_API int sgh_sum_rows_f32(const float *m, float *out, int rows, int cols, void *stream);
@@ -415,6 +450,9 @@ SGH_API int sgh_conv_dgrad_f32(sgh_conv_geom *g, const float *dy, const float *W
  * K a multiple of 16); SGH_EUNSUPPORTED otherwise, with dx untouched. */
 SGH_API int sgh_conv_dgrad_acc_f32(sgh_conv_geom *g, const float *dy, const float *W,
                                    float *dx, void *workspace, size_t ws_bytes, void *stream);
+/* 1 if sgh_conv_dgrad_acc_f32 covers this geometry, else 0: a caller that has to schedule the
+ * fallback (data gradient + Add) itself asks before it submits anything. */
+SGH_API int sgh_conv_dgrad_acc_supported(const sgh_conv_geom *g);
 /* The data gradient re-lays the weight tensor in its workspace before the matrix kernel runs:
  * a launch of a few microseconds per layer.  A caller that runs many data gradients while the
  * weights do not change (a backward pass) can have all of them re-laid by ONE launch up front:

@@ -83,6 +83,18 @@ SIGNATURES = {
     "sgh_prof_get": (C.c_int, [C.c_int, C.c_char_p, sz, C.POINTER(C.c_float), C.POINTER(C.c_double)]),
     "sgh_relu_bwd_f32": (C.c_int, [vp, vp, vp, sz, vp]),
     "sgh_relu_fwd_f32": (C.c_int, [vp, vp, sz, vp]),
+    "sgh_relu_fwd_f16": (C.c_int, [vp, vp, sz, vp]),
+    "sgh_relu_fwd_bf16": (C.c_int, [vp, vp, sz, vp]),
+    "sgh_softmax_ce_bwd_f16": (C.c_int, [vp, vp, vp, sz, sz, C.c_int, C.c_float, vp]),
+    "sgh_softmax_ce_bwd_bf16": (C.c_int, [vp, vp, vp, sz, sz, C.c_int, C.c_float, vp]),
+    "sgh_row_max_zero_seeded_f32": (C.c_int, [vp, vp, sz, sz, vp]),
+    "sgh_cast_f32_to_i32": (C.c_int, [vp, vp, sz, vp]),
+    "sgh_cast_i32_to_f32": (C.c_int, [vp, vp, sz, vp]),
+    "sgh_gemm_f16": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, vp, C.c_int,
+                               vp, C.c_int, C.c_float, vp, C.c_int, vp]),
+    "sgh_gemm_bf16": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, vp, C.c_int,
+                                vp, C.c_int, C.c_float, vp, C.c_int, vp]),
+    "sgh_conv_dgrad_acc_supported": (C.c_int, [C.POINTER(ConvGeom)]),
     "sgh_softmax_ce_bwd_f32": (C.c_int, [vp, vp, vp, sz, sz, C.c_int, C.c_float, vp]),
     "sgh_softmax_ce_label_errors": (C.c_int, [vp, C.POINTER(C.c_int)]),
     "sgh_softmax_fwd_f32": (C.c_int, [vp, vp, sz, sz, vp]),

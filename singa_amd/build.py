@@ -13,7 +13,7 @@ LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libsinga_hip.so")
 
 SOURCES = ["runtime.hip", "eltwise.hip", "pool.hip", "batchnorm.hip", "igemm.hip", "wgrad3x3.hip", "conv16.hip",
-    "wgrad_fewc.hip", "dgrad3x3.hip", "dgrad_fewc.hip", "half.hip", "tensor_fns.hip", "pointwise.hip", "fwd_fewc16.hip", "fwd_fewc.hip"]
+    "wgrad_fewc.hip", "dgrad3x3.hip", "dgrad_fewc.hip", "half.hip", "tensor_fns.hip", "pointwise.hip", "fwd_fewc16.hip", "fwd_fewc.hip", "gemm16.hip"]
 
 # Packed-FP32 VALU ops are disabled for every device code object of this library.
 HIPCC_FLAGS = [

@@ -5,6 +5,7 @@
 // results are comparable bit for bit where the reference is elementwise.
 #include "common.h"
 #include "sgd_math.h"
+#include "storage.h"
 
 // contraction is disabled per function where the reference rounds after each op
 #define SGH_NO_CONTRACT _Pragma("clang fp contract(off)")
@@ -378,21 +379,24 @@ __global__ __launch_bounds__(kBlock) void k_sgd_multi(const sgh_sgd_item *__rest
 // ---------------------------------------------------------------------------------------
 __device__ int g_label_errors = 0;
 
-__global__ __launch_bounds__(kBlock) void k_softmax_ce_bwd(const float *__restrict__ p, const int32_t *__restrict__ t,
-                                                          float *__restrict__ grad, size_t dim, int int_target,
+// S: the storage type of p and grad (fp32, or 16-bit with fp32 arithmetic and one rounding at the store)
+template <class S>
+__global__ __launch_bounds__(kBlock) void k_softmax_ce_bwd(const typename S::elem *__restrict__ p,
+                                                          const int32_t *__restrict__ t,
+                                                          typename S::elem *__restrict__ grad, size_t dim, int int_target,
                                                           float scale) {
   __shared__ float red[16];
   const size_t row = blockIdx.x;
-  const float *pr = p + row * dim;
-  float *gr = grad + row * dim;
+  const typename S::elem *pr = p + row * dim;
+  typename S::elem *gr = grad + row * dim;
   if (int_target) {
     const int label = t[row];
     const bool ok = label >= 0 && size_t(label) < dim;
     if (!ok && threadIdx.x == 0) atomicAdd(&g_label_errors, 1);
     for (size_t j = threadIdx.x; j < dim; j += kBlock) {
-      float v = pr[j];
+      float v = S::ld(pr + j);
       if (ok && j == size_t(label)) v = v - 1.0f;
-      gr[j] = v * scale;
+      S::st(gr + j, v * scale);
     }
   } else {
     const int32_t *tr = t + row * dim;
@@ -400,8 +404,8 @@ __global__ __launch_bounds__(kBlock) void k_softmax_ce_bwd(const float *__restri
     for (size_t j = threadIdx.x; j < dim; j += kBlock) s += float(tr[j]);
     s = sgh_block_sum(s, red);
     for (size_t j = threadIdx.x; j < dim; j += kBlock) {
-      float v = pr[j] - float(tr[j]) / s;
-      gr[j] = v * scale;
+      float v = S::ld(pr + j) - float(tr[j]) / s;
+      S::st(gr + j, v * scale);
     }
   }
 }
@@ -490,6 +494,34 @@ __global__ __launch_bounds__(kBlock) void k_add_row(const float *__restrict__ v,
   for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) m[i] += v[i % cols];
 }
 
+template <class S>
+int softmax_ce_bwd(const typename S::elem *p, const int32_t *t, typename S::elem *grad, size_t batch, size_t dim,
+                          int int_target, float scale, void *stream) {
+  if (batch == 0 || dim == 0) return SGH_OK;
+  if (!p || !t || !grad) return SGH_EINVAL;
+  if (batch > 0x7fffffffu) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_softmax_ce_bwd<S>, dim3((unsigned)batch), dim3(kBlock), 0, sgh_stream_of(stream), p, t, grad, dim,
+                     int_target, scale);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+// CastCopy between float and int tensors: (int)x truncates toward zero (v_cvt_i32_f32 saturates out-of-range
+// values and turns NaN into 0), (float)i rounds to nearest even
+__global__ __launch_bounds__(kBlock) void k_cast_f32_i32(const float *__restrict__ src, int32_t *__restrict__ dst, size_t n) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) dst[i] = int32_t(src[i]);
+}
+__global__ __launch_bounds__(kBlock) void k_cast_i32_f32(const int32_t *__restrict__ src, float *__restrict__ dst, size_t n) {
+  const size_t stride = size_t(gridDim.x) * kBlock;
+  for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) dst[i] = float(src[i]);
+}
+inline int cast_grid(size_t n) {
+  size_t blocks = (n + kBlock - 1) / kBlock;
+  const size_t cap = size_t(sgh_num_cus()) * 16;
+  return int(blocks > cap ? cap : (blocks < 1 ? 1 : blocks));
+}
+
 }  // namespace
 
 extern "C" {
@@ -501,6 +533,22 @@ int sgh_relu_bwd_f32(const float *dy, const float *x, float *dx, size_t n, void 
 
 int sgh_relu_fwd_f32(const float *x, float *y, size_t n, void *stream) {
   return launch_map1(x, y, n, ReluFwd{}, stream);
+}
+
+int sgh_cast_f32_to_i32(const float *src, int32_t *dst, size_t n, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!src || !dst) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_cast_f32_i32, dim3(cast_grid(n)), dim3(kBlock), 0, sgh_stream_of(stream), src, dst, n);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_cast_i32_to_f32(const int32_t *src, float *dst, size_t n, void *stream) {
+  if (n == 0) return SGH_OK;
+  if (!src || !dst) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_cast_i32_f32, dim3(cast_grid(n)), dim3(kBlock), 0, sgh_stream_of(stream), src, dst, n);
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
 }
 
 int sgh_clamp_f32(float low, float high, const float *x, float *out, size_t n, void *stream) {
@@ -607,13 +655,15 @@ int sgh_sgd_momentum_multi_f32(const sgh_sgd_item *table_dev, int count, size_t 
 
 int sgh_softmax_ce_bwd_f32(const float *p, const int32_t *t, float *grad, size_t batch, size_t dim, int int_target,
                            float scale, void *stream) {
-  if (batch == 0 || dim == 0) return SGH_OK;
-  if (!p || !t || !grad) return SGH_EINVAL;
-  if (batch > 0x7fffffffu) return SGH_EINVAL;
-  hipLaunchKernelGGL(k_softmax_ce_bwd, dim3((unsigned)batch), dim3(kBlock), 0, sgh_stream_of(stream), p, t, grad, dim,
-                     int_target, scale);
-  SGH_LAUNCH_CHECK();
-  return SGH_OK;
+  return softmax_ce_bwd<StF32>(p, t, grad, batch, dim, int_target, scale, stream);
+}
+int sgh_softmax_ce_bwd_f16(const uint16_t *p, const int32_t *t, uint16_t *grad, size_t batch, size_t dim, int int_target,
+                           float scale, void *stream) {
+  return softmax_ce_bwd<StF16>(p, t, grad, batch, dim, int_target, scale, stream);
+}
+int sgh_softmax_ce_bwd_bf16(const uint16_t *p, const int32_t *t, uint16_t *grad, size_t batch, size_t dim, int int_target,
+                            float scale, void *stream) {
+  return softmax_ce_bwd<StBF16>(p, t, grad, batch, dim, int_target, scale, stream);
 }
 
 int sgh_softmax_ce_label_errors(void *stream, int *count) {

@@ -100,6 +100,9 @@ int launch_map2_h(const uint16_t *a, const uint16_t *b, uint16_t *o, size_t n, F
 struct ReluBwd {
   __device__ __forceinline__ float operator()(float dy, float x) const { return x > 0.f ? dy : 0.f; }
 };
+struct ReluFwd {   // (math_kernel.cu:242-251: in > 0 ? in : 0)
+  __device__ __forceinline__ float operator()(float x, float) const { return x > 0.f ? x : 0.f; }
+};
 
 // dx = x > 0 ? dy0 + dy1 : 0: ReLU backward on a gradient that arrives as two summands (the two
 // branches of a residual block), so that the sum is never stored.  dx may alias dy0 or dy1.
@@ -442,6 +445,13 @@ int sgh_cast_f16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream)
 int sgh_cast_f32_to_bf16(const float *src, uint16_t *dst, size_t n, void *stream) { return cast_to16<BF16>(src, dst, n, stream); }
 int sgh_cast_bf16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream) { return cast_from16<BF16>(src, dst, n, stream); }
 
+// (both operands are x: the stored value where it is positive, else +0 -- exact, nothing is rounded)
+int sgh_relu_fwd_f16(const uint16_t *x, uint16_t *y, size_t n, void *stream) {
+  return launch_map2_h<F16>(x, x, y, n, ReluFwd{}, stream);
+}
+int sgh_relu_fwd_bf16(const uint16_t *x, uint16_t *y, size_t n, void *stream) {
+  return launch_map2_h<BF16>(x, x, y, n, ReluFwd{}, stream);
+}
 int sgh_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream) {
   sgh_prof_scope prof("relu_bwd/k_map2_h<ReluBwd>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<F16>(dy, x, dx, n, ReluBwd{}, stream);

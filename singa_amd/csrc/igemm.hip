@@ -1434,9 +1434,13 @@ int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, 
   return flush();
 }
 
+int sgh_conv_dgrad_acc_supported(const sgh_conv_geom *g) {
+  return g && conv_ok(g) && g->groups == 1 && dgrad_path(g) == kDgradTile3x3 ? 1 : 0;
+}
+
 int sgh_conv_dgrad_acc_f32(sgh_conv_geom *g, const float *dy, const float *W, float *dx, void *workspace,
                            size_t ws_bytes, void *stream) {
-  if (g && conv_ok(g) && (g->groups > 1 || dgrad_path(g) != kDgradTile3x3)) return SGH_EUNSUPPORTED;   // (the note stays for the fallback call)
+  if (g && conv_ok(g) && !sgh_conv_dgrad_acc_supported(g)) return SGH_EUNSUPPORTED;   // (the note stays for the fallback call)
   const bool prelaid = take_prelaid(g, 0, W, workspace);
   return conv_dgrad(g, dy, W, dx, workspace, ws_bytes, stream, true, prelaid);
 }

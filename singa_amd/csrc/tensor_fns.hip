@@ -35,12 +35,14 @@ __global__ __launch_bounds__(kBlock) void k_transform(const float *__restrict__ 
   }
 }
 
-// out[r] = max(0, max_c in[r][c]): the CPU function seeds the maximum with 0
-// (tensor_math_cpp.h:1132), and it is the CPU path that results are compared with
+// out[r] = max_c in[r][c], seeded with the row's first element like the reference's accelerator kernel
+// (src/core/tensor/math_kernel.cu:488-499); ZERO_SEEDED: max(0, ...), the reference's CPU function
+// (tensor_math_cpp.h:1132)
+template <bool ZERO_SEEDED>
 __global__ __launch_bounds__(kBlock) void k_row_max(const float *__restrict__ in, float *__restrict__ out, int ncol) {
   __shared__ float red[4];
   const float *row = in + size_t(blockIdx.x) * ncol;
-  float m = 0.f;
+  float m = ZERO_SEEDED ? 0.f : row[0];
   for (int c = threadIdx.x; c < ncol; c += kBlock) m = fmaxf(m, row[c]);
   m = sgh_wave_max(m);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
@@ -155,7 +157,15 @@ int sgh_transform_f32(const float *in, float *out, int ndim, const size_t *shape
 int sgh_row_max_f32(const float *in, float *out, size_t nrow, size_t ncol, void *stream) {
   if (nrow == 0) return SGH_OK;
   if (!in || !out || ncol == 0 || nrow > 0x7fffffffull || ncol > 0x7fffffffull) return SGH_EINVAL;
-  hipLaunchKernelGGL(k_row_max, dim3(unsigned(nrow)), dim3(kBlock), 0, sgh_stream_of(stream), in, out, int(ncol));
+  hipLaunchKernelGGL(k_row_max<false>, dim3(unsigned(nrow)), dim3(kBlock), 0, sgh_stream_of(stream), in, out, int(ncol));
+  SGH_LAUNCH_CHECK();
+  return SGH_OK;
+}
+
+int sgh_row_max_zero_seeded_f32(const float *in, float *out, size_t nrow, size_t ncol, void *stream) {
+  if (nrow == 0) return SGH_OK;
+  if (!in || !out || ncol == 0 || nrow > 0x7fffffffull || ncol > 0x7fffffffull) return SGH_EINVAL;
+  hipLaunchKernelGGL(k_row_max<true>, dim3(unsigned(nrow)), dim3(kBlock), 0, sgh_stream_of(stream), in, out, int(ncol));
   SGH_LAUNCH_CHECK();
   return SGH_OK;
 }

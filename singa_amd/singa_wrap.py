@@ -308,7 +308,7 @@ class Tensor(object):
         check(_L().sgh_memcpy(self._dev._h, self.ptr, a.ctypes.data, a.nbytes, 1), "sgh_memcpy H2D")
 
     def AsType(self, dtype):
-        """``Tensor::AsType`` (src/core/tensor/tensor.cc:197-214) between fp32 and a 16-bit type."""
+        """``Tensor::AsType`` (src/core/tensor/tensor.cc:197-214) between fp32 and a 16-bit type or int32."""
         if dtype == self._dtype:
             return self
         if self._transposed:
@@ -318,6 +318,10 @@ class Tensor(object):
             name = "sgh_cast_f32_to_%s" % _SUFFIX[dtype]
         elif dtype == kFloat32 and self._dtype in (kFloat16, kBFloat16):
             name = "sgh_cast_%s_to_f32" % _SUFFIX[self._dtype]
+        elif self._dtype == kFloat32 and dtype == kInt:      # (int)x: truncation toward zero
+            name = "sgh_cast_f32_to_i32"
+        elif self._dtype == kInt and dtype == kFloat32:
+            name = "sgh_cast_i32_to_f32"
         else:
             raise SingaHipError("AsType %r -> %r is not on the backward path" % (self._dtype, dtype))
         check(getattr(_L(), name)(self.ptr, out.ptr, self.Size(), self._dev.stream), name)
@@ -436,14 +440,17 @@ def Clamp(low, high, t):
     return out
 
 
-def RowMax(t):
-    """``singa.RowMax``: per row max(0, max over the row) (the CPU rule, tensor_math_cpp.h:1122-1140)."""
+def RowMax(t, cpu_rule=False):
+    """``singa.RowMax``: the maximum of every row, as the reference's accelerator kernel computes it
+    (src/core/tensor/math_kernel.cu:488-499).  ``cpu_rule=True`` (not in the reference signature) gives
+    max(0, row maximum), what the reference's CPU function returns (tensor_math_cpp.h:1122-1140)."""
     _need_f32("RowMax", t)
     t = Transform(t)
     if t.nDim() != 2:
         raise SingaHipError("RowMax expects a matrix")
     out = Tensor((t.shape(0),), t.device(), kFloat32)
-    check(_L().sgh_row_max_f32(t.ptr, out.ptr, t.shape(0), t.shape(1), t.device().stream), "sgh_row_max_f32")
+    name = "sgh_row_max_zero_seeded_f32" if cpu_rule else "sgh_row_max_f32"
+    check(getattr(_L(), name)(t.ptr, out.ptr, t.shape(0), t.shape(1), t.device().stream), name)
     return out
 
 
@@ -528,17 +535,17 @@ def _like(t):
 
 
 def ReLU(x):
-    _need_f32("ReLU", x)
+    fn, name = _fn("relu_fwd", x)   # (refuses other data types before anything is allocated)
     y = _like(x)
-    check(_L().sgh_relu_fwd_f32(x.ptr, y.ptr, x.Size(), x.device().stream), "sgh_relu_fwd_f32")
+    check(fn(x.ptr, y.ptr, x.Size(), x.device().stream), name)
     return y
 
 
 def ReLUBackward(dy, x):
     """``singa.ReLUBackward(dy, x)`` (python/singa/autograd.py:432-439)."""
     _same(dy, x)
-    dx = _like(dy)
     fn, name = _fn("relu_bwd", dy)
+    dx = _like(dy)
     check(fn(dy.ptr, x.ptr, dx.ptr, dy.Size(), dy.device().stream), name)
     return dx
 
@@ -564,10 +571,11 @@ def SoftMax(x):
     return p
 
 
-def _ce_dims(p, t):
+def _ce_dims(p, t, half_ok=False):
     if p.nDim() > 2 or t.nDim() > 2:
         raise SingaHipError("cross entropy expects at most 2-D tensors")
-    _need_f32("cross entropy", p)
+    if not (half_ok and p.data_type() in (kFloat16, kBFloat16)):
+        _need_f32("cross entropy", p)
     if t.data_type() != kInt:
         raise SingaHipError("the target tensor must hold int32 (the reference reads it as int)")
     batch = p.shape(0) if p.nDim() == 2 else 1
@@ -589,10 +597,10 @@ def CrossEntropyFwd(p, t):
 def SoftmaxCrossEntropyBwd(p, t, scale=1.0):
     """``singa.SoftmaxCrossEntropyBwd(p, t)`` (src/core/tensor/tensor.cc:1717-1721): returns a new
     tensor.  ``scale`` (not in the reference signature) fuses the ``dx /= N`` that follows it."""
-    batch, dim, int_target = _ce_dims(p, t)
+    batch, dim, int_target = _ce_dims(p, t, half_ok=True)
     g = _like(p)
-    check(_L().sgh_softmax_ce_bwd_f32(p.ptr, t.ptr, g.ptr, batch, dim, int(int_target), float(scale),
-                                      p.device().stream), "sgh_softmax_ce_bwd_f32")
+    fn, name = _fn("softmax_ce_bwd", p)   # 16-bit p: fp32 arithmetic on the stored values, one rounding
+    check(fn(p.ptr, t.ptr, g.ptr, batch, dim, int(int_target), float(scale), p.device().stream), name)
     return g
 
 
@@ -702,14 +710,15 @@ def Mult(A, B):
     flags of the views select the GEMM variant, no data is moved."""
     if A.nDim() != 2 or B.nDim() != 2 or A.shape(1) != B.shape(0):
         raise SingaHipError("Mult shape mismatch %s x %s" % (A.shape(), B.shape()))
-    _need_f32("Mult", A, B)
+    if A.data_type() != B.data_type():
+        raise SingaHipError("Mult: operands differ in data type")
+    fn, name = _fn("gemm", A)   # 16-bit operands: the 16-bit matrix instructions, fp32 accumulation, one rounding
     M, K, N = A.shape(0), A.shape(1), B.shape(1)
-    out = Tensor((M, N), A.device(), kFloat32)
+    out = Tensor((M, N), A.device(), A.data_type())
     tA, tB = A.transpose(), B.transpose()
     lda = M if tA else K
     ldb = K if tB else N
-    check(_L().sgh_gemm_f32(int(tA), int(tB), M, N, K, 1.0, A.ptr, lda, B.ptr, ldb, 0.0, out.ptr, N,
-                            A.device().stream), "sgh_gemm_f32")
+    check(fn(int(tA), int(tB), M, N, K, 1.0, A.ptr, lda, B.ptr, ldb, 0.0, out.ptr, N, A.device().stream), name)
     return out
 
 

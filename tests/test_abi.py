@@ -137,9 +137,13 @@ def test_fp32_only_wrappers_check_the_data_type_before_any_call():
         stream = None
 
     t = singa.from_device_pointer(0x1000, (4, 8), _NoDevice(), singa.kFloat16)
-    for call in (lambda: singa.ReLU(t), lambda: singa.SoftMax(t), lambda: singa.Mult(t, t.T()), lambda: singa.Sum(t, 0),
-                 lambda: singa.AddRow(t, t), lambda: t.__imul__(2.0)):
+    for call in (lambda: singa.SoftMax(t), lambda: singa.Sum(t, 0), lambda: singa.AddRow(t, t), lambda: t.__imul__(2.0)):
         with pytest.raises(singa.SingaHipError, match="float32"):
+            call()
+    # functions that exist for float32 and the 16-bit types refuse an int tensor the same way
+    i = singa.from_device_pointer(0x1000, (4, 8), _NoDevice(), singa.kInt)
+    for call in (lambda: singa.ReLU(i), lambda: singa.Mult(i, i.T()), lambda: singa.ReLUBackward(i, i)):
+        with pytest.raises(singa.SingaHipError, match="unsupported data type"):
             call()
 
 

@@ -96,6 +96,125 @@ def test_relu_backward_add_mult_axpy(singa, dev, kind, n):
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("n", SIZES)
+def test_relu_forward_16bit(singa, dev, kind, n):
+    """ReLU on a half tensor (src/core/tensor/math_kernel.cu:242-251: in > 0 ? in : 0): a select on the
+    stored values, so exact; -0.0, NaN and negative values give +0."""
+    xt, x = _to(singa, dev, _special(rng(77 + n), n), kind)
+    _same_bits(singa.ReLU(xt).to_numpy(), np.where(x > 0, x, np.float32(0)), "relu_fwd " + kind)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("batch,dim", [(1, 1), (3, 10), (128, 10), (64, 1000), (5, 4097)])
+def test_softmax_cross_entropy_backward_16bit(singa, dev, kind, batch, dim):
+    """SoftmaxCrossEntropyBwd on half probabilities (src/core/tensor/math_kernel.cu:588-611): the fp32
+    oracle applied to the stored values, its result rounded once -- bit for bit; label handling as in fp32
+    (index targets, array targets normalised by their row sum, out-of-range labels flagged and skipped)."""
+    from oracle import cpu_oracle as O
+    r = rng(batch * 31 + dim)
+    logits = r.standard_normal((batch, dim)).astype(np.float32)
+    p32 = np.exp(logits - logits.max(axis=1, keepdims=True))
+    p32 = (p32 / p32.sum(axis=1, keepdims=True)).astype(np.float32)
+    pt, p = _to(singa, dev, p32, kind)
+    labels = r.integers(0, dim, size=batch).astype(np.int32)
+    lt = singa.Tensor((batch,), dev, singa.kInt)
+    lt.CopyIntDataFromHostPtr(labels)
+    for scale in (1.0, 1.0 / batch):
+        want = O.softmax_ce_bwd(p, labels) * np.float32(scale)
+        _same_bits(singa.SoftmaxCrossEntropyBwd(pt, lt, scale).to_numpy(), _round(singa, want, kind),
+                   "softmax-CE bwd, index target, " + kind)
+    assert singa.LabelErrors(dev) == 0
+    # array target (multi-hot rows, each normalised by its sum); with dim == 1 the reference cannot tell it from an
+    # index target (int_target = t.Size() == batch, src/core/tensor/tensor.cc:1741-1758)
+    if dim > 1:
+        hot = (r.random((batch, dim)) < 0.3).astype(np.int32)
+        hot[np.arange(batch), labels] = 1          # no empty row
+        ht = singa.Tensor((batch, dim), dev, singa.kInt)
+        ht.CopyIntDataFromHostPtr(hot)
+        want = O.softmax_ce_bwd(p, hot)
+        _same_bits(singa.SoftmaxCrossEntropyBwd(pt, ht).to_numpy(), _round(singa, want, kind),
+                   "softmax-CE bwd, array target, " + kind)
+    # a label out of range leaves its row as p and is counted
+    if batch >= 3:
+        bad = labels.copy()
+        bad[1] = dim
+        bad[2] = -1
+        lt.CopyIntDataFromHostPtr(bad)
+        got = singa.SoftmaxCrossEntropyBwd(pt, lt).to_numpy()
+        _same_bits(got[1:3], p[1:3], "rows of out-of-range labels")
+        assert singa.LabelErrors(dev) == 2
+
+
+def _gemm_case(singa, dev, kind, M, N, K, tA, tB, r):
+    """A (M x K) and B (K x N) as the stored matrices a transposed view reads: [K][M] / [N][K]."""
+    a32 = (r.standard_normal((M, K)) / np.sqrt(max(K, 1))).astype(np.float32)
+    b32 = r.standard_normal((K, N)).astype(np.float32)
+    at, a = _to(singa, dev, np.ascontiguousarray(a32.T) if tA else a32, kind)
+    bt, b = _to(singa, dev, np.ascontiguousarray(b32.T) if tB else b32, kind)
+    A = at.T() if tA else at
+    B = bt.T() if tB else bt
+    got = singa.Mult(A, B)
+    assert got.data_type() == at.data_type() and got.shape() == [M, N]
+    want = (a.T if tA else a).astype(np.float64) @ (b.T if tB else b).astype(np.float64)
+    return got, want
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 7, 3), (64, 64, 32), (65, 63, 33), (128, 1000, 2048), (128, 2048, 1000),
+                                   (2048, 1000, 128), (100, 10, 4096), (3, 130, 257)])
+def test_gemm_16bit(singa, dev, kind, M, N, K):
+    """Mult on half matrices (cublasHgemm in the reference, tensor_math_cuda.h:1163-1187) for the four
+    transpose combinations: exact products of the stored values accumulated in fp32, one rounding -- held to
+    1e-2 normalised L2 against float64 (observed: the rounding of the result, 3e-4 / 2.5e-3), and to the
+    rounded float64 result within two units of the storage type's last place element by element."""
+    from util import nl2
+    r = rng(M * 7 + N * 3 + K)
+    for tA in (False, True):
+        for tB in (False, True):
+            got, want = _gemm_case(singa, dev, kind, M, N, K, tA, tB, r)
+            g = got.to_numpy().astype(np.float64)
+            assert nl2(g, want) <= 1e-2, (tA, tB, nl2(g, want))
+            ulp = (2.0 ** -10 if kind == "f16" else 2.0 ** -7) * np.maximum(np.abs(want), 1e-3)
+            assert np.all(np.abs(g - want) <= 2 * ulp + 1e-4), (tA, tB, float(np.max(np.abs(g - want) / ulp)))
+    # run-to-run identical, and a unit matrix reproduces the other operand bit for bit
+    r = rng(5)
+    eye = np.eye(64, dtype=np.float32)
+    b32 = r.standard_normal((64, 96)).astype(np.float32)
+    et, _ = _to(singa, dev, eye, kind)
+    bt, b = _to(singa, dev, b32, kind)
+    _same_bits(singa.Mult(et, bt).to_numpy(), b, "I * B")
+    _same_bits(singa.Mult(et, bt).to_numpy(), singa.Mult(et, bt).to_numpy(), "run to run")
+
+
+def test_gemm_16bit_alpha_beta_and_pitches(singa, dev):
+    """The C ABI directly: alpha / beta in fp32, row pitches larger than the rows, unaligned pointers
+    (the element-wise staging path) against float64."""
+    import ctypes as C
+    from singa_amd import _lib
+    r = rng(9)
+    M, N, K, lda, ldb, ldc = 37, 29, 45, 51, 33, 40
+    A = r.standard_normal((M, lda)).astype(np.float16)
+    B = r.standard_normal((K, ldb)).astype(np.float16)
+    C0 = r.standard_normal((M, ldc)).astype(np.float16)
+    # one leading element of padding makes every base pointer 2-byte aligned only
+    def dev_of(a):
+        t = singa.from_numpy(np.concatenate([[np.float16(0)], a.ravel()]).astype(np.float16), dev)
+        return t, t.ptr + 2
+    at, ap = dev_of(A)
+    bt, bp = dev_of(B)
+    ct, cp = dev_of(C0)
+    _lib.check(_lib.lib().sgh_gemm_f16(0, 0, M, N, K, 0.5, ap, lda, bp, ldb, -2.0, cp, ldc, dev.stream), "sgh_gemm_f16")
+    got = ct.to_numpy()[1:].reshape(M, ldc).astype(np.float64)
+    want = 0.5 * (A[:, :K].astype(np.float64) @ B[:, :N].astype(np.float64)) - 2.0 * C0[:, :N].astype(np.float64)
+    assert np.max(np.abs(got[:, :N] - want)) <= 2.0 ** -9 * np.max(np.abs(want)) + 1e-3
+    # the padding columns of C are untouched
+    assert np.array_equal(got[:, N:], C0[:, N:].astype(np.float64))
+    # bad arguments are rejected on the host
+    assert _lib.lib().sgh_gemm_f16(0, 0, M, N, K, 1.0, ap, K - 1, bp, ldb, 0.0, cp, ldc, dev.stream) < 0
+    assert _lib.lib().sgh_gemm_f16(0, 0, M, N, K, 1.0, ap, lda, bp, ldb, 0.0, cp, N - 1, dev.stream) < 0
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 28, 28), (16, 32, 8, 8), (3, 7, 4, 2),
                                    (16, 24, 14, 14), (2, 8, 6, 6),    # these two: planes of 8-byte vectors
                                    (8, 128, 14, 14), (16, 256, 7, 7), (4, 130, 5, 6), (32, 128, 8, 8),   # one-pass backward

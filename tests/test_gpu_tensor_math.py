@@ -409,8 +409,15 @@ def test_row_max_dot_and_sum(singa, dev):
     r = rng(33)
     for rows, cols in [(1, 1), (3, 7), (128, 1000), (17, 4097)]:
         m = randn(r, rows, cols)
-        m[0] = -np.abs(m[0]) - 1          # an all-negative row: the maximum starts at 0
-        assert_bit_equal(singa.RowMax(singa.from_numpy(m, dev)).to_numpy(), O.row_max(m), "row max")
+        m[0] = -np.abs(m[0]) - 1          # an all-negative row, where the reference's two backends differ
+        md = singa.from_numpy(m, dev)
+        # the CPU function seeds the maximum with 0 (tensor_math_cpp.h:1132): the oracle's rule
+        assert_bit_equal(singa.RowMax(md, cpu_rule=True).to_numpy(), O.row_max(m), "row max, CPU rule")
+        assert singa.RowMax(md, cpu_rule=True).to_numpy()[0] == 0.0
+        # the accelerator kernel seeds it with the row's first element (math_kernel.cu:488-499): the true
+        # maximum, which is the default here
+        assert_bit_equal(singa.RowMax(md).to_numpy(), m.max(axis=1), "row max, accelerator rule")
+        assert singa.RowMax(md).to_numpy()[0] < 0.0
     for n in (1, 100, 4096, 4097, 1 << 20, 5 * (1 << 20) + 3):
         a, b = randn(r, n), randn(r, n)
         ad, bd = singa.from_numpy(a, dev), singa.from_numpy(b, dev)
@@ -461,3 +468,24 @@ def test_clamp_and_the_half_precision_trip_of_a_gradient(singa, dev):
         assert np.array_equal(out[1:], want[1:].astype(np.float16).astype(np.float32))
     big = singa.from_numpy(np.array([70000.0, -1e-9, 3.0], np.float32), dev)
     assert np.array_equal(sgd.through_half(big).to_numpy(), np.array([np.inf, -0.0, 3.0], np.float32))   # no clipping: overflow
+
+
+def test_int_float_casts(singa, dev):
+    """AsType between float and int tensors (CastCopy<float, int> / <int, float>,
+    src/core/tensor/math_kernel.cu:280-292): (int)x truncates toward zero, (float)i rounds to nearest even."""
+    r = rng(41)
+    for n in (1, 5, 4097, 1 << 20):
+        f = (r.standard_normal(n) * 1000).astype(np.float32)
+        f[: min(n, 6)] = [0.5, -0.5, 1.999, -1.999, -0.0, 2147483520.0][: min(n, 6)]
+        it = singa.from_numpy(f, dev).AsType(singa.kInt)
+        assert it.data_type() == singa.kInt
+        assert np.array_equal(it.to_numpy(), np.trunc(f.astype(np.float64)).astype(np.int64).astype(np.int32))
+        i = r.integers(-2 ** 31, 2 ** 31 - 1, size=n, dtype=np.int64).astype(np.int32)
+        i[: min(n, 4)] = [0, -1, 16777217, -2 ** 31][: min(n, 4)]
+        t = singa.Tensor((n,), dev, singa.kInt)
+        t.CopyIntDataFromHostPtr(i)
+        assert_bit_equal(t.AsType(singa.kFloat32).to_numpy(), i.astype(np.float32), "int -> float")
+    # out of range saturates, NaN becomes 0 (the conversion instruction's rule; C leaves both undefined)
+    edge = np.array([3e9, -3e9, np.inf, -np.inf, np.nan], dtype=np.float32)
+    got = singa.from_numpy(edge, dev).AsType(singa.kInt).to_numpy()
+    assert got.tolist() == [2 ** 31 - 1, -2 ** 31, 2 ** 31 - 1, -2 ** 31, 0]
