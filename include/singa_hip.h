@@ -36,6 +36,8 @@ extern "C" {
 #define SGH_ELABEL (-4)     /* a class label was out of range (checked variant only) */
 #define SGH_ENOMEM (-5)
 #define SGH_ELIMIT (-6)     /* size beyond the fixed scratch of a non-allocating entry point */
+#define SGH_EEXCHANGE (-7)  /* a one-pass BatchNorm kernel's workgroups gave up waiting for each other (see
+                               sgh_bn_exchange_failures); returned by sgh_device_sync */
 
 /* Human-readable text for a return code (static storage). */
 SGH_API const char *sgh_error_string(int rc);
@@ -80,7 +82,9 @@ SGH_API void *sgh_device_aux_stream(sgh_device *dev);
 SGH_API int sgh_device_fork(sgh_device *dev, void **aux_stream);
 SGH_API int sgh_device_join(sgh_device *dev);
 SGH_API int sgh_block_used_on(sgh_device *dev, void *ptr, void *stream);
-/* Device::Sync (src/core/device/cuda_gpu.cc:206-209): blocks until the device's streams are idle. */
+/* Device::Sync (src/core/device/cuda_gpu.cc:206-209): blocks until the device's streams are idle.
+ * Returns SGH_EEXCHANGE (once) if a one-pass BatchNorm kernel that ran since the last look could not
+ * complete its exchange -- the outputs of that call are NaN; see sgh_bn_exchange_failures. */
 SGH_API int sgh_device_sync(sgh_device *dev);
 
 /* DeviceMemPool::Malloc / Free (include/singa/core/memory.h:41-45).  Size-bucketed cache:
@@ -461,9 +465,13 @@ SGH_API int sgh_conv_dgrad_acc_supported(const sgh_conv_geom *g);
  * weights.  The layer's next data gradient (sgh_conv_dgrad_*, sgh_conv_dgrad_acc_f32) skips its
  * own re-layout if, and only if, the note still holds: same W pointer, same workspace, and no
  * call since the prepare that may have changed a weight tensor -- every sgh_sgd_momentum_*,
- * sgh_axpy_*, sgh_memset_* and host-to-device / device-to-device sgh_memcpy call advances the
- * library's weight epoch, and so does sgh_conv_weights_changed(), which a caller that writes
- * weights by other means (its own kernels, a cast into a weight tensor) calls.  Otherwise the data gradient re-lays the weights
+ * sgh_axpy_*, sgh_memset_*, random fill, host-to-device / device-to-device sgh_memcpy,
+ * sgh_upload_async and sgh_graph_launch call (a recording may hold an update) advances the
+ * library's weight epoch; the elementwise entry points with an output tensor (sgh_add_*,
+ * sgh_sub_f32, sgh_div_f32, sgh_eltwise_mult_*, the scalar forms, sgh_clamp_f32, the casts)
+ * advance it when their output lies inside a prepared weight tensor (Tensor `*=` / `+=` on a
+ * weight); and so does sgh_conv_weights_changed(), which a caller that writes weights by other
+ * means (its own kernels) calls.  Otherwise the data gradient re-lays the weights
  * itself, as without a prepare.  A note is used once: the data gradient that reads it, and any
  * forward pass or weight gradient of the same geometry whose workspace overlaps the prepared one,
  * removes it.  The workspaces listed must be private to their layer from the prepare call to the
@@ -595,6 +603,22 @@ SGH_API int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma,
                            const float *save_mean, const float *save_invstd, float *dx,
                            float *dgamma, float *dbeta, int N, int C, int HW, void *workspace,
                            size_t ws_bytes, void *stream);
+/* The one-pass BatchNorm kernels (forward and backward; they read x, or x and dy, once) cut a channel
+ * into slices, one workgroup per slice, and the workgroups of a channel exchange their partial sums
+ * through the workspace while all of them are resident on the GPU.  That needs every slice of the oldest
+ * unfinished channel to be running: the plan only uses these kernels when that many workgroups fit the
+ * device at once (otherwise the two-pass kernels run), and workgroups are dispatched in index order.  The
+ * wait is bounded all the same: a workgroup that has polled `polls` times gives up, the channel's outputs
+ * become NaN, every kernel still ends normally, and a device-side counter records it.
+ *   sgh_bn_exchange_failures    waits for `stream`, returns the number of workgroups that gave up since
+ *                               the last look and clears it (sgh_device_sync looks too and returns
+ *                               SGH_EEXCHANGE).  0 in normal operation.
+ *   sgh_bn_exchange_spin_limit  sets `polls` for later launches (process-wide; <= 0 restores the default
+ *                               of 2^20).  For tests of the failure path: with a limit of 1 the first
+ *                               slices of a many-slice channel give up.
+ * No counterpart in the reference (cuDNN's kernels are closed). */
+SGH_API int sgh_bn_exchange_failures(void *stream, int *count);
+SGH_API void sgh_bn_exchange_spin_limit(int polls);
 /* sgh_bn_bwd_f32 for callers that cannot allocate device memory and have no workspace to pass
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  Same kernels, same results bit for bit; the per-channel partial

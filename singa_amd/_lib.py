@@ -175,6 +175,8 @@ SIGNATURES = {
     "sgh_conv_fwd_f16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
     "sgh_conv_fwd_bf16": (C.c_int, [C.POINTER(ConvGeom), vp, vp, vp, vp, vp, sz, vp]),
     "sgh_bn_workspace_bytes": (sz, [C.c_int, C.c_int, C.c_int]),
+    "sgh_bn_exchange_failures": (C.c_int, [vp, C.POINTER(C.c_int)]),
+    "sgh_bn_exchange_spin_limit": (None, [C.c_int]),
     "sgh_bn_fwd_train_f32": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
                                        C.c_int, C.c_int, vp, sz, vp]),
     "sgh_bn_relu_fwd_train_f32": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, C.c_float, vp, vp, vp, C.c_int,
@@ -212,6 +214,7 @@ SIGNATURES = {
 SGH_CONV_FWD, SGH_CONV_DGRAD, SGH_CONV_WGRAD = 0, 1, 2
 SGH_EUNSUPPORTED = -3
 SGH_ELIMIT = -6
+SGH_EEXCHANGE = -7
 
 
 class SingaHipError(RuntimeError):

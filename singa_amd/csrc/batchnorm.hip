@@ -475,9 +475,18 @@ __global__ __launch_bounds__(kResNT) void k_bn_bwd_resident(const typename S::el
 // channel's outputs become NaN.
 // x and dy are read once and dx written once: 3 tensor passes instead of 5.
 constexpr int kChipMaxG = 128, kChipSpinLimit = 1 << 20;
+// workgroups that gave up waiting for the other slices of their channel since the counter was last read
+// (sgh_bn_exchange_failures; sgh_device_sync reports it as SGH_EEXCHANGE)
+__device__ int g_bn_gave_up = 0;
+// the number of polls after which a workgroup gives up: kChipSpinLimit unless a test lowered it
+std::atomic<int> g_spin_limit{kChipSpinLimit};
+// set by every launch of a one-pass kernel whose channels have several slices: the counter is read back (a small
+// blocking copy) only when one has run since the last look
+std::atomic<bool> g_exchange_ran{false};
 #ifndef BN_CHIP_NL_ON
 #define BN_CHIP_NL_ON 1
 #endif
+
 // vectors per tensor and thread: 8 (64 registers of raw data), 5 for 16-byte vectors of 16-bit elements,
 // whose eight conversions per vector need more registers beside the data
 template <class S>
@@ -501,6 +510,17 @@ struct ChipPlan {
   int nl;           // vectors per tensor and thread kept in LDS (0: registers only)
   bool ragged;      // planes that are not whole vectors (7 x 7): see RAGGED in k_bn_bwd_onchip
 };
+
+// The exchange only terminates if all G workgroups of the oldest unfinished channel are running together.  A
+// 512-thread workgroup of these kernels fits twice on a CU (registers and LDS are budgeted for that), a
+// 1024-thread one once; with a run of channels per XCD (`xcd_runs` in the launchers: G <= 16 and C >= 8) the G
+// slices of a channel all land on one XCD, an eighth of the CUs.  A device with fewer CUs than that (a
+// partition) gets the two-pass kernels instead.
+inline bool chip_slices_fit(int G, int C, int nt) {
+  const long slots = long(sgh_num_cus()) * (nt == 512 ? 2 : 1);
+  const bool xcd_runs = G <= 16 && C >= 8;
+  return xcd_runs ? long(G) <= slots / 8 : long(G) <= slots;
+}
 
 template <class S>
 inline ChipPlan chip_plan(int N, int C, int HW) {
@@ -526,19 +546,21 @@ inline ChipPlan chip_plan(int N, int C, int HW) {
     G = (TV + long(p.nt) * per_thread - 1) / (long(p.nt) * per_thread);
   }
   p.nl = p.nt == 512 && lds_ok ? chip_nl<S>() : 0;
-  // few channels: thinner slices, so that there are two workgroups for every CU (at least one wavefront of vectors each)
-  const long want = (2L * sgh_num_cus() + C - 1) / C;
+  // few channels: thinner slices, so that there are two workgroups for every CU (at least one wavefront of vectors
+  // each) -- unless a channel fits one workgroup and there is a channel for every CU: then nothing is exchanged
+  const bool whole_channels = G == 1 && C >= sgh_num_cus();
+  const long want = whole_channels ? 1 : (2L * sgh_num_cus() + C - 1) / C;
   if (G < want) G = want;
   // whole rounds: as many slices as still fit into the rounds of (2 workgroups x CUs) that this many need
   const long slots = 2L * sgh_num_cus(), rounds = (long(C) * G + slots - 1) / slots;
   long fill = rounds * slots / C;
   if (fill > kChipMaxG) fill = kChipMaxG;
-  if (fill > G) G = fill;
+  if (fill > G && !whole_channels) G = fill;
   while (G > 1 && (TV + G - 1) / G < 64) --G;
   if (G > kChipMaxG || G < 1) return p;
   p.vpg = int((TV + G - 1) / G);
   p.G = int((TV + p.vpg - 1) / p.vpg);
-  p.ok = long(C) * p.G < 0x7fffffffL && !(p.ragged && p.nt != 512);
+  p.ok = long(C) * p.G < 0x7fffffffL && !(p.ragged && p.nt != 512) && chip_slices_fit(p.G, C, p.nt);
   return p;
 }
 
@@ -555,7 +577,8 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
                                                           typename S::elem *__restrict__ dx, float *__restrict__ dgamma,
                                                           float *__restrict__ dbeta, unsigned long long *__restrict__ ws,
                                                           BnShape s, int G, int vpg, unsigned long long ticket1,
-                                                          unsigned long long ticket2, int spin_limit, int xcd_runs) {
+                                                          unsigned long long ticket2, int spin_limit, int xcd_runs,
+                                                          int dephase_ticks) {
   typedef typename S::elem elem;
   constexpr int V = S::VEC, NV = chip_nv<S>();
   typedef typename RawVec<V * sizeof(elem)>::type raw;
@@ -569,6 +592,17 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
   const int unit = xcd_runs ? int(blockIdx.x & 7) * int(gridDim.x >> 3) + int(blockIdx.x >> 3) : int(blockIdx.x);
   const int c = unit / G, g = unit - c * G, t = threadIdx.x;
   if (c >= s.C) return;
+  // Launches of many rounds: all workgroups of the first round start together and stay in step -- everybody loads,
+  // then everybody waits for the exchange, then everybody stores -- and the later rounds inherit the rhythm, so the
+  // memory system idles through every exchange.  The odd channels of the first round start `dephase_ticks` (of the
+  // 100 MHz wall clock) late; from then on one half of the chip loads while the other half exchanges and stores.
+  if (dephase_ticks > 0 && int(blockIdx.x) < int(2 * 256) && (c & 1)) {
+    if (t == 0) {
+      const unsigned long long t0 = wall_clock64();
+      while (wall_clock64() - t0 < (unsigned long long)(dephase_ticks)) __builtin_amdgcn_s_sleep(16);
+    }
+    __syncthreads();
+  }
   unsigned long long *words = ws + size_t(c) * 2 * size_t(G);   // the channel's G slots
   if (G > 1 && t == 0) {
     const unsigned long long wa = __hip_atomic_load(words + 2 * g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -709,7 +743,10 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     // the same G numbers in the same order in every workgroup of the channel
     db = 0.f, dg = 0.f;
     for (int i = 0; i < G; ++i) db += part_a[i], dg += part_b[i];
-    if (gave_up) db = dg = __builtin_nanf("");
+    if (gave_up) {
+      db = dg = __builtin_nanf("");
+      if (t == 0) atomicAdd(&g_bn_gave_up, 1);
+    }
   }
   if (g == 0 && t == 0) {
     dbeta[c] = db;
@@ -731,8 +768,8 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     S::store16(reinterpret_cast<elem *>(&ov), o);                                                             \
     if constexpr (RAGGED)                                                                                     \
       __builtin_amdgcn_raw_buffer_store_b128(ov, rob, piece(n, r), 0, 0);                                     \
-    else                                                                                                      \
-      og[(size_t(n) * s.C + c) * PV + r] = ov;                                                                \
+    else   /* (non-temporal: 3-7 % on the 25-50 MB tensors, whose lines otherwise wait dirty in L2 for the end of the kernel) */ \
+      __builtin_nontemporal_store(ov, og + (size_t(n) * s.C + c) * PV + r);                                   \
   }
   if constexpr (NL > 0) {
 #pragma unroll
@@ -783,7 +820,7 @@ inline ChipPlan chip_fwd_plan(int N, int C, int HW, bool two) {
   if (G > kChipMaxG || G < 1) return p;
   p.vpg = int((TV + G - 1) / G);
   p.G = int((TV + p.vpg - 1) / p.vpg);
-  p.ok = long(C) * p.G < 0x7fffffffL;
+  p.ok = long(C) * p.G < 0x7fffffffL && chip_slices_fit(p.G, C, 512);
   return p;
 }
 
@@ -898,7 +935,10 @@ __global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem
   if (var < 0) var = 0;
   float mean = float(double(pivot) + dm);
   const float invstd = float(1.0 / sqrt(var + double(eps)));
-  if (G > 1 && gave_up) mean = __builtin_nanf("");
+  if (G > 1 && gave_up) {
+    mean = __builtin_nanf("");
+    if (t == 0) atomicAdd(&g_bn_gave_up, 1);
+  }
   if (g == 0 && t == 0) {
     save_mean[c] = mean;
     save_invstd[c] = invstd;
@@ -949,9 +989,10 @@ int launch_fwd_onchip(const typename S::elem *x, const typename S::elem *z, cons
   const int xcd_runs = p.G <= 16 && s.C >= 8 ? 1 : 0;
   const dim3 grid(xcd_runs ? unsigned((s.C + 7) / 8) * 8u * p.G : unsigned(s.C) * p.G);
   const unsigned long long t1 = next_ticket(), t2 = next_ticket();
+  if (p.G > 1) g_exchange_ran.store(true, std::memory_order_relaxed);
   hipLaunchKernelGGL((k_bn_fwd_onchip<S, ACT>), grid, dim3(512), 0, st, x, z, gamma, beta, running_mean, running_var, factor,
                      eps, y, save_mean, save_invstd, static_cast<unsigned long long *>(workspace), s, p.G, p.vpg, t1, t2,
-                     kChipSpinLimit, xcd_runs);
+                     g_spin_limit.load(std::memory_order_relaxed), xcd_runs);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -963,7 +1004,13 @@ int launch_onchip(const typename S::elem *dy, const typename S::elem *x, const f
   // (a run of channels per XCD needs the G workgroups of a channel resident on one XCD's 32 CUs together)
   const int xcd_runs = p.G <= 16 && s.C >= 8 ? 1 : 0;
   const dim3 grid(xcd_runs ? unsigned((s.C + 7) / 8) * 8u * p.G : unsigned(s.C) * p.G);
+  // from four rounds on, half of the first round starts 6 us late (fp32 64 x 64 x 112 x 112, seven rounds: 135 -> 128 us;
+  // two-round launches lose: 64 x 64 x 56 x 56 36 -> 41 us); SGH_BN_DEPHASE_US overrides the delay (0: off)
+  static const int dephase_env = getenv("SGH_BN_DEPHASE_US") ? atoi(getenv("SGH_BN_DEPHASE_US")) : 6;
+  const long rounds = (long(s.C) * p.G + 2L * sgh_num_cus() - 1) / (2L * sgh_num_cus());
+  const int dephase = p.G > 1 && rounds >= 4 && p.nt == 512 ? dephase_env * 100 : 0;
   const unsigned long long t1 = next_ticket(), t2 = next_ticket();
+  if (p.G > 1) g_exchange_ran.store(true, std::memory_order_relaxed);
   if constexpr (chip_nl<S>() > 0) {
     if (p.nl > 0) {
       constexpr int NL = chip_nl<S>();
@@ -977,24 +1024,24 @@ int launch_onchip(const typename S::elem *dy, const typename S::elem *x, const f
         attr = true;
       }
       hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, ws,
-                         s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
+                         s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
       return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
     }
   }
   if constexpr (S::VEC * sizeof(typename S::elem) == 16) {
     if (p.ragged) {
       hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512, 0, true>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean,
-                         save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
+                         save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
       return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
     }
   }
   if (p.ragged) return SGH_EUNSUPPORTED;
   if (p.nt == 512)
     hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean, save_invstd,
-                       dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
+                       dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
   else
     hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 1024>), grid, dim3(1024), 0, st, dy, x, gamma, beta, save_mean,
-                       save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, kChipSpinLimit, xcd_runs);
+                       save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -1045,26 +1092,57 @@ inline BnShape make_shape(int N, int C, int HW, int vec, int esize) {
   return s;
 }
 
-// bytes of workspace the backward pass of storage class S needs: the partial sums of the two-pass
-// kernels or the slots of the one-pass kernel, whichever the shape takes
+// Layout of a BatchNorm workspace (sgh_bn_workspace_bytes), three parts, each a multiple of 256 bytes:
+//   [0, twopass)            partial sums of the two-pass kernels, forward and backward, any storage type
+//   [twopass, + bwd words)  exchange words of the one-pass backward kernel
+//   [.., + fwd words)       exchange words of the one-pass forward kernel
+// A recorded one-pass launch tells which of its two tickets is next from what its own words hold, so every word
+// of a channel must be written by that kernel only between two replays: each one-pass kernel owns its part, and
+// nothing else writes there (a two-pass forward on the same handle between two replays of a recorded backward
+// used to overwrite the head of the backward words while they shared offset 0).
+inline size_t round256(size_t v) { return (v + 255) & ~size_t(255); }
+
+inline size_t twopass_workspace_bytes(int N, int C, int HW) {
+  const int s4 = make_shape(N, C, HW, 4, 4).S, s8 = make_shape(N, C, HW, 8, 2).S, s4h = make_shape(N, C, HW, 4, 2).S;
+  const int smax = s4 > s8 ? (s4 > s4h ? s4 : s4h) : (s8 > s4h ? s8 : s4h);
+  return round256(size_t(C) * smax * 2 * sizeof(float));
+}
+
+template <class S>
+inline size_t bwd_words_bytes_of(int N, int C, int HW) {
+  const ChipPlan cp = chip_plan<S>(N, C, HW);
+  return cp.ok ? chip_workspace_bytes(C, cp.G) : 0;
+}
+
+inline size_t bwd_words_bytes(int N, int C, int HW) {
+  const size_t b[3] = {bwd_words_bytes_of<StF32>(N, C, HW), bwd_words_bytes_of<StF16>(N, C, HW),
+                       bwd_words_bytes_of<StF16x4>(N, C, HW)};
+  size_t need = 0;
+  for (size_t v : b) need = v > need ? v : need;
+  return round256(need);
+}
+
+// where the one-pass forward kernel's words start
+inline size_t shared_workspace_bytes(int N, int C, int HW) {
+  return twopass_workspace_bytes(N, C, HW) + bwd_words_bytes(N, C, HW);
+}
+
+// bytes of workspace the backward pass of storage class S needs: the partial sums of the two-pass kernels, and
+// behind that part the words of the one-pass kernel where the shape takes it
 template <class S>
 inline size_t bwd_workspace_need(int N, int C, int HW) {
   const size_t two_pass = size_t(C) * make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem))).S * 2 * sizeof(float);
-  const ChipPlan cp = chip_plan<S>(N, C, HW);
-  const size_t chip = cp.ok ? chip_workspace_bytes(C, cp.G) : 0;
+  const size_t words = bwd_words_bytes_of<S>(N, C, HW);
+  const size_t chip = words ? twopass_workspace_bytes(N, C, HW) + words : 0;
   return two_pass > chip ? two_pass : chip;
 }
 
-// the part of a workspace that the two-pass kernels and the backward pass of every storage type use, a multiple
-// of 256 bytes (one size for every storage type: the largest of the fp32 and the 16-bit needs)
-inline size_t shared_workspace_bytes(int N, int C, int HW) {
-  const int s4 = make_shape(N, C, HW, 4, 4).S, s8 = make_shape(N, C, HW, 8, 2).S, s4h = make_shape(N, C, HW, 4, 2).S;
-  const int smax = s4 > s8 ? (s4 > s4h ? s4 : s4h) : (s8 > s4h ? s8 : s4h);
-  size_t need = size_t(C) * smax * 2 * sizeof(float);   // (the two-pass forward and backward)
-  const size_t b[3] = {bwd_workspace_need<StF32>(N, C, HW), bwd_workspace_need<StF16>(N, C, HW),
-                       bwd_workspace_need<StF16x4>(N, C, HW)};
-  for (size_t v : b) need = v > need ? v : need;
-  return (need + 255) & ~size_t(255);
+// the same for a caller that keeps the words at the start of a buffer of its own (sgh_bn_bwd_noalloc_f32)
+template <class S>
+inline size_t bwd_workspace_need_flat(int N, int C, int HW) {
+  const size_t two_pass = size_t(C) * make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem))).S * 2 * sizeof(float);
+  const size_t words = bwd_words_bytes_of<S>(N, C, HW);
+  return two_pass > words ? two_pass : words;
 }
 
 template <class S, int ACT>
@@ -1130,12 +1208,16 @@ int bn_fwd_infer(const typename S::elem *x, const float *gamma, const float *bet
 template <class S>
 int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *gamma, const float *beta,
            const float *save_mean, const float *save_invstd, typename S::elem *dx, float *dgamma, float *dbeta, int N,
-           int C, int HW, void *workspace, size_t ws_bytes, void *stream) {
+           int C, int HW, void *workspace, size_t ws_bytes, void *stream, bool flat_workspace = false) {
   if (!shape_ok(N, C, HW) || !dy || !x || !gamma || !save_mean || !save_invstd || !dx || !dgamma || !dbeta)
     return SGH_EINVAL;
   if (!sgh_aligned16(x) || !sgh_aligned16(dy) || !sgh_aligned16(dx)) return SGH_EINVAL;
   const BnShape s = make_shape(N, C, HW, S::VEC, int(sizeof(typename S::elem)));
-  if (!workspace || ws_bytes < bwd_workspace_need<S>(N, C, HW)) return SGH_EWORKSPACE;
+  if (!workspace || ws_bytes < (flat_workspace ? bwd_workspace_need_flat<S>(N, C, HW) : bwd_workspace_need<S>(N, C, HW)))
+    return SGH_EWORKSPACE;
+  // the one-pass kernel's words: a part of their own behind the two-pass partial sums (see the layout above);
+  // `flat_workspace`: at the start of a buffer whose owner clears them before every call
+  void *words = flat_workspace ? workspace : static_cast<char *>(workspace) + twopass_workspace_bytes(N, C, HW);
   float *part = static_cast<float *>(workspace);
   const dim3 grid(C * s.S), block(kBlock);
   hipStream_t st = sgh_stream_of(stream);
@@ -1147,12 +1229,15 @@ int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *g
   // (ragged planes of few elements -- 7 x 7 -- as well, unless the channels need more than two rounds of its
   // one workgroup per channel: f16 128 x 512 x 7 x 7 13.3 us there, 13.9 here, but 128 x 2048 x 7 x 7 42.6 against
   // 23.7 -- the LDS-resident kernel moves single elements)
-  const bool small_resident = resident_ok(N, C, HW, sizeof(typename S::elem)) &&
+  // (fp32 shapes that give every CU a whole channel -- no exchange, G = 1 -- run faster in registers: 64 x 256 x 14 x 14
+  // 11.5 -> 10.2 us, 64 x 512 x 7 x 7 10.2 -> 7.7 us, kernels alone on cold tensors)
+  const bool small_resident = !(cp.ok && cp.G == 1 && sizeof(typename S::elem) == 4) &&
+                              resident_ok(N, C, HW, sizeof(typename S::elem)) &&
                               (cp.ragged ? HW <= 64 && C <= 2 * sgh_num_cus() : long(N) * (HW / S::VEC) <= 4096);
   if (cp.ok && !small_resident && !sgh_env().bn_onchip_off) {
     if (!sgh_aligned16(workspace)) return SGH_EINVAL;
-    return beta ? launch_onchip<S, true>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, workspace, s, cp, st)
-                : launch_onchip<S, false>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, workspace, s, cp, st);
+    return beta ? launch_onchip<S, true>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, words, s, cp, st)
+                : launch_onchip<S, false>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, words, s, cp, st);
   }
   if (resident_ok(N, C, HW, sizeof(typename S::elem))) {
     const int rc = beta ? launch_resident<S, true>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, s, st)
@@ -1202,12 +1287,40 @@ int noalloc_scratch_of_current_device(float **out) {
 
 }  // namespace
 
+// Reads and clears the give-up counter of the current device if a multi-slice one-pass kernel has been launched
+// since the last look (so a caller that never runs one pays nothing); the stream(s) must be idle.
+int sgh_bn_take_exchange_failures(int *count) {
+  *count = 0;
+  if (!g_exchange_ran.exchange(false, std::memory_order_relaxed)) return SGH_OK;
+  int v = 0;
+  SGH_HIP_TRY(hipMemcpyFromSymbol(&v, HIP_SYMBOL(g_bn_gave_up), sizeof(int), 0, hipMemcpyDeviceToHost));
+  if (v != 0) {
+    const int zero = 0;
+    SGH_HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(g_bn_gave_up), &zero, sizeof(int), 0, hipMemcpyHostToDevice));
+  }
+  *count = v;
+  return SGH_OK;
+}
+
+void sgh_bn_mark_exchange_ran() { g_exchange_ran.store(true, std::memory_order_relaxed); }
+
 int sgh_bn_noalloc_setup() {
   float *p = nullptr;
   return noalloc_scratch_of_current_device(&p);
 }
 
 extern "C" {
+
+int sgh_bn_exchange_failures(void *stream, int *count) {
+  if (!count) return SGH_EINVAL;
+  SGH_HIP_TRY(hipStreamSynchronize(sgh_stream_of(stream)));
+  g_exchange_ran.store(true, std::memory_order_relaxed);   // (asked for explicitly: always look)
+  return sgh_bn_take_exchange_failures(count);
+}
+
+void sgh_bn_exchange_spin_limit(int polls) {
+  g_spin_limit.store(polls > 0 ? polls : kChipSpinLimit, std::memory_order_relaxed);
+}
 
 size_t sgh_bn_workspace_bytes(int N, int C, int HW) {
   if (!shape_ok(N, C, HW)) return 0;
@@ -1297,8 +1410,10 @@ int sgh_bn_bwd_f32(const float *dy, const float *x, const float *gamma, const fl
 int sgh_bn_bwd_noalloc_f32(const float *dy, const float *x, const float *gamma, const float *save_mean,
                            const float *save_invstd, float *dx, float *dgamma, float *dbeta, int N, int C, int HW,
                            void *stream) {
-  if (!shape_ok(N, C, HW)) return SGH_EINVAL;
-  const size_t need = bwd_workspace_need<StF32>(N, C, HW);
+  if (!shape_ok(N, C, HW) || !dy || !x || !gamma || !save_mean || !save_invstd || !dx || !dgamma || !dbeta)
+    return SGH_EINVAL;
+  if (!sgh_aligned16(x) || !sgh_aligned16(dy) || !sgh_aligned16(dx)) return SGH_EINVAL;   // (before anything is launched)
+  const size_t need = bwd_workspace_need_flat<StF32>(N, C, HW);
   if (need > sizeof(float) * 2 * size_t(kNoAllocMaxPairs)) return SGH_ELIMIT;
   float *part = nullptr;
   const int rc = noalloc_scratch_of_current_device(&part);
@@ -1315,7 +1430,7 @@ int sgh_bn_bwd_noalloc_f32(const float *dy, const float *x, const float *gamma, 
                        reinterpret_cast<unsigned long long *>(part), words);
     SGH_LAUNCH_CHECK();
   }
-  return bn_bwd<StF32>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, part, need, stream);
+  return bn_bwd<StF32>(dy, x, gamma, nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, part, need, stream, true);
 }
 int sgh_bn_bwd_f16(const uint16_t *dy, const uint16_t *x, const float *gamma, const float *save_mean,
                    const float *save_invstd, uint16_t *dx, float *dgamma, float *dbeta, int N, int C, int HW,

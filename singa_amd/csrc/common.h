@@ -49,12 +49,20 @@ bool sgh_stream_is_aux(hipStream_t s);
 // sgh_bn_bwd_noalloc_f32 (batchnorm.hip).  sgh_device_open calls it so that the entry point's first
 // call on a device finds the address ready; the entry point repeats the lookup if it was not.
 int sgh_bn_noalloc_setup();
+// batchnorm.hip: reads and clears the count of workgroups that gave up in a one-pass kernel's exchange (current
+// device, idle streams); and the note that such a kernel may have run without its launch being seen (a graph replay)
+int sgh_bn_take_exchange_failures(int *count);
+void sgh_bn_mark_exchange_ran();
 
 // Weight epoch: a host-side counter that every entry point which may change a weight tensor advances
 // (optimizer updates, Axpy, fills, casts, copies to the device, sgh_conv_weights_changed).  The note that
 // sgh_conv_dgrad_prepare_multi leaves in a geometry is honoured only within the epoch it was written in.
 unsigned long long sgh_weights_epoch();
 void sgh_weights_epoch_bump();
+// a weight tensor whose re-laid copy waits in a workspace / an elementwise entry point is about to write `bytes`
+// at `out`: advances the epoch if that is inside such a weight tensor
+void sgh_prepared_weights_add(const void *W, size_t bytes);
+void sgh_note_write(const void *out, size_t bytes);
 // True when the note in `g` covers a data gradient of storage type `dtype` (0 fp32, 1 binary16, 2 bfloat16)
 // reading weights `W` with workspace `workspace` now.
 bool sgh_prelaid_valid(const sgh_conv_geom *g, int dtype, const void *W, const void *workspace);

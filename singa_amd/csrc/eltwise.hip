@@ -552,35 +552,43 @@ int sgh_cast_i32_to_f32(const int32_t *src, float *dst, size_t n, void *stream) 
 }
 
 int sgh_clamp_f32(float low, float high, const float *x, float *out, size_t n, void *stream) {
+  sgh_note_write(out, n * sizeof(float));
   return launch_map1(x, out, n, ClampOp{low, high}, stream);
 }
 
 int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
+  sgh_note_write(out, n * sizeof(float));
   sgh_prof_scope prof("add/k_map2_1<AddOp>", 3.0 * n * sizeof(float), sgh_stream_of(stream));
   return launch_map2(a, b, out, n, AddOp{}, stream);
 }
 
 int sgh_add_relu_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
+  sgh_note_write(out, n * sizeof(float));
   return launch_map2(a, b, out, n, AddReluOp{}, stream);
 }
 
 int sgh_sub_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
+  sgh_note_write(out, n * sizeof(float));
   return launch_map2(a, b, out, n, SubOp{}, stream);
 }
 
 int sgh_div_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
+  sgh_note_write(out, n * sizeof(float));
   return launch_map2(a, b, out, n, DivOp{}, stream);
 }
 
 int sgh_add_scalar_f32(const float *a, float x, float *out, size_t n, void *stream) {
+  sgh_note_write(out, n * sizeof(float));
   return launch_map1(a, out, n, AddScalarOp{x}, stream);
 }
 
 int sgh_mult_scalar_f32(const float *a, float x, float *out, size_t n, void *stream) {
+  sgh_note_write(out, n * sizeof(float));
   return launch_map1(a, out, n, MulScalarOp{x}, stream);
 }
 
 int sgh_eltwise_mult_f32(const float *a, const float *b, int b_is_scalar, float *out, size_t n, void *stream) {
+  sgh_note_write(out, n * sizeof(float));
   if (n == 0) return SGH_OK;
   if (!a || !b || !out) return SGH_EINVAL;
   if (b_is_scalar) return launch_map1(a, out, n, MulScalarDevOp{b}, stream);

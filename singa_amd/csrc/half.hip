@@ -440,10 +440,10 @@ int sgh_sgd_momentum_master_bf16(float *p_master, const uint16_t *g, float *v, u
 }
 
 
-int sgh_cast_f32_to_f16(const float *src, uint16_t *dst, size_t n, void *stream) { return cast_to16<F16>(src, dst, n, stream); }
-int sgh_cast_f16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream) { return cast_from16<F16>(src, dst, n, stream); }
-int sgh_cast_f32_to_bf16(const float *src, uint16_t *dst, size_t n, void *stream) { return cast_to16<BF16>(src, dst, n, stream); }
-int sgh_cast_bf16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream) { return cast_from16<BF16>(src, dst, n, stream); }
+int sgh_cast_f32_to_f16(const float *src, uint16_t *dst, size_t n, void *stream) { sgh_note_write(dst, n * 2); return cast_to16<F16>(src, dst, n, stream); }
+int sgh_cast_f16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream) { sgh_note_write(dst, n * 4); return cast_from16<F16>(src, dst, n, stream); }
+int sgh_cast_f32_to_bf16(const float *src, uint16_t *dst, size_t n, void *stream) { sgh_note_write(dst, n * 2); return cast_to16<BF16>(src, dst, n, stream); }
+int sgh_cast_bf16_to_f32(const uint16_t *src, float *dst, size_t n, void *stream) { sgh_note_write(dst, n * 4); return cast_from16<BF16>(src, dst, n, stream); }
 
 // (both operands are x: the stored value where it is positive, else +0 -- exact, nothing is rounded)
 int sgh_relu_fwd_f16(const uint16_t *x, uint16_t *y, size_t n, void *stream) {
@@ -475,23 +475,29 @@ int sgh_relu_bwd_add_bf16(const uint16_t *dy0, const uint16_t *dy1, const uint16
   return launch_relu_bwd_add<StBF16>(dy0, dy1, x, dx, n, stream);
 }
 int sgh_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  sgh_note_write(out, n * 2);
   sgh_prof_scope prof("add/k_map2_h<AddOp>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<F16>(a, b, out, n, AddOp{}, stream);
 }
 int sgh_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  sgh_note_write(out, n * 2);
   sgh_prof_scope prof("add/k_map2_h<AddOp>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<BF16>(a, b, out, n, AddOp{}, stream);
 }
 int sgh_add_relu_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  sgh_note_write(out, n * 2);
   return launch_map2_h<F16>(a, b, out, n, AddReluOp<F16>{}, stream);
 }
 int sgh_add_relu_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  sgh_note_write(out, n * 2);
   return launch_map2_h<BF16>(a, b, out, n, AddReluOp<BF16>{}, stream);
 }
 int sgh_eltwise_mult_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  sgh_note_write(out, n * 2);
   return launch_map2_h<F16>(a, b, out, n, MulOp{}, stream);
 }
 int sgh_eltwise_mult_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
+  sgh_note_write(out, n * 2);
   return launch_map2_h<BF16>(a, b, out, n, MulOp{}, stream);
 }
 int sgh_axpy_f16(float alpha, const uint16_t *x, uint16_t *y, size_t n, void *stream) {

@@ -1395,6 +1395,7 @@ int sgh_conv_dgrad_prepare_multi(const sgh_conv_prepare_item *items, int count, 
       sgh_conv_geom *g = batch[i];
       g->prelaid_dtype = dtype, g->prelaid_W = t.it[i].W, g->prelaid_ws = t.it[i].Wt;
       g->prelaid_ws_bytes = batch_bytes[i], g->prelaid_epoch = sgh_weights_epoch();
+      sgh_prepared_weights_add(t.it[i].W, size_t(g->K) * g->C * g->R * g->S * (dtype == 0 ? 4 : 2));
     }
     t.count = 0;
     return SGH_OK;

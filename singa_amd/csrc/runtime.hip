@@ -46,7 +46,7 @@ struct sgh_device {
   size_t in_use = 0, cached = 0, driver_allocs = 0;
   // stream capture (sgh_graph_begin .. sgh_graph_end): blocks freed meanwhile are kept out of the
   // pool, because the captured kernels will write to them on every replay
-  bool capturing = false;
+  std::atomic<bool> capturing{false};   // (read by entry points that do not take the lock)
   std::vector<std::pair<void *, size_t>> held;
   std::unordered_set<void *> born;        // blocks handed out while recording
   std::vector<struct sgh_graph *> graphs;  // instantiated recordings of this device
@@ -112,8 +112,45 @@ const sgh_env_switches &sgh_env() {
 // ---- weight epoch and the prepared-weights note of a convolution geometry
 static std::atomic<unsigned long long> g_weights_epoch{1};
 
+// Weight tensors whose re-laid copies are waiting in a workspace (sgh_conv_dgrad_prepare_multi), as address
+// ranges.  Entry points that are known to update parameters advance the epoch outright; the elementwise ones,
+// which a backward pass also calls on activations between the prepare and the data gradients, advance it only
+// when their output lies inside one of these ranges (Tensor `*=`, `+=`, `-=` on a weight).
+static std::mutex g_prepared_mu;
+static std::vector<std::pair<const char *, size_t>> g_prepared;
+static std::atomic<int> g_prepared_count{0};
+
 unsigned long long sgh_weights_epoch() { return g_weights_epoch.load(std::memory_order_relaxed); }
-void sgh_weights_epoch_bump() { g_weights_epoch.fetch_add(1, std::memory_order_relaxed); }
+void sgh_weights_epoch_bump() {
+  g_weights_epoch.fetch_add(1, std::memory_order_relaxed);
+  if (g_prepared_count.load(std::memory_order_relaxed) != 0) {   // every note is void now
+    std::lock_guard<std::mutex> lk(g_prepared_mu);
+    g_prepared.clear();
+    g_prepared_count.store(0, std::memory_order_relaxed);
+  }
+}
+
+void sgh_prepared_weights_add(const void *W, size_t bytes) {
+  std::lock_guard<std::mutex> lk(g_prepared_mu);
+  if (g_prepared.size() >= 4096) g_prepared.clear();   // (notes of earlier epochs that nobody used up)
+  g_prepared.emplace_back(static_cast<const char *>(W), bytes);
+  g_prepared_count.store(int(g_prepared.size()), std::memory_order_relaxed);
+}
+
+void sgh_note_write(const void *out, size_t bytes) {
+  if (g_prepared_count.load(std::memory_order_relaxed) == 0 || !out) return;
+  bool hit = false;
+  {
+    std::lock_guard<std::mutex> lk(g_prepared_mu);
+    const char *o = static_cast<const char *>(out);
+    for (const auto &r : g_prepared)
+      if (o < r.first + r.second && r.first < o + bytes) {
+        hit = true;
+        break;
+      }
+  }
+  if (hit) sgh_weights_epoch_bump();
+}
 
 bool sgh_prelaid_valid(const sgh_conv_geom *g, int dtype, const void *W, const void *workspace) {
   return g->prelaid_W != nullptr && g->prelaid_W == W && g->prelaid_ws == workspace && g->prelaid_dtype == dtype &&
@@ -193,6 +230,8 @@ const char *sgh_error_string(int rc) {
     case SGH_ELABEL: return "class label out of range";
     case SGH_ENOMEM: return "out of device memory";
     case SGH_ELIMIT: return "size beyond the fixed scratch buffer of a non-allocating entry point";
+    case SGH_EEXCHANGE:
+      return "workgroups of a one-pass BatchNorm kernel gave up waiting for each other: the outputs of that call are NaN";
     default: break;
   }
   if (rc > 0) return hipGetErrorString(static_cast<hipError_t>(rc));
@@ -312,12 +351,11 @@ void *sgh_device_aux_stream(sgh_device *dev) {
 int sgh_device_fork(sgh_device *dev, void **aux_stream) {
   if (!dev || !aux_stream) return SGH_EINVAL;
   if (dev->capturing) return SGH_EUNSUPPORTED;
+  std::lock_guard<std::mutex> lk(dev->mu);   // (stream and event creation, and the record / wait pair, as one step)
   void *aux = sgh_device_aux_stream(dev);
   if (!aux) return SGH_ENOMEM;
-  if (!dev->fork_ev) {
-    SGH_HIP_TRY(hipEventCreateWithFlags(&dev->fork_ev, hipEventDisableTiming));
-    SGH_HIP_TRY(hipEventCreateWithFlags(&dev->join_ev, hipEventDisableTiming));
-  }
+  if (!dev->fork_ev) SGH_HIP_TRY(hipEventCreateWithFlags(&dev->fork_ev, hipEventDisableTiming));
+  if (!dev->join_ev) SGH_HIP_TRY(hipEventCreateWithFlags(&dev->join_ev, hipEventDisableTiming));
   SGH_HIP_TRY(hipEventRecord(dev->fork_ev, dev->stream));
   SGH_HIP_TRY(hipStreamWaitEvent(dev->aux, dev->fork_ev, 0));
   *aux_stream = aux;
@@ -326,11 +364,11 @@ int sgh_device_fork(sgh_device *dev, void **aux_stream) {
 
 int sgh_device_join(sgh_device *dev) {
   if (!dev) return SGH_EINVAL;
+  std::lock_guard<std::mutex> lk(dev->mu);
   if (!dev->aux || !dev->join_ev) return SGH_OK;   // never forked
   if (dev->capturing) return SGH_EUNSUPPORTED;
   SGH_HIP_TRY(hipEventRecord(dev->join_ev, dev->aux));
   SGH_HIP_TRY(hipStreamWaitEvent(dev->stream, dev->join_ev, 0));
-  std::lock_guard<std::mutex> lk(dev->mu);
   release_pending(dev);
   return SGH_OK;
 }
@@ -355,7 +393,12 @@ int sgh_device_sync(sgh_device *dev) {
   if (dev->capturing) return SGH_EUNSUPPORTED;  // nothing runs while the stream records
   std::lock_guard<std::mutex> lk(dev->mu);
   SGH_HIP_TRY(quiesce(dev));
-  return SGH_OK;
+  // workgroups of a one-pass BatchNorm kernel that gave up waiting for their channel's other slices left NaN
+  // behind: the first wait after such a launch says so
+  int gave_up = 0;
+  const int rc = sgh_bn_take_exchange_failures(&gave_up);
+  if (rc != SGH_OK) return rc;
+  return gave_up ? SGH_EEXCHANGE : SGH_OK;
 }
 
 int sgh_graph_begin(sgh_device *dev) {
@@ -396,6 +439,10 @@ int sgh_graph_end(sgh_device *dev, sgh_graph **out) {
 
 int sgh_graph_launch(sgh_graph *g) {
   if (!g || !g->exec || g->dev->capturing) return SGH_EINVAL;
+  // what the recording holds is not known here: it may update weights (prepared data-gradient weights must not
+  // outlive it) and it may run one-pass BatchNorm kernels (the next wait looks at their give-up counter)
+  sgh_weights_epoch_bump();
+  sgh_bn_mark_exchange_ran();
   SGH_HIP_TRY(hipGraphLaunch(g->exec, g->dev->stream));
   return SGH_OK;
 }

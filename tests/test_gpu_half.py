@@ -417,6 +417,95 @@ def test_recorded_batchnorm_forward_between_eager_backward_passes(singa, dev, ki
         dev.ResetGraph()
 
 
+@pytest.mark.parametrize("kind,shape", [("f16", (128, 48, 7, 7)), ("bf16", (128, 96, 7, 7)), ("f32", (64, 24, 28, 28)),
+                                        ("f16", (32, 16, 14, 14))])
+def test_recorded_batchnorm_backward_between_eager_forward_passes(singa, dev, kind, shape):
+    """The other direction: a recorded BatchNorm backward whose channels are cut into several slices (the one-pass
+    kernel with exchange words) is replayed with eager FORWARD calls on the same handle in between.  On planes
+    that are not whole vectors (7 x 7) the forward pass runs the two-pass kernels, which write their partial sums
+    at the start of the workspace; the backward kernel's words lie in a part of their own behind them, so every
+    replay finds all words of a channel in one state and stores the bits of the eager call."""
+    r = rng(sum(shape) + 11)
+    N, C, H, W = shape
+    x32, dy32 = (r.standard_normal(shape).astype(np.float32) for _ in range(2))
+    if kind == "f32":
+        xt, dyt = (singa.from_numpy(v, dev) for v in (x32, dy32))
+    else:
+        xt, dyt = (_to(singa, dev, v, kind)[0] for v in (x32, dy32))
+    gd = singa.from_numpy((1 + 0.3 * r.standard_normal(C)).astype(np.float32), dev)
+    bd = singa.from_numpy((0.2 * r.standard_normal(C)).astype(np.float32), dev)
+    rm, rv = singa.from_numpy(np.zeros(C, np.float32), dev), singa.from_numpy(np.ones(C, np.float32), dev)
+    h = singa.CudnnBatchNormHandle(0.9, xt)
+    for _ in range(2):   # (the pool holds the blocks the recorded call will take)
+        y, mean, var = singa.GpuBatchNormForwardTraining(h, xt, gd, bd, rm, rv)
+        want = [t.to_numpy() for t in singa.GpuBatchNormBackward(h, dyt, xt, gd, mean, var)]
+    assert all(np.isfinite(np.asarray(w, np.float32)).all() for w in want)
+    dev.Sync()
+    dev.EnableGraph(True)
+    dx, dg, db = singa.GpuBatchNormBackward(h, dyt, xt, gd, mean, var)
+    dev.EnableGraph(False)
+    try:
+        for i in range(6):
+            dx.SetFloatValue(0.0)
+            dev.RunGraph()
+            for got, w, what in zip((dx, dg, db), want, ("dx", "dgamma", "dbeta")):
+                _same_bits(got.to_numpy(), w, "%s of replay %d of the recorded backward, %s" % (what, i, kind))
+            if i != 3:   # (also two replays in a row)
+                y2, _, _ = singa.GpuBatchNormForwardTraining(h, xt, gd, bd, rm, rv)
+                _same_bits(y2.to_numpy(), y.to_numpy(), "eager forward between replays")
+        dev.Sync()       # (no workgroup gave up: the wait reports nothing)
+    finally:
+        dev.ResetGraph()
+
+
+def test_batchnorm_exchange_gives_up_visibly(singa, dev):
+    """The one-pass kernels' bounded wait: with the spin limit forced down to one poll from the host, workgroups
+    of a channel cut into many slices give up -- every kernel still ends normally, the channel's outputs are NaN,
+    and the next wait on the device returns SGH_EEXCHANGE instead of 0 (once); sgh_bn_exchange_failures counts
+    them.  With the default limit the same calls are clean and match the CPU oracle."""
+    import ctypes as C
+    from oracle import cpu_oracle as O
+    from singa_amd import _lib
+    from util import nl2
+    L = _lib.lib()
+    r = rng(77)
+    N, Cn, H, W = 32, 8, 112, 112     # 8 channels on a whole chip: 64 slices per channel
+    x = r.standard_normal((N, Cn, H, W)).astype(np.float32)
+    dy = r.standard_normal((N, Cn, H, W)).astype(np.float32)
+    g = (1 + 0.3 * r.standard_normal(Cn)).astype(np.float32)
+    b = (0.2 * r.standard_normal(Cn)).astype(np.float32)
+    xt, dyt, gd, bd = (singa.from_numpy(v, dev) for v in (x, dy, g, b))
+    rm, rv = singa.from_numpy(np.zeros(Cn, np.float32), dev), singa.from_numpy(np.ones(Cn, np.float32), dev)
+    h = singa.CudnnBatchNormHandle(0.9, xt)
+    y, mean, var = singa.GpuBatchNormForwardTraining(h, xt, gd, bd, rm, rv)
+    dev.Sync()
+    L.sgh_bn_exchange_spin_limit(1)
+    try:
+        dx, dg, db = singa.GpuBatchNormBackward(h, dyt, xt, gd, mean, var)
+        assert L.sgh_device_sync(dev._h) == _lib.SGH_EEXCHANGE          # the error code, not NaN-sniffing
+        assert b"gave up" in L.sgh_error_string(_lib.SGH_EEXCHANGE)
+        assert L.sgh_device_sync(dev._h) == 0                           # reported once
+        assert np.isnan(dg.to_numpy()).any() and np.isnan(dx.to_numpy()).any()
+        with pytest.raises(singa.SingaHipError, match="gave up"):
+            singa.GpuBatchNormBackward(h, dyt, xt, gd, mean, var)
+            dev.Sync()
+        # the forward kernel likewise; counted by the explicit query
+        singa.GpuBatchNormForwardTraining(h, xt, gd, bd, rm, rv)
+        n = C.c_int(-1)
+        _lib.check(L.sgh_bn_exchange_failures(dev.stream, C.byref(n)), "sgh_bn_exchange_failures")
+        assert n.value > 0
+        assert L.sgh_device_sync(dev._h) == 0                           # the query cleared the counter
+    finally:
+        L.sgh_bn_exchange_spin_limit(0)
+    dx, dg, db = singa.GpuBatchNormBackward(h, dyt, xt, gd, mean, var)
+    dev.Sync()
+    n = C.c_int(-1)
+    _lib.check(L.sgh_bn_exchange_failures(dev.stream, C.byref(n)), "sgh_bn_exchange_failures")
+    assert n.value == 0
+    dx_o, dg_o, db_o = O.bn_bwd(dy, x, g, mean.to_numpy(), var.to_numpy())
+    assert nl2(dx.to_numpy(), dx_o) <= 1e-3 and nl2(dg.to_numpy(), dg_o) <= 1e-3 and nl2(db.to_numpy(), db_o) <= 1e-3
+
+
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("case", [
     (2, 3, 8, 8, (2, 2), (2, 2), (0, 0)),
@@ -743,7 +832,6 @@ def test_set_value_on_16bit_tensors_stays_inside_the_tensor(singa, dev, kind):
 def test_fp32_only_functions_refuse_16bit_tensors(singa, dev):
     t = singa.Tensor((4, 8), dev, singa.kFloat16)
     t.SetFloatValue(1.0)
-    for call in (lambda: singa.ReLU(t), lambda: singa.SoftMax(t), lambda: singa.Mult(t, t.T()),
-                 lambda: singa.Sum(t, 0), lambda: t.__imul__(2.0)):
+    for call in (lambda: singa.SoftMax(t), lambda: singa.Sum(t, 0), lambda: t.__imul__(2.0)):
         with pytest.raises(singa.SingaHipError):
             call()

@@ -261,6 +261,33 @@ def test_prepared_weights_are_never_stale(singa, dev):
     # (3) prepared for one weight tensor, called with another
     singa.GpuConvPrepareBackward([(wd, h)])
     assert_bit_equal(singa.GpuConvBackwardx(dyd, other, xd, h).to_numpy(), fresh(other), "another weight tensor")
+    # (1d) in-place tensor arithmetic on the weight: `W *= s` (EltwiseMult with a scalar tensor on the right, the
+    # optimizer's own idiom, python/singa/opt.py:299-300) and `W += t`; the same ops on OTHER tensors leave the
+    # note alone (a backward pass runs many of them between the prepare and its data gradients)
+    half = singa.from_numpy(np.array([0.5], np.float32), dev)
+    acts, acts2, w2d = singa.from_numpy(x, dev), singa.from_numpy(x, dev), singa.from_numpy(w2, dev)
+    singa.GpuConvPrepareBackward([(wd, h)])
+    acts *= half
+    acts += acts2
+    wd *= half
+    assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), fresh(wd), "after W *= s")
+    singa.GpuConvPrepareBackward([(wd, h)])
+    wd += w2d
+    assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), fresh(wd), "after W += t")
+    # (1e) a replayed recording that holds an update: the library cannot see inside it
+    g = singa.from_numpy(w2, dev)
+    sgd2 = opt.SGD(lr=0.05, momentum=0.0)
+    sgd2.apply("w", wd, g)
+    dev.Sync()
+    dev.EnableGraph(True)
+    sgd2.apply("w", wd, g)
+    dev.EnableGraph(False)
+    try:
+        singa.GpuConvPrepareBackward([(wd, h)])
+        dev.RunGraph()
+        assert_bit_equal(singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy(), fresh(wd), "after a replayed update")
+    finally:
+        dev.ResetGraph()
 
 
 def test_conv_wgrad_is_deterministic(singa, dev):
