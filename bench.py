@@ -226,6 +226,33 @@ def main():
 
     if graph:
         dev.ResetGraph()
+    # What a SINGA tree with unchanged python/singa/autograd.py and opt.py would see through this library: one call
+    # per reference op (ReLU.backward and _BatchNorm2d.backward separately, `+=` as its own kernel, a weight
+    # re-layout inside every data gradient), everything on the one device stream, and SGD.apply parameter by
+    # parameter (python/singa/autograd.py:128-224, python/singa/opt.py:269-310).  A short second measurement
+    # after the timed region, reported beside the headline figure.
+    reference_tape = None
+    if not (args.no_fusion or args.with_forward):
+        saved = {f: getattr(hip, f) for f in ("fuse_bn_relu", "fuse_dgrad_add", "fuse_add_relu", "fuse_wgrad_bias",
+                                              "batch_relayout", "overlap_wgrad", "fuse_forward")}
+        hip.set_fusion(False)
+        net.sgd.op_by_op = True     # SGD.apply's own tensor ops, three launches per parameter
+        ref_steps = max(3, min(args.steps, 10))
+        for _ in range(2):
+            net.backward_and_update(fused_update=False)
+        sync()
+        t2 = time.perf_counter()
+        for _ in range(ref_steps):
+            net.backward_and_update(fused_update=False)
+        sync()
+        ref_ms = (time.perf_counter() - t2) / ref_steps * 1e3
+        reference_tape = {"value": round(args.batch / ref_ms * 1e3, 2), "unit": "imgs/s", "ms_per_step": round(ref_ms, 4),
+                          "steps": ref_steps,
+                          "tape": "one call per reference op on one stream, SGD.apply parameter by parameter through its own "
+                                  "Axpy / EltwiseMult ops (what unchanged autograd.py / opt.py issue)"}
+        for f, v in saved.items():
+            setattr(hip, f, v)
+        net.sgd.op_by_op = False
     # kernel-level pass (eager): every conv / GEMM launch bracketed by HIP events on the device stream
     prof_steps = max(1, min(args.steps, 5))
     hip.overlap_wgrad = False   # one kernel at a time on the device, so that an event pair brackets that kernel alone
@@ -297,6 +324,8 @@ def main():
         "host_enqueue_ms_per_step": round(t_enqueued / args.steps * 1e3, 4),
         "host_enqueue_ms_idle_queue": round(t_idle_enqueue * 1e3, 4),
     }
+    if reference_tape is not None:
+        out["reference_tape"] = reference_tape
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.config, args.cpu_sample_batch or args.batch, args.cpu_budget_s,
                                            args.cpu_single_thread_batch)

@@ -350,7 +350,8 @@ void *sgh_device_aux_stream(sgh_device *dev) {
 
 int sgh_device_fork(sgh_device *dev, void **aux_stream) {
   if (!dev || !aux_stream) return SGH_EINVAL;
-  if (dev->capturing) return SGH_EUNSUPPORTED;
+  // (while the main stream records, the event pair below pulls the auxiliary stream into the same recording: what
+  // is enqueued there afterwards becomes a branch of the graph, which sgh_device_join closes)
   std::lock_guard<std::mutex> lk(dev->mu);   // (stream and event creation, and the record / wait pair, as one step)
   void *aux = sgh_device_aux_stream(dev);
   if (!aux) return SGH_ENOMEM;
@@ -366,10 +367,9 @@ int sgh_device_join(sgh_device *dev) {
   if (!dev) return SGH_EINVAL;
   std::lock_guard<std::mutex> lk(dev->mu);
   if (!dev->aux || !dev->join_ev) return SGH_OK;   // never forked
-  if (dev->capturing) return SGH_EUNSUPPORTED;
   SGH_HIP_TRY(hipEventRecord(dev->join_ev, dev->aux));
   SGH_HIP_TRY(hipStreamWaitEvent(dev->stream, dev->join_ev, 0));
-  release_pending(dev);
+  if (!dev->capturing) release_pending(dev);   // (blocks freed during a recording stay with the graph)
   return SGH_OK;
 }
 

@@ -18,7 +18,7 @@ from ._lib import check
 
 class SGD(object):
 
-    def __init__(self, lr=0.1, momentum=0, dampening=0, weight_decay=0, nesterov=False):
+    def __init__(self, lr=0.1, momentum=0, dampening=0, weight_decay=0, nesterov=False, op_by_op=False):
         if momentum < 0.0:
             raise ValueError("Invalid momentum value: {}".format(momentum))
         if weight_decay < 0.0:
@@ -30,6 +30,11 @@ class SGD(object):
         self.dampening = float(dampening)
         self.weight_decay = float(weight_decay)
         self.nesterov = bool(nesterov)
+        # op_by_op: ``apply`` issues the reference's own tensor ops (Axpy with 1-element device tensors, the
+        # in-place product with the momentum tensor) instead of the fused kernel -- what unchanged
+        # python/singa/opt.py does through the Axpy / EltwiseMult entry points; bit-identical results
+        self.op_by_op = bool(op_by_op)
+        self._hyper = None
         self.moments = dict()
         self.masters = dict()
         self.step_counter = 0
@@ -56,11 +61,35 @@ class SGD(object):
                                                              param_grad.shape())
         if param_value.data_type() != param_grad.data_type():
             raise singa.SingaHipError("parameter and gradient differ in data type")
+        if self.op_by_op and param_value.data_type() == singa.kFloat32:
+            return self._apply_op_by_op(param_name, param_value, param_grad)
         v = self._moment(param_name, param_value) if self.momentum != 0 else None
         name = "sgh_sgd_momentum_" + singa._SUFFIX[param_value.data_type()]   # f32 / f16 / bf16
         check(getattr(_lib.lib(), name)(param_value.ptr, param_grad.ptr, v.ptr if v is not None else None,
                                         param_value.Size(), self.lr, self.momentum, self.dampening,
                                         self.weight_decay, int(self.nesterov), param_value.device().stream), name)
+
+    def _apply_op_by_op(self, param_name, param_value, param_grad):
+        """``SGD.apply`` as the reference writes it (python/singa/opt.py:269-310), op by op on 1-element device
+        tensors: 3 launches per parameter with momentum and no weight decay.  Unlike the fused kernel it may
+        overwrite the gradient tensor, as the reference does."""
+        dev = param_value.device()
+        if self._hyper is None:
+            mk = lambda v: singa.from_numpy(np.array([v], dtype=np.float32), dev)
+            self._hyper = {"decay": mk(self.weight_decay), "mom": mk(self.momentum), "alpha": mk(1.0 - self.dampening),
+                           "minus_lr": mk(0.0 - self.lr)}
+        h = self._hyper
+        if self.weight_decay != 0:
+            singa.Axpy(h["decay"], param_value, param_grad)            # g += wd * p
+        if self.momentum != 0:
+            buf = self._moment(param_name, param_value)
+            buf *= h["mom"]                                            # v *= mu      (EltwiseMult, scalar tensor)
+            singa.Axpy(h["alpha"], param_grad, buf)                    # v += (1 - damp) * g
+            if self.nesterov:
+                singa.Axpy(h["mom"], buf, param_grad)                  # g += mu * v
+            else:
+                param_grad = buf
+        singa.Axpy(h["minus_lr"], param_grad, param_value)             # p += (-lr) * g
 
     def apply_master(self, param_name, param_value, param_grad):
         """Mixed precision: ``param_value`` / ``param_grad`` are 16-bit; an fp32 master copy of the

@@ -132,6 +132,7 @@ class HipOps(object):
     # gradients of a backward pass run on the device's auxiliary stream beside the chain of data
     # gradients / BatchNorm / ReLU backward ops (matrix-bound work beside bandwidth-bound work)
     overlap_wgrad = True
+    graph_overlap = bool(int(__import__("os").environ.get("SGH_GRAPH_OVERLAP", "0")))
     _aux = None          # the auxiliary stream while a backward pass is under way
 
     def conv_bwd_w(self, dy, x, W, h):
@@ -169,9 +170,9 @@ class HipOps(object):
 
     def prepare_backward(self, convs, update_at_end=False):
         """`update_at_end`: no parameter is updated (no weight gradient read) before finish_backward."""
-        # (not while a graph is being recorded: a recording with a branch per layer replays slower than
-        # the plain chain, 6.4 against 5.9 ms for ResNet-18)
-        if self.overlap_wgrad and update_at_end and not self.dev.graph_enabled():
+        # (while a graph is being recorded only if `graph_overlap` says so: the weight gradients become a branch of
+        # the recording)
+        if self.overlap_wgrad and update_at_end and (self.graph_overlap or not self.dev.graph_enabled()):
             self._aux = self.dev.AuxStream()
         if self.batch_relayout:
             by_type = {}

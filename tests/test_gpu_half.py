@@ -714,6 +714,12 @@ def test_conv_dgrad_16bit_with_batched_weight_relayout(singa, dev, kind):
     (128, 256, 56, 64, 1, 1, 0),     # bottleneck reduce
     (128, 128, 56, 128, 3, 2, 1),    # stage transition, stride 2
     (128, 1024, 14, 256, 1, 1, 0),   # plane of 196 pixels: 24.5 octets
+    (128, 512, 7, 2048, 1, 1, 0),    # stage 4: bottleneck expand on 7 x 7 planes
+    (128, 2048, 7, 512, 1, 1, 0),    # ... reduce
+    (128, 512, 7, 512, 3, 1, 1),     # ... 3x3 on 49-pixel planes (pixel-major gradient copy)
+    (128, 512, 14, 512, 3, 2, 1),    # ... its stride-2 opening layer
+    (128, 256, 56, 512, 1, 2, 0),    # downsample convolutions: 1x1 stride 2 (one residue class, 2x2-block store)
+    (128, 1024, 14, 2048, 1, 2, 0),
 ])
 def test_conv_gradients_16bit_full_size_properties(singa, dev, kind, shape):
     """The 16-bit gradient kernels at the half-precision configuration's full batch (N = 128), too

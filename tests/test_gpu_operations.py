@@ -354,6 +354,12 @@ def test_conv_dgrad_is_deterministic(singa, dev, n, c, hw, k, stride):
     (64, 64, 56, 128, 3, 2, 1),    # stage transition: residue-class shared-tile dgrad, stride-2 slab wgrad
     (64, 256, 14, 512, 1, 2, 0),   # downsample: pointwise dgrad with dilating store
     (64, 64, 56, 128, 1, 2, 0),    # first downsample: 64 x 64 wavefront tiles
+    (64, 128, 28, 128, 3, 1, 1),   # the 3x3 layers of stages 2-4 at the full batch: shared-tile kernels on 28 x 28,
+    (64, 256, 14, 256, 3, 1, 1),   # 14 x 14 (tiles that straddle images, every tile shared between workgroups)
+    (64, 512, 7, 512, 3, 1, 1),    # and 7 x 7 planes (49 pixels: a tile covers 2.6 images)
+    (64, 128, 28, 256, 3, 2, 1),   # the stride-2 layers that open stages 3 and 4
+    (64, 256, 14, 512, 3, 2, 1),
+    (64, 128, 28, 256, 1, 2, 0),   # second downsample
 ])
 def test_conv_full_size_properties(singa, dev, shape):
     """Convolutions at the benchmark's full batch are too large for the CPU oracle inside a test,
@@ -542,6 +548,29 @@ def test_bn_reference_vectors(singa, dev, golden):
     y, mean, var = singa.GpuBatchNormForwardTraining(h, xd, gamma, beta, None, None)
     dx, _, _ = singa.GpuBatchNormBackward(h, xd, xd, gamma, mean, var)
     np.testing.assert_allclose(dx.to_numpy().ravel(), np.array(g["dx"], np.float32), atol=1e-6)
+
+
+def test_bn_2d_reference_vectors(singa, dev, golden):
+    """The reference's 2-D BatchNorm layer test (test/singa/test_batchnorm.cc:44-129) through the handle built from a
+    [batch, features] tensor (CudnnBatchNormHandle's is_2d case, src/model/operation/batchnorm.cc:27-43)."""
+    g = golden["bn_2d"]
+    x = np.array(g["x"], np.float32).reshape(g["x_shape"])
+    dy = np.array(g["dy"], np.float32).reshape(g["x_shape"])
+    xd = singa.from_numpy(x, dev)
+    h = singa.CudnnBatchNormHandle(1.0, xd)
+    assert h.is_2d and (h.height, h.width) == (1, 1)
+    mk = lambda v: singa.from_numpy(np.array(v, np.float32), dev)
+    rm, rv = mk(g["fwd_beta"]), mk(g["fwd_beta"])        # (the test seeds the running statistics with beta)
+    y, _, _ = singa.GpuBatchNormForwardTraining(h, xd, mk(g["fwd_gamma"]), mk(g["fwd_beta"]), rm, rv)
+    assert y.shape() == g["x_shape"]
+    np.testing.assert_allclose(y.to_numpy().ravel(), np.array(g["y"], np.float32), atol=g["tol"])
+    gamma = mk(g["bwd_gamma"])
+    _, mean, var = singa.GpuBatchNormForwardTraining(h, xd, gamma, mk(g["bwd_beta"]), None, None)
+    dx, ds, db = singa.GpuBatchNormBackward(h, singa.from_numpy(dy, dev), xd, gamma, mean, var)
+    assert dx.shape() == g["x_shape"] and ds.shape() == [2] and db.shape() == [2]
+    np.testing.assert_allclose(dx.to_numpy().ravel(), np.array(g["dx"], np.float32), atol=g["tol"])
+    np.testing.assert_allclose(ds.to_numpy(), np.array(g["dgamma"], np.float32), atol=g["tol"])
+    np.testing.assert_allclose(db.to_numpy(), np.array(g["dbeta"], np.float32), atol=g["tol"])
 
 
 @pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 56, 56), (64, 512, 7, 7), (16, 128, 28, 28),

@@ -29,6 +29,29 @@ def test_relu_reference_vector(singa, dev, golden):
     assert singa.ReLUBackward(dy, x).to_numpy().ravel().tolist() == g["dx"]
 
 
+def test_relu_layer_reference_vector(singa, dev, golden):
+    """The legacy Activation layer's ReLU vectors (test/singa/test_activation.cc:44-129)."""
+    g = golden["relu_layer"]
+    x, dy = singa.from_numpy(np.array(g["x"], np.float32), dev), singa.from_numpy(np.array(g["dy"], np.float32), dev)
+    assert singa.ReLU(x).to_numpy().tolist() == g["y"]
+    assert singa.ReLUBackward(dy, x).to_numpy().tolist() == g["dx"]
+
+
+def test_dense_backward_reference_vector(singa, dev, golden):
+    """Dense.Backward (test/singa/test_dense.cc:75-137) as autograd runs a Linear layer: db = Sum(dy, 0), the value the
+    reference test asserts; dx = dy . W^T and dW = x^T . dy (python/singa/autograd.py:613-623) against the oracle."""
+    g = golden["dense"]
+    x = np.array(g["x"], np.float32).reshape(g["x_shape"])
+    w = np.array(g["w"], np.float32).reshape(g["w_shape"])
+    dy = np.array(g["dy"], np.float32).reshape(g["dy_shape"])
+    xd, wd, dyd = (singa.from_numpy(v, dev) for v in (x, w, dy))
+    db = singa.Sum(dyd, 0).to_numpy()
+    for i, terms in enumerate(g["db_terms"]):
+        np.testing.assert_allclose(db[i], sum(float(dy.ravel()[k]) for k in terms), rtol=5e-7)
+    assert_bit_equal(singa.Mult(dyd, wd.T()).to_numpy(), O.sgemm(dy, w, transB=True), "dx = dy . W^T")
+    assert_bit_equal(singa.Mult(xd.T(), dyd).to_numpy(), O.sgemm(x, dy, transA=True), "dW = x^T . dy")
+
+
 @pytest.mark.parametrize("n", SIZES)
 def test_relu_backward(singa, dev, n):
     r = rng(n + 1)
@@ -147,12 +170,15 @@ def test_axpy_mult_add(singa, dev, n):
     assert_bit_equal(acc.to_numpy(), O.add(x, y), "+=")
 
 
-def test_sgd_reference_cases(singa, dev, golden):
+@pytest.mark.parametrize("op_by_op", [False, True])
+def test_sgd_reference_cases(singa, dev, golden, op_by_op):
+    """op_by_op: the reference's own sequence of tensor ops (Axpy with device scalars, the in-place product with the
+    momentum tensor) instead of the fused kernel -- what unchanged python/singa/opt.py runs on this library."""
     from singa_amd import opt
     g = golden["sgd"]
     shape = tuple(g["shape"])
     for c in g["cases"]:
-        sgd = opt.SGD(lr=c["lr"], momentum=c["mu"], weight_decay=c["wd"], nesterov=bool(c["nesterov"]))
+        sgd = opt.SGD(lr=c["lr"], momentum=c["mu"], weight_decay=c["wd"], nesterov=bool(c["nesterov"]), op_by_op=op_by_op)
         w = singa.from_numpy(np.full(shape, c["w0"], np.float32), dev)
         wo, vo = np.full(shape, c["w0"], np.float32), np.zeros(shape, np.float32)
         for _ in range(c["steps"]):
@@ -166,12 +192,13 @@ def test_sgd_reference_cases(singa, dev, golden):
 @pytest.mark.parametrize("n", [1, 5, 4096, 100003, 2359296])
 @pytest.mark.parametrize("cfg", [(0.05, 0.9, 0.0, 0.0, False), (0.1, 0.9, 0.1, 1e-4, False), (0.01, 0.8, 0.0, 5e-4, True),
                                  (0.05, 0.0, 0.0, 0.0, False)])
-def test_sgd_momentum_fused(singa, dev, n, cfg):
+@pytest.mark.parametrize("op_by_op", [False, True])
+def test_sgd_momentum_fused(singa, dev, n, cfg, op_by_op):
     lr, mu, damp, wd, nesterov = cfg
     from singa_amd import opt
     r = rng(n)
     p, v = randn(r, n), randn(r, n)
-    sgd = opt.SGD(lr=lr, momentum=mu, dampening=damp, weight_decay=wd, nesterov=nesterov)
+    sgd = opt.SGD(lr=lr, momentum=mu, dampening=damp, weight_decay=wd, nesterov=nesterov, op_by_op=op_by_op)
     pd = singa.from_numpy(p, dev)
     if mu != 0:
         sgd.moments["p"] = singa.from_numpy(v, dev)

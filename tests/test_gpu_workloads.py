@@ -134,7 +134,19 @@ def test_resnet50_bottleneck_16bit_step(dev, kind):
     print(kind, "GPU vs float64 model, worst:", ", ".join("%s=%.2e (oracle %.2e)" % (k, v, e_cpu[k]) for k, v in worst))
     print(kind, "largest GPU error / (2 x oracle error + u):", ", ".join("%s=%.2f" % (k, r) for r, k in ratio[:4]))
     assert ratio[0][0] <= 1.0, ratio[:4]
-    assert worst[0][1] < (1e-2 if kind == "f16" else 5e-2), worst
+    # the stated bar, tensor by tensor: 1e-2 for every gradient and updated parameter.  In bfloat16 (unit roundoff
+    # 2^-8) the fp32 oracle itself, rounding at the same points, does not hold it on some tensors -- last-place
+    # flips of stored gradients that compound over the layers behind them -- so a tensor may exceed 1e-2 only where
+    # the oracle's own distance from the float64 model is at least half the bar, and then stays within
+    # 2 x oracle + u (above) and 5e-2.  The set is printed and counted.
+    over = sorted(k for k, v in e_gpu.items() if v >= 1e-2)
+    print(kind, "%d of %d tensors above 1e-2: %s" % (len(over), len(e_gpu), ", ".join("%s=%.2e (oracle %.2e)" % (k, e_gpu[k], e_cpu[k]) for k in over)))
+    if kind == "f16":
+        assert not over, over
+    else:
+        assert all(e_cpu[k] >= 5e-3 for k in over), [(k, e_gpu[k], e_cpu[k]) for k in over if e_cpu[k] < 5e-3]
+        assert all(e_gpu[k] < 5e-2 for k in over)
+        assert len(over) <= len(e_gpu) // 4, len(over)
 
 
 @pytest.mark.parametrize("config,kind", [("resnet18_small", "f32"), ("resnet18_small", "f32-sum-in-relu"),
@@ -211,6 +223,47 @@ def test_two_stream_tape_at_full_size(dev, config, batch, kind):
         worst = max(nl2(a, b) for a, b in zip(one[1:], two[1:]))
         print("parameters after one step, full-chip against shared-chip split plan: nl2 <= %.2e" % worst)
         assert worst < 1e-3
+
+
+def test_resnet50_half_precision_tape_at_full_batch(dev):
+    """The half-precision configuration at its own size (ResNet-50, N = 128, binary16 storage) as one whole tape --
+    beyond the CPU oracle inside a test, so through what does not depend on size: every gradient and parameter
+    finite; the logits gradient of every image sums to 0 over the classes (softmax-CE) and its rows are those of
+    (p - onehot) / N computed from the tape's own probabilities; the step is run-to-run identical; and the input
+    gradient of the first step, which depends on no weight gradient, is bit-equal between the one-stream and the
+    two-stream tape."""
+    from singa_amd import singa_wrap as singa
+    x, labels = wl.make_inputs("resnet50", 128)
+
+    def run(overlap):
+        hip = wl.HalfHipOps(dev, singa.kFloat16)
+        hip.overlap_wgrad = overlap
+        net = wl.build("resnet50", hip, lr=0.01)
+        net.forward(hip.from_numpy(x), hip.from_numpy(labels))
+        p = hip.to_numpy(net.p).astype(np.float64)
+        dx = net.backward_and_update(keep_grads=True, fused_update=True)
+        grads = {k: np.asarray(hip.to_numpy(v), np.float32) for k, v in net.grad_log.items()}
+        return hip.to_numpy(dx), grads, [np.asarray(hip.to_numpy(q), np.float32) for _, q in net.params()], p
+
+    dx_a, grads_a, params_a, p = run(True)
+    assert dx_a.shape == (128, 3, 224, 224) and len(grads_a) > 160
+    assert np.isfinite(np.asarray(dx_a, np.float32)).all()
+    assert all(np.isfinite(v).all() for v in grads_a.values()) and all(np.isfinite(v).all() for v in params_a)
+    g = grads_a["logits"].astype(np.float64)
+    assert g.shape == (128, 1000) and np.abs(g.sum(axis=1)).max() < 1e-6
+    want = p.copy()
+    want[np.arange(128), labels] -= 1.0
+    assert nl2(g, want / 128) < 1e-6
+    dx_b, grads_b, params_b, _ = run(True)                      # run to run
+    assert np.array_equal(dx_a, dx_b)
+    assert all(np.array_equal(grads_a[k], grads_b[k]) for k in grads_a)
+    assert all(np.array_equal(a, b) for a, b in zip(params_a, params_b))
+    dx_c, grads_c, _, _ = run(False)                            # every kernel on one stream
+    assert np.array_equal(dx_a, dx_c)
+    # (the 16-bit weight gradients plan their split reduction by the stream they run on: last-place differences)
+    worst = max(nl2(grads_a[k], grads_c[k]) for k in grads_a)
+    print("gradients, two-stream against one-stream tape: nl2 <= %.2e" % worst)
+    assert worst < 1e-2
 
 
 def test_graph_replay_of_the_step(dev):

@@ -125,6 +125,49 @@ def test_relu(golden):
     assert O.relu_bwd(np.ones(3, np.float32), np.array([0.0, -0.0, 1e-30], np.float32)).tolist() == [0, 0, 1]
 
 
+def test_bn_2d_layer_vectors(golden):
+    """The legacy BatchNorm layer on a [batch, features] input (test/singa/test_batchnorm.cc:44-129): every
+    feature normalised over the batch, i.e. the 4-D case with planes of one element."""
+    g = golden["bn_2d"]
+    x, dy = _a(g["x"], g["x_shape"]), _a(g["dy"], g["x_shape"])
+    y, _, _ = O.bn_fwd_train(x, _a(g["fwd_gamma"]), _a(g["fwd_beta"]))
+    np.testing.assert_allclose(y.ravel(), _a(g["y"]), atol=g["tol"])
+    _, mean, invstd = O.bn_fwd_train(x, _a(g["bwd_gamma"]), _a(g["bwd_beta"]))
+    dx, dg, db = O.bn_bwd(dy, x, _a(g["bwd_gamma"]), mean, invstd)
+    np.testing.assert_allclose(dx.ravel(), _a(g["dx"]), atol=g["tol"])
+    np.testing.assert_allclose(dg, _a(g["dgamma"]), atol=g["tol"])
+    np.testing.assert_allclose(db, _a(g["dbeta"]), atol=g["tol"])
+    # the same numbers through the 4-D entry: [N, C] is [N, C, 1, 1]
+    dx4, dg4, db4 = O.bn_bwd(dy.reshape(2, 2, 1, 1), x.reshape(2, 2, 1, 1), _a(g["bwd_gamma"]), mean, invstd)
+    assert np.array_equal(dx4.ravel(), dx.ravel()) and np.array_equal(dg4, dg) and np.array_equal(db4, db)
+
+
+def test_dense_bias_gradient_vector(golden):
+    """Dense.Backward's bias gradient (test/singa/test_dense.cc:75-137): column sums of dy, the one thing the
+    reference test asserts; dx and dW (its assertions are commented out) against float64 instead."""
+    g = golden["dense"]
+    x, w, dy = _a(g["x"], g["x_shape"]), _a(g["w"], g["w_shape"]), _a(g["dy"], g["dy_shape"])
+    db = O.sum_rows(dy)
+    for i, terms in enumerate(g["db_terms"]):
+        exp = np.float32(0)
+        for k in terms:
+            exp = np.float32(exp + dy.ravel()[k])
+        np.testing.assert_allclose(db[i], exp, rtol=5e-7)   # EXPECT_FLOAT_EQ
+    dx = O.sgemm(dy, w, transB=True)      # dy . W^T  (python/singa/autograd.py:613-623)
+    dw = O.sgemm(x, dy, transA=True)      # x^T . dy
+    np.testing.assert_allclose(dx, dy.astype(np.float64) @ w.astype(np.float64).T, rtol=1e-6)
+    np.testing.assert_allclose(dw, x.astype(np.float64).T @ dy.astype(np.float64), rtol=1e-6)
+
+
+def test_relu_layer_vectors(golden):
+    g = golden["relu_layer"]
+    x, dy = _a(g["x"]), _a(g["dy"])
+    y, dx = O.relu_fwd(x), O.relu_bwd(dy, x)
+    for i in g["asserted_dx_elements"]:      # what the reference test checks (EXPECT_FLOAT_EQ)
+        assert y[i] == np.float32(g["y"][i]) and dx[i] == np.float32(g["dx"][i])
+    assert np.array_equal(y, _a(g["y"])) and np.array_equal(dx, _a(g["dx"]))
+
+
 def test_sgd_reference_cases(golden):
     g = golden["sgd"]
     shape = tuple(g["shape"])
