@@ -822,14 +822,15 @@ def GpuConvBackwardx(dy, W, x, h):
     return dx
 
 
-def GpuConvBackwardW(dy, x, W, h, stream=None):
+def GpuConvBackwardW(dy, x, W, h, stream=None, out=None):
     """`stream`: None = the device's stream.  Another stream (``HipGPU.Fork()``) runs the weight
     gradient beside whatever the main stream does next; it then works in a workspace of its own
     (``h.wgrad_workspace``); dy, x, the result and that workspace are announced to the pool
-    (``HipGPU.UsedOn``), so the caller may drop them whenever it likes."""
+    (``HipGPU.UsedOn``), so the caller may drop them whenever it likes.  `out`: the tensor that
+    receives the result (a caller that handed it out before the kernel was enqueued)."""
     h._check_dy(dy)
     h._check_x(x)
-    dW = _like(W)
+    dW = _like(W) if out is None else out
     fn, name = _fn("conv_wgrad", dy)
     ws = h.workspace
     if stream is not None:

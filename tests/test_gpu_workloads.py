@@ -266,11 +266,15 @@ def test_resnet50_half_precision_tape_at_full_batch(dev):
     assert worst < 1e-2
 
 
-def test_graph_replay_of_the_step(dev):
+@pytest.mark.parametrize("two_streams", [False, True])
+def test_graph_replay_of_the_step(dev, two_streams):
     """Graph mode (EnableGraph / RunGraph): one recorded backward+update step, replayed several
     times with eager work and synchronisations in between, leaves after every replay exactly the
-    parameters of a network that ran the same number of eager steps."""
+    parameters of a network that ran the same number of eager steps.  `two_streams`: the recording holds
+    the weight gradients as a branch on the auxiliary stream (fork / join while recording), in groups of
+    three layers; the eager steps it is compared with fork once per layer."""
     hip = wl.HipOps(dev)
+    hip.graph_overlap, hip.graph_wgrad_group = two_streams, 3
     x, labels = wl.make_inputs("resnet18_small", 2)
     nets = []
     for _ in range(2):
