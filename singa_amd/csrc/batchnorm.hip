@@ -546,6 +546,13 @@ inline ChipPlan chip_plan(int N, int C, int HW) {
     G = (TV + long(p.nt) * per_thread - 1) / (long(p.nt) * per_thread);
   }
   p.nl = p.nt == 512 && lds_ok ? chip_nl<S>() : 0;
+  // a channel that two workgroups of 512 threads would share but one of 1024 threads holds alone, with a channel for
+  // every CU: one workgroup per channel and nothing to exchange (16-bit 128 x 256 x 14 x 14: 3200 pieces per channel)
+  // -- 16.0 -> 15.0 us, 128 x 1024 x 14 x 14 50.6 -> 48.0 us
+  if (p.nt == 512 && G == 2 && p.nl == 0 && C >= sgh_num_cus() && TV <= 1024L * chip_nv<S>()) {
+    p.nt = 1024;
+    G = 1;
+  }
   // few channels: thinner slices, so that there are two workgroups for every CU (at least one wavefront of vectors
   // each) -- unless a channel fits one workgroup and there is a channel for every CU: then nothing is exchanged
   const bool whole_channels = G == 1 && C >= sgh_num_cus();
@@ -560,7 +567,7 @@ inline ChipPlan chip_plan(int N, int C, int HW) {
   if (G > kChipMaxG || G < 1) return p;
   p.vpg = int((TV + G - 1) / G);
   p.G = int((TV + p.vpg - 1) / p.vpg);
-  p.ok = long(C) * p.G < 0x7fffffffL && !(p.ragged && p.nt != 512) && chip_slices_fit(p.G, C, p.nt);
+  p.ok = long(C) * p.G < 0x7fffffffL && chip_slices_fit(p.G, C, p.nt);
   return p;
 }
 
@@ -1031,6 +1038,11 @@ int launch_onchip(const typename S::elem *dy, const typename S::elem *x, const f
     }
   }
   if constexpr (S::VEC * sizeof(typename S::elem) == 16) {
+    if (p.ragged && p.nt == 1024) {
+      hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 1024, 0, true>), grid, dim3(1024), 0, st, dy, x, gamma, beta, save_mean,
+                         save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
+      return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
+    }
     if (p.ragged) {
       hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512, 0, true>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean,
                          save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
@@ -1231,9 +1243,10 @@ int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *g
   // (ragged planes of few elements -- 7 x 7 -- as well, unless the channels need more than two rounds of its
   // one workgroup per channel: f16 128 x 512 x 7 x 7 13.3 us there, 13.9 here, but 128 x 2048 x 7 x 7 42.6 against
   // 23.7 -- the LDS-resident kernel moves single elements)
-  // (fp32 shapes that give every CU a whole channel -- no exchange, G = 1 -- run faster in registers: 64 x 256 x 14 x 14
-  // 11.5 -> 10.2 us, 64 x 512 x 7 x 7 10.2 -> 7.7 us, kernels alone on cold tensors)
-  const bool small_resident = !(cp.ok && cp.G == 1 && sizeof(typename S::elem) == 4) &&
+  // (shapes that give every CU a whole channel -- no exchange, G = 1 -- run faster in registers: fp32 64 x 256 x 14 x 14
+  // 11.5 -> 10.2 us, 64 x 512 x 7 x 7 10.2 -> 7.7 us, kernels alone on cold tensors; binary16 128 x 512 x 7 x 7 16.3 ->
+  // 13.6 us between events)
+  const bool small_resident = !(cp.ok && cp.G == 1) &&
                               resident_ok(N, C, HW, sizeof(typename S::elem)) &&
                               (cp.ragged ? HW <= 64 && C <= 2 * sgh_num_cus() : long(N) * (HW / S::VEC) <= 4096);
   if (cp.ok && !small_resident && !sgh_env().bn_onchip_off) {
