@@ -282,8 +282,8 @@ def main():
         "kernel": "%s MFMA conv dgrad + wgrad kernels (%s; %d launches/step)"
                   % ("16-bit" if half else "fp32", ", ".join(kernels), launches // prof_steps),
         "flop_per_step": flop / prof_steps, "kernel_ms_per_step": round(ms / prof_steps, 4),
-        "timing": "HIP event pair around every launch in %d extra steps with all kernels on one stream "
-                  "(the timed steps run the weight gradients on a second stream)" % prof_steps,
+        "timing": "HIP events attached to each dispatch (the kernel's own start and end) in %d extra steps with all "
+                  "kernels on one stream (the timed steps run the weight gradients on a second stream)" % prof_steps,
     }
     for k, v in conv.items():
         roofline[k + "_tflops"] = round(v["work"] / (v["ms"] * 1e-3) / 1e12, 3) if v["ms"] > 0 else 0.0
@@ -291,7 +291,7 @@ def main():
     ops_ms = sum(prof[k]["ms"] for k in ("conv_dgrad_op", "conv_wgrad_op") if k in prof)
     roofline["entry_points_ms_per_step"] = round(ops_ms / prof_steps, 4)
 
-    # the bandwidth-bound families: algorithmic bytes (minimal tensor traffic) / time between the event pair
+    # the bandwidth-bound families: algorithmic bytes (minimal tensor traffic) / time between the two events
     hbm = {}
     for k in ("bn_relu_bwd", "bn_bwd", "relu_bwd", "relu_bwd_add", "add", "pool_bwd", "sgd"):
         if k in prof and prof[k]["ms"] > 0:
@@ -321,7 +321,8 @@ def main():
                            else "one call per reference op"},
         "roofline": roofline,
         "hbm_kernels": {"peak_GB/s": PEAK_HBM_GBS, "bytes": "algorithmic (every tensor of the op once)",
-                        "timing": "HIP event pair around each entry point, same extra steps as the roofline", **hbm},
+                        "timing": "HIP events attached to the dispatch where the entry point is one kernel, a pair of markers "
+                                  "around it otherwise; same extra steps as the roofline", **hbm},
         "host_enqueue_ms_per_step": round(t_enqueued / args.steps * 1e3, 4),
         "host_enqueue_ms_idle_queue": round(t_idle_enqueue * 1e3, 4),
     }

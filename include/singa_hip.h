@@ -145,10 +145,14 @@ SGH_API int sgh_event_elapsed_ms(sgh_event *start, sgh_event *stop, float *ms);
 /* Kernel-level profiling: the per-node timing of SINGA's Graph (Device::SetVerbosity,
  * TimeProfilingDoExec, Graph::PrintTimeProfiling: src/core/scheduler/scheduler.cc:240-295) at
  * kernel granularity.  While enabled, every GEMM / implicit-GEMM launch of this library is
- * bracketed by an event pair on its own stream and tagged with its algorithmic FLOP count:
+ * timed by two events on its own stream and tagged with its algorithmic FLOP count:
  * "conv_wgrad" / "conv_dgrad" / "conv_fwd" cover the MFMA kernel alone, "conv_*_op" the whole
  * entry point (weight re-layout, split-K reduction and column-gather kernels included), "gemm"
- * a dense GEMM.  Records nest.  sgh_prof_enable(1) clears old records.
+ * a dense GEMM; the bandwidth-bound entry points ("bn_bwd", "bn_relu_bwd", "relu_bwd", "add",
+ * "pool_bwd", "sgd" ...) are tagged with their algorithmic bytes.  A record of a single kernel
+ * hands its events to the dispatch itself (hipExtLaunchKernelGGL), so they carry the kernel's
+ * own start and end; a record over several kernels is a pair of markers around them, which adds
+ * a few microseconds of queue time.  Records nest.  sgh_prof_enable(1) clears old records.
  * sgh_prof_get waits for record i to finish and returns its tag, duration and work. */
 SGH_API int sgh_prof_enable(int on);
 /* Drops the records taken so far and destroys their events (sgh_prof_enable(1) does the same before it starts;

@@ -1032,29 +1032,29 @@ int launch_onchip(const typename S::elem *dy, const typename S::elem *x, const f
           return SGH_EUNSUPPORTED;
         attr = true;
       }
-      hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, ws,
+      SGH_LAUNCH_TIMED(kern, grid, dim3(512), lds, st, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, ws,
                          s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
       return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
     }
   }
   if constexpr (S::VEC * sizeof(typename S::elem) == 16) {
     if (p.ragged && p.nt == 1024) {
-      hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 1024, 0, true>), grid, dim3(1024), 0, st, dy, x, gamma, beta, save_mean,
+      SGH_LAUNCH_TIMED((k_bn_bwd_onchip<S, RELU, 1024, 0, true>), grid, dim3(1024), 0, st, dy, x, gamma, beta, save_mean,
                          save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
       return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
     }
     if (p.ragged) {
-      hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512, 0, true>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean,
+      SGH_LAUNCH_TIMED((k_bn_bwd_onchip<S, RELU, 512, 0, true>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean,
                          save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
       return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
     }
   }
   if (p.ragged) return SGH_EUNSUPPORTED;
   if (p.nt == 512)
-    hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 512>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean, save_invstd,
+    SGH_LAUNCH_TIMED((k_bn_bwd_onchip<S, RELU, 512>), grid, dim3(512), 0, st, dy, x, gamma, beta, save_mean, save_invstd,
                        dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
   else
-    hipLaunchKernelGGL((k_bn_bwd_onchip<S, RELU, 1024>), grid, dim3(1024), 0, st, dy, x, gamma, beta, save_mean,
+    SGH_LAUNCH_TIMED((k_bn_bwd_onchip<S, RELU, 1024>), grid, dim3(1024), 0, st, dy, x, gamma, beta, save_mean,
                        save_invstd, dx, dgamma, dbeta, ws, s, p.G, p.vpg, t1, t2, g_spin_limit.load(std::memory_order_relaxed), xcd_runs, dephase);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
@@ -1077,8 +1077,8 @@ int launch_resident(const typename S::elem *dy, const typename S::elem *x, const
     attr = true;
   }
   const size_t lds = 2 * resident_half_bytes(s.N, s.HW, sizeof(typename S::elem));
-  hipLaunchKernelGGL(kern, dim3((s.C + 7) / 8 * 8), dim3(kResNT), lds, st, dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta,
-                     s);
+  SGH_LAUNCH_TIMED(kern, dim3((s.C + 7) / 8 * 8), dim3(kResNT), lds, st, dy, x, gamma, beta, save_mean, save_invstd, dx,
+                   dgamma, dbeta, s);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -1236,7 +1236,7 @@ int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *g
   const dim3 grid(C * s.S), block(kBlock);
   hipStream_t st = sgh_stream_of(stream);
   // algorithmic bytes: x and dy in, dx out (the fused form covers the ReLU backward as well)
-  sgh_prof_scope prof(beta ? "bn_relu_bwd/k_bn_bwd" : "bn_bwd/k_bn_bwd", 3.0 * N * C * HW * sizeof(typename S::elem), st);
+  sgh_prof_kernel_scope prof(beta ? "bn_relu_bwd/k_bn_bwd" : "bn_bwd/k_bn_bwd", 3.0 * N * C * HW * sizeof(typename S::elem), st);
   const ChipPlan cp = chip_plan<S>(N, C, HW);
   // (channels of at most 4096 vectors that fit in LDS are a little faster through the LDS-resident kernel below:
   // 13.4 against 14.9 us at 64 x 256 x 14 x 14 fp32)
@@ -1259,6 +1259,7 @@ int bn_bwd(const typename S::elem *dy, const typename S::elem *x, const float *g
                         : launch_resident<S, false>(dy, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, s, st);
     if (rc != SGH_EUNSUPPORTED) return rc;
   }
+  prof.span();   // two kernels
   if (beta) {
     hipLaunchKernelGGL((k_bn_bwd_partial<S, true>), grid, block, 0, st, dy, x, gamma, beta, save_mean, save_invstd, part, s);
     SGH_LAUNCH_CHECK();

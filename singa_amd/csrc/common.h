@@ -3,6 +3,7 @@
 #define SINGA_AMD_CSRC_COMMON_H_
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -87,6 +88,39 @@ struct sgh_prof_scope {
   sgh_prof_scope(const sgh_prof_scope &) = delete;
   sgh_prof_scope &operator=(const sgh_prof_scope &) = delete;
 };
+
+// Record for a scope that encloses ONE kernel launch made through SGH_LAUNCH_TIMED: the record's two events
+// are handed to that dispatch (hipExtLaunchKernelGGL), so they carry the kernel's own start and end rather
+// than two markers queued around it (which add a few microseconds to a short kernel).  A path with more
+// than one launch calls span() first and is then timed by markers like sgh_prof_scope; a scope that
+// launched nothing leaves a zero-length record.
+void sgh_prof_kernel_begin(const char *tag, double work);
+bool sgh_prof_kernel_take(hipEvent_t *start, hipEvent_t *stop);   // true once, for the launch after _begin
+void sgh_prof_kernel_span(hipStream_t s);
+void sgh_prof_kernel_end(hipStream_t s);
+struct sgh_prof_kernel_scope {
+  hipStream_t s;
+  bool on;
+  sgh_prof_kernel_scope(const char *tag, double work, hipStream_t s_) : s(s_), on(sgh_prof_on()) {
+    if (on) sgh_prof_kernel_begin(tag, work);
+  }
+  void span() {
+    if (on) sgh_prof_kernel_span(s);
+  }
+  ~sgh_prof_kernel_scope() {
+    if (on) sgh_prof_kernel_end(s);
+  }
+  sgh_prof_kernel_scope(const sgh_prof_kernel_scope &) = delete;
+  sgh_prof_kernel_scope &operator=(const sgh_prof_kernel_scope &) = delete;
+};
+#define SGH_LAUNCH_TIMED(kern, grid, block, lds, stream, ...)                                                    \
+  do {                                                                                                           \
+    hipEvent_t sgh_ev_a_, sgh_ev_b_;                                                                             \
+    if (sgh_prof_on() && sgh_prof_kernel_take(&sgh_ev_a_, &sgh_ev_b_))                                           \
+      hipExtLaunchKernelGGL(kern, grid, block, lds, stream, sgh_ev_a_, sgh_ev_b_, 0, __VA_ARGS__);               \
+    else                                                                                                         \
+      hipLaunchKernelGGL(kern, grid, block, lds, stream, __VA_ARGS__);                                           \
+  } while (0)
 
 // 3x3 (stride 1 or 2) weight gradient with a shared LDS input tile (wgrad3x3.hip).  *_run returns
 // SGH_EUNSUPPORTED for geometries it does not cover; *_workspace_bytes is 0 for those.

@@ -1155,7 +1155,7 @@ int launch_w(const W16Args &a, const W16Plan &p, hipStream_t s) {
     if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
     attr = true;
   }
-  hipLaunchKernelGGL(kern, dim3(unsigned(p.mtiles * p.ntiles) * unsigned(p.splits)), dim3(NT), lds, s, a);
+  SGH_LAUNCH_TIMED(kern, dim3(unsigned(p.mtiles * p.ntiles) * unsigned(p.splits)), dim3(NT), lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -1168,7 +1168,7 @@ int launch_d(const D16Args &a, const D16Plan &p, hipStream_t s) {
     if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
     attr = true;
   }
-  hipLaunchKernelGGL(kern, dim3(unsigned((p.tiles + 7) / 8) * 8u * unsigned(p.mtiles)), dim3(NT), lds, s, a);
+  SGH_LAUNCH_TIMED(kern, dim3(unsigned((p.tiles + 7) / 8) * 8u * unsigned(p.mtiles)), dim3(NT), lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -1182,7 +1182,7 @@ int launch_slab2(const S16Args &a, const D16Plan &p, hipStream_t s) {
     if (!allow_lds(kern, lds)) return SGH_EUNSUPPORTED;
     allowed = lds;
   }
-  hipLaunchKernelGGL(kern, dim3(unsigned((p.tiles + 7) / 8) * 8u * unsigned(p.mtiles)), dim3(NT), lds, s, a);
+  SGH_LAUNCH_TIMED(kern, dim3(unsigned((p.tiles + 7) / 8) * 8u * unsigned(p.mtiles)), dim3(NT), lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -1255,7 +1255,7 @@ int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
   a.chunks = p.chunks, a.chunks_per_split = p.cps;
   a.dy_elems = long(g->N) * g->K * g->P * g->Q, a.x_elems = long(g->N) * g->C * g->H * g->W;
   const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
-  sgh_prof_start("conv_wgrad16/k_wgrad16", flops, s);
+  sgh_prof_kernel_begin("conv_wgrad16/k_wgrad16", flops);
   int rc;
   if (p.bm == 128) {
     if (p.stride == 1) rc = bf16 ? launch_w<128, 1, true>(a, p, s) : launch_w<128, 1, false>(a, p, s);
@@ -1264,7 +1264,7 @@ int sgh_conv16_wgrad(const sgh_conv_geom *g, const uint16_t *dy, const uint16_t 
     if (p.stride == 1) rc = bf16 ? launch_w<64, 1, true>(a, p, s) : launch_w<64, 1, false>(a, p, s);
     else rc = bf16 ? launch_w<64, 2, true>(a, p, s) : launch_w<64, 2, false>(a, p, s);
   }
-  sgh_prof_stop(s);
+  sgh_prof_kernel_end(s);
   if (rc != SGH_OK) return rc;
   const size_t n = size_t(g->K) * a.CRS;
   if (n / 64 >= size_t(2 * sgh_num_cus()) || p.splits < 16) {
@@ -1317,12 +1317,12 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
     b.Wp = g->W + 1, b.HpWp = (g->H + 1) * (g->W + 1), b.SP = p.slab_sp, b.G = g->N * b.HpWp;
     b.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2), b.wt_bytes = unsigned(nw * 2);
     const double fl = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * 9;
-    sgh_prof_start(fwd_of ? "conv_fwd16/k_dgrad16_slab" : "conv_dgrad16/k_dgrad16_slab", fl, s);
+    sgh_prof_kernel_begin(fwd_of ? "conv_fwd16/k_dgrad16_slab" : "conv_dgrad16/k_dgrad16_slab", fl);
     int rc;
     if (p.slab == 1) rc = launch_slab<2, 2, 1, 4>(b, p, bf16, s);
     else if (p.slab == 2) rc = launch_slab<2, 2, 2, 4>(b, p, bf16, s);
     else rc = launch_slab<2, 2, 2, 2>(b, p, bf16, s);
-    sgh_prof_stop(s);
+    sgh_prof_kernel_end(s);
     return rc;
   }
   D16Args a{};
@@ -1339,7 +1339,7 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
   a.dy_bytes = unsigned(size_t(g->N) * g->K * g->P * g->Q * 2);
   a.wt_bytes = unsigned(nw * 2);
   const double flops = 2.0 * g->N * g->K * g->P * g->Q * double(g->C) * g->R * g->S;
-  sgh_prof_start(fwd_of ? "conv_fwd16/k_dgrad16" : "conv_dgrad16/k_dgrad16", flops, s);
+  sgh_prof_kernel_begin(fwd_of ? "conv_fwd16/k_dgrad16" : "conv_dgrad16/k_dgrad16", flops);
   int rc;
   if (p.pixk) {
     if (p.bm == 128) rc = bf16 ? launch_d<128, true, true>(a, p, s) : launch_d<128, false, true>(a, p, s);
@@ -1348,7 +1348,7 @@ int run_d16(const sgh_conv_geom *g, const sgh_conv_geom *fwd_of, const uint16_t 
     if (p.bm == 128) rc = bf16 ? launch_d<128, true, false>(a, p, s) : launch_d<128, false, false>(a, p, s);
     else rc = bf16 ? launch_d<64, true, false>(a, p, s) : launch_d<64, false, false>(a, p, s);
   }
-  sgh_prof_stop(s);
+  sgh_prof_kernel_end(s);
   return rc;
 }
 

@@ -438,7 +438,7 @@ int launch(const D3Args &a, const D3Plan &p, dim3 grid, hipStream_t s) {
       return SGH_EUNSUPPORTED;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(NT), p.lds, s, a);
+  SGH_LAUNCH_TIMED(kern, grid, dim3(NT), p.lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -484,7 +484,7 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   a.wt_bytes = unsigned(size_t(9) * KP * g->C * 4);
   dim3 grid(unsigned(p.dp_tiles + p.sk_wgs), 1, 1);
   int rc = SGH_EUNSUPPORTED;
-  sgh_prof_start(tag, 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
+  sgh_prof_kernel_begin(tag, 2.0 * g->N * g->K * g->P * g->Q * g->C * 9);
 #define D3_CASE(BM_, LOGP_, VR_) \
   if (!p.s2 && p.bm == BM_ && p.logp == LOGP_ && p.vr == VR_) rc = launch<BM_, LOGP_, VR_, false>(a, p, grid, s);
 #define D3_CASE_S2(LOGP_, VR_) \
@@ -502,7 +502,7 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   D3_CASE_S2(3, 32)
 #undef D3_CASE
 #undef D3_CASE_S2
-  sgh_prof_stop(s);
+  sgh_prof_kernel_end(s);
   if (rc != SGH_OK) return rc;
   if (p.sk_wgs > 0) {
     const int shared_tiles = p.tiles - p.dp_tiles;

@@ -382,7 +382,7 @@ int launch(const DFArgs &a, const DFPlan &p, dim3 grid, hipStream_t s) {
       return SGH_EUNSUPPORTED;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(NT), p.lds, s, a);
+  SGH_LAUNCH_TIMED(kern, grid, dim3(NT), p.lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -421,7 +421,7 @@ static int dgrad_fewc_run(const sgh_conv_geom *g, const void *dy, const float *W
   dim3 grid((g->P + TI - 1) / TI, g->N, 1);
   if (grid.y > 65535u) return SGH_EUNSUPPORTED;
   int rc = SGH_EUNSUPPORTED;
-  sgh_prof_start(tag, 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S, s);
+  sgh_prof_kernel_begin(tag, 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S);
   switch (p.qt) {
     case 1: rc = launch<1, S>(a, p, grid, s); break;
     case 2: rc = launch<2, S>(a, p, grid, s); break;
@@ -433,7 +433,7 @@ static int dgrad_fewc_run(const sgh_conv_geom *g, const void *dy, const float *W
     case 8: rc = launch<8, S>(a, p, grid, s); break;
     default: break;
   }
-  sgh_prof_stop(s);
+  sgh_prof_kernel_end(s);
   return rc;
 }
 
@@ -454,7 +454,7 @@ int launch16(const DF16Args &a, size_t lds, dim3 grid, hipStream_t s) {
       return SGH_EUNSUPPORTED;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
+  SGH_LAUNCH_TIMED(kern, grid, dim3(256), lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -473,7 +473,7 @@ int dgrad_fewc16_mfma(const sgh_conv_geom *g, const DFPlan &p, const uint16_t *d
   const dim3 grid((g->P + TI16 - 1) / TI16, g->N, 1);
   const size_t lds = size_t(SR16) * (p.qt * 16 + 8) * KP16 * sizeof(uint16_t);
   int rc = SGH_EUNSUPPORTED;
-  sgh_prof_start("conv_dgrad16/k_dgrad_fewc16", 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S, s);
+  sgh_prof_kernel_begin("conv_dgrad16/k_dgrad_fewc16", 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S);
   switch (p.qt) {
     case 1: rc = launch16<1, BF16>(a, lds, grid, s); break;
     case 2: rc = launch16<2, BF16>(a, lds, grid, s); break;
@@ -485,7 +485,7 @@ int dgrad_fewc16_mfma(const sgh_conv_geom *g, const DFPlan &p, const uint16_t *d
     case 8: rc = launch16<8, BF16>(a, lds, grid, s); break;
     default: break;
   }
-  sgh_prof_stop(s);
+  sgh_prof_kernel_end(s);
   return rc;
 }
 

@@ -94,13 +94,13 @@ int launch_map2(const float *a, const float *b, float *o, size_t n, F f, void *s
   if (!a || !b || !o) return SGH_EINVAL;
   if (sgh_aligned16(a) && sgh_aligned16(b) && sgh_aligned16(o)) {
     if (n * sizeof(float) >= kStreamBytes)
-      hipLaunchKernelGGL((k_map2_1<F, true>), dim3(grid_for(n >> 2)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o, n,
+      SGH_LAUNCH_TIMED((k_map2_1<F, true>), dim3(grid_for(n >> 2)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o, n,
                          f);
     else
-      hipLaunchKernelGGL((k_map2_1<F, false>), dim3(grid_for(n >> 2)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o,
+      SGH_LAUNCH_TIMED((k_map2_1<F, false>), dim3(grid_for(n >> 2)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o,
                          n, f);
   } else {
-    hipLaunchKernelGGL(k_map2_1_scalar<F>, dim3(grid_for(n)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o, n, f);
+    SGH_LAUNCH_TIMED(k_map2_1_scalar<F>, dim3(grid_for(n)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o, n, f);
   }
   SGH_LAUNCH_CHECK();
   return SGH_OK;
@@ -527,7 +527,7 @@ inline int cast_grid(size_t n) {
 extern "C" {
 
 int sgh_relu_bwd_f32(const float *dy, const float *x, float *dx, size_t n, void *stream) {
-  sgh_prof_scope prof("relu_bwd/k_map2_1<ReluBwd>", 3.0 * n * sizeof(float), sgh_stream_of(stream));
+  sgh_prof_kernel_scope prof("relu_bwd/k_map2_1<ReluBwd>", 3.0 * n * sizeof(float), sgh_stream_of(stream));
   return launch_map2(dy, x, dx, n, ReluBwd{}, stream);
 }
 
@@ -558,7 +558,7 @@ int sgh_clamp_f32(float low, float high, const float *x, float *out, size_t n, v
 
 int sgh_add_f32(const float *a, const float *b, float *out, size_t n, void *stream) {
   sgh_note_write(out, n * sizeof(float));
-  sgh_prof_scope prof("add/k_map2_1<AddOp>", 3.0 * n * sizeof(float), sgh_stream_of(stream));
+  sgh_prof_kernel_scope prof("add/k_map2_1<AddOp>", 3.0 * n * sizeof(float), sgh_stream_of(stream));
   return launch_map2(a, b, out, n, AddOp{}, stream);
 }
 
@@ -654,8 +654,8 @@ int sgh_sgd_momentum_multi_f32(const sgh_sgd_item *table_dev, int count, size_t 
   size_t chunks = total_n / kChunk + size_t(count);  // upper bound on sum of per-item chunk counts
   const size_t cap = size_t(sgh_num_cus()) * 8;
   if (chunks > cap) chunks = cap;
-  sgh_prof_scope prof("sgd/k_sgd_multi", 20.0 * total_n, sgh_stream_of(stream));   // p, g, v in; p, v out
-  hipLaunchKernelGGL(k_sgd_multi, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count,
+  sgh_prof_kernel_scope prof("sgd/k_sgd_multi", 20.0 * total_n, sgh_stream_of(stream));   // p, g, v in; p, v out
+  SGH_LAUNCH_TIMED(k_sgd_multi, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count,
                      SgdHyper{lr, mu, damp, wd}, nesterov);
   SGH_LAUNCH_CHECK();
   return SGH_OK;

@@ -91,7 +91,7 @@ int launch_map2_h(const uint16_t *a, const uint16_t *b, uint16_t *o, size_t n, F
   if (n == 0) return SGH_OK;
   if (!a || !b || !o) return SGH_EINVAL;
   const int vec = sgh_aligned16(a) && sgh_aligned16(b) && sgh_aligned16(o);
-  hipLaunchKernelGGL((k_map2_h<T, F>), dim3(grid_for(vec ? n >> 3 : n)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o,
+  SGH_LAUNCH_TIMED((k_map2_h<T, F>), dim3(grid_for(vec ? n >> 3 : n)), dim3(kBlock), 0, sgh_stream_of(stream), a, b, o,
                      n, f, vec);
   SGH_LAUNCH_CHECK();
   return SGH_OK;
@@ -153,7 +153,7 @@ int launch_relu_bwd_add(const typename S::elem *dy0, const typename S::elem *dy1
   if (n == 0) return SGH_OK;
   if (!dy0 || !dy1 || !x || !dx) return SGH_EINVAL;
   const int vec = sgh_aligned16(dy0) && sgh_aligned16(dy1) && sgh_aligned16(x) && sgh_aligned16(dx);
-  hipLaunchKernelGGL(k_relu_bwd_add<S>, dim3(grid_for(vec ? n / S::VEC : n)), dim3(kBlock), 0, sgh_stream_of(stream),
+  SGH_LAUNCH_TIMED(k_relu_bwd_add<S>, dim3(grid_for(vec ? n / S::VEC : n)), dim3(kBlock), 0, sgh_stream_of(stream),
                      dy0, dy1, x, dx, n, vec);
   SGH_LAUNCH_CHECK();
   return SGH_OK;
@@ -411,9 +411,9 @@ int sgh_sgd_momentum_multi_mixed(const sgh_sgd_mixed_item *table_dev, int count,
   if (chunks > cap) chunks = cap;
   const SgdHyper h{lr, mu, damp, wd};
   // fp32 items: p, g, v in, p, v out; 16-bit items: p, v (4) + g (2) in, p, v (4) + p16 (2) out: 20 bytes either way
-  sgh_prof_scope prof("sgd/k_sgd_multi_mixed", 20.0 * total_n, sgh_stream_of(stream));
-  if (bf16) hipLaunchKernelGGL(k_sgd_multi_mixed<BF16>, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count, h, nesterov);
-  else hipLaunchKernelGGL(k_sgd_multi_mixed<F16>, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count, h, nesterov);
+  sgh_prof_kernel_scope prof("sgd/k_sgd_multi_mixed", 20.0 * total_n, sgh_stream_of(stream));
+  if (bf16) SGH_LAUNCH_TIMED(k_sgd_multi_mixed<BF16>, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count, h, nesterov);
+  else SGH_LAUNCH_TIMED(k_sgd_multi_mixed<F16>, dim3(int(chunks)), dim3(kBlock), 0, sgh_stream_of(stream), table_dev, count, h, nesterov);
   SGH_LAUNCH_CHECK();
   return SGH_OK;
 }
@@ -453,35 +453,35 @@ int sgh_relu_fwd_bf16(const uint16_t *x, uint16_t *y, size_t n, void *stream) {
   return launch_map2_h<BF16>(x, x, y, n, ReluFwd{}, stream);
 }
 int sgh_relu_bwd_f16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream) {
-  sgh_prof_scope prof("relu_bwd/k_map2_h<ReluBwd>", 3.0 * n * 2, sgh_stream_of(stream));
+  sgh_prof_kernel_scope prof("relu_bwd/k_map2_h<ReluBwd>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<F16>(dy, x, dx, n, ReluBwd{}, stream);
 }
 int sgh_relu_bwd_bf16(const uint16_t *dy, const uint16_t *x, uint16_t *dx, size_t n, void *stream) {
-  sgh_prof_scope prof("relu_bwd/k_map2_h<ReluBwd>", 3.0 * n * 2, sgh_stream_of(stream));
+  sgh_prof_kernel_scope prof("relu_bwd/k_map2_h<ReluBwd>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<BF16>(dy, x, dx, n, ReluBwd{}, stream);
 }
 int sgh_relu_bwd_add_f32(const float *dy0, const float *dy1, const float *x, float *dx, size_t n, void *stream) {
-  sgh_prof_scope prof("relu_bwd_add/k_relu_bwd_add", 4.0 * n * 4, sgh_stream_of(stream));
+  sgh_prof_kernel_scope prof("relu_bwd_add/k_relu_bwd_add", 4.0 * n * 4, sgh_stream_of(stream));
   return launch_relu_bwd_add<StF32>(dy0, dy1, x, dx, n, stream);
 }
 int sgh_relu_bwd_add_f16(const uint16_t *dy0, const uint16_t *dy1, const uint16_t *x, uint16_t *dx, size_t n,
                          void *stream) {
-  sgh_prof_scope prof("relu_bwd_add/k_relu_bwd_add", 4.0 * n * 2, sgh_stream_of(stream));
+  sgh_prof_kernel_scope prof("relu_bwd_add/k_relu_bwd_add", 4.0 * n * 2, sgh_stream_of(stream));
   return launch_relu_bwd_add<StF16>(dy0, dy1, x, dx, n, stream);
 }
 int sgh_relu_bwd_add_bf16(const uint16_t *dy0, const uint16_t *dy1, const uint16_t *x, uint16_t *dx, size_t n,
                           void *stream) {
-  sgh_prof_scope prof("relu_bwd_add/k_relu_bwd_add", 4.0 * n * 2, sgh_stream_of(stream));
+  sgh_prof_kernel_scope prof("relu_bwd_add/k_relu_bwd_add", 4.0 * n * 2, sgh_stream_of(stream));
   return launch_relu_bwd_add<StBF16>(dy0, dy1, x, dx, n, stream);
 }
 int sgh_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
   sgh_note_write(out, n * 2);
-  sgh_prof_scope prof("add/k_map2_h<AddOp>", 3.0 * n * 2, sgh_stream_of(stream));
+  sgh_prof_kernel_scope prof("add/k_map2_h<AddOp>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<F16>(a, b, out, n, AddOp{}, stream);
 }
 int sgh_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {
   sgh_note_write(out, n * 2);
-  sgh_prof_scope prof("add/k_map2_h<AddOp>", 3.0 * n * 2, sgh_stream_of(stream));
+  sgh_prof_kernel_scope prof("add/k_map2_h<AddOp>", 3.0 * n * 2, sgh_stream_of(stream));
   return launch_map2_h<BF16>(a, b, out, n, AddOp{}, stream);
 }
 int sgh_add_relu_f16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n, void *stream) {

@@ -792,10 +792,10 @@ inline int launch_igemm(const LA &la, const LB &lb, const ST &st, int M, int N, 
                         int chunks_per_split, hipStream_t stream, const char *tag = nullptr, double flops = 0) {
   dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
   if (grid.y > 65535u || grid.z > 65535u) return SGH_EUNSUPPORTED;
-  if (tag) sgh_prof_start(tag, flops, stream);  // kernel-level record: this launch only
-  hipLaunchKernelGGL((k_igemm<BM, BN, LA, LB, ST, AK, BKc, ZCLASS, WGM, PF>), grid, dim3(NT), 0, stream, la, lb, st,
+  if (tag) sgh_prof_kernel_begin(tag, flops);  // kernel-level record: this launch only
+  SGH_LAUNCH_TIMED((k_igemm<BM, BN, LA, LB, ST, AK, BKc, ZCLASS, WGM, PF>), grid, dim3(NT), 0, stream, la, lb, st,
                      Ktotal, chunks_per_split);
-  if (tag) sgh_prof_stop(stream);
+  if (tag) sgh_prof_kernel_end(stream);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 

@@ -327,10 +327,10 @@ int sgh_pw_dgrad_run(const sgh_conv_geom *g, const float *dy, const float *W, fl
   a.ctiles = big ? (a.ncols + 63) / 64 : (a.ncols + 31) / 32;
   const long waves = long(a.mtiles) * a.ctiles;
   const unsigned blocks = unsigned((waves + 3) / 4);
-  sgh_prof_start("conv_dgrad/k_pw_dgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C, s);
-  if (big) hipLaunchKernelGGL((k_pw_dgrad<2, 2>), dim3(blocks), dim3(256), 0, s, a);
-  else hipLaunchKernelGGL((k_pw_dgrad<1, 1>), dim3(blocks), dim3(256), 0, s, a);
-  sgh_prof_stop(s);
+  sgh_prof_kernel_begin("conv_dgrad/k_pw_dgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C);
+  if (big) SGH_LAUNCH_TIMED((k_pw_dgrad<2, 2>), dim3(blocks), dim3(256), 0, s, a);
+  else SGH_LAUNCH_TIMED((k_pw_dgrad<1, 1>), dim3(blocks), dim3(256), 0, s, a);
+  sgh_prof_kernel_end(s);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -352,11 +352,11 @@ int sgh_pw_wgrad_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
   const int QP = (g->Q + 1) | 1;
   const size_t lds = size_t(2) * (128 + 64) * QP * sizeof(float);
   const dim3 grid(unsigned(p.mtiles * p.ntiles * p.splits));
-  sgh_prof_start("conv_wgrad/k_pw_wgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C, s);
-  if (g->Q == 7) hipLaunchKernelGGL(k_pw_wgrad<7>, grid, dim3(256), lds, s, a);
-  else if (g->Q == 14) hipLaunchKernelGGL(k_pw_wgrad<14>, grid, dim3(256), lds, s, a);
-  else hipLaunchKernelGGL(k_pw_wgrad<28>, grid, dim3(256), lds, s, a);
-  sgh_prof_stop(s);
+  sgh_prof_kernel_begin("conv_wgrad/k_pw_wgrad", 2.0 * g->N * g->K * g->P * g->Q * g->C);
+  if (g->Q == 7) SGH_LAUNCH_TIMED(k_pw_wgrad<7>, grid, dim3(256), lds, s, a);
+  else if (g->Q == 14) SGH_LAUNCH_TIMED(k_pw_wgrad<14>, grid, dim3(256), lds, s, a);
+  else SGH_LAUNCH_TIMED(k_pw_wgrad<28>, grid, dim3(256), lds, s, a);
+  sgh_prof_kernel_end(s);
   if (hipGetLastError() != hipSuccess) return SGH_EINVAL;
   const long n = long(g->K) * g->C;
   hipLaunchKernelGGL(k_pw_wgrad_reduce, dim3(unsigned((n + 15) / 16)), dim3(256), 0, s, a.part, dW, n, p.splits);

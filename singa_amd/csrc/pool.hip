@@ -580,7 +580,7 @@ int pool_bwd(const sgh_pool_geom *g, const typename S::elem *dy, const typename 
   if (g->is_max && !x) return SGH_EINVAL;
   const size_t total = size_t(g->N) * g->C * g->H * g->W;
   // algorithmic bytes: dy and (max pooling) x in, dx out
-  sgh_prof_scope prof(g->is_max ? "pool_bwd/k_pool_max_bwd" : "pool_bwd/k_pool_avg_bwd",
+  sgh_prof_kernel_scope prof(g->is_max ? "pool_bwd/k_pool_max_bwd" : "pool_bwd/k_pool_avg_bwd",
                       double(sizeof(typename S::elem)) *
                           (double(total) * (g->is_max ? 2 : 1) + double(g->N) * g->C * g->P * g->Q),
                       sgh_stream_of(stream));
@@ -590,7 +590,7 @@ int pool_bwd(const sgh_pool_geom *g, const typename S::elem *dy, const typename 
       sgh_aligned16(dx)) {
     const int bands = (g->H / 2 + 4 * kStripRows - 1) / (4 * kStripRows);
     const size_t lds = size_t(8 * kStripRows + 3) * (g->W + S::VEC) * sizeof(typename S::elem);   // <= 61 KB
-    hipLaunchKernelGGL(k_pool_max_bwd_3x3s2<S>, dim3(unsigned(size_t(g->N) * g->C * bands)), dim3(kBlock), lds,
+    SGH_LAUNCH_TIMED(k_pool_max_bwd_3x3s2<S>, dim3(unsigned(size_t(g->N) * g->C * bands)), dim3(kBlock), lds,
                        sgh_stream_of(stream), dy, x, dx, g->H, g->W, bands);
   } else if (g->is_max) {
     // band height: about 12 KB of x rows per workgroup (measured optimum: enough workgroups per CU to
@@ -613,18 +613,18 @@ int pool_bwd(const sgh_pool_geom *g, const typename S::elem *dy, const typename 
         kern = k_pool_max_bwd_tiled<2, 2, 2, 2, S>;
       else if (g->kernel_h == 3 && g->kernel_w == 3 && g->stride_h == 1 && g->stride_w == 1)
         kern = k_pool_max_bwd_tiled<3, 3, 1, 1, S>;
-      hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBlock), lds, sgh_stream_of(stream), dy, x, dx, to_g(g), TH,
+      SGH_LAUNCH_TIMED(kern, dim3((unsigned)blocks), dim3(kBlock), lds, sgh_stream_of(stream), dy, x, dx, to_g(g), TH,
                          bands, max_xrows, max_np);
     } else {
-      hipLaunchKernelGGL(k_pool_max_bwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
+      SGH_LAUNCH_TIMED(k_pool_max_bwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, x, dx,
                          to_g(g), total);
     }
   } else if (g->P == 1 && g->Q == 1 && g->pad_h == 0 && g->pad_w == 0 && g->kernel_h >= g->H && g->kernel_w >= g->W &&
              sgh_aligned16(dx))
-    hipLaunchKernelGGL(k_pool_avg_bwd_global<S>, dim3(grid_for((total + S::VEC - 1) / S::VEC)), dim3(kBlock), 0,
+    SGH_LAUNCH_TIMED(k_pool_avg_bwd_global<S>, dim3(grid_for((total + S::VEC - 1) / S::VEC)), dim3(kBlock), 0,
                        sgh_stream_of(stream), dy, dx, g->H * g->W, total);
   else
-    hipLaunchKernelGGL(k_pool_avg_bwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, dx, to_g(g),
+    SGH_LAUNCH_TIMED(k_pool_avg_bwd<S>, dim3(grid_for(total)), dim3(kBlock), 0, sgh_stream_of(stream), dy, dx, to_g(g),
                        total);
   SGH_LAUNCH_CHECK();
   return SGH_OK;

@@ -197,7 +197,51 @@ void sgh_prof_stop(hipStream_t s) {
   g_prof_open.pop_back();
 }
 
+// record whose events wait for the one launch of a sgh_prof_kernel_scope (-1: none); a record that turned
+// into a marker pair sits in g_prof_open like any other
+static long g_prof_kernel = -1;
+static bool g_prof_kernel_spanned = false;
+
+void sgh_prof_kernel_begin(const char *tag, double work) {
+  g_prof_kernel = -1;
+  g_prof_kernel_spanned = false;
+  if (!g_prof_on) return;
+  ProfRec r{tag, work, nullptr, nullptr};
+  if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) return;
+  g_prof_kernel = long(g_prof.size());
+  g_prof.push_back(r);
+}
+
+bool sgh_prof_kernel_take(hipEvent_t *start, hipEvent_t *stop) {
+  if (g_prof_kernel < 0) return false;
+  *start = g_prof[size_t(g_prof_kernel)].a;
+  *stop = g_prof[size_t(g_prof_kernel)].b;
+  g_prof_kernel = -1;
+  return true;
+}
+
+void sgh_prof_kernel_span(hipStream_t s) {
+  if (g_prof_kernel < 0) return;
+  (void)hipEventRecord(g_prof[size_t(g_prof_kernel)].a, s);
+  g_prof_open.push_back(size_t(g_prof_kernel));
+  g_prof_kernel = -1;
+  g_prof_kernel_spanned = true;
+}
+
+void sgh_prof_kernel_end(hipStream_t s) {
+  if (g_prof_kernel_spanned) {
+    g_prof_kernel_spanned = false;
+    sgh_prof_stop(s);
+  } else if (g_prof_kernel >= 0) {   // nothing was launched
+    (void)hipEventRecord(g_prof[size_t(g_prof_kernel)].a, s);
+    (void)hipEventRecord(g_prof[size_t(g_prof_kernel)].b, s);
+    g_prof_kernel = -1;
+  }
+}
+
 static void prof_clear() {
+  g_prof_kernel = -1;
+  g_prof_kernel_spanned = false;
   for (auto &r : g_prof) {
     if (r.a) (void)hipEventDestroy(r.a);
     if (r.b) (void)hipEventDestroy(r.b);

@@ -395,7 +395,7 @@ int launch(const W3Args &a, const W3Plan &p, dim3 grid, hipStream_t s) {
       return SGH_EUNSUPPORTED;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(NT), p.lds, s, a);
+  SGH_LAUNCH_TIMED(kern, grid, dim3(NT), p.lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -433,7 +433,7 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
   a.units_per_split = p.units_per_split;
   dim3 grid((g->K + p.bm - 1) / p.bm, (g->C + p.bc - 1) / p.bc, p.splits);
   int rc = SGH_EUNSUPPORTED;
-  sgh_prof_start("conv_wgrad/k_wgrad3x3", 2.0 * g->N * g->K * g->P * g->Q * g->C * 9, s);
+  sgh_prof_kernel_begin("conv_wgrad/k_wgrad3x3", 2.0 * g->N * g->K * g->P * g->Q * g->C * 9);
 #define W3_CASE(BM_, BC_, LOGP_, ROWS_) \
   if (p.bm == BM_ && p.bc == BC_ && p.logp == LOGP_ && p.rows == ROWS_) rc = launch<BM_, BC_, LOGP_, ROWS_>(a, p, grid, s);
   W3_CASE(128, 32, 6, 3)
@@ -448,7 +448,7 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
   W3_CASE(128, 32, 5, 9)
   W3_CASE(128, 32, 4, 15)
 #undef W3_CASE
-  sgh_prof_stop(s);
+  sgh_prof_kernel_end(s);
   if (rc != SGH_OK) return rc;
   // pairs per reduction workgroup: small layers take fewer pairs and more z-lanes per workgroup
   const long kc = long(g->K) * g->C;

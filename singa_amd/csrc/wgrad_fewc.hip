@@ -324,7 +324,7 @@ int launch(const WFArgs &a, const WFPlan &p, dim3 grid, hipStream_t s) {
       return SGH_EUNSUPPORTED;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(NT), p.lds, s, a);
+  SGH_LAUNCH_TIMED(kern, grid, dim3(NT), p.lds, s, a);
   return hipGetLastError() == hipSuccess ? SGH_OK : SGH_EINVAL;
 }
 
@@ -361,9 +361,9 @@ int sgh_wgrad_fewc_run(const sgh_conv_geom *g, const float *dy, const float *x, 
   a.total_units = p.total_units;
   a.units_per_split = p.units_per_split;
   dim3 grid((g->K + BM - 1) / BM, 1, p.splits);
-  sgh_prof_start("conv_wgrad/k_wgrad_fewc", 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S, s);
+  sgh_prof_kernel_begin("conv_wgrad/k_wgrad_fewc", 2.0 * g->N * g->K * g->P * g->Q * g->C * g->R * g->S);
   const int rc = g->stride_h == 1 ? launch<1>(a, p, grid, s) : launch<2>(a, p, grid, s);
-  sgh_prof_stop(s);
+  sgh_prof_kernel_end(s);
   if (rc != SGH_OK) return rc;
   const long n = long(g->K) * g->C * g->R * g->S;
   hipLaunchKernelGGL(k_wgrad_fewc_reduce, dim3(int((n + 15) / 16)), dim3(256), 0, s, a.part, dW, n, p.splits);
