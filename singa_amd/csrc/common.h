@@ -36,6 +36,7 @@ struct sgh_env_switches {
   bool dgrad3x3_off, wgrad3x3_off, dgrad_fewc_off, wgrad_fewc_off, dgrad_pointwise_off, conv16_off, bn_onchip_off, pw_dgrad_off, pw_wgrad_off, dgrad_fewc16_off, slab16_off, bn_ragged_off, fwd_fewc_off, bn_fwd_onchip_off;
   int dgrad_tile, wgrad_tile, pw_tile;   // -1: chosen from the geometry
   int dgrad3x3_bm;              // 0: chosen from the geometry, else 64 or 128
+  bool conv_xcd_off;            // tiles dealt to workgroups in launch order instead of per XCD
 };
 const sgh_env_switches &sgh_env();
 

@@ -53,9 +53,23 @@ struct D3Args {
   // reduction chunk of one tile (unit u = tile dp_tiles + u / nchunks, chunk u % nchunks).
   int ctiles, dp_tiles, sk_wgs;
   long sk_units;
+  int xcd_runs;           // whole-tile workgroups take their tiles in runs per XCD (whole_tile_of)
   float *partials;        // [sk_wgs][2][classes * BM * BN]: a workgroup's first / last incomplete tile
   unsigned dy_bytes, wt_bytes;
 };
+
+// Tile of whole-tile workgroup w.  Workgroup w runs on XCD w % 8 and every XCD has an L2 of its own, so the
+// j-th workgroup of XCD x takes tile ((j / 8) * 8 + x) * 8 + j % 8: an XCD works on runs of eight consecutive
+// tiles at a time, which share the halo rows of their dy slabs (and, for several channel tiles per pixel
+// tile, the whole slab) in its L2.  Measured on the ResNet-18 layers: the kernels fetch a third to a quarter of
+// the bytes into L2 (C64 56x56: 246 -> 65 MB per launch) at the same speed; whole contiguous ranges per XCD, and
+// the same treatment of the workgroups that share tiles, ran 1.5-3 % slower.  Only which hardware computes
+// which tile changes: results are identical.
+__device__ __forceinline__ int whole_tile_of(const D3Args &a, int w) {
+  if (!a.xcd_runs) return w;
+  const int x = w & 7, j = w >> 3;
+  return (((j >> 3) << 3) + x) * 8 + (j & 7);
+}
 
 // LOGP: log2 of the LDS row pitch (>= W + 2); VR: virtual rows held per channel.
 // BM: output channels per workgroup (64 or 128; the wavefront tile is (BM/2) x 32).
@@ -109,7 +123,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 4))) void
   for (bool again = true; again;) {
   int tile, ch_begin, ch_end, tile_rel = 0;
   if (!stream) {
-    tile = blockIdx.x;
+    tile = whole_tile_of(a, int(blockIdx.x));
     ch_begin = 0;
     ch_end = nchunks;
     again = false;
@@ -476,6 +490,7 @@ int sgh_dgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *wt, i
   a.Q = g->Q;
   a.total_pix = g->N * g->P * g->Q;
   a.ctiles = p.ctiles;
+  a.xcd_runs = p.dp_tiles % 64 == 0 && !sgh_env().conv_xcd_off;
   a.dp_tiles = p.dp_tiles;
   a.sk_wgs = p.sk_wgs;
   a.sk_units = p.sk_units;

@@ -102,6 +102,7 @@ const sgh_env_switches &sgh_env() {
     s.slab16_off = on("SGH_SLAB16_OFF");
     s.dgrad_tile = num("SGH_DGRAD_TILE", 0, 3), s.wgrad_tile = num("SGH_WGRAD_TILE", 0, 5);
     s.pw_tile = num("SGH_PW_TILE", 1, 2);
+    s.conv_xcd_off = on("SGH_CONV_XCD_OFF");
     const char *bm = getenv("SGH_DGRAD3X3_BM");
     s.dgrad3x3_bm = bm ? (atoi(bm) == 64 ? 64 : 128) : 0;
     return s;

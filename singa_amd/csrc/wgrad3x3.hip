@@ -41,6 +41,11 @@ struct W3Args {
   int RU;                // output rows per unit
   int units_per_image;   // ceil(P / RU)
   int total_units, units_per_split;
+  // 1-D grid of gx * gy * gz workgroups: k tile fastest, then channel tile, then split.  xcd: the j-th
+  // workgroup of XCD x (workgroup w runs on XCD w % 8) takes the logical id x * (count / 8) + j, so that the
+  // tiles of one split -- they read the same pixels of dy and x -- share that XCD's L2.  Only which hardware
+  // computes which partial changes.
+  int gx, gy, gz, xcd;
 };
 
 // LOGP: log2 of the LDS row pitch (>= W + 2 * pad_w); ROWS = RU + 2 slab rows.
@@ -87,8 +92,17 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int half = wave >> 2, w4 = wave & 3;
   const int wm = w4 / WGC, wc = w4 % WGC;
-  const int k0 = blockIdx.x * BM, c0 = blockIdx.y * BC;
-  const int u_begin = blockIdx.z * a.units_per_split;
+  int bx, by, bz;
+  {
+    const int w = int(blockIdx.x), count = a.gx * a.gy * a.gz;
+    const int lw = a.xcd && (count & 7) == 0 ? (w & 7) * (count >> 3) + (w >> 3) : w;
+    bz = lw / (a.gx * a.gy);
+    const int rem = lw - bz * (a.gx * a.gy);
+    by = rem / a.gx;
+    bx = rem - by * a.gx;
+  }
+  const int k0 = bx * BM, c0 = by * BC;
+  const int u_begin = bz * a.units_per_split;
   const int u_end = min(u_begin + a.units_per_split, a.total_units);
   const int PQ = a.P * a.Q, HW = a.H * a.W;
   const unsigned dy_img_bytes = unsigned(a.K) * PQ * 4u, x_img_bytes = unsigned(a.C) * HW * 4u;
@@ -277,7 +291,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         for (int v = 0; v < 16; ++v) acc[i][v] += xch[((i - T0) * 4 * 16 + v) * 64 + wbase];
     }
     // partial[z][tap][k][c]
-    float *pz = a.part + size_t(blockIdx.z) * 9 * a.K * a.C;
+    float *pz = a.part + size_t(bz) * 9 * a.K * a.C;
     const int c = c0 + wc * 32 + (lane & 31);
 #pragma unroll
     for (int i = 0; i < 9; ++i) {
@@ -431,7 +445,10 @@ int sgh_wgrad3x3_run(const sgh_conv_geom *g, const float *dy, const float *x, fl
   a.units_per_image = p.upi;
   a.total_units = p.total_units;
   a.units_per_split = p.units_per_split;
-  dim3 grid((g->K + p.bm - 1) / p.bm, (g->C + p.bc - 1) / p.bc, p.splits);
+  a.gx = (g->K + p.bm - 1) / p.bm, a.gy = (g->C + p.bc - 1) / p.bc, a.gz = p.splits;
+  a.xcd = sgh_env().conv_xcd_off ? 0 : 1;
+  if (long(a.gx) * a.gy * a.gz >= (long(1) << 31)) return SGH_EUNSUPPORTED;
+  dim3 grid(unsigned(a.gx * a.gy * a.gz), 1, 1);
   int rc = SGH_EUNSUPPORTED;
   sgh_prof_kernel_begin("conv_wgrad/k_wgrad3x3", 2.0 * g->N * g->K * g->P * g->Q * g->C * 9);
 #define W3_CASE(BM_, BC_, LOGP_, ROWS_) \
