@@ -146,6 +146,9 @@ def main():
     ap.add_argument("--with-forward", action="store_true",
                     help="time whole training steps -- forward pass, backward pass and update, inputs resident on the "
                          "device -- instead of the backward pass and update alone (the metric's name says so)")
+    ap.add_argument("--no-reference-tape", action="store_true",
+                    help="skip the second measurement of the unfused one-stream tape (profiler runs: keeps its "
+                         "kernels out of the trace)")
     ap.add_argument("--per-parameter-update", action="store_true",
                     help="update each parameter right after its gradient (one launch each) instead of one fused launch")
     args = ap.parse_args()
@@ -233,7 +236,7 @@ def main():
     # parameter (python/singa/autograd.py:128-224, python/singa/opt.py:269-310).  A short second measurement
     # after the timed region, reported beside the headline figure.
     reference_tape = None
-    if not (args.no_fusion or args.with_forward):
+    if not (args.no_fusion or args.with_forward or args.no_reference_tape):
         saved = {f: getattr(hip, f) for f in ("fuse_bn_relu", "fuse_dgrad_add", "fuse_add_relu", "fuse_wgrad_bias",
                                               "batch_relayout", "overlap_wgrad", "fuse_forward")}
         hip.set_fusion(False)
