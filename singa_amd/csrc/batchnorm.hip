@@ -529,6 +529,7 @@ inline ChipPlan chip_plan(int N, int C, int HW) {
   if (p.ragged && (S::VEC * sizeof(typename S::elem) != 16 || HW < S::VEC || sgh_env().bn_ragged_off ||
                    size_t(N) * C * HW * sizeof(typename S::elem) >= (size_t(1) << 31)))
     return p;
+  if (size_t(N) * C * HW * sizeof(typename S::elem) >= (size_t(1) << 32)) return p;   // (32-bit byte offsets)
   const long TV = long(N) * ((HW + S::VEC - 1) / S::VEC);        // vectors per channel
   // 512 threads (two workgroups per CU: one loads while the other waits or stores) unless that cuts the
   // channel into more slices than one wavefront can poll
@@ -570,6 +571,19 @@ inline ChipPlan chip_plan(int N, int C, int HW) {
   p.ok = long(C) * p.G < 0x7fffffffL && chip_slices_fit(p.G, C, p.nt);
   return p;
 }
+
+// (image, piece within the plane) of a thread's vectors: vector j of a thread is number first + j * NT of the
+// channel, so one division places the first and every later one is a step of NT / PV images and NT % PV pieces
+// with at most one carry -- a division by a run-time value per vector costs about twenty vector instructions,
+// a step four.
+struct ChipWalk {
+  int n, r;
+  __device__ __forceinline__ void step(int dn, int dr, int PV) {
+    n += dn;
+    r += dr;
+    if (r >= PV) r -= PV, ++n;
+  }
+};
 
 // RAGGED: planes that are not whole vectors.  A plane of HW elements is covered by ceil(HW / V) pieces of 16 bytes
 // at 2- or 4-byte alignment (buffer loads and stores take any); the last piece starts at HW - V, i.e. overlaps
@@ -624,7 +638,14 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
   const float mean = save_mean[c], invstd = save_invstd[c];
   const float gm = gamma[c], be = RELU ? beta[c] : 0.f;
   auto gate = [&](float d, float v) { return !RELU || S::stored_positive(bn_out(v, mean, invstd, gm, be)) ? d : 0.f; };
-  const raw *xg = reinterpret_cast<const raw *>(x), *dg_ = reinterpret_cast<const raw *>(dy);
+  // byte offsets within a tensor are 32 bits (the plan leaves larger tensors to the two-pass kernels): the
+  // addresses are then a uniform base plus a per-lane offset, with no 64-bit arithmetic per vector
+  const char *xb = reinterpret_cast<const char *>(x), *db_ = reinterpret_cast<const char *>(dy);
+  const unsigned CPV = unsigned(s.C) * unsigned(PV), cPV = unsigned(c) * unsigned(PV);
+  const int dn = NT / PV, dr = NT - dn * PV;
+  ChipWalk first;
+  first.n = (lo + t) / PV, first.r = (lo + t) - first.n * PV;
+  auto vec_bytes = [&](const ChipWalk &w) { return (unsigned(w.n) * CPV + cPV + unsigned(w.r)) * 16u; };
   const int tensor_bytes = RAGGED ? int(size_t(s.N) * s.C * s.HW * sizeof(elem)) : 0;
   const __amdgpu_buffer_rsrc_t rxb = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(x), 0, tensor_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rdb = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(dy), 0, tensor_bytes, 0x00020000);
@@ -644,33 +665,38 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     const rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(x), 0, int(bytes), 0x00020000);
     const rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(dy), 0, int(bytes), 0x00020000);
     const int wbase = __builtin_amdgcn_readfirstlane(t & ~63);
+    ChipWalk w = first;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
       const int iv = lo + j * NT + t;
       int voff = int(0x80000000u);   // (beyond the buffer: the slot reads as zero and is never used)
-      if (iv < hi) {
-        const int n = iv / PV, r = iv - n * PV;
-        voff = int((unsigned(n) * unsigned(s.C) + unsigned(c)) * unsigned(PV) + unsigned(r)) * 16;
-      }
+      if (iv < hi) voff = int(vec_bytes(w));
+      w.step(dn, dr, PV);
       typedef unsigned char __attribute__((address_space(3))) * lds_ptr;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(chip_lds + size_t((0 * NL + j) * NT + wbase) * 16), 16, voff, 0, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr)(chip_lds + size_t((1 * NL + j) * NT + wbase) * 16), 16, voff, 0, 0, 0);
     }
   }
   // every load of the slice is issued before the first value is used
+  ChipWalk wreg = first;   // the walk at the first register vector
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int iv = lo + (NL + i) * NT + t;
-    if (iv < hi) {
-      const int n = iv / PV, r = iv - n * PV;
-      if constexpr (RAGGED) {
-        xv[i] = __builtin_bit_cast(raw, __builtin_amdgcn_raw_buffer_load_b128(rxb, piece(n, r), 0, 0));
-        dv[i] = __builtin_bit_cast(raw, __builtin_amdgcn_raw_buffer_load_b128(rdb, piece(n, r), 0, 0));
-      } else {
-        const size_t off = (size_t(n) * s.C + c) * PV + r;
-        xv[i] = __builtin_nontemporal_load(xg + off);
-        dv[i] = __builtin_nontemporal_load(dg_ + off);
+  for (int j = 0; j < NL; ++j) wreg.step(dn, dr, PV);
+  {
+    ChipWalk w = wreg;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int iv = lo + (NL + i) * NT + t;
+      if (iv < hi) {
+        if constexpr (RAGGED) {
+          xv[i] = __builtin_bit_cast(raw, __builtin_amdgcn_raw_buffer_load_b128(rxb, piece(w.n, w.r), 0, 0));
+          dv[i] = __builtin_bit_cast(raw, __builtin_amdgcn_raw_buffer_load_b128(rdb, piece(w.n, w.r), 0, 0));
+        } else {
+          const unsigned off = vec_bytes(w);
+          xv[i] = __builtin_nontemporal_load(reinterpret_cast<const raw *>(xb + off));
+          dv[i] = __builtin_nontemporal_load(reinterpret_cast<const raw *>(db_ + off));
+        }
       }
+      w.step(dn, dr, PV);
     }
   }
   float a = 0.f, b = 0.f, b1 = 0.f;
@@ -705,10 +731,14 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
         BN_CHIP_ACCUMULATE(xl, dl, 0)
       }
   }
+  {
+    ChipWalk w = wreg;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int iv = lo + (NL + i) * NT + t;
-    if (iv < hi) BN_CHIP_ACCUMULATE(xv[i], dv[i], (iv % PV == PV - 1 ? tail_skip : 0))
+    for (int i = 0; i < NV; ++i) {
+      const int iv = lo + (NL + i) * NT + t;
+      if (iv < hi) BN_CHIP_ACCUMULATE(xv[i], dv[i], (w.r == PV - 1 ? tail_skip : 0))
+      if constexpr (RAGGED) w.step(dn, dr, PV);
+    }
   }
 #undef BN_CHIP_ACCUMULATE
   b += b1;
@@ -762,11 +792,10 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
   const float k = gm * invstd;
   const float rM = float(1.0 / (double(s.N) * s.HW));
   const float c0 = db * rM, c1 = dg * rM;
-  raw *og = reinterpret_cast<raw *>(dx);
-#define BN_CHIP_FINISH(IV, XR, DR)                                                                            \
+  char *ob = reinterpret_cast<char *>(dx);
+#define BN_CHIP_FINISH(W, XR, DR)                                                                             \
   {                                                                                                           \
-    const int n = (IV) / PV, r = (IV) - n * PV;                                                               \
-    float v[V], d[V], o[V];                                                                                   \
+    float v[V], d[V], o[V];                                                                                \
     S::template load16<false>(reinterpret_cast<const elem *>(&(XR)), v);                                      \
     S::template load16<false>(reinterpret_cast<const elem *>(&(DR)), d);                                      \
     _Pragma("unroll") for (int q = 0; q < V; ++q)                                                             \
@@ -774,25 +803,31 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     raw ov;                                                                                                   \
     S::store16(reinterpret_cast<elem *>(&ov), o);                                                             \
     if constexpr (RAGGED)                                                                                     \
-      __builtin_amdgcn_raw_buffer_store_b128(ov, rob, piece(n, r), 0, 0);                                     \
+      __builtin_amdgcn_raw_buffer_store_b128(ov, rob, piece((W).n, (W).r), 0, 0);                             \
     else   /* (non-temporal: 3-7 % on the 25-50 MB tensors, whose lines otherwise wait dirty in L2 for the end of the kernel) */ \
-      __builtin_nontemporal_store(ov, og + (size_t(n) * s.C + c) * PV + r);                                   \
+      __builtin_nontemporal_store(ov, reinterpret_cast<raw *>(ob + vec_bytes(W)));                            \
   }
   if constexpr (NL > 0) {
+    ChipWalk w = first;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
       const int iv = lo + j * NT + t;
       if (iv < hi) {
         const raw xl = *reinterpret_cast<const raw *>(chip_lds + size_t((0 * NL + j) * NT + t) * 16);
         const raw dl = *reinterpret_cast<const raw *>(chip_lds + size_t((1 * NL + j) * NT + t) * 16);
-        BN_CHIP_FINISH(iv, xl, dl)
+        BN_CHIP_FINISH(w, xl, dl)
       }
+      w.step(dn, dr, PV);
     }
   }
+  {
+    ChipWalk w = wreg;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int iv = lo + (NL + i) * NT + t;
-    if (iv < hi) BN_CHIP_FINISH(iv, xv[i], dv[i])
+    for (int i = 0; i < NV; ++i) {
+      const int iv = lo + (NL + i) * NT + t;
+      if (iv < hi) BN_CHIP_FINISH(w, xv[i], dv[i])
+      w.step(dn, dr, PV);
+    }
   }
 #undef BN_CHIP_FINISH
 }
