@@ -645,7 +645,7 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
   const int dn = NT / PV, dr = NT - dn * PV;
   ChipWalk first;
   first.n = (lo + t) / PV, first.r = (lo + t) - first.n * PV;
-  auto vec_bytes = [&](const ChipWalk &w) { return (unsigned(w.n) * CPV + cPV + unsigned(w.r)) * 16u; };
+  auto vec_bytes = [&](const ChipWalk &w) { return (unsigned(w.n) * CPV + cPV + unsigned(w.r)) * unsigned(sizeof(raw)); };
   const int tensor_bytes = RAGGED ? int(size_t(s.N) * s.C * s.HW * sizeof(elem)) : 0;
   const __amdgpu_buffer_rsrc_t rxb = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(x), 0, tensor_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rdb = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem *>(dy), 0, tensor_bytes, 0x00020000);
@@ -848,7 +848,7 @@ constexpr int chip_fwd_nv(bool two) {
 template <class S>
 inline ChipPlan chip_fwd_plan(int N, int C, int HW, bool two) {
   ChipPlan p{false, 0, 0, 512, 0, false};
-  if (HW % S::VEC != 0) return p;
+  if (HW % S::VEC != 0 || size_t(N) * C * HW * sizeof(typename S::elem) >= (size_t(1) << 32)) return p;
   const long TV = long(N) * (HW / S::VEC);
   const long per_wg = 512L * chip_fwd_nv<S>(two);
   long G = (TV + per_wg - 1) / per_wg;
@@ -896,14 +896,20 @@ __global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem
   const int PV = s.HW / V, TV = s.N * PV;
   const int lo = g * vpg, hi = min(lo + vpg, TV);
   const float pivot = S::ld(x + size_t(c) * s.HW);
-  const raw *xg = reinterpret_cast<const raw *>(x);
+  // the vectors of a thread are walked in steps of NT (ChipWalk), byte offsets are 32 bits from a uniform base
+  const char *xb = reinterpret_cast<const char *>(x);
+  const unsigned CPV = unsigned(s.C) * unsigned(PV), cPV = unsigned(c) * unsigned(PV);
+  const int dn = NT / PV, dr = NT - dn * PV;
+  ChipWalk first;
+  first.n = (lo + t) / PV, first.r = (lo + t) - first.n * PV;
+  auto vec_bytes = [&](const ChipWalk &w) { return (unsigned(w.n) * CPV + cPV + unsigned(w.r)) * unsigned(sizeof(raw)); };
   raw xv[NV];
+  {
+    ChipWalk w = first;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int iv = lo + i * NT + t;
-    if (iv < hi) {
-      const int n = iv / PV, r = iv - n * PV;
-      xv[i] = __builtin_nontemporal_load(xg + (size_t(n) * s.C + c) * PV + r);
+    for (int i = 0; i < NV; ++i) {
+      if (lo + i * NT + t < hi) xv[i] = __builtin_nontemporal_load(reinterpret_cast<const raw *>(xb + vec_bytes(w)));
+      w.step(dn, dr, PV);
     }
   }
   float a = 0.f, b = 0.f;
@@ -922,14 +928,12 @@ __global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem
   // the second tensor's slice is requested now and arrives during the block sums and the exchange
   raw zr[ACT == 2 ? NV : 1];
   if constexpr (ACT == 2) {
-    const raw *zg = reinterpret_cast<const raw *>(z);
+    const char *zb = reinterpret_cast<const char *>(z);
+    ChipWalk w = first;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int iv = lo + i * NT + t;
-      if (iv < hi) {
-        const int n = iv / PV, r = iv - n * PV;
-        zr[i] = __builtin_nontemporal_load(zg + (size_t(n) * s.C + c) * PV + r);
-      }
+      if (lo + i * NT + t < hi) zr[i] = __builtin_nontemporal_load(reinterpret_cast<const raw *>(zb + vec_bytes(w)));
+      w.step(dn, dr, PV);
     }
   }
   a = sgh_block_sum(a, red);
@@ -991,12 +995,12 @@ __global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem
     }
   }
   const float gm = gamma[c], be = beta[c];
-  raw *og = reinterpret_cast<raw *>(y);
+  char *ob = reinterpret_cast<char *>(y);
+  ChipWalk w = first;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
+  for (int i = 0; i < NV; ++i, w.step(dn, dr, PV)) {
     const int iv = lo + i * NT + t;
     if (iv < hi) {
-      const int n = iv / PV, r = iv - n * PV;
       float v[V], o[V], zv[V];
       S::template load16<false>(reinterpret_cast<const elem *>(&xv[i]), v);
       if constexpr (ACT == 2) S::template load16<false>(reinterpret_cast<const elem *>(&zr[i]), zv);
@@ -1005,7 +1009,7 @@ __global__ __launch_bounds__(512, 4) void k_bn_fwd_onchip(const typename S::elem
         o[q] = bn_fwd_value<S, ACT>(bn_out_rounded(v[q], mean, invstd, gm, be), ACT == 2 ? zv[q] : 0.f);
       raw ov;
       S::store16(reinterpret_cast<elem *>(&ov), o);
-      og[(size_t(n) * s.C + c) * PV + r] = ov;
+      *reinterpret_cast<raw *>(ob + vec_bytes(w)) = ov;
     }
   }
 }
