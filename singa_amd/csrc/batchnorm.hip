@@ -706,12 +706,16 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     float v[V], d[V];                                                                                         \
     S::template load16<false>(reinterpret_cast<const elem *>(&(XR)), v);                                      \
     S::template load16<false>(reinterpret_cast<const elem *>(&(DR)), d);                                      \
+    if constexpr (RELU) {   /* the gated gradient replaces the stored one (exactly: it is that value or zero), */ \
+                            /* so the second pass does not evaluate the gate again */                         \
+      _Pragma("unroll") for (int q = 0; q < V; ++q) d[q] = gate(d[q], v[q]);                                  \
+      S::store16(reinterpret_cast<elem *>(&(DR)), d);                                                         \
+    }                                                                                                         \
     if constexpr (RAGGED) {                                                                                   \
       _Pragma("unroll") for (int q = 0; q < V; ++q) d[q] = q < (SKIP) ? 0.f : d[q];                           \
     }                                                                                                         \
     _Pragma("unroll") for (int q = 0; q < V; q += 4) {                                                        \
-      const float d0 = gate(d[q], v[q]), d1 = gate(d[q + 1], v[q + 1]), d2 = gate(d[q + 2], v[q + 2]),        \
-                  d3 = gate(d[q + 3], v[q + 3]);                                                              \
+      const float d0 = d[q], d1 = d[q + 1], d2 = d[q + 2], d3 = d[q + 3];                                     \
       a += (d0 + d1) + (d2 + d3);                                                                             \
       b = __builtin_fmaf(d0, (v[q] - mean) * invstd, b);                                                      \
       b1 = __builtin_fmaf(d1, (v[q + 1] - mean) * invstd, b1);                                                \
@@ -727,8 +731,9 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     for (int j = 0; j < NL; ++j)
       if (lo + j * NT + t < hi) {
         const raw xl = *reinterpret_cast<const raw *>(chip_lds + size_t((0 * NL + j) * NT + t) * 16);
-        const raw dl = *reinterpret_cast<const raw *>(chip_lds + size_t((1 * NL + j) * NT + t) * 16);
+        raw dl = *reinterpret_cast<const raw *>(chip_lds + size_t((1 * NL + j) * NT + t) * 16);
         BN_CHIP_ACCUMULATE(xl, dl, 0)
+        if constexpr (RELU) *reinterpret_cast<raw *>(chip_lds + size_t((1 * NL + j) * NT + t) * 16) = dl;
       }
   }
   {
@@ -799,7 +804,7 @@ __global__ __launch_bounds__(NT, 4) void k_bn_bwd_onchip(const typename S::elem 
     S::template load16<false>(reinterpret_cast<const elem *>(&(XR)), v);                                      \
     S::template load16<false>(reinterpret_cast<const elem *>(&(DR)), d);                                      \
     _Pragma("unroll") for (int q = 0; q < V; ++q)                                                             \
-        o[q] = k * (gate(d[q], v[q]) - __builtin_fmaf((v[q] - mean) * invstd, c1, c0));                       \
+        o[q] = k * (d[q] - __builtin_fmaf((v[q] - mean) * invstd, c1, c0));   /* (d: gated in the first pass) */ \
     raw ov;                                                                                                   \
     S::store16(reinterpret_cast<elem *>(&ov), o);                                                             \
     if constexpr (RAGGED)                                                                                     \
