@@ -152,7 +152,9 @@ SGH_API int sgh_event_elapsed_ms(sgh_event *start, sgh_event *stop, float *ms);
  * "pool_bwd", "sgd" ...) are tagged with their algorithmic bytes.  A record of a single kernel
  * hands its events to the dispatch itself (hipExtLaunchKernelGGL), so they carry the kernel's
  * own start and end; a record over several kernels is a pair of markers around them, which adds
- * a few microseconds of queue time.  Records nest.  sgh_prof_enable(1) clears old records.
+ * a few microseconds of queue time.  Records nest.  No record is taken while a device records a
+ * graph (sgh_graph_begin .. sgh_graph_end): events inside a recording have no times.  The records
+ * belong to one host thread at a time.  sgh_prof_enable(1) clears old records.
  * sgh_prof_get waits for record i to finish and returns its tag, duration and work. */
 SGH_API int sgh_prof_enable(int on);
 /* Drops the records taken so far and destroys their events (sgh_prof_enable(1) does the same before it starts;

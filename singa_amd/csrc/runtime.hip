@@ -180,11 +180,12 @@ struct ProfRec {
 static std::vector<ProfRec> g_prof;
 static std::vector<size_t> g_prof_open;  // indices of records whose stop event is not recorded yet (nesting)
 static bool g_prof_on = false;
+static std::atomic<int> g_recording{0};   // devices whose stream is recording a graph: no profiling records meanwhile
 
-bool sgh_prof_on() { return g_prof_on; }
+bool sgh_prof_on() { return g_prof_on && g_recording.load(std::memory_order_relaxed) == 0; }
 
 void sgh_prof_start(const char *tag, double work, hipStream_t s) {
-  if (!g_prof_on) return;
+  if (!sgh_prof_on()) return;
   ProfRec r{tag, work, nullptr, nullptr};
   if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) return;
   (void)hipEventRecord(r.a, s);
@@ -193,7 +194,7 @@ void sgh_prof_start(const char *tag, double work, hipStream_t s) {
 }
 
 void sgh_prof_stop(hipStream_t s) {
-  if (!g_prof_on || g_prof_open.empty()) return;
+  if (!sgh_prof_on() || g_prof_open.empty()) return;
   (void)hipEventRecord(g_prof[g_prof_open.back()].b, s);
   g_prof_open.pop_back();
 }
@@ -206,7 +207,7 @@ static bool g_prof_kernel_spanned = false;
 void sgh_prof_kernel_begin(const char *tag, double work) {
   g_prof_kernel = -1;
   g_prof_kernel_spanned = false;
-  if (!g_prof_on) return;
+  if (!sgh_prof_on()) return;
   ProfRec r{tag, work, nullptr, nullptr};
   if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) return;
   g_prof_kernel = long(g_prof.size());
@@ -451,12 +452,14 @@ int sgh_graph_begin(sgh_device *dev) {
   // relaxed mode: the pool may still call hipMalloc while the stream records
   SGH_HIP_TRY(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeRelaxed));
   dev->capturing = true;
+  g_recording.fetch_add(1, std::memory_order_relaxed);
   return SGH_OK;
 }
 
 int sgh_graph_end(sgh_device *dev, sgh_graph **out) {
   if (!dev || !out || !dev->capturing) return SGH_EINVAL;
   dev->capturing = false;
+  g_recording.fetch_sub(1, std::memory_order_relaxed);
   hipGraph_t g = nullptr;
   hipError_t e = hipStreamEndCapture(dev->stream, &g);
   sgh_graph *gr = new (std::nothrow) sgh_graph();

@@ -316,6 +316,40 @@ def test_profiling_records_and_their_release(singa, dev):
     assert (dx.to_numpy() == 2.0).all()
 
 
+def test_no_profiling_records_inside_a_recording(singa, dev):
+    """While the device records a graph no profiling record is taken (events inside a recording have no
+    times); the recorded kernel replays with the right result, and records are taken again afterwards."""
+    import ctypes as C
+    from singa_amd import _lib
+    lib = _lib.lib()
+    m = 70000
+    x = singa.from_numpy(np.linspace(-1, 1, m, dtype=np.float32), dev)
+    dy = singa.Tensor((m,), dev); dy.SetFloatValue(3.0)
+    n = C.c_int(-1)
+    assert lib.sgh_prof_enable(1) == 0
+    try:
+        dev.EnableGraph(True)
+        dx = singa.ReLUBackward(dy, x)
+        dev.EnableGraph(False)
+        assert lib.sgh_prof_count(C.byref(n)) == 0 and n.value == 0
+        dev.RunGraph()
+        dev.Sync()
+        assert lib.sgh_prof_count(C.byref(n)) == 0 and n.value == 0
+        want = np.where(np.linspace(-1, 1, m, dtype=np.float32) > 0, np.float32(3.0), np.float32(0.0))
+        assert (dx.to_numpy() == want).all()
+        dx2 = singa.ReLUBackward(dy, x)     # eager again: one record, with a duration
+        dev.Sync()
+        assert lib.sgh_prof_count(C.byref(n)) == 0 and n.value == 1
+        buf = C.create_string_buffer(64)
+        ms, work = C.c_float(), C.c_double()
+        assert lib.sgh_prof_get(0, buf, 64, C.byref(ms), C.byref(work)) == 0 and ms.value > 0
+        assert (dx2.to_numpy() == want).all()
+    finally:
+        dev.ResetGraph()
+        lib.sgh_prof_enable(0)
+        lib.sgh_prof_clear()
+
+
 def test_upload_without_waiting(singa, dev):
     """sgh_upload_async: the host buffer may be overwritten as soon as the call returns, copies land
     in stream order (more uploads than staging slots in a row), oversize copies take the blocking path."""
