@@ -4,6 +4,8 @@ the CPU oracle, through the C ABI.
 Tolerances: max-pool routing and average pooling are bit-exact; conv and BatchNorm reductions
 are compared with the normalised L2 error ||gpu - cpu|| / ||cpu|| <= 1e-3 (fp32), the bound the
 task states for reductions whose summation order differs from the CPU's by construction."""
+import os
+
 import numpy as np
 import pytest
 
@@ -395,6 +397,44 @@ def test_conv_full_size_properties(singa, dev, shape):
     # linearity: dgrad(2*dy) == 2*dgrad(dy) exactly (scaling by a power of two)
     dx2 = singa.GpuConvBackwardx(singa.from_numpy(dy * 2, dev), wd, xd, h).to_numpy()
     assert_bit_equal(dx2, dx * 2, "dgrad linearity")
+
+
+_TILE_ORDER_CHILD = r'''
+import hashlib, sys, numpy as np
+sys.path.insert(0, sys.argv[1])
+from singa_amd import singa_wrap as singa
+dev = singa.create_hip_gpu_on(0)
+r = np.random.default_rng(99)
+for (N, C, H, K, st) in [(64, 64, 56, 64, 1), (64, 128, 28, 128, 1), (64, 64, 56, 128, 2), (8, 512, 7, 512, 1)]:
+    x = r.standard_normal((N, C, H, H)).astype(np.float32)
+    w = r.standard_normal((K, C, 3, 3)).astype(np.float32)
+    dy = r.standard_normal((N, K, H // st, H // st)).astype(np.float32)
+    xd, wd, dyd = singa.from_numpy(x, dev), singa.from_numpy(w, dev), singa.from_numpy(dy, dev)
+    h = singa.CudnnConvHandle(xd, (3, 3), (st, st), (1, 1), C, K, False)
+    dx = singa.GpuConvBackwardx(dyd, wd, xd, h).to_numpy()
+    dw = singa.GpuConvBackwardW(dyd, xd, wd, h).to_numpy()
+    print(hashlib.sha256(dx.tobytes()).hexdigest(), hashlib.sha256(dw.tobytes()).hexdigest(), flush=True)
+'''
+
+
+def test_conv_tile_order_per_xcd_changes_no_bit(tmp_path):
+    """The fp32 3x3 gradient kernels deal their tiles to workgroups per XCD (runs of eight neighbouring tiles in the
+    data gradient, the tiles of one reduction split in the weight gradient); SGH_CONV_XCD_OFF deals them in launch
+    order.  The switch is read once per process, so two child processes compute the same seeded gradients at full
+    size (enough tiles for whole rounds of the chip, where the order differs) and their results agree bit for bit."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = tmp_path / "tile_order_child.py"
+    script.write_text(_TILE_ORDER_CHILD)
+    outs = []
+    for off in (False, True):
+        env = dict(os.environ)
+        env.pop("SGH_CONV_XCD_OFF", None)
+        if off:
+            env["SGH_CONV_XCD_OFF"] = "1"
+        outs.append(subprocess.check_output([sys.executable, str(script), root], env=env, timeout=300).decode().split())
+    assert len(outs[0]) == 8 and outs[0] == outs[1]
 
 
 def test_conv_argument_checks(singa, dev):
