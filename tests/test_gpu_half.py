@@ -247,6 +247,29 @@ def test_batchnorm_16bit_storage(singa, dev, kind, shape):
     assert nl2(ds.to_numpy(), ds_o) < 1e-3 and nl2(db.to_numpy(), db_o) < 1e-3
 
 
+def _random_bn_shapes16(count, seed):
+    """Seeded shapes for the 16-bit one-pass BatchNorm kernels: planes of whole 16-byte vectors (8 elements), of whole
+    8-byte vectors only, and of neither (overlapping pieces); a thread's vectors stepping over several images or
+    lying in one plane; one slice per channel and many."""
+    r = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < count:
+        C = int(r.choice([1, 3, 8, 24, 64, 130, 256, 300]))
+        H = int(r.integers(1, 31))
+        W = H if r.random() < 0.5 else int(r.integers(1, 31))
+        N = int(r.integers(1, 65))
+        if not 4000 <= N * C * H * W <= 4_000_000:
+            continue
+        shapes.append((N, C, H, W))
+    return shapes
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", _random_bn_shapes16(24, 20241126))
+def test_batchnorm_16bit_shape_sweep(singa, dev, kind, shape):
+    test_batchnorm_16bit_storage(singa, dev, kind, shape)
+
+
 @pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("shape", [(4, 3, 5, 6), (2, 5, 7, 7), (8, 64, 28, 28), (3, 7, 4, 2), (16, 24, 14, 14)])
 def test_batchnorm_inference(singa, dev, kind, shape):

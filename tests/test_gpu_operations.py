@@ -649,6 +649,29 @@ def test_bn_vs_oracle(singa, dev, shape):
     assert_bit_equal(ds2.to_numpy(), ds.to_numpy())
 
 
+def _random_bn_shapes(count, seed):
+    """Seeded shapes aimed at the planning and indexing of the one-pass BatchNorm kernels: plane sizes that are
+    and are not whole 16-byte vectors, fewer / more vectors per plane than a workgroup has threads (so that a
+    thread's vectors step over several images, or several of them lie in one plane), channels in one slice and
+    in many, channel counts below and above the number of CUs."""
+    r = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < count:
+        C = int(r.choice([1, 2, 3, 8, 24, 64, 130, 256, 300]))
+        H = int(r.integers(1, 31))
+        W = H if r.random() < 0.5 else int(r.integers(1, 31))
+        N = int(r.integers(1, 49))
+        if not 2000 <= N * C * H * W <= 4_000_000:
+            continue
+        shapes.append((N, C, H, W))
+    return shapes
+
+
+@pytest.mark.parametrize("shape", _random_bn_shapes(36, 20241125))
+def test_bn_shape_sweep(singa, dev, shape):
+    test_bn_vs_oracle(singa, dev, shape)
+
+
 def _random_conv_cases(count, seed):
     """Seeded geometry sweep aimed at the planning logic of the specialised kernels: channel counts
     around the 32 / 64 / 128 tile edges, image sizes around the 16 / 32 / 64-column slab limits,
